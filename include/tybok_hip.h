@@ -1,0 +1,142 @@
+/*
+ * tybok_hip.h -- C ABI of libtybok_hip.so: MI355X (gfx950) kernels for tybok's fp8
+ * action-inference path.
+ *
+ * Conventions (the ones the reference's own native layer uses for its fused kernels,
+ * tybok/policies/fastwam/kernels/adit_fused_bindings.cpp:21-71):
+ *   - every pointer is a DEVICE pointer unless said otherwise; the caller owns every buffer,
+ *     workspace included; no entry point allocates, frees or synchronises;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); all work is enqueued
+ *     on it, so the calls are legal under stream capture (hipGraph);
+ *   - every entry point returns 0 on success or a negative TK_E* code; tk_last_error() gives
+ *     the message of the calling thread's last failure (the reference's host helpers throw
+ *     std::runtime_error and never exit(): tybok/policies/fastwam/kernels/coop_grid.h:20-27);
+ *   - reductions are fixed-order: the same inputs give the same bits on every run and under
+ *     graph replay (the reference's rule: tybok/policies/fastwam/kernels/vdit_gemm_core.cu:7-9).
+ *
+ * Workspace: one caller-owned buffer per stream of at least tk_workspace_bytes() bytes, passed
+ * once through tk_workspace_init() (which zeroes its arrival counters with a fill kernel).
+ * Entry points leave the counters zero on exit.  Two calls that may overlap in time (different
+ * streams) need different workspaces.
+ */
+#ifndef TYBOK_HIP_H
+#define TYBOK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TK_OK 0
+#define TK_EINVAL (-1)   /* bad shape / alignment / argument */
+#define TK_EWORKSPACE (-2) /* workspace too small */
+#define TK_ELAUNCH (-3)  /* HIP launch error */
+
+/* activation of the gated FFN */
+#define TK_ACT_SILU 0      /* SwiGLU: tybok/policies/smolvla/models/layers.py:75-76 */
+#define TK_ACT_GELU_TANH 1 /* GeGLU:  tybok/policies/pi05/models/layers.py:94-95 */
+
+/* suffix mask mode of the expert attention */
+#define TK_MASK_NONE 0   /* no suffix keys (cross-attention over the prefix only) */
+#define TK_MASK_BIDIR 1  /* every action token sees every action token (pi0.5) */
+#define TK_MASK_CAUSAL 2 /* action token i sees action tokens j <= i (SmolVLA) */
+
+/* element types */
+#define TK_BF16 0
+#define TK_F32 1
+
+int tk_version(void);
+const char* tk_last_error(void);
+
+/* Number of compute units of the current device (0 on error); diagnostic only. */
+int tk_device_cus(void);
+
+/* ---- workspace ------------------------------------------------------------------------- */
+/* Bytes that cover every entry point at the shapes of both policies (split-K partials,
+ * attention partials, the FFN's [M, I] intermediate, arrival counters). */
+size_t tk_workspace_bytes(void);
+/* Zero the arrival counters at the head of `ws` (fill kernel, capture-safe). Call once. */
+int tk_workspace_init(void* ws, size_t ws_bytes, void* stream);
+
+/* ---- fp8 weight packing ------------------------------------------------------------------ */
+/* The GEMM reads weights as 32x32-byte tiles in MFMA operand order: tile (nt, kt) holds rows
+ * 32*nt.. and k bytes 32*kt.., stored as 64 consecutive 16-byte lane chunks, so one wave loads a
+ * tile with one fully coalesced 1 KiB global_load_dwordx4.  Rows >= N and k >= K are zero.
+ * Replaces the reference's cached transposed copy `quantize_weight_rows_transposed`
+ * (tybok/policies/pi05/models/triton_expert_mlp_fp8.py:200-218): a layout-only, once-per-model
+ * transform of the checkpoint's row-major `[N, K]` e4m3fn weight
+ * (docs/fastWAM_weight_quantization.md:23-24).  Requires K % 16 == 0. */
+size_t tk_fp8w_packed_bytes(int N, int K);
+int tk_pack_fp8_weight(const void* w8_rowmajor, void* packed, int N, int K, void* stream);
+/* Gate and up weights ([I, K] each) packed into one buffer with their 32-row tiles interleaved
+ * (gate tile j, up tile j, gate tile j+1, ...), so one wave owns matching gate/up columns.
+ * Size = tk_fp8w_packed_bytes(2*I, K); requires I % 32 == 0. */
+int tk_pack_fp8_gate_up(const void* wg8_rowmajor, const void* wu8_rowmajor, void* packed, int I, int K,
+                        void* stream);
+
+/* ---- fp8-weight split-K GEMM ------------------------------------------------------------- */
+/* y[M, N] = bf16( (x[M, K] . W8[N, K]^T) * scale[n] )   (+ optional residual, see below)
+ * bf16 activations, e4m3fn weights (packed), fp32 per-output-channel scale, fp32 accumulate.
+ * Replaces `_w8a8_gemm` / `_down_fp8_splitk_kernel` + `_down_fp8_splitk_reduce_kernel`
+ * (tybok/policies/pi05/models/triton_prefill_mlp.py:62-130,
+ *  tybok/policies/pi05/models/triton_expert_mlp_fp8.py:312-435) with weight-only semantics
+ * (no activation quantisation).
+ *   x: bf16, row stride ldx elements (ldx % 8 == 0, 16-byte aligned); y: bf16, row stride ldy.
+ *   resid: NULL, or a [M, N] tensor (row stride ldr, type resid_dtype) added AFTER the bf16
+ *          rounding of the product: y = bf16(float(bf16(acc*scale)) + float(resid)) -- the
+ *          reference's in-place `out_emb += hidden_states`
+ *          (tybok/policies/smolvla/models/vlm_with_expert.py:386-408).
+ *   split_k: 0 = pick automatically; otherwise the number of K splits (>= 1).
+ */
+int tk_fp8w_gemm(const void* x, int ldx, const void* w_packed, const void* scale, void* y, int ldy,
+                 const void* resid, int ldr, int resid_dtype, int M, int N, int K, int split_k, void* ws,
+                 size_t ws_bytes, void* stream);
+
+/* ---- fused gated FFN ----------------------------------------------------------------------- */
+/* y[M, K] = down( act(gate(x)) * up(x) ) with fp8 weights, bf16 in/out:
+ *   g = bf16(x.Wg^T * sg), u = bf16(x.Wu^T * su), h = bf16(bf16(act(g)) * u), y = bf16(h.Wd^T * sd)
+ * Replaces `MLP.forward` / `GemmaMLP.forward` and the fused chains `triton_norm_gate_up` + down
+ * and `triton_mlp_fp8_chain` (tybok/policies/smolvla/models/layers.py:61-76,
+ * tybok/policies/pi05/models/layers.py:87-95, tybok/policies/smolvla/models/triton_mlp.py:30-144,
+ * tybok/policies/pi05/models/triton_expert_mlp_fp8.py:438-469).
+ *   wgu_packed: tk_pack_fp8_gate_up output; wd_packed: tk_pack_fp8_weight of [K, I].
+ *   resid/ldr/resid_dtype: as in tk_fp8w_gemm, applied to y.
+ * The [M, I] intermediate lives in the workspace (never returned). */
+int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void* sg, const void* su,
+                      const void* wd_packed, const void* sd, void* y, int ldy, const void* resid, int ldr,
+                      int resid_dtype, int M, int K, int I, int act, void* ws, size_t ws_bytes,
+                      void* stream);
+
+/* ---- action-expert attention over the cached prefix ------------------------------------------ */
+/* out[M, H*D] (bf16) = softmax(q.K^T * D^-0.5 + mask) . V over keys [prefix(P); suffix(S)].
+ * Replaces `EagerAttention._forward_eager` / `GemmaAttention._forward_eager`'s core and the fused
+ * `triton_self_attn` / `triton_cross_attn` / `_splitk_flash_kernel`
+ * (tybok/policies/smolvla/models/attention.py:136-187, tybok/policies/pi05/models/layers.py:166-191,
+ *  tybok/policies/smolvla/models/triton_attn.py:586-855,
+ *  tybok/policies/pi05/models/triton_expert_fused_qkv_rope_attn.py:322-433).
+ *   q:      bf16 [M, H, D], element strides (q_sm, q_sh), d contiguous.
+ *   k_pre/v_pre: [P, G, D] of kv_dtype (TK_BF16, or TK_F32 for the SmolVLA cross layers whose
+ *           expert K/V projections are fp32), element strides (pre_sl, pre_sh).
+ *   k_suf/v_suf: bf16 [S, G, D], strides (suf_sl, suf_sh); NULL when S == 0.
+ *   pad:    uint8 [P], 1 = prefix token visible (NULL = all visible).
+ *   mask_mode: TK_MASK_*; q head h reads kv head h / (H / G).
+ *   logits_bf16: 0 = fp32 logits (SmolVLA); 1 = logits rounded to bf16 before the softmax and
+ *           masked with the additive -2.3819763e38 (pi0.5).
+ *   D in {64, 128, 256}; masked logits use finfo(float32).min, so a fully masked row is uniform.
+ */
+int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* v_pre, int pre_sl,
+                   int pre_sh, int kv_dtype, const void* k_suf, const void* v_suf, int suf_sl, int suf_sh,
+                   const void* pad, void* out, int out_sm, int M, int P, int S, int H, int G, int D,
+                   int mask_mode, int logits_bf16, void* ws, size_t ws_bytes, void* stream);
+
+/* ---- diagnostics ------------------------------------------------------------------------------- */
+/* out_f32[256] = value of every e4m3fn code as decoded by the device's conversion instruction
+ * (the weight path of the GEMM); used to assert the OCP (not FNUZ) flavour on the box. */
+int tk_debug_decode_fp8(void* out_f32, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TYBOK_HIP_H */

@@ -1,0 +1,205 @@
+"""GPU parity of the HIP kernels (through the C ABI) against the CPU oracle on seeded inputs.
+
+Tolerances are the ones the task states for bf16 op outputs: rtol 2e-2 / atol 2e-2.
+"""
+
+import pytest
+import torch
+
+from oracle import fp8 as ofp8
+from oracle import ops as oops
+from oracle.inputs import GEMM_MS, GEMM_SHAPES, attn_case, ffn_case, gemm_case
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 2e-2, 2e-2
+
+
+def _close(got: torch.Tensor, want: torch.Tensor, what: str):
+    got = got.float().cpu()
+    want = want.float().cpu()
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite output"
+    err = (got - want).abs()
+    bound = ATOL + RTOL * want.abs()
+    worst = float((err - bound).max())
+    assert worst <= 0, f"{what}: max|err|={float(err.max()):.4g}, exceeds atol+rtol*|ref| by {worst:.4g}"
+
+
+@pytest.fixture(scope="module")
+def tk():
+    from tybok_amd import ops
+
+    return ops
+
+
+def test_device_decodes_ocp_e4m3fn(tk):
+    got = tk.decode_fp8_table().cpu()
+    want = torch.from_numpy(ofp8.e4m3fn_table())
+    ok = ~torch.isnan(want)
+    assert torch.equal(torch.isnan(got), torch.isnan(want)), "NaN codes differ: not the OCP e4m3fn flavour"
+    assert torch.equal(got[ok], want[ok])
+    assert torch.equal(torch.signbit(got[ok]), torch.signbit(want[ok]))
+
+
+def test_pack_layout(tk):
+    g = torch.Generator().manual_seed(0)
+    n, k = 80, 48  # ragged in both directions (3 n-tiles, 2 k-tiles)
+    codes = torch.randint(0, 256, (n, k), generator=g, dtype=torch.uint8)
+    packed = tk.pack_fp8_weight(codes.cuda(), torch.ones(n)).data.cpu()
+    kt_n = 2
+    ref = torch.zeros(3 * kt_n * 1024, dtype=torch.uint8)
+    for nt in range(3):
+        for kt in range(kt_n):
+            for lane in range(64):
+                row = nt * 32 + lane % 32
+                col = kt * 32 + 16 * (lane // 32)
+                if row < n and col < k:
+                    off = ((nt * kt_n + kt) * 64 + lane) * 16
+                    ref[off : off + 16] = codes[row, col : col + 16]
+    assert torch.equal(packed, ref)
+
+
+@pytest.mark.parametrize("k,n", GEMM_SHAPES)
+@pytest.mark.parametrize("m", GEMM_MS)
+def test_gemm_sweep(tk, m, k, n):
+    x, w8, s = gemm_case(m, k, n)
+    want = oops.lin_fp8w(x, w8, s)
+    pw = tk.pack_fp8_weight(w8.cuda(), s.cuda())
+    got = tk.fp8w_gemm(x.cuda(), pw)
+    torch.cuda.synchronize()
+    _close(got, want, f"gemm M={m} K={k} N={n}")
+
+
+@pytest.mark.parametrize("split", [1, 2, 5, 16])
+def test_gemm_split_k_equals_no_split_within_tolerance_and_is_deterministic(tk, split):
+    x, w8, s = gemm_case(50, 2048, 2048)
+    pw = tk.pack_fp8_weight(w8.cuda(), s.cuda())
+    xc = x.cuda()
+    a = tk.fp8w_gemm(xc, pw, split_k=split)
+    b = tk.fp8w_gemm(xc, pw, split_k=split)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b), "same launch twice must give the same bits (fixed-order reduction)"
+    _close(a, oops.lin_fp8w(x, w8, s), f"gemm split_k={split}")
+
+
+@pytest.mark.parametrize("m,k,n", [(3, 16, 32), (33, 48, 40), (50, 720, 720), (64, 80, 96), (241, 960, 2560), (130, 2048, 320)])
+def test_gemm_ragged_shapes(tk, m, k, n):
+    x, w8, s = gemm_case(m, k, n)
+    pw = tk.pack_fp8_weight(w8.cuda(), s.cuda())
+    got = tk.fp8w_gemm(x.cuda(), pw)
+    _close(got, oops.lin_fp8w(x, w8, s), f"gemm ragged M={m} K={k} N={n}")
+
+
+def test_gemm_strided_input_and_residual(tk):
+    x, w8, s = gemm_case(50, 720, 2048)
+    pw = tk.pack_fp8_weight(w8.cuda(), s.cuda())
+    wide = torch.zeros(50, 1440, dtype=torch.bfloat16, device="cuda")
+    wide[:, :720] = x.cuda()
+    g = torch.Generator().manual_seed(9)
+    for rdt in (torch.bfloat16, torch.float32):
+        resid = torch.randn(50, 2048, generator=g).to(rdt)
+        got = tk.fp8w_gemm(wide[:, :720], pw, resid=resid.cuda())
+        y = oops.lin_fp8w(x, w8, s)
+        y += resid  # the reference's in-place add: fp32 math, bf16 result
+        _close(got, y, f"gemm+resid {rdt}")
+
+
+def test_gemm_linearity_at_full_size(tk):
+    # size-independent property at the largest sweep shape: scaling x by 2 scales y by 2 bit-exactly
+    x, w8, s = gemm_case(64, 16384, 2048)
+    pw = tk.pack_fp8_weight(w8.cuda(), s.cuda())
+    a = tk.fp8w_gemm(x.cuda(), pw)
+    b = tk.fp8w_gemm((x * 2).cuda(), pw)
+    assert torch.equal((a.float() * 2).to(torch.bfloat16), b)
+
+
+def test_gemm_rejects_bad_arguments(tk):
+    x, w8, s = gemm_case(4, 32, 32)
+    pw = tk.pack_fp8_weight(w8.cuda(), s.cuda())
+    with pytest.raises(TypeError):
+        tk.fp8w_gemm(x.float().cuda(), pw)
+    with pytest.raises(ValueError):
+        tk.fp8w_gemm(x.cuda()[:, :16], pw)
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        tk.pack_fp8_weight(torch.zeros(32, 24, dtype=torch.uint8, device="cuda"), torch.ones(32))
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
+@pytest.mark.parametrize("m,k,i", [(50, 720, 2048), (50, 1024, 4096), (1, 720, 2048), (64, 960, 2560)])
+def test_gated_ffn(tk, act, m, k, i):
+    x, wg8, sg, wu8, su, wd8, sd = ffn_case(m, k, i, seed=0)
+    want = oops.gated_ffn(x, wg8, sg, wu8, su, wd8, sd, act)
+    wgu = tk.pack_fp8_gate_up(wg8.cuda(), sg, wu8.cuda(), su)
+    wd = tk.pack_fp8_weight(wd8.cuda(), sd)
+    got = tk.fp8w_gated_ffn(x.cuda(), wgu, wd, act)
+    again = tk.fp8w_gated_ffn(x.cuda(), wgu, wd, act)
+    assert torch.equal(got, again)
+    _close(got, want, f"ffn {act} M={m} K={k} I={i}")
+
+
+def test_gated_ffn_residual(tk):
+    x, wg8, sg, wu8, su, wd8, sd = ffn_case(50, 720, 2048, seed=1)
+    resid = torch.randn(50, 720, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
+    want = oops.gated_ffn(x, wg8, sg, wu8, su, wd8, sd, "silu")
+    want += resid
+    wgu = tk.pack_fp8_gate_up(wg8.cuda(), sg, wu8.cuda(), su)
+    wd = tk.pack_fp8_weight(wd8.cuda(), sd)
+    got = tk.fp8w_gated_ffn(x.cuda(), wgu, wd, "silu", resid=resid.cuda())
+    _close(got, want, "ffn+resid")
+
+
+ATTN_CASES = [
+    # m, p, h, g, d, mode, bf16_logits
+    (50, 241, 15, 5, 64, oops.MASK_BIDIR, False),   # config 3
+    (50, 241, 15, 5, 64, oops.MASK_CAUSAL, False),  # SmolVLA self layer, 3 cameras
+    (50, 177, 15, 5, 64, oops.MASK_CAUSAL, False),  # 2 cameras
+    (50, 712, 8, 1, 256, oops.MASK_BIDIR, True),    # pi0.5 expert
+    (7, 5, 4, 2, 64, oops.MASK_CAUSAL, False),      # tiny, ragged
+    (33, 95, 4, 4, 128, oops.MASK_BIDIR, False),
+]
+
+
+@pytest.mark.parametrize("m,p,h,g,d,mode,bl", ATTN_CASES)
+def test_expert_attention(tk, m, p, h, g, d, mode, bl):
+    q, k_pre, v_pre, k_suf, v_suf = attn_case(m, p, h, g, d, seed=0)
+    pad = torch.ones(p, dtype=torch.bool)
+    pad[torch.randperm(p, generator=torch.Generator().manual_seed(3))[: p // 7]] = False
+    want = oops.expert_attention(q, k_pre, v_pre, k_suf, v_suf, pad, mode, bf16_logits=bl)
+    got = tk.expert_attn(q.cuda(), k_pre.cuda(), v_pre.cuda(), k_suf.cuda(), v_suf.cuda(), pad.cuda(), mode, logits_bf16=bl)
+    again = tk.expert_attn(q.cuda(), k_pre.cuda(), v_pre.cuda(), k_suf.cuda(), v_suf.cuda(), pad.cuda(), mode, logits_bf16=bl)
+    assert torch.equal(got, again)
+    _close(got, want, f"attn M={m} P={p} H={h} G={g} D={d} mode={mode}")
+
+
+def test_cross_attention_fp32_kv(tk):
+    # SmolVLA cross layers: fp32 expert K/V over the prefix only, fp32 P.V
+    q, k_pre, v_pre, _, _ = attn_case(50, 241, 15, 5, 64, seed=1, kv_dtype=torch.float32)
+    pad = torch.ones(241, dtype=torch.bool)
+    pad[200:] = False
+    want = oops.expert_attention(q, k_pre, v_pre, None, None, pad, oops.MASK_NONE)
+    got = tk.expert_attn(q.cuda(), k_pre.cuda(), v_pre.cuda(), None, None, pad.cuda(), oops.MASK_NONE)
+    assert want.dtype == torch.float32
+    _close(got, want.to(torch.bfloat16), "cross attn fp32 kv")
+
+
+def test_attention_strided_kv_cache_views(tk):
+    # K/V as slices of a [L, G, D] cache buffer (suffix right behind the prefix), and head-major prefix
+    q, k_pre, v_pre, k_suf, v_suf = attn_case(50, 177, 15, 5, 64, seed=2)
+    kbuf = torch.cat([k_pre, k_suf]).cuda()
+    vbuf = torch.cat([v_pre, v_suf]).cuda()
+    want = oops.expert_attention(q, k_pre, v_pre, k_suf, v_suf, torch.ones(177, dtype=torch.bool), oops.MASK_CAUSAL)
+    got = tk.expert_attn(q.cuda(), kbuf[:177], vbuf[:177], kbuf[177:], vbuf[177:], None, oops.MASK_CAUSAL)
+    _close(got, want, "attn cache views")
+    k_hm = k_pre.permute(1, 0, 2).contiguous().cuda().permute(1, 0, 2)  # [P, G, D] view of [G, P, D]
+    v_hm = v_pre.permute(1, 0, 2).contiguous().cuda().permute(1, 0, 2)
+    got = tk.expert_attn(q.cuda(), k_hm, v_hm, k_suf.cuda(), v_suf.cuda(), None, oops.MASK_CAUSAL)
+    _close(got, want, "attn head-major prefix")
+
+
+def test_attention_fully_masked_prefix_is_uniform(tk):
+    q, k_pre, v_pre, _, _ = attn_case(50, 64, 15, 5, 64, seed=3)
+    none = torch.zeros(64, dtype=torch.bool)
+    want = oops.expert_attention(q, k_pre, v_pre, None, None, none, oops.MASK_NONE)
+    got = tk.expert_attn(q.cuda(), k_pre.cuda(), v_pre.cuda(), None, None, none.cuda(), oops.MASK_NONE)
+    _close(got, want, "attn fully masked")

@@ -1,0 +1,250 @@
+// extern "C" entry points of libtybok_hip.so (declared in include/tybok_hip.h).
+// Host-side argument checks, launch geometry, workspace carving.  No allocation, no sync.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/tybok_hip.h"
+#include "tk_common.h"
+#include "tk_kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// workspace carving (bytes)
+constexpr size_t kCounterBytes = TK_WS_COUNTER_BYTES;
+constexpr size_t kPartialOff = kCounterBytes;
+constexpr size_t kPartialBytes = 24ull << 20;  // split-K / kv-split fp32 partials
+constexpr size_t kHiddenOff = kPartialOff + kPartialBytes;
+constexpr size_t kHiddenBytes = TK_WS_TOTAL_BYTES - kHiddenOff;  // FFN [M, I] bf16 intermediate
+constexpr int kMaxCounters = (int)(kCounterBytes / 4);
+
+bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+int g_cus = -1;
+int device_cus() {
+  if (g_cus < 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    g_cus = n;
+  }
+  return g_cus;
+}
+
+// One GEMM launch (plain or gated).  `N` is the logical output width.
+int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, const float* s1, void* y, int ldy,
+                const void* resid, int ldr, int resid_dtype, int M, int N, int K, int split_k, int act, void* ws,
+                size_t ws_bytes, hipStream_t st) {
+  if (M <= 0 || N <= 0 || K <= 0) return fail(TK_EINVAL, "gemm: non-positive shape M=%d N=%d K=%d", M, N, K);
+  if (K % 16) return fail(TK_EINVAL, "gemm: K=%d must be a multiple of 16", K);
+  if (ldx % 8 || ldx < K) return fail(TK_EINVAL, "gemm: ldx=%d must be >= K and a multiple of 8", ldx);
+  if (ldy < N) return fail(TK_EINVAL, "gemm: ldy=%d < N=%d", ldy, N);
+  if (!x || !w_packed || !s0 || !y) return fail(TK_EINVAL, "gemm: null pointer");
+  if (!aligned16(x) || !aligned16(w_packed)) return fail(TK_EINVAL, "gemm: x and w_packed must be 16-byte aligned");
+  if (resid && resid_dtype != TK_BF16 && resid_dtype != TK_F32) return fail(TK_EINVAL, "gemm: bad resid_dtype");
+  const bool gated = s1 != nullptr;
+  if (gated && (N % 32)) return fail(TK_EINVAL, "gated gemm: I=%d must be a multiple of 32", N);
+
+  GemmArgs a;
+  a.x = (const u16*)x;
+  a.ldx = ldx;
+  a.w = (const uint8_t*)w_packed;
+  a.s0 = s0;
+  a.s1 = s1;
+  a.y = (u16*)y;
+  a.ldy = ldy;
+  a.resid = resid;
+  a.ldr = ldr;
+  a.resid_f32 = resid_dtype == TK_F32;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.KT = (K + 31) / 32;
+  a.ntiles = ((N + 31) / 32) * (gated ? 2 : 1);
+  a.act = act;
+
+  const int MT = M <= 32 ? 1 : 2;
+  const int mblocks = (M + 32 * MT - 1) / (32 * MT);
+  const int cus = device_cus();
+  int NT = 2;
+  if (!gated && ((a.ntiles + 1) / 2) * mblocks < cus / 2) NT = 1;  // few columns: finer strips
+  const int strips = (a.ntiles + NT - 1) / NT;
+  const int blocks0 = strips * mblocks;
+  const int NW = 4;
+  int ks = split_k;
+  if (ks <= 0) {
+    ks = 1;
+    if (blocks0 < cus) {
+      ks = (cus + blocks0 - 1) / blocks0;
+      const int max_by_k = a.KT / (NW * 2) > 1 ? a.KT / (NW * 2) : 1;  // keep >= 2 k tiles per wave
+      if (ks > max_by_k) ks = max_by_k;
+    }
+  }
+  if (ks > a.KT) ks = a.KT;
+  if (ks > 64) ks = 64;
+  a.ksplit = ks;
+  a.partial = nullptr;
+  a.counters = nullptr;
+  if (ks > 1) {
+    if (!ws) return fail(TK_EWORKSPACE, "gemm: split_k=%d needs a workspace", ks);
+    const size_t need = (size_t)blocks0 * ks * MT * NT * 4096;
+    if (blocks0 > kMaxCounters || need > kPartialBytes || ws_bytes < kPartialOff + need)
+      return fail(TK_EWORKSPACE, "gemm: workspace too small (need %zu partial bytes, %d counters)", need, blocks0);
+    a.partial = (float*)((char*)ws + kPartialOff);
+    a.counters = (int*)ws;
+  }
+  int rc = tk_launch_gemm(a, MT, NT, mblocks, st);
+  if (rc) return fail(TK_ELAUNCH, "gemm: launch failed (%s)", hipGetErrorString(hipGetLastError()));
+  return TK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tk_version(void) { return 1; }
+const char* tk_last_error(void) { return g_err; }
+int tk_device_cus(void) { return device_cus(); }
+
+size_t tk_workspace_bytes(void) { return TK_WS_TOTAL_BYTES; }
+
+int tk_workspace_init(void* ws, size_t ws_bytes, void* stream) {
+  if (!ws || ws_bytes < kCounterBytes) return fail(TK_EWORKSPACE, "workspace_init: need >= %zu bytes", kCounterBytes);
+  if (tk_launch_fill_zero((int*)ws, kMaxCounters, (hipStream_t)stream))
+    return fail(TK_ELAUNCH, "workspace_init: launch failed");
+  return TK_OK;
+}
+
+size_t tk_fp8w_packed_bytes(int N, int K) {
+  if (N <= 0 || K <= 0) return 0;
+  return (size_t)((N + 31) / 32) * ((K + 31) / 32) * 1024;
+}
+
+int tk_pack_fp8_weight(const void* w8, void* packed, int N, int K, void* stream) {
+  if (!w8 || !packed || N <= 0 || K <= 0) return fail(TK_EINVAL, "pack: bad argument");
+  if (K % 16) return fail(TK_EINVAL, "pack: K=%d must be a multiple of 16", K);
+  if (!aligned16(w8) || !aligned16(packed)) return fail(TK_EINVAL, "pack: pointers must be 16-byte aligned");
+  if (tk_launch_pack(w8, nullptr, packed, N, K, 0, (hipStream_t)stream)) return fail(TK_ELAUNCH, "pack: launch failed");
+  return TK_OK;
+}
+
+int tk_pack_fp8_gate_up(const void* wg8, const void* wu8, void* packed, int I, int K, void* stream) {
+  if (!wg8 || !wu8 || !packed || I <= 0 || K <= 0) return fail(TK_EINVAL, "pack_gate_up: bad argument");
+  if (K % 16 || I % 32) return fail(TK_EINVAL, "pack_gate_up: need K %% 16 == 0 and I %% 32 == 0 (K=%d I=%d)", K, I);
+  if (!aligned16(wg8) || !aligned16(wu8) || !aligned16(packed))
+    return fail(TK_EINVAL, "pack_gate_up: pointers must be 16-byte aligned");
+  if (tk_launch_pack(wg8, wu8, packed, I, K, 1, (hipStream_t)stream))
+    return fail(TK_ELAUNCH, "pack_gate_up: launch failed");
+  return TK_OK;
+}
+
+int tk_fp8w_gemm(const void* x, int ldx, const void* w_packed, const void* scale, void* y, int ldy, const void* resid,
+                 int ldr, int resid_dtype, int M, int N, int K, int split_k, void* ws, size_t ws_bytes, void* stream) {
+  return gemm_common(x, ldx, w_packed, (const float*)scale, nullptr, y, ldy, resid, ldr, resid_dtype, M, N, K, split_k,
+                     0, ws, ws_bytes, (hipStream_t)stream);
+}
+
+int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void* sg, const void* su,
+                      const void* wd_packed, const void* sd, void* y, int ldy, const void* resid, int ldr,
+                      int resid_dtype, int M, int K, int I, int act, void* ws, size_t ws_bytes, void* stream) {
+  if (act != TK_ACT_SILU && act != TK_ACT_GELU_TANH) return fail(TK_EINVAL, "ffn: unknown activation %d", act);
+  if (!sg || !su || !sd) return fail(TK_EINVAL, "ffn: null scale pointer");
+  if (I % 32) return fail(TK_EINVAL, "ffn: I=%d must be a multiple of 32", I);
+  if (!ws) return fail(TK_EWORKSPACE, "ffn: needs a workspace");
+  const size_t hbytes = (size_t)M * I * 2;
+  if (hbytes > kHiddenBytes || ws_bytes < kHiddenOff + hbytes)
+    return fail(TK_EWORKSPACE, "ffn: workspace too small for the [%d, %d] intermediate", M, I);
+  void* hbuf = (char*)ws + kHiddenOff;
+  // gate/up + activation-multiply -> h[M, I] (bf16, workspace)
+  int rc = gemm_common(x, ldx, wgu_packed, (const float*)sg, (const float*)su, hbuf, I, nullptr, 0, 0, M, I, K, 0, act,
+                       ws, ws_bytes, (hipStream_t)stream);
+  if (rc) return rc;
+  // down projection (+ residual)
+  return gemm_common(hbuf, I, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, M, K, I, 0, 0, ws,
+                     ws_bytes, (hipStream_t)stream);
+}
+
+int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* v_pre, int pre_sl, int pre_sh,
+                   int kv_dtype, const void* k_suf, const void* v_suf, int suf_sl, int suf_sh, const void* pad,
+                   void* out, int out_sm, int M, int P, int S, int H, int G, int D, int mask_mode, int logits_bf16,
+                   void* ws, size_t ws_bytes, void* stream) {
+  if (M <= 0 || P < 0 || S < 0 || P + S <= 0 || H <= 0 || G <= 0 || H % G)
+    return fail(TK_EINVAL, "attn: bad shape M=%d P=%d S=%d H=%d G=%d", M, P, S, H, G);
+  if (D != 64 && D != 128 && D != 256) return fail(TK_EINVAL, "attn: head_dim %d not in {64,128,256}", D);
+  if (kv_dtype != TK_BF16 && kv_dtype != TK_F32) return fail(TK_EINVAL, "attn: bad kv_dtype");
+  if (kv_dtype == TK_F32 && (S != 0 || D != 64))
+    return fail(TK_EINVAL, "attn: fp32 K/V is supported for prefix-only attention with head_dim 64");
+  if (mask_mode < 0 || mask_mode > 2) return fail(TK_EINVAL, "attn: bad mask_mode %d", mask_mode);
+  if (S > 0 && mask_mode == TK_MASK_NONE) return fail(TK_EINVAL, "attn: suffix keys need a suffix mask mode");
+  if (!q || !out || (P > 0 && (!k_pre || !v_pre)) || (S > 0 && (!k_suf || !v_suf)))
+    return fail(TK_EINVAL, "attn: null pointer");
+  if (q_sm % 8 || q_sh % 8 || pre_sl % 8 || pre_sh % 8 || (S > 0 && (suf_sl % 8 || suf_sh % 8)))
+    return fail(TK_EINVAL, "attn: strides must be multiples of 8 elements");
+  if (!aligned16(q) || !aligned16(k_pre) || !aligned16(v_pre) || !aligned16(k_suf) || !aligned16(v_suf))
+    return fail(TK_EINVAL, "attn: q/k/v must be 16-byte aligned");
+  if (out_sm < H * D) return fail(TK_EINVAL, "attn: out_sm=%d < H*D", out_sm);
+
+  AttnArgs a;
+  a.q = (const u16*)q;
+  a.q_sm = q_sm;
+  a.q_sh = q_sh;
+  a.k_pre = k_pre;
+  a.v_pre = v_pre;
+  a.pre_sl = pre_sl;
+  a.pre_sh = pre_sh;
+  a.k_suf = (const u16*)k_suf;
+  a.v_suf = (const u16*)v_suf;
+  a.suf_sl = suf_sl;
+  a.suf_sh = suf_sh;
+  a.pad = (const uint8_t*)pad;
+  a.out = (u16*)out;
+  a.out_sm = out_sm;
+  a.M = M;
+  a.P = P;
+  a.S = S;
+  a.H = H;
+  a.G = G;
+  a.mask_mode = mask_mode;
+  a.logits_bf16 = logits_bf16;
+  a.scale = 1.0f / sqrtf((float)D);
+
+  const int ntiles = (P + S + 31) / 32;
+  const int mtiles = (M + 31) / 32;
+  // one 32-key tile per wave and round: split the keys over blocks once a block would need
+  // more than two rounds
+  int splits = (ntiles + 7) / 8;
+  if (splits < 1) splits = 1;
+  if (splits > 8) splits = 8;
+  a.kv_splits = splits;
+  a.partial = nullptr;
+  a.counters = nullptr;
+  if (splits > 1) {
+    const int blocks = H * mtiles;
+    const size_t need = (size_t)blocks * splits * (64 + (size_t)(D / 32) * 1024) * 4;
+    if (!ws || blocks > kMaxCounters || need > kPartialBytes || ws_bytes < kPartialOff + need)
+      return fail(TK_EWORKSPACE, "attn: workspace too small (need %zu bytes)", need);
+    a.partial = (float*)((char*)ws + kPartialOff);
+    a.counters = (int*)ws;
+  }
+  if (tk_launch_attn(a, D, kv_dtype == TK_F32, (hipStream_t)stream))
+    return fail(TK_ELAUNCH, "attn: launch failed (%s)", hipGetErrorString(hipGetLastError()));
+  return TK_OK;
+}
+
+int tk_debug_decode_fp8(void* out_f32, void* stream) {
+  if (!out_f32) return fail(TK_EINVAL, "decode: null pointer");
+  if (tk_launch_decode_fp8((float*)out_f32, (hipStream_t)stream)) return fail(TK_ELAUNCH, "decode: launch failed");
+  return TK_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,63 @@
+// Shared device helpers for the gfx950 kernels (wave64, MFMA 32x32x16 bf16, OCP fp8).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16;
+
+#define TK_WAVE 64
+
+// Workspace layout (bytes): [counters][scratch ...]
+#define TK_WS_COUNTER_BYTES (64 * 1024)  // 16384 int32 arrival counters
+#define TK_WS_TOTAL_BYTES (64ull * 1024 * 1024)
+
+__device__ __forceinline__ float bf16_bits_to_f32(u16 b) { return __uint_as_float(((unsigned)b) << 16); }
+
+// fp32 -> bf16 bits, round-to-nearest-even (NaN kept quiet), same as torch's cast.
+__device__ __forceinline__ u16 f32_to_bf16_bits(float f) {
+  unsigned u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (u16)(u >> 16);
+}
+__device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+// 4 e4m3fn bytes (one dword) -> 4 bf16 (exact: every e4m3 value is a bf16 value).
+__device__ __forceinline__ void fp8x4_to_bf16x4(int v, bf16x2& lo, bf16x2& hi) {
+  lo = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v, 1.0f, false);
+  hi = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v, 1.0f, true);
+}
+
+// 8 e4m3fn bytes (two dwords) -> one MFMA operand of 8 bf16.
+__device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(int a, int b) {
+  bf16x2 p0, p1, p2, p3;
+  fp8x4_to_bf16x4(a, p0, p1);
+  fp8x4_to_bf16x4(b, p2, p3);
+  bf16x8 r;
+  r[0] = p0[0]; r[1] = p0[1]; r[2] = p1[0]; r[3] = p1[1];
+  r[4] = p2[0]; r[5] = p2[1]; r[6] = p3[0]; r[7] = p3[1];
+  return r;
+}
+
+__device__ __forceinline__ bf16x8 as_bf16x8(i32x4 v) {
+  union { i32x4 i; bf16x8 b; } u;
+  u.i = v;
+  return u.b;
+}
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float gelu_tanh_f(float x) {
+  const float c0 = 0.7978845608028654f;  // sqrt(2/pi)
+  float inner = c0 * (x + 0.044715f * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+// C layout of v_mfma_f32_32x32x16: lane l, register i holds
+//   column = l % 32, row = 8*(i/4) + 4*(l/32) + (i%4).
+__device__ __forceinline__ int mfma32_row(int lane, int i) { return 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3); }

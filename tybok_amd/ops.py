@@ -1,0 +1,241 @@
+"""Tensor-level wrappers over the C ABI: torch supplies device memory and the stream, nothing else.
+
+Every function enqueues on ``torch.cuda.current_stream()`` and is legal under graph capture as
+long as the output / workspace tensors were allocated before the capture (or come from the
+capture's private pool).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import native
+
+ACT = {"silu": 0, "gelu_tanh": 1}
+MASK_NONE, MASK_BIDIR, MASK_CAUSAL = 0, 1, 2
+_BF16, _F32 = 0, 1
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+class Workspace:
+    """Caller-owned scratch of the library (split-K partials, FFN intermediate, counters).
+
+    One per stream that may run kernels concurrently.  Created before graph capture.
+    """
+
+    def __init__(self, device: torch.device | str = "cuda"):
+        lib = native.lib()
+        self.nbytes = int(lib.tk_workspace_bytes())
+        self.buf = torch.empty(self.nbytes, dtype=torch.uint8, device=device)
+        native.check(lib.tk_workspace_init(self.buf.data_ptr(), self.nbytes, _stream()), "tk_workspace_init")
+
+    @property
+    def ptr(self) -> int:
+        return self.buf.data_ptr()
+
+
+_default_ws: dict[int, Workspace] = {}
+
+
+def default_workspace(device: torch.device | str | None = None) -> Workspace:
+    dev = torch.device(device if device is not None else "cuda")
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    ws = _default_ws.get(idx)
+    if ws is None:
+        ws = Workspace(torch.device("cuda", idx))
+        _default_ws[idx] = ws
+    return ws
+
+
+@dataclass
+class PackedWeight:
+    """An fp8 e4m3fn ``[N, K]`` weight in the library's tile order plus its fp32 row scales."""
+
+    data: torch.Tensor  # uint8, packed tiles
+    scale: torch.Tensor  # fp32 [N]
+    n: int
+    k: int
+
+
+@dataclass
+class PackedGateUp:
+    """Gate and up weights (``[I, K]`` each) with interleaved 32-row tiles."""
+
+    data: torch.Tensor
+    scale_gate: torch.Tensor
+    scale_up: torch.Tensor
+    i: int
+    k: int
+
+
+def _as_fp8_bytes(w8: torch.Tensor) -> torch.Tensor:
+    if w8.dtype == torch.float8_e4m3fn:
+        w8 = w8.view(torch.uint8)
+    if w8.dtype != torch.uint8:
+        raise TypeError(f"expected float8_e4m3fn or uint8 codes, got {w8.dtype}")
+    if not w8.is_cuda:
+        raise ValueError("weight must be on the GPU")
+    return w8.contiguous()
+
+
+def pack_fp8_weight(w8: torch.Tensor, scale: torch.Tensor) -> PackedWeight:
+    """Row-major e4m3fn ``[N, K]`` (+ fp32 ``[N]`` scale) -> :class:`PackedWeight` (once per model)."""
+    lib = native.lib()
+    codes = _as_fp8_bytes(w8)
+    n, k = codes.shape
+    out = torch.empty(int(lib.tk_fp8w_packed_bytes(n, k)), dtype=torch.uint8, device=codes.device)
+    native.check(lib.tk_pack_fp8_weight(codes.data_ptr(), out.data_ptr(), n, k, _stream()), "tk_pack_fp8_weight")
+    return PackedWeight(out, scale.to(device=codes.device, dtype=torch.float32).contiguous(), n, k)
+
+
+def pack_fp8_gate_up(wg8: torch.Tensor, sg: torch.Tensor, wu8: torch.Tensor, su: torch.Tensor) -> PackedGateUp:
+    lib = native.lib()
+    cg, cu = _as_fp8_bytes(wg8), _as_fp8_bytes(wu8)
+    if cg.shape != cu.shape:
+        raise ValueError("gate and up weights must have the same shape")
+    i, k = cg.shape
+    out = torch.empty(int(lib.tk_fp8w_packed_bytes(2 * i, k)), dtype=torch.uint8, device=cg.device)
+    native.check(
+        lib.tk_pack_fp8_gate_up(cg.data_ptr(), cu.data_ptr(), out.data_ptr(), i, k, _stream()), "tk_pack_fp8_gate_up"
+    )
+    f32 = dict(device=cg.device, dtype=torch.float32)
+    return PackedGateUp(out, sg.to(**f32).contiguous(), su.to(**f32).contiguous(), i, k)
+
+
+def _check_act(x: torch.Tensor, k: int) -> tuple[int, int]:
+    if x.dtype != torch.bfloat16 or not x.is_cuda:
+        raise TypeError("activations must be bf16 CUDA tensors")
+    if x.dim() != 2 or x.shape[1] != k or x.stride(1) != 1:
+        raise ValueError(f"activations must be [M, {k}] with unit inner stride, got {tuple(x.shape)}")
+    return x.shape[0], x.stride(0)
+
+
+def _resid_args(resid: torch.Tensor | None, m: int, n: int) -> tuple[int | None, int, int]:
+    if resid is None:
+        return None, 0, 0
+    if resid.shape != (m, n) or resid.stride(1) != 1:
+        raise ValueError("residual must be [M, N] with unit inner stride")
+    if resid.dtype == torch.bfloat16:
+        return resid.data_ptr(), resid.stride(0), _BF16
+    if resid.dtype == torch.float32:
+        return resid.data_ptr(), resid.stride(0), _F32
+    raise TypeError("residual must be bf16 or fp32")
+
+
+def fp8w_gemm(
+    x: torch.Tensor,
+    w: PackedWeight,
+    *,
+    resid: torch.Tensor | None = None,
+    out: torch.Tensor | None = None,
+    split_k: int = 0,
+    ws: Workspace | None = None,
+) -> torch.Tensor:
+    """``bf16((x @ W8^T) * scale)`` (+ residual) for ``x [M, K]`` bf16."""
+    lib = native.lib()
+    m, ldx = _check_act(x, w.k)
+    if out is None:
+        out = torch.empty(m, w.n, dtype=torch.bfloat16, device=x.device)
+    rp, ldr, rdt = _resid_args(resid, m, w.n)
+    ws = ws or default_workspace(x.device)
+    rc = lib.tk_fp8w_gemm(
+        x.data_ptr(), ldx, w.data.data_ptr(), w.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt,
+        m, w.n, w.k, split_k, ws.ptr, ws.nbytes, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_fp8w_gemm")
+    return out
+
+
+def fp8w_gated_ffn(
+    x: torch.Tensor,
+    wgu: PackedGateUp,
+    wd: PackedWeight,
+    act: str = "silu",
+    *,
+    resid: torch.Tensor | None = None,
+    out: torch.Tensor | None = None,
+    ws: Workspace | None = None,
+) -> torch.Tensor:
+    """``down(act(gate(x)) * up(x))`` (+ residual) for ``x [M, K]`` bf16."""
+    lib = native.lib()
+    m, ldx = _check_act(x, wgu.k)
+    if wd.k != wgu.i or wd.n != wgu.k:
+        raise ValueError("down weight must be [K, I]")
+    if out is None:
+        out = torch.empty(m, wd.n, dtype=torch.bfloat16, device=x.device)
+    rp, ldr, rdt = _resid_args(resid, m, wd.n)
+    ws = ws or default_workspace(x.device)
+    rc = lib.tk_fp8w_gated_ffn(
+        x.data_ptr(), ldx, wgu.data.data_ptr(), wgu.scale_gate.data_ptr(), wgu.scale_up.data_ptr(),
+        wd.data.data_ptr(), wd.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt,
+        m, wgu.k, wgu.i, ACT[act], ws.ptr, ws.nbytes, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_fp8w_gated_ffn")
+    return out
+
+
+def expert_attn(
+    q: torch.Tensor,
+    k_pre: torch.Tensor,
+    v_pre: torch.Tensor,
+    k_suf: torch.Tensor | None,
+    v_suf: torch.Tensor | None,
+    prefix_pad: torch.Tensor | None,
+    mask_mode: int,
+    *,
+    logits_bf16: bool = False,
+    out: torch.Tensor | None = None,
+    ws: Workspace | None = None,
+) -> torch.Tensor:
+    """Attention of ``q [M, H, D]`` over ``[k_pre; k_suf]`` (``[P|S, G, D]`` views, any strides with
+    a contiguous head dim).  ``prefix_pad``: uint8/bool ``[P]`` or None.  Returns bf16 ``[M, H*D]``."""
+    lib = native.lib()
+    if q.dtype != torch.bfloat16 or q.dim() != 3 or q.stride(2) != 1:
+        raise TypeError("q must be bf16 [M, H, D] with a contiguous head dim")
+    m, h, d = q.shape
+    p, g = k_pre.shape[0], k_pre.shape[1]
+    if k_pre.dtype != v_pre.dtype or k_pre.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("prefix K/V must both be bf16 or both fp32")
+    if k_pre.stride() != v_pre.stride() or k_pre.stride(2) != 1:
+        raise ValueError("prefix K and V must share strides and have a contiguous head dim")
+    s = 0
+    suf_sl = suf_sh = 0
+    if k_suf is not None:
+        assert v_suf is not None
+        if k_suf.dtype != torch.bfloat16 or v_suf.dtype != torch.bfloat16:
+            raise TypeError("suffix K/V must be bf16")
+        if k_suf.stride() != v_suf.stride() or k_suf.stride(2) != 1:
+            raise ValueError("suffix K and V must share strides and have a contiguous head dim")
+        s = k_suf.shape[0]
+        suf_sl, suf_sh = k_suf.stride(0), k_suf.stride(1)
+    pad = None
+    if prefix_pad is not None:
+        pad = prefix_pad.view(torch.uint8) if prefix_pad.dtype == torch.bool else prefix_pad
+        if pad.dtype != torch.uint8 or pad.numel() != p or not pad.is_contiguous():
+            raise ValueError("prefix_pad must be a contiguous uint8/bool [P]")
+    if out is None:
+        out = torch.empty(m, h * d, dtype=torch.bfloat16, device=q.device)
+    ws = ws or default_workspace(q.device)
+    rc = lib.tk_expert_attn(
+        q.data_ptr(), q.stride(0), q.stride(1), k_pre.data_ptr(), v_pre.data_ptr(), k_pre.stride(0), k_pre.stride(1),
+        _F32 if k_pre.dtype == torch.float32 else _BF16, _ptr(k_suf), _ptr(v_suf), suf_sl, suf_sh, _ptr(pad),
+        out.data_ptr(), out.stride(0), m, p, s, h, g, d, mask_mode, int(logits_bf16), ws.ptr, ws.nbytes, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_expert_attn")
+    return out
+
+
+def decode_fp8_table(device: torch.device | str = "cuda") -> torch.Tensor:
+    """Values of all 256 e4m3fn codes as the device's conversion instruction decodes them."""
+    out = torch.empty(256, dtype=torch.float32, device=device)
+    native.check(native.lib().tk_debug_decode_fp8(out.data_ptr(), _stream()), "tk_debug_decode_fp8")
+    return out
