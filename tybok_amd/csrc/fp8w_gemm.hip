@@ -5,9 +5,14 @@
 //     tile with ONE coalesced 1 KiB global_load_dwordx4 straight into operand registers.
 //   * e4m3 -> bf16 is exact and done in registers (v_cvt_scalef32_pk_bf16_fp8, scale 1.0), the
 //     product runs on v_mfma_f32_32x32x16_bf16 with fp32 accumulation.
-//   * x (bf16, tiny, L2 resident) is read directly in A-operand order: 32 contiguous bytes/lane.
-//   * A block owns NT n-tiles x MT m-tiles and a contiguous range of k-tiles; its NW waves take
-//     k-tiles round-robin, so concurrently issued loads of a block are contiguous in memory.
+//   * A block owns NT n-tiles x MT m-tiles and a contiguous range of k-tiles; per round its NW
+//     waves take NW*TPW consecutive k-tiles (TPW each).  The activations of a round
+//     (MT*32 rows x NW*TPW*32 columns, bf16) are staged ONCE per block through LDS with fully
+//     coalesced 16-byte loads (whole 128-byte lines per row) and read back in A-operand order:
+//     reading them per lane from global memory costs one cache-line lookup per row and
+//     instruction and caps a CU at a fraction of its L1 fill rate.
+//   * Columns past the block's K range (K tail, next split) are zeroed in LDS, so the weight
+//     loads need no masking: a zero activation column cancels whatever tile was read.
 //   * Reductions are fixed-order: waves through LDS (w = 0..NW-1), K splits through an fp32
 //     partial buffer summed by the last-arriving block in split order (no float atomics).
 #include "tk_common.h"
@@ -15,17 +20,32 @@
 
 namespace {
 
-template <int MT, int NT>
-struct Frag {
-  i32x4 w[NT];
-  i32x4 xa[MT][2];
-};
+// LDS-only barrier: waits for this wave's LDS traffic, not for the global prefetch queue
+// (a full __syncthreads() would drain vmcnt and serialise the weight stream every round).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
-template <int MT, int NT, int NW, bool GATED, int PF>
+template <int MT, int NT, int NW, bool GATED, int PF, int TPW>
 __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   constexpr int TILES = MT * NT;
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  constexpr int RKT = NW * TPW;               // k tiles per block round
+  constexpr int ROWB = RKT * 64;              // bytes of one activation row per round
+  constexpr int PITCH = ROWB + 16;            // LDS row pitch (bytes), keeps 16-byte alignment
+  constexpr int ROWS = MT * 32;
+  constexpr int XBUF = ROWS * PITCH;          // bytes per staging buffer
+  constexpr int PPR = ROWB / 16;              // 16-byte pieces per row
+  constexpr int XPT = ROWS * PPR / (NW * 64); // pieces per thread and round
+  constexpr int RED_BYTES = 2 * NW * 16 * 64 * 4;
+  constexpr int LDS_BYTES = 2 * XBUF > RED_BYTES ? 2 * XBUF : RED_BYTES;
+  static_assert(ROWS * PPR % (NW * 64) == 0, "staging pieces must divide evenly");
+  __shared__ __align__(16) unsigned char lds[LDS_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
   const int strip = blockIdx.x;
   const int split = blockIdx.y;
   const int mblock = blockIdx.z;
@@ -34,24 +54,51 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 
   const int kt_lo = (int)(((long long)split * a.KT) / a.ksplit);
   const int kt_hi = (int)(((long long)(split + 1) * a.KT) / a.ksplit);
+  const int nrounds = (kt_hi - kt_lo + RKT - 1) / RKT;
+  const int k_end = kt_hi * 32 < a.K ? kt_hi * 32 : a.K;  // first activation column this block must not use
 
-  // weight tile streams of this wave
+  // weight tile streams of this wave; a strip may hang over the last n tile: clamp to a valid
+  // tile (its results are never stored) so every load is unconditional.
   const uint8_t* wbase[NT];
-  bool nt_ok[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     int ntg = strip * NT + nt;
-    nt_ok[nt] = ntg < a.ntiles;
+    if (ntg > a.ntiles - 1) ntg = a.ntiles - 1;
     wbase[nt] = a.w + ((size_t)ntg * a.KT) * 1024 + lane * 16;
   }
-  // activation rows of this lane
-  const u16* xrow[MT];
-  bool m_ok[MT];
+
+  // staging pieces of this thread: piece p -> (row p / PPR, 16-byte column p % PPR).  Rows >= M
+  // are clamped to M-1 (an output row depends only on its own activation row; rows >= M are
+  // never stored).
+  const u16* xsrc[XPT];
+  int xcol[XPT];   // first element (k index) of the piece within a round
+  int xdst[XPT];   // LDS byte offset within a staging buffer
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    int m = (mblock * MT + mt) * 32 + l32;
-    m_ok[mt] = m < a.M;
-    xrow[mt] = a.x + (size_t)m * a.ldx + 16 * half;
+  for (int i = 0; i < XPT; ++i) {
+    const int p = tid + i * NW * 64;
+    const int r = p / PPR, c = p % PPR;
+    int m = mblock * ROWS + r;
+    if (m > a.M - 1) m = a.M - 1;
+    xsrc[i] = a.x + (size_t)m * a.ldx;
+    xcol[i] = c * 8;
+    xdst[i] = r * PITCH + c * 16;
+  }
+
+  // scales of the columns this wave will finish, fetched before the loop so the epilogue does not
+  // start with a cold miss
+  float sc_pre[2] = {0.f, 0.f};
+  {
+    const int n0 = GATED ? (strip * NT / 2) * 32 + l32 : strip * NT * 32 + l32;
+    if (!GATED) {
+#pragma unroll
+      for (int nt = 0; nt < (NT < 2 ? NT : 2); ++nt) {
+        const int n = n0 + nt * 32;
+        sc_pre[nt] = n < a.N ? a.s0[n] : 0.f;
+      }
+    } else {
+      sc_pre[0] = n0 < a.N ? a.s0[n0] : 0.f;
+      sc_pre[1] = n0 < a.N ? a.s1[n0] : 0.f;
+    }
   }
 
   f32x16 acc[MT][NT];
@@ -62,62 +109,113 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
 
-  auto load = [&](Frag<MT, NT>& f, int kt) {
+  struct WFrag {
+    i32x4 w[TPW][NT];
+  };
+  auto wload = [&](WFrag& f, int r) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      i32x4 v = {0, 0, 0, 0};
-      if (nt_ok[nt]) v = *(const i32x4*)(wbase[nt] + (size_t)kt * 1024);
-      f.w[nt] = v;
-    }
-    const bool k_ok = (kt * 32 + 16 * half) < a.K;
+    for (int j = 0; j < TPW; ++j) {
+      int kt = kt_lo + r * RKT + wave * TPW + j;
+      if (kt > a.KT - 1) kt = a.KT - 1;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      i32x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
-      if (m_ok[mt] && k_ok) {
-        const i32x4* p = (const i32x4*)(xrow[mt] + kt * 32);
-        v0 = p[0];
-        v1 = p[1];
-      }
-      f.xa[mt][0] = v0;
-      f.xa[mt][1] = v1;
+      for (int nt = 0; nt < NT; ++nt) f.w[j][nt] = *(const i32x4*)(wbase[nt] + (size_t)kt * 1024);
     }
   };
-  auto compute = [&](const Frag<MT, NT>& f) {
-    bf16x8 wb[NT][2];
+  struct XFrag {
+    i32x4 v[XPT];
+  };
+  auto xload = [&](XFrag& f, int r) {
+    const int k0 = (kt_lo + r * RKT) * 32;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      wb[nt][0] = fp8x8_to_bf16x8(f.w[nt][0], f.w[nt][1]);
-      wb[nt][1] = fp8x8_to_bf16x8(f.w[nt][2], f.w[nt][3]);
+    for (int i = 0; i < XPT; ++i) {
+      int k = k0 + xcol[i];
+      if (k > a.K - 8) k = a.K - 8;  // keep the address inside the row; the value is dropped below
+      f.v[i] = *(const i32x4*)(xsrc[i] + k);
     }
+  };
+  auto xstore = [&](const XFrag& f, int r, int b) {
+    const int k0 = (kt_lo + r * RKT) * 32;
+    const i32x4 z = {0, 0, 0, 0};
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int i = 0; i < XPT; ++i) {
+      const bool ok = (k0 + xcol[i]) < k_end;
+      *(i32x4*)(lds + b * XBUF + xdst[i]) = ok ? f.v[i] : z;
+    }
+  };
+  auto compute = [&](const WFrag& f, int b) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+    for (int j = 0; j < TPW; ++j) {
+      i32x4 xa[MT][2];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(f.xa[mt][j]), wb[nt][j], acc[mt][nt], 0, 0, 0);
+      for (int mt = 0; mt < MT; ++mt) {
+        const i32x4* p = (const i32x4*)(lds + b * XBUF + (mt * 32 + l32) * PITCH + ((wave * TPW + j) * 32 + 16 * half) * 2);
+        xa[mt][0] = p[0];
+        xa[mt][1] = p[1];
+      }
+      bf16x8 wb[NT][2];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        wb[nt][0] = fp8x8_to_bf16x8(f.w[j][nt][0], f.w[j][nt][1]);
+        wb[nt][1] = fp8x8_to_bf16x8(f.w[j][nt][2], f.w[j][nt][3]);
+      }
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(xa[mt][h2]), wb[nt][h2], acc[mt][nt], 0, 0, 0);
+    }
   };
 
-  // software pipeline: PF k-tiles of this wave in flight
-  Frag<MT, NT> buf[PF];
-  const int kt0 = kt_lo + wave;
-#pragma unroll
-  for (int p = 0; p < PF; ++p)
-    if (kt0 + p * NW < kt_hi) load(buf[p], kt0 + p * NW);
-  for (int kt = kt0; kt < kt_hi; kt += NW * PF) {
+  // Software pipeline over block rounds: PF rounds in flight.  A round's activations and weights
+  // are requested together (memory returns in order, so waiting for one means waiting for
+  // everything requested before it).  The steady-state loop runs while a whole group of PF rounds
+  // can prefetch and has no branch, so the compiler keeps precise vmcnt waits; the tail (at most
+  // 2*PF-1 rounds) uses block-uniform conditions and requests nothing that is not consumed (a
+  // redundant request would have to be waited for at the first barrier after the loop).
+  if (nrounds > 0) {
+    WFrag wbuf[PF];
+    XFrag xbuf[PF];
 #pragma unroll
     for (int p = 0; p < PF; ++p) {
-      const int k = kt + p * NW;
-      if (k < kt_hi) {
-        compute(buf[p]);
-        const int kn = k + PF * NW;
-        if (kn < kt_hi) load(buf[p], kn);
+      if (p < nrounds) {
+        xload(xbuf[p], p);
+        wload(wbuf[p], p);
+      }
+    }
+    int it = 0;
+    for (; it + 2 * PF <= nrounds; it += PF) {
+#pragma unroll
+      for (int p = 0; p < PF; ++p) {
+        const int r = it + p;
+        xstore(xbuf[p], r, r & 1);
+        lds_barrier();
+        compute(wbuf[p], r & 1);
+        xload(xbuf[p], r + PF);
+        wload(wbuf[p], r + PF);
+        __builtin_amdgcn_sched_barrier(0);  // keep the refill right behind its stage's MFMAs
+      }
+    }
+    const int rem = nrounds - it;  // in [0, 2*PF)
+#pragma unroll
+    for (int q = 0; q < 2 * PF - 1; ++q) {
+      if (q < rem) {  // block-uniform
+        const int r = it + q;
+        xstore(xbuf[q % PF], r, r & 1);
+        lds_barrier();
+        compute(wbuf[q % PF], r & 1);
+        if (q + PF < rem) {
+          xload(xbuf[q % PF], r + PF);
+          wload(wbuf[q % PF], r + PF);
+        }
       }
     }
   }
+  __syncthreads();  // staging buffers are dead; the reduction reuses the LDS
 
   // ---- in-block reduction over waves (fixed order), tile by tile, double-buffered LDS ----
-  __shared__ float red[2][NW][16][64];
+  float (*red)[NW][16][64] = (float (*)[NW][16][64])lds;
   constexpr int OWN = GATED ? 2 * ((TILES / 2 + NW - 1) / NW) : (TILES + NW - 1) / NW;
   float own[OWN][16];
 #pragma unroll
@@ -159,19 +257,20 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       if (wave == owner) {
         float* dst = a.partial + (((size_t)blk_lin * a.ksplit + split) * TILES + t) * 1024 + lane;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i * 64] = own[slot][i];
+        for (int i = 0; i < 16; ++i) st_agent(dst + i * 64, own[slot][i]);
       }
     }
+    // The partials were written through to device-coherent memory (agent-scope stores), so no
+    // cache flush is needed: wait until they are acknowledged, then count this block in.
     __shared__ int s_last;
-    __threadfence();
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (threadIdx.x == 0) {
-      int old = atomicAdd(a.counters + blk_lin, 1);
+      int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       s_last = (old == a.ksplit - 1);
     }
     __syncthreads();
     if (!s_last) return;
-    __threadfence();
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
       const int owner = GATED ? (t / 2) % NW : t % NW;
@@ -182,11 +281,12 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
         for (int s = 0; s < a.ksplit; ++s) {
           const float* src = a.partial + (((size_t)blk_lin * a.ksplit + s) * TILES + t) * 1024 + lane;
 #pragma unroll
-          for (int i = 0; i < 16; ++i) own[slot][i] += __builtin_nontemporal_load(src + i * 64);
+          for (int i = 0; i < 16; ++i) own[slot][i] += ld_agent(src + i * 64);
         }
       }
     }
-    if (threadIdx.x == 0) a.counters[blk_lin] = 0;  // leave the counter ready for the next launch
+    if (threadIdx.x == 0)  // leave the counter ready for the next launch
+      __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
   // ---- epilogue ----
@@ -198,7 +298,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       const int slot = t / NW;
       const int n = (strip * NT + nt) * 32 + l32;
       if (n >= a.N) continue;
-      const float sc = a.s0[n];
+      const float sc = nt < 2 ? sc_pre[nt < 2 ? nt : 0] : a.s0[n];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int m = (mblock * MT + mt) * 32 + mfma32_row(lane, i);
@@ -223,7 +323,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       const int sg = (u / NW) * 2, su = sg + 1;
       const int col = ((strip * NT + nt) / 2) * 32 + l32;  // logical column in [0, I)
       if (col >= a.N) continue;
-      const float scg = a.s0[col], scu = a.s1[col];
+      const float scg = nt == 0 ? sc_pre[0] : a.s0[col], scu = nt == 0 ? sc_pre[1] : a.s1[col];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int m = (mblock * MT + mt) * 32 + mfma32_row(lane, i);
@@ -277,7 +377,7 @@ __global__ void decode_fp8_kernel(float* out) {
 
 template <int MT, int NT, int NW, bool GATED, int PF>
 int launch(const GemmArgs& a, dim3 grid, hipStream_t st) {
-  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, NW, GATED, PF>), grid, dim3(NW * 64), 0, st, a);
+  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, NW, GATED, PF, 1>), grid, dim3(NW * 64), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -58,6 +58,15 @@ __device__ __forceinline__ float gelu_tanh_f(float x) {
   return 0.5f * x * (1.0f + tanhf(inner));
 }
 
+// Device-coherent (agent-scope, cache write-through / cache-bypassing) accesses used for data that
+// one block hands to another inside a kernel: with them the hand-off needs no L2 flush.
+__device__ __forceinline__ void st_agent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_agent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // C layout of v_mfma_f32_32x32x16: lane l, register i holds
 //   column = l % 32, row = 8*(i/4) + 4*(l/32) + (i%4).
 __device__ __forceinline__ int mfma32_row(int lane, int i) { return 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3); }

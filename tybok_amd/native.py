@@ -11,7 +11,10 @@ import ctypes
 import os
 from ctypes import c_char_p, c_int, c_size_t, c_void_p
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libtybok_hip.so")
+# TYBOK_HIP_LIB points at an alternative build of the same ABI (kernel experiments); default in-tree.
+_LIB_PATH = os.environ.get("TYBOK_HIP_LIB") or os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "_lib", "libtybok_hip.so"
+)
 _lib: ctypes.CDLL | None = None
 
 # name -> (restype, argtypes); mirrors include/tybok_hip.h one to one
