@@ -1,0 +1,89 @@
+"""Seeded cases shared by the golden-vector writer and the tests (weights and inputs are
+regenerated from seeds; only the reference's outputs are stored as fixtures)."""
+
+from __future__ import annotations
+
+import torch
+
+SMOLVLA_CASES = {
+    # reduced depth: 4 VLM/expert layers (self, cross, self, cross), 2 vision layers, 2 cameras,
+    # padded language tail, random noise, 3 Euler steps
+    "small": dict(num_vlm_layers=4, vision_layers=2, cameras=2, num_steps=3, seed=11, noise="randn", lang_pad=8),
+    # full depth (config 4 of the benchmark): 16 + 16 layers, 12 vision layers, 3 cameras, 10 steps, zero noise
+    "full": dict(num_vlm_layers=16, vision_layers=12, cameras=3, num_steps=10, seed=0, noise="zeros", lang_pad=0),
+}
+
+PI05_CASES = {
+    # reduced depth: 3 VLM/expert layers, 2 vision layers, 2 cameras, padded language tail, 3 steps
+    "small": dict(depth=3, vision_layers=2, cameras=2, num_steps=3, seed=12, noise="randn", lang_pad=60),
+}
+
+
+def smolvla_build(case: dict):
+    from tybok_amd.policies.smolvla.config import SmolVLAConfig, TextConfig, VisionConfig, VLMConfig
+    from tybok_amd.policies.smolvla.weights import random_state_dict
+
+    cfg = SmolVLAConfig(
+        num_vlm_layers=case["num_vlm_layers"],
+        num_steps=case["num_steps"],
+        vlm_config=VLMConfig(text_config=TextConfig(), vision_config=VisionConfig(num_hidden_layers=case["vision_layers"])),
+        image_features=[f"observation.images.camera{i + 1}" for i in range(case["cameras"])],
+    )
+    sd = random_state_dict(cfg, seed=case["seed"])
+    return cfg, sd, smolvla_inputs(cfg, case)
+
+
+def smolvla_inputs(cfg, case: dict) -> dict:
+    g = torch.Generator().manual_seed(case["seed"] + 1000)
+    w, h = cfg.resize_imgs_with_padding
+    n = case["cameras"]
+    images = [torch.randint(0, 256, (1, 3, h, w), generator=g, dtype=torch.uint8).float() / 255.0 for _ in range(n)]
+    tokens = torch.randint(0, cfg.vlm_config.text_config.vocab_size, (1, cfg.tokenizer_max_length), generator=g)
+    lang_masks = torch.ones(1, cfg.tokenizer_max_length, dtype=torch.bool)
+    if case["lang_pad"]:
+        lang_masks[:, -case["lang_pad"] :] = False
+    state = torch.zeros(1, cfg.max_state_dim)
+    state[:, :6] = torch.randn(1, 6, generator=g)
+    if case["noise"] == "zeros":
+        noise = torch.zeros(1, cfg.chunk_size, cfg.max_action_dim)
+    else:
+        noise = torch.randn(1, cfg.chunk_size, cfg.max_action_dim, generator=g)
+    return dict(
+        images=images,
+        img_masks=[torch.ones(1, dtype=torch.bool) for _ in range(n)],
+        lang_tokens=tokens,
+        lang_masks=lang_masks,
+        state=state,
+        noise=noise,
+    )
+
+
+def pi05_build(case: dict):
+    from tybok_amd.policies.pi05.config import PI05Config
+    from tybok_amd.policies.pi05.weights import random_state_dict
+
+    cfg = PI05Config.shaped(depth=case["depth"], vision_layers=case["vision_layers"], cameras=case["cameras"], num_steps=case["num_steps"])
+    sd = random_state_dict(cfg, seed=case["seed"])
+    return cfg, sd, pi05_inputs(cfg, case)
+
+
+def pi05_inputs(cfg, case: dict) -> dict:
+    g = torch.Generator().manual_seed(case["seed"] + 1000)
+    h, w = cfg.image_resolution
+    n = case["cameras"]
+    images = [torch.randint(0, 256, (1, 3, h, w), generator=g, dtype=torch.uint8).float() / 255.0 for _ in range(n)]
+    tokens = torch.randint(0, cfg.vocab_size, (1, cfg.tokenizer_max_length), generator=g)
+    lang_masks = torch.ones(1, cfg.tokenizer_max_length, dtype=torch.bool)
+    if case["lang_pad"]:
+        lang_masks[:, -case["lang_pad"] :] = False
+    if case["noise"] == "zeros":
+        noise = torch.zeros(1, cfg.chunk_size, cfg.max_action_dim)
+    else:
+        noise = torch.randn(1, cfg.chunk_size, cfg.max_action_dim, generator=g)
+    return dict(
+        images=images,
+        img_masks=[torch.ones(1, dtype=torch.bool) for _ in range(n)],
+        lang_tokens=tokens,
+        lang_masks=lang_masks,
+        noise=noise,
+    )

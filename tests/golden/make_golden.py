@@ -1,0 +1,162 @@
+"""Write golden vectors for the model-level wiring from the reference's own torch modules.
+
+Run ONCE in the build container (the reference is not available elsewhere):
+
+    python tests/golden/make_golden.py [smolvla|pi05|all]
+
+For each case the reference's eager model classes (``/root/reference/tybok/policies/<model>/models``)
+are constructed on the CPU from plain config dataclasses (no checkpoint, no tokenizer), loaded with
+the seeded random state dict of ``tybok_amd.policies.<model>.weights.random_state_dict`` and run on
+seeded inputs.  Only outputs are stored (``tests/golden/<case>.npz``): the final action chunk, the
+step-0 velocity, and a few slices of prefix embedding / prefix KV.  Inputs and weights are
+regenerated from the same seeds by ``tests/golden/cases.py``.
+"""
+
+from __future__ import annotations
+
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, HERE)
+
+import cases  # noqa: E402
+
+REFERENCE_ROOT = "/root/reference"
+
+
+def _import_reference():
+    if REFERENCE_ROOT not in sys.path:
+        sys.path.insert(0, REFERENCE_ROOT)
+
+
+def _load(module: torch.nn.Module, sd: dict) -> None:
+    missing = []
+    own = dict(module.named_parameters())
+    for name, p in own.items():
+        if name not in sd:
+            missing.append(name)
+            continue
+        assert tuple(p.shape) == tuple(sd[name].shape), (name, tuple(p.shape), tuple(sd[name].shape))
+        assert p.dtype == sd[name].dtype, (name, p.dtype, sd[name].dtype)
+        p.data.copy_(sd[name])
+    extra = sorted(set(sd) - set(own))
+    assert not missing, f"reference parameters without a value: {missing[:5]} (+{len(missing)})"
+    assert not extra, f"state dict entries the reference does not have: {extra[:5]} (+{len(extra)})"
+
+
+def smolvla_case(name: str) -> dict:
+    _import_reference()
+    from tybok.policies.smolvla import config as rcfg
+    from tybok.policies.smolvla.models.flow_matching import VLAFlowMatching, make_att_2d_masks
+
+    case = cases.SMOLVLA_CASES[name]
+    cfg, sd, inputs = cases.smolvla_build(case)
+    vis = cfg.vlm_config.vision_config
+    ref_cfg = rcfg.SmolVLAConfig(
+        num_vlm_layers=cfg.num_vlm_layers,
+        num_steps=cfg.num_steps,
+        vlm_config=rcfg.VLMConfig(
+            text_config=rcfg.TextConfig(), vision_config=rcfg.VisionConfig(num_hidden_layers=vis.num_hidden_layers)
+        ),
+    )
+    default = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)  # the engine builds the model under a bf16 default
+    try:
+        model = VLAFlowMatching(ref_cfg, tokenizer=None)
+    finally:
+        torch.set_default_dtype(default)
+    model.eval()
+    _load(model, sd)
+    images = [img * 2.0 - 1.0 for img in inputs["images"]]  # prepare_images at the model resolution
+    out: dict[str, np.ndarray] = {}
+    with torch.inference_mode():
+        embs, pads, att = model.embed_prefix(images, inputs["img_masks"], inputs["lang_tokens"], inputs["lang_masks"], state=inputs["state"])
+        out["prefix_embs_head"] = embs[0, :4].float().numpy()
+        out["prefix_embs_tail"] = embs[0, -50:, :64].float().numpy()
+        out["pad_masks"] = pads.numpy()
+        mask2d = make_att_2d_masks(pads, att)
+        pos = torch.cumsum(pads, dim=1) - 1
+        _, kv = model.vlm_with_expert.forward(
+            attention_mask=mask2d, position_ids=pos, past_key_values=None, inputs_embeds=[embs, None], use_cache=True, fill_kv_cache=True
+        )
+        last = cfg.num_vlm_layers - 1
+        out["k_first"] = kv[0]["key_states"][0, ::16].float().numpy()
+        out["v_last"] = kv[last]["value_states"][0, ::16].float().numpy()
+        x0 = torch.zeros(1, cfg.chunk_size, cfg.max_action_dim)
+        v_half = model.denoise_step(prefix_pad_masks=pads, past_key_values=kv, x_t=x0, timestep=torch.tensor([0.5], dtype=torch.float32))
+        out["v_t_half"] = v_half[0].float().numpy()
+        chunk = model.sample_actions(images, inputs["img_masks"], inputs["lang_tokens"], inputs["lang_masks"], inputs["state"], noise=inputs["noise"])
+        out["chunk"] = chunk[0].float().numpy()
+    return out
+
+
+def pi05_case(name: str) -> dict:
+    _import_reference()
+    from tybok.policies.pi05 import config as rcfg
+    from tybok.policies.pi05.models.flow_matching import PI05FlowMatching, make_att_2d_masks, prepare_attention_masks_4d
+
+    case = cases.PI05_CASES[name]
+    cfg, sd, inputs = cases.pi05_build(case)
+    rcfg.GEMMA_VARIANTS["golden_vlm"] = dict(cfg.paligemma_dims)
+    rcfg.GEMMA_VARIANTS["golden_expert"] = dict(cfg.expert_dims)
+    ref_cfg = rcfg.PI05Config(
+        paligemma_variant="golden_vlm", action_expert_variant="golden_expert", num_steps=cfg.num_steps,
+        tokenizer_max_length=cfg.tokenizer_max_length,
+    )  # fmt: skip
+    ref_cfg._image_features = list(cfg.image_features)
+    default = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        model = PI05FlowMatching(ref_cfg)
+    finally:
+        torch.set_default_dtype(default)
+    vt = model.paligemma_with_expert.paligemma.model.vision_tower.vision_model
+    vt.encoder.layers = vt.encoder.layers[: cfg.vision_layers]
+    model.eval()
+    _load(model, sd)
+    images = [img * 2.0 - 1.0 for img in inputs["images"]]
+    out: dict[str, np.ndarray] = {}
+    with torch.inference_mode():
+        embs, pads, att = model.embed_prefix(images, inputs["img_masks"], inputs["lang_tokens"], inputs["lang_masks"])
+        out["prefix_embs_head"] = embs[0, :4].float().numpy()
+        out["prefix_embs_tail"] = embs[0, -8:, :64].float().numpy()
+        mask4d = prepare_attention_masks_4d(make_att_2d_masks(pads, att))
+        pos = torch.cumsum(pads, dim=1) - 1
+        _, kv = model.paligemma_with_expert.forward(
+            attention_mask=mask4d, position_ids=pos, past_key_values=None, inputs_embeds=[embs, None], use_cache=True
+        )
+        out["k_first"] = kv[0][0][0, 0, ::32].float().numpy()
+        out["v_last"] = kv[-1][1][0, 0, ::32].float().numpy()
+        x0 = torch.zeros(1, cfg.chunk_size, cfg.max_action_dim)
+        v_half = model.denoise_step(prefix_pad_masks=pads, past_key_values=kv, x_t=x0, timestep=torch.tensor([0.5], dtype=torch.float32))
+        out["v_t_half"] = v_half[0].float().numpy()
+        chunk = model.sample_actions(images, inputs["img_masks"], inputs["lang_tokens"], inputs["lang_masks"], noise=inputs["noise"])
+        out["chunk"] = chunk[0].float().numpy()
+    return out
+
+
+def main() -> None:
+    which = sys.argv[1] if len(sys.argv) > 1 else "all"
+    torch.manual_seed(0)
+    jobs = []
+    if which in ("smolvla", "all"):
+        jobs += [("smolvla", n) for n in cases.SMOLVLA_CASES]
+    if which in ("pi05", "all"):
+        jobs += [("pi05", n) for n in cases.PI05_CASES]
+    for model, name in jobs:
+        t0 = time.time()
+        out = smolvla_case(name) if model == "smolvla" else pi05_case(name)
+        path = os.path.join(HERE, f"{model}_{name}.npz")
+        np.savez_compressed(path, **out)
+        print(f"{model}:{name}: wrote {path} ({os.path.getsize(path) / 1024:.0f} KiB) in {time.time() - t0:.1f}s", flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,59 @@
+"""Pins oracle/smolvla.py (model wiring) to golden vectors written from the reference's own torch
+modules (tests/golden/make_golden.py).  CPU only."""
+
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "golden"))
+
+import cases  # noqa: E402
+from oracle import smolvla as O  # noqa: E402
+
+
+def _shape(cfg) -> O.SmolVLAShape:
+    return O.SmolVLAShape(
+        num_vlm_layers=cfg.num_vlm_layers,
+        vis_layers=cfg.vlm_config.vision_config.num_hidden_layers,
+        num_steps=cfg.num_steps,
+    )
+
+
+def _run(name: str):
+    case = cases.SMOLVLA_CASES[name]
+    cfg, sd, inp = cases.smolvla_build(case)
+    shape = _shape(cfg)
+    w = O.Weights(sd)
+    trace: dict = {}
+    with torch.no_grad():
+        images = O.prepare_images(inp["images"])
+        chunk = O.sample_actions(w, shape, images, inp["img_masks"], inp["lang_tokens"], inp["lang_masks"], inp["state"], inp["noise"], trace=trace)
+        x0 = torch.zeros(1, shape.chunk, shape.max_action_dim)
+        v_half = O.denoise_step(w, shape, trace["pad_masks"], trace["kv"], trace["ekv"], x0, 0.5)
+    return cfg, chunk, v_half, trace
+
+
+def _maxdiff(a, b) -> float:
+    return float(np.abs(np.asarray(a, dtype=np.float64) - np.asarray(b, dtype=np.float64)).max())
+
+
+@pytest.mark.parametrize("name", ["small", "full"])
+def test_oracle_matches_reference_golden(name):
+    gold = np.load(os.path.join(HERE, "golden", f"smolvla_{name}.npz"))
+    cfg, chunk, v_half, trace = _run(name)
+    embs = trace["prefix_embs"]
+    assert _maxdiff(embs[0, :4].float().numpy(), gold["prefix_embs_head"]) == 0.0
+    assert _maxdiff(embs[0, -50:, :64].float().numpy(), gold["prefix_embs_tail"]) == 0.0
+    assert np.array_equal(trace["pad_masks"].numpy(), gold["pad_masks"])
+    last = cfg.num_vlm_layers - 1
+    assert _maxdiff(trace["kv"][0][0][0, ::16].float().numpy(), gold["k_first"]) == 0.0
+    assert _maxdiff(trace["kv"][last][1][0, ::16].float().numpy(), gold["v_last"]) <= 1e-6
+    # same torch ops in the same order on the same machine: the restatement reproduces the
+    # reference's chunk to fp32 round-off
+    assert _maxdiff(v_half[0].numpy(), gold["v_t_half"]) <= 1e-5
+    assert _maxdiff(chunk[0].numpy(), gold["chunk"]) <= 1e-5
+    assert float(np.abs(gold["chunk"]).max()) > 0.1  # the case is not degenerate
