@@ -88,11 +88,15 @@ int tk_pack_fp8_gate_up(const void* wg8_rowmajor, const void* wu8_rowmajor, void
  *          rounding of the product: y = bf16(float(bf16(acc*scale)) + float(resid)) -- the
  *          reference's in-place `out_emb += hidden_states`
  *          (tybok/policies/smolvla/models/vlm_with_expert.py:386-408).
+ *   gate:  NULL, or bf16 [N]: the product is multiplied by gate[n] (one more bf16 rounding)
+ *          before the residual is added: y = bf16(resid + bf16(bf16(acc*scale) * gate[n])) -- the
+ *          AdaRMS gated residual `x + y * gate` of pi0.5 (tybok/policies/pi05/models/layers.py:27-31,
+ *          tybok/policies/pi05/models/triton_expert_residual.py:26-60).
  *   split_k: 0 = pick automatically; otherwise the number of K splits (>= 1).
  */
 int tk_fp8w_gemm(const void* x, int ldx, const void* w_packed, const void* scale, void* y, int ldy,
-                 const void* resid, int ldr, int resid_dtype, int M, int N, int K, int split_k, void* ws,
-                 size_t ws_bytes, void* stream);
+                 const void* resid, int ldr, int resid_dtype, const void* gate, int M, int N, int K, int split_k,
+                 void* ws, size_t ws_bytes, void* stream);
 
 /* ---- fused gated FFN ----------------------------------------------------------------------- */
 /* y[M, K] = down( act(gate(x)) * up(x) ) with fp8 weights, bf16 in/out:
@@ -102,12 +106,12 @@ int tk_fp8w_gemm(const void* x, int ldx, const void* w_packed, const void* scale
  * tybok/policies/pi05/models/layers.py:87-95, tybok/policies/smolvla/models/triton_mlp.py:30-144,
  * tybok/policies/pi05/models/triton_expert_mlp_fp8.py:438-469).
  *   wgu_packed: tk_pack_fp8_gate_up output; wd_packed: tk_pack_fp8_weight of [K, I].
- *   resid/ldr/resid_dtype: as in tk_fp8w_gemm, applied to y.
+ *   resid/ldr/resid_dtype/gate: as in tk_fp8w_gemm, applied to y.
  * The [M, I] intermediate lives in the workspace (never returned). */
 int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void* sg, const void* su,
                       const void* wd_packed, const void* sd, void* y, int ldy, const void* resid, int ldr,
-                      int resid_dtype, int M, int K, int I, int act, void* ws, size_t ws_bytes,
-                      void* stream);
+                      int resid_dtype, const void* gate, int M, int K, int I, int act, void* ws,
+                      size_t ws_bytes, void* stream);
 
 /* ---- action-expert attention over the cached prefix ------------------------------------------ */
 /* out[M, H*D] (bf16) = softmax(q.K^T * D^-0.5 + mask) . V over keys [prefix(P); suffix(S)].

@@ -203,3 +203,21 @@ def test_attention_fully_masked_prefix_is_uniform(tk):
     want = oops.expert_attention(q, k_pre, v_pre, None, None, none, oops.MASK_NONE)
     got = tk.expert_attn(q.cuda(), k_pre.cuda(), v_pre.cuda(), None, None, none.cuda(), oops.MASK_NONE)
     _close(got, want, "attn fully masked")
+
+
+def test_gated_residual_epilogue(tk):
+    # pi0.5 AdaRMS gated residual: y = resid + bf16(ffn(x) * gate)
+    x, wg8, sg, wu8, su, wd8, sd = ffn_case(50, 1024, 4096, seed=3)
+    g = torch.Generator().manual_seed(4)
+    resid = torch.randn(50, 1024, generator=g).to(torch.bfloat16)
+    gate = torch.randn(1024, generator=g).to(torch.bfloat16)
+    want = resid + oops.gated_ffn(x, wg8, sg, wu8, su, wd8, sd, "gelu_tanh") * gate
+    wgu = tk.pack_fp8_gate_up(wg8.cuda(), sg, wu8.cuda(), su)
+    wd = tk.pack_fp8_weight(wd8.cuda(), sd)
+    got = tk.fp8w_gated_ffn(x.cuda(), wgu, wd, "gelu_tanh", resid=resid.cuda(), gate=gate.cuda())
+    _close(got, want, "ffn gated residual")
+    pw = tk.pack_fp8_weight(wd8.cuda(), sd)
+    h = torch.randn(50, 4096, generator=g).to(torch.bfloat16)
+    want = resid + oops.lin_fp8w(h, wd8, sd) * gate
+    got = tk.fp8w_gemm(h.cuda(), pw, resid=resid.cuda(), gate=gate.cuda())
+    _close(got, want, "gemm gated residual")

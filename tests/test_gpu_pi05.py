@@ -1,0 +1,106 @@
+"""pi0.5 backend on the GPU against the CPU oracle: model-level parity per tier, engine API,
+hipGraph replay == eager."""
+
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "golden"))
+
+import cases  # noqa: E402
+from oracle import pi05 as O  # noqa: E402
+from oracle.smolvla import Weights  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+def _shape(cfg) -> O.PI05Shape:
+    return O.PI05Shape(depth=cfg.paligemma_dims["depth"], vis_layers=cfg.vision_layers, num_steps=cfg.num_steps)
+
+
+def _oracle_chunk(cfg, sd, inp, llm_fp8, exp_fp8):
+    shape = _shape(cfg)
+    w = Weights(sd, O.fp8_linear_names(shape, llm_fp8, exp_fp8))
+    with torch.no_grad():
+        return O.sample_actions(w, shape, [i * 2.0 - 1.0 for i in inp["images"]], inp["img_masks"], inp["lang_tokens"], inp["lang_masks"], inp["noise"])
+
+
+def _gpu_chunk(cfg, sd, inp, **tiers):
+    from tybok_amd.policies.pi05.model import PI05Model
+
+    model = PI05Model(cfg, sd, "cuda", **tiers)
+    with torch.inference_mode():
+        out = model.sample_actions(
+            [(i * 2.0 - 1.0).cuda() for i in inp["images"]], [m.cuda() for m in inp["img_masks"]], inp["lang_tokens"].cuda(),
+            inp["lang_masks"].cuda(), inp["noise"].cuda(),
+        )  # fmt: skip
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+TIERS = [
+    dict(fused_expert=False, fp8_expert_mlp=False, fp8_llm_mlp=False),
+    dict(fused_expert=True, fp8_expert_mlp=False, fp8_llm_mlp=False),
+    dict(fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True),
+]
+
+
+@pytest.mark.parametrize("tiers", TIERS, ids=["eager", "attn", "full"])
+def test_small_model_chunk_matches_oracle(tiers):
+    cfg, sd, inp = cases.pi05_build(cases.PI05_CASES["small"])
+    want = _oracle_chunk(cfg, sd, inp, tiers["fp8_llm_mlp"], tiers["fp8_expert_mlp"])
+    got = _gpu_chunk(cfg, sd, inp, **tiers)
+    err = float((got - want).abs().max())
+    print(f"pi05 small {tiers}: max|err| = {err:.4g}, |chunk|max = {float(want.abs().max()):.3g}")
+    assert torch.isfinite(got).all()
+    assert err <= 1e-2 * max(1.0, float(want.abs().max()))
+    if not any(tiers.values()):
+        gold = torch.from_numpy(np.load(os.path.join(HERE, "golden", "pi05_small.npz"))["chunk"])[None]
+        assert float((got - gold).abs().max()) <= 1e-2 * max(1.0, float(gold.abs().max()))
+
+
+def test_zero_noise_chunk_within_bound():
+    # zero noise, full fp8 path, reduced depth (the full-depth run is the benchmark's job)
+    case = dict(cases.PI05_CASES["small"], noise="zeros", depth=4, num_steps=10, seed=21)
+    cfg, sd, inp = cases.pi05_build(case)
+    want = _oracle_chunk(cfg, sd, inp, True, True)
+    got = _gpu_chunk(cfg, sd, inp, fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True)
+    err = float((got - want).abs().max())
+    print(f"pi05 zero-noise fp8: max|err| = {err:.4g}, |chunk|max = {float(want.abs().max()):.3g}")
+    assert err <= 1e-2
+
+
+@pytest.fixture(scope="module")
+def ckpt(tmp_path_factory):
+    from tybok_amd.policies.synthetic import write_pi05_checkpoint
+
+    return write_pi05_checkpoint(str(tmp_path_factory.mktemp("pi05_ckpt")), cameras=2, seed=6, depth=2, vision_layers=2, num_steps=3)
+
+
+def test_engine_api_and_graph_equals_eager(ckpt):
+    from tybok_amd.registry import create_engine
+
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True)
+    eager = create_engine(ckpt, device="cuda", graph=False, warmup=False, **flags)
+    graph = create_engine(ckpt, device="cuda", graph=True, warmup=True, **flags)
+    assert graph.graph_enabled and list(graph._graph_runner.keys()) == [(2, 200)]
+    spec = eager.describe()
+    assert spec["model_type"] == "pi05" and spec["resize"] == [224, 224] and spec["pad_mode"] == "center"
+    assert spec["cameras"] == ["base_0_rgb", "left_wrist_0_rgb"] and spec["action_dim"] == 7 and spec["chunk_size"] == 50
+    frame = eager._profile_frame(seed=1)
+    noise = torch.zeros(1, 50, 7)
+    a = eager.predict_action_chunk(frame, noise=noise)
+    assert a.shape == (50, 7) and np.isfinite(a).all()
+    for _ in range(3):
+        assert np.array_equal(a, graph.predict_action_chunk(frame, noise=noise))
+        assert np.array_equal(a, eager.predict_action_chunk(frame, noise=noise))
+    chunk, normalized = graph.predict_action_chunk(frame, noise=noise, return_normalized=True)
+    assert np.array_equal(chunk, a) and normalized.shape == (50, 7)
+    with pytest.raises(NotImplementedError):
+        create_engine(ckpt, device="cuda", warmup=False, pad_free=True)
+    with pytest.raises(NotImplementedError):
+        create_engine(ckpt, device="cuda", warmup=False, rtc_config={"enabled": True})

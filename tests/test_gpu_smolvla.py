@@ -1,0 +1,121 @@
+"""SmolVLA backend on the GPU against the CPU oracle: model-level parity per tier, engine API,
+hipGraph replay == eager, camera-count graph keys."""
+
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "golden"))
+
+import cases  # noqa: E402
+from oracle import smolvla as O  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_chunk(cfg, sd, inp, llm_fp8: bool, exp_fp8: bool):
+    shape = O.SmolVLAShape(num_vlm_layers=cfg.num_vlm_layers, vis_layers=cfg.vlm_config.vision_config.num_hidden_layers, num_steps=cfg.num_steps)
+    w = O.Weights(sd, O.fp8_linear_names(shape, llm_fp8, exp_fp8))
+    with torch.no_grad():
+        return O.sample_actions(w, shape, O.prepare_images(inp["images"]), inp["img_masks"], inp["lang_tokens"], inp["lang_masks"], inp["state"], inp["noise"])
+
+
+def _gpu_chunk(cfg, sd, inp, **tiers):
+    from tybok_amd.policies.smolvla.model import SmolVLAModel
+
+    model = SmolVLAModel(cfg, sd, "cuda", **tiers)
+    dev = lambda t: t.cuda()  # noqa: E731
+    with torch.inference_mode():
+        out = model.sample_actions(
+            [dev(i * 2.0 - 1.0) for i in inp["images"]], [dev(m) for m in inp["img_masks"]], dev(inp["lang_tokens"]),
+            dev(inp["lang_masks"]), dev(inp["state"]), dev(inp["noise"]),
+        )  # fmt: skip
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+TIERS = [
+    dict(fused_expert=False, fp8_expert_mlp=False, fp8_llm_mlp=False),  # plain torch on the GPU
+    dict(fused_expert=True, fp8_expert_mlp=False, fp8_llm_mlp=False),   # HIP attention
+    dict(fused_expert=False, fp8_expert_mlp=True, fp8_llm_mlp=False),   # HIP fp8 expert FFN
+    dict(fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True),     # the full fp8 path
+]
+
+
+@pytest.mark.parametrize("tiers", TIERS, ids=["eager", "attn", "fp8ffn", "full"])
+def test_small_model_chunk_matches_oracle(tiers):
+    cfg, sd, inp = cases.smolvla_build(cases.SMOLVLA_CASES["small"])
+    want = _oracle_chunk(cfg, sd, inp, tiers["fp8_llm_mlp"], tiers["fp8_expert_mlp"])
+    got = _gpu_chunk(cfg, sd, inp, **tiers)
+    err = float((got - want).abs().max())
+    print(f"small {tiers}: max|err| = {err:.4g}, |chunk|max = {float(want.abs().max()):.3g}")
+    assert torch.isfinite(got).all()
+    # random noise drives |chunk| up to ~4: the 1e-2 bound of the zero-noise case scales with it
+    assert err <= 1e-2 * max(1.0, float(want.abs().max()))
+
+
+def test_full_model_zero_noise_chunk_matches_oracle_and_golden():
+    # benchmark config 4: 16+16 layers, 3 cameras, 10 steps, zero noise, full fp8 path
+    cfg, sd, inp = cases.smolvla_build(cases.SMOLVLA_CASES["full"])
+    want = _oracle_chunk(cfg, sd, inp, True, True)
+    got = _gpu_chunk(cfg, sd, inp, fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True)
+    err = float((got - want).abs().max())
+    print(f"full fp8: max|err| = {err:.4g}, |chunk|max = {float(want.abs().max()):.3g}")
+    assert err <= 1e-2
+    # the bf16 (no fp8) GPU path against the reference's own output for the same tensors
+    gold = torch.from_numpy(np.load(os.path.join(HERE, "golden", "smolvla_full.npz"))["chunk"])[None]
+    got16 = _gpu_chunk(cfg, sd, inp, fused_expert=True, fp8_expert_mlp=False, fp8_llm_mlp=False)
+    err16 = float((got16 - gold).abs().max())
+    print(f"full bf16 vs reference golden: max|err| = {err16:.4g}")
+    assert err16 <= 1e-2
+
+
+@pytest.fixture(scope="module")
+def ckpt(tmp_path_factory):
+    from tybok_amd.policies.synthetic import write_smolvla_checkpoint
+
+    return write_smolvla_checkpoint(str(tmp_path_factory.mktemp("smolvla_ckpt")), cameras=3, seed=5, num_vlm_layers=4, vision_layers=2, num_steps=3)
+
+
+def test_engine_api_graph_equals_eager_and_camera_keys(ckpt):
+    from tybok_amd.registry import create_engine
+
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True)
+    eager = create_engine(ckpt, device="cuda", graph=False, warmup=False, **flags)
+    graph = create_engine(ckpt, device="cuda", graph=True, graph_cameras=(2, 3), warmup=True, seed=3, **flags)
+    assert graph.graph_enabled and sorted(graph._graph_runner.keys()) == [(2,), (3,)]
+    spec = eager.describe()
+    assert spec == {"model_type": "smolvla", "cameras": ["camera1", "camera2", "camera3"], "resize": [512, 512], "action_dim": 6, "chunk_size": 50}
+    noise = torch.zeros(1, 50, 6)
+    for cams in (3, 2):
+        frame = eager._profile_frame(cameras=cams, seed=cams)
+        a = eager.predict_action_chunk(frame, noise=noise)
+        assert a.shape == (50, 6) and a.dtype == np.float32 and np.isfinite(a).all()
+        # several replays interleaved with eager work: every replay equals the eager result bit for bit
+        for _ in range(3):
+            b = graph.predict_action_chunk(frame, noise=noise)
+            assert np.array_equal(a, b)
+            assert np.array_equal(a, eager.predict_action_chunk(frame, noise=noise))
+    # select_action drains a queue of chunk_size actions before inferring again
+    first = graph.select_action(frame, noise=noise)
+    assert first.shape == (6,) and np.array_equal(first, b[0])
+    assert np.array_equal(graph.select_action(frame, noise=noise), b[1])
+    # implicit noise: seeded engine RNG, drawn outside the graph -> two calls differ
+    c1 = graph.predict_action_chunk(frame)
+    c2 = graph.predict_action_chunk(frame)
+    assert not np.array_equal(c1, c2)
+
+
+def test_engine_rejects_flags_it_does_not_implement(ckpt):
+    from tybok_amd.registry import create_engine
+
+    with pytest.raises(NotImplementedError):
+        create_engine(ckpt, device="cuda", warmup=False, tl_fused_vit=True)
+    with pytest.raises(NotImplementedError):
+        create_engine(ckpt, device="cuda", warmup=False, compile_model=True)
+    with pytest.raises(ValueError):
+        create_engine(ckpt, device="cuda", warmup=False, sampler="heun")

@@ -299,11 +299,13 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       const int n = (strip * NT + nt) * 32 + l32;
       if (n >= a.N) continue;
       const float sc = nt < 2 ? sc_pre[nt < 2 ? nt : 0] : a.s0[n];
+      const float gt = a.gate ? bf16_bits_to_f32(a.gate[n]) : 1.0f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int m = (mblock * MT + mt) * 32 + mfma32_row(lane, i);
         if (m < a.M) {
           u16 r = f32_to_bf16_bits(own[slot][i] * sc);
+          if (a.gate) r = f32_to_bf16_bits(bf16_bits_to_f32(r) * gt);
           if (a.resid) {
             float rv = a.resid_f32 ? ((const float*)a.resid)[(size_t)m * a.ldr + n]
                                    : bf16_bits_to_f32(((const u16*)a.resid)[(size_t)m * a.ldr + n]);

@@ -43,8 +43,8 @@ int device_cus() {
 
 // One GEMM launch (plain or gated).  `N` is the logical output width.
 int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, const float* s1, void* y, int ldy,
-                const void* resid, int ldr, int resid_dtype, int M, int N, int K, int split_k, int act, void* ws,
-                size_t ws_bytes, hipStream_t st) {
+                const void* resid, int ldr, int resid_dtype, const void* gate, int M, int N, int K, int split_k,
+                int act, void* ws, size_t ws_bytes, hipStream_t st) {
   if (M <= 0 || N <= 0 || K <= 0) return fail(TK_EINVAL, "gemm: non-positive shape M=%d N=%d K=%d", M, N, K);
   if (K % 16) return fail(TK_EINVAL, "gemm: K=%d must be a multiple of 16", K);
   if (ldx % 8 || ldx < K) return fail(TK_EINVAL, "gemm: ldx=%d must be >= K and a multiple of 8", ldx);
@@ -66,6 +66,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   a.resid = resid;
   a.ldr = ldr;
   a.resid_f32 = resid_dtype == TK_F32;
+  a.gate = (const u16*)gate;
   a.M = M;
   a.N = N;
   a.K = K;
@@ -149,14 +150,16 @@ int tk_pack_fp8_gate_up(const void* wg8, const void* wu8, void* packed, int I, i
 }
 
 int tk_fp8w_gemm(const void* x, int ldx, const void* w_packed, const void* scale, void* y, int ldy, const void* resid,
-                 int ldr, int resid_dtype, int M, int N, int K, int split_k, void* ws, size_t ws_bytes, void* stream) {
-  return gemm_common(x, ldx, w_packed, (const float*)scale, nullptr, y, ldy, resid, ldr, resid_dtype, M, N, K, split_k,
-                     0, ws, ws_bytes, (hipStream_t)stream);
+                 int ldr, int resid_dtype, const void* gate, int M, int N, int K, int split_k, void* ws, size_t ws_bytes,
+                 void* stream) {
+  return gemm_common(x, ldx, w_packed, (const float*)scale, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, N, K,
+                     split_k, 0, ws, ws_bytes, (hipStream_t)stream);
 }
 
 int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void* sg, const void* su,
                       const void* wd_packed, const void* sd, void* y, int ldy, const void* resid, int ldr,
-                      int resid_dtype, int M, int K, int I, int act, void* ws, size_t ws_bytes, void* stream) {
+                      int resid_dtype, const void* gate, int M, int K, int I, int act, void* ws, size_t ws_bytes,
+                      void* stream) {
   if (act != TK_ACT_SILU && act != TK_ACT_GELU_TANH) return fail(TK_EINVAL, "ffn: unknown activation %d", act);
   if (!sg || !su || !sd) return fail(TK_EINVAL, "ffn: null scale pointer");
   if (I % 32) return fail(TK_EINVAL, "ffn: I=%d must be a multiple of 32", I);
@@ -166,12 +169,12 @@ int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void
     return fail(TK_EWORKSPACE, "ffn: workspace too small for the [%d, %d] intermediate", M, I);
   void* hbuf = (char*)ws + kHiddenOff;
   // gate/up + activation-multiply -> h[M, I] (bf16, workspace)
-  int rc = gemm_common(x, ldx, wgu_packed, (const float*)sg, (const float*)su, hbuf, I, nullptr, 0, 0, M, I, K, 0, act,
-                       ws, ws_bytes, (hipStream_t)stream);
+  int rc = gemm_common(x, ldx, wgu_packed, (const float*)sg, (const float*)su, hbuf, I, nullptr, 0, 0, nullptr, M, I, K, 0,
+                       act, ws, ws_bytes, (hipStream_t)stream);
   if (rc) return rc;
   // down projection (+ residual)
-  return gemm_common(hbuf, I, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, M, K, I, 0, 0, ws,
-                     ws_bytes, (hipStream_t)stream);
+  return gemm_common(hbuf, I, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, K, I, 0, 0,
+                     ws, ws_bytes, (hipStream_t)stream);
 }
 
 int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* v_pre, int pre_sl, int pre_sh,

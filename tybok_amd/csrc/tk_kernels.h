@@ -14,6 +14,7 @@ struct GemmArgs {
   const void* resid;
   int ldr;
   int resid_f32;
+  const unsigned short* gate;  // bf16 [N] per-column gate applied before the residual, or nullptr
   int M, N, K;  // N: logical output columns (gated: the intermediate size I)
   int KT;       // k tiles of 32
   int ntiles;   // n tiles of 32 in the packed buffer (gated: 2 * I / 32)

@@ -29,13 +29,13 @@ SIGNATURES: dict[str, tuple] = {
     "tk_pack_fp8_gate_up": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "tk_fp8w_gemm": (
         c_int,
-        [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-         c_void_p, c_size_t, c_void_p],
+        [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
+         c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
     "tk_fp8w_gated_ffn": (
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
-         c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
+         c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
     "tk_expert_attn": (
         c_int,

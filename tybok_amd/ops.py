@@ -131,16 +131,25 @@ def _resid_args(resid: torch.Tensor | None, m: int, n: int) -> tuple[int | None,
     raise TypeError("residual must be bf16 or fp32")
 
 
+def _gate_ptr(gate: torch.Tensor | None, n: int) -> int | None:
+    if gate is None:
+        return None
+    if gate.dtype != torch.bfloat16 or gate.numel() != n or not gate.is_contiguous():
+        raise ValueError(f"gate must be a contiguous bf16 tensor of {n} elements")
+    return gate.data_ptr()
+
+
 def fp8w_gemm(
     x: torch.Tensor,
     w: PackedWeight,
     *,
     resid: torch.Tensor | None = None,
+    gate: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
     split_k: int = 0,
     ws: Workspace | None = None,
 ) -> torch.Tensor:
-    """``bf16((x @ W8^T) * scale)`` (+ residual) for ``x [M, K]`` bf16."""
+    """``bf16((x @ W8^T) * scale)`` (``* gate[n]``, ``+ residual``) for ``x [M, K]`` bf16."""
     lib = native.lib()
     m, ldx = _check_act(x, w.k)
     if out is None:
@@ -149,7 +158,7 @@ def fp8w_gemm(
     ws = ws or default_workspace(x.device)
     rc = lib.tk_fp8w_gemm(
         x.data_ptr(), ldx, w.data.data_ptr(), w.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt,
-        m, w.n, w.k, split_k, ws.ptr, ws.nbytes, _stream(),
+        _gate_ptr(gate, w.n), m, w.n, w.k, split_k, ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip
     native.check(rc, "tk_fp8w_gemm")
     return out
@@ -162,10 +171,11 @@ def fp8w_gated_ffn(
     act: str = "silu",
     *,
     resid: torch.Tensor | None = None,
+    gate: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
     ws: Workspace | None = None,
 ) -> torch.Tensor:
-    """``down(act(gate(x)) * up(x))`` (+ residual) for ``x [M, K]`` bf16."""
+    """``down(act(gate(x)) * up(x))`` (``* gate[n]``, ``+ residual``) for ``x [M, K]`` bf16."""
     lib = native.lib()
     m, ldx = _check_act(x, wgu.k)
     if wd.k != wgu.i or wd.n != wgu.k:
@@ -177,10 +187,20 @@ def fp8w_gated_ffn(
     rc = lib.tk_fp8w_gated_ffn(
         x.data_ptr(), ldx, wgu.data.data_ptr(), wgu.scale_gate.data_ptr(), wgu.scale_up.data_ptr(),
         wd.data.data_ptr(), wd.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt,
-        m, wgu.k, wgu.i, ACT[act], ws.ptr, ws.nbytes, _stream(),
+        _gate_ptr(gate, wd.n), m, wgu.k, wgu.i, ACT[act], ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip
     native.check(rc, "tk_fp8w_gated_ffn")
     return out
+
+
+def _eff_strides(t: torch.Tensor) -> tuple[int, int]:
+    """(row, head) element strides of a ``[L, G, D]`` view; a size-1 dim never advances, so its
+    stride is reported as 0 whatever torch recorded for it."""
+    return (t.stride(0) if t.shape[0] > 1 else 0, t.stride(1) if t.shape[1] > 1 else 0)
+
+
+def _same_layout(k: torch.Tensor, v: torch.Tensor) -> bool:
+    return k.shape == v.shape and k.stride(2) == 1 and v.stride(2) == 1 and _eff_strides(k) == _eff_strides(v)
 
 
 def expert_attn(
@@ -205,7 +225,7 @@ def expert_attn(
     p, g = k_pre.shape[0], k_pre.shape[1]
     if k_pre.dtype != v_pre.dtype or k_pre.dtype not in (torch.bfloat16, torch.float32):
         raise TypeError("prefix K/V must both be bf16 or both fp32")
-    if k_pre.stride() != v_pre.stride() or k_pre.stride(2) != 1:
+    if not _same_layout(k_pre, v_pre):
         raise ValueError("prefix K and V must share strides and have a contiguous head dim")
     s = 0
     suf_sl = suf_sh = 0
@@ -213,10 +233,10 @@ def expert_attn(
         assert v_suf is not None
         if k_suf.dtype != torch.bfloat16 or v_suf.dtype != torch.bfloat16:
             raise TypeError("suffix K/V must be bf16")
-        if k_suf.stride() != v_suf.stride() or k_suf.stride(2) != 1:
+        if not _same_layout(k_suf, v_suf):
             raise ValueError("suffix K and V must share strides and have a contiguous head dim")
         s = k_suf.shape[0]
-        suf_sl, suf_sh = k_suf.stride(0), k_suf.stride(1)
+        suf_sl, suf_sh = _eff_strides(k_suf)
     pad = None
     if prefix_pad is not None:
         pad = prefix_pad.view(torch.uint8) if prefix_pad.dtype == torch.bool else prefix_pad
@@ -226,7 +246,7 @@ def expert_attn(
         out = torch.empty(m, h * d, dtype=torch.bfloat16, device=q.device)
     ws = ws or default_workspace(q.device)
     rc = lib.tk_expert_attn(
-        q.data_ptr(), q.stride(0), q.stride(1), k_pre.data_ptr(), v_pre.data_ptr(), k_pre.stride(0), k_pre.stride(1),
+        q.data_ptr(), q.stride(0), q.stride(1), k_pre.data_ptr(), v_pre.data_ptr(), *_eff_strides(k_pre),
         _F32 if k_pre.dtype == torch.float32 else _BF16, _ptr(k_suf), _ptr(v_suf), suf_sl, suf_sh, _ptr(pad),
         out.data_ptr(), out.stride(0), m, p, s, h, g, d, mask_mode, int(logits_bf16), ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip

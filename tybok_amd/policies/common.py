@@ -1,0 +1,123 @@
+"""Pieces shared by the two backends: dataset-statistics (un)normalisation, the task tokenizers
+and the safetensors parameter loader.  Behaviour follows the reference's per-backend copies
+(tybok/policies/smolvla/preprocess.py:36-182, tybok/policies/smolvla/tokenizer.py:31-87,
+tybok/policies/smolvla/models/policy.py:38-68).
+"""
+
+from __future__ import annotations
+
+import glob
+import hashlib
+import os
+from dataclasses import dataclass, field
+
+import torch
+
+OBS_STATE = "observation.state"
+OBS_LANGUAGE_TOKENS = "observation.language.tokens"
+OBS_LANGUAGE_ATTENTION_MASK = "observation.language.attention_mask"
+ACTION = "action"
+
+
+@dataclass
+class Normalizer:
+    """Per-feature MEAN_STD (un)normalisation; identity when the key has no statistics."""
+
+    norm_map: dict[str, str]
+    stats: dict[str, dict[str, torch.Tensor]] = field(default_factory=dict)
+    eps: float = 1e-8
+
+    @classmethod
+    def from_files(cls, pattern: str, norm_map: dict[str, str]) -> "Normalizer":
+        stats: dict[str, dict[str, torch.Tensor]] = {}
+        for file in sorted(glob.glob(pattern)):
+            from safetensors import safe_open
+
+            with safe_open(file, "pt", "cpu") as f:
+                for flat in f.keys():
+                    key, stat = flat.rsplit(".", 1)
+                    stats.setdefault(key, {})[stat] = f.get_tensor(flat).float()
+        return cls(norm_map=norm_map, stats=stats)
+
+    def _apply(self, t: torch.Tensor, key: str, ftype: str, inverse: bool) -> torch.Tensor:
+        mode = self.norm_map.get(ftype, "IDENTITY")
+        if mode == "IDENTITY" or key not in self.stats:
+            return t
+        if mode != "MEAN_STD":
+            raise ValueError(f"Unsupported normalization mode: {mode}")
+        mean, std = self.stats[key].get("mean"), self.stats[key].get("std")
+        if mean is None or std is None:
+            raise ValueError("MEAN_STD normalization mode requires mean and std stats")
+        mean, std = mean.to(t.device), std.to(t.device)
+        return t * std + mean if inverse else (t - mean) / (std + self.eps)
+
+    def normalize(self, t, key, ftype):
+        return self._apply(t, key, ftype, False)
+
+    def unnormalize(self, t, key, ftype):
+        return self._apply(t, key, ftype, True)
+
+
+def load_normalizer(checkpoint_dir: str, norm_map: dict[str, str]) -> Normalizer:
+    return Normalizer.from_files(
+        os.path.join(checkpoint_dir, "policy_preprocessor_step_*_normalizer_processor.safetensors"), norm_map
+    )
+
+
+def load_unnormalizer(checkpoint_dir: str, norm_map: dict[str, str]) -> Normalizer:
+    return Normalizer.from_files(
+        os.path.join(checkpoint_dir, "policy_postprocessor_step_*_unnormalizer_processor.safetensors"), norm_map
+    )
+
+
+class FileTokenizer:
+    """``tokenizers`` tokenizer loaded from ``tokenizer.json``: truncation + right padding to ``max_length``."""
+
+    def __init__(self, tokenizer_dir: str, max_length: int, pad_token: str, append_newline: bool = True):
+        from tokenizers import Tokenizer
+
+        self.tok = Tokenizer.from_file(os.path.join(tokenizer_dir, "tokenizer.json"))
+        self.max_length = max_length
+        self.tok.enable_truncation(max_length=max_length)
+        pad_id = self.tok.token_to_id(pad_token)
+        self.tok.enable_padding(pad_id=pad_id if pad_id is not None else 0, pad_token=pad_token, length=max_length, direction="right")
+
+    def encode_task(self, task: str) -> tuple[torch.Tensor, torch.Tensor]:
+        enc = self.tok.encode(task)
+        return torch.tensor([enc.ids], dtype=torch.long), torch.tensor([enc.attention_mask], dtype=torch.bool)
+
+
+class SyntheticTokenizer:
+    """Stand-in for random-init checkpoints (no ``tokenizer.json``): ``max_length`` token ids drawn
+    from a generator seeded by the task string, all unmasked.  Deterministic per task."""
+
+    def __init__(self, vocab_size: int, max_length: int):
+        self.vocab_size, self.max_length = int(vocab_size), int(max_length)
+
+    def encode_task(self, task: str) -> tuple[torch.Tensor, torch.Tensor]:
+        seed = int.from_bytes(hashlib.sha256(task.encode("utf-8")).digest()[:4], "little")
+        g = torch.Generator().manual_seed(seed)
+        ids = torch.randint(0, self.vocab_size, (1, self.max_length), generator=g)
+        return ids, torch.ones(1, self.max_length, dtype=torch.bool)
+
+
+def load_state_dict(checkpoint_dir: str, wanted: dict[str, tuple], remap: dict[str, str] | None = None) -> dict[str, torch.Tensor]:
+    """Read every ``*.safetensors`` of the checkpoint (processor statistics aside) and return the
+    tensors whose names (minus a leading ``model.``) are in ``wanted``; raises if one is missing."""
+    from safetensors import safe_open
+
+    out: dict[str, torch.Tensor] = {}
+    for file in sorted(glob.glob(os.path.join(checkpoint_dir, "*.safetensors"))):
+        if "processor" in os.path.basename(file):
+            continue
+        with safe_open(file, "pt", "cpu") as f:
+            for name in f.keys():
+                key = (remap or {}).get(name, name)
+                for cand in (key, key[len("model.") :] if key.startswith("model.") else None):
+                    if cand in wanted:
+                        out[cand] = f.get_tensor(name)
+                        break
+    missing = [k for k in wanted if k not in out]
+    if missing:
+        raise FileNotFoundError(f"{len(missing)} parameters missing from {checkpoint_dir} (e.g. {missing[0]})")
+    return out

@@ -1,0 +1,342 @@
+"""pi0.5 policy engine, registered as ``model_type="pi05"``.
+
+Constructor keywords, ``describe()`` keys and the ``predict_action_chunk`` / ``select_action``
+semantics are the reference's (tybok/policies/pi05/engine.py:104-132, 472-481, 668-741).  Tier
+flags wired to the HIP kernels:
+
+* ``tl_fused_expert``     expert denoising attention on ``tk_expert_attn`` (bf16 logits)
+* ``tl_fp8_expert_mlp``   expert GeGLU FFN on e4m3fn weights with the gated residual fused
+* ``tl_fp8_llm_mlp``      VLM prefill GeGLU FFN on e4m3fn weights
+
+The prefix-side tiers (``tl_fused_vit``, ``tl_llm_flash_attn``, ``vit_mlp_dtype``, ``pad_free``,
+``skip_empty_images``), ``compile_model`` and Real-Time Chunking are not implemented here and are
+rejected when requested.
+"""
+
+from __future__ import annotations
+
+import logging
+import os
+from collections import deque
+from typing import Any
+
+import numpy as np
+import torch
+import torch.nn.functional as F  # noqa: N812
+
+from ...base import PolicyEngine
+from ...graph import CaptureSession, GraphRunner
+from ...image_utils import resize_with_pad_center
+from ...registry import register, reject_unsupported_flags
+from ..common import (
+    ACTION,
+    OBS_LANGUAGE_ATTENTION_MASK,
+    OBS_LANGUAGE_TOKENS,
+    OBS_STATE,
+    FileTokenizer,
+    SyntheticTokenizer,
+    load_normalizer,
+    load_state_dict,
+    load_unnormalizer,
+)
+from .config import PI05Config
+from .model import PI05Model
+from .weights import parameter_inventory, random_state_dict
+
+log = logging.getLogger("tybok.pi05")
+
+# the checkpoint stores the VLM embedding table under the tied lm_head
+# (tybok/policies/pi05/models/policy.py:35-42)
+_KEY_REMAP = {
+    "model.paligemma_with_expert.paligemma.lm_head.weight": "model.paligemma_with_expert.paligemma.model.language_model.embed_tokens.weight",
+    "paligemma_with_expert.paligemma.lm_head.weight": "paligemma_with_expert.paligemma.model.language_model.embed_tokens.weight",
+}
+
+
+def build_prompt(task: str, normalized_state: torch.Tensor) -> str:
+    """``"Task: <task>, State: <256-bin ints>;\\nAction: "`` (tybok/policies/pi05/preprocess.py:112-123)."""
+    state = normalized_state.detach().cpu().numpy()
+    bins = np.linspace(-1, 1, 256 + 1)[:-1]
+    digits = np.digitize(state, bins=bins) - 1
+    text = task.strip().replace("_", " ").replace("\n", " ")
+    return f"Task: {text}, State: {' '.join(map(str, digits.tolist()))};\nAction: "
+
+
+@register("pi05")
+class PI05Engine(PolicyEngine):
+    _UNSUPPORTED_FLAGS = {
+        "tl_llm_fused_attn": False,
+        "tl_vit_oproj": False,
+        "tl_fused_vit": False,
+        "tl_llm_flash_attn": False,
+        "vit_mlp_dtype": None,
+        "skip_empty_images": False,
+        "pad_free": False,
+        "pack_qkv": False,
+        "text_fused": False,
+        "text_fused_split": False,
+        "action_fused": False,
+        "action_fused_split": False,
+        "video_fused": False,
+        "video_fused_split": False,
+        "action_pre_fused": False,
+        "video_pre_fused": False,
+        "require_fused": False,
+        "text_encoder_dir": None,
+        "vae_dir": None,
+    }
+
+    def __init__(
+        self,
+        checkpoint_dir: str,
+        device: str = "auto",
+        compile_model: bool = False,
+        warmup: bool = True,
+        graph: bool = False,
+        graph_cameras: tuple[int, ...] | None = None,
+        num_steps: int | None = None,
+        seed: int | None = None,
+        sampler: str = "euler",
+        cache_expert_prefix_kv: bool = True,
+        profile: bool = False,
+        overlap: bool = True,
+        tl_fused_vit: bool = False,
+        tl_llm_flash_attn: bool = False,
+        tl_fused_expert: bool = False,
+        tl_fp8_llm_mlp: bool = False,
+        tl_fp8_expert_mlp: bool = False,
+        vit_mlp_dtype: str | None = None,
+        skip_empty_images: bool = False,
+        pad_free: bool = False,
+        camera_alias: dict[str, str] | None = None,
+        tokenizer_dir: str | None = None,
+        rtc_config: dict | None = None,
+        **kwargs: Any,
+    ):
+        super().__init__(checkpoint_dir, device=device)
+        reject_unsupported_flags(type(self), "pi05", kwargs)
+        reject_unsupported_flags(
+            type(self), "pi05",
+            dict(tl_fused_vit=tl_fused_vit, tl_llm_flash_attn=tl_llm_flash_attn, vit_mlp_dtype=vit_mlp_dtype,
+                 skip_empty_images=skip_empty_images, pad_free=pad_free),
+        )  # fmt: skip
+        if sampler != "euler":
+            raise ValueError(f"sampler {sampler!r} not supported for pi05 (only 'euler')")
+        if compile_model:
+            raise NotImplementedError("--compile is not supported by this backend (the HIP tiers replace it)")
+        if rtc_config and rtc_config.get("enabled"):
+            raise NotImplementedError("Real-Time Chunking is not implemented by this backend")
+        hip_flags = [n for n, on in (("--tl-fused-expert", tl_fused_expert), ("--tl-fp8-llm-mlp", tl_fp8_llm_mlp), ("--tl-fp8-expert-mlp", tl_fp8_expert_mlp)) if on]
+        if hip_flags and not str(self.device).startswith("cuda"):
+            # same gate as the reference's _require_fp8_mma (engine.py:51-71), for this hardware
+            raise RuntimeError(f"{' / '.join(hip_flags)} run gfx950 HIP kernels, but the engine is running on {self.device!r}")
+        self.compile_model = False
+        self.config = PI05Config.from_pretrained(checkpoint_dir, tokenizer_dir=tokenizer_dir)
+        if num_steps is not None:
+            self.config.num_steps = int(num_steps)
+
+        tok_dir = self.config.tokenizer_dir
+        if tok_dir and os.path.isfile(os.path.join(tok_dir, "tokenizer.json")):
+            self.tokenizer = FileTokenizer(tok_dir, self.config.tokenizer_max_length, "<pad>")
+        elif self.config.random_init is not None:
+            self.tokenizer = SyntheticTokenizer(self.config.vocab_size, self.config.tokenizer_max_length)
+        else:
+            raise FileNotFoundError("no tokenizer.json: pass --tokenizer-dir")
+
+        if self.config.random_init is not None:
+            sd = random_state_dict(self.config, seed=int(self.config.random_init.get("seed", 0)))
+        else:
+            sd = load_state_dict(checkpoint_dir, {n: s for n, s, _, _ in parameter_inventory(self.config)}, remap=_KEY_REMAP)
+        self.tl_fused_expert = bool(tl_fused_expert)
+        self.tl_fp8_llm_mlp = bool(tl_fp8_llm_mlp)
+        self.tl_fp8_expert_mlp = bool(tl_fp8_expert_mlp)
+        self.model = PI05Model(
+            self.config, sd, self.device,
+            fused_expert=self.tl_fused_expert, fp8_expert_mlp=self.tl_fp8_expert_mlp, fp8_llm_mlp=self.tl_fp8_llm_mlp,
+        )  # fmt: skip
+        del sd
+
+        norm_map = self.config.normalization_mapping
+        self.normalizer = load_normalizer(checkpoint_dir, norm_map)
+        self.unnormalizer = load_unnormalizer(checkpoint_dir, norm_map)
+        self.camera_alias: dict[str, str] = {}
+        for src, dst in (camera_alias or {}).items():
+            s = src if src.startswith("observation.images.") else f"observation.images.{src}"
+            d = dst if dst.startswith("observation.images.") else f"observation.images.{dst}"
+            if d not in self.config.image_features:
+                raise ValueError(f"camera_alias target {dst!r} is not an expected image feature")
+            self.camera_alias[s] = d
+
+        self.seed = seed
+        self._noise_gen: torch.Generator | None = None
+        if seed is not None:
+            self._noise_gen = torch.Generator(device=self.device).manual_seed(int(seed))
+        self._action_queue: deque[torch.Tensor] = deque(maxlen=self.config.n_action_steps)
+        self.rtc_processor = None
+
+        self.graph_requested = bool(graph)
+        self.graph_enabled = self.graph_requested and str(self.device).startswith("cuda")
+        self.overlap = False  # prefill x step-0 two-stream overlap is not implemented; accepted, inert
+        self._sess = CaptureSession(self.device)
+        self._graph_runner = GraphRunner(self._capture_graph, self.device, label="pi05 graph", logger=log)
+        if warmup:
+            self._warmup()
+        if self.graph_enabled:
+            key = (len(self.config.image_features), self.config.tokenizer_max_length)
+            if not self._graph_runner.precapture([key]):
+                log.warning("graph capture failed; falling back to eager")
+                self.graph_enabled = False
+                self._graph_runner.clear()
+        if profile:
+            try:
+                self.profile()
+            except Exception as e:  # noqa: BLE001 - never fail startup on a diagnostic
+                log.warning(f"profile failed: {e}")
+
+    # ------------------------------------------------------------------ API
+    def supports_rtc(self) -> bool:
+        return False
+
+    def describe(self) -> dict[str, Any]:
+        return {
+            "model_type": "pi05",
+            "cameras": [k[len("observation.images.") :] for k in self.config.real_camera_keys],
+            "resize": [self.config.image_resolution[1], self.config.image_resolution[0]],
+            "pad_mode": "center",
+            "action_dim": int(self.config.action_feature_shape[0]),
+            "chunk_size": int(self.config.chunk_size),
+            "rtc": False,
+        }
+
+    @torch.inference_mode()
+    def predict_action_chunk(self, frame: dict[str, Any], noise: torch.Tensor | None = None, *, return_normalized: bool = False, **rtc: Any) -> Any:
+        if any(v is not None for v in rtc.values()):
+            raise NotImplementedError("Real-Time Chunking guidance arguments are not supported by this backend")
+        batch = self._batch_from_frame(frame)
+        actions = self._infer(batch, self._prepare_noise(noise))[:, :, : self.config.action_feature_shape[0]]
+        chunk = self.unnormalizer.unnormalize(actions, ACTION, "ACTION").cpu().numpy()[0]
+        return (chunk, actions.cpu().numpy()[0]) if return_normalized else chunk
+
+    @torch.inference_mode()
+    def select_action(self, frame: dict[str, Any], noise: torch.Tensor | None = None) -> np.ndarray:
+        if not self._action_queue:
+            batch = self._batch_from_frame(frame)
+            actions = self._infer(batch, self._prepare_noise(noise))[:, : self.config.n_action_steps, : self.config.action_feature_shape[0]]
+            self._action_queue.extend(actions.transpose(0, 1))
+        action = self._action_queue.popleft()
+        return self.unnormalizer.unnormalize(action, ACTION, "ACTION").cpu().numpy()[0]
+
+    def validate(self, reference_dir: str) -> dict[str, float]:
+        def load(name: str):
+            path = os.path.join(reference_dir, name)
+            if not os.path.exists(path):
+                raise FileNotFoundError(f"reference dump {path} missing")
+            return torch.load(path, weights_only=True)
+
+        frame, ref = load("frame.pt"), load("chunk.pt")
+        noise = torch.zeros(1, self.config.chunk_size, self.config.action_feature_shape[0])
+        chunk = torch.from_numpy(self.predict_action_chunk(frame, noise=noise))
+        diff = (chunk - ref["chunk_post"].float().cpu().reshape(chunk.shape)).abs()
+        return {"chunk_post.max": float(diff.max()), "chunk_post.mean": float(diff.mean())}
+
+    # ------------------------------------------------------------------ request plumbing
+    def _batch_from_frame(self, frame: dict[str, Any]) -> dict[str, torch.Tensor]:
+        """Batch dimension, state normalisation, state-in-prompt tokenisation (preprocess.py:159-189)."""
+        frame = dict(frame)
+        for src, dst in self.camera_alias.items():
+            if src in frame and dst not in frame:
+                frame[dst] = frame.pop(src)
+        batch: dict[str, torch.Tensor] = {}
+        for key, value in frame.items():
+            if key.startswith("observation.") and isinstance(value, torch.Tensor):
+                batch[key] = value.unsqueeze(0) if value.ndim in (1, 3) else value
+        if OBS_STATE in batch:
+            batch[OBS_STATE] = self.normalizer.normalize(batch[OBS_STATE], OBS_STATE, "STATE")
+        if OBS_LANGUAGE_TOKENS not in batch:
+            state = batch.get(OBS_STATE)
+            if state is None:
+                raise ValueError("state is required for PI05")
+            task = frame.get("task", "")
+            if not isinstance(task, str):
+                raise ValueError(f"task must be a string, got {type(task).__name__}")
+            prompt = build_prompt(task, state[0] if state.ndim == 2 else state)
+            batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK] = self.tokenizer.encode_task(prompt)
+        return {k: v.to(self.device) for k, v in batch.items()}
+
+    def _prepare_noise(self, noise: torch.Tensor | None) -> torch.Tensor | None:
+        if noise is None:
+            return None
+        noise = noise.to(self.device, dtype=torch.float32)
+        if noise.shape[-1] != self.config.max_action_dim:
+            noise = F.pad(noise, (0, self.config.max_action_dim - noise.shape[-1]))
+        return noise
+
+    def prepare_images(self, batch: dict[str, torch.Tensor]):
+        """Centre-padded resize to 224x224, [0,1] -> [-1,1]; missing slots become -1 images with a zero mask (policy.py:170-234)."""
+        h, w = self.config.image_resolution
+        present = [k for k in self.config.image_features if k in batch]
+        if not present:
+            raise ValueError(f"All image features are missing from the batch (expected {self.config.image_features})")
+        images, masks = [], []
+        for key in present:
+            img = resize_with_pad_center(batch[key].float(), h, w) * 2.0 - 1.0
+            images.append(img)
+            masks.append(torch.ones(img.shape[0], dtype=torch.bool, device=img.device))
+        for _ in [k for k in self.config.image_features if k not in batch]:
+            images.append(torch.ones_like(images[-1]) * -1)
+            masks.append(torch.zeros_like(masks[-1]))
+        return images, masks
+
+    def _sample_noise(self, out: torch.Tensor | None = None) -> torch.Tensor:
+        shape = (1, self.config.chunk_size, self.config.max_action_dim)
+        return torch.normal(0.0, 1.0, size=shape, dtype=torch.float32, device=self.device, generator=self._noise_gen, out=out)
+
+    def _infer(self, batch: dict[str, torch.Tensor], noise: torch.Tensor | None) -> torch.Tensor:
+        images, img_masks = self.prepare_images(batch)
+        tokens, masks = batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK]
+        if self.graph_enabled and self._graph_runner:
+            entry = self._graph_runner.entry((len(images), int(tokens.shape[1])))
+            return self._run_graph(entry, images, img_masks, tokens, masks, noise)
+        if noise is None:
+            noise = self._sample_noise()
+        return self.model.sample_actions(images, img_masks, tokens, masks, noise)
+
+    # ------------------------------------------------------------------ hipGraph path
+    def _capture_graph(self, key, request=None) -> dict[str, Any]:
+        """One graph of the whole inference core for ``key = (n_cams, lang_len)`` (engine.py:542-606)."""
+        n_cams, lang_len = int(key[0]), int(key[1])
+        h, w = self.config.image_resolution
+        dev = self.device
+        static: dict[str, Any] = {
+            "images": [torch.zeros(1, 3, h, w, dtype=torch.float32, device=dev) for _ in range(n_cams)],
+            "img_masks": [torch.ones(1, dtype=torch.bool, device=dev) for _ in range(n_cams)],
+            "tokens": torch.zeros(1, lang_len, dtype=torch.int64, device=dev),
+            "masks": torch.ones(1, lang_len, dtype=torch.bool, device=dev),
+            "noise": torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, dtype=torch.float32, device=dev),
+            "out": torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, dtype=torch.float32, device=dev),
+        }
+        model = self.model
+
+        def core() -> None:
+            static["out"].copy_(model.sample_actions(static["images"], static["img_masks"], static["tokens"], static["masks"], static["noise"]))
+
+        log.info(f"capturing one graph for {n_cams} camera(s), lang={lang_len}, steps={self.config.num_steps}")
+        graph = self._sess.prime_and_capture(core)
+        self._sess.sync()
+        return {"graph": graph, "statics": static}
+
+    def _run_graph(self, entry, images, img_masks, tokens, masks, noise) -> torch.Tensor:
+        static = entry["statics"]
+        with self._graph_runner.copy_inputs():
+            for i, (img, mask) in enumerate(zip(images, img_masks)):
+                static["images"][i].copy_(img)
+                static["img_masks"][i].copy_(mask)
+            static["tokens"].copy_(tokens)
+            static["masks"].copy_(masks)
+            if noise is None:
+                self._sample_noise(out=static["noise"])
+            else:
+                static["noise"].copy_(noise)
+        self._graph_runner.wait_inputs()
+        entry["graph"].replay()
+        return static["out"].clone()

@@ -1,0 +1,242 @@
+"""pi0.5 flow-matching model on one MI355X.
+
+Same computation as the reference's ``PI05FlowMatching`` + ``PaliGemmaWithExpertModel`` +
+``GemmaDecoder`` (tybok/policies/pi05/models/flow_matching.py:261-838,
+tybok/policies/pi05/models/paligemma_with_expert.py:129-276, tybok/policies/pi05/models/gemma.py,
+tybok/policies/pi05/models/layers.py), with the reference's seams wired to the HIP kernels:
+
+* ``fp8_expert_mlp`` / ``fp8_llm_mlp``  -- the GeGLU FFN of the expert / VLM layers runs as
+  ``tk_fp8w_gated_ffn`` on e4m3fn weights; for the expert the AdaRMS gated residual
+  ``x + y * gate`` is fused into the down projection's epilogue (the seam of
+  ``_forward_fp8_mlp`` / ``make_fp8_mlp_forward``: layers.py:397-419, triton_prefill_mlp.py:145-166);
+* ``fused_expert``  -- the denoising attention over ``[prefix KV; suffix]`` runs as
+  ``tk_expert_attn`` with bf16 logits (the seam of ``_forward_fused_attn``: layers.py:330-371).
+
+The per-step AdaRMS modulations ``dense(time_mlp(time_emb))`` depend only on the step index and
+are computed once (the reference's static path does the same: flow_matching.py:321-358).
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F  # noqa: N812
+
+from ... import ops as tk
+from ..smolvla.model import GatedMLP, sinusoidal_time_embedding
+from .config import PI05Config
+from .weights import EXP, PROJ, VIS, VLM
+
+BF16 = torch.bfloat16
+EPS = 1e-6
+MASK_VALUE = -2.3819763e38  # additive mask of the openpi attention
+_ROPE_POSITIONS = 2048
+
+
+def gemma_norm(x: torch.Tensor, weight: torch.Tensor | None = None, modulation: torch.Tensor | None = None):
+    """Gemma RMSNorm (``* (1 + w)``) or AdaRMS (``* (1 + scale) + shift``, returns the gate) -- layers.py:51-84."""
+    dim = x.shape[-1]
+    var = torch.mean(torch.square(x.float()), dim=-1, keepdim=True)
+    normed = x * torch.rsqrt(var + EPS)
+    if modulation is None:
+        return (normed * (1.0 + weight.float())).to(x.dtype), None
+    mod = modulation.unsqueeze(1) if (x.dim() == 3 and modulation.dim() == 2) else modulation
+    if mod.shape[-1] == 2 * dim:
+        scale, shift = mod.chunk(2, dim=-1)
+        return (normed * (1 + scale.float()) + shift.float()).to(x.dtype), None
+    scale, shift, gate = mod.chunk(3, dim=-1)
+    return (normed * (1 + scale.float()) + shift.float()).to(x.dtype), gate.to(x.dtype)
+
+
+def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """``x [B,H,L,D]`` rotated in its own dtype with ``cos/sin [B,L,D]`` (rope.py:44-75)."""
+    half = x.shape[-1] // 2
+    rot = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+    return x * cos.unsqueeze(1) + rot * sin.unsqueeze(1)
+
+
+def attention_core(q, k, v, add_mask, scaling: float) -> torch.Tensor:
+    """bf16 logits, fp32 softmax (layers.py:179-191): ``q [B,H,Lq,D]``, ``k/v [B,G,Lk,D]`` -> ``[B,Lq,H*D]``."""
+    b, h, lq, d = q.shape
+    g = k.shape[1]
+    if h != g:
+        k = k[:, :, None].expand(b, g, h // g, k.shape[2], d).reshape(b, h, k.shape[2], d)
+        v = v[:, :, None].expand(b, g, h // g, v.shape[2], d).reshape(b, h, v.shape[2], d)
+    logits = torch.matmul(q, k.transpose(2, 3)) * scaling + add_mask
+    probs = F.softmax(logits, dim=-1, dtype=torch.float32).to(q.dtype)
+    return torch.matmul(probs, v).transpose(1, 2).reshape(b, lq, h * d)
+
+
+class PI05Model:
+    def __init__(
+        self,
+        cfg: PI05Config,
+        state_dict: dict[str, torch.Tensor],
+        device: str | torch.device,
+        *,
+        fused_expert: bool = False,
+        fp8_expert_mlp: bool = False,
+        fp8_llm_mlp: bool = False,
+    ):
+        self.cfg = cfg
+        self.device = torch.device(device)
+        self.fused_expert = bool(fused_expert)
+        self.fp8_expert_mlp = bool(fp8_expert_mlp)
+        self.fp8_llm_mlp = bool(fp8_llm_mlp)
+        self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp
+        if self.use_hip and self.device.type != "cuda":
+            raise RuntimeError("the fused / fp8 tiers run HIP kernels and need a GPU device")
+        self.vd, self.ed = cfg.paligemma_dims, cfg.expert_dims
+        self.depth = self.vd["depth"]
+        self.head_dim = self.vd["head_dim"]
+        mlp_keys = tuple(f".mlp.{p}_proj.weight" for p in ("gate", "up", "down"))
+        self.p = {k: v.to(self.device) for k, v in state_dict.items() if not k.endswith(mlp_keys)}
+        self.vlm_mlp = [GatedMLP(state_dict, f"{VLM}layers.{i}.mlp.", self.device, self.fp8_llm_mlp, act="gelu_tanh") for i in range(self.depth)]
+        self.exp_mlp = [GatedMLP(state_dict, f"{EXP}layers.{i}.mlp.", self.device, self.fp8_expert_mlp, act="gelu_tanh") for i in range(self.ed["depth"])]
+        self.ws = tk.default_workspace(self.device) if self.use_hip else None
+
+        inv = 1.0 / (10000.0 ** (torch.arange(0, self.head_dim, 2, dtype=torch.int64).float() / self.head_dim))
+        inv = inv.to(BF16).float()  # the reference's inverse frequencies go through a bf16 buffer
+        freqs = torch.arange(_ROPE_POSITIONS, dtype=torch.float32)[:, None] * inv[None, :]
+        emb = torch.cat([freqs, freqs], dim=-1)
+        self.rope_cos, self.rope_sin = emb.cos().to(self.device), emb.sin().to(self.device)
+        self.embed_scale = torch.tensor(self.vd["width"] ** 0.5, dtype=BF16, device=self.device)
+        self.patch_w = self.p[VIS + "embeddings.patch_embedding.weight"].reshape(cfg.vision_hidden, -1)
+        self.set_num_steps(cfg.num_steps)
+
+    def lin(self, name: str, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(x, self.p[name + ".weight"], self.p.get(name + ".bias"))
+
+    def set_num_steps(self, n: int) -> None:
+        """Per-step AdaRMS modulations of every expert norm (computed on the device, once)."""
+        self.num_steps = int(n)
+        dt = -1.0 / self.num_steps
+        self.mods: list[list[tuple[torch.Tensor, torch.Tensor]]] = []
+        self.final_mods: list[torch.Tensor] = []
+        with torch.inference_mode():
+            for step in range(self.num_steps):
+                t = torch.tensor(1.0 + step * dt, dtype=torch.float32).expand(1)
+                te = sinusoidal_time_embedding(t, self.ed["width"], self.cfg.min_period, self.cfg.max_period).float().to(self.device)
+                cond = F.silu(self.lin("time_mlp_out", F.silu(self.lin("time_mlp_in", te))))
+                self.mods.append(
+                    [
+                        (self.lin(f"{EXP}layers.{i}.input_layernorm.dense", cond), self.lin(f"{EXP}layers.{i}.post_attention_layernorm.dense", cond))
+                        for i in range(self.ed["depth"])
+                    ]
+                )
+                self.final_mods.append(self.lin(EXP + "norm.dense", cond))
+
+    def rope_tables(self, pos: torch.Tensor, dtype) -> tuple[torch.Tensor, torch.Tensor]:
+        return self.rope_cos[pos].to(dtype), self.rope_sin[pos].to(dtype)
+
+    # ------------------------------------------------------------------ vision + prefix
+    def embed_image(self, image: torch.Tensor) -> torch.Tensor:
+        """``[1, 3, 224, 224]`` fp32 in [-1, 1] -> ``[1, 256, vlm_width]`` fp32 (SigLIP tower + projector, fp32)."""
+        cfg, p = self.cfg, self.p
+        b = image.shape[0]
+        ps = cfg.vision_patch
+        n_h, n_w = image.shape[2] // ps, image.shape[3] // ps
+        x = image.float().view(b, 3, n_h, ps, n_w, ps).permute(0, 2, 4, 1, 3, 5).reshape(b, n_h * n_w, 3 * ps * ps)
+        x = F.linear(x, self.patch_w, p[VIS + "embeddings.patch_embedding.bias"])
+        x = x + p[VIS + "embeddings.position_embedding.weight"][None]
+        vh, heads = cfg.vision_hidden, cfg.vision_heads
+        hd = vh // heads
+        for i in range(cfg.vision_layers):
+            lp = f"{VIS}encoder.layers.{i}."
+            h = F.layer_norm(x, (vh,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], EPS)
+            q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
+            k = self.lin(lp + "self_attn.k_proj", h).view(b, -1, heads, hd).transpose(1, 2)
+            v = self.lin(lp + "self_attn.v_proj", h).view(b, -1, heads, hd).transpose(1, 2)
+            att = torch.softmax(torch.matmul(q, k.transpose(2, 3)) * hd**-0.5, dim=-1)
+            a = torch.matmul(att, v).transpose(1, 2).reshape(b, -1, vh)
+            x = x + self.lin(lp + "self_attn.out_proj", a)
+            h = F.layer_norm(x, (vh,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS)
+            x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
+        x = F.layer_norm(x, (vh,), p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], EPS)
+        return self.lin(PROJ, x)
+
+    def embed_prefix(self, images, img_masks, tokens, masks):
+        """-> ``(embs fp32 [1,P,W], pad_masks [1,P])``; every prefix token attends to every valid one."""
+        embs, pads = [], []
+        for img, m in zip(images, img_masks):
+            e = self.embed_image(img)
+            embs.append(e)
+            pads.append(m[:, None].expand(e.shape[0], e.shape[1]))
+        lang = F.embedding(tokens, self.p[VLM + "embed_tokens.weight"]) * self.embed_scale
+        embs.append(lang)
+        pads.append(masks)
+        return torch.cat(embs, dim=1), torch.cat(pads, dim=1)
+
+    def _attn_proj(self, lp: str, h: torch.Tensor, cos, sin):
+        b, length = h.shape[0], h.shape[1]
+        q = self.lin(lp + "q_proj", h).view(b, length, -1, self.head_dim).transpose(1, 2)
+        k = self.lin(lp + "k_proj", h).view(b, length, -1, self.head_dim).transpose(1, 2)
+        v = self.lin(lp + "v_proj", h).view(b, length, -1, self.head_dim).transpose(1, 2)
+        return apply_rope(q, cos, sin), apply_rope(k, cos, sin), v
+
+    def prefill(self, embs: torch.Tensor, pad_masks: torch.Tensor):
+        """VLM prefill -> per-layer post-RoPE ``(K, V)`` bf16 ``[1, G, P, D]``."""
+        mask = pad_masks[:, None, :] & pad_masks[:, :, None]
+        add = torch.where(mask[:, None], 0.0, MASK_VALUE)
+        pos = torch.cumsum(pad_masks, dim=1) - 1
+        hidden = embs.to(BF16)
+        cos, sin = self.rope_tables(pos, hidden.dtype)
+        kv = []
+        scaling = self.head_dim**-0.5
+        for i in range(self.depth):
+            lp = f"{VLM}layers.{i}."
+            h, _ = gemma_norm(hidden, weight=self.p[lp + "input_layernorm.weight"])
+            q, k, v = self._attn_proj(lp + "self_attn.", h, cos, sin)
+            kv.append((k, v))
+            hidden = hidden + self.lin(lp + "self_attn.o_proj", attention_core(q, k, v, add, scaling))
+            h, _ = gemma_norm(hidden, weight=self.p[lp + "post_attention_layernorm.weight"])
+            hidden = self.vlm_mlp[i](h, hidden)
+        return kv
+
+    # ------------------------------------------------------------------ denoising
+    def denoise_step(self, prefix_pad, kv, x_t, step: int) -> torch.Tensor:
+        """Velocity fp32 ``[1, chunk, max_action_dim]`` at denoising step ``step`` (flow_matching.py:505-556)."""
+        hidden = self.lin("action_in_proj", x_t).to(BF16)
+        b, s = hidden.shape[0], hidden.shape[1]
+        p_len = prefix_pad.shape[1]
+        pos = prefix_pad.sum(dim=-1)[:, None] + torch.arange(s, device=self.device)[None, :]
+        cos, sin = self.rope_tables(pos, hidden.dtype)
+        scaling = self.head_dim**-0.5
+        if not self.fused_expert:
+            vis = torch.cat([prefix_pad[:, None, :].expand(b, s, p_len), torch.ones(b, s, s, dtype=torch.bool, device=self.device)], dim=2)
+            add = torch.where(vis[:, None], 0.0, MASK_VALUE)
+        for i in range(self.ed["depth"]):
+            lp = f"{EXP}layers.{i}."
+            mod_in, mod_post = self.mods[step][i]
+            h, gate = gemma_norm(hidden, modulation=mod_in)
+            q, k, v = self._attn_proj(lp + "self_attn.", h, cos, sin)
+            if self.fused_expert:
+                pk, pv = kv[i]
+                att = tk.expert_attn(
+                    q[0].transpose(0, 1), pk[0].transpose(0, 1), pv[0].transpose(0, 1), k[0].transpose(0, 1), v[0].transpose(0, 1),
+                    prefix_pad[0], tk.MASK_BIDIR, logits_bf16=True, ws=self.ws,
+                )[None]  # fmt: skip
+            else:
+                att = attention_core(q, torch.cat([kv[i][0], k], dim=2), torch.cat([kv[i][1], v], dim=2), add, scaling)
+            hidden = hidden + self.lin(lp + "self_attn.o_proj", att) * gate
+            h, gate = gemma_norm(hidden, modulation=mod_post)
+            mlp = self.exp_mlp[i]
+            if mlp.fp8:
+                y = tk.fp8w_gated_ffn(h.view(b * s, -1), mlp.wgu, mlp.wd, "gelu_tanh", resid=hidden.view(b * s, -1), gate=gate.reshape(-1), ws=self.ws)
+                hidden = y.view(b, s, -1)
+            else:
+                a = F.gelu(F.linear(h, mlp.wg), approximate="tanh") * F.linear(h, mlp.wu)
+                hidden = hidden + F.linear(a, mlp.wdn) * gate
+        out, _ = gemma_norm(hidden, modulation=self.final_mods[step])
+        return self.lin("action_out_proj", out.to(torch.float32))
+
+    def sample_actions(self, images, img_masks, tokens, masks, noise, trace: dict | None = None) -> torch.Tensor:
+        """Prefix embed, prefill, Euler loop -> ``[1, chunk, max_action_dim]`` fp32."""
+        embs, pads = self.embed_prefix(images, img_masks, tokens, masks)
+        kv = self.prefill(embs, pads)
+        if trace is not None:
+            trace.update(prefix_embs=embs, pad_masks=pads, kv=kv)
+        dt = -1.0 / self.num_steps
+        x_t = noise
+        for step in range(self.num_steps):
+            x_t = x_t + dt * self.denoise_step(pads, kv, x_t, step)
+        return x_t

@@ -1,0 +1,348 @@
+"""SmolVLA policy engine, registered as ``model_type="smolvla"``.
+
+Constructor keywords, ``describe()`` keys and the ``predict_action_chunk`` / ``select_action``
+semantics are the reference's (tybok/policies/smolvla/engine.py:78-96, 332-400), so the worker and
+gateway need no change.  The tier flags select the HIP kernels:
+
+* ``tl_fused_expert``     expert denoising attention on ``tk_expert_attn``
+* ``tl_fp8_expert_mlp``   expert gated FFN on e4m3fn weights (``tk_fp8w_gated_ffn``)
+* ``tl_fp8_llm_mlp``      VLM prefill gated FFN on e4m3fn weights
+
+The reference's SmolVLA backend rejects the two fp8 flags (engine.py:47-55); here they are
+implemented, because the fp8 action-inference path is what this backend is for.
+``tl_llm_fused_attn`` / ``tl_vit_oproj`` (prefill / vision fusions) and ``compile_model`` have no
+implementation here and are rejected when requested.
+"""
+
+from __future__ import annotations
+
+import logging
+import os
+from collections import deque
+from typing import Any
+
+import numpy as np
+import torch
+import torch.nn.functional as F  # noqa: N812
+
+from ...base import PolicyEngine
+from ...graph import CaptureSession, GraphRunner, camera_counts
+from ...image_utils import resize_with_pad
+from ...registry import register
+from ..common import (
+    ACTION,
+    OBS_LANGUAGE_ATTENTION_MASK,
+    OBS_LANGUAGE_TOKENS,
+    OBS_STATE,
+    FileTokenizer,
+    SyntheticTokenizer,
+    load_normalizer,
+    load_state_dict,
+    load_unnormalizer,
+)
+from .config import SmolVLAConfig
+from .model import SmolVLAModel
+from .weights import parameter_inventory, random_state_dict
+
+log = logging.getLogger("tybok.smolvla")
+
+
+@register("smolvla")
+class SmolVLAEngine(PolicyEngine):
+    # flags owned by other backends or not implemented here: inert default -> accepted, else rejected
+    _UNSUPPORTED_FLAGS = {
+        "tl_llm_fused_attn": False,
+        "tl_vit_oproj": False,
+        "tl_fused_vit": False,
+        "tl_llm_flash_attn": False,
+        "vit_mlp_dtype": None,
+        "skip_empty_images": False,
+        "pad_free": False,
+        "pack_qkv": False,
+        "text_fused": False,
+        "text_fused_split": False,
+        "action_fused": False,
+        "action_fused_split": False,
+        "video_fused": False,
+        "video_fused_split": False,
+        "action_pre_fused": False,
+        "video_pre_fused": False,
+        "require_fused": False,
+        "text_encoder_dir": None,
+        "vae_dir": None,
+    }
+
+    def __init__(
+        self,
+        checkpoint_dir: str,
+        device: str = "auto",
+        compile_model: bool = False,
+        warmup: bool = True,
+        graph: bool = False,
+        graph_cameras: tuple[int, ...] | None = None,
+        num_steps: int | None = None,
+        seed: int | None = None,
+        sampler: str = "euler",
+        cache_expert_prefix_kv: bool = True,
+        profile: bool = False,
+        overlap: bool = True,
+        camera_alias: dict[str, str] | None = None,
+        tl_llm_fused_attn: bool = False,
+        tl_vit_oproj: bool = False,
+        tl_fused_expert: bool = False,
+        tl_fp8_llm_mlp: bool = False,
+        tl_fp8_expert_mlp: bool = False,
+    ):
+        super().__init__(checkpoint_dir, device=device)
+        if sampler != "euler":
+            raise ValueError(f"unknown sampler {sampler!r} (this backend implements 'euler')")
+        if compile_model:
+            raise NotImplementedError("--compile is not supported by this backend (the HIP tiers replace it)")
+        if tl_llm_fused_attn or tl_vit_oproj:
+            raise NotImplementedError("--tl-llm-fused-attn / --tl-vit-oproj are not implemented by this backend")
+        self.compile_model = False
+        self.config = SmolVLAConfig.from_pretrained(checkpoint_dir)
+        if self.config.vlm_config is None:
+            raise ValueError(
+                f"Could not locate the VLM backbone config for {self.config.vlm_model_name!r}; "
+                "check `vlm_model_name` in the checkpoint config.json"
+            )
+        if num_steps is not None:
+            self.config.num_steps = int(num_steps)
+        self.config.cache_expert_prefix_kv = bool(cache_expert_prefix_kv)
+        hip_flags = [n for n, on in (("--tl-fused-expert", tl_fused_expert), ("--tl-fp8-llm-mlp", tl_fp8_llm_mlp), ("--tl-fp8-expert-mlp", tl_fp8_expert_mlp)) if on]
+        if hip_flags and not str(self.device).startswith("cuda"):
+            raise RuntimeError(f"{' / '.join(hip_flags)} run gfx950 HIP kernels, but the engine is running on {self.device!r}")
+
+        vocab = self.config.vlm_config.text_config.vocab_size
+        tok_dir = self.config.vlm_dir or checkpoint_dir
+        if os.path.isfile(os.path.join(tok_dir, "tokenizer.json")):
+            self.tokenizer = FileTokenizer(tok_dir, self.config.tokenizer_max_length, "<|im_end|>")
+        elif self.config.random_init is not None:
+            self.tokenizer = SyntheticTokenizer(vocab, self.config.tokenizer_max_length)
+        else:
+            raise FileNotFoundError(f"no tokenizer.json under {tok_dir}")
+
+        if self.config.random_init is not None:
+            sd = random_state_dict(self.config, seed=int(self.config.random_init.get("seed", 0)))
+        else:
+            sd = load_state_dict(checkpoint_dir, {n: s for n, s, _, _ in parameter_inventory(self.config)})
+        self.tl_fused_expert = bool(tl_fused_expert)
+        self.tl_fp8_llm_mlp = bool(tl_fp8_llm_mlp)
+        self.tl_fp8_expert_mlp = bool(tl_fp8_expert_mlp)
+        self.model = SmolVLAModel(
+            self.config, sd, self.device,
+            fused_expert=self.tl_fused_expert, fp8_expert_mlp=self.tl_fp8_expert_mlp, fp8_llm_mlp=self.tl_fp8_llm_mlp,
+        )  # fmt: skip
+        del sd
+
+        norm_map = self.config.normalization_mapping
+        self.normalizer = load_normalizer(checkpoint_dir, norm_map)
+        self.unnormalizer = load_unnormalizer(checkpoint_dir, norm_map)
+        self.camera_alias = self._resolve_alias(camera_alias)
+
+        self.seed = seed
+        self._noise_gen: torch.Generator | None = None
+        if seed is not None:
+            self._noise_gen = torch.Generator(device=self.device).manual_seed(int(seed))
+        self._action_queue: deque[torch.Tensor] = deque(maxlen=self.config.n_action_steps)
+
+        self.graph_requested = bool(graph)
+        self.graph_enabled = self.graph_requested and str(self.device).startswith("cuda")
+        self.overlap = False  # prefill x step-0 two-stream overlap is not implemented; accepted, inert
+        self._sess = CaptureSession(self.device)
+        self._graph_runner = GraphRunner(self._capture_graph, self.device, label="smolvla graph", logger=log)
+        self._graph_fallback_warned = False
+
+        if warmup:
+            self._warmup()
+        if self.graph_enabled:
+            max_cams = len(self.config.image_features)
+            counts = camera_counts(graph_cameras, default=max_cams, max_images=max_cams)
+            if not self._graph_runner.precapture([(n,) for n in counts]):
+                log.warning("graph capture failed for all requested camera counts; falling back to eager mode")
+                self.graph_enabled = False
+                self._graph_runner.clear()
+        if profile:
+            try:
+                self.profile()
+            except Exception as e:  # noqa: BLE001 - never fail startup on a diagnostic
+                log.warning(f"profile failed: {e}")
+
+    # ------------------------------------------------------------------ API
+    def describe(self) -> dict[str, Any]:
+        return {
+            "model_type": "smolvla",
+            "cameras": [k[len("observation.images.") :] for k in self.config.image_features],
+            "resize": list(self.config.resize_imgs_with_padding),
+            "action_dim": int(self.config.action_feature_shape[0]),
+            "chunk_size": int(self.config.chunk_size),
+        }
+
+    @torch.inference_mode()
+    def predict_action_chunk(self, frame: dict[str, Any], noise: torch.Tensor | None = None) -> np.ndarray:
+        batch = self._batch_from_frame(frame)
+        actions = self._infer(batch, self._prepare_noise(noise))
+        actions = actions[:, :, : self.config.action_feature_shape[0]]
+        return self.unnormalizer.unnormalize(actions, ACTION, "ACTION").cpu().numpy()[0]
+
+    @torch.inference_mode()
+    def select_action(self, frame: dict[str, Any], noise: torch.Tensor | None = None) -> np.ndarray:
+        if not self._action_queue:
+            batch = self._batch_from_frame(frame)
+            actions = self._infer(batch, self._prepare_noise(noise))[:, :, : self.config.action_feature_shape[0]]
+            self._action_queue.extend(actions.transpose(0, 1)[: self.config.n_action_steps])
+        action = self._action_queue.popleft()
+        return self.unnormalizer.unnormalize(action, ACTION, "ACTION").cpu().numpy()[0]
+
+    def validate(self, reference_dir: str) -> dict[str, float]:
+        """Max/mean-abs errors of the full zero-noise chunk against ``chunk.pt`` of a reference dump
+        (``frame.pt`` + ``chunk.pt``: tybok/policies/smolvla/engine.py:668-673, 738-752)."""
+
+        def load(name: str):
+            path = os.path.join(reference_dir, name)
+            if not os.path.exists(path):
+                raise FileNotFoundError(f"reference dump {path} missing")
+            return torch.load(path, weights_only=True)
+
+        frame, ref = load("frame.pt"), load("chunk.pt")
+        noise = torch.zeros(1, self.config.chunk_size, self.config.action_feature_shape[0])
+        chunk = torch.from_numpy(self.predict_action_chunk(frame, noise=noise))
+        diff = (chunk - ref["chunk_post"].float().cpu().reshape(chunk.shape)).abs()
+        return {"chunk_post.max": float(diff.max()), "chunk_post.mean": float(diff.mean())}
+
+    # ------------------------------------------------------------------ request plumbing
+    def _resolve_alias(self, camera_alias: dict[str, str] | None) -> dict[str, str]:
+        full: dict[str, str] = {}
+        for src, dst in (camera_alias or {}).items():
+            s = src if src.startswith("observation.images.") else f"observation.images.{src}"
+            d = dst if dst.startswith("observation.images.") else f"observation.images.{dst}"
+            if d not in self.config.image_features:
+                raise ValueError(f"camera_alias target {dst!r} is not an expected image feature")
+            if s in self.config.image_features:
+                raise ValueError(f"camera_alias source {src!r} is already an expected image feature")
+            full[s] = d
+        return full
+
+    def _batch_from_frame(self, frame: dict[str, Any]) -> dict[str, torch.Tensor]:
+        """Batch dimension, task tokens, device move, state normalisation (preprocess.py:138-171)."""
+        frame = dict(frame)
+        for src, dst in self.camera_alias.items():
+            if src in frame and dst not in frame:
+                frame[dst] = frame.pop(src)
+        batch: dict[str, torch.Tensor] = {}
+        for key, value in frame.items():
+            if key.startswith("observation.") and isinstance(value, torch.Tensor):
+                batch[key] = value.unsqueeze(0) if value.ndim in (1, 3) else value
+        if OBS_LANGUAGE_TOKENS not in batch:
+            task = frame.get("task", "")
+            if isinstance(task, str) and not task.endswith("\n"):
+                task = f"{task}\n"
+            batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK] = self.tokenizer.encode_task(task)
+        batch = {k: v.to(self.device) for k, v in batch.items()}
+        if OBS_STATE in batch:
+            batch[OBS_STATE] = self.normalizer.normalize(batch[OBS_STATE], OBS_STATE, "STATE")
+        return batch
+
+    def _prepare_noise(self, noise: torch.Tensor | None) -> torch.Tensor | None:
+        if noise is None:
+            return None
+        noise = noise.to(self.device, dtype=torch.float32)
+        if noise.shape[-1] != self.config.max_action_dim:
+            noise = F.pad(noise, (0, self.config.max_action_dim - noise.shape[-1]))
+        return noise
+
+    def prepare_images(self, batch: dict[str, torch.Tensor]):
+        """Resize (left/top pad) to the model resolution, [0,1] -> [-1,1]; masks all true (policy.py:117-163)."""
+        w, h = self.config.resize_imgs_with_padding
+        present = [k for k in self.config.image_features if k in batch]
+        if not present:
+            raise ValueError(f"All image features are missing from the batch (expected {self.config.image_features})")
+        images, masks = [], []
+        for key in present:
+            img = resize_with_pad(batch[key], h, w, pad_value=0) * 2.0 - 1.0
+            images.append(img)
+            masks.append(torch.ones(img.shape[0], dtype=torch.bool, device=img.device))
+        missing = [k for k in self.config.image_features if k not in batch]
+        for _ in range(min(len(missing), self.config.empty_cameras)):
+            images.append(torch.ones_like(images[-1]) * -1)
+            masks.append(torch.zeros_like(masks[-1]))
+        return images, masks
+
+    def prepare_state(self, batch: dict[str, torch.Tensor]) -> torch.Tensor:
+        state = batch[OBS_STATE]
+        if state.shape[-1] < self.config.max_state_dim:
+            state = F.pad(state, (0, self.config.max_state_dim - state.shape[-1]))
+        return state
+
+    def _sample_noise(self, out: torch.Tensor | None = None) -> torch.Tensor:
+        shape = (1, self.config.chunk_size, self.config.max_action_dim)
+        return torch.normal(0.0, 1.0, size=shape, dtype=torch.float32, device=self.device, generator=self._noise_gen, out=out)
+
+    def _infer(self, batch: dict[str, torch.Tensor], noise: torch.Tensor | None) -> torch.Tensor:
+        images, img_masks = self.prepare_images(batch)
+        state = self.prepare_state(batch)
+        tokens, lang_masks = batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK]
+        if self.graph_enabled and self._graph_runner:
+            entry = None
+            try:
+                entry = self._graph_runner.entry((len(images),))
+            except Exception as e:  # noqa: BLE001 - unseen shape that cannot be captured: eager for this request
+                if not self._graph_fallback_warned:
+                    log.warning(f"graph replay skipped ({e}); falling back to eager for this request")
+                    self._graph_fallback_warned = True
+            if entry is not None:
+                return self._run_graph(entry, images, img_masks, tokens, lang_masks, state, noise)
+        if noise is None:
+            noise = self._sample_noise()
+        return self.model.sample_actions(images, img_masks, tokens, lang_masks, state, noise)
+
+    # ------------------------------------------------------------------ hipGraph path
+    def _prefix_len_for(self, n_cams: int) -> int:
+        return n_cams * self.config.vlm_config.image_seq_len + self.config.tokenizer_max_length + 1
+
+    def _capture_graph(self, key, request=None) -> dict[str, Any]:
+        """One graph of the whole inference core for ``key = (n_cams,)`` (engine.py:408-472)."""
+        n_cams = int(key[0])
+        w, h = self.config.resize_imgs_with_padding
+        dev = self.device
+        static: dict[str, Any] = {
+            "images": [torch.zeros(1, 3, h, w, dtype=torch.float32, device=dev) for _ in range(n_cams)],
+            "img_masks": [torch.ones(1, dtype=torch.bool, device=dev) for _ in range(n_cams)],
+            "lang_tokens": torch.zeros(1, self.config.tokenizer_max_length, dtype=torch.long, device=dev),
+            "lang_masks": torch.ones(1, self.config.tokenizer_max_length, dtype=torch.bool, device=dev),
+            "state": torch.zeros(1, self.config.max_state_dim, dtype=torch.float32, device=dev),
+            "noise": torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, dtype=torch.float32, device=dev),
+            "out": torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, dtype=torch.float32, device=dev),
+        }
+        model = self.model
+
+        def core() -> None:
+            static["out"].copy_(
+                model.sample_actions(
+                    static["images"], static["img_masks"], static["lang_tokens"], static["lang_masks"], static["state"], static["noise"]
+                )
+            )
+
+        log.info(f"capturing one graph for {n_cams} camera(s) (prefix_len={self._prefix_len_for(n_cams)}, steps={self.config.num_steps})")
+        graph = self._sess.prime_and_capture(core)
+        self._sess.sync()
+        return {"graph": graph, "statics": static}
+
+    def _run_graph(self, entry, images, img_masks, tokens, lang_masks, state, noise) -> torch.Tensor:
+        """Copy the request into the static buffers (copy stream), replay, return a copy of the output."""
+        static = entry["statics"]
+        with self._graph_runner.copy_inputs():
+            for i, (img, mask) in enumerate(zip(images, img_masks)):
+                static["images"][i].copy_(img)
+                static["img_masks"][i].copy_(mask)
+            static["lang_tokens"].copy_(tokens)
+            static["lang_masks"].copy_(lang_masks)
+            static["state"].copy_(state)
+            if noise is None:
+                self._sample_noise(out=static["noise"])  # noise is drawn outside the graph
+            else:
+                static["noise"].copy_(noise)
+        self._graph_runner.wait_inputs()
+        entry["graph"].replay()
+        return static["out"].clone()

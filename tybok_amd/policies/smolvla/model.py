@@ -1,0 +1,313 @@
+"""SmolVLA flow-matching model on one MI355X.
+
+Same computation as the reference's ``VLAFlowMatching`` + ``SmolVLMWithExpertModel``
+(tybok/policies/smolvla/models/flow_matching.py:86-644,
+tybok/policies/smolvla/models/vlm_with_expert.py:41-511), with the reference's seams wired to
+the HIP kernels of this package:
+
+* ``fp8_expert_mlp`` / ``fp8_llm_mlp``  -- the gated FFN of the expert / VLM layers runs as
+  ``tk_fp8w_gated_ffn`` on e4m3fn weights (second residual fused), the seam where the reference
+  calls ``triton_norm_gate_up`` + ``down_proj`` (vlm_with_expert.py:391-408);
+* ``fused_expert``  -- the denoising self/cross attention runs as ``tk_expert_attn`` over the
+  cached prefix KV, the seam of ``triton_self_attn`` / ``triton_cross_attn``
+  (vlm_with_expert.py:166-190, 275-297).
+
+Everything else (norms, projections, RoPE, vision tower) is plain torch on the GPU.  The model
+is capture-clean: every constant is built at construction time, nothing copies from the host or
+synchronises inside :meth:`sample_actions`.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F  # noqa: N812
+
+from ... import ops as tk
+from ...quant import quantize_weight_rows
+from .config import SmolVLAConfig
+from .weights import CONNECTOR, EXP, TXT, VIS
+
+BF16 = torch.bfloat16
+_ROPE_POSITIONS = 16384
+
+
+def sinusoidal_time_embedding(time: torch.Tensor, dim: int, min_period: float, max_period: float) -> torch.Tensor:
+    """``cat(sin, cos)(2*pi*t/period)`` in float64 (flow_matching.py:27-42)."""
+    frac = torch.linspace(0.0, 1.0, dim // 2, dtype=torch.float64)
+    period = min_period * (max_period / min_period) ** frac
+    ang = (1.0 / period * 2 * math.pi)[None, :] * time.to(torch.float64)[:, None]
+    return torch.cat([torch.sin(ang), torch.cos(ang)], dim=1)
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """Llama RMSNorm: fp32 statistics, cast back, then the weight (layers.py:22-27)."""
+    x32 = x.to(torch.float32)
+    var = x32.pow(2).mean(-1, keepdim=True)
+    return weight * (x32 * torch.rsqrt(var + eps)).to(x.dtype)
+
+
+def eager_attention(mask: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    """fp32-score GQA attention (attention.py:136-187): ``q [B,Lq,H,D]``, ``k/v [B,Lk,G,D]``, bool ``mask [B,Lq,Lk]``."""
+    b, lq, h, d = q.shape
+    g = k.shape[2]
+    rep = h // g
+    kf = k[:, :, :, None, :].expand(b, k.shape[1], g, rep, d).reshape(b, k.shape[1], h, d)
+    vf = v[:, :, :, None, :].expand(b, v.shape[1], g, rep, d).reshape(b, v.shape[1], h, d)
+    scores = torch.matmul(q.float().transpose(1, 2), kf.float().permute(0, 2, 3, 1)) * d**-0.5
+    scores = torch.where(mask[:, None], scores, torch.finfo(torch.float32).min)
+    probs = F.softmax(scores, dim=-1).to(vf.dtype)
+    out = torch.matmul(probs, vf.permute(0, 2, 1, 3))
+    return out.permute(0, 2, 1, 3).reshape(b, lq, h * d)
+
+
+class GatedMLP:
+    """gate/up/down of one decoder layer: bf16 torch linears, or fp8 weights on the HIP kernel."""
+
+    def __init__(self, sd: dict, prefix: str, device, fp8: bool, act: str = "silu"):
+        self.act = act
+        self.fp8 = fp8
+        wg, wu, wd = (sd[prefix + n + ".weight"] for n in ("gate_proj", "up_proj", "down_proj"))
+        if fp8:
+            g8, sg = quantize_weight_rows(wg.to(device))
+            u8, su = quantize_weight_rows(wu.to(device))
+            d8, sdn = quantize_weight_rows(wd.to(device))
+            self.wgu = tk.pack_fp8_gate_up(g8, sg, u8, su)
+            self.wd = tk.pack_fp8_weight(d8, sdn)
+        else:
+            self.wg, self.wu, self.wdn = wg.to(device), wu.to(device), wd.to(device)
+
+    def __call__(self, x: torch.Tensor, resid: torch.Tensor) -> torch.Tensor:
+        """``down(act(gate(x)) * up(x)) + resid`` for ``x [B, L, hidden]`` bf16 (in-place add semantics)."""
+        if self.fp8:
+            b, length, hidden = x.shape
+            y = tk.fp8w_gated_ffn(x.reshape(b * length, hidden), self.wgu, self.wd, self.act, resid=resid.reshape(b * length, hidden))
+            return y.view(b, length, hidden)
+        a = F.silu(F.linear(x, self.wg)) if self.act == "silu" else F.gelu(F.linear(x, self.wg), approximate="tanh")
+        out = F.linear(a * F.linear(x, self.wu), self.wdn)
+        out += resid
+        return out
+
+
+class SmolVLAModel:
+    def __init__(
+        self,
+        cfg: SmolVLAConfig,
+        state_dict: dict[str, torch.Tensor],
+        device: str | torch.device,
+        *,
+        fused_expert: bool = False,
+        fp8_expert_mlp: bool = False,
+        fp8_llm_mlp: bool = False,
+    ):
+        assert cfg.vlm_config is not None
+        self.cfg = cfg
+        self.device = torch.device(device)
+        self.fused_expert = bool(fused_expert)
+        self.fp8_expert_mlp = bool(fp8_expert_mlp)
+        self.fp8_llm_mlp = bool(fp8_llm_mlp)
+        self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp
+        if self.use_hip and self.device.type != "cuda":
+            raise RuntimeError("the fused / fp8 tiers run HIP kernels and need a GPU device")
+        t = cfg.vlm_config.text_config
+        self.heads, self.kv_heads, self.head_dim = t.num_attention_heads, t.num_key_value_heads, t.head_dim
+        self.eps = t.rms_norm_eps
+        self.num_layers = cfg.num_vlm_layers
+        mlp_keys = tuple(f".mlp.{p}_proj.weight" for p in ("gate", "up", "down"))
+        # everything except the MLP weights (owned by GatedMLP, possibly as fp8) moves as is
+        self.p = {k: v.to(self.device) for k, v in state_dict.items() if not k.endswith(mlp_keys)}
+        self.vlm_mlp = [GatedMLP(state_dict, f"{TXT}layers.{i}.mlp.", self.device, self.fp8_llm_mlp) for i in range(self.num_layers)]
+        self.exp_mlp = [GatedMLP(state_dict, f"{EXP}layers.{i}.mlp.", self.device, self.fp8_expert_mlp) for i in range(cfg.n_expert_layers)]
+        self.ws = tk.default_workspace(self.device) if self.use_hip else None
+
+        # constants (built once: nothing below copies from the host at inference time)
+        d_half = self.head_dim // 2
+        exponents = (2.0 / (d_half * 2)) * torch.arange(d_half, dtype=torch.float32)
+        radians = torch.arange(_ROPE_POSITIONS, dtype=torch.float32)[:, None] / (10_000.0**exponents)[None, :]
+        self.rope_sin = torch.sin(radians).to(self.device)
+        self.rope_cos = torch.cos(radians).to(self.device)
+        self.set_num_steps(cfg.num_steps)
+        v = cfg.vlm_config.vision_config
+        side = v.image_size // v.patch_size
+        self.vis_pos = torch.arange(side * side, device=self.device)
+        self.img_scale = torch.tensor(t.hidden_size**0.5, dtype=BF16, device=self.device)
+        self.patch_w = self.p[VIS + "embeddings.patch_embedding.weight"].reshape(v.hidden_size, -1)
+
+    def set_num_steps(self, n: int) -> None:
+        self.num_steps = int(n)
+        dt = -1.0 / self.num_steps
+        embs = []
+        for step in range(self.num_steps):
+            t = torch.tensor(1.0 + step * dt, dtype=torch.float32).expand(1)
+            embs.append(sinusoidal_time_embedding(t, self.cfg.expert_hidden_size, self.cfg.min_period, self.cfg.max_period).float())
+        self.time_embs = [e.to(self.device) for e in embs]
+
+    # ------------------------------------------------------------------ helpers
+    def lin(self, name: str, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(x, self.p[name + ".weight"], self.p.get(name + ".bias"))
+
+    def rope(self, x: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        """Half-split RoPE of ``x [B, L, H, D]`` at integer ``positions [B, L]`` (rope.py:51-73)."""
+        d_half = x.shape[-1] // 2
+        pos = positions.clamp(0, _ROPE_POSITIONS - 1)
+        sin = self.rope_sin[pos][..., None, :]
+        cos = self.rope_cos[pos][..., None, :]
+        x32 = x.to(torch.float32)
+        a, b = x32[..., :d_half], x32[..., d_half:]
+        return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1).to(x.dtype)
+
+    # ------------------------------------------------------------------ vision + prefix
+    def embed_image(self, image: torch.Tensor) -> torch.Tensor:
+        """``[1, 3, H, W]`` in [-1, 1] -> ``[1, 64, hidden]`` bf16 (vision.py; plain torch)."""
+        cfg = self.cfg.vlm_config
+        v = cfg.vision_config
+        p = self.p
+        b = image.shape[0]
+        ps = v.patch_size
+        n_h, n_w = image.shape[2] // ps, image.shape[3] // ps
+        # non-overlapping patch convolution as one GEMM over unfolded patches
+        x = image.to(BF16).view(b, 3, n_h, ps, n_w, ps).permute(0, 2, 4, 1, 3, 5).reshape(b, n_h * n_w, 3 * ps * ps)
+        x = F.linear(x, self.patch_w, p[VIS + "embeddings.patch_embedding.bias"])
+        x = x + p[VIS + "embeddings.position_embedding.weight"][self.vis_pos][None]
+        heads = v.num_attention_heads
+        hd = v.hidden_size // heads
+        for i in range(v.num_hidden_layers):
+            lp = f"{VIS}encoder.layers.{i}."
+            h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], v.layer_norm_eps)
+            q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
+            k = self.lin(lp + "self_attn.k_proj", h).view(b, -1, heads, hd).transpose(1, 2)
+            val = self.lin(lp + "self_attn.v_proj", h).view(b, -1, heads, hd).transpose(1, 2)
+            att = torch.softmax(torch.matmul(q, k.transpose(2, 3)).float() * hd**-0.5, dim=-1).to(val.dtype)
+            a = torch.matmul(att, val).transpose(1, 2).reshape(b, -1, v.hidden_size)
+            x = x + self.lin(lp + "self_attn.out_proj", a)
+            h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
+            x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
+        x = F.layer_norm(x, (v.hidden_size,), p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], v.layer_norm_eps)
+        s = cfg.scale_factor
+        seq, dim = x.shape[1], x.shape[2]
+        side = int(seq**0.5)
+        x = x.view(b, side, side, dim).view(b, side, side // s, dim * s).permute(0, 2, 1, 3)
+        x = x.reshape(b, side // s, side // s, dim * s * s).permute(0, 2, 1, 3).reshape(b, seq // (s * s), dim * s * s)
+        return self.lin(CONNECTOR, x)
+
+    def embed_prefix(self, images, img_masks, lang_tokens, lang_masks, state):
+        """-> ``(embs fp32 [1,P,hidden], pad_masks bool [1,P], att_masks bool [1,P])`` (flow_matching.py:160-257)."""
+        embs, pads = [], []
+        for img, m in zip(images, img_masks):
+            e = self.embed_image(img) * self.img_scale
+            embs.append(e)
+            pads.append(m[:, None].expand(e.shape[0], e.shape[1]))
+        lang = F.embedding(lang_tokens, self.p[TXT + "embed_tokens.weight"])
+        lang = lang * math.sqrt(lang.shape[-1])
+        embs.append(lang)
+        pads.append(lang_masks)
+        st = self.lin("state_proj", state)[:, None, :]
+        embs.append(st)
+        pads.append(torch.ones(st.shape[0], 1, dtype=torch.bool, device=self.device))
+        embs = torch.cat(embs, dim=1)
+        pads = torch.cat(pads, dim=1)
+        att = torch.zeros(pads.shape, dtype=torch.bool, device=self.device)
+        att[:, -1] = True  # image / language tokens do not attend to the state token
+        return embs, pads, att
+
+    @staticmethod
+    def make_att_2d_masks(pad_masks: torch.Tensor, att_masks: torch.Tensor) -> torch.Tensor:
+        c = torch.cumsum(att_masks, dim=1)
+        return (c[:, None, :] <= c[:, :, None]) & (pad_masks[:, None, :] & pad_masks[:, :, None])
+
+    def _layer_tail(self, prefix: str, mlp: GatedMLP, att_out: torch.Tensor, hidden: torch.Tensor) -> torch.Tensor:
+        out = self.lin(prefix + "self_attn.o_proj", att_out.to(BF16))
+        out += hidden  # first residual; downcasts an fp32 hidden exactly like the reference's in-place add
+        h = rms_norm(out, self.p[prefix + "post_attention_layernorm.weight"], self.eps)
+        return mlp(h, out)
+
+    def prefill(self, embs, pad_masks, att_masks):
+        """VLM prefill -> ``(K, V)`` bf16 ``[layers, 1, P, G, D]`` (post-RoPE prefix cache)."""
+        mask = self.make_att_2d_masks(pad_masks, att_masks)
+        pos = torch.cumsum(pad_masks, dim=1) - 1
+        b, length = embs.shape[0], embs.shape[1]
+        keys = torch.empty(self.num_layers, b, length, self.kv_heads, self.head_dim, dtype=BF16, device=self.device)
+        values = torch.empty_like(keys)
+        hidden = embs
+        for i in range(self.num_layers):
+            lp = f"{TXT}layers.{i}."
+            h = rms_norm(hidden, self.p[lp + "input_layernorm.weight"], self.eps).to(BF16)
+            q = self.rope(self.lin(lp + "self_attn.q_proj", h).view(b, length, -1, self.head_dim), pos)
+            k = self.rope(self.lin(lp + "self_attn.k_proj", h).view(b, length, -1, self.head_dim), pos)
+            v = self.lin(lp + "self_attn.v_proj", h).view(b, length, -1, self.head_dim)
+            keys[i].copy_(k)
+            values[i].copy_(v)
+            att = eager_attention(mask, q, k, v)
+            hidden = self._layer_tail(lp, self.vlm_mlp[i], att, hidden)
+        return keys, values
+
+    def expert_prefix_kv(self, keys, values):
+        """fp32 expert K/V projections of the prefix for the cross layers (flow_matching.py:553-578)."""
+        out = {}
+        for i in range(self.num_layers):
+            if not self.cfg.is_cross_layer(i):
+                continue
+            lp = f"{EXP}layers.{i}.self_attn."
+            b, length = keys.shape[1], keys.shape[2]
+            ek = self.lin(lp + "k_proj", keys[i].float().reshape(b, length, -1)).view(b, length, -1, self.head_dim)
+            ev = self.lin(lp + "v_proj", values[i].float().reshape(b, length, -1)).view(b, length, -1, self.head_dim)
+            out[i] = (ek, ev)
+        return out
+
+    # ------------------------------------------------------------------ denoising
+    def embed_suffix(self, x_t: torch.Tensor, time_emb: torch.Tensor) -> torch.Tensor:
+        a = self.lin("action_in_proj", x_t)
+        te = time_emb[:, None, :].expand_as(a)
+        h = self.lin("action_time_mlp_in", torch.cat([a, te], dim=2))
+        return self.lin("action_time_mlp_out", F.silu(h))
+
+    def denoise_step(self, prefix_pad, keys, values, ekv, x_t, time_emb):
+        """Velocity ``v_t`` fp32 ``[1, chunk, max_action_dim]`` (flow_matching.py:316-350)."""
+        hidden = self.embed_suffix(x_t, time_emb)
+        b, s = hidden.shape[0], hidden.shape[1]
+        p_len = prefix_pad.shape[1]
+        pos = prefix_pad.sum(dim=-1)[:, None] + torch.arange(s, device=self.device)[None, :]
+        pos0 = pos - pos.min(dim=1, keepdim=True).values
+        if not self.fused_expert:
+            causal = torch.ones(s, s, dtype=torch.bool, device=self.device).tril()[None]
+            full_mask = torch.cat([prefix_pad[:, None, :].expand(b, s, p_len), causal], dim=2)
+        for i in range(self.num_layers):
+            lp = f"{EXP}layers.{i}."
+            h = rms_norm(hidden, self.p[lp + "input_layernorm.weight"], self.eps).to(BF16)
+            q = self.lin(lp + "self_attn.q_proj", h).view(b, s, -1, self.head_dim)
+            if not self.cfg.is_cross_layer(i):
+                k = self.rope(self.lin(lp + "self_attn.k_proj", h).view(b, s, -1, self.head_dim), pos)
+                v = self.lin(lp + "self_attn.v_proj", h).view(b, s, -1, self.head_dim)
+                q = self.rope(q, pos)
+                if self.fused_expert:
+                    att = tk.expert_attn(q[0], keys[i, 0], values[i, 0], k[0], v[0], prefix_pad[0], tk.MASK_CAUSAL, ws=self.ws)[None]
+                else:
+                    att = eager_attention(full_mask, q, torch.cat([keys[i], k], dim=1), torch.cat([values[i], v], dim=1))
+            else:
+                q = self.rope(q, pos0)
+                ek, ev = ekv[i]
+                if self.fused_expert:
+                    att = tk.expert_attn(q[0], ek[0], ev[0], None, None, prefix_pad[0], tk.MASK_NONE, ws=self.ws)[None]
+                else:
+                    att = eager_attention(prefix_pad[:, None, :].expand(b, s, p_len), q, ek, ev)
+            hidden = self._layer_tail(lp, self.exp_mlp[i], att, hidden)
+        out = rms_norm(hidden, self.p[EXP + "norm.weight"], self.eps)
+        return self.lin("action_out_proj", out.to(torch.float32))
+
+    def sample_actions_core(self, embs, pads, att, noise, trace: dict | None = None) -> torch.Tensor:
+        keys, values = self.prefill(embs, pads, att)
+        ekv = self.expert_prefix_kv(keys, values)
+        if trace is not None:
+            trace.update(prefix_embs=embs, pad_masks=pads, keys=keys, values=values, ekv=ekv)
+        dt = -1.0 / self.num_steps
+        x_t = noise
+        for step in range(self.num_steps):
+            v_t = self.denoise_step(pads, keys, values, ekv, x_t, self.time_embs[step])
+            x_t = x_t + dt * v_t
+        return x_t
+
+    def sample_actions(self, images, img_masks, lang_tokens, lang_masks, state, noise, trace: dict | None = None) -> torch.Tensor:
+        """Prefix embed, prefill, expert prefix KV, Euler loop -> ``[1, chunk, max_action_dim]`` fp32."""
+        embs, pads, att = self.embed_prefix(images, img_masks, lang_tokens, lang_masks, state)
+        return self.sample_actions_core(embs, pads, att, noise, trace)
