@@ -1,0 +1,257 @@
+"""Benchmark of the fp8 action-inference hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one ``predict_action_chunk`` request of the SmolVLA-shaped policy (random init, 16+16
+layers, 3 cameras, 10 Euler steps, zero noise, fp8 MLP weights, HIP attention, hipGraph) with the
+observation already resident in HBM.  ``value`` is the p50 latency over the K timed requests.
+
+The same JSON line carries
+* ``roofline``      -- the fp8-weight GEMM at the sweep's largest weight-streaming shape
+  (M=50, K=2048, N=16384): algorithmic bytes / average launch duration, measured with events on
+  the launching stream over a graph of back-to-back launches that rotate through > 1 GB of
+  distinct weight copies (cold HBM);
+* ``cpu_baseline``  -- the CPU oracle (a torch restatement of the reference's eager path) timed on
+  the host cores for one request of the same workload;
+* extra fields: 2-camera and pi0.5-shaped p50, the GEMM sweep, the PCIe-inclusive latency.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+GEMM_SHAPES = ((960, 2560), (720, 2048), (2048, 16384), (16384, 2048), (2048, 2048))  # (K, N)
+
+
+def bytes_gemm(m: int, k: int, n: int) -> int:
+    return k * n + 4 * n + 2 * m * k + 2 * m * n
+
+
+def spin_up(ms: float = 150.0) -> None:
+    """Keep the GPU busy long enough for its clocks to leave the idle state."""
+    import torch
+
+    a = torch.randn(4096, 4096, device="cuda", dtype=torch.bfloat16)
+    t0 = time.time()
+    while (time.time() - t0) * 1e3 < ms:
+        for _ in range(10):
+            a @ a
+        torch.cuda.synchronize()
+
+
+def gemm_launch_us(m: int, k: int, n: int, launches: int = 100, reps: int = 10, cold: bool = True) -> float:
+    """Average duration (us) of one fp8-weight GEMM launch inside a replayed graph."""
+    import torch
+
+    from tybok_amd import ops as tk
+    from tybok_amd.quant import quantize_weight_rows
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16).cuda()
+    w8, s = quantize_weight_rows(torch.randn(n, k, generator=g) * 0.02)
+    base = tk.pack_fp8_weight(w8.cuda(), s.cuda())
+    copies = max(2, int(1.1e9 // (k * n))) if cold else 1
+    pws = [base] + [tk.PackedWeight(base.data.clone(), base.scale, base.n, base.k) for _ in range(copies - 1)]
+    out = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(3):
+            tk.fp8w_gemm(x, pws[i % copies], out=out)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    # the engines capture under inference_mode; capturing outside it afterwards trips torch's
+    # graph-safe RNG state (an in-place update of an inference tensor)
+    with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
+        for i in range(launches):
+            tk.fp8w_gemm(x, pws[i % copies], out=out)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * launches)
+
+
+def device_frame(engine, cameras: int, seed: int = 0) -> dict:
+    """Synthetic observation (uint8-valued images / 255, random state) already on the GPU."""
+    import torch
+
+    spec = engine.describe()
+    g = torch.Generator().manual_seed(seed)
+    w, h = spec["resize"]
+    images = {cam: (torch.randint(0, 256, (3, h, w), generator=g, dtype=torch.uint8).float() / 255.0) for cam in spec["cameras"][:cameras]}
+    state = torch.randn(6 if spec["model_type"] == "smolvla" else 8, generator=g)
+    frame = engine.make_frame(images, state, "pick up the cube")
+    return {k: (v.cuda() if hasattr(v, "cuda") else v) for k, v in frame.items()}
+
+
+def time_requests(engine, frame, noise, steps: int, warmup: int) -> tuple[list[float], float]:
+    import torch
+
+    for _ in range(warmup):
+        engine.predict_action_chunk(frame, noise=noise)
+    torch.cuda.synchronize()
+    samples = []
+    t_start = time.perf_counter()
+    for _ in range(steps):
+        t0 = time.perf_counter()
+        engine.predict_action_chunk(frame, noise=noise)
+        torch.cuda.synchronize()
+        samples.append((time.perf_counter() - t0) * 1e3)
+    total_ms = (time.perf_counter() - t_start) * 1e3
+    return samples, total_ms
+
+
+def cpu_baseline_smolvla(cameras: int) -> dict:
+    """One request of the benchmark workload on the host cores through the CPU oracle."""
+    import torch
+
+    from oracle import smolvla as O
+    from tybok_amd.policies.smolvla.config import SmolVLAConfig, VLMConfig
+    from tybok_amd.policies.smolvla.weights import random_state_dict
+
+    cfg = SmolVLAConfig(vlm_config=VLMConfig(), image_features=[f"observation.images.camera{i + 1}" for i in range(cameras)])
+    sd = random_state_dict(cfg, seed=0)
+    shape = O.SmolVLAShape()
+    w = O.Weights(sd, O.fp8_linear_names(shape, True, True))
+    g = torch.Generator().manual_seed(0)
+    images = [torch.randint(0, 256, (1, 3, 512, 512), generator=g, dtype=torch.uint8).float() / 255.0 for _ in range(cameras)]
+    tokens = torch.randint(0, shape.vocab, (1, shape.tok_len), generator=g)
+    state = torch.zeros(1, shape.max_state_dim)
+    noise = torch.zeros(1, shape.chunk, shape.max_action_dim)
+    masks = [torch.ones(1, dtype=torch.bool)] * cameras
+    t0 = time.perf_counter()
+    with torch.no_grad():
+        O.sample_actions(w, shape, O.prepare_images(images), masks, tokens, torch.ones(1, shape.tok_len, dtype=torch.bool), state, noise)
+    ms = (time.perf_counter() - t0) * 1e3
+    return {
+        "value": round(ms, 1),
+        "unit": "ms",
+        "cores": int(torch.get_num_threads()),
+        "kind": "port",
+        "sample": f"1 predict_action_chunk of the same SmolVLA-shaped workload ({cameras} cameras, 10 steps, fp8 MLP weights), CPU oracle, no warm-up",
+    }
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--skip-pi05", action="store_true")
+    ap.add_argument("--skip-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path is batch-1 and single-device (--gpus must be 1)")
+
+    import torch
+
+    from tybok_amd.policies.synthetic import write_pi05_checkpoint, write_smolvla_checkpoint
+    from tybok_amd.registry import create_engine
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True)
+    tmp = tempfile.mkdtemp(prefix="tybok_bench_")
+
+    # ---- SmolVLA-shaped chunk (headline) ----
+    ckpt = write_smolvla_checkpoint(os.path.join(tmp, "smolvla"), cameras=3, seed=0)
+    engine = create_engine(ckpt, device="cuda", graph=True, graph_cameras=(2, 3), warmup=True, **flags)
+    noise = torch.zeros(1, 50, 6, device="cuda")
+    spin_up()
+    frame3 = device_frame(engine, 3)
+    samples3, total_ms = time_requests(engine, frame3, noise, args.steps, args.warmup)
+    frame2 = device_frame(engine, 2)
+    samples2, _ = time_requests(engine, frame2, noise, max(5, args.steps // 2), 2)
+    host_frame = {k: (v.cpu() if hasattr(v, "cpu") else v) for k, v in frame3.items()}
+    samples_host, _ = time_requests(engine, host_frame, noise.cpu(), max(5, args.steps // 2), 2)
+    graph_ok = bool(engine.graph_enabled)
+    del engine
+    torch.cuda.empty_cache()
+
+    # ---- pi0.5-shaped chunk ----
+    pi05_p50 = None
+    if not args.skip_pi05:
+        ckpt5 = write_pi05_checkpoint(os.path.join(tmp, "pi05"), cameras=2, seed=0)
+        eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **flags)
+        frame5 = device_frame(eng5, 2)
+        s5, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
+        pi05_p50 = float(np.percentile(s5, 50))
+        del eng5
+        torch.cuda.empty_cache()
+
+    # ---- fp8 GEMM roofline (dominant weight-streaming kernel) + sweep ----
+    spin_up()
+    sweep = {}
+    for k, n in GEMM_SHAPES:
+        us = gemm_launch_us(50, k, n)
+        sweep[f"K{k}_N{n}"] = {"us": round(us, 2), "GBps": round(bytes_gemm(50, k, n) / us / 1e3, 1)}
+    rk, rn = 2048, 16384
+    r_us = sweep[f"K{rk}_N{rn}"]["us"]
+    achieved = bytes_gemm(50, rk, rn) / r_us / 1e3
+    roofline = {
+        "bound": "hbm",
+        "kernel": "fp8w_gemm_kernel (M=50, K=2048, N=16384, cold weights)",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "bytes_per_launch": bytes_gemm(50, rk, rn),
+        "us_per_launch": r_us,
+    }
+    traffic_file = os.path.join(ROOT, "profiles", "fp8w_gemm_traffic.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file, encoding="utf-8") as f:
+            roofline["traffic"] = json.load(f).get("hbm_bytes_per_launch")
+
+    cpu = None if args.skip_cpu else cpu_baseline_smolvla(3)
+
+    p50 = float(np.percentile(samples3, 50))
+    line = {
+        "metric": "p50 predict_action_chunk latency (ms) + fp8 GEMM achieved HBM GB/s vs peak",
+        "value": round(p50, 3),
+        "unit": "ms",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(total_ms / args.steps, 3),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 activations x fp8-e4m3 weights, fp32 accumulate",
+        "data": "synthetic (random-init weights, uniform-noise images, random token ids, zero noise)",
+        "config": {
+            "workload": "SmolVLA-shaped predict_action_chunk: 16+16 layers, 3 cameras 512x512, 48 tokens, chunk 50, 10 Euler steps, fp8 MLP weights, hipGraph",
+            "inputs": "HBM-resident observation",
+            "graph": graph_ok,
+        },
+        "p95_ms": round(float(np.percentile(samples3, 95)), 3),
+        "smolvla_2cam_p50_ms": round(float(np.percentile(samples2, 50)), 3),
+        "smolvla_3cam_host_inputs_p50_ms": round(float(np.percentile(samples_host, 50)), 3),
+        "pi05_2cam_p50_ms": None if pi05_p50 is None else round(pi05_p50, 3),
+        "gemm_sweep_M50": sweep,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
