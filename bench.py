@@ -155,6 +155,7 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-pi05", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--gemm-only", action="store_true", help="only the roofline GEMM loop plus a plain copy of known size (for rocprofv3 runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is batch-1 and single-device (--gpus must be 1)")
@@ -167,6 +168,16 @@ def main() -> None:
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     torch.cuda.set_device(0)
+    if args.gemm_only:
+        # counter calibration: one device-to-device copy of 256 MiB reads and writes exactly that much
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        spin_up()
+        us = gemm_launch_us(50, 2048, 16384, launches=20, reps=args.steps)
+        print(json.dumps({"gemm_only": {"M": 50, "K": 2048, "N": 16384, "us": round(us, 2), "GBps": round(bytes_gemm(50, 2048, 16384) / us / 1e3, 1)}}), flush=True)
+        return
     flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True)
     tmp = tempfile.mkdtemp(prefix="tybok_bench_")
 
