@@ -113,6 +113,50 @@ int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void
                       int resid_dtype, const void* gate, int M, int K, int I, int act, void* ws,
                       size_t ws_bytes, void* stream);
 
+/* y = tk_fp8w_gated_ffn(rms_norm(x, norm_w, norm_eps), ...): the post-attention RMSNorm runs inside
+ * the gate/up launch while the activations are staged (bf16 x: bf16(w * bf16(x * rstd)), fp32
+ * statistics), as the reference's `triton_norm_gate_up(x, norm_w, eps, gate_w, up_w)` folds it
+ * (tybok/policies/smolvla/models/triton_mlp.py:105-144, call site vlm_with_expert.py:391-408).
+ *   norm_w: bf16 [K], 16-byte aligned.  Other arguments as tk_fp8w_gated_ffn. */
+int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float norm_eps, const void* wgu_packed,
+                           const void* sg, const void* su, const void* wd_packed, const void* sd, void* y, int ldy,
+                           const void* resid, int ldr, int resid_dtype, const void* gate, int M, int K, int I,
+                           int act, void* ws, size_t ws_bytes, void* stream);
+
+/* ---- bf16-weight expert projections (norm prologue, rotary epilogue, residual epilogue) ----- */
+/* Bytes of a packed bf16 [N, K] weight (2 KiB per 32x32 tile). */
+size_t tk_bf16w_packed_bytes(int N, int K);
+/* Row-major bf16 [N, K] -> tile order.  rope_half = 0 keeps the natural n-tile order; rope_half =
+ * head_dim/2 orders the tiles so that each pair of adjacent tiles holds columns (c, c + rope_half)
+ * of one head (2*rope_half must divide N).  Offline, once per weight; the same role as the
+ * reference's `_packed_qkv_interleaved` (tybok/policies/pi05/models/
+ * triton_expert_fused_qkv_rope_attn.py:226-251). */
+int tk_pack_bf16_weight(const void* w, void* packed, int N, int K, int rope_half, void* stream);
+/* y[M, N] (bf16) = epilogue( prologue(x)[M, K] . W[N, K]^T ) with bf16 weights.
+ *   prologue: norm_w == NULL -> x is bf16, used as is.  Otherwise Llama RMSNorm with fp32
+ *             statistics: x bf16 (x_dtype TK_BF16) -> bf16(w * bf16(x * rstd)); x fp32 (TK_F32,
+ *             the first expert layer) -> bf16(w * (x * rstd)).
+ *   epilogue: rope_pos == NULL -> y = bf16(acc) (+ residual: bf16(y + resid), bf16 or fp32 resid)
+ *             -- the o_proj + in-place residual add of a decoder layer
+ *             (tybok/policies/smolvla/models/vlm_with_expert.py:380-389).
+ *             rope_pos != NULL -> half-split rotary embedding on columns < rope_cols: the pair
+ *             (c, c + rope_half) of each head at row m becomes, in fp32 from the bf16-rounded
+ *             projection, (a*cos - b*sin, b*cos + a*sin) with cos/sin = table[pos[m]][c % rope_half],
+ *             rounded to bf16; columns >= rope_cols (the v projection) pass through.  W must have
+ *             been packed with the same rope_half.  One launch for the concatenated q|k|v weight:
+ *             `triton_self_attn`'s norm + q/k/v + RoPE phase and `triton_qkv_rope_fused`
+ *             (tybok/policies/smolvla/models/triton_attn.py:99-172,586-655,
+ *              tybok/policies/pi05/models/triton_expert_fused_qkv_rope_attn.py:254-320;
+ *              eager: tybok/policies/smolvla/models/rope.py:51-73).
+ *   rope_pos: int32 [M] (clamped into [0, rope_positions)); rope_cos/rope_sin: fp32
+ *             [rope_positions, rope_half].
+ * Built for the action-chunk tile shape (any M, tiled 64 rows at a time); the norm prologue is
+ * built together with the rotary epilogue only. */
+int tk_bf16w_linear(const void* x, int ldx, int x_dtype, const void* w_packed, const void* norm_w, float norm_eps,
+                    const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions,
+                    int rope_cols, int rope_half, void* y, int ldy, const void* resid, int ldr, int resid_dtype,
+                    int M, int N, int K, int split_k, void* ws, size_t ws_bytes, void* stream);
+
 /* ---- action-expert attention over the cached prefix ------------------------------------------ */
 /* out[M, H*D] (bf16) = softmax(q.K^T * D^-0.5 + mask) . V over keys [prefix(P); suffix(S)].
  * Replaces `EagerAttention._forward_eager` / `GemmaAttention._forward_eager`'s core and the fused

@@ -1,0 +1,160 @@
+"""GPU parity of the fused expert-layer launches (norm + q|k|v + RoPE, o_proj + residual,
+norm + gated FFN) against compositions of the CPU oracle's ops on seeded inputs.
+
+Tolerance: rtol 2e-2 / atol 2e-2 on bf16 outputs, as for the other op tests.
+"""
+
+import pytest
+import torch
+import torch.nn.functional as F  # noqa: N812
+
+from oracle import ops as oops
+from oracle.inputs import ffn_case
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 2e-2, 2e-2
+BF16 = torch.bfloat16
+
+
+def _close(got, want, what):
+    got, want = got.float().cpu(), want.float().cpu()
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite output"
+    err = (got - want).abs()
+    worst = float((err - (ATOL + RTOL * want.abs())).max())
+    assert worst <= 0, f"{what}: max|err|={float(err.max()):.4g}, exceeds atol+rtol*|ref| by {worst:.4g}"
+
+
+@pytest.fixture(scope="module")
+def tk():
+    from tybok_amd import ops
+
+    return ops
+
+
+def _tables(tk, positions: int, d_half: int, base: float = 10_000.0):
+    # the table the oracle's rope_half_split evaluates per call, for every position
+    exponents = (2.0 / (d_half * 2)) * torch.arange(d_half, dtype=torch.float32)
+    radians = torch.arange(positions, dtype=torch.float32)[:, None] / (base**exponents)[None, :]
+    return tk.RopeTables(torch.cos(radians).cuda(), torch.sin(radians).cuda())
+
+
+def _qkv_case(m, k, heads, kv_heads, d, x_dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    n = (heads + 2 * kv_heads) * d
+    x = torch.randn(m, k, generator=g) * 1.7
+    x = x.to(x_dtype)
+    norm_w = (1.0 + 0.2 * torch.randn(k, generator=g)).to(BF16)
+    w = (torch.randn(n, k, generator=g) * k**-0.5).to(BF16)
+    pos = torch.randint(0, 400, (m,), generator=g, dtype=torch.int32)
+    return x, norm_w, w, pos, n
+
+
+def _qkv_oracle(x, norm_w, w, pos, heads, kv_heads, d, eps):
+    m = x.shape[0]
+    h = x if norm_w is None else oops.rms_norm_llama(x, norm_w, eps).to(BF16)
+    y = F.linear(h, w)
+    rc = (heads + kv_heads) * d
+    qk = oops.rope_half_split(y[:, :rc].reshape(1, m, heads + kv_heads, d), pos[None].long())
+    return torch.cat([qk.reshape(m, rc), y[:, rc:]], dim=1)
+
+
+@pytest.mark.parametrize("x_dtype", [BF16, torch.float32])
+@pytest.mark.parametrize(
+    "m,k,heads,kv_heads,d",
+    [
+        (50, 720, 15, 5, 64),  # SmolVLA expert self-attention layer
+        (50, 1024, 8, 1, 256),  # pi0.5 expert geometry
+        (7, 48, 2, 1, 64),  # tiny, one ragged k tile
+        (100, 720, 15, 5, 64),  # two row blocks
+    ],
+)
+def test_norm_qkv_rope(tk, m, k, heads, kv_heads, d, x_dtype):
+    eps = 1e-5
+    x, norm_w, w, pos, n = _qkv_case(m, k, heads, kv_heads, d, x_dtype, seed=10)
+    want = _qkv_oracle(x, norm_w, w, pos, heads, kv_heads, d, eps)
+    pw = tk.pack_bf16_weight(w.cuda(), rope_half=d // 2)
+    rope = _tables(tk, 512, d // 2)
+    kw = dict(norm_w=norm_w.cuda(), eps=eps, rope=rope, rope_pos=pos.cuda(), rope_cols=(heads + kv_heads) * d)
+    got = tk.bf16w_linear(x.cuda(), pw, **kw)
+    again = tk.bf16w_linear(x.cuda(), pw, **kw)
+    assert torch.equal(got, again), "two launches on the same input differ"
+    _close(got, want, f"norm+qkv+rope M={m} K={k} D={d} x={x_dtype}")
+
+
+def test_qkv_rope_without_norm_and_query_only(tk):
+    # cross layers project queries only (no k/v columns), positions 0..M-1
+    m, k, heads, d = 50, 720, 15, 64
+    x, _, w, _, _ = _qkv_case(m, k, heads, 0, d, BF16, seed=11)
+    pos = torch.arange(m, dtype=torch.int32)
+    want = _qkv_oracle(x, None, w, pos, heads, 0, d, 0.0)
+    pw = tk.pack_bf16_weight(w.cuda(), rope_half=d // 2)
+    got = tk.bf16w_linear(x.cuda(), pw, rope=_tables(tk, 64, d // 2), rope_pos=pos.cuda(), rope_cols=heads * d)
+    _close(got, want, "q+rope")
+
+
+def test_rope_positions_are_clamped_into_the_table(tk):
+    m, k, heads, d = 8, 64, 1, 64
+    x, _, w, _, _ = _qkv_case(m, k, heads, 0, d, BF16, seed=12)
+    pos = torch.tensor([-5, 0, 3, 15, 16, 99, 7, 1], dtype=torch.int32)
+    want = _qkv_oracle(x, None, w, pos.clamp(0, 15), heads, 0, d, 0.0)
+    pw = tk.pack_bf16_weight(w.cuda(), rope_half=d // 2)
+    got = tk.bf16w_linear(x.cuda(), pw, rope=_tables(tk, 16, d // 2), rope_pos=pos.cuda(), rope_cols=d)
+    _close(got, want, "clamped positions")
+
+
+@pytest.mark.parametrize("resid_dtype", [None, BF16, torch.float32])
+@pytest.mark.parametrize("m,k,n", [(50, 960, 720), (50, 2048, 1024), (9, 80, 40), (130, 960, 720)])
+def test_o_proj_residual(tk, m, k, n, resid_dtype):
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(m, k, generator=g).to(BF16)
+    w = (torch.randn(n, k, generator=g) * k**-0.5).to(BF16)
+    want = F.linear(x, w)
+    resid = None
+    if resid_dtype is not None:
+        resid = torch.randn(m, n, generator=g).to(resid_dtype)
+        want += resid  # in-place: an fp32 residual is added in fp32 and rounded to bf16 once
+    pw = tk.pack_bf16_weight(w.cuda())
+    got = tk.bf16w_linear(x.cuda(), pw, resid=None if resid is None else resid.cuda())
+    _close(got, want, f"o_proj M={m} K={k} N={n} resid={resid_dtype}")
+    for split in (1, 3):
+        forced = tk.bf16w_linear(x.cuda(), pw, resid=None if resid is None else resid.cuda(), split_k=split)
+        _close(forced, want, f"o_proj split_k={split}")
+
+
+@pytest.mark.parametrize("act,m,k,i", [("silu", 50, 720, 2048), ("gelu_tanh", 50, 1024, 4096), ("silu", 1, 720, 2048)])
+def test_norm_gated_ffn(tk, act, m, k, i):
+    eps = 1e-5
+    x, wg8, sg, wu8, su, wd8, sd = ffn_case(m, k, i, seed=14)
+    g = torch.Generator().manual_seed(15)
+    x = (x.float() * 2.5).to(BF16)
+    norm_w = (1.0 + 0.2 * torch.randn(k, generator=g)).to(BF16)
+    resid = torch.randn(m, k, generator=g).to(BF16)
+    want = oops.gated_ffn(oops.rms_norm_llama(x, norm_w, eps), wg8, sg, wu8, su, wd8, sd, act)
+    want += resid
+    wgu = tk.pack_fp8_gate_up(wg8.cuda(), sg, wu8.cuda(), su)
+    wd = tk.pack_fp8_weight(wd8.cuda(), sd)
+    got = tk.fp8w_gated_ffn(x.cuda(), wgu, wd, act, resid=resid.cuda(), norm_w=norm_w.cuda(), eps=eps)
+    _close(got, want, f"norm+ffn {act} M={m}")
+    # the fused norm must equal normalising first and calling the plain entry point, bit for bit
+    # (same rounding points, same GEMM)
+    h = oops.rms_norm_llama(x, norm_w, eps).cuda()
+    two_step = tk.fp8w_gated_ffn(h, wgu, wd, act, resid=resid.cuda())
+    mism = (got != two_step).float().mean().item()
+    assert mism < 0.02, f"fused norm differs from norm-then-FFN on {mism:.1%} of the outputs"
+
+
+def test_fused_layer_argument_checks(tk):
+    w = torch.zeros(128, 64, dtype=BF16, device="cuda")
+    x = torch.zeros(4, 64, dtype=BF16, device="cuda")
+    pw_rope = tk.pack_bf16_weight(w, rope_half=32)
+    with pytest.raises(ValueError):
+        tk.bf16w_linear(x, pw_rope)  # pair-ordered weight without the rotary epilogue
+    with pytest.raises(TypeError):
+        tk.bf16w_linear(x.float(), tk.pack_bf16_weight(w))  # fp32 input without a norm
+    with pytest.raises(RuntimeError):
+        tk.pack_bf16_weight(torch.zeros(96, 64, dtype=BF16, device="cuda"), rope_half=32)  # 64 does not divide 96
+    rope = _tables(tk, 16, 32)
+    with pytest.raises(RuntimeError):
+        tk.bf16w_linear(x, pw_rope, rope=rope, rope_pos=torch.zeros(4, dtype=torch.int32, device="cuda"), rope_cols=32)

@@ -28,20 +28,33 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-template <int MT, int NT, int NW, bool GATED, int PF, int TPW>
+// EPI: 0 plain (scale, optional per-column gate, optional residual), 1 gated (gate/up tile pairs ->
+//      act(g)*u), 2 rope (tile pairs hold columns (i, i + D/2) of one head -> rotary embedding).
+// W16: weights are bf16 (two 16-byte operand chunks per lane and k tile) instead of e4m3.
+// PRO: 0 none, 1 RMSNorm of bf16 activations, 2 RMSNorm of fp32 activations -- applied while the
+//      activations are staged into LDS, with the reference's rounding points:
+//      bf16 input: bf16(w * bf16(x * rstd));  fp32 input: bf16(w * (x * rstd)).
+template <int MT, int NT, int NW, int EPI, int PF, int TPW, bool W16, int PRO>
 __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
+  constexpr bool GATED = EPI == 1;
+  constexpr bool PAIRED = EPI != 0;  // both n tiles of a pair are finished by the same wave
+  constexpr bool XF32 = PRO == 2;
   constexpr int TILES = MT * NT;
   constexpr int RKT = NW * TPW;               // k tiles per block round
-  constexpr int ROWB = RKT * 64;              // bytes of one activation row per round
+  constexpr int ROWB = RKT * 64;              // bytes of one staged (bf16) activation row per round
   constexpr int PITCH = ROWB + 16;            // LDS row pitch (bytes), keeps 16-byte alignment
   constexpr int ROWS = MT * 32;
   constexpr int XBUF = ROWS * PITCH;          // bytes per staging buffer
-  constexpr int PPR = ROWB / 16;              // 16-byte pieces per row
+  constexpr int PPR = ROWB / 16;              // 8-element pieces per row
   constexpr int XPT = ROWS * PPR / (NW * 64); // pieces per thread and round
   constexpr int RED_BYTES = 2 * NW * 16 * 64 * 4;
   constexpr int LDS_BYTES = 2 * XBUF > RED_BYTES ? 2 * XBUF : RED_BYTES;
+  constexpr int WCH = W16 ? 2 : 1;            // 16-byte operand chunks per lane, n tile and k tile
+  constexpr int WTILE = W16 ? 2048 : 1024;    // bytes of one packed 32x32 tile
   static_assert(ROWS * PPR % (NW * 64) == 0, "staging pieces must divide evenly");
+  static_assert(!PAIRED || NT == 2, "paired epilogues need two n tiles per strip");
   __shared__ __align__(16) unsigned char lds[LDS_BYTES];
+  __shared__ float rstd_s[ROWS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -64,30 +77,32 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   for (int nt = 0; nt < NT; ++nt) {
     int ntg = strip * NT + nt;
     if (ntg > a.ntiles - 1) ntg = a.ntiles - 1;
-    wbase[nt] = a.w + ((size_t)ntg * a.KT) * 1024 + lane * 16;
+    wbase[nt] = a.w + ((size_t)ntg * a.KT) * WTILE + lane * 16;
   }
 
-  // staging pieces of this thread: piece p -> (row p / PPR, 16-byte column p % PPR).  Rows >= M
+  // staging pieces of this thread: piece p -> (row p / PPR, 8-element column p % PPR).  Rows >= M
   // are clamped to M-1 (an output row depends only on its own activation row; rows >= M are
   // never stored).
-  const u16* xsrc[XPT];
+  const char* xsrc[XPT];
   int xcol[XPT];   // first element (k index) of the piece within a round
   int xdst[XPT];   // LDS byte offset within a staging buffer
+  int xrow[XPT];
 #pragma unroll
   for (int i = 0; i < XPT; ++i) {
     const int p = tid + i * NW * 64;
     const int r = p / PPR, c = p % PPR;
     int m = mblock * ROWS + r;
     if (m > a.M - 1) m = a.M - 1;
-    xsrc[i] = a.x + (size_t)m * a.ldx;
+    xsrc[i] = (const char*)a.x + (size_t)m * a.ldx * (XF32 ? 4 : 2);
     xcol[i] = c * 8;
     xdst[i] = r * PITCH + c * 16;
+    xrow[i] = r;
   }
 
   // scales of the columns this wave will finish, fetched before the loop so the epilogue does not
   // start with a cold miss
-  float sc_pre[2] = {0.f, 0.f};
-  {
+  float sc_pre[2] = {1.f, 1.f};
+  if (!W16) {
     const int n0 = GATED ? (strip * NT / 2) * 32 + l32 : strip * NT * 32 + l32;
     if (!GATED) {
 #pragma unroll
@@ -110,7 +125,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
 
   struct WFrag {
-    i32x4 w[TPW][NT];
+    i32x4 w[TPW][NT][WCH];
   };
   auto wload = [&](WFrag& f, int r) {
 #pragma unroll
@@ -118,11 +133,14 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       int kt = kt_lo + r * RKT + wave * TPW + j;
       if (kt > a.KT - 1) kt = a.KT - 1;
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) f.w[j][nt] = *(const i32x4*)(wbase[nt] + (size_t)kt * 1024);
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int c = 0; c < WCH; ++c) f.w[j][nt][c] = *(const i32x4*)(wbase[nt] + (size_t)kt * WTILE + c * 1024);
     }
   };
   struct XFrag {
-    i32x4 v[XPT];
+    i32x4 v[XPT][XF32 ? 2 : 1];
+    i32x4 nw[PRO ? XPT : 1];  // norm weights of the piece's 8 columns
   };
   auto xload = [&](XFrag& f, int r) {
     const int k0 = (kt_lo + r * RKT) * 32;
@@ -130,16 +148,53 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     for (int i = 0; i < XPT; ++i) {
       int k = k0 + xcol[i];
       if (k > a.K - 8) k = a.K - 8;  // keep the address inside the row; the value is dropped below
-      f.v[i] = *(const i32x4*)(xsrc[i] + k);
+      if (XF32) {
+        const i32x4* p = (const i32x4*)(xsrc[i] + (size_t)k * 4);
+        f.v[i][0] = p[0];
+        f.v[i][XF32 ? 1 : 0] = p[1];
+      } else {
+        f.v[i][0] = *(const i32x4*)(xsrc[i] + (size_t)k * 2);
+      }
+      if (PRO) f.nw[i] = *(const i32x4*)(a.norm_w + k);
     }
   };
+  float my_rstd[XPT];
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) my_rstd[i] = 1.f;
   auto xstore = [&](const XFrag& f, int r, int b) {
     const int k0 = (kt_lo + r * RKT) * 32;
     const i32x4 z = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < XPT; ++i) {
       const bool ok = (k0 + xcol[i]) < k_end;
-      *(i32x4*)(lds + b * XBUF + xdst[i]) = ok ? f.v[i] : z;
+      i32x4 out;
+      if (PRO == 0) {
+        out = f.v[i][0];
+      } else {
+        union { i32x4 v; u16 h[8]; } nwu, o;
+        nwu.v = f.nw[i];
+        float xv[8];
+        if (XF32) {
+          union { i32x4 v; float f[4]; } lo, hi;
+          lo.v = f.v[i][0];
+          hi.v = f.v[i][XF32 ? 1 : 0];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { xv[e] = lo.f[e]; xv[4 + e] = hi.f[e]; }
+        } else {
+          union { i32x4 v; u16 h[8]; } xu;
+          xu.v = f.v[i][0];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) xv[e] = bf16_bits_to_f32(xu.h[e]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float n = xv[e] * my_rstd[i];
+          if (!XF32) n = round_bf16(n);
+          o.h[e] = f32_to_bf16_bits(bf16_bits_to_f32(nwu.h[e]) * n);
+        }
+        out = o.v;
+      }
+      *(i32x4*)(lds + b * XBUF + xdst[i]) = ok ? out : z;
     }
   };
   auto compute = [&](const WFrag& f, int b) {
@@ -155,8 +210,13 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       bf16x8 wb[NT][2];
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        wb[nt][0] = fp8x8_to_bf16x8(f.w[j][nt][0], f.w[j][nt][1]);
-        wb[nt][1] = fp8x8_to_bf16x8(f.w[j][nt][2], f.w[j][nt][3]);
+        if (W16) {
+          wb[nt][0] = as_bf16x8(f.w[j][nt][0]);
+          wb[nt][1] = as_bf16x8(f.w[j][nt][W16 ? 1 : 0]);
+        } else {
+          wb[nt][0] = fp8x8_to_bf16x8(f.w[j][nt][0][0], f.w[j][nt][0][1]);
+          wb[nt][1] = fp8x8_to_bf16x8(f.w[j][nt][0][2], f.w[j][nt][0][3]);
+        }
       }
 #pragma unroll
       for (int h2 = 0; h2 < 2; ++h2)
@@ -172,18 +232,48 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   // are requested together (memory returns in order, so waiting for one means waiting for
   // everything requested before it).  The steady-state loop runs while a whole group of PF rounds
   // can prefetch and has no branch, so the compiler keeps precise vmcnt waits; the tail (at most
-  // 2*PF-1 rounds) uses block-uniform conditions and requests nothing that is not consumed (a
-  // redundant request would have to be waited for at the first barrier after the loop).
-  if (nrounds > 0) {
-    WFrag wbuf[PF];
-    XFrag xbuf[PF];
+  // 2*PF-1 rounds) uses block-uniform conditions and requests nothing that is not consumed.
+  WFrag wbuf[PF];
+  XFrag xbuf[PF];
 #pragma unroll
-    for (int p = 0; p < PF; ++p) {
-      if (p < nrounds) {
-        xload(xbuf[p], p);
-        wload(wbuf[p], p);
+  for (int p = 0; p < PF; ++p) {
+    if (p < nrounds) {
+      xload(xbuf[p], p);
+      wload(wbuf[p], p);
+    }
+  }
+  if (PRO) {
+    // per-row 1/rms over the whole K (every block needs it for its rows, whatever its k range)
+    constexpr int TPR = NW * 64 / ROWS;  // threads per row
+    const int r = tid / TPR, q = tid % TPR;
+    int m = mblock * ROWS + r;
+    if (m > a.M - 1) m = a.M - 1;
+    const char* row = (const char*)a.x + (size_t)m * a.ldx * (XF32 ? 4 : 2);
+    float ss = 0.f;
+#pragma unroll 8
+    for (int p = q; p < a.K / 8; p += TPR) {
+      if (XF32) {
+        const float4* p4 = (const float4*)(row + (size_t)p * 32);
+        float4 u0 = p4[0], u1 = p4[1];
+        ss += u0.x * u0.x + u0.y * u0.y + u0.z * u0.z + u0.w * u0.w + u1.x * u1.x + u1.y * u1.y + u1.z * u1.z + u1.w * u1.w;
+      } else {
+        union { i32x4 v; u16 h[8]; } xu;
+        xu.v = *(const i32x4*)(row + (size_t)p * 16);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float f = bf16_bits_to_f32(xu.h[e]);
+          ss += f * f;
+        }
       }
     }
+#pragma unroll
+    for (int o = TPR / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    if (q == 0) rstd_s[r] = rsqrtf(ss / (float)a.K + a.norm_eps);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) my_rstd[i] = rstd_s[xrow[i]];
+  }
+  if (nrounds > 0) {
     int it = 0;
     for (; it + 2 * PF <= nrounds; it += PF) {
 #pragma unroll
@@ -216,7 +306,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 
   // ---- in-block reduction over waves (fixed order), tile by tile, double-buffered LDS ----
   float (*red)[NW][16][64] = (float (*)[NW][16][64])lds;
-  constexpr int OWN = GATED ? 2 * ((TILES / 2 + NW - 1) / NW) : (TILES + NW - 1) / NW;
+  constexpr int OWN = PAIRED ? 2 * ((TILES / 2 + NW - 1) / NW) : (TILES + NW - 1) / NW;
   float own[OWN][16];
 #pragma unroll
   for (int o = 0; o < OWN; ++o)
@@ -226,8 +316,8 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
     const int mt = t / NT, nt = t % NT;
-    const int owner = GATED ? (t / 2) % NW : t % NW;
-    const int slot = GATED ? ((t / 2) / NW) * 2 + (t & 1) : t / NW;
+    const int owner = PAIRED ? (t / 2) % NW : t % NW;
+    const int slot = PAIRED ? ((t / 2) / NW) * 2 + (t & 1) : t / NW;
     if (NW > 1) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) red[t & 1][wave][i][lane] = acc[mt][nt][i];
@@ -252,8 +342,8 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   if (a.ksplit > 1) {
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-      const int owner = GATED ? (t / 2) % NW : t % NW;
-      const int slot = GATED ? ((t / 2) / NW) * 2 + (t & 1) : t / NW;
+      const int owner = PAIRED ? (t / 2) % NW : t % NW;
+      const int slot = PAIRED ? ((t / 2) / NW) * 2 + (t & 1) : t / NW;
       if (wave == owner) {
         float* dst = a.partial + (((size_t)blk_lin * a.ksplit + split) * TILES + t) * 1024 + lane;
 #pragma unroll
@@ -273,8 +363,8 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     if (!s_last) return;
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-      const int owner = GATED ? (t / 2) % NW : t % NW;
-      const int slot = GATED ? ((t / 2) / NW) * 2 + (t & 1) : t / NW;
+      const int owner = PAIRED ? (t / 2) % NW : t % NW;
+      const int slot = PAIRED ? ((t / 2) / NW) * 2 + (t & 1) : t / NW;
       if (wave == owner) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) own[slot][i] = 0.f;
@@ -290,7 +380,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   }
 
   // ---- epilogue ----
-  if (!GATED) {
+  if (EPI == 0) {
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
       const int mt = t / NT, nt = t % NT;
@@ -298,7 +388,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       const int slot = t / NW;
       const int n = (strip * NT + nt) * 32 + l32;
       if (n >= a.N) continue;
-      const float sc = nt < 2 ? sc_pre[nt < 2 ? nt : 0] : a.s0[n];
+      const float sc = sc_pre[nt < 2 ? nt : 0];
       const float gt = a.gate ? bf16_bits_to_f32(a.gate[n]) : 1.0f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -315,17 +405,17 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
         }
       }
     }
-  } else {
+  } else if (EPI == 1) {
     // tiles come in (gate, up) pairs over the same logical columns
 #pragma unroll
     for (int u = 0; u < TILES / 2; ++u) {
       if (wave != u % NW) continue;
       const int t = 2 * u;
-      const int mt = t / NT, nt = t % NT;
+      const int mt = t / NT;
       const int sg = (u / NW) * 2, su = sg + 1;
-      const int col = ((strip * NT + nt) / 2) * 32 + l32;  // logical column in [0, I)
+      const int col = strip * 32 + l32;  // logical column in [0, I)
       if (col >= a.N) continue;
-      const float scg = nt == 0 ? sc_pre[0] : a.s0[col], scu = nt == 0 ? sc_pre[1] : a.s1[col];
+      const float scg = sc_pre[0], scu = sc_pre[1];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int m = (mblock * MT + mt) * 32 + mfma32_row(lane, i);
@@ -334,6 +424,42 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
           float up = round_bf16(own[su][i] * scu);
           float act = a.act == 0 ? silu_f(g) : gelu_tanh_f(g);
           a.y[(size_t)m * a.ldy + col] = f32_to_bf16_bits(round_bf16(act) * up);
+        }
+      }
+    }
+  } else {
+    // the two tiles of a strip hold columns (c, c + rope_half) of one head: logical tile of
+    // physical tile (strip, j) is (strip / PO) * 2 * PO + strip % PO + j * PO with PO = rope_half / 32
+    const int po = a.rope_half >> 5;
+    const int lt0 = (strip / po) * 2 * po + strip % po;
+    const int ca = lt0 * 32 + l32, cb = ca + a.rope_half;
+    const int fi = ca % (2 * a.rope_half);  // rotary frequency index of the pair
+    const bool rot = ca < a.rope_cols;
+#pragma unroll
+    for (int u = 0; u < TILES / 2; ++u) {
+      if (wave != u % NW) continue;
+      const int mt = (2 * u) / NT;
+      const int sa = (u / NW) * 2, sb = sa + 1;
+      if (cb >= a.N) continue;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = (mblock * MT + mt) * 32 + mfma32_row(lane, i);
+        if (m < a.M) {
+          float va = round_bf16(own[sa][i] * sc_pre[0]);
+          float vb = round_bf16(own[sb][i] * sc_pre[1]);
+          if (rot) {
+            int pos = a.rope_pos[m];
+            pos = pos < 0 ? 0 : (pos > a.rope_positions - 1 ? a.rope_positions - 1 : pos);
+            const float cs = a.rope_cos[(size_t)pos * a.rope_half + fi];
+            const float sn = a.rope_sin[(size_t)pos * a.rope_half + fi];
+            // separately rounded products, as an elementwise fp32 implementation computes them
+            const float ra = __fsub_rn(__fmul_rn(va, cs), __fmul_rn(vb, sn));
+            const float rb = __fadd_rn(__fmul_rn(vb, cs), __fmul_rn(va, sn));
+            va = ra;
+            vb = rb;
+          }
+          a.y[(size_t)m * a.ldy + ca] = f32_to_bf16_bits(va);
+          a.y[(size_t)m * a.ldy + cb] = f32_to_bf16_bits(vb);
         }
       }
     }
@@ -362,6 +488,31 @@ __global__ void pack_kernel(const uint8_t* __restrict__ w0, const uint8_t* __res
   *(i32x4*)(out + c * 16) = v;
 }
 
+// bf16 [N, K] row-major -> 2 KiB tiles: chunk c (0/1) of lane l = 8 bf16 at k = 32*kt + 16*(l/32) + 8*c,
+// stored as [c][lane] so each of the two loads of a tile is one coalesced 1 KiB read.  With
+// pair_off = PO > 0, physical n tile (2p + j) holds logical n tile (p / PO) * 2 * PO + p % PO + j * PO,
+// i.e. the two tiles of a strip hold columns (c, c + 32*PO) -- the rotary pairs of one head.
+__global__ void pack_bf16_kernel(const unsigned short* __restrict__ w, uint8_t* __restrict__ out, int N, int K, int KT,
+                                 long long nchunks, int pair_off) {
+  long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= nchunks) return;
+  const int lane = (int)(c & 63);
+  const int ch = (int)((c >> 6) & 1);
+  const long long tile = c >> 7;
+  const int kt = (int)(tile % KT);
+  const int ntp = (int)(tile / KT);
+  int nt = ntp;
+  if (pair_off > 0) {
+    const int p = ntp >> 1, j = ntp & 1;
+    nt = (p / pair_off) * 2 * pair_off + p % pair_off + j * pair_off;
+  }
+  const int n = nt * 32 + (lane & 31);
+  const int k = kt * 32 + 16 * (lane >> 5) + 8 * ch;
+  i32x4 v = {0, 0, 0, 0};
+  if (n < N && k < K) v = *(const i32x4*)(w + (size_t)n * K + k);
+  *(i32x4*)(out + c * 16) = v;
+}
+
 __global__ void fill_zero_kernel(int* p, int n) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0;
@@ -377,9 +528,9 @@ __global__ void decode_fp8_kernel(float* out) {
   out[c] = bf16_bits_to_f32((u16)(cv.u & 0xffff));
 }
 
-template <int MT, int NT, int NW, bool GATED, int PF>
+template <int MT, int NT, int EPI, bool W16, int PRO>
 int launch(const GemmArgs& a, dim3 grid, hipStream_t st) {
-  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, NW, GATED, PF, 1>), grid, dim3(NW * 64), 0, st, a);
+  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, 4, 1, W16, PRO>), grid, dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
@@ -387,13 +538,38 @@ int launch(const GemmArgs& a, dim3 grid, hipStream_t st) {
 
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st) {
   dim3 grid((a.ntiles + NT - 1) / NT, a.ksplit, mblocks);
-  const bool gated = a.s1 != nullptr;
-  if (gated) {
-    if (NT != 2) return -1;
-    return MT == 1 ? launch<1, 2, 4, true, 4>(a, grid, st) : launch<2, 2, 4, true, 4>(a, grid, st);
+  const int epi = a.s1 != nullptr ? 1 : (a.rope_pos != nullptr ? 2 : 0);
+  const int pro = a.norm_w == nullptr ? 0 : (a.x_f32 ? 2 : 1);
+  if (a.w16) {
+    // bf16-weight linears of the expert layers (M > 32 only: the action chunk)
+    if (MT != 2 || NT != 2) return -1;
+    if (epi == 2) {
+      if (pro == 1) return launch<2, 2, 2, true, 1>(a, grid, st);
+      if (pro == 2) return launch<2, 2, 2, true, 2>(a, grid, st);
+      return launch<2, 2, 2, true, 0>(a, grid, st);
+    }
+    if (epi == 0 && pro == 0) return launch<2, 2, 0, true, 0>(a, grid, st);
+    return -1;
   }
-  if (NT == 1) return MT == 1 ? launch<1, 1, 4, false, 4>(a, grid, st) : launch<2, 1, 4, false, 4>(a, grid, st);
-  return MT == 1 ? launch<1, 2, 4, false, 4>(a, grid, st) : launch<2, 2, 4, false, 4>(a, grid, st);
+  if (epi == 2 || pro == 2) return -1;
+  if (epi == 1) {
+    if (NT != 2) return -1;
+    if (pro == 1) return MT == 1 ? launch<1, 2, 1, false, 1>(a, grid, st) : launch<2, 2, 1, false, 1>(a, grid, st);
+    return MT == 1 ? launch<1, 2, 1, false, 0>(a, grid, st) : launch<2, 2, 1, false, 0>(a, grid, st);
+  }
+  if (pro) return -1;
+  if (NT == 1) return MT == 1 ? launch<1, 1, 0, false, 0>(a, grid, st) : launch<2, 1, 0, false, 0>(a, grid, st);
+  return MT == 1 ? launch<1, 2, 0, false, 0>(a, grid, st) : launch<2, 2, 0, false, 0>(a, grid, st);
+}
+
+int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st) {
+  const int KT = (K + 31) / 32;
+  const int ntiles = (N + 31) / 32;
+  const long long nchunks = (long long)ntiles * KT * 128;
+  const long long blocks = (nchunks + 255) / 256;
+  hipLaunchKernelGGL(pack_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const unsigned short*)w, (uint8_t*)out, N,
+                     K, KT, nchunks, pair_off);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
 int tk_launch_pack(const void* w0, const void* w1, void* out, int N, int K, int interleave, hipStream_t st) {

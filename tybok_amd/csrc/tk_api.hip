@@ -41,23 +41,49 @@ int device_cus() {
   return g_cus;
 }
 
-// One GEMM launch (plain or gated).  `N` is the logical output width.
+// Optional pieces of a GEMM launch beyond y = bf16((x . W^T) * scale).
+struct GemmExtra {
+  int x_f32 = 0;                  // activations are fp32 (norm prologue only)
+  int w16 = 0;                    // bf16 weight tiles
+  const void* norm_w = nullptr;   // RMSNorm prologue
+  float norm_eps = 0.f;
+  const int* rope_pos = nullptr;  // rotary epilogue
+  const float* rope_cos = nullptr;
+  const float* rope_sin = nullptr;
+  int rope_positions = 0, rope_cols = 0, rope_half = 0;
+};
+
+// One GEMM launch (plain, gated or rotary).  `N` is the logical output width.
 int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, const float* s1, void* y, int ldy,
                 const void* resid, int ldr, int resid_dtype, const void* gate, int M, int N, int K, int split_k,
-                int act, void* ws, size_t ws_bytes, hipStream_t st) {
+                int act, void* ws, size_t ws_bytes, hipStream_t st, const GemmExtra& e = GemmExtra()) {
   if (M <= 0 || N <= 0 || K <= 0) return fail(TK_EINVAL, "gemm: non-positive shape M=%d N=%d K=%d", M, N, K);
   if (K % 16) return fail(TK_EINVAL, "gemm: K=%d must be a multiple of 16", K);
   if (ldx % 8 || ldx < K) return fail(TK_EINVAL, "gemm: ldx=%d must be >= K and a multiple of 8", ldx);
   if (ldy < N) return fail(TK_EINVAL, "gemm: ldy=%d < N=%d", ldy, N);
-  if (!x || !w_packed || !s0 || !y) return fail(TK_EINVAL, "gemm: null pointer");
+  if (!x || !w_packed || (!s0 && !e.w16) || !y) return fail(TK_EINVAL, "gemm: null pointer");
   if (!aligned16(x) || !aligned16(w_packed)) return fail(TK_EINVAL, "gemm: x and w_packed must be 16-byte aligned");
   if (resid && resid_dtype != TK_BF16 && resid_dtype != TK_F32) return fail(TK_EINVAL, "gemm: bad resid_dtype");
+  if (resid && ldr < N) return fail(TK_EINVAL, "gemm: ldr=%d < N=%d", ldr, N);
   const bool gated = s1 != nullptr;
+  const bool rope = e.rope_pos != nullptr;
   if (gated && (N % 32)) return fail(TK_EINVAL, "gated gemm: I=%d must be a multiple of 32", N);
+  if (e.x_f32 && !e.norm_w) return fail(TK_EINVAL, "gemm: fp32 activations need the norm prologue");
+  if (e.norm_w && !aligned16(e.norm_w)) return fail(TK_EINVAL, "gemm: norm weight must be 16-byte aligned");
+  if (rope) {
+    if (gated || resid || gate) return fail(TK_EINVAL, "gemm: the rotary epilogue excludes gate/residual epilogues");
+    if (!e.rope_cos || !e.rope_sin || e.rope_positions <= 0) return fail(TK_EINVAL, "gemm: null rotary table");
+    if (e.rope_half < 32 || e.rope_half % 32) return fail(TK_EINVAL, "gemm: rope_half=%d must be a multiple of 32", e.rope_half);
+    if (N % (2 * e.rope_half) || e.rope_cols % (2 * e.rope_half) || e.rope_cols > N)
+      return fail(TK_EINVAL, "gemm: N=%d and rope_cols=%d must be multiples of the head size %d", N, e.rope_cols, 2 * e.rope_half);
+  }
 
   GemmArgs a;
-  a.x = (const u16*)x;
+  memset(&a, 0, sizeof(a));
+  a.x = x;
   a.ldx = ldx;
+  a.x_f32 = e.x_f32;
+  a.w16 = e.w16;
   a.w = (const uint8_t*)w_packed;
   a.s0 = s0;
   a.s1 = s1;
@@ -73,12 +99,24 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   a.KT = (K + 31) / 32;
   a.ntiles = ((N + 31) / 32) * (gated ? 2 : 1);
   a.act = act;
+  a.norm_w = (const u16*)e.norm_w;
+  a.norm_eps = e.norm_eps;
+  a.rope_pos = e.rope_pos;
+  a.rope_cos = e.rope_cos;
+  a.rope_sin = e.rope_sin;
+  a.rope_positions = e.rope_positions;
+  a.rope_cols = e.rope_cols;
+  a.rope_half = e.rope_half;
 
-  const int MT = M <= 32 ? 1 : 2;
-  const int mblocks = (M + 32 * MT - 1) / (32 * MT);
   const int cus = device_cus();
+  int MT = M <= 32 ? 1 : 2;
   int NT = 2;
-  if (!gated && ((a.ntiles + 1) / 2) * mblocks < cus / 2) NT = 1;  // few columns: finer strips
+  if (e.w16) {
+    MT = 2;  // the bf16-weight kernels exist for the action-chunk tile shape only
+  } else if (!gated && ((a.ntiles + 1) / 2) * ((M + 32 * MT - 1) / (32 * MT)) < cus / 2) {
+    NT = 1;  // few columns: finer strips
+  }
+  const int mblocks = (M + 32 * MT - 1) / (32 * MT);
   const int strips = (a.ntiles + NT - 1) / NT;
   const int blocks0 = strips * mblocks;
   const int NW = 4;
@@ -105,6 +143,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
     a.counters = (int*)ws;
   }
   int rc = tk_launch_gemm(a, MT, NT, mblocks, st);
+  if (rc == -1) return fail(TK_EINVAL, "gemm: this combination of weight type, prologue and epilogue is not built");
   if (rc) return fail(TK_ELAUNCH, "gemm: launch failed (%s)", hipGetErrorString(hipGetLastError()));
   return TK_OK;
 }
@@ -173,6 +212,65 @@ int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void
                        act, ws, ws_bytes, (hipStream_t)stream);
   if (rc) return rc;
   // down projection (+ residual)
+  return gemm_common(hbuf, I, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, K, I, 0, 0,
+                     ws, ws_bytes, (hipStream_t)stream);
+}
+
+size_t tk_bf16w_packed_bytes(int N, int K) {
+  if (N <= 0 || K <= 0) return 0;
+  return (size_t)((N + 31) / 32) * ((K + 31) / 32) * 2048;
+}
+
+int tk_pack_bf16_weight(const void* w, void* packed, int N, int K, int rope_half, void* stream) {
+  if (!w || !packed || N <= 0 || K <= 0) return fail(TK_EINVAL, "pack_bf16: bad argument");
+  if (K % 16) return fail(TK_EINVAL, "pack_bf16: K=%d must be a multiple of 16", K);
+  if (!aligned16(w) || !aligned16(packed)) return fail(TK_EINVAL, "pack_bf16: pointers must be 16-byte aligned");
+  if (rope_half && (rope_half % 32 || N % (2 * rope_half)))
+    return fail(TK_EINVAL, "pack_bf16: rope_half=%d must be a multiple of 32 and 2*rope_half divide N=%d", rope_half, N);
+  if (tk_launch_pack_bf16(w, packed, N, K, rope_half / 32, (hipStream_t)stream))
+    return fail(TK_ELAUNCH, "pack_bf16: launch failed");
+  return TK_OK;
+}
+
+int tk_bf16w_linear(const void* x, int ldx, int x_dtype, const void* w_packed, const void* norm_w, float norm_eps,
+                    const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions, int rope_cols,
+                    int rope_half, void* y, int ldy, const void* resid, int ldr, int resid_dtype, int M, int N, int K,
+                    int split_k, void* ws, size_t ws_bytes, void* stream) {
+  if (x_dtype != TK_BF16 && x_dtype != TK_F32) return fail(TK_EINVAL, "bf16w_linear: bad x_dtype");
+  GemmExtra e;
+  e.x_f32 = x_dtype == TK_F32;
+  e.w16 = 1;
+  e.norm_w = norm_w;
+  e.norm_eps = norm_eps;
+  e.rope_pos = (const int*)rope_pos;
+  e.rope_cos = (const float*)rope_cos;
+  e.rope_sin = (const float*)rope_sin;
+  e.rope_positions = rope_positions;
+  e.rope_cols = rope_cols;
+  e.rope_half = rope_half;
+  if (!rope_pos && norm_w) return fail(TK_EINVAL, "bf16w_linear: the norm prologue is built for the rotary projection only");
+  return gemm_common(x, ldx, w_packed, nullptr, nullptr, y, ldy, resid, ldr, resid_dtype, nullptr, M, N, K, split_k, 0, ws,
+                     ws_bytes, (hipStream_t)stream, e);
+}
+
+int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float norm_eps, const void* wgu_packed,
+                           const void* sg, const void* su, const void* wd_packed, const void* sd, void* y, int ldy,
+                           const void* resid, int ldr, int resid_dtype, const void* gate, int M, int K, int I, int act,
+                           void* ws, size_t ws_bytes, void* stream) {
+  if (act != TK_ACT_SILU && act != TK_ACT_GELU_TANH) return fail(TK_EINVAL, "ffn: unknown activation %d", act);
+  if (!sg || !su || !sd || !norm_w) return fail(TK_EINVAL, "ffn: null scale or norm pointer");
+  if (I % 32) return fail(TK_EINVAL, "ffn: I=%d must be a multiple of 32", I);
+  if (!ws) return fail(TK_EWORKSPACE, "ffn: needs a workspace");
+  const size_t hbytes = (size_t)M * I * 2;
+  if (hbytes > kHiddenBytes || ws_bytes < kHiddenOff + hbytes)
+    return fail(TK_EWORKSPACE, "ffn: workspace too small for the [%d, %d] intermediate", M, I);
+  void* hbuf = (char*)ws + kHiddenOff;
+  GemmExtra e;
+  e.norm_w = norm_w;
+  e.norm_eps = norm_eps;
+  int rc = gemm_common(x, ldx, wgu_packed, (const float*)sg, (const float*)su, hbuf, I, nullptr, 0, 0, nullptr, M, I, K, 0,
+                       act, ws, ws_bytes, (hipStream_t)stream, e);
+  if (rc) return rc;
   return gemm_common(hbuf, I, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, K, I, 0, 0,
                      ws, ws_bytes, (hipStream_t)stream);
 }

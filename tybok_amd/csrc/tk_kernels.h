@@ -4,8 +4,10 @@
 #include <stdint.h>
 
 struct GemmArgs {
-  const unsigned short* x;  // bf16 [M, K]
+  const void* x;  // bf16 (or fp32 when x_f32) [M, K]
   int ldx;
+  int x_f32;
+  int w16;  // weights are bf16 tiles (2 KiB) instead of e4m3 tiles (1 KiB)
   const uint8_t* w;  // packed 32x32-byte tiles, tile (nt, kt) at ((nt*KT)+kt)*1024
   const float* s0;   // scale (plain) or gate scale (gated)
   const float* s1;   // up scale (gated) or nullptr
@@ -22,6 +24,17 @@ struct GemmArgs {
   float* partial;
   int* counters;
   int act;
+  // RMSNorm prologue (norm_w != nullptr): bf16 [K] weight, eps
+  const unsigned short* norm_w;
+  float norm_eps;
+  // rotary epilogue (rope_pos != nullptr): int32 [M] positions, fp32 [positions, rope_half] tables,
+  // columns < rope_cols are rotated in pairs (c, c + rope_half)
+  const int* rope_pos;
+  const float* rope_cos;
+  const float* rope_sin;
+  int rope_positions;  // rows of the tables (positions are clamped into them)
+  int rope_cols;
+  int rope_half;
 };
 
 struct AttnArgs {
@@ -46,6 +59,7 @@ struct AttnArgs {
 
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st);
 int tk_launch_pack(const void* w0, const void* w1, void* out, int N, int K, int interleave, hipStream_t st);
+int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st);
 int tk_launch_fill_zero(int* p, int n, hipStream_t st);
 int tk_launch_decode_fp8(float* out, hipStream_t st);
 int tk_launch_attn(AttnArgs a, int D, int kv_f32, hipStream_t st);

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
 
 # TYBOK_HIP_LIB points at an alternative build of the same ABI (kernel experiments); default in-tree.
 _LIB_PATH = os.environ.get("TYBOK_HIP_LIB") or os.path.join(
@@ -36,6 +36,18 @@ SIGNATURES: dict[str, tuple] = {
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
          c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
+    ),  # fmt: skip
+    "tk_fp8w_norm_gated_ffn": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+         c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
+    ),  # fmt: skip
+    "tk_bf16w_packed_bytes": (c_size_t, [c_int, c_int]),
+    "tk_pack_bf16_weight": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "tk_bf16w_linear": (
+        c_int,
+        [c_void_p, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+         c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
     "tk_expert_attn": (
         c_int,

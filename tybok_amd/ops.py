@@ -77,6 +77,32 @@ class PackedGateUp:
     k: int
 
 
+@dataclass
+class PackedBf16Weight:
+    """A bf16 ``[N, K]`` weight in tile order; ``rope_half`` > 0 means rotary pair order."""
+
+    data: torch.Tensor
+    n: int
+    k: int
+    rope_half: int = 0
+
+
+@dataclass
+class RopeTables:
+    """fp32 ``[positions, rope_half]`` cos / sin tables of a half-split rotary embedding."""
+
+    cos: torch.Tensor
+    sin: torch.Tensor
+
+    @property
+    def positions(self) -> int:
+        return self.cos.shape[0]
+
+    @property
+    def half(self) -> int:
+        return self.cos.shape[1]
+
+
 def _as_fp8_bytes(w8: torch.Tensor) -> torch.Tensor:
     if w8.dtype == torch.float8_e4m3fn:
         w8 = w8.view(torch.uint8)
@@ -172,10 +198,13 @@ def fp8w_gated_ffn(
     *,
     resid: torch.Tensor | None = None,
     gate: torch.Tensor | None = None,
+    norm_w: torch.Tensor | None = None,
+    eps: float = 0.0,
     out: torch.Tensor | None = None,
     ws: Workspace | None = None,
 ) -> torch.Tensor:
-    """``down(act(gate(x)) * up(x))`` (``* gate[n]``, ``+ residual``) for ``x [M, K]`` bf16."""
+    """``down(act(gate(x)) * up(x))`` (``* gate[n]``, ``+ residual``) for ``x [M, K]`` bf16;
+    with ``norm_w`` the input is first RMS-normalised inside the gate/up launch."""
     lib = native.lib()
     m, ldx = _check_act(x, wgu.k)
     if wd.k != wgu.i or wd.n != wgu.k:
@@ -184,12 +213,95 @@ def fp8w_gated_ffn(
         out = torch.empty(m, wd.n, dtype=torch.bfloat16, device=x.device)
     rp, ldr, rdt = _resid_args(resid, m, wd.n)
     ws = ws or default_workspace(x.device)
+    if norm_w is not None:
+        rc = lib.tk_fp8w_norm_gated_ffn(
+            x.data_ptr(), ldx, _norm_ptr(norm_w, wgu.k), float(eps), wgu.data.data_ptr(), wgu.scale_gate.data_ptr(),
+            wgu.scale_up.data_ptr(), wd.data.data_ptr(), wd.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt,
+            _gate_ptr(gate, wd.n), m, wgu.k, wgu.i, ACT[act], ws.ptr, ws.nbytes, _stream(),
+        )  # fmt: skip
+        native.check(rc, "tk_fp8w_norm_gated_ffn")
+        return out
     rc = lib.tk_fp8w_gated_ffn(
         x.data_ptr(), ldx, wgu.data.data_ptr(), wgu.scale_gate.data_ptr(), wgu.scale_up.data_ptr(),
         wd.data.data_ptr(), wd.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt,
         _gate_ptr(gate, wd.n), m, wgu.k, wgu.i, ACT[act], ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip
     native.check(rc, "tk_fp8w_gated_ffn")
+    return out
+
+
+def pack_bf16_weight(w: torch.Tensor, rope_half: int = 0) -> PackedBf16Weight:
+    """Row-major bf16 ``[N, K]`` -> :class:`PackedBf16Weight` (once per model)."""
+    lib = native.lib()
+    if w.dtype != torch.bfloat16 or not w.is_cuda or w.dim() != 2:
+        raise TypeError("expected a bf16 CUDA matrix")
+    w = w.contiguous()
+    n, k = w.shape
+    out = torch.empty(int(lib.tk_bf16w_packed_bytes(n, k)), dtype=torch.uint8, device=w.device)
+    native.check(lib.tk_pack_bf16_weight(w.data_ptr(), out.data_ptr(), n, k, rope_half, _stream()), "tk_pack_bf16_weight")
+    return PackedBf16Weight(out, n, k, rope_half)
+
+
+def _norm_ptr(norm_w: torch.Tensor | None, k: int) -> int | None:
+    if norm_w is None:
+        return None
+    if norm_w.dtype != torch.bfloat16 or norm_w.numel() != k or not norm_w.is_contiguous():
+        raise ValueError(f"norm weight must be a contiguous bf16 tensor of {k} elements")
+    return norm_w.data_ptr()
+
+
+def bf16w_linear(
+    x: torch.Tensor,
+    w: PackedBf16Weight,
+    *,
+    norm_w: torch.Tensor | None = None,
+    eps: float = 0.0,
+    rope: RopeTables | None = None,
+    rope_pos: torch.Tensor | None = None,
+    rope_cols: int = 0,
+    resid: torch.Tensor | None = None,
+    out: torch.Tensor | None = None,
+    split_k: int = 0,
+    ws: Workspace | None = None,
+) -> torch.Tensor:
+    """``x [M, K] @ W^T`` with bf16 weights; optional RMSNorm prologue (``x`` bf16 or fp32), and
+    either a rotary epilogue (``rope`` tables, int32 ``rope_pos [M]``, columns ``< rope_cols``
+    rotated) or a residual epilogue."""
+    lib = native.lib()
+    if not x.is_cuda or x.dim() != 2 or x.shape[1] != w.k or x.stride(1) != 1:
+        raise ValueError(f"activations must be CUDA [M, {w.k}] with unit inner stride")
+    if x.dtype == torch.float32:
+        if norm_w is None:
+            raise TypeError("fp32 activations are accepted with the norm prologue only")
+        xdt = _F32
+    elif x.dtype == torch.bfloat16:
+        xdt = _BF16
+    else:
+        raise TypeError("activations must be bf16 or fp32")
+    m = x.shape[0]
+    if out is None:
+        out = torch.empty(m, w.n, dtype=torch.bfloat16, device=x.device)
+    rp, ldr, rdt = _resid_args(resid, m, w.n)
+    pos_p = cos_p = sin_p = None
+    positions = half = 0
+    if rope is not None:
+        if rope_pos is None or rope_pos.dtype != torch.int32 or rope_pos.numel() != m or not rope_pos.is_contiguous():
+            raise ValueError("rope_pos must be a contiguous int32 [M]")
+        if rope.half != w.rope_half:
+            raise ValueError("weight was packed for a different rotary head size")
+        if rope.cos.dtype != torch.float32 or not rope.cos.is_contiguous() or not rope.sin.is_contiguous():
+            raise ValueError("rotary tables must be contiguous fp32")
+        pos_p, cos_p, sin_p = rope_pos.data_ptr(), rope.cos.data_ptr(), rope.sin.data_ptr()
+        positions, half = rope.positions, rope.half
+    elif w.rope_half:
+        raise ValueError("a weight packed in rotary pair order needs the rotary epilogue")
+    ws = ws or default_workspace(x.device)
+    rc = lib.tk_bf16w_linear(
+        x.data_ptr(), x.stride(0), xdt, w.data.data_ptr(), _norm_ptr(norm_w, w.k), float(eps), pos_p, cos_p, sin_p,
+        positions, rope_cols, half, out.data_ptr(), out.stride(0), rp, ldr, rdt, m, w.n, w.k, split_k, ws.ptr, ws.nbytes,
+        _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_bf16w_linear")
     return out
 
 

@@ -8,11 +8,13 @@ the HIP kernels of this package:
 * ``fp8_expert_mlp`` / ``fp8_llm_mlp``  -- the gated FFN of the expert / VLM layers runs as
   ``tk_fp8w_gated_ffn`` on e4m3fn weights (second residual fused), the seam where the reference
   calls ``triton_norm_gate_up`` + ``down_proj`` (vlm_with_expert.py:391-408);
-* ``fused_expert``  -- the denoising self/cross attention runs as ``tk_expert_attn`` over the
-  cached prefix KV, the seam of ``triton_self_attn`` / ``triton_cross_attn``
-  (vlm_with_expert.py:166-190, 275-297).
+* ``fused_expert``  -- a denoising expert layer is five launches: input RMSNorm + packed q|k|v
+  projection + RoPE (``tk_bf16w_linear``), attention over the cached prefix KV
+  (``tk_expert_attn``), o_proj + residual (``tk_bf16w_linear``), and -- with ``fp8_expert_mlp`` --
+  post-attention RMSNorm + gate/up, down + residual (``tk_fp8w_norm_gated_ffn``); the seam of
+  ``triton_self_attn`` / ``triton_cross_attn`` (vlm_with_expert.py:166-190, 275-297).
 
-Everything else (norms, projections, RoPE, vision tower) is plain torch on the GPU.  The model
+Everything else (VLM prefill, vision tower, action/time projections) is plain torch on the GPU.  The model
 is capture-clean: every constant is built at construction time, nothing copies from the host or
 synchronises inside :meth:`sample_actions`.
 """
@@ -120,6 +122,8 @@ class SmolVLAModel:
         self.vlm_mlp = [GatedMLP(state_dict, f"{TXT}layers.{i}.mlp.", self.device, self.fp8_llm_mlp) for i in range(self.num_layers)]
         self.exp_mlp = [GatedMLP(state_dict, f"{EXP}layers.{i}.mlp.", self.device, self.fp8_expert_mlp) for i in range(cfg.n_expert_layers)]
         self.ws = tk.default_workspace(self.device) if self.use_hip else None
+        if self.fused_expert:
+            self._pack_expert_projections()
 
         # constants (built once: nothing below copies from the host at inference time)
         d_half = self.head_dim // 2
@@ -127,6 +131,7 @@ class SmolVLAModel:
         radians = torch.arange(_ROPE_POSITIONS, dtype=torch.float32)[:, None] / (10_000.0**exponents)[None, :]
         self.rope_sin = torch.sin(radians).to(self.device)
         self.rope_cos = torch.cos(radians).to(self.device)
+        self.rope_tables = tk.RopeTables(self.rope_cos, self.rope_sin) if self.fused_expert else None
         self.set_num_steps(cfg.num_steps)
         v = cfg.vlm_config.vision_config
         side = v.image_size // v.patch_size
@@ -142,6 +147,17 @@ class SmolVLAModel:
             t = torch.tensor(1.0 + step * dt, dtype=torch.float32).expand(1)
             embs.append(sinusoidal_time_embedding(t, self.cfg.expert_hidden_size, self.cfg.min_period, self.cfg.max_period).float())
         self.time_embs = [e.to(self.device) for e in embs]
+
+    def _pack_expert_projections(self) -> None:
+        """bf16 expert attention weights in tile order: q|k|v concatenated (self layers) or q alone
+        (cross layers) in rotary pair order, o_proj in natural order."""
+        self.exp_qkv, self.exp_o = [], []
+        for i in range(self.num_layers):
+            lp = f"{EXP}layers.{i}.self_attn."
+            names = ("q_proj",) if self.cfg.is_cross_layer(i) else ("q_proj", "k_proj", "v_proj")
+            w = torch.cat([self.p[lp + n + ".weight"] for n in names], dim=0).to(BF16)
+            self.exp_qkv.append(tk.pack_bf16_weight(w, rope_half=self.head_dim // 2))
+            self.exp_o.append(tk.pack_bf16_weight(self.p[lp + "o_proj.weight"].to(BF16)))
 
     # ------------------------------------------------------------------ helpers
     def lin(self, name: str, x: torch.Tensor) -> torch.Tensor:
@@ -262,13 +278,54 @@ class SmolVLAModel:
         h = self.lin("action_time_mlp_in", torch.cat([a, te], dim=2))
         return self.lin("action_time_mlp_out", F.silu(h))
 
-    def denoise_step(self, prefix_pad, keys, values, ekv, x_t, time_emb):
+    def suffix_positions(self, prefix_pad: torch.Tensor, s: int) -> tuple[torch.Tensor, torch.Tensor]:
+        """Positions of the action tokens: after the valid prefix (self layers) and from 0 (cross layers)."""
+        pos = prefix_pad.sum(dim=-1)[:, None] + torch.arange(s, device=self.device)[None, :]
+        pos0 = pos - pos.min(dim=1, keepdim=True).values
+        return pos, pos0
+
+    def _denoise_step_fused(self, prefix_pad, keys, values, ekv, hidden, pos32, pos0_32):
+        """Expert stack on the fused launches; ``hidden [S, E]`` fp32 in, bf16 out."""
+        h_q, h_kv, d = self.heads, self.kv_heads, self.head_dim
+        nq, nkv = h_q * d, h_kv * d
+        s = hidden.shape[0]
+        pad = prefix_pad[0]
+        for i in range(self.num_layers):
+            lp = f"{EXP}layers.{i}."
+            cross = self.cfg.is_cross_layer(i)
+            qkv = tk.bf16w_linear(
+                hidden, self.exp_qkv[i], norm_w=self.p[lp + "input_layernorm.weight"], eps=self.eps, rope=self.rope_tables,
+                rope_pos=pos0_32 if cross else pos32, rope_cols=nq if cross else nq + nkv, ws=self.ws,
+            )  # fmt: skip
+            q = qkv[:, :nq].view(s, h_q, d)
+            if cross:
+                ek, ev = ekv[i]
+                att = tk.expert_attn(q, ek[0], ev[0], None, None, pad, tk.MASK_NONE, ws=self.ws)
+            else:
+                k = qkv[:, nq : nq + nkv].view(s, h_kv, d)
+                v = qkv[:, nq + nkv :].view(s, h_kv, d)
+                att = tk.expert_attn(q, keys[i, 0], values[i, 0], k, v, pad, tk.MASK_CAUSAL, ws=self.ws)
+            out = tk.bf16w_linear(att, self.exp_o[i], resid=hidden, ws=self.ws)
+            mlp = self.exp_mlp[i]
+            post_w = self.p[lp + "post_attention_layernorm.weight"]
+            if mlp.fp8:
+                hidden = tk.fp8w_gated_ffn(out, mlp.wgu, mlp.wd, mlp.act, resid=out, norm_w=post_w, eps=self.eps, ws=self.ws)
+            else:
+                hidden = mlp(rms_norm(out, post_w, self.eps)[None], out[None])[0]
+        return hidden
+
+    def denoise_step(self, prefix_pad, keys, values, ekv, x_t, time_emb, positions=None):
         """Velocity ``v_t`` fp32 ``[1, chunk, max_action_dim]`` (flow_matching.py:316-350)."""
         hidden = self.embed_suffix(x_t, time_emb)
         b, s = hidden.shape[0], hidden.shape[1]
         p_len = prefix_pad.shape[1]
-        pos = prefix_pad.sum(dim=-1)[:, None] + torch.arange(s, device=self.device)[None, :]
-        pos0 = pos - pos.min(dim=1, keepdim=True).values
+        pos, pos0 = positions if positions is not None else self.suffix_positions(prefix_pad, s)
+        if self.fused_expert and b == 1:
+            clamp = lambda t: t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)  # noqa: E731
+            pos32, pos0_32 = (pos, pos0) if pos.dtype == torch.int32 else (clamp(pos), clamp(pos0))
+            hidden = self._denoise_step_fused(prefix_pad, keys, values, ekv, hidden[0], pos32, pos0_32)[None]
+            out = rms_norm(hidden, self.p[EXP + "norm.weight"], self.eps)
+            return self.lin("action_out_proj", out.to(torch.float32))
         if not self.fused_expert:
             causal = torch.ones(s, s, dtype=torch.bool, device=self.device).tril()[None]
             full_mask = torch.cat([prefix_pad[:, None, :].expand(b, s, p_len), causal], dim=2)
@@ -302,8 +359,11 @@ class SmolVLAModel:
             trace.update(prefix_embs=embs, pad_masks=pads, keys=keys, values=values, ekv=ekv)
         dt = -1.0 / self.num_steps
         x_t = noise
+        positions = self.suffix_positions(pads, noise.shape[1])
+        if self.fused_expert and noise.shape[0] == 1:
+            positions = tuple(t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32) for t in positions)
         for step in range(self.num_steps):
-            v_t = self.denoise_step(pads, keys, values, ekv, x_t, self.time_embs[step])
+            v_t = self.denoise_step(pads, keys, values, ekv, x_t, self.time_embs[step], positions)
             x_t = x_t + dt * v_t
         return x_t
 
