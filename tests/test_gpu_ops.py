@@ -83,7 +83,7 @@ def test_gemm_split_k_equals_no_split_within_tolerance_and_is_deterministic(tk, 
     _close(a, oops.lin_fp8w(x, w8, s), f"gemm split_k={split}")
 
 
-@pytest.mark.parametrize("m,k,n", [(3, 16, 32), (33, 48, 40), (50, 720, 720), (64, 80, 96), (241, 960, 2560), (130, 2048, 320)])
+@pytest.mark.parametrize("m,k,n", [(3, 16, 32), (5, 32, 37), (40, 96, 130), (33, 48, 40), (50, 720, 720), (64, 80, 96), (241, 960, 2560), (130, 2048, 320)])
 def test_gemm_ragged_shapes(tk, m, k, n):
     x, w8, s = gemm_case(m, k, n)
     pw = tk.pack_fp8_weight(w8.cuda(), s.cuda())

@@ -18,6 +18,23 @@
 #include "tk_common.h"
 #include "tk_kernels.h"
 
+#ifdef TK_PHASE_TIMING
+// development aid (never built into the shipped library): per-block phase timestamps
+__device__ long long tk_phase_stamps[8 * 8192];
+#define TK_MARK(i)                                                                                       \
+  do {                                                                                                   \
+    if (threadIdx.x == 0) {                                                                              \
+      const int b_ = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;                     \
+      if (b_ < 8192) tk_phase_stamps[b_ * 8 + (i)] = wall_clock64();                                     \
+    }                                                                                                    \
+  } while (0)
+extern "C" int tk_debug_read_phases(void* host_out) {
+  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(tk_phase_stamps), sizeof(long long) * 8 * 8192);
+}
+#else
+#define TK_MARK(i)
+#endif
+
 namespace {
 
 // LDS-only barrier: waits for this wave's LDS traffic, not for the global prefetch queue
@@ -65,6 +82,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   const int half = lane >> 5;
   const int l32 = lane & 31;
 
+  TK_MARK(0);
   const int kt_lo = (int)(((long long)split * a.KT) / a.ksplit);
   const int kt_hi = (int)(((long long)(split + 1) * a.KT) / a.ksplit);
   const int nrounds = (kt_hi - kt_lo + RKT - 1) / RKT;
@@ -97,23 +115,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     xcol[i] = c * 8;
     xdst[i] = r * PITCH + c * 16;
     xrow[i] = r;
-  }
-
-  // scales of the columns this wave will finish, fetched before the loop so the epilogue does not
-  // start with a cold miss
-  float sc_pre[2] = {1.f, 1.f};
-  if (!W16) {
-    const int n0 = GATED ? (strip * NT / 2) * 32 + l32 : strip * NT * 32 + l32;
-    if (!GATED) {
-#pragma unroll
-      for (int nt = 0; nt < (NT < 2 ? NT : 2); ++nt) {
-        const int n = n0 + nt * 32;
-        sc_pre[nt] = n < a.N ? a.s0[n] : 0.f;
-      }
-    } else {
-      sc_pre[0] = n0 < a.N ? a.s0[n0] : 0.f;
-      sc_pre[1] = n0 < a.N ? a.s1[n0] : 0.f;
-    }
   }
 
   f32x16 acc[MT][NT];
@@ -171,7 +172,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       if (PRO == 0) {
         out = f.v[i][0];
       } else {
-        union { i32x4 v; u16 h[8]; } nwu, o;
+        union { i32x4 v; unsigned u[4]; } nwu, o;
         nwu.v = f.nw[i];
         float xv[8];
         if (XF32) {
@@ -181,16 +182,23 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) { xv[e] = lo.f[e]; xv[4 + e] = hi.f[e]; }
         } else {
-          union { i32x4 v; u16 h[8]; } xu;
+          union { i32x4 v; unsigned u[4]; } xu;
           xu.v = f.v[i][0];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) xv[e] = bf16_bits_to_f32(xu.h[e]);
+          for (int e = 0; e < 4; ++e) {
+            xv[2 * e] = __uint_as_float(xu.u[e] << 16);
+            xv[2 * e + 1] = __uint_as_float(xu.u[e] & 0xffff0000u);
+          }
         }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float n = xv[e] * my_rstd[i];
-          if (!XF32) n = round_bf16(n);
-          o.h[e] = f32_to_bf16_bits(bf16_bits_to_f32(nwu.h[e]) * n);
+        for (int e = 0; e < 4; ++e) {
+          float n0 = xv[2 * e] * my_rstd[i], n1 = xv[2 * e + 1] * my_rstd[i];
+          if (!XF32) {  // a bf16 input is normalised back to bf16 before the weight multiply
+            const unsigned u = pack_bf16x2(n0, n1);
+            n0 = __uint_as_float(u << 16);
+            n1 = __uint_as_float(u & 0xffff0000u);
+          }
+          o.u[e] = pack_bf16x2(__uint_as_float(nwu.u[e] << 16) * n0, __uint_as_float(nwu.u[e] & 0xffff0000u) * n1);
         }
         out = o.v;
       }
@@ -224,7 +232,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt)
-            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(xa[mt][h2]), wb[nt][h2], acc[mt][nt], 0, 0, 0);
+            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[nt][h2], as_bf16x8(xa[mt][h2]), acc[mt][nt], 0, 0, 0);
     }
   };
 
@@ -242,30 +250,35 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       wload(wbuf[p], p);
     }
   }
+  TK_MARK(1);
   if (PRO) {
     // per-row 1/rms over the whole K (every block needs it for its rows, whatever its k range)
     constexpr int TPR = NW * 64 / ROWS;  // threads per row
     const int r = tid / TPR, q = tid % TPR;
-    int m = mblock * ROWS + r;
-    if (m > a.M - 1) m = a.M - 1;
-    const char* row = (const char*)a.x + (size_t)m * a.ldx * (XF32 ? 4 : 2);
-    float ss = 0.f;
+    const int m = mblock * ROWS + r;
+    const char* row = (const char*)a.x + (size_t)(m < a.M ? m : 0) * a.ldx * (XF32 ? 4 : 2);
+    const int npieces = m < a.M ? a.K / 8 : 0;  // rows past M are never stored: skip their reads
+    float ss0 = 0.f, ss1 = 0.f;
 #pragma unroll 8
-    for (int p = q; p < a.K / 8; p += TPR) {
+    for (int p = q; p < npieces; p += TPR) {
       if (XF32) {
-        const float4* p4 = (const float4*)(row + (size_t)p * 32);
-        float4 u0 = p4[0], u1 = p4[1];
-        ss += u0.x * u0.x + u0.y * u0.y + u0.z * u0.z + u0.w * u0.w + u1.x * u1.x + u1.y * u1.y + u1.z * u1.z + u1.w * u1.w;
-      } else {
-        union { i32x4 v; u16 h[8]; } xu;
-        xu.v = *(const i32x4*)(row + (size_t)p * 16);
+        const f32x4* p4 = (const f32x4*)(row + (size_t)p * 32);
+        const f32x4 u0 = p4[0], u1 = p4[1];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float f = bf16_bits_to_f32(xu.h[e]);
-          ss += f * f;
+        for (int e = 0; e < 4; ++e) {
+          ss0 = fmaf(u0[e], u0[e], ss0);
+          ss1 = fmaf(u1[e], u1[e], ss1);
         }
+      } else {
+        union { i32x4 v; bf16x2 h[4]; } xu;
+        xu.v = *(const i32x4*)(row + (size_t)p * 16);
+        ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[0], xu.h[0], ss0, false);
+        ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[1], xu.h[1], ss1, false);
+        ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[2], xu.h[2], ss0, false);
+        ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[3], xu.h[3], ss1, false);
       }
     }
+    float ss = ss0 + ss1;
 #pragma unroll
     for (int o = TPR / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
     if (q == 0) rstd_s[r] = rsqrtf(ss / (float)a.K + a.norm_eps);
@@ -273,6 +286,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 #pragma unroll
     for (int i = 0; i < XPT; ++i) my_rstd[i] = rstd_s[xrow[i]];
   }
+  TK_MARK(2);
   if (nrounds > 0) {
     int it = 0;
     for (; it + 2 * PF <= nrounds; it += PF) {
@@ -303,55 +317,47 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     }
   }
   __syncthreads();  // staging buffers are dead; the reduction reuses the LDS
+  TK_MARK(3);
 
-  // ---- in-block reduction over waves (fixed order), tile by tile, double-buffered LDS ----
-  float (*red)[NW][16][64] = (float (*)[NW][16][64])lds;
-  constexpr int OWN = PAIRED ? 2 * ((TILES / 2 + NW - 1) / NW) : (TILES + NW - 1) / NW;
-  float own[OWN][16];
-#pragma unroll
-  for (int o = 0; o < OWN; ++o)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) own[o][i] = 0.f;
+  // The accumulators hold C^T tiles: lane l of a tile owns activation row m = l % 32 and, in
+  // register i, output column n = 8*(i/4) + 4*(l/32) + i%4 -- register group g = i/4 is four
+  // consecutive columns.  From here on wave w owns group g = w of EVERY tile: all four waves take
+  // part in the reductions and in the epilogue, and everything moves as 8- or 16-byte vectors.
+  static_assert(NW == 4, "one wave per register group");
+  const int ng = wave * 8 + half * 4;  // first of this lane's four columns within an n tile
 
+  // ---- in-block reduction over waves (fixed order w = 0..3), tile by tile, double-buffered ----
+  f32x4 (*red)[NW][4][64] = (f32x4 (*)[NW][4][64])lds;
+  f32x4 own[TILES];
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
     const int mt = t / NT, nt = t % NT;
-    const int owner = PAIRED ? (t / 2) % NW : t % NW;
-    const int slot = PAIRED ? ((t / 2) / NW) * 2 + (t & 1) : t / NW;
-    if (NW > 1) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) red[t & 1][wave][i][lane] = acc[mt][nt][i];
-      __syncthreads();
-      if (wave == owner) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          float s = 0.f;
-#pragma unroll
-          for (int w = 0; w < NW; ++w) s += red[t & 1][w][i][lane];
-          own[slot][i] = s;
-        }
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) own[slot][i] = acc[mt][nt][i];
+    for (int g = 0; g < 4; ++g) {
+      f32x4 v = {acc[mt][nt][4 * g], acc[mt][nt][4 * g + 1], acc[mt][nt][4 * g + 2], acc[mt][nt][4 * g + 3]};
+      red[t & 1][wave][g][lane] = v;
     }
+    __syncthreads();
+    f32x4 sum = red[t & 1][0][wave][lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) sum += red[t & 1][w][wave][lane];
+    own[t] = sum;
   }
 
   // ---- K-split reduction through global partials; the last-arriving block finishes ----
+  TK_MARK(4);
   const int blk_lin = mblock * gridDim.x + strip;
   if (a.ksplit > 1) {
+    // partial layout: [(block, split)][tile][group][lane][4 floats], written and read as 8-byte
+    // device-coherent accesses (write-through, so the hand-off needs no cache flush)
+    unsigned long long* pbase = (unsigned long long*)a.partial + ((size_t)wave * 64 + lane) * 2;
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-      const int owner = PAIRED ? (t / 2) % NW : t % NW;
-      const int slot = PAIRED ? ((t / 2) / NW) * 2 + (t & 1) : t / NW;
-      if (wave == owner) {
-        float* dst = a.partial + (((size_t)blk_lin * a.ksplit + split) * TILES + t) * 1024 + lane;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) st_agent(dst + i * 64, own[slot][i]);
-      }
+      unsigned long long* dst = pbase + (((size_t)blk_lin * a.ksplit + split) * TILES + t) * 512;
+      st_agent64(dst, own[t][0], own[t][1]);
+      st_agent64(dst + 1, own[t][2], own[t][3]);
     }
-    // The partials were written through to device-coherent memory (agent-scope stores), so no
-    // cache flush is needed: wait until they are acknowledged, then count this block in.
+    // wait until the partials are acknowledged, then count this block in
     __shared__ int s_last;
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
@@ -360,45 +366,71 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       s_last = (old == a.ksplit - 1);
     }
     __syncthreads();
+    TK_MARK(5);
     if (!s_last) return;
+    if (threadIdx.x == 0)  // leave the counter ready for the next launch
+      __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-    for (int t = 0; t < TILES; ++t) {
-      const int owner = PAIRED ? (t / 2) % NW : t % NW;
-      const int slot = PAIRED ? ((t / 2) / NW) * 2 + (t & 1) : t / NW;
-      if (wave == owner) {
+    for (int t = 0; t < TILES; ++t) own[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // sum in split order; four splits' loads are in flight together
+    constexpr int SB = 4;
+    for (int s0 = 0; s0 < a.ksplit; s0 += SB) {
+      unsigned long long raw[SB][TILES][2];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) own[slot][i] = 0.f;
-        for (int s = 0; s < a.ksplit; ++s) {
-          const float* src = a.partial + (((size_t)blk_lin * a.ksplit + s) * TILES + t) * 1024 + lane;
+      for (int j = 0; j < SB; ++j) {
+        const int sj = s0 + j < a.ksplit ? s0 + j : a.ksplit - 1;
 #pragma unroll
-          for (int i = 0; i < 16; ++i) own[slot][i] += ld_agent(src + i * 64);
+        for (int t = 0; t < TILES; ++t) {
+          const unsigned long long* src = pbase + (((size_t)blk_lin * a.ksplit + sj) * TILES + t) * 512;
+          raw[j][t][0] = ld_agent64(src);
+          raw[j][t][1] = ld_agent64(src + 1);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < SB; ++j) {
+        if (s0 + j < a.ksplit) {
+#pragma unroll
+          for (int t = 0; t < TILES; ++t) {
+            own[t][0] += __uint_as_float((unsigned)raw[j][t][0]);
+            own[t][1] += __uint_as_float((unsigned)(raw[j][t][0] >> 32));
+            own[t][2] += __uint_as_float((unsigned)raw[j][t][1]);
+            own[t][3] += __uint_as_float((unsigned)(raw[j][t][1] >> 32));
+          }
         }
       }
     }
-    if (threadIdx.x == 0)  // leave the counter ready for the next launch
-      __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
-  // ---- epilogue ----
+  // ---- epilogue: this lane finishes row m (per m tile), columns n0 .. n0+3 of each n tile ----
+  TK_MARK(6);
   if (EPI == 0) {
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
       const int mt = t / NT, nt = t % NT;
-      if (wave != t % NW) continue;
-      const int slot = t / NW;
-      const int n = (strip * NT + nt) * 32 + l32;
-      if (n >= a.N) continue;
-      const float sc = sc_pre[nt < 2 ? nt : 0];
-      const float gt = a.gate ? bf16_bits_to_f32(a.gate[n]) : 1.0f;
+      const int m = (mblock * MT + mt) * 32 + l32;
+      const int n0 = (strip * NT + nt) * 32 + ng;
+      if (m >= a.M || n0 >= a.N) continue;
+      if (a.vec) {  // N % 4 == 0 and every row pitch / pointer allows 8-byte accesses
+        f32x4 v = own[t];
+        if (!W16) v *= *(const f32x4*)(a.s0 + n0);
+        i32x2 r = pack_bf16x4(v);
+        if (a.gate) r = pack_bf16x4(unpack_bf16x4(r) * unpack_bf16x4(*(const i32x2*)(a.gate + n0)));
+        if (a.resid) {
+          const f32x4 rv = a.resid_f32 ? *(const f32x4*)((const float*)a.resid + (size_t)m * a.ldr + n0)
+                                       : unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n0));
+          r = pack_bf16x4(unpack_bf16x4(r) + rv);
+        }
+        *(i32x2*)(a.y + (size_t)m * a.ldy + n0) = r;
+      } else {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int m = (mblock * MT + mt) * 32 + mfma32_row(lane, i);
-        if (m < a.M) {
-          u16 r = f32_to_bf16_bits(own[slot][i] * sc);
-          if (a.gate) r = f32_to_bf16_bits(bf16_bits_to_f32(r) * gt);
+        for (int j = 0; j < 4; ++j) {
+          const int n = n0 + j;
+          if (n >= a.N) continue;
+          u16 r = f32_to_bf16_bits(own[t][j] * (W16 ? 1.0f : a.s0[n]));
+          if (a.gate) r = f32_to_bf16_bits(bf16_bits_to_f32(r) * bf16_bits_to_f32(a.gate[n]));
           if (a.resid) {
-            float rv = a.resid_f32 ? ((const float*)a.resid)[(size_t)m * a.ldr + n]
-                                   : bf16_bits_to_f32(((const u16*)a.resid)[(size_t)m * a.ldr + n]);
+            const float rv = a.resid_f32 ? ((const float*)a.resid)[(size_t)m * a.ldr + n]
+                                         : bf16_bits_to_f32(((const u16*)a.resid)[(size_t)m * a.ldr + n]);
             r = f32_to_bf16_bits(bf16_bits_to_f32(r) + rv);
           }
           a.y[(size_t)m * a.ldy + n] = r;
@@ -406,25 +438,21 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       }
     }
   } else if (EPI == 1) {
-    // tiles come in (gate, up) pairs over the same logical columns
+    // tiles come in (gate, up) pairs over the same logical columns; I % 32 == 0
+    const int col = strip * 32 + ng;  // logical column in [0, I)
+    if (col < a.N) {
+      const f32x4 scg = *(const f32x4*)(a.s0 + col), scu = *(const f32x4*)(a.s1 + col);
 #pragma unroll
-    for (int u = 0; u < TILES / 2; ++u) {
-      if (wave != u % NW) continue;
-      const int t = 2 * u;
-      const int mt = t / NT;
-      const int sg = (u / NW) * 2, su = sg + 1;
-      const int col = strip * 32 + l32;  // logical column in [0, I)
-      if (col >= a.N) continue;
-      const float scg = sc_pre[0], scu = sc_pre[1];
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = (mblock * MT + mt) * 32 + l32;
+        if (m >= a.M) continue;
+        const f32x4 g = unpack_bf16x4(pack_bf16x4(own[mt * 2] * scg));
+        const f32x4 up = unpack_bf16x4(pack_bf16x4(own[mt * 2 + 1] * scu));
+        f32x4 act;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int m = (mblock * MT + mt) * 32 + mfma32_row(lane, i);
-        if (m < a.M) {
-          float g = round_bf16(own[sg][i] * scg);
-          float up = round_bf16(own[su][i] * scu);
-          float act = a.act == 0 ? silu_f(g) : gelu_tanh_f(g);
-          a.y[(size_t)m * a.ldy + col] = f32_to_bf16_bits(round_bf16(act) * up);
-        }
+        for (int j = 0; j < 4; ++j) act[j] = a.act == 0 ? silu_f(g[j]) : gelu_tanh_f(g[j]);
+        act = unpack_bf16x4(pack_bf16x4(act));
+        *(i32x2*)(a.y + (size_t)m * a.ldy + col) = pack_bf16x4(act * up);
       }
     }
   } else {
@@ -432,38 +460,37 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     // physical tile (strip, j) is (strip / PO) * 2 * PO + strip % PO + j * PO with PO = rope_half / 32
     const int po = a.rope_half >> 5;
     const int lt0 = (strip / po) * 2 * po + strip % po;
-    const int ca = lt0 * 32 + l32, cb = ca + a.rope_half;
-    const int fi = ca % (2 * a.rope_half);  // rotary frequency index of the pair
+    const int ca = lt0 * 32 + ng, cb = ca + a.rope_half;
+    const int fi = ca % (2 * a.rope_half);  // rotary frequency index of the first pair
     const bool rot = ca < a.rope_cols;
+    if (cb + 3 < a.N) {
 #pragma unroll
-    for (int u = 0; u < TILES / 2; ++u) {
-      if (wave != u % NW) continue;
-      const int mt = (2 * u) / NT;
-      const int sa = (u / NW) * 2, sb = sa + 1;
-      if (cb >= a.N) continue;
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = (mblock * MT + mt) * 32 + l32;
+        if (m >= a.M) continue;
+        f32x4 va = unpack_bf16x4(pack_bf16x4(own[mt * 2]));
+        f32x4 vb = unpack_bf16x4(pack_bf16x4(own[mt * 2 + 1]));
+        if (rot) {
+          int pos = a.rope_pos[m];
+          pos = pos < 0 ? 0 : (pos > a.rope_positions - 1 ? a.rope_positions - 1 : pos);
+          const f32x4 cs = *(const f32x4*)(a.rope_cos + (size_t)pos * a.rope_half + fi);
+          const f32x4 sn = *(const f32x4*)(a.rope_sin + (size_t)pos * a.rope_half + fi);
+          f32x4 ra, rb;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int m = (mblock * MT + mt) * 32 + mfma32_row(lane, i);
-        if (m < a.M) {
-          float va = round_bf16(own[sa][i] * sc_pre[0]);
-          float vb = round_bf16(own[sb][i] * sc_pre[1]);
-          if (rot) {
-            int pos = a.rope_pos[m];
-            pos = pos < 0 ? 0 : (pos > a.rope_positions - 1 ? a.rope_positions - 1 : pos);
-            const float cs = a.rope_cos[(size_t)pos * a.rope_half + fi];
-            const float sn = a.rope_sin[(size_t)pos * a.rope_half + fi];
+          for (int j = 0; j < 4; ++j) {
             // separately rounded products, as an elementwise fp32 implementation computes them
-            const float ra = __fsub_rn(__fmul_rn(va, cs), __fmul_rn(vb, sn));
-            const float rb = __fadd_rn(__fmul_rn(vb, cs), __fmul_rn(va, sn));
-            va = ra;
-            vb = rb;
+            ra[j] = __fsub_rn(__fmul_rn(va[j], cs[j]), __fmul_rn(vb[j], sn[j]));
+            rb[j] = __fadd_rn(__fmul_rn(vb[j], cs[j]), __fmul_rn(va[j], sn[j]));
           }
-          a.y[(size_t)m * a.ldy + ca] = f32_to_bf16_bits(va);
-          a.y[(size_t)m * a.ldy + cb] = f32_to_bf16_bits(vb);
+          va = ra;
+          vb = rb;
         }
+        *(i32x2*)(a.y + (size_t)m * a.ldy + ca) = pack_bf16x4(va);
+        *(i32x2*)(a.y + (size_t)m * a.ldy + cb) = pack_bf16x4(vb);
       }
     }
   }
+  TK_MARK(7);
 }
 
 __global__ void pack_kernel(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1, uint8_t* __restrict__ out,

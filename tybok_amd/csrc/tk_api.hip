@@ -29,6 +29,7 @@ constexpr size_t kHiddenBytes = TK_WS_TOTAL_BYTES - kHiddenOff;  // FFN [M, I] b
 constexpr int kMaxCounters = (int)(kCounterBytes / 4);
 
 bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+bool aligned8(const void* p) { return (((uintptr_t)p) & 7) == 0; }
 
 int g_cus = -1;
 int device_cus() {
@@ -99,6 +100,12 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   a.KT = (K + 31) / 32;
   a.ntiles = ((N + 31) / 32) * (gated ? 2 : 1);
   a.act = act;
+  a.vec = N % 4 == 0 && ldy % 4 == 0 && aligned8(y) && (e.w16 || aligned16(s0)) && (!gate || aligned8(gate)) &&
+          (!resid || (ldr % 4 == 0 && (resid_dtype == TK_F32 ? aligned16(resid) : aligned8(resid))));
+  if ((gated || rope) && (ldy % 4 || !aligned8(y) || (gated && (!aligned16(s0) || !aligned16(s1)))))
+    return fail(TK_EINVAL, "gemm: this epilogue needs ldy %% 4 == 0, an 8-byte aligned y and 16-byte aligned scales");
+  if (rope && (!aligned16(e.rope_cos) || !aligned16(e.rope_sin)))
+    return fail(TK_EINVAL, "gemm: rotary tables must be 16-byte aligned");
   a.norm_w = (const u16*)e.norm_w;
   a.norm_eps = e.norm_eps;
   a.rope_pos = e.rope_pos;
@@ -122,11 +129,23 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   const int NW = 4;
   int ks = split_k;
   if (ks <= 0) {
+    // Launch-cost model (microseconds, measured per phase on MI355X): the k loop costs about
+    // 0.35 per block round (NW k tiles) with a floor of one memory round trip; splitting K adds a
+    // partial write, an arrival count and a partial read-back (about 2 + 0.05 per split) and only
+    // pays while the grid still fits the device twice over.
     ks = 1;
     if (blocks0 < cus) {
-      ks = (cus + blocks0 - 1) / blocks0;
-      const int max_by_k = a.KT / (NW * 2) > 1 ? a.KT / (NW * 2) : 1;  // keep >= 2 k tiles per wave
-      if (ks > max_by_k) ks = max_by_k;
+      float best = 1e30f;
+      for (int c = 1; c <= 64 && c * NW <= a.KT && (c == 1 || blocks0 * c <= 2 * cus); ++c) {
+        const int rounds = (a.KT + c * NW - 1) / (c * NW);
+        float t = rounds * 0.35f;
+        if (t < 1.0f) t = 1.0f;
+        if (c > 1) t += 2.0f + 0.05f * c;
+        if (t < best - 1e-3f) {
+          best = t;
+          ks = c;
+        }
+      }
     }
   }
   if (ks > a.KT) ks = a.KT;

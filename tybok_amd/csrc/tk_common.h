@@ -7,6 +7,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned short u16;
@@ -25,6 +26,23 @@ __device__ __forceinline__ u16 f32_to_bf16_bits(float f) {
   if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40);
   u += 0x7fffu + ((u >> 16) & 1u);
   return (u16)(u >> 16);
+}
+// two fp32 -> packed bf16 pair (lo = a, hi = b), round-to-nearest-even in one v_cvt_pk_bf16_f32
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
+  f32x2 v = {a, b};
+  union { bf16x2 h; unsigned u; } r;
+  r.h = __builtin_convertvector(v, bf16x2);
+  return r.u;
+}
+// four fp32 <-> four bf16 in two dwords
+__device__ __forceinline__ i32x2 pack_bf16x4(f32x4 v) {
+  i32x2 r = {(int)pack_bf16x2(v[0], v[1]), (int)pack_bf16x2(v[2], v[3])};
+  return r;
+}
+__device__ __forceinline__ f32x4 unpack_bf16x4(i32x2 r) {
+  f32x4 v = {__uint_as_float((unsigned)r[0] << 16), __uint_as_float((unsigned)r[0] & 0xffff0000u),
+             __uint_as_float((unsigned)r[1] << 16), __uint_as_float((unsigned)r[1] & 0xffff0000u)};
+  return v;
 }
 __device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
@@ -64,6 +82,14 @@ __device__ __forceinline__ void st_agent(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ float ld_agent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// two floats as one 8-byte device-coherent access
+__device__ __forceinline__ void st_agent64(unsigned long long* p, float lo, float hi) {
+  const unsigned long long v = (unsigned long long)__float_as_uint(lo) | ((unsigned long long)__float_as_uint(hi) << 32);
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long ld_agent64(const unsigned long long* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 

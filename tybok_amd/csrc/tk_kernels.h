@@ -24,6 +24,7 @@ struct GemmArgs {
   float* partial;
   int* counters;
   int act;
+  int vec;  // the plain epilogue may use 8/16-byte accesses (alignment and N % 4 checked by the host)
   // RMSNorm prologue (norm_w != nullptr): bf16 [K] weight, eps
   const unsigned short* norm_w;
   float norm_eps;
