@@ -150,14 +150,31 @@ int tk_pack_bf16_weight(const void* w, void* packed, int N, int K, int rope_half
  *              eager: tybok/policies/smolvla/models/rope.py:51-73).
  *   rope_pos: int32 [M] (clamped into [0, rope_positions)); rope_cos/rope_sin: fp32
  *             [rope_positions, rope_half].
+ *   vt:       optional (rotary epilogue only): the columns n >= vt_col0 (the value projection;
+ *             vt_col0 a head boundary >= rope_cols) are also written transposed,
+ *             vt[(n - vt_col0) * vt_ld + m], the suffix V^T operand of tk_expert_attn; entries
+ *             m >= M of a row are left as they are (keep them zero).
  * Built for the action-chunk tile shape (any M, tiled 64 rows at a time); the norm prologue is
  * built together with the rotary epilogue only. */
 int tk_bf16w_linear(const void* x, int ldx, int x_dtype, const void* w_packed, const void* norm_w, float norm_eps,
                     const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions,
-                    int rope_cols, int rope_half, void* y, int ldy, const void* resid, int ldr, int resid_dtype,
-                    int M, int N, int K, int split_k, void* ws, size_t ws_bytes, void* stream);
+                    int rope_cols, int rope_half, void* vt, int vt_col0, int vt_ld, void* y, int ldy,
+                    const void* resid, int ldr, int resid_dtype, int M, int N, int K, int split_k, void* ws,
+                    size_t ws_bytes, void* stream);
 
 /* ---- action-expert attention over the cached prefix ------------------------------------------ */
+/* Lays one layer's prefix K/V out for tk_expert_attn, once per request (the counterpart of the
+ * reference filling its static per-layer prefix cache after the VLM prefill,
+ * tybok/policies/smolvla/models/flow_matching.py:553-578):
+ *   k, v:   [L, G, D] of kv_dtype with element strides (sl, sh), d contiguous.
+ *   vt_hi:  bf16 [G, D, vt_ld] <- V transposed (keys contiguous), zero-filled from L to vt_ld;
+ *           vt_ld >= L rounded up to 32, a multiple of 8.
+ *   TK_BF16: k is used in place by the attention (k may be NULL here); k_hi/k_lo/vt_lo unused.
+ *   TK_F32 (the SmolVLA cross layers, whose expert K/V projections are fp32): K -> k_hi + k_lo
+ *           (bf16 [L, G, D] contiguous each, x = hi + lo to 16 mantissa bits), V^T -> vt_hi + vt_lo. */
+int tk_attn_prepare_kv(const void* k, const void* v, int kv_dtype, int sl, int sh, int L, int G, int D, void* k_hi,
+                       void* k_lo, void* vt_hi, void* vt_lo, int vt_ld, void* stream);
+
 /* out[M, H*D] (bf16) = softmax(q.K^T * D^-0.5 + mask) . V over keys [prefix(P); suffix(S)].
  * Replaces `EagerAttention._forward_eager` / `GemmaAttention._forward_eager`'s core and the fused
  * `triton_self_attn` / `triton_cross_attn` / `_splitk_flash_kernel`
@@ -165,19 +182,26 @@ int tk_bf16w_linear(const void* x, int ldx, int x_dtype, const void* w_packed, c
  *  tybok/policies/smolvla/models/triton_attn.py:586-855,
  *  tybok/policies/pi05/models/triton_expert_fused_qkv_rope_attn.py:322-433).
  *   q:      bf16 [M, H, D], element strides (q_sm, q_sh), d contiguous.
- *   k_pre/v_pre: [P, G, D] of kv_dtype (TK_BF16, or TK_F32 for the SmolVLA cross layers whose
- *           expert K/V projections are fp32), element strides (pre_sl, pre_sh).
- *   k_suf/v_suf: bf16 [S, G, D], strides (suf_sl, suf_sh); NULL when S == 0.
+ *   k_pre:  bf16 [P, G, D], element strides (pre_sl, pre_sh).
+ *   vt_pre: bf16 V^T [G, D, >= P rounded up to 32] (zero padded), element strides (pre_vt_sh, pre_vt_sd),
+ *           keys contiguous -- tk_attn_prepare_kv's output.
+ *   k_pre_lo / vt_pre_lo: low planes of fp32 K/V (same strides), or NULL for bf16 K/V; only with
+ *           S == 0 and D == 64 (the SmolVLA cross layers).
+ *   k_suf:  bf16 [S, G, D], strides (suf_sl, suf_sh); vt_suf: bf16 V^T [G, D, >= S rounded up to
+ *           32] (zero padded), strides (suf_vt_sh, suf_vt_sd) -- tk_bf16w_linear's `vt` output.
+ *           Both NULL when S == 0.
  *   pad:    uint8 [P], 1 = prefix token visible (NULL = all visible).
  *   mask_mode: TK_MASK_*; q head h reads kv head h / (H / G).
  *   logits_bf16: 0 = fp32 logits (SmolVLA); 1 = logits rounded to bf16 before the softmax and
  *           masked with the additive -2.3819763e38 (pi0.5).
  *   D in {64, 128, 256}; masked logits use finfo(float32).min, so a fully masked row is uniform.
+ *   out:    8-byte aligned, out_sm a multiple of 4.
  */
-int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* v_pre, int pre_sl,
-                   int pre_sh, int kv_dtype, const void* k_suf, const void* v_suf, int suf_sl, int suf_sh,
-                   const void* pad, void* out, int out_sm, int M, int P, int S, int H, int G, int D,
-                   int mask_mode, int logits_bf16, void* ws, size_t ws_bytes, void* stream);
+int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* k_pre_lo, int pre_sl, int pre_sh,
+                   const void* vt_pre, const void* vt_pre_lo, int pre_vt_sd, int pre_vt_sh, const void* k_suf,
+                   int suf_sl, int suf_sh, const void* vt_suf, int suf_vt_sd, int suf_vt_sh, const void* pad, void* out,
+                   int out_sm, int M, int P, int S, int H, int G, int D, int mask_mode, int logits_bf16, void* ws,
+                   size_t ws_bytes, void* stream);
 
 /* ---- diagnostics ------------------------------------------------------------------------------- */
 /* out_f32[256] = value of every e4m3fn code as decoded by the device's conversion instruction

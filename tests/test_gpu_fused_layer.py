@@ -81,6 +81,13 @@ def test_norm_qkv_rope(tk, m, k, heads, kv_heads, d, x_dtype):
     again = tk.bf16w_linear(x.cuda(), pw, **kw)
     assert torch.equal(got, again), "two launches on the same input differ"
     _close(got, want, f"norm+qkv+rope M={m} K={k} D={d} x={x_dtype}")
+    # the value columns also come out transposed (the attention kernel's suffix V^T operand)
+    v0 = (heads + kv_heads) * d
+    vt = torch.zeros(kv_heads * d, (m + 31) // 32 * 32, dtype=BF16, device="cuda")
+    with_vt = tk.bf16w_linear(x.cuda(), pw, vt_out=vt, vt_col0=v0, **kw)
+    assert torch.equal(with_vt, got)
+    assert torch.equal(vt[:, :m], got[:, v0:].t()), "transposed value output differs from the value columns"
+    assert not vt[:, m:].any(), "padding columns of V^T were written"
 
 
 def test_qkv_rope_without_norm_and_query_only(tk):

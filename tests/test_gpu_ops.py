@@ -166,8 +166,8 @@ def test_expert_attention(tk, m, p, h, g, d, mode, bl):
     pad = torch.ones(p, dtype=torch.bool)
     pad[torch.randperm(p, generator=torch.Generator().manual_seed(3))[: p // 7]] = False
     want = oops.expert_attention(q, k_pre, v_pre, k_suf, v_suf, pad, mode, bf16_logits=bl)
-    got = tk.expert_attn(q.cuda(), k_pre.cuda(), v_pre.cuda(), k_suf.cuda(), v_suf.cuda(), pad.cuda(), mode, logits_bf16=bl)
-    again = tk.expert_attn(q.cuda(), k_pre.cuda(), v_pre.cuda(), k_suf.cuda(), v_suf.cuda(), pad.cuda(), mode, logits_bf16=bl)
+    got = tk.expert_attn_plain(q.cuda(), k_pre.cuda(), v_pre.cuda(), k_suf.cuda(), v_suf.cuda(), pad.cuda(), mode, logits_bf16=bl)
+    again = tk.expert_attn_plain(q.cuda(), k_pre.cuda(), v_pre.cuda(), k_suf.cuda(), v_suf.cuda(), pad.cuda(), mode, logits_bf16=bl)
     assert torch.equal(got, again)
     _close(got, want, f"attn M={m} P={p} H={h} G={g} D={d} mode={mode}")
 
@@ -178,7 +178,7 @@ def test_cross_attention_fp32_kv(tk):
     pad = torch.ones(241, dtype=torch.bool)
     pad[200:] = False
     want = oops.expert_attention(q, k_pre, v_pre, None, None, pad, oops.MASK_NONE)
-    got = tk.expert_attn(q.cuda(), k_pre.cuda(), v_pre.cuda(), None, None, pad.cuda(), oops.MASK_NONE)
+    got = tk.expert_attn_plain(q.cuda(), k_pre.cuda(), v_pre.cuda(), None, None, pad.cuda(), oops.MASK_NONE)
     assert want.dtype == torch.float32
     _close(got, want.to(torch.bfloat16), "cross attn fp32 kv")
 
@@ -189,11 +189,11 @@ def test_attention_strided_kv_cache_views(tk):
     kbuf = torch.cat([k_pre, k_suf]).cuda()
     vbuf = torch.cat([v_pre, v_suf]).cuda()
     want = oops.expert_attention(q, k_pre, v_pre, k_suf, v_suf, torch.ones(177, dtype=torch.bool), oops.MASK_CAUSAL)
-    got = tk.expert_attn(q.cuda(), kbuf[:177], vbuf[:177], kbuf[177:], vbuf[177:], None, oops.MASK_CAUSAL)
+    got = tk.expert_attn_plain(q.cuda(), kbuf[:177], vbuf[:177], kbuf[177:], vbuf[177:], None, oops.MASK_CAUSAL)
     _close(got, want, "attn cache views")
     k_hm = k_pre.permute(1, 0, 2).contiguous().cuda().permute(1, 0, 2)  # [P, G, D] view of [G, P, D]
     v_hm = v_pre.permute(1, 0, 2).contiguous().cuda().permute(1, 0, 2)
-    got = tk.expert_attn(q.cuda(), k_hm, v_hm, k_suf.cuda(), v_suf.cuda(), None, oops.MASK_CAUSAL)
+    got = tk.expert_attn_plain(q.cuda(), k_hm, v_hm, k_suf.cuda(), v_suf.cuda(), None, oops.MASK_CAUSAL)
     _close(got, want, "attn head-major prefix")
 
 
@@ -201,7 +201,7 @@ def test_attention_fully_masked_prefix_is_uniform(tk):
     q, k_pre, v_pre, _, _ = attn_case(50, 64, 15, 5, 64, seed=3)
     none = torch.zeros(64, dtype=torch.bool)
     want = oops.expert_attention(q, k_pre, v_pre, None, None, none, oops.MASK_NONE)
-    got = tk.expert_attn(q.cuda(), k_pre.cuda(), v_pre.cuda(), None, None, none.cuda(), oops.MASK_NONE)
+    got = tk.expert_attn_plain(q.cuda(), k_pre.cuda(), v_pre.cuda(), None, None, none.cuda(), oops.MASK_NONE)
     _close(got, want, "attn fully masked")
 
 

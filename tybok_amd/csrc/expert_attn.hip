@@ -2,17 +2,25 @@
 //
 //   out[M, H*D] = softmax(q . K^T * D^-0.5 (+mask)) . V        (GQA: q head h -> kv head h/(H/G))
 //
-// Tiny and latency-bound (50 queries, a few hundred keys), so the grid is (head, 32-query tile,
-// kv split) and the four waves of a block take 32-key tiles round-robin:
-//   * S^T[key, q] = K . Q^T on v_mfma_f32_32x32x16_bf16: K rows are read from global memory in
-//     A-operand order (16 bytes per lane), Q is held in registers as the B operand.  In this
-//     orientation one lane owns one query column, so the softmax max/sum are in-lane plus one
-//     cross-half exchange (wavefront reduction), and P^T is already the B operand of P.V.
-//   * V tiles go through wave-private LDS (coalesced 16-byte rows in, key-strided 2-byte reads
-//     out) to form the A operand of O^T[d, q] += V^T . P^T.
-//   * fp32 K/V (SmolVLA cross layers) are split into bf16 hi + lo planes; P too (3 MFMAs).
+// Tiny and latency-bound (50 queries, a few hundred keys): the kernel is built so that a wave
+// issues every global load it needs up front and then runs a short, branch-light instruction
+// stream.  Grid = (head, 32-query tile, kv split); the four waves of a block take 32-key tiles
+// round-robin (normally one tile per wave).
+//   * Both MFMA operands stream from global memory in operand order, 16 bytes per lane, with no
+//     LDS staging: K rows as the A operand of S^T[key, q] = K . Q^T, and V from a TRANSPOSED
+//     cache V^T[kv head, d, key] as the A operand of O^T[d, q] += V^T . P^T.  The prefix V^T is
+//     laid out once per request (tk_attn_prepare_kv), the suffix V^T by the projection kernel's
+//     epilogue.  Keys beyond a segment's length read zero-padded V^T columns.
+//   * In this orientation one lane owns one query column, so the softmax max/sum are in-lane plus
+//     one cross-half exchange, and P^T is already the B operand of P.V.  K rows are assigned to
+//     lanes through a fixed permutation so that accumulator registers 8s..8s+7 of a lane are
+//     eight CONSECUTIVE keys -- exactly one 16-byte chunk of a V^T row.
+//   * fp32 K/V (SmolVLA cross layers) come as bf16 hi + lo planes (x = hi + lo to 16 mantissa
+//     bits), split once per request; P is split the same way in registers (3 MFMAs for P.V).
 //   * Online softmax per wave, then a fixed-order merge over waves (LDS) and kv splits (global
-//     partials, last-arriving block) -- deterministic, no atomics on data.
+//     partials handed over with device-coherent accesses, last-arriving block finishes) --
+//     deterministic, no atomics on data.  Wave w owns rows d = 8w + 4*(lane/32) + 0..3 of every
+//     output d tile in the merges and writes them as one 8-byte store per query.
 #include <math.h>
 #include "tk_common.h"
 #include "tk_kernels.h"
@@ -23,25 +31,24 @@ constexpr float kF32Min = -3.4028234663852886e38f;    // finfo(float32).min
 constexpr float kOpenpiMask = -2.3819763e38f;         // additive mask of the pi0.5 path
 constexpr int kNW = 4;
 
+// K row held by MFMA row r of a key tile: swaps bits 2 and 3 of r (see the header comment)
+__device__ __forceinline__ int key_of_row(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
+
 __device__ __forceinline__ bf16x8 pack_bf16x8(const float* v) {
-  union { u16 h[8]; bf16x8 b; } u;
+  union { unsigned u[4]; bf16x8 b; } r;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) u.h[j] = f32_to_bf16_bits(v[j]);
-  return u.b;
+  for (int j = 0; j < 4; ++j) r.u[j] = pack_bf16x2(v[2 * j], v[2 * j + 1]);
+  return r.b;
 }
 
-template <int D, bool KVF32>
+template <int D, bool SPLIT>
 __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
   constexpr int DT = D / 32;                 // d tiles of the output
   constexpr int DS = D / 16;                 // k steps of Q.K^T
-  constexpr int DCH = D > 128 ? 128 : D;     // d columns staged per V pass
-  constexpr int NPASS = D / DCH;
-  constexpr int VP = DCH + 8;                // LDS row pitch (u16 elements)
-  constexpr int PLANES = KVF32 ? 2 : 1;
-  constexpr int STAGE_BYTES = kNW * PLANES * 32 * VP * 2;
-  constexpr int MERGE_BYTES = kNW * 2 * 16 * 64 * 4 + kNW * 2 * 32 * 4;
-  constexpr int SMEM = STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES;
-  __shared__ __align__(16) unsigned char smem[SMEM];
+  constexpr int PL = SPLIT ? 2 : 1;          // operand planes (hi, lo)
+  constexpr int PF = D <= 128 ? 2 : 1;       // key tiles in flight per wave
+  __shared__ __align__(16) f32x4 red[2][kNW][4][64];
+  __shared__ float st_m[kNW][32], st_l[kNW][32];
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -51,24 +58,57 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
   const int mtile = blockIdx.y;
   const int split = blockIdx.z;
   const int g = h / (a.H / a.G);
-  const int L = a.P + a.S;
-  const int ntiles = (L + 31) / 32;
+  const int tp = (a.P + 31) >> 5;            // prefix tiles; suffix tiles follow
+  const int ntiles = tp + ((a.S + 31) >> 5);
   const int t_lo = (split * ntiles) / a.kv_splits;
   const int t_hi = ((split + 1) * ntiles) / a.kv_splits;
   const int qi = mtile * 32 + l32;
   const bool q_ok = qi < a.M;
 
-  // ---- Q as B operand, resident in registers ----
-  bf16x8 qf[DS];
-  {
-    const u16* qp = a.q + (size_t)qi * a.q_sm + (size_t)h * a.q_sh + 8 * half;
+  struct Stage {
+    i32x4 k[PL][DS];
+    i32x4 v[PL][DT][2];
+    int pad;
+  };
+  // every load of a key tile, issued back to back (t is wave-uniform)
+  auto load = [&](Stage& st, int t) {
+    const bool pre = t < tp;
+    const int tt = pre ? t : t - tp;
+    const int len = pre ? a.P : a.S;
+    int kr = tt * 32 + key_of_row(l32);
+    if (kr > len - 1) kr = len - 1;  // masked below; keeps the address valid and the value finite
+    const size_t koff = (size_t)kr * (pre ? a.pre_sl : a.suf_sl) + (size_t)g * (pre ? a.pre_sh : a.suf_sh) + 8 * half;
+    const size_t vsd = pre ? a.pre_vt_sd : a.suf_vt_sd;
+    const size_t voff = (size_t)g * (pre ? a.pre_vt_sh : a.suf_vt_sh) + (size_t)l32 * vsd + tt * 32 + 8 * half;
 #pragma unroll
-    for (int st = 0; st < DS; ++st) {
-      i32x4 v = {0, 0, 0, 0};
-      if (q_ok) v = *(const i32x4*)(qp + 16 * st);
-      qf[st] = as_bf16x8(v);
+    for (int pl = 0; pl < PL; ++pl) {
+      const u16* kb = pre ? (pl ? a.k_pre_lo : a.k_pre) : a.k_suf;
+      const u16* vb = pre ? (pl ? a.vt_pre_lo : a.vt_pre) : a.vt_suf;
+#pragma unroll
+      for (int s = 0; s < DS; ++s) st.k[pl][s] = *(const i32x4*)(kb + koff + 16 * s);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) st.v[pl][dt][s] = *(const i32x4*)(vb + voff + (size_t)dt * 32 * vsd + 16 * s);
     }
+    st.pad = 1;
+    if (pre && a.pad) {
+      const int key = tt * 32 + l32;
+      st.pad = key < a.P ? a.pad[key] : 0;
+    }
+  };
+
+  // ---- Q as B operand, resident in registers; the first tiles' loads go out with it ----
+  bf16x8 qf[DS];
+  Stage stg[PF];
+  {
+    const u16* qp = a.q + (size_t)(q_ok ? qi : a.M - 1) * a.q_sm + (size_t)h * a.q_sh + 8 * half;
+#pragma unroll
+    for (int s = 0; s < DS; ++s) qf[s] = as_bf16x8(*(const i32x4*)(qp + 16 * s));
   }
+#pragma unroll
+  for (int p = 0; p < PF; ++p)
+    if (t_lo + wave + kNW * p < t_hi) load(stg[p], t_lo + wave + kNW * p);
 
   f32x16 o[DT];
 #pragma unroll
@@ -77,65 +117,33 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
     for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  u16* vstage = (u16*)smem + (size_t)wave * PLANES * 32 * VP;
-
-  for (int t = t_lo + wave; t < t_hi; t += kNW) {
+  auto process = [&](const Stage& st, int t) {
+    const bool pre = t < tp;
+    const int tt = pre ? t : t - tp;
+    const int len = pre ? a.P : a.S;
     // ---- S^T tile = K . Q^T ----
     f32x16 sT;
 #pragma unroll
     for (int i = 0; i < 16; ++i) sT[i] = 0.f;
-    {
-      const int kr = t * 32 + l32;
-      const bool k_ok = kr < L;
-      const bool in_pre = kr < a.P;
-      if (KVF32) {
-        const float* kp = (const float*)a.k_pre + (size_t)kr * a.pre_sl + (size_t)g * a.pre_sh + 8 * half;
 #pragma unroll
-        for (int st = 0; st < DS; ++st) {
-          float f[8], lo[8];
+    for (int s = 0; s < DS; ++s)
 #pragma unroll
-          for (int j = 0; j < 8; ++j) f[j] = 0.f;
-          if (k_ok) {
-            const float4* p4 = (const float4*)(kp + 16 * st);
-            float4 x0 = p4[0], x1 = p4[1];
-            f[0] = x0.x; f[1] = x0.y; f[2] = x0.z; f[3] = x0.w;
-            f[4] = x1.x; f[5] = x1.y; f[6] = x1.z; f[7] = x1.w;
-          }
-#pragma unroll
-          for (int j = 0; j < 8; ++j) lo[j] = f[j] - round_bf16(f[j]);
-          sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pack_bf16x8(f), qf[st], sT, 0, 0, 0);
-          sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pack_bf16x8(lo), qf[st], sT, 0, 0, 0);
-        }
-      } else {
-        const u16* kp = in_pre ? (const u16*)a.k_pre + (size_t)kr * a.pre_sl + (size_t)g * a.pre_sh
-                               : a.k_suf + (size_t)(kr - a.P) * a.suf_sl + (size_t)g * a.suf_sh;
-        kp += 8 * half;
-#pragma unroll
-        for (int st = 0; st < DS; ++st) {
-          i32x4 v = {0, 0, 0, 0};
-          if (k_ok) v = *(const i32x4*)(kp + 16 * st);
-          sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(v), qf[st], sT, 0, 0, 0);
-        }
-      }
-    }
+      for (int pl = 0; pl < PL; ++pl) sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(st.k[pl][s]), qf[s], sT, 0, 0, 0);
 
     // ---- scale, mask, online softmax (one query column per lane) ----
+    const unsigned pmask = (unsigned)__ballot(st.pad != 0);  // lanes 0..31: keys of this tile
     float p[16];
     float tmax = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int key = t * 32 + mfma32_row(lane, i);
+      const int kl = 16 * (i >> 3) + 8 * half + (i & 7);  // key within the tile held by register i
+      const int key = tt * 32 + kl;
       float s = sT[i];
       if (a.logits_bf16) s = round_bf16(s);
       s *= a.scale;
-      bool vis;
-      if (key < a.P) {
-        vis = a.pad ? (a.pad[key < L ? key : 0] != 0) : true;
-      } else {
-        vis = (a.mask_mode == 1) || ((key - a.P) <= qi);
-      }
+      const bool vis = pre ? ((pmask >> kl) & 1u) != 0 : (a.mask_mode == 1 || key <= qi);
       if (!vis) s = a.logits_bf16 ? (s + kOpenpiMask) : kF32Min;
-      if (key >= L) s = -INFINITY;
+      if (key >= len) s = -INFINITY;
       p[i] = s;
       tmax = fmaxf(tmax, s);
     }
@@ -151,209 +159,224 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
     lsum += __shfl_xor(lsum, 32);
     l_run = l_run * alpha + lsum;
     m_run = m_new;
+    if (alpha != 1.0f) {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+        for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+    }
 
-    // P^T as B operand: step s uses registers 8s..8s+7 (keys 8*(2s+j/4) + 4*half + j%4)
+    // P^T as B operand: step s uses registers 8s..8s+7 = keys 16s + 8*half + 0..7
     bf16x8 pb[2], pbl[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       pb[s] = pack_bf16x8(p + 8 * s);
-      if (KVF32) {
+      if (SPLIT) {
         float lo[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) lo[j] = p[8 * s + j] - round_bf16(p[8 * s + j]);
         pbl[s] = pack_bf16x8(lo);
       }
     }
+    // ---- O^T += V^T . P^T ----
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(st.v[0][dt][s]), pb[s], o[dt], 0, 0, 0);
+        if (SPLIT) {
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(st.v[PL - 1][dt][s]), pb[s], o[dt], 0, 0, 0);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(st.v[0][dt][s]), pbl[s], o[dt], 0, 0, 0);
+        }
+      }
+  };
 
-    // ---- O^T += V^T . P^T, V staged through wave-private LDS ----
+  for (int t = t_lo + wave; t < t_hi; t += kNW * PF) {
 #pragma unroll
-    for (int pass = 0; pass < NPASS; ++pass) {
-      constexpr int CH_PER_ROW = DCH / 8;  // 16-byte chunks per staged row
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int c0 = 0; c0 < 32 * CH_PER_ROW; c0 += 64) {
-        const int c = c0 + lane;
-        const int kl = c / CH_PER_ROW;
-        const int dc = c % CH_PER_ROW;
-        const int kv = t * 32 + kl;
-        const int dcol = pass * DCH + dc * 8;
-        if (KVF32) {
-          float f[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j) f[j] = 0.f;
-          if (kv < L) {
-            const float4* p4 =
-                (const float4*)((const float*)a.v_pre + (size_t)kv * a.pre_sl + (size_t)g * a.pre_sh + dcol);
-            float4 x0 = p4[0], x1 = p4[1];
-            f[0] = x0.x; f[1] = x0.y; f[2] = x0.z; f[3] = x0.w;
-            f[4] = x1.x; f[5] = x1.y; f[6] = x1.z; f[7] = x1.w;
-          }
-          float lo[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j) lo[j] = f[j] - round_bf16(f[j]);
-          union { bf16x8 b; i32x4 i; } uh, ul;
-          uh.b = pack_bf16x8(f);
-          ul.b = pack_bf16x8(lo);
-          *(i32x4*)(vstage + (size_t)kl * VP + dc * 8) = uh.i;
-          *(i32x4*)(vstage + (size_t)(32 + kl) * VP + dc * 8) = ul.i;
-        } else {
-          i32x4 v = {0, 0, 0, 0};
-          if (kv < L) {
-            const u16* vp = kv < a.P ? (const u16*)a.v_pre + (size_t)kv * a.pre_sl + (size_t)g * a.pre_sh
-                                     : a.v_suf + (size_t)(kv - a.P) * a.suf_sl + (size_t)g * a.suf_sh;
-            v = *(const i32x4*)(vp + dcol);
-          }
-          *(i32x4*)(vstage + (size_t)kl * VP + dc * 8) = v;
-        }
+    for (int p = 0; p < PF; ++p) {
+      const int tc = t + kNW * p;
+      if (tc < t_hi) {  // wave-uniform
+        process(stg[p], tc);
+        if (tc + kNW * PF < t_hi) load(stg[p], tc + kNW * PF);
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int dl = 0; dl < DCH / 32; ++dl) {
-        const int dt = pass * (DCH / 32) + dl;
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-          union { u16 hh[8]; bf16x8 b; } va, vl;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const int kl = 8 * (2 * s + (j >> 2)) + 4 * half + (j & 3);
-            va.hh[j] = vstage[(size_t)kl * VP + dl * 32 + l32];
-            if (KVF32) vl.hh[j] = vstage[(size_t)(32 + kl) * VP + dl * 32 + l32];
-          }
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va.b, pb[s], o[dt], 0, 0, 0);
-          if (KVF32) {
-            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vl.b, pb[s], o[dt], 0, 0, 0);
-            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va.b, pbl[s], o[dt], 0, 0, 0);
-          }
-        }
-      }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
   }
 
-  // ---- merge the four waves in fixed order (LDS), two d tiles per round ----
-  float* st_m = (float*)smem;                 // [kNW][32]
-  float* st_l = st_m + kNW * 32;              // [kNW][32]
-  float* obuf = st_l + kNW * 32;              // [kNW][2][16][64]
-  __syncthreads();                            // staging region is dead from here on
+  // ---- merge the four waves in fixed order (LDS) ----
   if (half == 0) {
-    st_m[wave * 32 + l32] = m_run;
-    st_l[wave * 32 + l32] = l_run;
+    st_m[wave][l32] = m_run;
+    st_l[wave][l32] = l_run;
   }
-  const int blk_lin = mtile * a.H + h;
-  float* part_stats = a.partial;  // [blk][split][2][32]
-  float* part_o = a.partial + (size_t)gridDim.x * gridDim.y * a.kv_splits * 64;  // [blk][split][DT][16][64]
-  float bm = 0.f, bl = 0.f;       // block-level (m, l) of this lane's query
+  f32x4 own[DT];
+  float ew[kNW];
+  float bm = -INFINITY, bl = 0.f;  // block-level (m, l) of this lane's query
 #pragma unroll
-  for (int r = 0; r < DT / 2; ++r) {
+  for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
-    for (int dd = 0; dd < 2; ++dd)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) obuf[((wave * 2 + dd) * 16 + i) * 64 + lane] = o[2 * r + dd][i];
-    __syncthreads();
-    if (wave < 2) {
-      const int dd = wave;
-      const int dt = 2 * r + dd;
-      float mw[kNW], ew[kNW];
-      float mt = -INFINITY;
-#pragma unroll
-      for (int w = 0; w < kNW; ++w) {
-        mw[w] = st_m[w * 32 + l32];
-        mt = fmaxf(mt, mw[w]);
-      }
-      float lt = 0.f;
-#pragma unroll
-      for (int w = 0; w < kNW; ++w) {
-        ew[w] = (mw[w] == -INFINITY) ? 0.f : __expf(mw[w] - mt);
-        lt += st_l[w * 32 + l32] * ew[w];
-      }
-      bm = mt;
-      bl = lt;
-      float accv[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float s = 0.f;
-#pragma unroll
-        for (int w = 0; w < kNW; ++w) s += obuf[((w * 2 + dd) * 16 + i) * 64 + lane] * ew[w];
-        accv[i] = s;
-      }
-      if (a.kv_splits == 1) {
-        if (q_ok) {
-          const float inv = 1.0f / lt;
-          u16* op = a.out + (size_t)qi * a.out_sm + (size_t)h * D + dt * 32;
-#pragma unroll
-          for (int i = 0; i < 16; ++i) op[mfma32_row(lane, i)] = f32_to_bf16_bits(accv[i] * inv);
-        }
-      } else {
-        float* dst = part_o + ((((size_t)blk_lin * a.kv_splits + split) * DT + dt) * 16) * 64 + lane;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i * 64] = accv[i];
-      }
+    for (int gq = 0; gq < 4; ++gq) {
+      f32x4 v = {o[dt][4 * gq], o[dt][4 * gq + 1], o[dt][4 * gq + 2], o[dt][4 * gq + 3]};
+      red[dt & 1][wave][gq][lane] = v;
     }
     __syncthreads();
+    if (dt == 0) {
+      float mw[kNW];
+#pragma unroll
+      for (int w = 0; w < kNW; ++w) {
+        mw[w] = st_m[w][l32];
+        bm = fmaxf(bm, mw[w]);
+      }
+#pragma unroll
+      for (int w = 0; w < kNW; ++w) {
+        ew[w] = (mw[w] == -INFINITY) ? 0.f : __expf(mw[w] - bm);
+        bl += st_l[w][l32] * ew[w];
+      }
+    }
+    f32x4 sum = red[dt & 1][0][wave][lane] * ew[0];
+#pragma unroll
+    for (int w = 1; w < kNW; ++w) sum += red[dt & 1][w][wave][lane] * ew[w];
+    own[dt] = sum;
   }
-  if (a.kv_splits == 1) return;
+
+  // this lane's output: query qi, columns d0 .. d0+3 of every d tile
+  u16* op = a.out + (size_t)(q_ok ? qi : 0) * a.out_sm + (size_t)h * D + 8 * wave + 4 * half;
+  if (a.kv_splits == 1) {
+    if (q_ok) {
+      const float inv = 1.0f / bl;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *(i32x2*)(op + dt * 32) = pack_bf16x4(own[dt] * inv);
+    }
+    return;
+  }
 
   // ---- kv-split merge by the last-arriving block ----
+  // partials per (block, split): [2][32] stats, then [DT][4 groups][64 lanes][4 floats]
+  const int blk_lin = mtile * a.H + h;
+  constexpr size_t PSTRIDE = 64 + (size_t)DT * 1024;  // floats
+  float* pmine = a.partial + ((size_t)blk_lin * a.kv_splits + split) * PSTRIDE;
   if (wave == 0 && half == 0) {
-    float* ps = part_stats + ((size_t)blk_lin * a.kv_splits + split) * 64;
-    ps[l32] = bm;
-    ps[32 + l32] = bl;
+    st_agent(pmine + l32, bm);
+    st_agent(pmine + 32 + l32, bl);
+  }
+  {
+    unsigned long long* dst = (unsigned long long*)(pmine + 64) + ((size_t)wave * 64 + lane) * 2;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      st_agent64(dst + (size_t)dt * 512, own[dt][0], own[dt][1]);
+      st_agent64(dst + (size_t)dt * 512 + 1, own[dt][2], own[dt][3]);
+    }
   }
   __shared__ int s_last;
-  __threadfence();
+  __builtin_amdgcn_s_waitcnt(0);  // partials acknowledged (written through) before the count
   __syncthreads();
   if (threadIdx.x == 0) {
-    int old = atomicAdd(a.counters + blk_lin, 1);
+    int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s_last = (old == a.kv_splits - 1);
   }
   __syncthreads();
   if (!s_last) return;
-  __threadfence();
+  if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+  constexpr int MAXS = 8;  // the host never asks for more kv splits
+  const float* pblk = a.partial + (size_t)blk_lin * a.kv_splits * PSTRIDE;
+  float ms[MAXS], ls[MAXS], es[MAXS];
+#pragma unroll
+  for (int s = 0; s < MAXS; ++s) {
+    const int sc = s < a.kv_splits ? s : a.kv_splits - 1;
+    ms[s] = ld_agent(pblk + (size_t)sc * PSTRIDE + l32);
+    ls[s] = ld_agent(pblk + (size_t)sc * PSTRIDE + 32 + l32);
+  }
   float mt = -INFINITY;
-  for (int s = 0; s < a.kv_splits; ++s) mt = fmaxf(mt, part_stats[((size_t)blk_lin * a.kv_splits + s) * 64 + l32]);
+#pragma unroll
+  for (int s = 0; s < MAXS; ++s)
+    if (s < a.kv_splits) mt = fmaxf(mt, ms[s]);
   float lt = 0.f;
-  for (int s = 0; s < a.kv_splits; ++s) {
-    const float* ps = part_stats + ((size_t)blk_lin * a.kv_splits + s) * 64;
-    const float e = (ps[l32] == -INFINITY) ? 0.f : __expf(ps[l32] - mt);
-    lt += ps[32 + l32] * e;
+#pragma unroll
+  for (int s = 0; s < MAXS; ++s) {
+    es[s] = (s < a.kv_splits && ms[s] != -INFINITY) ? __expf(ms[s] - mt) : 0.f;
+    if (s < a.kv_splits) lt += ls[s] * es[s];
   }
   const float inv = 1.0f / lt;
-  for (int dt = wave; dt < DT; dt += kNW) {
-    float accv[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) accv[i] = 0.f;
-    for (int s = 0; s < a.kv_splits; ++s) {
-      const float ms = part_stats[((size_t)blk_lin * a.kv_splits + s) * 64 + l32];
-      const float e = (ms == -INFINITY) ? 0.f : __expf(ms - mt);
-      const float* src = part_o + ((((size_t)blk_lin * a.kv_splits + s) * DT + dt) * 16) * 64 + lane;
+  for (int dt = 0; dt < DT; ++dt) {
+    unsigned long long raw[MAXS][2];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) accv[i] += src[i * 64] * e;
+    for (int s = 0; s < MAXS; ++s) {
+      const int sc = s < a.kv_splits ? s : a.kv_splits - 1;
+      const unsigned long long* src =
+          (const unsigned long long*)(pblk + (size_t)sc * PSTRIDE + 64) + (size_t)dt * 512 + ((size_t)wave * 64 + lane) * 2;
+      raw[s][0] = ld_agent64(src);
+      raw[s][1] = ld_agent64(src + 1);
     }
-    if (q_ok) {
-      u16* op = a.out + (size_t)qi * a.out_sm + (size_t)h * D + dt * 32;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < 16; ++i) op[mfma32_row(lane, i)] = f32_to_bf16_bits(accv[i] * inv);
+    for (int s = 0; s < MAXS; ++s) {
+      if (s < a.kv_splits) {
+        f32x4 v = {__uint_as_float((unsigned)raw[s][0]), __uint_as_float((unsigned)(raw[s][0] >> 32)),
+                   __uint_as_float((unsigned)raw[s][1]), __uint_as_float((unsigned)(raw[s][1] >> 32))};
+        acc += v * es[s];
+      }
     }
+    if (q_ok) *(i32x2*)(op + dt * 32) = pack_bf16x4(acc * inv);
   }
-  if (threadIdx.x == 0) a.counters[blk_lin] = 0;
 }
 
-template <int D, bool KVF32>
+// Lays a [L, G, D] K/V pair out for the attention kernel: V transposed to [G, D, ld] (keys
+// contiguous, zero-filled from L to ld), and -- for fp32 sources -- K and V^T split into bf16
+// hi + lo planes.  One thread per (key, kv head, 8 d columns).
+__global__ void kv_prepare_kernel(KvPrepArgs p) {
+  const int chunks = p.D / 8;
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long total = (long long)p.ld * p.G * chunks;
+  if (idx >= total) return;
+  const int dc = (int)(idx % chunks);
+  const int g = (int)((idx / chunks) % p.G);
+  const int key = (int)(idx / ((long long)chunks * p.G));
+  float kf[8], vf[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) kf[j] = vf[j] = 0.f;
+  if (key < p.L) {
+    const size_t off = (size_t)key * p.sl + (size_t)g * p.sh + dc * 8;
+    if (p.f32) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        kf[j] = ((const float*)p.k)[off + j];
+        vf[j] = ((const float*)p.v)[off + j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) vf[j] = bf16_bits_to_f32(((const u16*)p.v)[off + j]);
+    }
+  }
+  const size_t vt0 = ((size_t)g * p.D + dc * 8) * p.ld + key;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const u16 hi = f32_to_bf16_bits(vf[j]);
+    p.vt_hi[vt0 + (size_t)j * p.ld] = hi;
+    if (p.f32) p.vt_lo[vt0 + (size_t)j * p.ld] = f32_to_bf16_bits(vf[j] - bf16_bits_to_f32(hi));
+  }
+  if (p.f32 && key < p.L) {
+    const size_t ko = ((size_t)key * p.G + g) * p.D + dc * 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const u16 hi = f32_to_bf16_bits(kf[j]);
+      p.k_hi[ko + j] = hi;
+      p.k_lo[ko + j] = f32_to_bf16_bits(kf[j] - bf16_bits_to_f32(hi));
+    }
+  }
+}
+
+template <int D, bool SPLIT>
 int launch_attn(const AttnArgs& a, hipStream_t st) {
   dim3 grid(a.H, (a.M + 31) / 32, a.kv_splits);
-  hipLaunchKernelGGL((expert_attn_kernel<D, KVF32>), grid, dim3(kNW * 64), 0, st, a);
+  hipLaunchKernelGGL((expert_attn_kernel<D, SPLIT>), grid, dim3(kNW * 64), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
 }  // namespace
 
-int tk_launch_attn(AttnArgs a, int D, int kv_f32, hipStream_t st) {
-  if (kv_f32) {
+int tk_launch_attn(AttnArgs a, int D, hipStream_t st) {
+  const bool split = a.k_pre_lo != nullptr;
+  if (split) {
     if (D == 64) return launch_attn<64, true>(a, st);
     return -1;
   }
@@ -361,4 +384,10 @@ int tk_launch_attn(AttnArgs a, int D, int kv_f32, hipStream_t st) {
   if (D == 128) return launch_attn<128, false>(a, st);
   if (D == 256) return launch_attn<256, false>(a, st);
   return -1;
+}
+
+int tk_launch_kv_prepare(KvPrepArgs p, hipStream_t st) {
+  const long long total = (long long)p.ld * p.G * (p.D / 8);
+  hipLaunchKernelGGL(kv_prepare_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, p);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
 }

@@ -485,8 +485,19 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
           va = ra;
           vb = rb;
         }
-        *(i32x2*)(a.y + (size_t)m * a.ldy + ca) = pack_bf16x4(va);
-        *(i32x2*)(a.y + (size_t)m * a.ldy + cb) = pack_bf16x4(vb);
+        const i32x2 pa = pack_bf16x4(va), pbv = pack_bf16x4(vb);
+        *(i32x2*)(a.y + (size_t)m * a.ldy + ca) = pa;
+        *(i32x2*)(a.y + (size_t)m * a.ldy + cb) = pbv;
+        if (a.vt && ca >= a.vt_col0) {  // tile-uniform: vt_col0 is a multiple of the head size
+          // value columns, transposed for the attention kernel (lanes = consecutive rows m)
+          u16* va_t = a.vt + (size_t)(ca - a.vt_col0) * a.vt_ld + m;
+          u16* vb_t = a.vt + (size_t)(cb - a.vt_col0) * a.vt_ld + m;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            va_t[(size_t)j * a.vt_ld] = (u16)(((unsigned)pa[j >> 1]) >> (16 * (j & 1)));
+            vb_t[(size_t)j * a.vt_ld] = (u16)(((unsigned)pbv[j >> 1]) >> (16 * (j & 1)));
+          }
+        }
       }
     }
   }

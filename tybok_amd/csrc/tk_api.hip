@@ -52,6 +52,8 @@ struct GemmExtra {
   const float* rope_cos = nullptr;
   const float* rope_sin = nullptr;
   int rope_positions = 0, rope_cols = 0, rope_half = 0;
+  void* vt = nullptr;  // transposed copy of the columns >= vt_col0 (rotary epilogue)
+  int vt_col0 = 0, vt_ld = 0;
 };
 
 // One GEMM launch (plain, gated or rotary).  `N` is the logical output width.
@@ -106,6 +108,11 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
     return fail(TK_EINVAL, "gemm: this epilogue needs ldy %% 4 == 0, an 8-byte aligned y and 16-byte aligned scales");
   if (rope && (!aligned16(e.rope_cos) || !aligned16(e.rope_sin)))
     return fail(TK_EINVAL, "gemm: rotary tables must be 16-byte aligned");
+  if (e.vt) {
+    if (!rope) return fail(TK_EINVAL, "gemm: the transposed value output belongs to the rotary epilogue");
+    if (e.vt_col0 < e.rope_cols || e.vt_col0 > N || e.vt_col0 % (2 * e.rope_half) || e.vt_ld < M)
+      return fail(TK_EINVAL, "gemm: vt_col0=%d must be a head boundary in [rope_cols, N] and vt_ld=%d >= M", e.vt_col0, e.vt_ld);
+  }
   a.norm_w = (const u16*)e.norm_w;
   a.norm_eps = e.norm_eps;
   a.rope_pos = e.rope_pos;
@@ -114,6 +121,9 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   a.rope_positions = e.rope_positions;
   a.rope_cols = e.rope_cols;
   a.rope_half = e.rope_half;
+  a.vt = (u16*)e.vt;
+  a.vt_col0 = e.vt_col0;
+  a.vt_ld = e.vt_ld;
 
   const int cus = device_cus();
   int MT = M <= 32 ? 1 : 2;
@@ -253,8 +263,8 @@ int tk_pack_bf16_weight(const void* w, void* packed, int N, int K, int rope_half
 
 int tk_bf16w_linear(const void* x, int ldx, int x_dtype, const void* w_packed, const void* norm_w, float norm_eps,
                     const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions, int rope_cols,
-                    int rope_half, void* y, int ldy, const void* resid, int ldr, int resid_dtype, int M, int N, int K,
-                    int split_k, void* ws, size_t ws_bytes, void* stream) {
+                    int rope_half, void* vt, int vt_col0, int vt_ld, void* y, int ldy, const void* resid, int ldr,
+                    int resid_dtype, int M, int N, int K, int split_k, void* ws, size_t ws_bytes, void* stream) {
   if (x_dtype != TK_BF16 && x_dtype != TK_F32) return fail(TK_EINVAL, "bf16w_linear: bad x_dtype");
   GemmExtra e;
   e.x_f32 = x_dtype == TK_F32;
@@ -267,6 +277,9 @@ int tk_bf16w_linear(const void* x, int ldx, int x_dtype, const void* w_packed, c
   e.rope_positions = rope_positions;
   e.rope_cols = rope_cols;
   e.rope_half = rope_half;
+  e.vt = vt;
+  e.vt_col0 = vt_col0;
+  e.vt_ld = vt_ld;
   if (!rope_pos && norm_w) return fail(TK_EINVAL, "bf16w_linear: the norm prologue is built for the rotary projection only");
   return gemm_common(x, ldx, w_packed, nullptr, nullptr, y, ldy, resid, ldr, resid_dtype, nullptr, M, N, K, split_k, 0, ws,
                      ws_bytes, (hipStream_t)stream, e);
@@ -294,38 +307,75 @@ int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float nor
                      ws, ws_bytes, (hipStream_t)stream);
 }
 
-int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* v_pre, int pre_sl, int pre_sh,
-                   int kv_dtype, const void* k_suf, const void* v_suf, int suf_sl, int suf_sh, const void* pad,
-                   void* out, int out_sm, int M, int P, int S, int H, int G, int D, int mask_mode, int logits_bf16,
-                   void* ws, size_t ws_bytes, void* stream) {
+int tk_attn_prepare_kv(const void* k, const void* v, int kv_dtype, int sl, int sh, int L, int G, int D, void* k_hi,
+                       void* k_lo, void* vt_hi, void* vt_lo, int vt_ld, void* stream) {
+  if (L <= 0 || G <= 0 || D <= 0 || D % 8) return fail(TK_EINVAL, "prepare_kv: bad shape L=%d G=%d D=%d", L, G, D);
+  if (kv_dtype != TK_BF16 && kv_dtype != TK_F32) return fail(TK_EINVAL, "prepare_kv: bad kv_dtype");
+  if (vt_ld < ((L + 31) / 32) * 32 || vt_ld % 8) return fail(TK_EINVAL, "prepare_kv: vt_ld=%d must be >= L rounded up to 32", vt_ld);
+  if (!v || !vt_hi) return fail(TK_EINVAL, "prepare_kv: null pointer");
+  if (kv_dtype == TK_F32 && (!k || !k_hi || !k_lo || !vt_lo)) return fail(TK_EINVAL, "prepare_kv: fp32 sources need all four planes");
+  KvPrepArgs p;
+  p.k = k;
+  p.v = v;
+  p.f32 = kv_dtype == TK_F32;
+  p.sl = sl;
+  p.sh = sh;
+  p.L = L;
+  p.G = G;
+  p.D = D;
+  p.k_hi = (u16*)k_hi;
+  p.k_lo = (u16*)k_lo;
+  p.vt_hi = (u16*)vt_hi;
+  p.vt_lo = (u16*)vt_lo;
+  p.ld = vt_ld;
+  if (tk_launch_kv_prepare(p, (hipStream_t)stream)) return fail(TK_ELAUNCH, "prepare_kv: launch failed");
+  return TK_OK;
+}
+
+int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* k_pre_lo, int pre_sl, int pre_sh,
+                   const void* vt_pre, const void* vt_pre_lo, int pre_vt_sd, int pre_vt_sh, const void* k_suf, int suf_sl,
+                   int suf_sh, const void* vt_suf, int suf_vt_sd, int suf_vt_sh, const void* pad, void* out, int out_sm,
+                   int M, int P, int S, int H, int G, int D, int mask_mode, int logits_bf16, void* ws, size_t ws_bytes,
+                   void* stream) {
   if (M <= 0 || P < 0 || S < 0 || P + S <= 0 || H <= 0 || G <= 0 || H % G)
     return fail(TK_EINVAL, "attn: bad shape M=%d P=%d S=%d H=%d G=%d", M, P, S, H, G);
   if (D != 64 && D != 128 && D != 256) return fail(TK_EINVAL, "attn: head_dim %d not in {64,128,256}", D);
-  if (kv_dtype != TK_BF16 && kv_dtype != TK_F32) return fail(TK_EINVAL, "attn: bad kv_dtype");
-  if (kv_dtype == TK_F32 && (S != 0 || D != 64))
-    return fail(TK_EINVAL, "attn: fp32 K/V is supported for prefix-only attention with head_dim 64");
+  const bool split = k_pre_lo != nullptr || vt_pre_lo != nullptr;
+  if (split && (!k_pre_lo || !vt_pre_lo)) return fail(TK_EINVAL, "attn: hi/lo planes need both K and V^T low planes");
+  if (split && (S != 0 || D != 64))
+    return fail(TK_EINVAL, "attn: hi/lo (fp32) K/V is supported for prefix-only attention with head_dim 64");
   if (mask_mode < 0 || mask_mode > 2) return fail(TK_EINVAL, "attn: bad mask_mode %d", mask_mode);
   if (S > 0 && mask_mode == TK_MASK_NONE) return fail(TK_EINVAL, "attn: suffix keys need a suffix mask mode");
-  if (!q || !out || (P > 0 && (!k_pre || !v_pre)) || (S > 0 && (!k_suf || !v_suf)))
+  if (!q || !out || (P > 0 && (!k_pre || !vt_pre)) || (S > 0 && (!k_suf || !vt_suf)))
     return fail(TK_EINVAL, "attn: null pointer");
-  if (q_sm % 8 || q_sh % 8 || pre_sl % 8 || pre_sh % 8 || (S > 0 && (suf_sl % 8 || suf_sh % 8)))
+  if (q_sm % 8 || q_sh % 8 || (P > 0 && (pre_sl % 8 || pre_sh % 8 || pre_vt_sd % 8 || pre_vt_sh % 8)) ||
+      (S > 0 && (suf_sl % 8 || suf_sh % 8 || suf_vt_sd % 8 || suf_vt_sh % 8)))
     return fail(TK_EINVAL, "attn: strides must be multiples of 8 elements");
-  if (!aligned16(q) || !aligned16(k_pre) || !aligned16(v_pre) || !aligned16(k_suf) || !aligned16(v_suf))
-    return fail(TK_EINVAL, "attn: q/k/v must be 16-byte aligned");
-  if (out_sm < H * D) return fail(TK_EINVAL, "attn: out_sm=%d < H*D", out_sm);
+  if (!aligned16(q) || !aligned16(k_pre) || !aligned16(vt_pre) || !aligned16(k_pre_lo) || !aligned16(vt_pre_lo) ||
+      !aligned16(k_suf) || !aligned16(vt_suf))
+    return fail(TK_EINVAL, "attn: q/k/v^T must be 16-byte aligned");
+  if ((P > 0 && pre_vt_sd < ((P + 31) / 32) * 32) || (S > 0 && suf_vt_sd < ((S + 31) / 32) * 32))
+    return fail(TK_EINVAL, "attn: a V^T row must hold the segment length rounded up to 32 keys (zero padded)");
+  if (out_sm < H * D || out_sm % 4 || !aligned8(out)) return fail(TK_EINVAL, "attn: out_sm=%d must be >= H*D, a multiple of 4, out 8-byte aligned", out_sm);
 
   AttnArgs a;
   a.q = (const u16*)q;
   a.q_sm = q_sm;
   a.q_sh = q_sh;
-  a.k_pre = k_pre;
-  a.v_pre = v_pre;
+  a.k_pre = (const u16*)k_pre;
+  a.k_pre_lo = (const u16*)k_pre_lo;
+  a.vt_pre = (const u16*)vt_pre;
+  a.vt_pre_lo = (const u16*)vt_pre_lo;
   a.pre_sl = pre_sl;
   a.pre_sh = pre_sh;
+  a.pre_vt_sd = pre_vt_sd;
+  a.pre_vt_sh = pre_vt_sh;
   a.k_suf = (const u16*)k_suf;
-  a.v_suf = (const u16*)v_suf;
+  a.vt_suf = (const u16*)vt_suf;
   a.suf_sl = suf_sl;
   a.suf_sh = suf_sh;
+  a.suf_vt_sd = suf_vt_sd;
+  a.suf_vt_sh = suf_vt_sh;
   a.pad = (const uint8_t*)pad;
   a.out = (u16*)out;
   a.out_sm = out_sm;
@@ -338,11 +388,11 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
   a.logits_bf16 = logits_bf16;
   a.scale = 1.0f / sqrtf((float)D);
 
-  const int ntiles = (P + S + 31) / 32;
+  const int ntiles = (P + 31) / 32 + (S + 31) / 32;
   const int mtiles = (M + 31) / 32;
-  // one 32-key tile per wave and round: split the keys over blocks once a block would need
-  // more than two rounds
-  int splits = (ntiles + 7) / 8;
+  // one 32-key tile per wave: split the keys over blocks of four waves (at most 8 splits, beyond
+  // that a wave loops over several tiles)
+  int splits = (ntiles + 3) / 4;
   if (splits < 1) splits = 1;
   if (splits > 8) splits = 8;
   a.kv_splits = splits;
@@ -356,8 +406,8 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
     a.partial = (float*)((char*)ws + kPartialOff);
     a.counters = (int*)ws;
   }
-  if (tk_launch_attn(a, D, kv_dtype == TK_F32, (hipStream_t)stream))
-    return fail(TK_ELAUNCH, "attn: launch failed (%s)", hipGetErrorString(hipGetLastError()));
+  int rc = tk_launch_attn(a, D, (hipStream_t)stream);
+  if (rc) return fail(TK_ELAUNCH, "attn: launch failed (%s)", hipGetErrorString(hipGetLastError()));
   return TK_OK;
 }
 

@@ -36,17 +36,25 @@ struct GemmArgs {
   int rope_positions;  // rows of the tables (positions are clamped into them)
   int rope_cols;
   int rope_half;
+  // rotary epilogue only: columns >= vt_col0 are also written transposed, vt[(n - vt_col0) * vt_ld + m]
+  unsigned short* vt;
+  int vt_col0;
+  int vt_ld;
 };
 
 struct AttnArgs {
   const unsigned short* q;
   int q_sm, q_sh;
-  const void* k_pre;
-  const void* v_pre;
-  int pre_sl, pre_sh;
+  // prefix: K [P, G, D] (element strides pre_sl, pre_sh) and V^T [G, D, >= roundup(P, 32)]
+  // (element strides pre_vt_sh, pre_vt_sd); the *_lo planes are nullptr unless K/V were fp32
+  const unsigned short* k_pre;
+  const unsigned short* k_pre_lo;
+  const unsigned short* vt_pre;
+  const unsigned short* vt_pre_lo;
+  int pre_sl, pre_sh, pre_vt_sd, pre_vt_sh;
   const unsigned short* k_suf;
-  const unsigned short* v_suf;
-  int suf_sl, suf_sh;
+  const unsigned short* vt_suf;
+  int suf_sl, suf_sh, suf_vt_sd, suf_vt_sh;
   const uint8_t* pad;
   unsigned short* out;
   int out_sm;
@@ -58,9 +66,23 @@ struct AttnArgs {
   float scale;
 };
 
+struct KvPrepArgs {
+  const void* k;  // [L, G, D] with element strides (sl, sh); fp32 when f32, else bf16 (k unused)
+  const void* v;
+  int f32;
+  int sl, sh;
+  int L, G, D;
+  unsigned short* k_hi;  // [L, G, D] contiguous (fp32 sources only)
+  unsigned short* k_lo;
+  unsigned short* vt_hi;  // [G, D, ld]
+  unsigned short* vt_lo;  // fp32 sources only
+  int ld;
+};
+
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st);
 int tk_launch_pack(const void* w0, const void* w1, void* out, int N, int K, int interleave, hipStream_t st);
 int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st);
 int tk_launch_fill_zero(int* p, int n, hipStream_t st);
 int tk_launch_decode_fp8(float* out, hipStream_t st);
-int tk_launch_attn(AttnArgs a, int D, int kv_f32, hipStream_t st);
+int tk_launch_attn(AttnArgs a, int D, hipStream_t st);
+int tk_launch_kv_prepare(KvPrepArgs p, hipStream_t st);

@@ -259,6 +259,8 @@ def bf16w_linear(
     rope: RopeTables | None = None,
     rope_pos: torch.Tensor | None = None,
     rope_cols: int = 0,
+    vt_out: torch.Tensor | None = None,
+    vt_col0: int = 0,
     resid: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
     split_k: int = 0,
@@ -266,7 +268,8 @@ def bf16w_linear(
 ) -> torch.Tensor:
     """``x [M, K] @ W^T`` with bf16 weights; optional RMSNorm prologue (``x`` bf16 or fp32), and
     either a rotary epilogue (``rope`` tables, int32 ``rope_pos [M]``, columns ``< rope_cols``
-    rotated) or a residual epilogue."""
+    rotated; with ``vt_out [N - vt_col0, >= M]`` the columns from ``vt_col0`` on are also written
+    transposed) or a residual epilogue."""
     lib = native.lib()
     if not x.is_cuda or x.dim() != 2 or x.shape[1] != w.k or x.stride(1) != 1:
         raise ValueError(f"activations must be CUDA [M, {w.k}] with unit inner stride")
@@ -295,11 +298,16 @@ def bf16w_linear(
         positions, half = rope.positions, rope.half
     elif w.rope_half:
         raise ValueError("a weight packed in rotary pair order needs the rotary epilogue")
+    vt_p, vt_ld = None, 0
+    if vt_out is not None:
+        if vt_out.dtype != torch.bfloat16 or vt_out.dim() != 2 or vt_out.stride(1) != 1 or vt_out.shape[0] != w.n - vt_col0:
+            raise ValueError("vt_out must be bf16 [N - vt_col0, >= M] with unit inner stride")
+        vt_p, vt_ld = vt_out.data_ptr(), vt_out.stride(0)
     ws = ws or default_workspace(x.device)
     rc = lib.tk_bf16w_linear(
         x.data_ptr(), x.stride(0), xdt, w.data.data_ptr(), _norm_ptr(norm_w, w.k), float(eps), pos_p, cos_p, sin_p,
-        positions, rope_cols, half, out.data_ptr(), out.stride(0), rp, ldr, rdt, m, w.n, w.k, split_k, ws.ptr, ws.nbytes,
-        _stream(),
+        positions, rope_cols, half, vt_p, vt_col0, vt_ld, out.data_ptr(), out.stride(0), rp, ldr, rdt, m, w.n, w.k,
+        split_k, ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip
     native.check(rc, "tk_bf16w_linear")
     return out
@@ -315,12 +323,62 @@ def _same_layout(k: torch.Tensor, v: torch.Tensor) -> bool:
     return k.shape == v.shape and k.stride(2) == 1 and v.stride(2) == 1 and _eff_strides(k) == _eff_strides(v)
 
 
+@dataclass
+class PrefixKV:
+    """One layer's prefix K/V in the attention kernel's layout (see :func:`prepare_prefix_kv`)."""
+
+    k: torch.Tensor  # bf16 [P, G, D] (any row / head strides, d contiguous)
+    vt: torch.Tensor  # bf16 [G, D, P rounded up to 32], zero padded
+    k_lo: torch.Tensor | None = None  # low planes when the source was fp32
+    vt_lo: torch.Tensor | None = None
+
+    @property
+    def length(self) -> int:
+        return self.k.shape[0]
+
+
+@dataclass
+class SuffixKV:
+    """The action tokens' own K ``[S, G, D]`` and V^T ``[G, D, >= S rounded up to 32]`` (zero padded)."""
+
+    k: torch.Tensor
+    vt: torch.Tensor
+
+
+def _pad32(n: int) -> int:
+    return (n + 31) // 32 * 32
+
+
+def prepare_prefix_kv(k: torch.Tensor, v: torch.Tensor) -> PrefixKV:
+    """``k, v [P, G, D]`` (bf16 or fp32 views sharing strides) -> :class:`PrefixKV`, one launch.
+
+    bf16: ``k`` is used in place, ``v`` is transposed.  fp32: both are split into bf16 hi + lo planes.
+    """
+    lib = native.lib()
+    if k.dtype != v.dtype or k.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("prefix K/V must both be bf16 or both fp32")
+    if not _same_layout(k, v):
+        raise ValueError("prefix K and V must share strides and have a contiguous head dim")
+    p, g, d = k.shape
+    sl, sh = _eff_strides(k)
+    bf = dict(dtype=torch.bfloat16, device=k.device)
+    vt = torch.empty(g, d, _pad32(p), **bf)
+    if k.dtype == torch.float32:
+        k_hi, k_lo, vt_lo = torch.empty(p, g, d, **bf), torch.empty(p, g, d, **bf), torch.empty_like(vt)
+        rc = lib.tk_attn_prepare_kv(k.data_ptr(), v.data_ptr(), _F32, sl, sh, p, g, d, k_hi.data_ptr(), k_lo.data_ptr(),
+                                    vt.data_ptr(), vt_lo.data_ptr(), vt.shape[2], _stream())  # fmt: skip
+        native.check(rc, "tk_attn_prepare_kv")
+        return PrefixKV(k_hi, vt, k_lo, vt_lo)
+    rc = lib.tk_attn_prepare_kv(None, v.data_ptr(), _BF16, sl, sh, p, g, d, None, None, vt.data_ptr(), None, vt.shape[2],
+                                _stream())  # fmt: skip
+    native.check(rc, "tk_attn_prepare_kv")
+    return PrefixKV(k, vt)
+
+
 def expert_attn(
     q: torch.Tensor,
-    k_pre: torch.Tensor,
-    v_pre: torch.Tensor,
-    k_suf: torch.Tensor | None,
-    v_suf: torch.Tensor | None,
+    prefix: PrefixKV | None,
+    suffix: SuffixKV | None,
     prefix_pad: torch.Tensor | None,
     mask_mode: int,
     *,
@@ -328,42 +386,81 @@ def expert_attn(
     out: torch.Tensor | None = None,
     ws: Workspace | None = None,
 ) -> torch.Tensor:
-    """Attention of ``q [M, H, D]`` over ``[k_pre; k_suf]`` (``[P|S, G, D]`` views, any strides with
-    a contiguous head dim).  ``prefix_pad``: uint8/bool ``[P]`` or None.  Returns bf16 ``[M, H*D]``."""
+    """Attention of ``q [M, H, D]`` over ``[prefix; suffix]`` keys.  ``prefix_pad``: uint8/bool
+    ``[P]`` or None.  Returns bf16 ``[M, H*D]``."""
     lib = native.lib()
     if q.dtype != torch.bfloat16 or q.dim() != 3 or q.stride(2) != 1:
         raise TypeError("q must be bf16 [M, H, D] with a contiguous head dim")
     m, h, d = q.shape
-    p, g = k_pre.shape[0], k_pre.shape[1]
-    if k_pre.dtype != v_pre.dtype or k_pre.dtype not in (torch.bfloat16, torch.float32):
-        raise TypeError("prefix K/V must both be bf16 or both fp32")
-    if not _same_layout(k_pre, v_pre):
-        raise ValueError("prefix K and V must share strides and have a contiguous head dim")
+    bf = torch.bfloat16
+
+    def _vt_ok(vt: torch.Tensor, g: int, length: int) -> bool:
+        return vt.dtype == bf and vt.dim() == 3 and vt.shape[:2] == (g, d) and vt.stride(2) == 1 and vt.shape[2] >= _pad32(length)
+
+    p = g = 0
+    kp = kpl = vp = vpl = None
+    pre_sl = pre_sh = pre_sd = pre_vsh = 0
+    if prefix is not None:
+        p, g = prefix.k.shape[0], prefix.k.shape[1]
+        if prefix.k.dtype != bf or prefix.k.shape[2] != d or prefix.k.stride(2) != 1 or not _vt_ok(prefix.vt, g, p):
+            raise ValueError("prefix must hold bf16 K [P, G, D] and V^T [G, D, >= P rounded up to 32]")
+        pre_sl, pre_sh = _eff_strides(prefix.k)
+        pre_vsh, pre_sd = prefix.vt.stride(0) if g > 1 else 0, prefix.vt.stride(1)
+        kp, vp = prefix.k.data_ptr(), prefix.vt.data_ptr()
+        if prefix.k_lo is not None:
+            if prefix.vt_lo is None or prefix.k_lo.stride() != prefix.k.stride() or prefix.vt_lo.stride() != prefix.vt.stride():
+                raise ValueError("low planes must mirror the high planes' layout")
+            kpl, vpl = prefix.k_lo.data_ptr(), prefix.vt_lo.data_ptr()
     s = 0
-    suf_sl = suf_sh = 0
-    if k_suf is not None:
-        assert v_suf is not None
-        if k_suf.dtype != torch.bfloat16 or v_suf.dtype != torch.bfloat16:
-            raise TypeError("suffix K/V must be bf16")
-        if not _same_layout(k_suf, v_suf):
-            raise ValueError("suffix K and V must share strides and have a contiguous head dim")
-        s = k_suf.shape[0]
-        suf_sl, suf_sh = _eff_strides(k_suf)
+    ks = vs = None
+    suf_sl = suf_sh = suf_sd = suf_vsh = 0
+    if suffix is not None:
+        s, gs = suffix.k.shape[0], suffix.k.shape[1]
+        if prefix is not None and gs != g:
+            raise ValueError("prefix and suffix must have the same number of kv heads")
+        g = gs
+        if suffix.k.dtype != bf or suffix.k.shape[2] != d or suffix.k.stride(2) != 1 or not _vt_ok(suffix.vt, g, s):
+            raise ValueError("suffix must hold bf16 K [S, G, D] and V^T [G, D, >= S rounded up to 32]")
+        suf_sl, suf_sh = _eff_strides(suffix.k)
+        suf_vsh, suf_sd = suffix.vt.stride(0) if g > 1 else 0, suffix.vt.stride(1)
+        ks, vs = suffix.k.data_ptr(), suffix.vt.data_ptr()
     pad = None
     if prefix_pad is not None:
         pad = prefix_pad.view(torch.uint8) if prefix_pad.dtype == torch.bool else prefix_pad
         if pad.dtype != torch.uint8 or pad.numel() != p or not pad.is_contiguous():
             raise ValueError("prefix_pad must be a contiguous uint8/bool [P]")
     if out is None:
-        out = torch.empty(m, h * d, dtype=torch.bfloat16, device=q.device)
+        out = torch.empty(m, h * d, dtype=bf, device=q.device)
     ws = ws or default_workspace(q.device)
     rc = lib.tk_expert_attn(
-        q.data_ptr(), q.stride(0), q.stride(1), k_pre.data_ptr(), v_pre.data_ptr(), *_eff_strides(k_pre),
-        _F32 if k_pre.dtype == torch.float32 else _BF16, _ptr(k_suf), _ptr(v_suf), suf_sl, suf_sh, _ptr(pad),
-        out.data_ptr(), out.stride(0), m, p, s, h, g, d, mask_mode, int(logits_bf16), ws.ptr, ws.nbytes, _stream(),
+        q.data_ptr(), q.stride(0), q.stride(1), kp, kpl, pre_sl, pre_sh, vp, vpl, pre_sd, pre_vsh, ks, suf_sl, suf_sh,
+        vs, suf_sd, suf_vsh, _ptr(pad), out.data_ptr(), out.stride(0), m, p, s, h, max(g, 1), d, mask_mode,
+        int(logits_bf16), ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip
     native.check(rc, "tk_expert_attn")
     return out
+
+
+def expert_attn_plain(
+    q: torch.Tensor,
+    k_pre: torch.Tensor | None,
+    v_pre: torch.Tensor | None,
+    k_suf: torch.Tensor | None,
+    v_suf: torch.Tensor | None,
+    prefix_pad: torch.Tensor | None,
+    mask_mode: int,
+    **kw,
+) -> torch.Tensor:
+    """:func:`expert_attn` on plain ``[L, G, D]`` K/V tensors: lays the prefix out with
+    :func:`prepare_prefix_kv` and transposes the suffix values with torch, then calls the kernel."""
+    prefix = prepare_prefix_kv(k_pre, v_pre) if k_pre is not None and k_pre.shape[0] > 0 else None
+    suffix = None
+    if k_suf is not None and k_suf.shape[0] > 0:
+        s, g, d = k_suf.shape
+        vt = torch.zeros(g, d, _pad32(s), dtype=torch.bfloat16, device=k_suf.device)
+        vt[:, :, :s] = v_suf.permute(1, 2, 0)
+        suffix = SuffixKV(k_suf, vt)
+    return expert_attn(q, prefix, suffix, prefix_pad, mask_mode, **kw)
 
 
 def decode_fp8_table(device: torch.device | str = "cuda") -> torch.Tensor:

@@ -93,6 +93,7 @@ class PI05Model:
         self.vlm_mlp = [GatedMLP(state_dict, f"{VLM}layers.{i}.mlp.", self.device, self.fp8_llm_mlp, act="gelu_tanh") for i in range(self.depth)]
         self.exp_mlp = [GatedMLP(state_dict, f"{EXP}layers.{i}.mlp.", self.device, self.fp8_expert_mlp, act="gelu_tanh") for i in range(self.ed["depth"])]
         self.ws = tk.default_workspace(self.device) if self.use_hip else None
+        self.vt_suf = None  # zero-padded V^T of the action tokens, allocated on first use
 
         inv = 1.0 / (10000.0 ** (torch.arange(0, self.head_dim, 2, dtype=torch.int64).float() / self.head_dim))
         inv = inv.to(BF16).float()  # the reference's inverse frequencies go through a bf16 buffer
@@ -193,10 +194,20 @@ class PI05Model:
         return kv
 
     # ------------------------------------------------------------------ denoising
-    def denoise_step(self, prefix_pad, kv, x_t, step: int) -> torch.Tensor:
+    def attention_caches(self, kv) -> list:
+        """Per-layer prefix K/V in the attention kernel's layout (V transposed), once per request."""
+        return [tk.prepare_prefix_kv(k[0].transpose(0, 1), v[0].transpose(0, 1)) for k, v in kv]
+
+    def denoise_step(self, prefix_pad, kv, x_t, step: int, caches: list | None = None) -> torch.Tensor:
         """Velocity fp32 ``[1, chunk, max_action_dim]`` at denoising step ``step`` (flow_matching.py:505-556)."""
         hidden = self.lin("action_in_proj", x_t).to(BF16)
         b, s = hidden.shape[0], hidden.shape[1]
+        if self.fused_expert:
+            if caches is None:
+                caches = self.attention_caches(kv)
+            if self.vt_suf is None or self.vt_suf.shape[2] < (s + 31) // 32 * 32:
+                g = kv[0][0].shape[1]
+                self.vt_suf = torch.zeros(g, self.head_dim, (s + 31) // 32 * 32, dtype=BF16, device=self.device)
         p_len = prefix_pad.shape[1]
         pos = prefix_pad.sum(dim=-1)[:, None] + torch.arange(s, device=self.device)[None, :]
         cos, sin = self.rope_tables(pos, hidden.dtype)
@@ -210,10 +221,10 @@ class PI05Model:
             h, gate = gemma_norm(hidden, modulation=mod_in)
             q, k, v = self._attn_proj(lp + "self_attn.", h, cos, sin)
             if self.fused_expert:
-                pk, pv = kv[i]
+                self.vt_suf[:, :, :s].copy_(v[0].transpose(1, 2))
                 att = tk.expert_attn(
-                    q[0].transpose(0, 1), pk[0].transpose(0, 1), pv[0].transpose(0, 1), k[0].transpose(0, 1), v[0].transpose(0, 1),
-                    prefix_pad[0], tk.MASK_BIDIR, logits_bf16=True, ws=self.ws,
+                    q[0].transpose(0, 1), caches[i], tk.SuffixKV(k[0].transpose(0, 1), self.vt_suf), prefix_pad[0],
+                    tk.MASK_BIDIR, logits_bf16=True, ws=self.ws,
                 )[None]  # fmt: skip
             else:
                 att = attention_core(q, torch.cat([kv[i][0], k], dim=2), torch.cat([kv[i][1], v], dim=2), add, scaling)
@@ -237,6 +248,7 @@ class PI05Model:
             trace.update(prefix_embs=embs, pad_masks=pads, kv=kv)
         dt = -1.0 / self.num_steps
         x_t = noise
+        caches = self.attention_caches(kv) if self.fused_expert else None
         for step in range(self.num_steps):
-            x_t = x_t + dt * self.denoise_step(pads, kv, x_t, step)
+            x_t = x_t + dt * self.denoise_step(pads, kv, x_t, step, caches)
         return x_t

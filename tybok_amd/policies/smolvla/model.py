@@ -124,6 +124,9 @@ class SmolVLAModel:
         self.ws = tk.default_workspace(self.device) if self.use_hip else None
         if self.fused_expert:
             self._pack_expert_projections()
+            # V^T of the action tokens [G, D, chunk rounded up to 32]; the projection kernel writes
+            # columns < chunk, the zero padding beyond is never touched
+            self.vt_suf = torch.zeros(self.kv_heads, self.head_dim, (cfg.chunk_size + 31) // 32 * 32, dtype=BF16, device=self.device)
 
         # constants (built once: nothing below copies from the host at inference time)
         d_half = self.head_dim // 2
@@ -284,7 +287,19 @@ class SmolVLAModel:
         pos0 = pos - pos.min(dim=1, keepdim=True).values
         return pos, pos0
 
-    def _denoise_step_fused(self, prefix_pad, keys, values, ekv, hidden, pos32, pos0_32):
+    def attention_caches(self, keys, values, ekv) -> list:
+        """Per-layer prefix K/V in the attention kernel's layout, once per request: V transposed
+        (self layers, bf16 cache) or K and V^T split into bf16 hi + lo planes (cross layers, fp32)."""
+        caches = []
+        for i in range(self.num_layers):
+            if self.cfg.is_cross_layer(i):
+                ek, ev = ekv[i]
+                caches.append(tk.prepare_prefix_kv(ek[0], ev[0]))
+            else:
+                caches.append(tk.prepare_prefix_kv(keys[i, 0], values[i, 0]))
+        return caches
+
+    def _denoise_step_fused(self, prefix_pad, caches, hidden, pos32, pos0_32):
         """Expert stack on the fused launches; ``hidden [S, E]`` fp32 in, bf16 out."""
         h_q, h_kv, d = self.heads, self.kv_heads, self.head_dim
         nq, nkv = h_q * d, h_kv * d
@@ -295,16 +310,15 @@ class SmolVLAModel:
             cross = self.cfg.is_cross_layer(i)
             qkv = tk.bf16w_linear(
                 hidden, self.exp_qkv[i], norm_w=self.p[lp + "input_layernorm.weight"], eps=self.eps, rope=self.rope_tables,
-                rope_pos=pos0_32 if cross else pos32, rope_cols=nq if cross else nq + nkv, ws=self.ws,
+                rope_pos=pos0_32 if cross else pos32, rope_cols=nq if cross else nq + nkv,
+                vt_out=None if cross else self.vt_suf.view(nkv, -1), vt_col0=nq + nkv, ws=self.ws,
             )  # fmt: skip
             q = qkv[:, :nq].view(s, h_q, d)
             if cross:
-                ek, ev = ekv[i]
-                att = tk.expert_attn(q, ek[0], ev[0], None, None, pad, tk.MASK_NONE, ws=self.ws)
+                att = tk.expert_attn(q, caches[i], None, pad, tk.MASK_NONE, ws=self.ws)
             else:
-                k = qkv[:, nq : nq + nkv].view(s, h_kv, d)
-                v = qkv[:, nq + nkv :].view(s, h_kv, d)
-                att = tk.expert_attn(q, keys[i, 0], values[i, 0], k, v, pad, tk.MASK_CAUSAL, ws=self.ws)
+                suffix = tk.SuffixKV(qkv[:, nq : nq + nkv].view(s, h_kv, d), self.vt_suf)
+                att = tk.expert_attn(q, caches[i], suffix, pad, tk.MASK_CAUSAL, ws=self.ws)
             out = tk.bf16w_linear(att, self.exp_o[i], resid=hidden, ws=self.ws)
             mlp = self.exp_mlp[i]
             post_w = self.p[lp + "post_attention_layernorm.weight"]
@@ -314,7 +328,7 @@ class SmolVLAModel:
                 hidden = mlp(rms_norm(out, post_w, self.eps)[None], out[None])[0]
         return hidden
 
-    def denoise_step(self, prefix_pad, keys, values, ekv, x_t, time_emb, positions=None):
+    def denoise_step(self, prefix_pad, keys, values, ekv, x_t, time_emb, positions=None, caches=None):
         """Velocity ``v_t`` fp32 ``[1, chunk, max_action_dim]`` (flow_matching.py:316-350)."""
         hidden = self.embed_suffix(x_t, time_emb)
         b, s = hidden.shape[0], hidden.shape[1]
@@ -323,12 +337,13 @@ class SmolVLAModel:
         if self.fused_expert and b == 1:
             clamp = lambda t: t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)  # noqa: E731
             pos32, pos0_32 = (pos, pos0) if pos.dtype == torch.int32 else (clamp(pos), clamp(pos0))
-            hidden = self._denoise_step_fused(prefix_pad, keys, values, ekv, hidden[0], pos32, pos0_32)[None]
+            if caches is None:
+                caches = self.attention_caches(keys, values, ekv)
+            hidden = self._denoise_step_fused(prefix_pad, caches, hidden[0], pos32, pos0_32)[None]
             out = rms_norm(hidden, self.p[EXP + "norm.weight"], self.eps)
             return self.lin("action_out_proj", out.to(torch.float32))
-        if not self.fused_expert:
-            causal = torch.ones(s, s, dtype=torch.bool, device=self.device).tril()[None]
-            full_mask = torch.cat([prefix_pad[:, None, :].expand(b, s, p_len), causal], dim=2)
+        causal = torch.ones(s, s, dtype=torch.bool, device=self.device).tril()[None]
+        full_mask = torch.cat([prefix_pad[:, None, :].expand(b, s, p_len), causal], dim=2)
         for i in range(self.num_layers):
             lp = f"{EXP}layers.{i}."
             h = rms_norm(hidden, self.p[lp + "input_layernorm.weight"], self.eps).to(BF16)
@@ -337,17 +352,11 @@ class SmolVLAModel:
                 k = self.rope(self.lin(lp + "self_attn.k_proj", h).view(b, s, -1, self.head_dim), pos)
                 v = self.lin(lp + "self_attn.v_proj", h).view(b, s, -1, self.head_dim)
                 q = self.rope(q, pos)
-                if self.fused_expert:
-                    att = tk.expert_attn(q[0], keys[i, 0], values[i, 0], k[0], v[0], prefix_pad[0], tk.MASK_CAUSAL, ws=self.ws)[None]
-                else:
-                    att = eager_attention(full_mask, q, torch.cat([keys[i], k], dim=1), torch.cat([values[i], v], dim=1))
+                att = eager_attention(full_mask, q, torch.cat([keys[i], k], dim=1), torch.cat([values[i], v], dim=1))
             else:
                 q = self.rope(q, pos0)
                 ek, ev = ekv[i]
-                if self.fused_expert:
-                    att = tk.expert_attn(q[0], ek[0], ev[0], None, None, prefix_pad[0], tk.MASK_NONE, ws=self.ws)[None]
-                else:
-                    att = eager_attention(prefix_pad[:, None, :].expand(b, s, p_len), q, ek, ev)
+                att = eager_attention(prefix_pad[:, None, :].expand(b, s, p_len), q, ek, ev)
             hidden = self._layer_tail(lp, self.exp_mlp[i], att, hidden)
         out = rms_norm(hidden, self.p[EXP + "norm.weight"], self.eps)
         return self.lin("action_out_proj", out.to(torch.float32))
@@ -362,8 +371,9 @@ class SmolVLAModel:
         positions = self.suffix_positions(pads, noise.shape[1])
         if self.fused_expert and noise.shape[0] == 1:
             positions = tuple(t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32) for t in positions)
+        caches = self.attention_caches(keys, values, ekv) if self.fused_expert and noise.shape[0] == 1 else None
         for step in range(self.num_steps):
-            v_t = self.denoise_step(pads, keys, values, ekv, x_t, self.time_embs[step], positions)
+            v_t = self.denoise_step(pads, keys, values, ekv, x_t, self.time_embs[step], positions, caches)
             x_t = x_t + dt * v_t
         return x_t
 
