@@ -178,7 +178,7 @@ def main() -> None:
         us = gemm_launch_us(50, 2048, 16384, launches=20, reps=args.steps)
         print(json.dumps({"gemm_only": {"M": 50, "K": 2048, "N": 16384, "us": round(us, 2), "GBps": round(bytes_gemm(50, 2048, 16384) / us / 1e3, 1)}}), flush=True)
         return
-    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True)
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_fused_attn=True)
     tmp = tempfile.mkdtemp(prefix="tybok_bench_")
 
     # ---- SmolVLA-shaped chunk (headline) ----

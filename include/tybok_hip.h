@@ -191,6 +191,10 @@ int tk_attn_prepare_kv(const void* k, const void* v, int kv_dtype, int sl, int s
  *           32] (zero padded), strides (suf_vt_sh, suf_vt_sd) -- tk_bf16w_linear's `vt` output.
  *           Both NULL when S == 0.
  *   pad:    uint8 [P], 1 = prefix token visible (NULL = all visible).
+ *   mask2d: optional uint8 [M, mask_ld] (mask_ld >= P rounded up to 32, a multiple of 8): byte
+ *           (m, p) != 0 = prefix key p visible to query m; replaces `pad`.  This is the 2-D mask of
+ *           the VLM prefill (`make_att_2d_masks`, tybok/policies/smolvla/models/flow_matching.py:44-83,
+ *           `triton_prefill_layer`'s mask2d, tybok/policies/smolvla/models/triton_attn.py:465-583).
  *   mask_mode: TK_MASK_*; q head h reads kv head h / (H / G).
  *   logits_bf16: 0 = fp32 logits (SmolVLA); 1 = logits rounded to bf16 before the softmax and
  *           masked with the additive -2.3819763e38 (pi0.5).
@@ -199,9 +203,9 @@ int tk_attn_prepare_kv(const void* k, const void* v, int kv_dtype, int sl, int s
  */
 int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* k_pre_lo, int pre_sl, int pre_sh,
                    const void* vt_pre, const void* vt_pre_lo, int pre_vt_sd, int pre_vt_sh, const void* k_suf,
-                   int suf_sl, int suf_sh, const void* vt_suf, int suf_vt_sd, int suf_vt_sh, const void* pad, void* out,
-                   int out_sm, int M, int P, int S, int H, int G, int D, int mask_mode, int logits_bf16, void* ws,
-                   size_t ws_bytes, void* stream);
+                   int suf_sl, int suf_sh, const void* vt_suf, int suf_vt_sd, int suf_vt_sh, const void* pad,
+                   const void* mask2d, int mask_ld, void* out, int out_sm, int M, int P, int S, int H, int G, int D,
+                   int mask_mode, int logits_bf16, void* ws, size_t ws_bytes, void* stream);
 
 /* ---- diagnostics ------------------------------------------------------------------------------- */
 /* out_f32[256] = value of every e4m3fn code as decoded by the device's conversion instruction

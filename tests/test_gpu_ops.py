@@ -205,6 +205,27 @@ def test_attention_fully_masked_prefix_is_uniform(tk):
     _close(got, want, "attn fully masked")
 
 
+@pytest.mark.parametrize("p,h,g,d", [(241, 15, 5, 64), (177, 15, 5, 64), (40, 4, 2, 128), (1024, 12, 12, 64)])
+def test_prefill_attention_with_2d_mask(tk, p, h, g, d):
+    # the VLM prefill: every token is a query, keys are the same tokens, visibility from the
+    # block-causal 2-D mask (image/language tokens see each other, the state token sees all) & padding
+    q, k, v, _, _ = attn_case(p, p, h, g, d, seed=4)
+    gen = torch.Generator().manual_seed(5)
+    pad = torch.rand(p, generator=gen) > 0.1
+    att = torch.zeros(p, dtype=torch.bool)
+    att[-1] = True
+    mask = oops.make_att_2d_masks(pad[None], att[None])[0]
+    want = oops.eager_attention(mask[None], q[None], k[None], v[None])[0]
+    p_pad = (p + 31) // 32 * 32
+    m2 = torch.zeros(p, p_pad, dtype=torch.uint8)
+    m2[:, :p] = mask
+    pre = tk.prepare_prefix_kv(k.cuda(), v.cuda())
+    got = tk.expert_attn(q.cuda(), pre, None, None, oops.MASK_NONE, mask2d=m2.cuda())
+    again = tk.expert_attn(q.cuda(), pre, None, None, oops.MASK_NONE, mask2d=m2.cuda())
+    assert torch.equal(got, again)
+    _close(got, want, f"prefill attention P={p} H={h} D={d}")
+
+
 def test_gated_residual_epilogue(tk):
     # pi0.5 AdaRMS gated residual: y = resid + bf16(ffn(x) * gate)
     x, wg8, sg, wu8, su, wd8, sd = ffn_case(50, 1024, 4096, seed=3)

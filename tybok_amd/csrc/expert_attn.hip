@@ -69,6 +69,7 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
     i32x4 k[PL][DS];
     i32x4 v[PL][DT][2];
     int pad;
+    unsigned long long m2[2];  // per-query visibility bytes of the tile's keys (mask2d)
   };
   // every load of a key tile, issued back to back (t is wave-uniform)
   auto load = [&](Stage& st, int t) {
@@ -92,7 +93,12 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
         for (int s = 0; s < 2; ++s) st.v[pl][dt][s] = *(const i32x4*)(vb + voff + (size_t)dt * 32 * vsd + 16 * s);
     }
     st.pad = 1;
-    if (pre && a.pad) {
+    if (pre && a.mask2d) {
+      // eight consecutive keys per byte run: registers 8s..8s+7 of this lane
+      const uint8_t* mp = a.mask2d + (size_t)(q_ok ? qi : a.M - 1) * a.mask_ld + tt * 32 + 8 * half;
+      st.m2[0] = *(const unsigned long long*)mp;
+      st.m2[1] = *(const unsigned long long*)(mp + 16);
+    } else if (pre && a.pad) {
       const int key = tt * 32 + l32;
       st.pad = key < a.P ? a.pad[key] : 0;
     }
@@ -141,7 +147,10 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
       float s = sT[i];
       if (a.logits_bf16) s = round_bf16(s);
       s *= a.scale;
-      const bool vis = pre ? ((pmask >> kl) & 1u) != 0 : (a.mask_mode == 1 || key <= qi);
+      bool vis;
+      if (!pre) vis = a.mask_mode == 1 || key <= qi;
+      else if (a.mask2d) vis = ((st.m2[i >> 3] >> (8 * (i & 7))) & 0xffull) != 0;
+      else vis = ((pmask >> kl) & 1u) != 0;
       if (!vis) s = a.logits_bf16 ? (s + kOpenpiMask) : kF32Min;
       if (key >= len) s = -INFINITY;
       p[i] = s;

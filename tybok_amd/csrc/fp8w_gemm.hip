@@ -40,6 +40,9 @@ namespace {
 // LDS-only barrier: waits for this wave's LDS traffic, not for the global prefetch queue
 // (a full __syncthreads() would drain vmcnt and serialise the weight stream every round).
 __device__ __forceinline__ void lds_barrier() {
+#ifdef TK_EXP_NOBARRIER
+  return;
+#endif
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -144,6 +147,9 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     i32x4 nw[PRO ? XPT : 1];  // norm weights of the piece's 8 columns
   };
   auto xload = [&](XFrag& f, int r) {
+#ifdef TK_EXP_NOX
+    if (r > 0) return;
+#endif
     const int k0 = (kt_lo + r * RKT) * 32;
 #pragma unroll
     for (int i = 0; i < XPT; ++i) {
@@ -243,12 +249,14 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   // 2*PF-1 rounds) uses block-uniform conditions and requests nothing that is not consumed.
   WFrag wbuf[PF];
   XFrag xbuf[PF];
+  // (unconditional even when the block has fewer than PF rounds -- the addresses are clamped to
+  // valid tiles: a branch here would make the compiler's wait-count analysis assume, at the head
+  // of the steady-state loop, that the first stage's loads might be the youngest in flight, and
+  // drain the whole queue once per pass)
 #pragma unroll
   for (int p = 0; p < PF; ++p) {
-    if (p < nrounds) {
-      xload(xbuf[p], p);
-      wload(wbuf[p], p);
-    }
+    xload(xbuf[p], p);
+    wload(wbuf[p], p);
   }
   TK_MARK(1);
   if (PRO) {
@@ -566,9 +574,15 @@ __global__ void decode_fp8_kernel(float* out) {
   out[c] = bf16_bits_to_f32((u16)(cv.u & 0xffff));
 }
 
+#ifndef TK_EXP_PF
+#define TK_EXP_PF 4
+#endif
+#ifndef TK_EXP_TPW
+#define TK_EXP_TPW 1
+#endif
 template <int MT, int NT, int EPI, bool W16, int PRO>
 int launch(const GemmArgs& a, dim3 grid, hipStream_t st) {
-  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, 4, 1, W16, PRO>), grid, dim3(256), 0, st, a);
+  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, TK_EXP_PF, TK_EXP_TPW, W16, PRO>), grid, dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -334,9 +334,9 @@ int tk_attn_prepare_kv(const void* k, const void* v, int kv_dtype, int sl, int s
 
 int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* k_pre_lo, int pre_sl, int pre_sh,
                    const void* vt_pre, const void* vt_pre_lo, int pre_vt_sd, int pre_vt_sh, const void* k_suf, int suf_sl,
-                   int suf_sh, const void* vt_suf, int suf_vt_sd, int suf_vt_sh, const void* pad, void* out, int out_sm,
-                   int M, int P, int S, int H, int G, int D, int mask_mode, int logits_bf16, void* ws, size_t ws_bytes,
-                   void* stream) {
+                   int suf_sh, const void* vt_suf, int suf_vt_sd, int suf_vt_sh, const void* pad, const void* mask2d,
+                   int mask_ld, void* out, int out_sm, int M, int P, int S, int H, int G, int D, int mask_mode,
+                   int logits_bf16, void* ws, size_t ws_bytes, void* stream) {
   if (M <= 0 || P < 0 || S < 0 || P + S <= 0 || H <= 0 || G <= 0 || H % G)
     return fail(TK_EINVAL, "attn: bad shape M=%d P=%d S=%d H=%d G=%d", M, P, S, H, G);
   if (D != 64 && D != 128 && D != 256) return fail(TK_EINVAL, "attn: head_dim %d not in {64,128,256}", D);
@@ -356,6 +356,8 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
     return fail(TK_EINVAL, "attn: q/k/v^T must be 16-byte aligned");
   if ((P > 0 && pre_vt_sd < ((P + 31) / 32) * 32) || (S > 0 && suf_vt_sd < ((S + 31) / 32) * 32))
     return fail(TK_EINVAL, "attn: a V^T row must hold the segment length rounded up to 32 keys (zero padded)");
+  if (mask2d && (mask_ld % 8 || mask_ld < ((P + 31) / 32) * 32 || !aligned8(mask2d)))
+    return fail(TK_EINVAL, "attn: mask2d rows must be 8-byte aligned and hold P rounded up to 32 bytes");
   if (out_sm < H * D || out_sm % 4 || !aligned8(out)) return fail(TK_EINVAL, "attn: out_sm=%d must be >= H*D, a multiple of 4, out 8-byte aligned", out_sm);
 
   AttnArgs a;
@@ -377,6 +379,8 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
   a.suf_vt_sd = suf_vt_sd;
   a.suf_vt_sh = suf_vt_sh;
   a.pad = (const uint8_t*)pad;
+  a.mask2d = (const uint8_t*)mask2d;
+  a.mask_ld = mask_ld;
   a.out = (u16*)out;
   a.out_sm = out_sm;
   a.M = M;
@@ -395,6 +399,8 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
   int splits = (ntiles + 3) / 4;
   if (splits < 1) splits = 1;
   if (splits > 8) splits = 8;
+  // many query tiles already fill the device: keep whole key ranges in one block (no partials)
+  while (splits > 1 && H * mtiles * splits > 2 * device_cus()) --splits;
   a.kv_splits = splits;
   a.partial = nullptr;
   a.counters = nullptr;

@@ -56,6 +56,8 @@ struct AttnArgs {
   const unsigned short* vt_suf;
   int suf_sl, suf_sh, suf_vt_sd, suf_vt_sh;
   const uint8_t* pad;
+  const uint8_t* mask2d;  // [M, mask_ld] per-(query, prefix key) visibility; overrides pad when set
+  int mask_ld;
   unsigned short* out;
   int out_sm;
   int M, P, S, H, G;

@@ -58,8 +58,8 @@ SIGNATURES: dict[str, tuple] = {
     "tk_expert_attn": (
         c_int,
         [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int,
-         c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-         c_int, c_void_p, c_size_t, c_void_p],
+         c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+         c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
     "tk_debug_decode_fp8": (c_int, [c_void_p, c_void_p]),
 }

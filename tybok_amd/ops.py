@@ -382,12 +382,14 @@ def expert_attn(
     prefix_pad: torch.Tensor | None,
     mask_mode: int,
     *,
+    mask2d: torch.Tensor | None = None,
     logits_bf16: bool = False,
     out: torch.Tensor | None = None,
     ws: Workspace | None = None,
 ) -> torch.Tensor:
     """Attention of ``q [M, H, D]`` over ``[prefix; suffix]`` keys.  ``prefix_pad``: uint8/bool
-    ``[P]`` or None.  Returns bf16 ``[M, H*D]``."""
+    ``[P]`` or None; ``mask2d``: uint8/bool ``[M, >= P rounded up to 32]`` per-(query, prefix key)
+    visibility, replaces ``prefix_pad``.  Returns bf16 ``[M, H*D]``."""
     lib = native.lib()
     if q.dtype != torch.bfloat16 or q.dim() != 3 or q.stride(2) != 1:
         raise TypeError("q must be bf16 [M, H, D] with a contiguous head dim")
@@ -429,12 +431,18 @@ def expert_attn(
         pad = prefix_pad.view(torch.uint8) if prefix_pad.dtype == torch.bool else prefix_pad
         if pad.dtype != torch.uint8 or pad.numel() != p or not pad.is_contiguous():
             raise ValueError("prefix_pad must be a contiguous uint8/bool [P]")
+    m2_p, m2_ld = None, 0
+    if mask2d is not None:
+        m2 = mask2d.view(torch.uint8) if mask2d.dtype == torch.bool else mask2d
+        if m2.dtype != torch.uint8 or m2.dim() != 2 or m2.shape[0] != m or m2.stride(1) != 1 or m2.shape[1] < _pad32(p):
+            raise ValueError("mask2d must be uint8/bool [M, >= P rounded up to 32] with unit inner stride")
+        m2_p, m2_ld = m2.data_ptr(), m2.stride(0)
     if out is None:
         out = torch.empty(m, h * d, dtype=bf, device=q.device)
     ws = ws or default_workspace(q.device)
     rc = lib.tk_expert_attn(
         q.data_ptr(), q.stride(0), q.stride(1), kp, kpl, pre_sl, pre_sh, vp, vpl, pre_sd, pre_vsh, ks, suf_sl, suf_sh,
-        vs, suf_sd, suf_vsh, _ptr(pad), out.data_ptr(), out.stride(0), m, p, s, h, max(g, 1), d, mask_mode,
+        vs, suf_sd, suf_vsh, _ptr(pad), m2_p, m2_ld, out.data_ptr(), out.stride(0), m, p, s, h, max(g, 1), d, mask_mode,
         int(logits_bf16), ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip
     native.check(rc, "tk_expert_attn")

@@ -51,7 +51,6 @@ log = logging.getLogger("tybok.smolvla")
 class SmolVLAEngine(PolicyEngine):
     # flags owned by other backends or not implemented here: inert default -> accepted, else rejected
     _UNSUPPORTED_FLAGS = {
-        "tl_llm_fused_attn": False,
         "tl_vit_oproj": False,
         "tl_fused_vit": False,
         "tl_llm_flash_attn": False,
@@ -98,8 +97,8 @@ class SmolVLAEngine(PolicyEngine):
             raise ValueError(f"unknown sampler {sampler!r} (this backend implements 'euler')")
         if compile_model:
             raise NotImplementedError("--compile is not supported by this backend (the HIP tiers replace it)")
-        if tl_llm_fused_attn or tl_vit_oproj:
-            raise NotImplementedError("--tl-llm-fused-attn / --tl-vit-oproj are not implemented by this backend")
+        if tl_vit_oproj:
+            raise NotImplementedError("--tl-vit-oproj is not implemented by this backend")
         self.compile_model = False
         self.config = SmolVLAConfig.from_pretrained(checkpoint_dir)
         if self.config.vlm_config is None:
@@ -110,7 +109,14 @@ class SmolVLAEngine(PolicyEngine):
         if num_steps is not None:
             self.config.num_steps = int(num_steps)
         self.config.cache_expert_prefix_kv = bool(cache_expert_prefix_kv)
-        hip_flags = [n for n, on in (("--tl-fused-expert", tl_fused_expert), ("--tl-fp8-llm-mlp", tl_fp8_llm_mlp), ("--tl-fp8-expert-mlp", tl_fp8_expert_mlp)) if on]
+        hip_flags = [
+            n
+            for n, on in (
+                ("--tl-fused-expert", tl_fused_expert), ("--tl-fp8-llm-mlp", tl_fp8_llm_mlp),
+                ("--tl-fp8-expert-mlp", tl_fp8_expert_mlp), ("--tl-llm-fused-attn", tl_llm_fused_attn),
+            )
+            if on
+        ]  # fmt: skip
         if hip_flags and not str(self.device).startswith("cuda"):
             raise RuntimeError(f"{' / '.join(hip_flags)} run gfx950 HIP kernels, but the engine is running on {self.device!r}")
 
@@ -130,9 +136,13 @@ class SmolVLAEngine(PolicyEngine):
         self.tl_fused_expert = bool(tl_fused_expert)
         self.tl_fp8_llm_mlp = bool(tl_fp8_llm_mlp)
         self.tl_fp8_expert_mlp = bool(tl_fp8_expert_mlp)
+        # --tl-llm-fused-attn: the VLM prefill layers on the fused HIP launches (norm + q/k/v + RoPE +
+        # KV write, attention under the 2-D prefix mask, o_proj + residual)
+        self.tl_llm_fused_attn = bool(tl_llm_fused_attn)
         self.model = SmolVLAModel(
             self.config, sd, self.device,
             fused_expert=self.tl_fused_expert, fp8_expert_mlp=self.tl_fp8_expert_mlp, fp8_llm_mlp=self.tl_fp8_llm_mlp,
+            fused_prefill=self.tl_llm_fused_attn,
         )  # fmt: skip
         del sd
 

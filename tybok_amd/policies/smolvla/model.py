@@ -102,6 +102,7 @@ class SmolVLAModel:
         fused_expert: bool = False,
         fp8_expert_mlp: bool = False,
         fp8_llm_mlp: bool = False,
+        fused_prefill: bool = False,
     ):
         assert cfg.vlm_config is not None
         self.cfg = cfg
@@ -109,7 +110,8 @@ class SmolVLAModel:
         self.fused_expert = bool(fused_expert)
         self.fp8_expert_mlp = bool(fp8_expert_mlp)
         self.fp8_llm_mlp = bool(fp8_llm_mlp)
-        self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp
+        self.fused_prefill = bool(fused_prefill)
+        self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp or self.fused_prefill
         if self.use_hip and self.device.type != "cuda":
             raise RuntimeError("the fused / fp8 tiers run HIP kernels and need a GPU device")
         t = cfg.vlm_config.text_config
@@ -122,6 +124,8 @@ class SmolVLAModel:
         self.vlm_mlp = [GatedMLP(state_dict, f"{TXT}layers.{i}.mlp.", self.device, self.fp8_llm_mlp) for i in range(self.num_layers)]
         self.exp_mlp = [GatedMLP(state_dict, f"{EXP}layers.{i}.mlp.", self.device, self.fp8_expert_mlp) for i in range(cfg.n_expert_layers)]
         self.ws = tk.default_workspace(self.device) if self.use_hip else None
+        if self.fused_prefill:
+            self.vlm_qkv, self.vlm_o = self._pack_attention_weights(TXT, lambda i: False)
         if self.fused_expert:
             self._pack_expert_projections()
             # V^T of the action tokens [G, D, chunk rounded up to 32]; the projection kernel writes
@@ -134,7 +138,7 @@ class SmolVLAModel:
         radians = torch.arange(_ROPE_POSITIONS, dtype=torch.float32)[:, None] / (10_000.0**exponents)[None, :]
         self.rope_sin = torch.sin(radians).to(self.device)
         self.rope_cos = torch.cos(radians).to(self.device)
-        self.rope_tables = tk.RopeTables(self.rope_cos, self.rope_sin) if self.fused_expert else None
+        self.rope_tables = tk.RopeTables(self.rope_cos, self.rope_sin) if self.fused_expert or self.fused_prefill else None
         self.set_num_steps(cfg.num_steps)
         v = cfg.vlm_config.vision_config
         side = v.image_size // v.patch_size
@@ -151,16 +155,20 @@ class SmolVLAModel:
             embs.append(sinusoidal_time_embedding(t, self.cfg.expert_hidden_size, self.cfg.min_period, self.cfg.max_period).float())
         self.time_embs = [e.to(self.device) for e in embs]
 
-    def _pack_expert_projections(self) -> None:
-        """bf16 expert attention weights in tile order: q|k|v concatenated (self layers) or q alone
-        (cross layers) in rotary pair order, o_proj in natural order."""
-        self.exp_qkv, self.exp_o = [], []
+    def _pack_attention_weights(self, stack: str, q_only) -> tuple[list, list]:
+        """bf16 attention weights of a decoder stack in tile order: q|k|v concatenated (or q alone
+        where ``q_only(i)``) in rotary pair order, o_proj in natural order."""
+        qkv, o = [], []
         for i in range(self.num_layers):
-            lp = f"{EXP}layers.{i}.self_attn."
-            names = ("q_proj",) if self.cfg.is_cross_layer(i) else ("q_proj", "k_proj", "v_proj")
+            lp = f"{stack}layers.{i}.self_attn."
+            names = ("q_proj",) if q_only(i) else ("q_proj", "k_proj", "v_proj")
             w = torch.cat([self.p[lp + n + ".weight"] for n in names], dim=0).to(BF16)
-            self.exp_qkv.append(tk.pack_bf16_weight(w, rope_half=self.head_dim // 2))
-            self.exp_o.append(tk.pack_bf16_weight(self.p[lp + "o_proj.weight"].to(BF16)))
+            qkv.append(tk.pack_bf16_weight(w, rope_half=self.head_dim // 2))
+            o.append(tk.pack_bf16_weight(self.p[lp + "o_proj.weight"].to(BF16)))
+        return qkv, o
+
+    def _pack_expert_projections(self) -> None:
+        self.exp_qkv, self.exp_o = self._pack_attention_weights(EXP, self.cfg.is_cross_layer)
 
     # ------------------------------------------------------------------ helpers
     def lin(self, name: str, x: torch.Tensor) -> torch.Tensor:
@@ -213,8 +221,13 @@ class SmolVLAModel:
     def embed_prefix(self, images, img_masks, lang_tokens, lang_masks, state):
         """-> ``(embs fp32 [1,P,hidden], pad_masks bool [1,P], att_masks bool [1,P])`` (flow_matching.py:160-257)."""
         embs, pads = [], []
-        for img, m in zip(images, img_masks):
-            e = self.embed_image(img) * self.img_scale
+        if len(images) > 1 and all(img.shape == images[0].shape for img in images):
+            # one pass of the vision tower over all cameras: rows are independent, and the tower's
+            # GEMMs fill the device three times better than one 1024-patch image at a time
+            per_image = (self.embed_image(torch.cat(list(images), dim=0)) * self.img_scale).split(images[0].shape[0], dim=0)
+        else:
+            per_image = [self.embed_image(img) * self.img_scale for img in images]
+        for e, m in zip(per_image, img_masks):
             embs.append(e)
             pads.append(m[:, None].expand(e.shape[0], e.shape[1]))
         lang = F.embedding(lang_tokens, self.p[TXT + "embed_tokens.weight"])
@@ -261,6 +274,40 @@ class SmolVLAModel:
             hidden = self._layer_tail(lp, self.vlm_mlp[i], att, hidden)
         return keys, values
 
+    def prefill_fused(self, embs, pad_masks, att_masks):
+        """VLM prefill on the fused launches (per layer: norm + q|k|v + RoPE, attention under the
+        2-D prefix mask, o_proj + residual, gated FFN) -> ``(K, V, V^T)``: K / V are ``[layers, 1, P,
+        G, D]`` views of the per-layer projection outputs, V^T ``[layers, G, D, P rounded up to 32]``
+        is the attention kernel's value layout (written by the projection epilogue)."""
+        p_len = embs.shape[1]
+        p_pad = (p_len + 31) // 32 * 32
+        h_q, h_kv, d = self.heads, self.kv_heads, self.head_dim
+        nq, nkv = h_q * d, h_kv * d
+        mask2d = torch.zeros(p_len, p_pad, dtype=torch.uint8, device=self.device)
+        mask2d[:, :p_len] = self.make_att_2d_masks(pad_masks, att_masks)[0]
+        pos32 = (torch.cumsum(pad_masks, dim=1) - 1)[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
+        qkv_all = torch.empty(self.num_layers, p_len, nq + 2 * nkv, dtype=BF16, device=self.device)
+        vt_all = torch.zeros(self.num_layers, nkv, p_pad, dtype=BF16, device=self.device)
+        hidden = embs[0]
+        for i in range(self.num_layers):
+            lp = f"{TXT}layers.{i}."
+            qkv = tk.bf16w_linear(
+                hidden, self.vlm_qkv[i], norm_w=self.p[lp + "input_layernorm.weight"], eps=self.eps, rope=self.rope_tables,
+                rope_pos=pos32, rope_cols=nq + nkv, vt_out=vt_all[i], vt_col0=nq + nkv, out=qkv_all[i], ws=self.ws,
+            )  # fmt: skip
+            cache = tk.PrefixKV(qkv[:, nq : nq + nkv].view(p_len, h_kv, d), vt_all[i].view(h_kv, d, p_pad))
+            att = tk.expert_attn(qkv[:, :nq].view(p_len, h_q, d), cache, None, None, tk.MASK_NONE, mask2d=mask2d, ws=self.ws)
+            out = tk.bf16w_linear(att, self.vlm_o[i], resid=hidden, ws=self.ws)
+            mlp = self.vlm_mlp[i]
+            post_w = self.p[lp + "post_attention_layernorm.weight"]
+            if mlp.fp8:
+                hidden = tk.fp8w_gated_ffn(out, mlp.wgu, mlp.wd, mlp.act, resid=out, norm_w=post_w, eps=self.eps, ws=self.ws)
+            else:
+                hidden = mlp(rms_norm(out, post_w, self.eps)[None], out[None])[0]
+        keys = qkv_all[:, None, :, nq : nq + nkv].unflatten(-1, (h_kv, d))
+        values = qkv_all[:, None, :, nq + nkv :].unflatten(-1, (h_kv, d))
+        return keys, values, vt_all.view(self.num_layers, h_kv, d, p_pad)
+
     def expert_prefix_kv(self, keys, values):
         """fp32 expert K/V projections of the prefix for the cross layers (flow_matching.py:553-578)."""
         out = {}
@@ -287,14 +334,17 @@ class SmolVLAModel:
         pos0 = pos - pos.min(dim=1, keepdim=True).values
         return pos, pos0
 
-    def attention_caches(self, keys, values, ekv) -> list:
+    def attention_caches(self, keys, values, ekv, vt=None) -> list:
         """Per-layer prefix K/V in the attention kernel's layout, once per request: V transposed
-        (self layers, bf16 cache) or K and V^T split into bf16 hi + lo planes (cross layers, fp32)."""
+        (self layers, bf16 cache; ``vt`` when the prefill already produced it) or K and V^T split
+        into bf16 hi + lo planes (cross layers, fp32)."""
         caches = []
         for i in range(self.num_layers):
             if self.cfg.is_cross_layer(i):
                 ek, ev = ekv[i]
                 caches.append(tk.prepare_prefix_kv(ek[0], ev[0]))
+            elif vt is not None:
+                caches.append(tk.PrefixKV(keys[i, 0], vt[i]))
             else:
                 caches.append(tk.prepare_prefix_kv(keys[i, 0], values[i, 0]))
         return caches
@@ -362,7 +412,11 @@ class SmolVLAModel:
         return self.lin("action_out_proj", out.to(torch.float32))
 
     def sample_actions_core(self, embs, pads, att, noise, trace: dict | None = None) -> torch.Tensor:
-        keys, values = self.prefill(embs, pads, att)
+        vt = None
+        if self.fused_prefill and embs.shape[0] == 1:
+            keys, values, vt = self.prefill_fused(embs, pads, att)
+        else:
+            keys, values = self.prefill(embs, pads, att)
         ekv = self.expert_prefix_kv(keys, values)
         if trace is not None:
             trace.update(prefix_embs=embs, pad_masks=pads, keys=keys, values=values, ekv=ekv)
@@ -371,7 +425,7 @@ class SmolVLAModel:
         positions = self.suffix_positions(pads, noise.shape[1])
         if self.fused_expert and noise.shape[0] == 1:
             positions = tuple(t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32) for t in positions)
-        caches = self.attention_caches(keys, values, ekv) if self.fused_expert and noise.shape[0] == 1 else None
+        caches = self.attention_caches(keys, values, ekv, vt) if self.fused_expert and noise.shape[0] == 1 else None
         for step in range(self.num_steps):
             v_t = self.denoise_step(pads, keys, values, ekv, x_t, self.time_embs[step], positions, caches)
             x_t = x_t + dt * v_t
