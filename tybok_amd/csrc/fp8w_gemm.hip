@@ -67,7 +67,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   constexpr int XBUF = ROWS * PITCH;          // bytes per staging buffer
   constexpr int PPR = ROWB / 16;              // 8-element pieces per row
   constexpr int XPT = ROWS * PPR / (NW * 64); // pieces per thread and round
-  constexpr int RED_BYTES = 2 * NW * 16 * 64 * 4;
+  constexpr int RED_BYTES = TILES * NW * 16 * 64 * 4;  // every wave's partial tiles at once
   constexpr int LDS_BYTES = 2 * XBUF > RED_BYTES ? 2 * XBUF : RED_BYTES;
   constexpr int WCH = W16 ? 2 : 1;            // 16-byte operand chunks per lane, n tile and k tile
   constexpr int WTILE = W16 ? 2048 : 1024;    // bytes of one packed 32x32 tile
@@ -334,8 +334,50 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   static_assert(NW == 4, "one wave per register group");
   const int ng = wave * 8 + half * 4;  // first of this lane's four columns within an n tile
 
-  // ---- in-block reduction over waves (fixed order w = 0..3), tile by tile, double-buffered ----
-  f32x4 (*red)[NW][4][64] = (f32x4 (*)[NW][4][64])lds;
+  // ---- epilogue operands: requested now, consumed after the reductions ----
+  f32x4 e_sc[NT];     // EPI 0: column scales; EPI 1: e_sc[0] gate scale, e_sc[1] up scale
+  f32x4 e_rv[TILES];  // EPI 0: residual values; EPI 2: [2*mt] cos, [2*mt+1] sin of this lane's row
+  i32x2 e_gate[NT];   // EPI 0: per-column gate (bf16 x4)
+  if (EPI == 0) {
+    if (a.vec) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        int n0 = (strip * NT + nt) * 32 + ng;
+        if (n0 > a.N - 4) n0 = a.N - 4;  // columns past N are never stored
+        if (!W16) e_sc[nt] = *(const f32x4*)(a.s0 + n0);
+        if (a.gate) e_gate[nt] = *(const i32x2*)(a.gate + n0);
+        if (a.resid) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            int m = (mblock * MT + mt) * 32 + l32;
+            if (m > a.M - 1) m = a.M - 1;
+            e_rv[mt * NT + nt] = a.resid_f32 ? *(const f32x4*)((const float*)a.resid + (size_t)m * a.ldr + n0)
+                                             : unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n0));
+          }
+        }
+      }
+    }
+  } else if (EPI == 1) {
+    int col = strip * 32 + ng;
+    if (col > a.N - 4) col = a.N - 4;
+    e_sc[0] = *(const f32x4*)(a.s0 + col);
+    e_sc[NT - 1] = *(const f32x4*)(a.s1 + col);
+  } else {
+    const int po = a.rope_half >> 5;
+    const int fi = (((strip / po) * 2 * po + strip % po) * 32 + ng) % (2 * a.rope_half);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      int m = (mblock * MT + mt) * 32 + l32;
+      if (m > a.M - 1) m = a.M - 1;
+      int pos = a.rope_pos[m];
+      pos = pos < 0 ? 0 : (pos > a.rope_positions - 1 ? a.rope_positions - 1 : pos);
+      e_rv[2 * mt] = *(const f32x4*)(a.rope_cos + (size_t)pos * a.rope_half + fi);
+      e_rv[2 * mt + 1] = *(const f32x4*)(a.rope_sin + (size_t)pos * a.rope_half + fi);
+    }
+  }
+
+  // ---- in-block reduction over waves (fixed order w = 0..3): one exchange for all tiles ----
+  f32x4 (*red)[NW][4][64] = (f32x4 (*)[NW][4][64])lds;  // [tile][wave][group][lane]
   f32x4 own[TILES];
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
@@ -343,12 +385,15 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       f32x4 v = {acc[mt][nt][4 * g], acc[mt][nt][4 * g + 1], acc[mt][nt][4 * g + 2], acc[mt][nt][4 * g + 3]};
-      red[t & 1][wave][g][lane] = v;
+      red[t][wave][g][lane] = v;
     }
-    __syncthreads();
-    f32x4 sum = red[t & 1][0][wave][lane];
+  }
+  __syncthreads();
 #pragma unroll
-    for (int w = 1; w < NW; ++w) sum += red[t & 1][w][wave][lane];
+  for (int t = 0; t < TILES; ++t) {
+    f32x4 sum = red[t][0][wave][lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) sum += red[t][w][wave][lane];
     own[t] = sum;
   }
 
@@ -420,14 +465,10 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       if (m >= a.M || n0 >= a.N) continue;
       if (a.vec) {  // N % 4 == 0 and every row pitch / pointer allows 8-byte accesses
         f32x4 v = own[t];
-        if (!W16) v *= *(const f32x4*)(a.s0 + n0);
+        if (!W16) v *= e_sc[nt];
         i32x2 r = pack_bf16x4(v);
-        if (a.gate) r = pack_bf16x4(unpack_bf16x4(r) * unpack_bf16x4(*(const i32x2*)(a.gate + n0)));
-        if (a.resid) {
-          const f32x4 rv = a.resid_f32 ? *(const f32x4*)((const float*)a.resid + (size_t)m * a.ldr + n0)
-                                       : unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n0));
-          r = pack_bf16x4(unpack_bf16x4(r) + rv);
-        }
+        if (a.gate) r = pack_bf16x4(unpack_bf16x4(r) * unpack_bf16x4(e_gate[nt]));
+        if (a.resid) r = pack_bf16x4(unpack_bf16x4(r) + e_rv[t]);
         *(i32x2*)(a.y + (size_t)m * a.ldy + n0) = r;
       } else {
 #pragma unroll
@@ -449,7 +490,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     // tiles come in (gate, up) pairs over the same logical columns; I % 32 == 0
     const int col = strip * 32 + ng;  // logical column in [0, I)
     if (col < a.N) {
-      const f32x4 scg = *(const f32x4*)(a.s0 + col), scu = *(const f32x4*)(a.s1 + col);
+      const f32x4 scg = e_sc[0], scu = e_sc[NT - 1];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         const int m = (mblock * MT + mt) * 32 + l32;
@@ -469,7 +510,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     const int po = a.rope_half >> 5;
     const int lt0 = (strip / po) * 2 * po + strip % po;
     const int ca = lt0 * 32 + ng, cb = ca + a.rope_half;
-    const int fi = ca % (2 * a.rope_half);  // rotary frequency index of the first pair
     const bool rot = ca < a.rope_cols;
     if (cb + 3 < a.N) {
 #pragma unroll
@@ -479,10 +519,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
         f32x4 va = unpack_bf16x4(pack_bf16x4(own[mt * 2]));
         f32x4 vb = unpack_bf16x4(pack_bf16x4(own[mt * 2 + 1]));
         if (rot) {
-          int pos = a.rope_pos[m];
-          pos = pos < 0 ? 0 : (pos > a.rope_positions - 1 ? a.rope_positions - 1 : pos);
-          const f32x4 cs = *(const f32x4*)(a.rope_cos + (size_t)pos * a.rope_half + fi);
-          const f32x4 sn = *(const f32x4*)(a.rope_sin + (size_t)pos * a.rope_half + fi);
+          const f32x4 cs = e_rv[2 * mt], sn = e_rv[2 * mt + 1];
           f32x4 ra, rb;
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
