@@ -87,6 +87,41 @@ def gemm_launch_us(m: int, k: int, n: int, launches: int = 100, reps: int = 10, 
     return e0.elapsed_time(e1) * 1e3 / (reps * launches)
 
 
+def attn_launch_us(launches: int = 100, reps: int = 10) -> float:
+    """Average duration (us) of one action-expert attention launch (50 queries, 241 prefix + 50
+    own keys, 15/5 heads of 64, causal suffix) inside a replayed graph."""
+    import torch
+
+    from oracle.inputs import attn_case
+    from tybok_amd import ops as tk
+
+    q, k_pre, v_pre, k_suf, v_suf = (t.cuda() for t in attn_case())
+    prefix = tk.prepare_prefix_kv(k_pre, v_pre)
+    vt = torch.zeros(5, 64, 64, dtype=torch.bfloat16, device="cuda")
+    vt[:, :, :50] = v_suf.permute(1, 2, 0)
+    suffix = tk.SuffixKV(k_suf, vt)
+    out = torch.empty(50, 960, dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(3):
+            tk.expert_attn(q, prefix, suffix, None, tk.MASK_CAUSAL, out=out)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
+        for _ in range(launches):
+            tk.expert_attn(q, prefix, suffix, None, tk.MASK_CAUSAL, out=out)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * launches)
+
+
 def device_frame(engine, cameras: int, seed: int = 0) -> dict:
     """Synthetic observation (uint8-valued images / 255, random state) already on the GPU."""
     import torch
@@ -156,6 +191,8 @@ def main() -> None:
     ap.add_argument("--skip-pi05", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--gemm-only", action="store_true", help="only the roofline GEMM loop plus a plain copy of known size (for rocprofv3 runs)")
+    ap.add_argument("--gemm-shape", type=int, nargs=3, metavar=("M", "K", "N"), default=(50, 2048, 16384), help="shape of the --gemm-only loop")
+    ap.add_argument("--attn-only", action="store_true", help="only the action-expert attention loop (for rocprofv3 runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is batch-1 and single-device (--gpus must be 1)")
@@ -175,8 +212,14 @@ def main() -> None:
         for _ in range(3):
             dst.copy_(src)
         spin_up()
-        us = gemm_launch_us(50, 2048, 16384, launches=20, reps=args.steps)
-        print(json.dumps({"gemm_only": {"M": 50, "K": 2048, "N": 16384, "us": round(us, 2), "GBps": round(bytes_gemm(50, 2048, 16384) / us / 1e3, 1)}}), flush=True)
+        gm, gk, gn = args.gemm_shape
+        us = gemm_launch_us(gm, gk, gn, launches=20, reps=args.steps)
+        print(json.dumps({"gemm_only": {"M": gm, "K": gk, "N": gn, "us": round(us, 2), "GBps": round(bytes_gemm(gm, gk, gn) / us / 1e3, 1)}}), flush=True)
+        return
+    if args.attn_only:
+        spin_up()
+        us = attn_launch_us(launches=20, reps=args.steps)
+        print(json.dumps({"attn_only": {"M": 50, "P": 241, "S": 50, "H": 15, "G": 5, "D": 64, "us": round(us, 2)}}), flush=True)
         return
     flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_fused_attn=True)
     tmp = tempfile.mkdtemp(prefix="tybok_bench_")
@@ -200,7 +243,8 @@ def main() -> None:
     pi05_p50 = None
     if not args.skip_pi05:
         ckpt5 = write_pi05_checkpoint(os.path.join(tmp, "pi05"), cameras=2, seed=0)
-        eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **flags)
+        flags5 = {k: v for k, v in flags.items() if k != "tl_llm_fused_attn"}  # a SmolVLA-only tier
+        eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **flags5)
         frame5 = device_frame(eng5, 2)
         s5, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
         pi05_p50 = float(np.percentile(s5, 50))
@@ -249,7 +293,7 @@ def main() -> None:
         "dtype": "bf16 activations x fp8-e4m3 weights, fp32 accumulate",
         "data": "synthetic (random-init weights, uniform-noise images, random token ids, zero noise)",
         "config": {
-            "workload": "SmolVLA-shaped predict_action_chunk: 16+16 layers, 3 cameras 512x512, 48 tokens, chunk 50, 10 Euler steps, fp8 MLP weights, hipGraph",
+            "workload": "SmolVLA-shaped predict_action_chunk: 16+16 layers, 3 cameras 512x512, 48 tokens, chunk 50, 10 Euler steps, fp8 MLP weights, fused expert + prefill tiers, hipGraph",
             "inputs": "HBM-resident observation",
             "graph": graph_ok,
         },
