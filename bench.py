@@ -221,7 +221,7 @@ def main() -> None:
         us = attn_launch_us(launches=20, reps=args.steps)
         print(json.dumps({"attn_only": {"M": 50, "P": 241, "S": 50, "H": 15, "G": 5, "D": 64, "us": round(us, 2)}}), flush=True)
         return
-    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_fused_attn=True)
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_fused_attn=True, tl_vit_oproj=True)
     tmp = tempfile.mkdtemp(prefix="tybok_bench_")
 
     # ---- SmolVLA-shaped chunk (headline) ----
@@ -243,7 +243,7 @@ def main() -> None:
     pi05_p50 = None
     if not args.skip_pi05:
         ckpt5 = write_pi05_checkpoint(os.path.join(tmp, "pi05"), cameras=2, seed=0)
-        flags5 = {k: v for k, v in flags.items() if k != "tl_llm_fused_attn"}  # a SmolVLA-only tier
+        flags5 = {k: v for k, v in flags.items() if k not in ("tl_llm_fused_attn", "tl_vit_oproj")}  # a SmolVLA-only tier
         eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **flags5)
         frame5 = device_frame(eng5, 2)
         s5, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)

@@ -207,6 +207,16 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
                    const void* mask2d, int mask_ld, void* out, int out_sm, int M, int P, int S, int H, int G, int D,
                    int mask_mode, int logits_bf16, void* ws, size_t ws_bytes, void* stream);
 
+/* B independent unmasked attentions in one launch (the vision tower's self-attention, one problem
+ * per camera image): out[b][M, H*D] = softmax(q[b].K[b]^T * D^-0.5) . V[b].  Layouts as the prefix
+ * operands of tk_expert_attn (K [P, G, D]; V^T [G, D, >= P rounded up to 32], zero padded), with
+ * element strides q_sb / k_sb / vt_sb / out_sb between problems.  logits_bf16 = 1 rounds q.K^T to
+ * bf16 before the fp32 scale and softmax, as a bf16 matmul followed by `.float() * scale` does
+ * (tybok/policies/smolvla/models/vision.py:197-257). */
+int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const void* k, long long k_sb, int k_sl, int k_sh,
+                    const void* vt, long long vt_sb, int vt_sd, int vt_sh, void* out, long long out_sb, int out_sm, int B,
+                    int M, int P, int H, int G, int D, int logits_bf16, void* ws, size_t ws_bytes, void* stream);
+
 /* ---- diagnostics ------------------------------------------------------------------------------- */
 /* out_f32[256] = value of every e4m3fn code as decoded by the device's conversion instruction
  * (the weight path of the GEMM); used to assert the OCP (not FNUZ) flavour on the box. */

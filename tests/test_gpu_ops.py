@@ -226,6 +226,20 @@ def test_prefill_attention_with_2d_mask(tk, p, h, g, d):
     _close(got, want, f"prefill attention P={p} H={h} D={d}")
 
 
+def test_batched_vision_attention(tk):
+    # three images' self-attention in one launch, bf16-rounded logits as the torch bf16 matmul path gives
+    b, m, h, d = 3, 256, 12, 64
+    g = torch.Generator().manual_seed(6)
+    qkv = torch.randn(b, m, 3, h, d, generator=g).to(torch.bfloat16)
+    q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))  # [b, h, m, d]
+    att = torch.softmax(torch.matmul(q, k.transpose(2, 3)).float() * d**-0.5, dim=-1).to(v.dtype)
+    want = torch.matmul(att, v).transpose(1, 2).reshape(b, m, h * d)
+    dev = qkv.cuda()
+    vt = dev[:, :, 2].permute(0, 2, 3, 1).contiguous()
+    got = tk.batched_attn(dev[:, :, 0], dev[:, :, 1], vt, logits_bf16=True)
+    _close(got, want, "batched vision attention")
+
+
 def test_gated_residual_epilogue(tk):
     # pi0.5 AdaRMS gated residual: y = resid + bf16(ffn(x) * gate)
     x, wg8, sg, wu8, su, wd8, sd = ffn_case(50, 1024, 4096, seed=3)

@@ -55,8 +55,14 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
   const int half = lane >> 5;
   const int l32 = lane & 31;
   const int h = blockIdx.x;
-  const int mtile = blockIdx.y;
+  const int mtiles = (a.M + 31) >> 5;
+  const int bi = blockIdx.y / mtiles;        // problem of a batched launch
+  const int mtile = blockIdx.y % mtiles;
   const int split = blockIdx.z;
+  a.q += bi * a.q_sb;
+  a.k_pre += bi * a.k_sb;
+  a.vt_pre += bi * a.vt_sb;
+  a.out += bi * a.out_sb;
   const int g = h / (a.H / a.G);
   const int tp = (a.P + 31) >> 5;            // prefix tiles; suffix tiles follow
   const int ntiles = tp + ((a.S + 31) >> 5);
@@ -259,7 +265,7 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
 
   // ---- kv-split merge by the last-arriving block ----
   // partials per (block, split): [2][32] stats, then [DT][4 groups][64 lanes][4 floats]
-  const int blk_lin = mtile * a.H + h;
+  const int blk_lin = blockIdx.y * a.H + h;
   constexpr size_t PSTRIDE = 64 + (size_t)DT * 1024;  // floats
   float* pmine = a.partial + ((size_t)blk_lin * a.kv_splits + split) * PSTRIDE;
   if (wave == 0 && half == 0) {
@@ -376,7 +382,7 @@ __global__ void kv_prepare_kernel(KvPrepArgs p) {
 
 template <int D, bool SPLIT>
 int launch_attn(const AttnArgs& a, hipStream_t st) {
-  dim3 grid(a.H, (a.M + 31) / 32, a.kv_splits);
+  dim3 grid(a.H, ((a.M + 31) / 32) * (a.batch > 0 ? a.batch : 1), a.kv_splits);
   hipLaunchKernelGGL((expert_attn_kernel<D, SPLIT>), grid, dim3(kNW * 64), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }

@@ -332,7 +332,7 @@ int tk_attn_prepare_kv(const void* k, const void* v, int kv_dtype, int sl, int s
   return TK_OK;
 }
 
-int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* k_pre_lo, int pre_sl, int pre_sh,
+static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb, long long out_sb, const void* q, int q_sm, int q_sh, const void* k_pre, const void* k_pre_lo, int pre_sl, int pre_sh,
                    const void* vt_pre, const void* vt_pre_lo, int pre_vt_sd, int pre_vt_sh, const void* k_suf, int suf_sl,
                    int suf_sh, const void* vt_suf, int suf_vt_sd, int suf_vt_sh, const void* pad, const void* mask2d,
                    int mask_ld, void* out, int out_sm, int M, int P, int S, int H, int G, int D, int mask_mode,
@@ -384,6 +384,11 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
   a.out = (u16*)out;
   a.out_sm = out_sm;
   a.M = M;
+  a.batch = batch;
+  a.q_sb = q_sb;
+  a.k_sb = k_sb;
+  a.vt_sb = vt_sb;
+  a.out_sb = out_sb;
   a.P = P;
   a.S = S;
   a.H = H;
@@ -393,7 +398,7 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
   a.scale = 1.0f / sqrtf((float)D);
 
   const int ntiles = (P + 31) / 32 + (S + 31) / 32;
-  const int mtiles = (M + 31) / 32;
+  const int mtiles = ((M + 31) / 32) * (batch > 0 ? batch : 1);
   // one 32-key tile per wave: split the keys over blocks of four waves (at most 8 splits, beyond
   // that a wave loops over several tiles)
   int splits = (ntiles + 3) / 4;
@@ -415,6 +420,26 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
   int rc = tk_launch_attn(a, D, (hipStream_t)stream);
   if (rc) return fail(TK_ELAUNCH, "attn: launch failed (%s)", hipGetErrorString(hipGetLastError()));
   return TK_OK;
+}
+
+int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* k_pre_lo, int pre_sl, int pre_sh,
+                   const void* vt_pre, const void* vt_pre_lo, int pre_vt_sd, int pre_vt_sh, const void* k_suf, int suf_sl,
+                   int suf_sh, const void* vt_suf, int suf_vt_sd, int suf_vt_sh, const void* pad, const void* mask2d,
+                   int mask_ld, void* out, int out_sm, int M, int P, int S, int H, int G, int D, int mask_mode,
+                   int logits_bf16, void* ws, size_t ws_bytes, void* stream) {
+  return attn_impl(0, 0, 0, 0, 0, q, q_sm, q_sh, k_pre, k_pre_lo, pre_sl, pre_sh, vt_pre, vt_pre_lo, pre_vt_sd, pre_vt_sh, k_suf,
+                   suf_sl, suf_sh, vt_suf, suf_vt_sd, suf_vt_sh, pad, mask2d, mask_ld, out, out_sm, M, P, S, H, G, D, mask_mode,
+                   logits_bf16, ws, ws_bytes, stream);
+}
+
+int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const void* k, long long k_sb, int k_sl, int k_sh,
+                    const void* vt, long long vt_sb, int vt_sd, int vt_sh, void* out, long long out_sb, int out_sm, int B,
+                    int M, int P, int H, int G, int D, int logits_bf16, void* ws, size_t ws_bytes, void* stream) {
+  if (B <= 0) return fail(TK_EINVAL, "batched_attn: B=%d", B);
+  if (q_sb % 8 || k_sb % 8 || vt_sb % 8 || out_sb % 4) return fail(TK_EINVAL, "batched_attn: batch strides must keep 16-byte alignment");
+  return attn_impl(B, q_sb, k_sb, vt_sb, out_sb, q, q_sm, q_sh, k, nullptr, k_sl, k_sh, vt, nullptr, vt_sd, vt_sh, nullptr, 0, 0,
+                   nullptr, 0, 0, nullptr, nullptr, 0, out, out_sm, M, P, 0, H, G, D, TK_MASK_NONE, logits_bf16, ws, ws_bytes,
+                   stream);
 }
 
 int tk_debug_decode_fp8(void* out_f32, void* stream) {

@@ -61,6 +61,9 @@ struct AttnArgs {
   unsigned short* out;
   int out_sm;
   int M, P, S, H, G;
+  // independent problems in one launch (prefix-only): element strides between them, 0 = single
+  int batch;
+  long long q_sb, k_sb, vt_sb, out_sb;
   int mask_mode, logits_bf16;
   int kv_splits;
   float* partial;

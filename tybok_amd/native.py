@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_longlong, c_size_t, c_void_p
 
 # TYBOK_HIP_LIB points at an alternative build of the same ABI (kernel experiments); default in-tree.
 _LIB_PATH = os.environ.get("TYBOK_HIP_LIB") or os.path.join(
@@ -54,6 +54,11 @@ SIGNATURES: dict[str, tuple] = {
         c_int,
         [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
          c_void_p],
+    ),  # fmt: skip
+    "tk_batched_attn": (
+        c_int,
+        [c_void_p, c_longlong, c_int, c_int, c_void_p, c_longlong, c_int, c_int, c_void_p, c_longlong, c_int, c_int,
+         c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
     "tk_expert_attn": (
         c_int,

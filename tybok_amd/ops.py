@@ -449,6 +449,40 @@ def expert_attn(
     return out
 
 
+def batched_attn(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    vt: torch.Tensor,
+    *,
+    logits_bf16: bool = False,
+    out: torch.Tensor | None = None,
+    ws: Workspace | None = None,
+) -> torch.Tensor:
+    """``B`` independent unmasked attentions: ``q [B, M, H, D]``, ``k [B, P, G, D]`` (views with a
+    contiguous head dim), ``vt [B, G, D, >= P rounded up to 32]`` (V transposed, zero padded) ->
+    bf16 ``[B, M, H*D]``."""
+    lib = native.lib()
+    bf = torch.bfloat16
+    if q.dtype != bf or k.dtype != bf or vt.dtype != bf or q.dim() != 4 or k.dim() != 4 or vt.dim() != 4:
+        raise TypeError("q, k, vt must be 4-D bf16 tensors")
+    b, m, h, d = q.shape
+    p, g = k.shape[1], k.shape[2]
+    if k.shape[0] != b or k.shape[3] != d or vt.shape[:3] != (b, g, d) or vt.shape[3] < _pad32(p):
+        raise ValueError("k must be [B, P, G, D] and vt [B, G, D, >= P rounded up to 32]")
+    if q.stride(3) != 1 or k.stride(3) != 1 or vt.stride(3) != 1:
+        raise ValueError("q, k need a contiguous head dim and vt contiguous keys")
+    if out is None:
+        out = torch.empty(b, m, h * d, dtype=bf, device=q.device)
+    ws = ws or default_workspace(q.device)
+    rc = lib.tk_batched_attn(
+        q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), k.data_ptr(), k.stride(0), k.stride(1), k.stride(2) if g > 1 else 0,
+        vt.data_ptr(), vt.stride(0), vt.stride(2), vt.stride(1) if g > 1 else 0, out.data_ptr(), out.stride(0), out.stride(1),
+        b, m, p, h, g, d, int(logits_bf16), ws.ptr, ws.nbytes, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_batched_attn")
+    return out
+
+
 def expert_attn_plain(
     q: torch.Tensor,
     k_pre: torch.Tensor | None,

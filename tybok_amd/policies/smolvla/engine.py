@@ -4,14 +4,16 @@ Constructor keywords, ``describe()`` keys and the ``predict_action_chunk`` / ``s
 semantics are the reference's (tybok/policies/smolvla/engine.py:78-96, 332-400), so the worker and
 gateway need no change.  The tier flags select the HIP kernels:
 
-* ``tl_fused_expert``     expert denoising attention on ``tk_expert_attn``
+* ``tl_fused_expert``     expert layers on the fused launches: norm + q|k|v + RoPE
+                          (``tk_bf16w_linear``), ``tk_expert_attn``, o_proj + residual
 * ``tl_fp8_expert_mlp``   expert gated FFN on e4m3fn weights (``tk_fp8w_gated_ffn``)
 * ``tl_fp8_llm_mlp``      VLM prefill gated FFN on e4m3fn weights
+* ``tl_llm_fused_attn``   VLM prefill layers on the same fused launches (2-D prefix mask)
+* ``tl_vit_oproj``        vision tower with packed q|k|v and ``tk_batched_attn``
 
 The reference's SmolVLA backend rejects the two fp8 flags (engine.py:47-55); here they are
 implemented, because the fp8 action-inference path is what this backend is for.
-``tl_llm_fused_attn`` / ``tl_vit_oproj`` (prefill / vision fusions) and ``compile_model`` have no
-implementation here and are rejected when requested.
+``compile_model`` has no implementation here and is rejected when requested.
 """
 
 from __future__ import annotations
@@ -51,7 +53,6 @@ log = logging.getLogger("tybok.smolvla")
 class SmolVLAEngine(PolicyEngine):
     # flags owned by other backends or not implemented here: inert default -> accepted, else rejected
     _UNSUPPORTED_FLAGS = {
-        "tl_vit_oproj": False,
         "tl_fused_vit": False,
         "tl_llm_flash_attn": False,
         "vit_mlp_dtype": None,
@@ -97,8 +98,6 @@ class SmolVLAEngine(PolicyEngine):
             raise ValueError(f"unknown sampler {sampler!r} (this backend implements 'euler')")
         if compile_model:
             raise NotImplementedError("--compile is not supported by this backend (the HIP tiers replace it)")
-        if tl_vit_oproj:
-            raise NotImplementedError("--tl-vit-oproj is not implemented by this backend")
         self.compile_model = False
         self.config = SmolVLAConfig.from_pretrained(checkpoint_dir)
         if self.config.vlm_config is None:
@@ -114,6 +113,7 @@ class SmolVLAEngine(PolicyEngine):
             for n, on in (
                 ("--tl-fused-expert", tl_fused_expert), ("--tl-fp8-llm-mlp", tl_fp8_llm_mlp),
                 ("--tl-fp8-expert-mlp", tl_fp8_expert_mlp), ("--tl-llm-fused-attn", tl_llm_fused_attn),
+                ("--tl-vit-oproj", tl_vit_oproj),
             )
             if on
         ]  # fmt: skip
@@ -139,10 +139,13 @@ class SmolVLAEngine(PolicyEngine):
         # --tl-llm-fused-attn: the VLM prefill layers on the fused HIP launches (norm + q/k/v + RoPE +
         # KV write, attention under the 2-D prefix mask, o_proj + residual)
         self.tl_llm_fused_attn = bool(tl_llm_fused_attn)
+        # --tl-vit-oproj: vision tower with q/k/v packed into one GEMM and the self-attention on the
+        # HIP kernel (the reference's tier packs q/k/v and fuses out_proj over the SDPA layout)
+        self.tl_vit_oproj = bool(tl_vit_oproj)
         self.model = SmolVLAModel(
             self.config, sd, self.device,
             fused_expert=self.tl_fused_expert, fp8_expert_mlp=self.tl_fp8_expert_mlp, fp8_llm_mlp=self.tl_fp8_llm_mlp,
-            fused_prefill=self.tl_llm_fused_attn,
+            fused_prefill=self.tl_llm_fused_attn, fused_vit=self.tl_vit_oproj,
         )  # fmt: skip
         del sd
 

@@ -103,6 +103,7 @@ class SmolVLAModel:
         fp8_expert_mlp: bool = False,
         fp8_llm_mlp: bool = False,
         fused_prefill: bool = False,
+        fused_vit: bool = False,
     ):
         assert cfg.vlm_config is not None
         self.cfg = cfg
@@ -111,7 +112,8 @@ class SmolVLAModel:
         self.fp8_expert_mlp = bool(fp8_expert_mlp)
         self.fp8_llm_mlp = bool(fp8_llm_mlp)
         self.fused_prefill = bool(fused_prefill)
-        self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp or self.fused_prefill
+        self.fused_vit = bool(fused_vit)
+        self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp or self.fused_prefill or self.fused_vit
         if self.use_hip and self.device.type != "cuda":
             raise RuntimeError("the fused / fp8 tiers run HIP kernels and need a GPU device")
         t = cfg.vlm_config.text_config
@@ -126,6 +128,14 @@ class SmolVLAModel:
         self.ws = tk.default_workspace(self.device) if self.use_hip else None
         if self.fused_prefill:
             self.vlm_qkv, self.vlm_o = self._pack_attention_weights(TXT, lambda i: False)
+        if self.fused_vit:
+            # vision q|k|v as one projection (one GEMM over all cameras' patches instead of three)
+            self.vis_qkv = []
+            for i in range(cfg.vlm_config.vision_config.num_hidden_layers):
+                lp = f"{VIS}encoder.layers.{i}.self_attn."
+                w = torch.cat([self.p[lp + n + "_proj.weight"] for n in "qkv"], dim=0).contiguous()
+                b = torch.cat([self.p[lp + n + "_proj.bias"] for n in "qkv"], dim=0).contiguous()
+                self.vis_qkv.append((w, b))
         if self.fused_expert:
             self._pack_expert_projections()
             # V^T of the action tokens [G, D, chunk rounded up to 32]; the projection kernel writes
@@ -202,6 +212,17 @@ class SmolVLAModel:
         for i in range(v.num_hidden_layers):
             lp = f"{VIS}encoder.layers.{i}."
             h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], v.layer_norm_eps)
+            if self.fused_vit:
+                # packed q|k|v GEMM, then the HIP attention (one problem per camera): q.K^T rounded to
+                # bf16 before the fp32 scale and softmax, exactly what the bf16 matmul below produces
+                w_qkv, b_qkv = self.vis_qkv[i]
+                qkv = F.linear(h, w_qkv, b_qkv).view(b, -1, 3, heads, hd)
+                vt = qkv[:, :, 2].permute(0, 2, 3, 1).contiguous()
+                a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, ws=self.ws)
+                x = x + self.lin(lp + "self_attn.out_proj", a)
+                h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
+                x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
+                continue
             q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
             k = self.lin(lp + "self_attn.k_proj", h).view(b, -1, heads, hd).transpose(1, 2)
             val = self.lin(lp + "self_attn.v_proj", h).view(b, -1, heads, hd).transpose(1, 2)
