@@ -117,8 +117,12 @@ int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void
  * the gate/up launch while the activations are staged (bf16 x: bf16(w * bf16(x * rstd)), fp32
  * statistics), as the reference's `triton_norm_gate_up(x, norm_w, eps, gate_w, up_w)` folds it
  * (tybok/policies/smolvla/models/triton_mlp.py:105-144, call site vlm_with_expert.py:391-408).
- *   norm_w: bf16 [K], 16-byte aligned.  Other arguments as tk_fp8w_gated_ffn. */
-int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float norm_eps, const void* wgu_packed,
+ *   norm_w: bf16 [K], 16-byte aligned; or NULL with ada_scale / ada_shift (fp32 [K] each): the
+ *           adaptive RMSNorm of pi0.5, bf16((x * rstd) * (1 + scale) + shift) in fp32, as
+ *           `triton_norm_gate_up_fp8` folds it (tybok/policies/pi05/models/triton_expert_mlp_fp8.py:54-197;
+ *           eager: tybok/policies/pi05/models/layers.py:51-84).  Other arguments as tk_fp8w_gated_ffn. */
+int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float norm_eps, const void* ada_scale,
+                           const void* ada_shift, const void* wgu_packed,
                            const void* sg, const void* su, const void* wd_packed, const void* sd, void* y, int ldy,
                            const void* resid, int ldr, int resid_dtype, const void* gate, int M, int K, int I,
                            int act, void* ws, size_t ws_bytes, void* stream);
@@ -150,6 +154,15 @@ int tk_pack_bf16_weight(const void* w, void* packed, int N, int K, int rope_half
  *              eager: tybok/policies/smolvla/models/rope.py:51-73).
  *   rope_pos: int32 [M] (clamped into [0, rope_positions)); rope_cos/rope_sin: fp32
  *             [rope_positions, rope_half].
+ *   ada_scale / ada_shift: fp32 [K], instead of norm_w: adaptive RMSNorm prologue (pi0.5),
+ *             bf16((x * rstd) * (1 + scale) + shift) with every step rounded in fp32
+ *             (tybok/policies/pi05/models/layers.py:51-84).
+ *   rope_bf16: 1 = rotate in bf16 arithmetic, every product and the sum rounded to bf16 and the
+ *             tables holding bf16 values: pi0.5's `x * cos + rotate_half(x) * sin` on bf16 tensors
+ *             (tybok/policies/pi05/models/rope.py:59-75).
+ *   gate:     optional bf16 [N], plain epilogue only: y = bf16(bf16(acc) * gate[n]) before the
+ *             residual -- pi0.5's gated residual `res + o_proj(att) * gate`
+ *             (tybok/policies/pi05/models/triton_expert_residual.py:26-60).
  *   vt:       optional (rotary epilogue only): the columns n >= vt_col0 (the value projection;
  *             vt_col0 a head boundary >= rope_cols) are also written transposed,
  *             vt[(n - vt_col0) * vt_ld + m], the suffix V^T operand of tk_expert_attn; entries
@@ -157,10 +170,10 @@ int tk_pack_bf16_weight(const void* w, void* packed, int N, int K, int rope_half
  * Built for the action-chunk tile shape (any M, tiled 64 rows at a time); the norm prologue is
  * built together with the rotary epilogue only. */
 int tk_bf16w_linear(const void* x, int ldx, int x_dtype, const void* w_packed, const void* norm_w, float norm_eps,
-                    const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions,
-                    int rope_cols, int rope_half, void* vt, int vt_col0, int vt_ld, void* y, int ldy,
-                    const void* resid, int ldr, int resid_dtype, int M, int N, int K, int split_k, void* ws,
-                    size_t ws_bytes, void* stream);
+                    const void* ada_scale, const void* ada_shift, const void* rope_pos, const void* rope_cos,
+                    const void* rope_sin, int rope_positions, int rope_cols, int rope_half, int rope_bf16, void* vt,
+                    int vt_col0, int vt_ld, void* y, int ldy, const void* resid, int ldr, int resid_dtype,
+                    const void* gate, int M, int N, int K, int split_k, void* ws, size_t ws_bytes, void* stream);
 
 /* ---- action-expert attention over the cached prefix ------------------------------------------ */
 /* Lays one layer's prefix K/V out for tk_expert_attn, once per request (the counterpart of the

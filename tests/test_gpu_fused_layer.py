@@ -152,6 +152,52 @@ def test_norm_gated_ffn(tk, act, m, k, i):
     assert mism < 0.02, f"fused norm differs from norm-then-FFN on {mism:.1%} of the outputs"
 
 
+@pytest.mark.parametrize("m,k,heads,kv_heads,d", [(50, 1024, 8, 1, 256), (19, 96, 2, 1, 64)])
+def test_adarms_qkv_rope_bf16_arithmetic(tk, m, k, heads, kv_heads, d):
+    # the pi0.5 expert projection: adaptive RMSNorm prologue, rotate-half RoPE in bf16 arithmetic
+    eps = 1e-6
+    x, _, w, pos, n = _qkv_case(m, k, heads, kv_heads, d, BF16, seed=16)
+    g = torch.Generator().manual_seed(17)
+    mod = 0.3 * torch.randn(1, 3 * k, generator=g)
+    h, _ = oops.gemma_rms_norm(x[None], eps, modulation=mod)
+    y = F.linear(h[0], w)
+    rc = (heads + kv_heads) * d
+    cos, sin = oops.gemma_rope_cos_sin(d, pos[None].long(), BF16)
+    qk = oops.gemma_apply_rope(y[:, :rc].reshape(1, m, heads + kv_heads, d).transpose(1, 2), cos, sin)
+    want = torch.cat([qk.transpose(1, 2).reshape(m, rc), y[:, rc:]], dim=1)
+    cos_t, sin_t = oops.gemma_rope_cos_sin(d, torch.arange(512)[None], BF16)
+    rope = tk.RopeTables(cos_t[0, :, : d // 2].float().contiguous().cuda(), sin_t[0, :, : d // 2].float().contiguous().cuda())
+    scale, shift = mod[0, :k].contiguous().cuda(), mod[0, k : 2 * k].contiguous().cuda()
+    pw = tk.pack_bf16_weight(w.cuda(), rope_half=d // 2)
+    got = tk.bf16w_linear(x.cuda(), pw, ada=(scale, shift), eps=eps, rope=rope, rope_pos=pos.cuda(), rope_cols=rc, rope_bf16=True)
+    _close(got, want, f"adarms+qkv+rope(bf16) M={m} K={k} D={d}")
+    mism = (got.cpu() != want).float().mean().item()
+    assert mism < 0.03, f"{mism:.1%} of the outputs differ from the eager composition (expected: rare 1-ulp flips)"
+
+
+def test_gated_residual_o_proj_and_adarms_ffn(tk):
+    m, k, n = 50, 2048, 1024
+    g = torch.Generator().manual_seed(18)
+    x = torch.randn(m, k, generator=g).to(BF16)
+    w = (torch.randn(n, k, generator=g) * k**-0.5).to(BF16)
+    gate = torch.randn(n, generator=g).to(BF16)
+    resid = torch.randn(m, n, generator=g).to(BF16)
+    want = resid + F.linear(x, w) * gate
+    got = tk.bf16w_linear(x.cuda(), tk.pack_bf16_weight(w.cuda()), resid=resid.cuda(), gate=gate.cuda())
+    _close(got, want, "o_proj gated residual")
+    # adaptive norm + GeGLU FFN + gated residual
+    eps = 1e-6
+    xx, wg8, sg, wu8, su, wd8, sd = ffn_case(m, 1024, 4096, seed=19)
+    mod = 0.3 * torch.randn(1, 3 * 1024, generator=g)
+    h, gt = oops.gemma_rms_norm(xx[None], eps, modulation=mod)
+    want = xx + oops.gated_ffn(h[0], wg8, sg, wu8, su, wd8, sd, "gelu_tanh") * gt[0]
+    wgu = tk.pack_fp8_gate_up(wg8.cuda(), sg, wu8.cuda(), su)
+    wd = tk.pack_fp8_weight(wd8.cuda(), sd)
+    scale, shift = mod[0, :1024].contiguous().cuda(), mod[0, 1024:2048].contiguous().cuda()
+    got = tk.fp8w_gated_ffn(xx.cuda(), wgu, wd, "gelu_tanh", resid=xx.cuda(), gate=gt[0].contiguous().cuda(), ada=(scale, shift), eps=eps)
+    _close(got, want, "adarms + GeGLU FFN + gated residual")
+
+
 def test_fused_layer_argument_checks(tk):
     w = torch.zeros(128, 64, dtype=BF16, device="cuda")
     x = torch.zeros(4, 64, dtype=BF16, device="cuda")

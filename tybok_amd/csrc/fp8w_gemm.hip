@@ -51,7 +51,8 @@ __device__ __forceinline__ void lds_barrier() {
 // EPI: 0 plain (scale, optional per-column gate, optional residual), 1 gated (gate/up tile pairs ->
 //      act(g)*u), 2 rope (tile pairs hold columns (i, i + D/2) of one head -> rotary embedding).
 // W16: weights are bf16 (two 16-byte operand chunks per lane and k tile) instead of e4m3.
-// PRO: 0 none, 1 RMSNorm of bf16 activations, 2 RMSNorm of fp32 activations -- applied while the
+// PRO: 0 none, 1 RMSNorm of bf16 activations, 2 RMSNorm of fp32 activations, 3 adaptive RMSNorm of
+//      bf16 activations: bf16((x * rstd) * (1 + scale[k]) + shift[k]) in fp32 -- applied while the
 //      activations are staged into LDS, with the reference's rounding points:
 //      bf16 input: bf16(w * bf16(x * rstd));  fp32 input: bf16(w * (x * rstd)).
 template <int MT, int NT, int NW, int EPI, int PF, int TPW, bool W16, int PRO>
@@ -142,9 +143,10 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
         for (int c = 0; c < WCH; ++c) f.w[j][nt][c] = *(const i32x4*)(wbase[nt] + (size_t)kt * WTILE + c * 1024);
     }
   };
+  constexpr bool ADA = PRO == 3;
   struct XFrag {
     i32x4 v[XPT][XF32 ? 2 : 1];
-    i32x4 nw[PRO ? XPT : 1];  // norm weights of the piece's 8 columns
+    i32x4 nw[PRO ? XPT : 1][ADA ? 4 : 1];  // norm weights of the piece's 8 columns (ADA: fp32 scale, shift)
   };
   auto xload = [&](XFrag& f, int r) {
 #ifdef TK_EXP_NOX
@@ -162,7 +164,14 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       } else {
         f.v[i][0] = *(const i32x4*)(xsrc[i] + (size_t)k * 2);
       }
-      if (PRO) f.nw[i] = *(const i32x4*)(a.norm_w + k);
+      if (ADA) {
+        f.nw[i][0] = *(const i32x4*)(a.ada_scale + k);
+        f.nw[i][ADA ? 1 : 0] = *(const i32x4*)(a.ada_scale + k + 4);
+        f.nw[i][ADA ? 2 : 0] = *(const i32x4*)(a.ada_shift + k);
+        f.nw[i][ADA ? 3 : 0] = *(const i32x4*)(a.ada_shift + k + 4);
+      } else if (PRO) {
+        f.nw[i][0] = *(const i32x4*)(a.norm_w + k);
+      }
     }
   };
   float my_rstd[XPT];
@@ -177,9 +186,26 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       i32x4 out;
       if (PRO == 0) {
         out = f.v[i][0];
+      } else if (ADA) {
+        union { i32x4 v; unsigned u[4]; } xu, o;
+        union { i32x4 v[2]; float f[8]; } sc, sh;
+        xu.v = f.v[i][0];
+        sc.v[0] = f.nw[i][0];
+        sc.v[1] = f.nw[i][ADA ? 1 : 0];
+        sh.v[0] = f.nw[i][ADA ? 2 : 0];
+        sh.v[1] = f.nw[i][ADA ? 3 : 0];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          // separately rounded fp32 operations, as the elementwise reference computes them
+          const float x0 = __uint_as_float(xu.u[e] << 16), x1 = __uint_as_float(xu.u[e] & 0xffff0000u);
+          const float y0 = __fadd_rn(__fmul_rn(__fmul_rn(x0, my_rstd[i]), __fadd_rn(1.0f, sc.f[2 * e])), sh.f[2 * e]);
+          const float y1 = __fadd_rn(__fmul_rn(__fmul_rn(x1, my_rstd[i]), __fadd_rn(1.0f, sc.f[2 * e + 1])), sh.f[2 * e + 1]);
+          o.u[e] = pack_bf16x2(y0, y1);
+        }
+        out = o.v;
       } else {
         union { i32x4 v; unsigned u[4]; } nwu, o;
-        nwu.v = f.nw[i];
+        nwu.v = f.nw[i][0];
         float xv[8];
         if (XF32) {
           union { i32x4 v; float f[4]; } lo, hi;
@@ -521,11 +547,20 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
         if (rot) {
           const f32x4 cs = e_rv[2 * mt], sn = e_rv[2 * mt + 1];
           f32x4 ra, rb;
+          if (a.rope_bf16) {
+            // bf16 arithmetic (x * cos + rotate_half(x) * sin on bf16 tensors): every product and
+            // the sum round to bf16; the tables hold bf16 values
+            const f32x4 ac = unpack_bf16x4(pack_bf16x4(va * cs)), bs = unpack_bf16x4(pack_bf16x4(vb * sn));
+            const f32x4 bc = unpack_bf16x4(pack_bf16x4(vb * cs)), as = unpack_bf16x4(pack_bf16x4(va * sn));
+            ra = ac - bs;
+            rb = bc + as;
+          } else {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            // separately rounded products, as an elementwise fp32 implementation computes them
-            ra[j] = __fsub_rn(__fmul_rn(va[j], cs[j]), __fmul_rn(vb[j], sn[j]));
-            rb[j] = __fadd_rn(__fmul_rn(vb[j], cs[j]), __fmul_rn(va[j], sn[j]));
+            for (int j = 0; j < 4; ++j) {
+              // separately rounded products, as an elementwise fp32 implementation computes them
+              ra[j] = __fsub_rn(__fmul_rn(va[j], cs[j]), __fmul_rn(vb[j], sn[j]));
+              rb[j] = __fadd_rn(__fmul_rn(vb[j], cs[j]), __fmul_rn(va[j], sn[j]));
+            }
           }
           va = ra;
           vb = rb;
@@ -628,13 +663,14 @@ int launch(const GemmArgs& a, dim3 grid, hipStream_t st) {
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st) {
   dim3 grid((a.ntiles + NT - 1) / NT, a.ksplit, mblocks);
   const int epi = a.s1 != nullptr ? 1 : (a.rope_pos != nullptr ? 2 : 0);
-  const int pro = a.norm_w == nullptr ? 0 : (a.x_f32 ? 2 : 1);
+  const int pro = a.ada_scale != nullptr ? 3 : (a.norm_w == nullptr ? 0 : (a.x_f32 ? 2 : 1));
   if (a.w16) {
     // bf16-weight linears of the expert layers (M > 32 only: the action chunk)
     if (MT != 2 || NT != 2) return -1;
     if (epi == 2) {
       if (pro == 1) return launch<2, 2, 2, true, 1>(a, grid, st);
       if (pro == 2) return launch<2, 2, 2, true, 2>(a, grid, st);
+      if (pro == 3) return launch<2, 2, 2, true, 3>(a, grid, st);
       return launch<2, 2, 2, true, 0>(a, grid, st);
     }
     if (epi == 0 && pro == 0) return launch<2, 2, 0, true, 0>(a, grid, st);
@@ -644,6 +680,7 @@ int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st) {
   if (epi == 1) {
     if (NT != 2) return -1;
     if (pro == 1) return MT == 1 ? launch<1, 2, 1, false, 1>(a, grid, st) : launch<2, 2, 1, false, 1>(a, grid, st);
+    if (pro == 3) return MT == 1 ? launch<1, 2, 1, false, 3>(a, grid, st) : launch<2, 2, 1, false, 3>(a, grid, st);
     return MT == 1 ? launch<1, 2, 1, false, 0>(a, grid, st) : launch<2, 2, 1, false, 0>(a, grid, st);
   }
   if (pro) return -1;

@@ -48,10 +48,12 @@ struct GemmExtra {
   int w16 = 0;                    // bf16 weight tiles
   const void* norm_w = nullptr;   // RMSNorm prologue
   float norm_eps = 0.f;
+  const void* ada_scale = nullptr;  // adaptive RMSNorm prologue (fp32 [K] scale / shift)
+  const void* ada_shift = nullptr;
   const int* rope_pos = nullptr;  // rotary epilogue
   const float* rope_cos = nullptr;
   const float* rope_sin = nullptr;
-  int rope_positions = 0, rope_cols = 0, rope_half = 0;
+  int rope_positions = 0, rope_cols = 0, rope_half = 0, rope_bf16 = 0;
   void* vt = nullptr;  // transposed copy of the columns >= vt_col0 (rotary epilogue)
   int vt_col0 = 0, vt_ld = 0;
 };
@@ -72,6 +74,9 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   const bool rope = e.rope_pos != nullptr;
   if (gated && (N % 32)) return fail(TK_EINVAL, "gated gemm: I=%d must be a multiple of 32", N);
   if (e.x_f32 && !e.norm_w) return fail(TK_EINVAL, "gemm: fp32 activations need the norm prologue");
+  if ((e.ada_scale != nullptr) != (e.ada_shift != nullptr)) return fail(TK_EINVAL, "gemm: adaptive norm needs both scale and shift");
+  if (e.ada_scale && (e.norm_w || e.x_f32 || !aligned16(e.ada_scale) || !aligned16(e.ada_shift)))
+    return fail(TK_EINVAL, "gemm: adaptive norm takes bf16 activations, no norm weight, 16-byte aligned scale / shift");
   if (e.norm_w && !aligned16(e.norm_w)) return fail(TK_EINVAL, "gemm: norm weight must be 16-byte aligned");
   if (rope) {
     if (gated || resid || gate) return fail(TK_EINVAL, "gemm: the rotary epilogue excludes gate/residual epilogues");
@@ -115,6 +120,9 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   }
   a.norm_w = (const u16*)e.norm_w;
   a.norm_eps = e.norm_eps;
+  a.ada_scale = (const float*)e.ada_scale;
+  a.ada_shift = (const float*)e.ada_shift;
+  a.rope_bf16 = e.rope_bf16;
   a.rope_pos = e.rope_pos;
   a.rope_cos = e.rope_cos;
   a.rope_sin = e.rope_sin;
@@ -262,35 +270,41 @@ int tk_pack_bf16_weight(const void* w, void* packed, int N, int K, int rope_half
 }
 
 int tk_bf16w_linear(const void* x, int ldx, int x_dtype, const void* w_packed, const void* norm_w, float norm_eps,
-                    const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions, int rope_cols,
-                    int rope_half, void* vt, int vt_col0, int vt_ld, void* y, int ldy, const void* resid, int ldr,
-                    int resid_dtype, int M, int N, int K, int split_k, void* ws, size_t ws_bytes, void* stream) {
+                    const void* ada_scale, const void* ada_shift, const void* rope_pos, const void* rope_cos,
+                    const void* rope_sin, int rope_positions, int rope_cols, int rope_half, int rope_bf16, void* vt,
+                    int vt_col0, int vt_ld, void* y, int ldy, const void* resid, int ldr, int resid_dtype, const void* gate,
+                    int M, int N, int K, int split_k, void* ws, size_t ws_bytes, void* stream) {
   if (x_dtype != TK_BF16 && x_dtype != TK_F32) return fail(TK_EINVAL, "bf16w_linear: bad x_dtype");
   GemmExtra e;
   e.x_f32 = x_dtype == TK_F32;
   e.w16 = 1;
   e.norm_w = norm_w;
   e.norm_eps = norm_eps;
+  e.ada_scale = ada_scale;
+  e.ada_shift = ada_shift;
   e.rope_pos = (const int*)rope_pos;
   e.rope_cos = (const float*)rope_cos;
   e.rope_sin = (const float*)rope_sin;
   e.rope_positions = rope_positions;
   e.rope_cols = rope_cols;
   e.rope_half = rope_half;
+  e.rope_bf16 = rope_bf16;
   e.vt = vt;
   e.vt_col0 = vt_col0;
   e.vt_ld = vt_ld;
-  if (!rope_pos && norm_w) return fail(TK_EINVAL, "bf16w_linear: the norm prologue is built for the rotary projection only");
-  return gemm_common(x, ldx, w_packed, nullptr, nullptr, y, ldy, resid, ldr, resid_dtype, nullptr, M, N, K, split_k, 0, ws,
+  if (!rope_pos && (norm_w || ada_scale))
+    return fail(TK_EINVAL, "bf16w_linear: the norm prologues are built for the rotary projection only");
+  return gemm_common(x, ldx, w_packed, nullptr, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, N, K, split_k, 0, ws,
                      ws_bytes, (hipStream_t)stream, e);
 }
 
-int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float norm_eps, const void* wgu_packed,
+int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float norm_eps, const void* ada_scale,
+                           const void* ada_shift, const void* wgu_packed,
                            const void* sg, const void* su, const void* wd_packed, const void* sd, void* y, int ldy,
                            const void* resid, int ldr, int resid_dtype, const void* gate, int M, int K, int I, int act,
                            void* ws, size_t ws_bytes, void* stream) {
   if (act != TK_ACT_SILU && act != TK_ACT_GELU_TANH) return fail(TK_EINVAL, "ffn: unknown activation %d", act);
-  if (!sg || !su || !sd || !norm_w) return fail(TK_EINVAL, "ffn: null scale or norm pointer");
+  if (!sg || !su || !sd || (!norm_w && !ada_scale)) return fail(TK_EINVAL, "ffn: null scale or norm pointer");
   if (I % 32) return fail(TK_EINVAL, "ffn: I=%d must be a multiple of 32", I);
   if (!ws) return fail(TK_EWORKSPACE, "ffn: needs a workspace");
   const size_t hbytes = (size_t)M * I * 2;
@@ -300,6 +314,8 @@ int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float nor
   GemmExtra e;
   e.norm_w = norm_w;
   e.norm_eps = norm_eps;
+  e.ada_scale = ada_scale;
+  e.ada_shift = ada_shift;
   int rc = gemm_common(x, ldx, wgu_packed, (const float*)sg, (const float*)su, hbuf, I, nullptr, 0, 0, nullptr, M, I, K, 0,
                        act, ws, ws_bytes, (hipStream_t)stream, e);
   if (rc) return rc;

@@ -28,6 +28,9 @@ struct GemmArgs {
   // RMSNorm prologue (norm_w != nullptr): bf16 [K] weight, eps
   const unsigned short* norm_w;
   float norm_eps;
+  // adaptive RMSNorm prologue (ada_scale != nullptr): fp32 [K] scale and shift, same eps
+  const float* ada_scale;
+  const float* ada_shift;
   // rotary epilogue (rope_pos != nullptr): int32 [M] positions, fp32 [positions, rope_half] tables,
   // columns < rope_cols are rotated in pairs (c, c + rope_half)
   const int* rope_pos;
@@ -36,6 +39,7 @@ struct GemmArgs {
   int rope_positions;  // rows of the tables (positions are clamped into them)
   int rope_cols;
   int rope_half;
+  int rope_bf16;  // rotate in bf16 arithmetic (tables hold bf16 values)
   // rotary epilogue only: columns >= vt_col0 are also written transposed, vt[(n - vt_col0) * vt_ld + m]
   unsigned short* vt;
   int vt_col0;

@@ -39,16 +39,16 @@ SIGNATURES: dict[str, tuple] = {
     ),  # fmt: skip
     "tk_fp8w_norm_gated_ffn": (
         c_int,
-        [c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-         c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
+        [c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
     "tk_bf16w_packed_bytes": (c_size_t, [c_int, c_int]),
     "tk_pack_bf16_weight": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tk_bf16w_linear": (
         c_int,
-        [c_void_p, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-         c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p,
-         c_size_t, c_void_p],
+        [c_void_p, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+         c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
+         c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
     "tk_attn_prepare_kv": (
         c_int,

@@ -200,11 +200,13 @@ def fp8w_gated_ffn(
     gate: torch.Tensor | None = None,
     norm_w: torch.Tensor | None = None,
     eps: float = 0.0,
+    ada: tuple[torch.Tensor, torch.Tensor] | None = None,
     out: torch.Tensor | None = None,
     ws: Workspace | None = None,
 ) -> torch.Tensor:
     """``down(act(gate(x)) * up(x))`` (``* gate[n]``, ``+ residual``) for ``x [M, K]`` bf16;
-    with ``norm_w`` the input is first RMS-normalised inside the gate/up launch."""
+    with ``norm_w`` (RMSNorm) or ``ada = (scale, shift)`` (adaptive RMSNorm) the input is first
+    normalised inside the gate/up launch."""
     lib = native.lib()
     m, ldx = _check_act(x, wgu.k)
     if wd.k != wgu.i or wd.n != wgu.k:
@@ -213,9 +215,9 @@ def fp8w_gated_ffn(
         out = torch.empty(m, wd.n, dtype=torch.bfloat16, device=x.device)
     rp, ldr, rdt = _resid_args(resid, m, wd.n)
     ws = ws or default_workspace(x.device)
-    if norm_w is not None:
+    if norm_w is not None or ada is not None:
         rc = lib.tk_fp8w_norm_gated_ffn(
-            x.data_ptr(), ldx, _norm_ptr(norm_w, wgu.k), float(eps), wgu.data.data_ptr(), wgu.scale_gate.data_ptr(),
+            x.data_ptr(), ldx, _norm_ptr(norm_w, wgu.k), float(eps), *_ada_ptrs(ada, wgu.k), wgu.data.data_ptr(), wgu.scale_gate.data_ptr(),
             wgu.scale_up.data_ptr(), wd.data.data_ptr(), wd.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt,
             _gate_ptr(gate, wd.n), m, wgu.k, wgu.i, ACT[act], ws.ptr, ws.nbytes, _stream(),
         )  # fmt: skip
@@ -250,18 +252,31 @@ def _norm_ptr(norm_w: torch.Tensor | None, k: int) -> int | None:
     return norm_w.data_ptr()
 
 
+def _ada_ptrs(ada, k: int) -> tuple[int | None, int | None]:
+    if ada is None:
+        return None, None
+    scale, shift = ada
+    for t in (scale, shift):
+        if t.dtype != torch.float32 or t.numel() != k or t.stride(-1) != 1:
+            raise ValueError(f"adaptive-norm scale / shift must be fp32 vectors of {k} contiguous elements")
+    return scale.data_ptr(), shift.data_ptr()
+
+
 def bf16w_linear(
     x: torch.Tensor,
     w: PackedBf16Weight,
     *,
     norm_w: torch.Tensor | None = None,
     eps: float = 0.0,
+    ada: tuple[torch.Tensor, torch.Tensor] | None = None,
     rope: RopeTables | None = None,
     rope_pos: torch.Tensor | None = None,
     rope_cols: int = 0,
+    rope_bf16: bool = False,
     vt_out: torch.Tensor | None = None,
     vt_col0: int = 0,
     resid: torch.Tensor | None = None,
+    gate: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
     split_k: int = 0,
     ws: Workspace | None = None,
@@ -269,7 +284,9 @@ def bf16w_linear(
     """``x [M, K] @ W^T`` with bf16 weights; optional RMSNorm prologue (``x`` bf16 or fp32), and
     either a rotary epilogue (``rope`` tables, int32 ``rope_pos [M]``, columns ``< rope_cols``
     rotated; with ``vt_out [N - vt_col0, >= M]`` the columns from ``vt_col0`` on are also written
-    transposed) or a residual epilogue."""
+    transposed) or a (gated) residual epilogue.  ``ada = (scale, shift)``, fp32 ``[K]`` each,
+    selects the adaptive RMSNorm prologue instead of ``norm_w``; ``rope_bf16`` the bf16-arithmetic
+    rotation."""
     lib = native.lib()
     if not x.is_cuda or x.dim() != 2 or x.shape[1] != w.k or x.stride(1) != 1:
         raise ValueError(f"activations must be CUDA [M, {w.k}] with unit inner stride")
@@ -305,9 +322,9 @@ def bf16w_linear(
         vt_p, vt_ld = vt_out.data_ptr(), vt_out.stride(0)
     ws = ws or default_workspace(x.device)
     rc = lib.tk_bf16w_linear(
-        x.data_ptr(), x.stride(0), xdt, w.data.data_ptr(), _norm_ptr(norm_w, w.k), float(eps), pos_p, cos_p, sin_p,
-        positions, rope_cols, half, vt_p, vt_col0, vt_ld, out.data_ptr(), out.stride(0), rp, ldr, rdt, m, w.n, w.k,
-        split_k, ws.ptr, ws.nbytes, _stream(),
+        x.data_ptr(), x.stride(0), xdt, w.data.data_ptr(), _norm_ptr(norm_w, w.k), float(eps), *_ada_ptrs(ada, w.k),
+        pos_p, cos_p, sin_p, positions, rope_cols, half, int(rope_bf16), vt_p, vt_col0, vt_ld, out.data_ptr(),
+        out.stride(0), rp, ldr, rdt, _gate_ptr(gate, w.n), m, w.n, w.k, split_k, ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip
     native.check(rc, "tk_bf16w_linear")
     return out

@@ -100,6 +100,18 @@ class PI05Model:
         freqs = torch.arange(_ROPE_POSITIONS, dtype=torch.float32)[:, None] * inv[None, :]
         emb = torch.cat([freqs, freqs], dim=-1)
         self.rope_cos, self.rope_sin = emb.cos().to(self.device), emb.sin().to(self.device)
+        if self.fused_expert:
+            # the fused rotary epilogue reads fp32 tables holding the bf16 values the eager path uses
+            half = self.head_dim // 2
+            self.rope_tables_hip = tk.RopeTables(
+                self.rope_cos[:, :half].to(BF16).float().contiguous(), self.rope_sin[:, :half].to(BF16).float().contiguous()
+            )
+            self.exp_qkv, self.exp_o = [], []
+            for i in range(self.ed["depth"]):
+                lp = f"{EXP}layers.{i}.self_attn."
+                w = torch.cat([self.p[lp + n + "_proj.weight"] for n in "qkv"], dim=0).to(BF16)
+                self.exp_qkv.append(tk.pack_bf16_weight(w, rope_half=half))
+                self.exp_o.append(tk.pack_bf16_weight(self.p[lp + "o_proj.weight"].to(BF16)))
         self.embed_scale = torch.tensor(self.vd["width"] ** 0.5, dtype=BF16, device=self.device)
         self.patch_w = self.p[VIS + "embeddings.patch_embedding.weight"].reshape(cfg.vision_hidden, -1)
         self.set_num_steps(cfg.num_steps)
@@ -125,6 +137,14 @@ class PI05Model:
                     ]
                 )
                 self.final_mods.append(self.lin(EXP + "norm.dense", cond))
+            # (scale, shift, gate) of every modulation as separate contiguous vectors for the fused launches
+            w = self.ed["width"]
+
+            def split(mod: torch.Tensor):
+                m = mod.reshape(-1).float()
+                return m[:w].contiguous(), m[w : 2 * w].contiguous(), m[2 * w :].to(BF16).contiguous()
+
+            self.mods_split = [[(split(a), split(b)) for a, b in step] for step in self.mods]
 
     def rope_tables(self, pos: torch.Tensor, dtype) -> tuple[torch.Tensor, torch.Tensor]:
         return self.rope_cos[pos].to(dtype), self.rope_sin[pos].to(dtype)
@@ -198,6 +218,28 @@ class PI05Model:
         """Per-layer prefix K/V in the attention kernel's layout (V transposed), once per request."""
         return [tk.prepare_prefix_kv(k[0].transpose(0, 1), v[0].transpose(0, 1)) for k, v in kv]
 
+    def _denoise_layers_fused(self, prefix_pad, caches, hidden, pos, step: int) -> torch.Tensor:
+        """Expert stack on the fused launches (per layer: AdaRMS + q|k|v + RoPE, attention, o_proj with
+        gated residual, AdaRMS + GeGLU FFN with gated residual); ``hidden [S, W]`` bf16."""
+        heads, d = self.ed["num_heads"], self.head_dim
+        g = self.vt_suf.shape[0]
+        nq, nkv = heads * d, g * d
+        s = hidden.shape[0]
+        pos32 = pos[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
+        pad = prefix_pad[0]
+        for i in range(self.ed["depth"]):
+            (sc_in, sh_in, gate_in), (sc_post, sh_post, gate_post) = self.mods_split[step][i]
+            qkv = tk.bf16w_linear(
+                hidden, self.exp_qkv[i], ada=(sc_in, sh_in), eps=EPS, rope=self.rope_tables_hip, rope_pos=pos32,
+                rope_cols=nq + nkv, rope_bf16=True, vt_out=self.vt_suf.view(nkv, -1), vt_col0=nq + nkv, ws=self.ws,
+            )  # fmt: skip
+            suffix = tk.SuffixKV(qkv[:, nq : nq + nkv].view(s, g, d), self.vt_suf)
+            att = tk.expert_attn(qkv[:, :nq].view(s, heads, d), caches[i], suffix, pad, tk.MASK_BIDIR, logits_bf16=True, ws=self.ws)
+            hidden = tk.bf16w_linear(att, self.exp_o[i], resid=hidden, gate=gate_in, ws=self.ws)
+            mlp = self.exp_mlp[i]
+            hidden = tk.fp8w_gated_ffn(hidden, mlp.wgu, mlp.wd, "gelu_tanh", resid=hidden, gate=gate_post, ada=(sc_post, sh_post), eps=EPS, ws=self.ws)
+        return hidden
+
     def denoise_step(self, prefix_pad, kv, x_t, step: int, caches: list | None = None) -> torch.Tensor:
         """Velocity fp32 ``[1, chunk, max_action_dim]`` at denoising step ``step`` (flow_matching.py:505-556)."""
         hidden = self.lin("action_in_proj", x_t).to(BF16)
@@ -210,6 +252,10 @@ class PI05Model:
                 self.vt_suf = torch.zeros(g, self.head_dim, (s + 31) // 32 * 32, dtype=BF16, device=self.device)
         p_len = prefix_pad.shape[1]
         pos = prefix_pad.sum(dim=-1)[:, None] + torch.arange(s, device=self.device)[None, :]
+        if self.fused_expert and b == 1 and all(m.fp8 for m in self.exp_mlp):
+            hidden = self._denoise_layers_fused(prefix_pad, caches, hidden[0], pos, step)[None]
+            out, _ = gemma_norm(hidden, modulation=self.final_mods[step])
+            return self.lin("action_out_proj", out.to(torch.float32))
         cos, sin = self.rope_tables(pos, hidden.dtype)
         scaling = self.head_dim**-0.5
         if not self.fused_expert:
