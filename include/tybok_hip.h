@@ -230,6 +230,20 @@ int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const voi
                     const void* vt, long long vt_sb, int vt_sd, int vt_sh, void* out, long long out_sb, int out_sm, int B,
                     int M, int P, int H, int G, int D, int logits_bf16, void* ws, size_t ws_bytes, void* stream);
 
+/* ---- tail of a denoising step ---------------------------------------------------------------- */
+/* Final norm of the expert hidden state + fp32 action projection + Euler update in one launch:
+ *   h = norm(x) (bf16 row; norm_w: Llama RMSNorm bf16(w * bf16(x * rstd)); or ada_scale / ada_shift:
+ *   adaptive RMSNorm bf16((x * rstd) * (1 + scale) + shift)),  v = float(h) . W^T + bias (fp32),
+ *   x_out = x_t + dt * v.
+ * Replaces the tail of `denoise_step` and the `x_t + dt * v_t` of the Euler loop
+ * (tybok/policies/smolvla/models/flow_matching.py:343-350,612-620,
+ *  tybok/policies/pi05/models/flow_matching.py:547-556,228-240).
+ *   x: bf16 [M, K] (row pitch ldx); w: fp32 [N, K]; bias: fp32 [N] or NULL; N must divide 256.
+ *   v_out: fp32 [M, N] or NULL; x_t / x_out: fp32 [M, N] or both NULL (x_out may alias x_t). */
+int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps,
+                   const void* w, const void* bias, void* v_out, const void* x_t, void* x_out, float dt, int M, int N,
+                   int K, void* stream);
+
 /* ---- diagnostics ------------------------------------------------------------------------------- */
 /* out_f32[256] = value of every e4m3fn code as decoded by the device's conversion instruction
  * (the weight path of the GEMM); used to assert the OCP (not FNUZ) flavour on the box. */

@@ -211,3 +211,30 @@ def test_fused_layer_argument_checks(tk):
     rope = _tables(tk, 16, 32)
     with pytest.raises(RuntimeError):
         tk.bf16w_linear(x, pw_rope, rope=rope, rope_pos=torch.zeros(4, dtype=torch.int32, device="cuda"), rope_cols=32)
+
+
+@pytest.mark.parametrize("adaptive", [False, True])
+def test_step_tail_norm_projection_euler(tk, adaptive):
+    m, k, n = 50, 720 if not adaptive else 1024, 32
+    g = torch.Generator().manual_seed(20)
+    x = (torch.randn(m, k, generator=g) * 2.0).to(BF16)
+    w = torch.randn(n, k, generator=g) * k**-0.5
+    b = torch.randn(n, generator=g)
+    x_t = torch.randn(m, n, generator=g)
+    dt = -0.1
+    if adaptive:
+        mod = 0.3 * torch.randn(1, 3 * k, generator=g)
+        h, _ = oops.gemma_rms_norm(x[None], 1e-6, modulation=mod)
+        h = h[0]
+        kw = dict(ada=(mod[0, :k].contiguous().cuda(), mod[0, k : 2 * k].contiguous().cuda()), eps=1e-6)
+    else:
+        norm_w = (1.0 + 0.2 * torch.randn(k, generator=g)).to(BF16)
+        h = oops.rms_norm_llama(x, norm_w, 1e-5)
+        kw = dict(norm_w=norm_w.cuda(), eps=1e-5)
+    v_want = F.linear(h.float(), w, b)
+    x_want = x_t + dt * v_want
+    v, x_new = tk.expert_tail(x.cuda(), w.cuda(), b.cuda(), x_t=x_t.cuda(), dt=dt, want_v=True, **kw)
+    assert float((v.cpu() - v_want).abs().max()) < 2e-3, "velocity differs from norm + fp32 linear"
+    assert float((x_new.cpu() - x_want).abs().max()) < 2e-4, "Euler update differs"
+    v_only, none = tk.expert_tail(x.cuda(), w.cuda(), b.cuda(), **kw)
+    assert none is None and torch.equal(v_only, v)

@@ -311,27 +311,34 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
     if (s < a.kv_splits) lt += ls[s] * es[s];
   }
   const float inv = 1.0f / lt;
+  // several d tiles' partials in flight together: the read-back costs round trips, not bandwidth
+  constexpr int DTB = DT >= 4 ? 4 : DT;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) {
-    unsigned long long raw[MAXS][2];
+  for (int d0 = 0; d0 < DT; d0 += DTB) {
+    unsigned long long raw[DTB][MAXS][2];
 #pragma unroll
-    for (int s = 0; s < MAXS; ++s) {
-      const int sc = s < a.kv_splits ? s : a.kv_splits - 1;
-      const unsigned long long* src =
-          (const unsigned long long*)(pblk + (size_t)sc * PSTRIDE + 64) + (size_t)dt * 512 + ((size_t)wave * 64 + lane) * 2;
-      raw[s][0] = ld_agent64(src);
-      raw[s][1] = ld_agent64(src + 1);
-    }
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int dd = 0; dd < DTB; ++dd)
 #pragma unroll
-    for (int s = 0; s < MAXS; ++s) {
-      if (s < a.kv_splits) {
-        f32x4 v = {__uint_as_float((unsigned)raw[s][0]), __uint_as_float((unsigned)(raw[s][0] >> 32)),
-                   __uint_as_float((unsigned)raw[s][1]), __uint_as_float((unsigned)(raw[s][1] >> 32))};
-        acc += v * es[s];
+      for (int s = 0; s < MAXS; ++s) {
+        const int sc = s < a.kv_splits ? s : a.kv_splits - 1;
+        const unsigned long long* src = (const unsigned long long*)(pblk + (size_t)sc * PSTRIDE + 64) +
+                                        (size_t)(d0 + dd) * 512 + ((size_t)wave * 64 + lane) * 2;
+        raw[dd][s][0] = ld_agent64(src);
+        raw[dd][s][1] = ld_agent64(src + 1);
       }
+#pragma unroll
+    for (int dd = 0; dd < DTB; ++dd) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < MAXS; ++s) {
+        if (s < a.kv_splits) {
+          f32x4 v = {__uint_as_float((unsigned)raw[dd][s][0]), __uint_as_float((unsigned)(raw[dd][s][0] >> 32)),
+                     __uint_as_float((unsigned)raw[dd][s][1]), __uint_as_float((unsigned)(raw[dd][s][1] >> 32))};
+          acc += v * es[s];
+        }
+      }
+      if (q_ok) *(i32x2*)(op + (d0 + dd) * 32) = pack_bf16x4(acc * inv);
     }
-    if (q_ok) *(i32x2*)(op + dt * 32) = pack_bf16x4(acc * inv);
   }
 }
 

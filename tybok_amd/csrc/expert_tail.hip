@@ -1,0 +1,75 @@
+// Tail of a denoising step on gfx950: final (adaptive) RMSNorm of the expert hidden state, the fp32
+// action projection, and the Euler update, in one launch.
+//
+//   h[m, :]  = norm(x[m, :])                       bf16, the reference's rounding points
+//   v[m, n]  = sum_k float(h[m, k]) * W[n, k] + b[n]            fp32
+//   x_out[m, n] = x_t[m, n] + dt * v[m, n]                      fp32 (product and sum rounded separately)
+//
+// Tiny (50 rows x 32 outputs x 720..1024 inputs): one block per row, the normalised row lives in
+// LDS, each thread owns one (output, k-slice) pair and the slices are summed in a fixed order.
+#include "tk_common.h"
+#include "tk_kernels.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+__global__ __launch_bounds__(kThreads) void expert_tail_kernel(TailArgs a) {
+  extern __shared__ float hrow[];  // [K] normalised row, as fp32 values of bf16 numbers
+  __shared__ float red[kThreads / 64];
+  __shared__ float part[kThreads];
+  const int m = blockIdx.x;
+  const int tid = threadIdx.x;
+  const u16* x = a.x + (size_t)m * a.ldx;
+
+  float ss = 0.f;
+  for (int k = tid; k < a.K; k += kThreads) {
+    const float f = bf16_bits_to_f32(x[k]);
+    ss = fmaf(f, f, ss);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < kThreads / 64; ++w) tot += red[w];
+  const float rstd = rsqrtf(tot / (float)a.K + a.eps);
+
+  for (int k = tid; k < a.K; k += kThreads) {
+    const float f = bf16_bits_to_f32(x[k]);
+    float h;
+    if (a.ada_scale) {
+      // adaptive: bf16((x * rstd) * (1 + scale) + shift), fp32 steps rounded separately
+      h = round_bf16(__fadd_rn(__fmul_rn(__fmul_rn(f, rstd), __fadd_rn(1.0f, a.ada_scale[k])), a.ada_shift[k]));
+    } else {
+      // Llama RMSNorm on a bf16 row: bf16(w * bf16(x * rstd))
+      h = round_bf16(bf16_bits_to_f32(a.norm_w[k]) * round_bf16(f * rstd));
+    }
+    hrow[k] = h;
+  }
+  __syncthreads();
+
+  // thread -> (output n, k slice): slices of an output are consecutive threads
+  const int slices = kThreads / a.N;  // host guarantees N divides kThreads and N <= kThreads
+  const int n = tid / slices, sl = tid % slices;
+  const float* w = a.w + (size_t)n * a.K;
+  float acc = 0.f;
+  for (int k = sl; k < a.K; k += slices) acc = fmaf(hrow[k], w[k], acc);
+  part[tid] = acc;
+  __syncthreads();
+  if (sl == 0) {
+    float v = 0.f;
+    for (int j = 0; j < slices; ++j) v += part[tid + j];
+    if (a.bias) v += a.bias[n];
+    if (a.v_out) a.v_out[(size_t)m * a.N + n] = v;
+    if (a.x_out) a.x_out[(size_t)m * a.N + n] = __fadd_rn(a.x_t[(size_t)m * a.N + n], __fmul_rn(a.dt, v));
+  }
+}
+
+}  // namespace
+
+int tk_launch_tail(TailArgs a, hipStream_t st) {
+  hipLaunchKernelGGL(expert_tail_kernel, dim3(a.M), dim3(kThreads), (size_t)a.K * sizeof(float), st, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}

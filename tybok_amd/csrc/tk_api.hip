@@ -458,6 +458,36 @@ int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const voi
                    stream);
 }
 
+int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps,
+                   const void* w, const void* bias, void* v_out, const void* x_t, void* x_out, float dt, int M, int N, int K,
+                   void* stream) {
+  if (M <= 0 || N <= 0 || K <= 0 || ldx < K) return fail(TK_EINVAL, "tail: bad shape M=%d N=%d K=%d ldx=%d", M, N, K, ldx);
+  if (N > 256 || 256 % N) return fail(TK_EINVAL, "tail: N=%d must divide 256", N);
+  if (K > 16384) return fail(TK_EINVAL, "tail: K=%d too large for the row buffer", K);
+  if (!x || !w || (!norm_w && !(ada_scale && ada_shift)) || (norm_w && (ada_scale || ada_shift)))
+    return fail(TK_EINVAL, "tail: needs x, w and exactly one of norm_w or ada_scale + ada_shift");
+  if (x_out && !x_t) return fail(TK_EINVAL, "tail: x_out needs x_t");
+  if (!v_out && !x_out) return fail(TK_EINVAL, "tail: no output requested");
+  TailArgs a;
+  a.x = (const u16*)x;
+  a.ldx = ldx;
+  a.norm_w = (const u16*)norm_w;
+  a.ada_scale = (const float*)ada_scale;
+  a.ada_shift = (const float*)ada_shift;
+  a.eps = eps;
+  a.w = (const float*)w;
+  a.bias = (const float*)bias;
+  a.v_out = (float*)v_out;
+  a.x_t = (const float*)x_t;
+  a.x_out = (float*)x_out;
+  a.dt = dt;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  if (tk_launch_tail(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "tail: launch failed");
+  return TK_OK;
+}
+
 int tk_debug_decode_fp8(void* out_f32, void* stream) {
   if (!out_f32) return fail(TK_EINVAL, "decode: null pointer");
   if (tk_launch_decode_fp8((float*)out_f32, (hipStream_t)stream)) return fail(TK_ELAUNCH, "decode: launch failed");

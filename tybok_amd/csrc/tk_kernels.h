@@ -88,6 +88,23 @@ struct KvPrepArgs {
   int ld;
 };
 
+struct TailArgs {
+  const unsigned short* x;  // bf16 [M, K]
+  int ldx;
+  const unsigned short* norm_w;  // bf16 [K] (RMSNorm) or nullptr with ada_scale / ada_shift
+  const float* ada_scale;
+  const float* ada_shift;
+  float eps;
+  const float* w;     // fp32 [N, K]
+  const float* bias;  // fp32 [N] or nullptr
+  float* v_out;       // fp32 [M, N] or nullptr
+  const float* x_t;   // fp32 [M, N] (with x_out)
+  float* x_out;       // fp32 [M, N] or nullptr
+  float dt;
+  int M, N, K;
+};
+
+int tk_launch_tail(TailArgs a, hipStream_t st);
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st);
 int tk_launch_pack(const void* w0, const void* w1, void* out, int N, int K, int interleave, hipStream_t st);
 int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st);

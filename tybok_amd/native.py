@@ -55,6 +55,11 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
          c_void_p],
     ),  # fmt: skip
+    "tk_expert_tail": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+         c_int, c_int, c_int, c_void_p],
+    ),  # fmt: skip
     "tk_batched_attn": (
         c_int,
         [c_void_p, c_longlong, c_int, c_int, c_void_p, c_longlong, c_int, c_int, c_void_p, c_longlong, c_int, c_int,

@@ -522,6 +522,44 @@ def expert_attn_plain(
     return expert_attn(q, prefix, suffix, prefix_pad, mask_mode, **kw)
 
 
+def expert_tail(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    bias: torch.Tensor | None,
+    *,
+    norm_w: torch.Tensor | None = None,
+    ada: tuple[torch.Tensor, torch.Tensor] | None = None,
+    eps: float,
+    x_t: torch.Tensor | None = None,
+    dt: float = 0.0,
+    want_v: bool = False,
+) -> tuple[torch.Tensor | None, torch.Tensor | None]:
+    """Final norm of ``x [M, K]`` bf16, fp32 projection with ``w [N, K]`` (+ ``bias``), and -- with
+    ``x_t [M, N]`` -- the Euler update ``x_t + dt * v``.  Returns ``(v or None, x_new or None)``."""
+    lib = native.lib()
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or x.stride(1) != 1:
+        raise TypeError("x must be bf16 [M, K] with unit inner stride")
+    m, k = x.shape
+    if w.dtype != torch.float32 or w.shape[1] != k or not w.is_contiguous():
+        raise ValueError("w must be contiguous fp32 [N, K]")
+    n = w.shape[0]
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != n or not bias.is_contiguous()):
+        raise ValueError("bias must be contiguous fp32 [N]")
+    f32 = dict(dtype=torch.float32, device=x.device)
+    v = torch.empty(m, n, **f32) if (want_v or x_t is None) else None
+    x_new = None
+    if x_t is not None:
+        if x_t.dtype != torch.float32 or x_t.shape != (m, n) or not x_t.is_contiguous():
+            raise ValueError("x_t must be contiguous fp32 [M, N]")
+        x_new = torch.empty(m, n, **f32)
+    rc = lib.tk_expert_tail(
+        x.data_ptr(), x.stride(0), _norm_ptr(norm_w, k), *_ada_ptrs(ada, k), float(eps), w.data_ptr(), _ptr(bias), _ptr(v),
+        _ptr(x_t), _ptr(x_new), float(dt), m, n, k, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_expert_tail")
+    return v, x_new
+
+
 def decode_fp8_table(device: torch.device | str = "cuda") -> torch.Tensor:
     """Values of all 256 e4m3fn codes as the device's conversion instruction decodes them."""
     out = torch.empty(256, dtype=torch.float32, device=device)

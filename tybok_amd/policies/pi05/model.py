@@ -145,6 +145,7 @@ class PI05Model:
                 return m[:w].contiguous(), m[w : 2 * w].contiguous(), m[2 * w :].to(BF16).contiguous()
 
             self.mods_split = [[(split(a), split(b)) for a, b in step] for step in self.mods]
+            self.final_split = [split(m)[:2] for m in self.final_mods]
 
     def rope_tables(self, pos: torch.Tensor, dtype) -> tuple[torch.Tensor, torch.Tensor]:
         return self.rope_cos[pos].to(dtype), self.rope_sin[pos].to(dtype)
@@ -178,8 +179,12 @@ class PI05Model:
     def embed_prefix(self, images, img_masks, tokens, masks):
         """-> ``(embs fp32 [1,P,W], pad_masks [1,P])``; every prefix token attends to every valid one."""
         embs, pads = [], []
-        for img, m in zip(images, img_masks):
-            e = self.embed_image(img)
+        if len(images) > 1 and all(img.shape == images[0].shape for img in images):
+            # one pass of the vision tower over all cameras (rows are independent)
+            per_image = self.embed_image(torch.cat(list(images), dim=0)).split(images[0].shape[0], dim=0)
+        else:
+            per_image = [self.embed_image(img) for img in images]
+        for e, m in zip(per_image, img_masks):
             embs.append(e)
             pads.append(m[:, None].expand(e.shape[0], e.shape[1]))
         lang = F.embedding(tokens, self.p[VLM + "embed_tokens.weight"]) * self.embed_scale
@@ -253,9 +258,9 @@ class PI05Model:
         p_len = prefix_pad.shape[1]
         pos = prefix_pad.sum(dim=-1)[:, None] + torch.arange(s, device=self.device)[None, :]
         if self.fused_expert and b == 1 and all(m.fp8 for m in self.exp_mlp):
-            hidden = self._denoise_layers_fused(prefix_pad, caches, hidden[0], pos, step)[None]
-            out, _ = gemma_norm(hidden, modulation=self.final_mods[step])
-            return self.lin("action_out_proj", out.to(torch.float32))
+            hidden = self._denoise_layers_fused(prefix_pad, caches, hidden[0], pos, step)
+            v, _ = tk.expert_tail(hidden, self.p["action_out_proj.weight"], self.p["action_out_proj.bias"], ada=self.final_split[step], eps=EPS)
+            return v[None]
         cos, sin = self.rope_tables(pos, hidden.dtype)
         scaling = self.head_dim**-0.5
         if not self.fused_expert:

@@ -164,6 +164,17 @@ class SmolVLAModel:
             t = torch.tensor(1.0 + step * dt, dtype=torch.float32).expand(1)
             embs.append(sinusoidal_time_embedding(t, self.cfg.expert_hidden_size, self.cfg.min_period, self.cfg.max_period).float())
         self.time_embs = [e.to(self.device) for e in embs]
+        if getattr(self, "fused_expert", False):
+            # Suffix embedding with its constants folded (exact algebra, evaluated in float64):
+            #   mlp_in(cat[in_proj(x), te]) = (Wa Win) x + (Wa b_in + Wt te + b_mlp)
+            # so a step embeds the noisy actions with two small GEMMs and one SiLU.
+            f64 = lambda name: self.p[name].to(torch.float64)  # noqa: E731
+            w_in, b_in = f64("action_in_proj.weight"), f64("action_in_proj.bias")
+            w_mlp, b_mlp = f64("action_time_mlp_in.weight"), f64("action_time_mlp_in.bias")
+            e = w_in.shape[0]
+            w_a, w_t = w_mlp[:, :e], w_mlp[:, e:]
+            self.suffix_w = (w_a @ w_in).float().contiguous()
+            self.suffix_b = [(w_a @ b_in + w_t @ te[0].to(torch.float64) + b_mlp).float().contiguous() for te in self.time_embs]
 
     def _pack_attention_weights(self, stack: str, q_only) -> tuple[list, list]:
         """bf16 attention weights of a decoder stack in tile order: q|k|v concatenated (or q alone
@@ -399,6 +410,19 @@ class SmolVLAModel:
                 hidden = mlp(rms_norm(out, post_w, self.eps)[None], out[None])[0]
         return hidden
 
+    def fused_euler_step(self, prefix_pad, caches, x_t, step: int, positions, dt: float) -> torch.Tensor:
+        """One Euler step on the fused launches: folded suffix embedding, expert stack, then final
+        norm + action projection + ``x_t + dt * v_t`` in one launch.  ``x_t [1, chunk, A]`` fp32."""
+        pos32, pos0_32 = positions
+        h = F.silu(F.linear(x_t[0], self.suffix_w, self.suffix_b[step]))
+        hidden = F.linear(h, self.p["action_time_mlp_out.weight"], self.p["action_time_mlp_out.bias"])
+        hidden = self._denoise_step_fused(prefix_pad, caches, hidden, pos32, pos0_32)
+        _, x_new = tk.expert_tail(
+            hidden, self.p["action_out_proj.weight"], self.p["action_out_proj.bias"], norm_w=self.p[EXP + "norm.weight"],
+            eps=self.eps, x_t=x_t[0], dt=dt,
+        )  # fmt: skip
+        return x_new[None]
+
     def denoise_step(self, prefix_pad, keys, values, ekv, x_t, time_emb, positions=None, caches=None):
         """Velocity ``v_t`` fp32 ``[1, chunk, max_action_dim]`` (flow_matching.py:316-350)."""
         hidden = self.embed_suffix(x_t, time_emb)
@@ -447,7 +471,11 @@ class SmolVLAModel:
         if self.fused_expert and noise.shape[0] == 1:
             positions = tuple(t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32) for t in positions)
         caches = self.attention_caches(keys, values, ekv, vt) if self.fused_expert and noise.shape[0] == 1 else None
+        fused_loop = caches is not None and x_t.dtype == torch.float32 and x_t.is_contiguous()
         for step in range(self.num_steps):
+            if fused_loop:
+                x_t = self.fused_euler_step(pads, caches, x_t, step, positions, dt)
+                continue
             v_t = self.denoise_step(pads, keys, values, ekv, x_t, self.time_embs[step], positions, caches)
             x_t = x_t + dt * v_t
         return x_t
