@@ -75,6 +75,7 @@ def gemm_launch_us(m: int, k: int, n: int, launches: int = 100, reps: int = 10, 
     with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
         for i in range(launches):
             tk.fp8w_gemm(x, pws[i % copies], out=out)
+    spin_up(60.0)  # capture and allocation idle the GPU long enough for its clocks to drop
     for _ in range(3):
         graph.replay()
     torch.cuda.synchronize()
@@ -110,6 +111,7 @@ def attn_launch_us(launches: int = 100, reps: int = 10) -> float:
     with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
         for _ in range(launches):
             tk.expert_attn(q, prefix, suffix, None, tk.MASK_CAUSAL, out=out)
+    spin_up(60.0)  # capture and allocation idle the GPU long enough for its clocks to drop
     for _ in range(3):
         graph.replay()
     torch.cuda.synchronize()
