@@ -25,11 +25,27 @@
 #include "tk_common.h"
 #include "tk_kernels.h"
 
+#ifdef TK_PHASE_TIMING
+// development aid (never built into the shipped library): per-block phase timestamps
+__device__ long long tk_attn_stamps[8 * 8192];
+#define TA_MARK(i)                                                                   \
+  do {                                                                               \
+    if (threadIdx.x == 0) {                                                          \
+      const int b_ = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x; \
+      if (b_ < 8192) tk_attn_stamps[b_ * 8 + (i)] = wall_clock64();                  \
+    }                                                                                \
+  } while (0)
+extern "C" int tk_debug_read_attn_phases(void* host_out) {
+  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(tk_attn_stamps), sizeof(long long) * 8 * 8192);
+}
+#else
+#define TA_MARK(i)
+#endif
+
 namespace {
 
 constexpr float kF32Min = -3.4028234663852886e38f;    // finfo(float32).min
 constexpr float kOpenpiMask = -2.3819763e38f;         // additive mask of the pi0.5 path
-constexpr int kNW = 4;
 
 // K row held by MFMA row r of a key tile: swaps bits 2 and 3 of r (see the header comment)
 __device__ __forceinline__ int key_of_row(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
@@ -41,12 +57,16 @@ __device__ __forceinline__ bf16x8 pack_bf16x8(const float* v) {
   return r.b;
 }
 
-template <int D, bool SPLIT>
-__global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
+// NWV waves per block, one 32-key tile each per pass.  With few key tiles (the action expert:
+// 8-10) a block of 8 or 12 waves covers the whole key range, so the waves merge through LDS only and
+// the global partial hand-off between kv splits (two more round trips) is not needed.
+template <int D, bool SPLIT, int NWV>
+__global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
+  constexpr int kNW = NWV;
   constexpr int DT = D / 32;                 // d tiles of the output
   constexpr int DS = D / 16;                 // k steps of Q.K^T
   constexpr int PL = SPLIT ? 2 : 1;          // operand planes (hi, lo)
-  constexpr int PF = D <= 128 ? 2 : 1;       // key tiles in flight per wave
+  constexpr int PF = (NWV > 4 || D > 128) ? 1 : 2;  // key tiles in flight per wave
   __shared__ __align__(16) f32x4 red[2][kNW][4][64];
   __shared__ float st_m[kNW][32], st_l[kNW][32];
 
@@ -64,6 +84,7 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
   a.vt_pre += bi * a.vt_sb;
   a.out += bi * a.out_sb;
   const int g = h / (a.H / a.G);
+  TA_MARK(0);
   const int tp = (a.P + 31) >> 5;            // prefix tiles; suffix tiles follow
   const int ntiles = tp + ((a.S + 31) >> 5);
   const int t_lo = (split * ntiles) / a.kv_splits;
@@ -122,6 +143,7 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
   for (int p = 0; p < PF; ++p)
     if (t_lo + wave + kNW * p < t_hi) load(stg[p], t_lo + wave + kNW * p);
 
+  TA_MARK(1);
   f32x16 o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
@@ -217,11 +239,16 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
     }
   }
 
+  TA_MARK(2);
   // ---- merge the four waves in fixed order (LDS) ----
   if (half == 0) {
     st_m[wave][l32] = m_run;
     st_l[wave][l32] = l_run;
   }
+  // waves 0..3 own the four register groups (output rows 8w + 4*(lane/32) + 0..3 of every d tile);
+  // further waves only contribute their tiles
+  const bool owner = wave < 4;
+  const int wg = wave & 3;
   f32x4 own[DT];
   float ew[kNW];
   float bm = -INFINITY, bl = 0.f;  // block-level (m, l) of this lane's query
@@ -246,16 +273,20 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
         bl += st_l[w][l32] * ew[w];
       }
     }
-    f32x4 sum = red[dt & 1][0][wave][lane] * ew[0];
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    if (owner) {
+      sum = red[dt & 1][0][wg][lane] * ew[0];
 #pragma unroll
-    for (int w = 1; w < kNW; ++w) sum += red[dt & 1][w][wave][lane] * ew[w];
+      for (int w = 1; w < kNW; ++w) sum += red[dt & 1][w][wg][lane] * ew[w];
+    }
     own[dt] = sum;
   }
 
+  TA_MARK(3);
   // this lane's output: query qi, columns d0 .. d0+3 of every d tile
-  u16* op = a.out + (size_t)(q_ok ? qi : 0) * a.out_sm + (size_t)h * D + 8 * wave + 4 * half;
+  u16* op = a.out + (size_t)(q_ok ? qi : 0) * a.out_sm + (size_t)h * D + 8 * wg + 4 * half;
   if (a.kv_splits == 1) {
-    if (q_ok) {
+    if (q_ok && owner) {
       const float inv = 1.0f / bl;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) *(i32x2*)(op + dt * 32) = pack_bf16x4(own[dt] * inv);
@@ -272,7 +303,7 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
     st_agent(pmine + l32, bm);
     st_agent(pmine + 32 + l32, bl);
   }
-  {
+  if (owner) {
     unsigned long long* dst = (unsigned long long*)(pmine + 64) + ((size_t)wave * 64 + lane) * 2;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
@@ -288,7 +319,8 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
     s_last = (old == a.kv_splits - 1);
   }
   __syncthreads();
-  if (!s_last) return;
+  TA_MARK(4);
+  if (!s_last || !owner) return;
   if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
   constexpr int MAXS = 8;  // the host never asks for more kv splits
@@ -310,6 +342,7 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
     es[s] = (s < a.kv_splits && ms[s] != -INFINITY) ? __expf(ms[s] - mt) : 0.f;
     if (s < a.kv_splits) lt += ls[s] * es[s];
   }
+  TA_MARK(5);
   const float inv = 1.0f / lt;
   // several d tiles' partials in flight together: the read-back costs round trips, not bandwidth
   constexpr int DTB = DT >= 4 ? 4 : DT;
@@ -340,6 +373,7 @@ __global__ __launch_bounds__(kNW * 64) void expert_attn_kernel(AttnArgs a) {
       if (q_ok) *(i32x2*)(op + (d0 + dd) * 32) = pack_bf16x4(acc * inv);
     }
   }
+  TA_MARK(6);
 }
 
 // Lays a [L, G, D] K/V pair out for the attention kernel: V transposed to [G, D, ld] (keys
@@ -387,24 +421,36 @@ __global__ void kv_prepare_kernel(KvPrepArgs p) {
   }
 }
 
-template <int D, bool SPLIT>
+template <int D, bool SPLIT, int NWV>
 int launch_attn(const AttnArgs& a, hipStream_t st) {
   dim3 grid(a.H, ((a.M + 31) / 32) * (a.batch > 0 ? a.batch : 1), a.kv_splits);
-  hipLaunchKernelGGL((expert_attn_kernel<D, SPLIT>), grid, dim3(kNW * 64), 0, st, a);
+  hipLaunchKernelGGL((expert_attn_kernel<D, SPLIT, NWV>), grid, dim3(NWV * 64), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
 }  // namespace
 
-int tk_launch_attn(AttnArgs a, int D, hipStream_t st) {
+int tk_attn_waves(int D, int split_planes, int ntiles) {
+  // a block of 8 or 12 waves when that covers every key tile (D = 64 only: register budget)
+  if (D != 64) return 4;
+  if (ntiles <= 8 && ntiles > 4) return 8;
+  if (!split_planes && ntiles <= 12 && ntiles > 8) return 12;
+  return 4;
+}
+
+int tk_launch_attn(AttnArgs a, int D, int waves, hipStream_t st) {
   const bool split = a.k_pre_lo != nullptr;
   if (split) {
-    if (D == 64) return launch_attn<64, true>(a, st);
-    return -1;
+    if (D != 64) return -1;
+    return waves == 8 ? launch_attn<64, true, 8>(a, st) : launch_attn<64, true, 4>(a, st);
   }
-  if (D == 64) return launch_attn<64, false>(a, st);
-  if (D == 128) return launch_attn<128, false>(a, st);
-  if (D == 256) return launch_attn<256, false>(a, st);
+  if (D == 64) {
+    if (waves == 12) return launch_attn<64, false, 12>(a, st);
+    if (waves == 8) return launch_attn<64, false, 8>(a, st);
+    return launch_attn<64, false, 4>(a, st);
+  }
+  if (D == 128) return launch_attn<128, false, 4>(a, st);
+  if (D == 256) return launch_attn<256, false, 4>(a, st);
   return -1;
 }
 

@@ -417,7 +417,8 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   const int mtiles = ((M + 31) / 32) * (batch > 0 ? batch : 1);
   // one 32-key tile per wave: split the keys over blocks of four waves (at most 8 splits, beyond
   // that a wave loops over several tiles)
-  int splits = (ntiles + 3) / 4;
+  const int waves = tk_attn_waves(D, split ? 1 : 0, ntiles);
+  int splits = (ntiles + waves - 1) / waves;
   if (splits < 1) splits = 1;
   if (splits > 8) splits = 8;
   // many query tiles already fill the device: keep whole key ranges in one block (no partials)
@@ -433,7 +434,7 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
     a.partial = (float*)((char*)ws + kPartialOff);
     a.counters = (int*)ws;
   }
-  int rc = tk_launch_attn(a, D, (hipStream_t)stream);
+  int rc = tk_launch_attn(a, D, waves, (hipStream_t)stream);
   if (rc) return fail(TK_ELAUNCH, "attn: launch failed (%s)", hipGetErrorString(hipGetLastError()));
   return TK_OK;
 }

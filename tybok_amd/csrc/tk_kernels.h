@@ -110,5 +110,6 @@ int tk_launch_pack(const void* w0, const void* w1, void* out, int N, int K, int 
 int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st);
 int tk_launch_fill_zero(int* p, int n, hipStream_t st);
 int tk_launch_decode_fp8(float* out, hipStream_t st);
-int tk_launch_attn(AttnArgs a, int D, hipStream_t st);
+int tk_attn_waves(int D, int split_planes, int ntiles);
+int tk_launch_attn(AttnArgs a, int D, int waves, hipStream_t st);
 int tk_launch_kv_prepare(KvPrepArgs p, hipStream_t st);
