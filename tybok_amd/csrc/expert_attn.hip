@@ -71,14 +71,25 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   __shared__ float st_m[kNW][32], st_l[kNW][32];
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keeps tile indices scalar
   const int half = lane >> 5;
   const int l32 = lane & 31;
-  const int h = blockIdx.x;
   const int mtiles = (a.M + 31) >> 5;
-  const int bi = blockIdx.y / mtiles;        // problem of a batched launch
-  const int mtile = blockIdx.y % mtiles;
+  int h = blockIdx.x;
+  int bi = blockIdx.y / mtiles;              // problem of a batched launch
+  int mtile = blockIdx.y % mtiles;
   const int split = blockIdx.z;
+  if (a.xcd_remap) {
+    // Large batched launches (vision tower): a 1-D grid whose workgroups the dispatcher deals
+    // round-robin to the 8 XCDs.  All query tiles of one (problem, head) pair are given to the same
+    // XCD, so that pair's K / V^T (re-read by every query tile) stays in that XCD's L2.
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int pair = (slot / mtiles) * 8 + xcd;
+    if (pair >= a.batch * a.H) return;
+    mtile = slot % mtiles;
+    bi = pair / a.H;
+    h = pair % a.H;
+  }
   a.q += bi * a.q_sb;
   a.k_pre += bi * a.k_sb;
   a.vt_pre += bi * a.vt_sb;
@@ -119,16 +130,17 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
 #pragma unroll
         for (int s = 0; s < 2; ++s) st.v[pl][dt][s] = *(const i32x4*)(vb + voff + (size_t)dt * 32 * vsd + 16 * s);
     }
-    st.pad = 1;
-    if (pre && a.mask2d) {
-      // eight consecutive keys per byte run: registers 8s..8s+7 of this lane
-      const uint8_t* mp = a.mask2d + (size_t)(q_ok ? qi : a.M - 1) * a.mask_ld + tt * 32 + 8 * half;
-      st.m2[0] = *(const unsigned long long*)mp;
-      st.m2[1] = *(const unsigned long long*)(mp + 16);
-    } else if (pre && a.pad) {
-      const int key = tt * 32 + l32;
-      st.pad = key < a.P ? a.pad[key] : 0;
-    }
+    // visibility operands, always requested (from a harmless valid address when unused): a branch
+    // around a load would make the compiler wait for every outstanding load before each tile
+    const bool use_m2 = pre && a.mask2d != nullptr;
+    const bool use_pad = pre && a.mask2d == nullptr && a.pad != nullptr;
+    const int key = tt * 32 + l32;
+    const uint8_t* mp = use_m2 ? a.mask2d + (size_t)(q_ok ? qi : a.M - 1) * a.mask_ld + tt * 32 + 8 * half : (const uint8_t*)a.q;
+    st.m2[0] = *(const unsigned long long*)mp;  // eight consecutive keys: registers 8s..8s+7 of this lane
+    st.m2[1] = *(const unsigned long long*)(mp + (use_m2 ? 16 : 8));
+    const uint8_t* pp = (use_pad && key < a.P) ? a.pad + key : (const uint8_t*)a.q;
+    const int padv = *pp;
+    st.pad = use_pad ? (key < a.P ? padv : 0) : 1;
   };
 
   // ---- Q as B operand, resident in registers; the first tiles' loads go out with it ----
@@ -139,11 +151,16 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
 #pragma unroll
     for (int s = 0; s < DS; ++s) qf[s] = as_bf16x8(*(const i32x4*)(qp + 16 * s));
   }
+  // tiles of this wave: t_lo + wave + kNW * i, i < nt_w; indices past the end are clamped to a valid
+  // tile so that every prefetch is unconditional (never processed)
+  const int nt_w = t_hi - t_lo > wave ? (t_hi - t_lo - wave + kNW - 1) / kNW : 0;
+  auto tile_of = [&](int i) {
+    const int t = t_lo + wave + kNW * i;
+    return t < t_hi ? t : (t_hi > 0 ? t_hi - 1 : 0);
+  };
 #pragma unroll
-  for (int p = 0; p < PF; ++p)
-    if (t_lo + wave + kNW * p < t_hi) load(stg[p], t_lo + wave + kNW * p);
+  for (int p = 0; p < PF; ++p) load(stg[p], tile_of(p));
 
-  TA_MARK(1);
   f32x16 o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
@@ -165,24 +182,47 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
       for (int pl = 0; pl < PL; ++pl) sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(st.k[pl][s]), qf[s], sT, 0, 0, 0);
 
     // ---- scale, mask, online softmax (one query column per lane) ----
-    const unsigned pmask = (unsigned)__ballot(st.pad != 0);  // lanes 0..31: keys of this tile
+    // Register i of this lane holds key kl(i) = 16*(i/8) + 8*half + i%8 of the tile.  Visibility and
+    // range are first reduced to two 16-bit masks (bit i = register i) with wave-uniform branches, so
+    // the per-element code below is straight-line selects.
+    unsigned vbits, ibits;
+    {
+      const int k0 = tt * 32 + 8 * half;  // key of register 0; registers 8..15 are 16 keys further
+      const int left = len - k0;          // keys from k0 on that exist
+      const unsigned lo8 = left >= 8 ? 0xffu : (left > 0 ? (1u << left) - 1u : 0u);
+      const unsigned hi8 = left >= 24 ? 0xffu : (left > 16 ? (1u << (left - 16)) - 1u : 0u);
+      ibits = lo8 | (hi8 << 8);
+      if (!pre) {
+        if (a.mask_mode == 1) {
+          vbits = 0xffffu;
+        } else {  // causal among the suffix tokens: key <= query
+          const int c = qi - k0 + 1;  // visible keys from k0 on
+          const unsigned cl = c >= 8 ? 0xffu : (c > 0 ? (1u << c) - 1u : 0u);
+          const unsigned ch = c >= 24 ? 0xffu : (c > 16 ? (1u << (c - 16)) - 1u : 0u);
+          vbits = cl | (ch << 8);
+        }
+      } else if (a.mask2d) {
+        // one byte (0 or 1) per key: gather bit 0 of the 8 bytes of each word
+        const unsigned long long gather = 0x0102040810204080ull, ones = 0x0101010101010101ull;
+        vbits = (unsigned)(((st.m2[0] & ones) * gather) >> 56) | ((unsigned)(((st.m2[1] & ones) * gather) >> 56) << 8);
+      } else {
+        const unsigned pmask = (unsigned)__ballot(st.pad != 0);  // lanes 0..31: keys of this tile
+        vbits = ((pmask >> (8 * half)) & 0xffu) | (((pmask >> (16 + 8 * half)) & 0xffu) << 8);
+      }
+    }
+    const bool lb = a.logits_bf16 != 0;
     float p[16];
     float tmax = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int kl = 16 * (i >> 3) + 8 * half + (i & 7);  // key within the tile held by register i
-      const int key = tt * 32 + kl;
-      float s = sT[i];
-      if (a.logits_bf16) s = round_bf16(s);
-      s *= a.scale;
-      bool vis;
-      if (!pre) vis = a.mask_mode == 1 || key <= qi;
-      else if (a.mask2d) vis = ((st.m2[i >> 3] >> (8 * (i & 7))) & 0xffull) != 0;
-      else vis = ((pmask >> kl) & 1u) != 0;
-      if (!vis) s = a.logits_bf16 ? (s + kOpenpiMask) : kF32Min;
-      if (key >= len) s = -INFINITY;
-      p[i] = s;
-      tmax = fmaxf(tmax, s);
+      float sv = sT[i];
+      sv = lb ? round_bf16(sv) : sv;
+      sv *= a.scale;
+      const float masked = lb ? sv + kOpenpiMask : kF32Min;
+      sv = (vbits >> i) & 1u ? sv : masked;
+      sv = (ibits >> i) & 1u ? sv : -INFINITY;
+      p[i] = sv;
+      tmax = fmaxf(tmax, sv);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
     const float m_new = fmaxf(m_run, tmax);
@@ -196,12 +236,10 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
     lsum += __shfl_xor(lsum, 32);
     l_run = l_run * alpha + lsum;
     m_run = m_new;
-    if (alpha != 1.0f) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
-    }
+      for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
 
     // P^T as B operand: step s uses registers 8s..8s+7 = keys 16s + 8*half + 0..7
     bf16x8 pb[2], pbl[2];
@@ -228,13 +266,22 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
       }
   };
 
-  for (int t = t_lo + wave; t < t_hi; t += kNW * PF) {
+  {
+    // software pipeline over this wave's tiles: the steady-state loop has no branch (precise
+    // wait counts), the tail (< 2*PF tiles) uses wave-uniform conditions
+    int i = 0;
+    for (; i + 2 * PF <= nt_w; i += PF) {
 #pragma unroll
-    for (int p = 0; p < PF; ++p) {
-      const int tc = t + kNW * p;
-      if (tc < t_hi) {  // wave-uniform
-        process(stg[p], tc);
-        if (tc + kNW * PF < t_hi) load(stg[p], tc + kNW * PF);
+      for (int p = 0; p < PF; ++p) {
+        process(stg[p], tile_of(i + p));
+        load(stg[p], tile_of(i + p + PF));
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 2 * PF - 1; ++q) {
+      if (i + q < nt_w) {
+        process(stg[q % PF], tile_of(i + q));
+        if (i + q + PF < nt_w) load(stg[q % PF], tile_of(i + q + PF));
       }
     }
   }
@@ -424,6 +471,7 @@ __global__ void kv_prepare_kernel(KvPrepArgs p) {
 template <int D, bool SPLIT, int NWV>
 int launch_attn(const AttnArgs& a, hipStream_t st) {
   dim3 grid(a.H, ((a.M + 31) / 32) * (a.batch > 0 ? a.batch : 1), a.kv_splits);
+  if (a.xcd_remap) grid = dim3(8 * ((a.batch * a.H + 7) / 8) * ((a.M + 31) / 32), 1, 1);
   hipLaunchKernelGGL((expert_attn_kernel<D, SPLIT, NWV>), grid, dim3(NWV * 64), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }

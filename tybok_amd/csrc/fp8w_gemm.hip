@@ -79,7 +79,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps k-tile indices scalar
   const int strip = blockIdx.x;
   const int split = blockIdx.y;
   const int mblock = blockIdx.z;

@@ -424,6 +424,7 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   // many query tiles already fill the device: keep whole key ranges in one block (no partials)
   while (splits > 1 && H * mtiles * splits > 2 * device_cus()) --splits;
   a.kv_splits = splits;
+  a.xcd_remap = (batch > 0 && splits == 1 && H * mtiles >= 2 * device_cus()) ? 1 : 0;
   a.partial = nullptr;
   a.counters = nullptr;
   if (splits > 1) {

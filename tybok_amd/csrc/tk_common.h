@@ -20,20 +20,15 @@ typedef unsigned short u16;
 
 __device__ __forceinline__ float bf16_bits_to_f32(u16 b) { return __uint_as_float(((unsigned)b) << 16); }
 
-// fp32 -> bf16 bits, round-to-nearest-even (NaN kept quiet), same as torch's cast.
-__device__ __forceinline__ u16 f32_to_bf16_bits(float f) {
-  unsigned u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (u16)(u >> 16);
-}
 // two fp32 -> packed bf16 pair (lo = a, hi = b), round-to-nearest-even in one v_cvt_pk_bf16_f32
+// (NaN stays a quiet NaN), same as torch's cast.
 __device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
   f32x2 v = {a, b};
   union { bf16x2 h; unsigned u; } r;
   r.h = __builtin_convertvector(v, bf16x2);
   return r.u;
 }
+__device__ __forceinline__ u16 f32_to_bf16_bits(float f) { return (u16)pack_bf16x2(f, 0.f); }
 // four fp32 <-> four bf16 in two dwords
 __device__ __forceinline__ i32x2 pack_bf16x4(f32x4 v) {
   i32x2 r = {(int)pack_bf16x2(v[0], v[1]), (int)pack_bf16x2(v[2], v[3])};
@@ -44,7 +39,7 @@ __device__ __forceinline__ f32x4 unpack_bf16x4(i32x2 r) {
              __uint_as_float((unsigned)r[1] << 16), __uint_as_float((unsigned)r[1] & 0xffff0000u)};
   return v;
 }
-__device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+__device__ __forceinline__ float round_bf16(float f) { return __uint_as_float(pack_bf16x2(f, 0.f) << 16); }
 
 // 4 e4m3fn bytes (one dword) -> 4 bf16 (exact: every e4m3 value is a bf16 value).
 __device__ __forceinline__ void fp8x4_to_bf16x4(int v, bf16x2& lo, bf16x2& hi) {

@@ -67,6 +67,7 @@ struct AttnArgs {
   int M, P, S, H, G;
   // independent problems in one launch (prefix-only): element strides between them, 0 = single
   int batch;
+  int xcd_remap;  // batched, unsplit launches: 1-D grid with (problem, head) pairs pinned to an XCD
   long long q_sb, k_sb, vt_sb, out_sb;
   int mask_mode, logits_bf16;
   int kv_splits;
