@@ -94,12 +94,11 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   a.k_pre += bi * a.k_sb;
   a.vt_pre += bi * a.vt_sb;
   a.out += bi * a.out_sb;
-  const int g = h / (a.H / a.G);
+  const int g = (h * a.gqa_mul) >> 16;       // h / (H / G) without a runtime divide
   TA_MARK(0);
   const int tp = (a.P + 31) >> 5;            // prefix tiles; suffix tiles follow
-  const int ntiles = tp + ((a.S + 31) >> 5);
-  const int t_lo = (split * ntiles) / a.kv_splits;
-  const int t_hi = ((split + 1) * ntiles) / a.kv_splits;
+  const int t_lo = split * a.tile_q + (split < a.tile_r ? split : a.tile_r);
+  const int t_hi = t_lo + a.tile_q + (split < a.tile_r ? 1 : 0);
   const int qi = mtile * 32 + l32;
   const bool q_ok = qi < a.M;
 

@@ -87,8 +87,10 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   const int l32 = lane & 31;
 
   TK_MARK(0);
-  const int kt_lo = (int)(((long long)split * a.KT) / a.ksplit);
-  const int kt_hi = (int)(((long long)(split + 1) * a.KT) / a.ksplit);
+  // k tiles of this split: KT = ksplit * kt_q + kt_r, the first kt_r splits take one more (host-side
+  // division: a 64-bit divide here costs some 300 scalar instructions before the first load)
+  const int kt_lo = split * a.kt_q + (split < a.kt_r ? split : a.kt_r);
+  const int kt_hi = kt_lo + a.kt_q + (split < a.kt_r ? 1 : 0);
   const int nrounds = (kt_hi - kt_lo + RKT - 1) / RKT;
   const int k_end = kt_hi * 32 < a.K ? kt_hi * 32 : a.K;  // first activation column this block must not use
 

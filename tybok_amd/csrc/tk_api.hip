@@ -169,6 +169,8 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   if (ks > a.KT) ks = a.KT;
   if (ks > 64) ks = 64;
   a.ksplit = ks;
+  a.kt_q = a.KT / ks;
+  a.kt_r = a.KT % ks;
   a.partial = nullptr;
   a.counters = nullptr;
   if (ks > 1) {
@@ -424,6 +426,9 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   // many query tiles already fill the device: keep whole key ranges in one block (no partials)
   while (splits > 1 && H * mtiles * splits > 2 * device_cus()) --splits;
   a.kv_splits = splits;
+  a.tile_q = ntiles / splits;
+  a.tile_r = ntiles % splits;
+  a.gqa_mul = (65536 + H / G - 1) / (H / G);
   a.xcd_remap = (batch > 0 && splits == 1 && H * mtiles >= 2 * device_cus()) ? 1 : 0;
   a.partial = nullptr;
   a.counters = nullptr;

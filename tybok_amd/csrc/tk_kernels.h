@@ -21,6 +21,7 @@ struct GemmArgs {
   int KT;       // k tiles of 32
   int ntiles;   // n tiles of 32 in the packed buffer (gated: 2 * I / 32)
   int ksplit;
+  int kt_q, kt_r;  // KT = ksplit * kt_q + kt_r
   float* partial;
   int* counters;
   int act;
@@ -71,6 +72,8 @@ struct AttnArgs {
   long long q_sb, k_sb, vt_sb, out_sb;
   int mask_mode, logits_bf16;
   int kv_splits;
+  int tile_q, tile_r;  // key tiles = kv_splits * tile_q + tile_r
+  int gqa_mul;         // kv head of query head h = (h * gqa_mul) >> 16
   float* partial;
   int* counters;
   float scale;
