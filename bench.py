@@ -245,7 +245,8 @@ def main() -> None:
     pi05_p50 = None
     if not args.skip_pi05:
         ckpt5 = write_pi05_checkpoint(os.path.join(tmp, "pi05"), cameras=2, seed=0)
-        flags5 = {k: v for k, v in flags.items() if k not in ("tl_llm_fused_attn", "tl_vit_oproj")}  # a SmolVLA-only tier
+        flags5 = {k: v for k, v in flags.items() if k not in ("tl_llm_fused_attn", "tl_vit_oproj")}  # SmolVLA-only tiers
+        flags5["tl_llm_flash_attn"] = True  # pi0.5's name for the fused prefill
         eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **flags5)
         frame5 = device_frame(eng5, 2)
         s5, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)

@@ -46,10 +46,12 @@ TIERS = [
     dict(fused_expert=False, fp8_expert_mlp=False, fp8_llm_mlp=False),
     dict(fused_expert=True, fp8_expert_mlp=False, fp8_llm_mlp=False),
     dict(fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True),
+    dict(fused_expert=False, fp8_expert_mlp=False, fp8_llm_mlp=False, fused_prefill=True),
+    dict(fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True, fused_prefill=True),
 ]
 
 
-@pytest.mark.parametrize("tiers", TIERS, ids=["eager", "attn", "full"])
+@pytest.mark.parametrize("tiers", TIERS, ids=["eager", "attn", "full", "prefill", "full+prefill"])
 def test_small_model_chunk_matches_oracle(tiers):
     cfg, sd, inp = cases.pi05_build(cases.PI05_CASES["small"])
     want = _oracle_chunk(cfg, sd, inp, tiers["fp8_llm_mlp"], tiers["fp8_expert_mlp"])
@@ -72,6 +74,10 @@ def test_zero_noise_chunk_within_bound():
     err = float((got - want).abs().max())
     print(f"pi05 zero-noise fp8: max|err| = {err:.4g}, |chunk|max = {float(want.abs().max()):.3g}")
     assert err <= 1e-2
+    got = _gpu_chunk(cfg, sd, inp, fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True, fused_prefill=True)
+    err = float((got - want).abs().max())
+    print(f"pi05 zero-noise fp8 + fused prefill: max|err| = {err:.4g}")
+    assert err <= 1e-2
 
 
 @pytest.fixture(scope="module")
@@ -84,7 +90,7 @@ def ckpt(tmp_path_factory):
 def test_engine_api_and_graph_equals_eager(ckpt):
     from tybok_amd.registry import create_engine
 
-    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True)
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_flash_attn=True)
     eager = create_engine(ckpt, device="cuda", graph=False, warmup=False, **flags)
     graph = create_engine(ckpt, device="cuda", graph=True, warmup=True, **flags)
     assert graph.graph_enabled and list(graph._graph_runner.keys()) == [(2, 200)]

@@ -7,8 +7,10 @@ flags wired to the HIP kernels:
 * ``tl_fused_expert``     expert denoising attention on ``tk_expert_attn`` (bf16 logits)
 * ``tl_fp8_expert_mlp``   expert GeGLU FFN on e4m3fn weights with the gated residual fused
 * ``tl_fp8_llm_mlp``      VLM prefill GeGLU FFN on e4m3fn weights
+* ``tl_llm_flash_attn``   VLM prefill layers on the fused launches (norm + q|k|v + RoPE, attention
+                          under the pad mask, o_proj + residual), K/V cache written by the projection
 
-The prefix-side tiers (``tl_fused_vit``, ``tl_llm_flash_attn``, ``vit_mlp_dtype``, ``pad_free``,
+The prefix-side tiers (``tl_fused_vit``, ``vit_mlp_dtype``, ``pad_free``,
 ``skip_empty_images``), ``compile_model`` and Real-Time Chunking are not implemented here and are
 rejected when requested.
 """
@@ -68,7 +70,6 @@ class PI05Engine(PolicyEngine):
         "tl_llm_fused_attn": False,
         "tl_vit_oproj": False,
         "tl_fused_vit": False,
-        "tl_llm_flash_attn": False,
         "vit_mlp_dtype": None,
         "skip_empty_images": False,
         "pad_free": False,
@@ -117,7 +118,7 @@ class PI05Engine(PolicyEngine):
         reject_unsupported_flags(type(self), "pi05", kwargs)
         reject_unsupported_flags(
             type(self), "pi05",
-            dict(tl_fused_vit=tl_fused_vit, tl_llm_flash_attn=tl_llm_flash_attn, vit_mlp_dtype=vit_mlp_dtype,
+            dict(tl_fused_vit=tl_fused_vit, vit_mlp_dtype=vit_mlp_dtype,
                  skip_empty_images=skip_empty_images, pad_free=pad_free),
         )  # fmt: skip
         if sampler != "euler":
@@ -126,7 +127,14 @@ class PI05Engine(PolicyEngine):
             raise NotImplementedError("--compile is not supported by this backend (the HIP tiers replace it)")
         if rtc_config and rtc_config.get("enabled"):
             raise NotImplementedError("Real-Time Chunking is not implemented by this backend")
-        hip_flags = [n for n, on in (("--tl-fused-expert", tl_fused_expert), ("--tl-fp8-llm-mlp", tl_fp8_llm_mlp), ("--tl-fp8-expert-mlp", tl_fp8_expert_mlp)) if on]
+        hip_flags = [
+            n
+            for n, on in (
+                ("--tl-fused-expert", tl_fused_expert), ("--tl-fp8-llm-mlp", tl_fp8_llm_mlp),
+                ("--tl-fp8-expert-mlp", tl_fp8_expert_mlp), ("--tl-llm-flash-attn", tl_llm_flash_attn),
+            )
+            if on
+        ]  # fmt: skip
         if hip_flags and not str(self.device).startswith("cuda"):
             # same gate as the reference's _require_fp8_mma (engine.py:51-71), for this hardware
             raise RuntimeError(f"{' / '.join(hip_flags)} run gfx950 HIP kernels, but the engine is running on {self.device!r}")
@@ -153,6 +161,7 @@ class PI05Engine(PolicyEngine):
         self.model = PI05Model(
             self.config, sd, self.device,
             fused_expert=self.tl_fused_expert, fp8_expert_mlp=self.tl_fp8_expert_mlp, fp8_llm_mlp=self.tl_fp8_llm_mlp,
+            fused_prefill=bool(tl_llm_flash_attn),
         )  # fmt: skip
         del sd
 

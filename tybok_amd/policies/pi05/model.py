@@ -76,13 +76,15 @@ class PI05Model:
         fused_expert: bool = False,
         fp8_expert_mlp: bool = False,
         fp8_llm_mlp: bool = False,
+        fused_prefill: bool = False,
     ):
         self.cfg = cfg
         self.device = torch.device(device)
         self.fused_expert = bool(fused_expert)
         self.fp8_expert_mlp = bool(fp8_expert_mlp)
         self.fp8_llm_mlp = bool(fp8_llm_mlp)
-        self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp
+        self.fused_prefill = bool(fused_prefill)
+        self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp or self.fused_prefill
         if self.use_hip and self.device.type != "cuda":
             raise RuntimeError("the fused / fp8 tiers run HIP kernels and need a GPU device")
         self.vd, self.ed = cfg.paligemma_dims, cfg.expert_dims
@@ -100,18 +102,32 @@ class PI05Model:
         freqs = torch.arange(_ROPE_POSITIONS, dtype=torch.float32)[:, None] * inv[None, :]
         emb = torch.cat([freqs, freqs], dim=-1)
         self.rope_cos, self.rope_sin = emb.cos().to(self.device), emb.sin().to(self.device)
-        if self.fused_expert:
+        half = self.head_dim // 2
+
+        def pack_stack(stack: str, depth: int):
+            qkv, o = [], []
+            for i in range(depth):
+                lp = f"{stack}layers.{i}.self_attn."
+                w = torch.cat([self.p[lp + n + "_proj.weight"] for n in "qkv"], dim=0).to(BF16)
+                qkv.append(tk.pack_bf16_weight(w, rope_half=half))
+                o.append(tk.pack_bf16_weight(self.p[lp + "o_proj.weight"].to(BF16)))
+            return qkv, o
+
+        if self.fused_expert or self.fused_prefill:
             # the fused rotary epilogue reads fp32 tables holding the bf16 values the eager path uses
-            half = self.head_dim // 2
             self.rope_tables_hip = tk.RopeTables(
                 self.rope_cos[:, :half].to(BF16).float().contiguous(), self.rope_sin[:, :half].to(BF16).float().contiguous()
             )
-            self.exp_qkv, self.exp_o = [], []
-            for i in range(self.ed["depth"]):
-                lp = f"{EXP}layers.{i}.self_attn."
-                w = torch.cat([self.p[lp + n + "_proj.weight"] for n in "qkv"], dim=0).to(BF16)
-                self.exp_qkv.append(tk.pack_bf16_weight(w, rope_half=half))
-                self.exp_o.append(tk.pack_bf16_weight(self.p[lp + "o_proj.weight"].to(BF16)))
+        if self.fused_expert:
+            self.exp_qkv, self.exp_o = pack_stack(EXP, self.ed["depth"])
+        if self.fused_prefill:
+            self.vlm_qkv, self.vlm_o = pack_stack(VLM, self.depth)
+            # Gemma RMSNorm x * rstd * (1 + w) is the adaptive norm with scale = w and shift = 0
+            zeros = torch.zeros(self.vd["width"], dtype=torch.float32, device=self.device)
+            self.vlm_norms = [
+                tuple((self.p[f"{VLM}layers.{i}.{n}.weight"].float().contiguous(), zeros) for n in ("input_layernorm", "post_attention_layernorm"))
+                for i in range(self.depth)
+            ]
         self.embed_scale = torch.tensor(self.vd["width"] ** 0.5, dtype=BF16, device=self.device)
         self.patch_w = self.p[VIS + "embeddings.patch_embedding.weight"].reshape(cfg.vision_hidden, -1)
         self.set_num_steps(cfg.num_steps)
@@ -218,6 +234,41 @@ class PI05Model:
             hidden = self.vlm_mlp[i](h, hidden)
         return kv
 
+    def prefill_fused(self, embs: torch.Tensor, pad_masks: torch.Tensor):
+        """VLM prefill on the fused launches (norm + q|k|v + RoPE, attention under the pad x pad mask,
+        o_proj + residual, GeGLU FFN) -> ``(kv, caches)``: ``kv`` per-layer ``(K, V) [1, G, P, D]`` views
+        of the projection outputs, ``caches`` the same keys with V^T in the attention kernel's layout."""
+        p_len = embs.shape[1]
+        p_pad = (p_len + 31) // 32 * 32
+        heads, g, d = self.vd["num_heads"], self.vd["num_kv_heads"], self.head_dim
+        nq, nkv = heads * d, g * d
+        mask2d = torch.zeros(p_len, p_pad, dtype=torch.uint8, device=self.device)
+        mask2d[:, :p_len] = pad_masks[0][:, None] & pad_masks[0][None, :]
+        pos32 = (torch.cumsum(pad_masks, dim=1) - 1)[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
+        qkv_all = torch.empty(self.depth, p_len, nq + 2 * nkv, dtype=BF16, device=self.device)
+        vt_all = torch.zeros(self.depth, nkv, p_pad, dtype=BF16, device=self.device)
+        hidden = embs[0].to(BF16)
+        kv, caches = [], []
+        for i in range(self.depth):
+            norm_in, norm_post = self.vlm_norms[i]
+            qkv = tk.bf16w_linear(
+                hidden, self.vlm_qkv[i], ada=norm_in, eps=EPS, rope=self.rope_tables_hip, rope_pos=pos32, rope_cols=nq + nkv,
+                rope_bf16=True, vt_out=vt_all[i], vt_col0=nq + nkv, out=qkv_all[i], ws=self.ws,
+            )  # fmt: skip
+            k = qkv[:, nq : nq + nkv].view(p_len, g, d)
+            cache = tk.PrefixKV(k, vt_all[i].view(g, d, p_pad))
+            att = tk.expert_attn(qkv[:, :nq].view(p_len, heads, d), cache, None, None, tk.MASK_NONE, mask2d=mask2d, logits_bf16=True, ws=self.ws)
+            out = tk.bf16w_linear(att, self.vlm_o[i], resid=hidden, ws=self.ws)
+            mlp = self.vlm_mlp[i]
+            if mlp.fp8:
+                hidden = tk.fp8w_gated_ffn(out, mlp.wgu, mlp.wd, "gelu_tanh", resid=out, ada=norm_post, eps=EPS, ws=self.ws)
+            else:
+                h, _ = gemma_norm(out[None], weight=self.p[f"{VLM}layers.{i}.post_attention_layernorm.weight"])
+                hidden = mlp(h, out[None])[0]
+            kv.append((k.transpose(0, 1)[None], qkv[:, nq + nkv :].view(p_len, g, d).transpose(0, 1)[None]))
+            caches.append(cache)
+        return kv, caches
+
     # ------------------------------------------------------------------ denoising
     def attention_caches(self, kv) -> list:
         """Per-layer prefix K/V in the attention kernel's layout (V transposed), once per request."""
@@ -294,12 +345,17 @@ class PI05Model:
     def sample_actions(self, images, img_masks, tokens, masks, noise, trace: dict | None = None) -> torch.Tensor:
         """Prefix embed, prefill, Euler loop -> ``[1, chunk, max_action_dim]`` fp32."""
         embs, pads = self.embed_prefix(images, img_masks, tokens, masks)
-        kv = self.prefill(embs, pads)
+        caches = None
+        if self.fused_prefill and embs.shape[0] == 1:
+            kv, caches = self.prefill_fused(embs, pads)
+        else:
+            kv = self.prefill(embs, pads)
         if trace is not None:
             trace.update(prefix_embs=embs, pad_masks=pads, kv=kv)
         dt = -1.0 / self.num_steps
         x_t = noise
-        caches = self.attention_caches(kv) if self.fused_expert else None
+        if caches is None or not self.fused_expert:
+            caches = self.attention_caches(kv) if self.fused_expert else None
         for step in range(self.num_steps):
             x_t = x_t + dt * self.denoise_step(pads, kv, x_t, step, caches)
         return x_t
