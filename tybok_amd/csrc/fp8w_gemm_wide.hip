@@ -1,0 +1,399 @@
+// fp8-weight GEMM for many rows (M > 64: the VLM prefill) on gfx950.
+//
+// Same operands and packed weight tiles as the skinny kernel (fp8w_gemm.hip), other balance: with
+// hundreds of rows the product is MFMA-bound, so the block tile is large enough that neither
+// operand is re-read often:
+//   * a block of 4 waves owns 128 rows x 8 packed n tiles (256 packed columns) and a range of k
+//     tiles; wave w owns n tiles 2w, 2w+1 for all 128 rows: 8 accumulator tiles of 32x32, and per
+//     k tile 16 MFMAs against 2 weight loads (straight from global memory into operand registers,
+//     1 KiB coalesced per tile, e4m3 -> bf16 in registers) and 8 LDS operand reads;
+//   * the activations of a round (128 rows x 64 columns) are staged once per block through LDS with
+//     whole 128-byte lines per row, double buffered, one LDS barrier per round;
+//   * blocks that share weights (same n tiles and k range, different rows) get consecutive slots of
+//     ONE XCD, so the weight tiles are read from HBM once and served from that XCD's L2 afterwards;
+//   * K splits (few column blocks, long K: the down projection) hand fp32 partials through the
+//     workspace; the last-arriving block sums them in split order -- bit-deterministic.
+// The epilogues compute exactly what the skinny kernel's do (same rounding points).
+#include "tk_common.h"
+#include "tk_kernels.h"
+
+namespace {
+
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+constexpr int MT = 4;   // m tiles per block (and per wave)
+constexpr int NT = 2;   // n tiles per wave
+constexpr int NW = 4;   // waves per block
+constexpr int RK = 2;   // k tiles per round
+constexpr int PF = 4;   // rounds in flight (even: round r uses LDS buffer r % 2)
+
+// EPI: 0 plain (scale, optional per-column gate, optional residual), 1 gated (gate/up tile pairs).
+template <int EPI>
+__global__ __launch_bounds__(NW * 64) void fp8w_wide_kernel(GemmArgs a, int nblk_m, int ngroups) {
+  constexpr int ROWS = MT * 32;
+  constexpr int ROWB = RK * 64;            // bytes of one staged activation row per round
+  constexpr int PITCH = ROWB + 16;         // conflict-free 16-byte operand reads, 16-byte aligned
+  constexpr int XBUF = ROWS * PITCH;
+  constexpr int PPR = ROWB / 16;           // 16-byte pieces per staged row
+  constexpr int XPT = ROWS * PPR / (NW * 64);
+  constexpr int TILES = MT * NT;
+  __shared__ __align__(16) unsigned char lds[2 * XBUF];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5;
+  const int l32 = lane & 31;
+
+  // slot s of XCD x (blocks are dealt to the 8 XCDs round-robin) -> group (s / nblk_m) * 8 + x, m block
+  // s % nblk_m: the nblk_m blocks of a group (same weights) run back to back on one XCD
+  const unsigned id = blockIdx.x;
+  const unsigned slot = id >> 3;
+  const int mblock = (int)(slot % (unsigned)nblk_m);
+  const int group = (int)((slot / (unsigned)nblk_m) * 8 + (id & 7));
+  if (group >= ngroups) return;
+  const int split = group % a.ksplit;
+  const int nblk = group / a.ksplit;
+
+  const int kt_lo = split * a.kt_q + (split < a.kt_r ? split : a.kt_r);
+  const int kt_hi = kt_lo + a.kt_q + (split < a.kt_r ? 1 : 0);
+  const int nrounds = (kt_hi - kt_lo + RK - 1) / RK;
+  const int k_end = kt_hi * 32 < a.K ? kt_hi * 32 : a.K;
+
+  const int strip = nblk * NW + wave;  // this wave's pair of packed n tiles
+  const uint8_t* wbase[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    int ntg = strip * NT + nt;
+    if (ntg > a.ntiles - 1) ntg = a.ntiles - 1;  // overhanging tiles are computed on valid data, never stored
+    wbase[nt] = a.w + ((size_t)ntg * a.KT) * 1024 + lane * 16;
+  }
+
+  const char* xsrc[XPT];
+  int xcol[XPT], xdst[XPT];
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) {
+    const int p = tid + i * NW * 64;
+    const int r = p / PPR, c = p % PPR;
+    int m = mblock * ROWS + r;
+    if (m > a.M - 1) m = a.M - 1;  // rows past M: valid data, never stored
+    xsrc[i] = (const char*)a.x + (size_t)m * a.ldx * 2;
+    xcol[i] = c * 8;
+    xdst[i] = r * PITCH + c * 16;
+  }
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
+
+  struct WFrag {
+    i32x4 w[RK][NT];
+  };
+  struct XFrag {
+    i32x4 v[XPT];
+  };
+  auto wload = [&](WFrag& f, int r) {
+#pragma unroll
+    for (int j = 0; j < RK; ++j) {
+      int kt = kt_lo + r * RK + j;
+      if (kt > a.KT - 1) kt = a.KT - 1;  // its activation columns are zeroed
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) f.w[j][nt] = *(const i32x4*)(wbase[nt] + (size_t)kt * 1024);
+    }
+  };
+  auto xload = [&](XFrag& f, int r) {
+    const int k0 = (kt_lo + r * RK) * 32;
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) {
+      int k = k0 + xcol[i];
+      if (k > a.K - 8) k = a.K - 8;
+      f.v[i] = *(const i32x4*)(xsrc[i] + (size_t)k * 2);
+    }
+  };
+  auto xstore = [&](const XFrag& f, int r, int b) {
+    const int k0 = (kt_lo + r * RK) * 32;
+    const i32x4 z = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) *(i32x4*)(lds + b * XBUF + xdst[i]) = (k0 + xcol[i]) < k_end ? f.v[i] : z;
+  };
+  // Operand fragments and converted weights of two k tiles: while the MFMAs of one k tile run,
+  // the LDS reads and the e4m3 -> bf16 conversions of the next one are issued between them.
+  i32x4 xa[2][MT][2];
+  bf16x8 wb[2][NT][2];
+  auto xread = [&](int set, int b, int j) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const i32x4* p = (const i32x4*)(lds + b * XBUF + (mt * 32 + l32) * PITCH + (j * 32 + 16 * half) * 2);
+      xa[set][mt][0] = p[0];
+      xa[set][mt][1] = p[1];
+    }
+  };
+  auto wcvt = [&](int set, const WFrag& f, int j) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      wb[set][nt][0] = fp8x8_to_bf16x8(f.w[j][nt][0], f.w[j][nt][1]);
+      wb[set][nt][1] = fp8x8_to_bf16x8(f.w[j][nt][2], f.w[j][nt][3]);
+    }
+  };
+  auto mma = [&](int set) {
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[set][nt][h2], as_bf16x8(xa[set][mt][h2]), acc[mt][nt], 0, 0, 0);
+  };
+  // scheduling hint for a phase of 16 MFMAs, 8 LDS reads and 16 conversions: spread the reads and
+  // the conversions between the MFMAs instead of waiting for each read right before its MFMA
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS read
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // VALU
+    }
+  };
+  static_assert(RK == 2 && PF % 2 == 0, "a round is two phases; buffer parity follows the pipeline slot");
+
+  // PF rounds in flight; every load is unconditional (clamped addresses; columns past the block's k
+  // range are zeroed when staged), so the loop bodies have no branch and the compiler keeps precise
+  // wait counts.  Round r: phase A multiplies k tile 0 while k tile 1's operands are fetched from
+  // LDS; phase B stages round r+1 into the other LDS buffer, passes the round's only barrier (a wave
+  // can write buffer b for round r+2 only after every wave has passed the barrier of round r+1, i.e.
+  // has its round-r operands in registers), fetches round r+1's first operands and multiplies k tile 1.
+  WFrag wbuf[PF];
+  XFrag xbuf[PF];
+#pragma unroll
+  for (int p = 0; p < PF; ++p) {
+    xload(xbuf[p], p);
+    wload(wbuf[p], p);
+  }
+  xstore(xbuf[0], 0, 0);
+  xload(xbuf[0], PF);
+  lds_barrier();
+  xread(0, 0, 0);
+  wcvt(0, wbuf[0], 0);
+  auto round = [&](int p, int r) {
+    const int b = p & 1;  // == r & 1: rounds advance PF at a time
+    const int pn = (p + 1) % PF;
+    __builtin_amdgcn_sched_barrier(0);
+    xread(1, b, 1);
+    wcvt(1, wbuf[p], 1);
+    mma(0);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    wload(wbuf[p], r + PF);
+    xstore(xbuf[pn], r + 1, b ^ 1);
+    xload(xbuf[pn], r + 1 + PF);
+    lds_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    xread(0, b ^ 1, 0);
+    wcvt(0, wbuf[pn], 0);
+    mma(1);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  {
+    int it = 0;
+    for (; it + PF <= nrounds; it += PF) {
+#pragma unroll
+      for (int p = 0; p < PF; ++p) round(p, it + p);
+    }
+    const int rem = nrounds - it;  // in [0, PF)
+#pragma unroll
+    for (int q = 0; q < PF - 1; ++q)
+      if (q < rem) round(q, it + q);  // block-uniform
+  }
+
+  // ---- K-split hand-off: fp32 partials [(block, split)][wave][tile][group][lane][4] ----
+  const int blk_lin = nblk * nblk_m + mblock;
+  if (a.ksplit > 1) {
+    unsigned long long* pbase = (unsigned long long*)a.partial + ((size_t)wave * TILES * 4 * 64 + lane) * 2;
+    unsigned long long* mine = pbase + ((size_t)blk_lin * a.ksplit + split) * (NW * TILES * 4 * 64 * 2);
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& c = acc[t / NT][t % NT];
+        unsigned long long* dst = mine + (size_t)(t * 4 + g) * 128;
+        st_agent64(dst, c[4 * g], c[4 * g + 1]);
+        st_agent64(dst + 1, c[4 * g + 2], c[4 * g + 3]);
+      }
+    __shared__ int s_last;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (old == a.ksplit - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
+    for (int s = 0; s < a.ksplit; ++s) {  // split order, whoever arrived last
+      const unsigned long long* src = pbase + ((size_t)blk_lin * a.ksplit + s) * (NW * TILES * 4 * 64 * 2);
+      unsigned long long raw[TILES][4][2];
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          raw[t][g][0] = ld_agent64(src + (size_t)(t * 4 + g) * 128);
+          raw[t][g][1] = ld_agent64(src + (size_t)(t * 4 + g) * 128 + 1);
+        }
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f32x16& c = acc[t / NT][t % NT];
+          c[4 * g] += __uint_as_float((unsigned)raw[t][g][0]);
+          c[4 * g + 1] += __uint_as_float((unsigned)(raw[t][g][0] >> 32));
+          c[4 * g + 2] += __uint_as_float((unsigned)raw[t][g][1]);
+          c[4 * g + 3] += __uint_as_float((unsigned)(raw[t][g][1] >> 32));
+        }
+    }
+  }
+
+  // ---- epilogue: lane l of a tile owns row m = l % 32 and, per register group g, four
+  // consecutive columns 8g + 4*(l/32) .. +3 (the accumulators hold C^T) ----
+  if (EPI == 0) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n0 = (strip * NT + nt) * 32 + 8 * g + 4 * half;
+        if (n0 >= a.N) continue;
+        const f32x4 sc = *(const f32x4*)(a.s0 + n0);
+        f32x4 gt = {0.f, 0.f, 0.f, 0.f};
+        if (a.gate) gt = unpack_bf16x4(*(const i32x2*)(a.gate + n0));
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const int m = (mblock * MT + mt) * 32 + l32;
+          if (m >= a.M) continue;
+          const f32x16& c = acc[mt][nt];
+          f32x4 v = {c[4 * g], c[4 * g + 1], c[4 * g + 2], c[4 * g + 3]};
+          i32x2 r = pack_bf16x4(v * sc);
+          if (a.gate) r = pack_bf16x4(unpack_bf16x4(r) * gt);
+          if (a.resid) {
+            const f32x4 rv = a.resid_f32 ? *(const f32x4*)((const float*)a.resid + (size_t)m * a.ldr + n0)
+                                         : unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n0));
+            r = pack_bf16x4(unpack_bf16x4(r) + rv);
+          }
+          *(i32x2*)(a.y + (size_t)m * a.ldy + n0) = r;
+        }
+      }
+  } else {
+    // tile pair (gate, up) of logical columns strip*32 ..; I % 32 == 0
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int col = strip * 32 + 8 * g + 4 * half;
+      if (col >= a.N) continue;
+      const f32x4 scg = *(const f32x4*)(a.s0 + col), scu = *(const f32x4*)(a.s1 + col);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = (mblock * MT + mt) * 32 + l32;
+        if (m >= a.M) continue;
+        const f32x16& cg = acc[mt][0];
+        const f32x16& cu = acc[mt][1];
+        const f32x4 vg = {cg[4 * g], cg[4 * g + 1], cg[4 * g + 2], cg[4 * g + 3]};
+        const f32x4 vu = {cu[4 * g], cu[4 * g + 1], cu[4 * g + 2], cu[4 * g + 3]};
+        const f32x4 gg = unpack_bf16x4(pack_bf16x4(vg * scg));
+        const f32x4 up = unpack_bf16x4(pack_bf16x4(vu * scu));
+        f32x4 act;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) act[j] = a.act == 0 ? silu_f(gg[j]) : gelu_tanh_f(gg[j]);
+        act = unpack_bf16x4(pack_bf16x4(act));
+        *(i32x2*)(a.y + (size_t)m * a.ldy + col) = pack_bf16x4(act * up);
+      }
+    }
+  }
+}
+
+// One block per row: out = bf16 norm of the bf16 row, with the rounding points of the skinny
+// kernel's prologues: RMSNorm bf16(w * bf16(x * rstd)); adaptive bf16((x * rstd) * (1 + scale) + shift).
+__global__ __launch_bounds__(256) void norm_rows_kernel(NormRowsArgs a) {
+  __shared__ float part[4];
+  const int tid = threadIdx.x;
+  const char* row = (const char*)a.x + (size_t)blockIdx.x * a.ldx * 2;
+  const int pieces = a.K / 8;
+  float ss0 = 0.f, ss1 = 0.f;
+  for (int p = tid; p < pieces; p += 256) {
+    union { i32x4 v; bf16x2 h[4]; } xu;
+    xu.v = *(const i32x4*)(row + (size_t)p * 16);
+    ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[0], xu.h[0], ss0, false);
+    ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[1], xu.h[1], ss1, false);
+    ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[2], xu.h[2], ss0, false);
+    ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[3], xu.h[3], ss1, false);
+  }
+  float ss = ss0 + ss1;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+  if ((tid & 63) == 0) part[tid >> 6] = ss;
+  __syncthreads();
+  ss = (part[0] + part[1]) + (part[2] + part[3]);
+  const float rstd = rsqrtf(ss / (float)a.K + a.eps);
+  char* dst = (char*)a.out + (size_t)blockIdx.x * a.ldo * 2;
+  for (int p = tid; p < pieces; p += 256) {
+    union { i32x4 v; unsigned u[4]; } xu, o;
+    xu.v = *(const i32x4*)(row + (size_t)p * 16);
+    if (a.ada_scale) {
+      union { i32x4 v[2]; float f[8]; } sc, sh;
+      sc.v[0] = *(const i32x4*)(a.ada_scale + p * 8);
+      sc.v[1] = *(const i32x4*)(a.ada_scale + p * 8 + 4);
+      sh.v[0] = *(const i32x4*)(a.ada_shift + p * 8);
+      sh.v[1] = *(const i32x4*)(a.ada_shift + p * 8 + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float x0 = __uint_as_float(xu.u[e] << 16), x1 = __uint_as_float(xu.u[e] & 0xffff0000u);
+        const float y0 = __fadd_rn(__fmul_rn(__fmul_rn(x0, rstd), __fadd_rn(1.0f, sc.f[2 * e])), sh.f[2 * e]);
+        const float y1 = __fadd_rn(__fmul_rn(__fmul_rn(x1, rstd), __fadd_rn(1.0f, sc.f[2 * e + 1])), sh.f[2 * e + 1]);
+        o.u[e] = pack_bf16x2(y0, y1);
+      }
+    } else {
+      union { i32x4 v; unsigned u[4]; } nw;
+      nw.v = *(const i32x4*)(a.norm_w + p * 8);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const unsigned u = pack_bf16x2(__uint_as_float(xu.u[e] << 16) * rstd, __uint_as_float(xu.u[e] & 0xffff0000u) * rstd);
+        o.u[e] = pack_bf16x2(__uint_as_float(nw.u[e] << 16) * __uint_as_float(u << 16),
+                             __uint_as_float(nw.u[e] & 0xffff0000u) * __uint_as_float(u & 0xffff0000u));
+      }
+    }
+    *(i32x4*)(dst + (size_t)p * 16) = o.v;
+  }
+}
+
+}  // namespace
+
+int tk_wide_rows() { return MT * 32; }
+int tk_wide_cols() { return NW * NT * 32; }
+
+int tk_launch_gemm_wide(GemmArgs a, hipStream_t st) {
+  const int nblk_m = (a.M + MT * 32 - 1) / (MT * 32);
+  const int nblk_n = (a.ntiles + NW * NT - 1) / (NW * NT);
+  const int ngroups = nblk_n * a.ksplit;
+  const unsigned blocks = (unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m;
+  if (a.s1)
+    hipLaunchKernelGGL(fp8w_wide_kernel<1>, dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
+  else
+    hipLaunchKernelGGL(fp8w_wide_kernel<0>, dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st) {
+  hipLaunchKernelGGL(norm_rows_kernel, dim3(a.M), dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}

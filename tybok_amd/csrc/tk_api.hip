@@ -23,8 +23,10 @@ int fail(int code, const char* fmt, ...) {
 // workspace carving (bytes)
 constexpr size_t kCounterBytes = TK_WS_COUNTER_BYTES;
 constexpr size_t kPartialOff = kCounterBytes;
-constexpr size_t kPartialBytes = 24ull << 20;  // split-K / kv-split fp32 partials
-constexpr size_t kHiddenOff = kPartialOff + kPartialBytes;
+constexpr size_t kPartialBytes = 56ull << 20;  // split-K / kv-split fp32 partials
+constexpr size_t kNormOff = kPartialOff + kPartialBytes;
+constexpr size_t kNormBytes = 8ull << 20;  // normalised activations of a many-row GEMM
+constexpr size_t kHiddenOff = kNormOff + kNormBytes;
 constexpr size_t kHiddenBytes = TK_WS_TOTAL_BYTES - kHiddenOff;  // FFN [M, I] bf16 intermediate
 constexpr int kMaxCounters = (int)(kCounterBytes / 4);
 
@@ -134,6 +136,57 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   a.vt_ld = e.vt_ld;
 
   const int cus = device_cus();
+  const bool has_norm = e.norm_w || e.ada_scale;
+  if (!e.w16 && !rope && !e.x_f32 && a.vec && M > 64 &&
+      (!has_norm || (ws && ws_bytes >= kNormOff + (size_t)M * K * 2 && (size_t)M * K * 2 <= kNormBytes))) {
+    // many rows: MFMA-bound kernel with a 128 x 256 block tile
+    if (has_norm) {
+      NormRowsArgs nr;
+      nr.x = (const u16*)x;
+      nr.ldx = ldx;
+      nr.norm_w = (const u16*)e.norm_w;
+      nr.ada_scale = (const float*)e.ada_scale;
+      nr.ada_shift = (const float*)e.ada_shift;
+      nr.eps = e.norm_eps;
+      nr.out = (u16*)((char*)ws + kNormOff);
+      nr.ldo = K;
+      nr.M = M;
+      nr.K = K;
+      if (tk_launch_norm_rows(nr, st)) return fail(TK_ELAUNCH, "gemm: norm launch failed");
+      a.x = nr.out;
+      a.ldx = K;
+      a.norm_w = nullptr;
+      a.ada_scale = a.ada_shift = nullptr;
+    }
+    const int blocks0 = ((a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols()) * ((M + tk_wide_rows() - 1) / tk_wide_rows());
+    int ks = split_k;
+    if (ks <= 0) {
+      // fill the device once; a split keeps at least 16 k tiles and its partials must fit
+      ks = cus / blocks0;
+      if (ks > a.KT / 16) ks = a.KT / 16;
+      if (ks < 1) ks = 1;
+    }
+    const size_t per_split = (size_t)tk_wide_rows() * tk_wide_cols() * 4;
+    if (ks > 1 && ws) {
+      const size_t fit = kPartialBytes / (per_split * blocks0);
+      const size_t have = ws_bytes > kPartialOff ? (ws_bytes - kPartialOff) / (per_split * blocks0) : 0;
+      if ((size_t)ks > fit) ks = (int)fit;
+      if ((size_t)ks > have) ks = (int)have;
+      if (ks < 1) ks = 1;
+    }
+    if (ks > a.KT) ks = a.KT;
+    if (ks > 1 && (!ws || blocks0 > kMaxCounters)) {
+      if (split_k > 1) return fail(TK_EWORKSPACE, "gemm: split_k=%d needs a workspace", ks);
+      ks = 1;
+    }
+    a.ksplit = ks;
+    a.kt_q = a.KT / ks;
+    a.kt_r = a.KT % ks;
+    a.partial = ks > 1 ? (float*)((char*)ws + kPartialOff) : nullptr;
+    a.counters = ks > 1 ? (int*)ws : nullptr;
+    if (tk_launch_gemm_wide(a, st)) return fail(TK_ELAUNCH, "gemm: launch failed (%s)", hipGetErrorString(hipGetLastError()));
+    return TK_OK;
+  }
   int MT = M <= 32 ? 1 : 2;
   int NT = 2;
   if (e.w16) {

@@ -16,7 +16,7 @@ typedef unsigned short u16;
 
 // Workspace layout (bytes): [counters][scratch ...]
 #define TK_WS_COUNTER_BYTES (64 * 1024)  // 16384 int32 arrival counters
-#define TK_WS_TOTAL_BYTES (64ull * 1024 * 1024)
+#define TK_WS_TOTAL_BYTES (128ull * 1024 * 1024)
 
 __device__ __forceinline__ float bf16_bits_to_f32(u16 b) { return __uint_as_float(((unsigned)b) << 16); }
 
@@ -65,10 +65,12 @@ __device__ __forceinline__ bf16x8 as_bf16x8(i32x4 v) {
 }
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+// gelu(x, approximate="tanh") = 0.5 x (1 + tanh(z)) = x / (1 + exp(-2z)), z = sqrt(2/pi) (x + 0.044715 x^3):
+// the same function through one exponential instead of a tanh expansion.
 __device__ __forceinline__ float gelu_tanh_f(float x) {
   const float c0 = 0.7978845608028654f;  // sqrt(2/pi)
-  float inner = c0 * (x + 0.044715f * x * x * x);
-  return 0.5f * x * (1.0f + tanhf(inner));
+  const float inner = c0 * (x + 0.044715f * x * x * x);
+  return x / (1.0f + __expf(-2.0f * inner));
 }
 
 // Device-coherent (agent-scope, cache write-through / cache-bypassing) accesses used for data that

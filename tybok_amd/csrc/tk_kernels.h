@@ -108,7 +108,23 @@ struct TailArgs {
   int M, N, K;
 };
 
+struct NormRowsArgs {
+  const unsigned short* x;  // bf16 [M, K]
+  int ldx;
+  const unsigned short* norm_w;  // bf16 [K] (RMSNorm) or nullptr with ada_scale / ada_shift
+  const float* ada_scale;
+  const float* ada_shift;
+  float eps;
+  unsigned short* out;  // bf16 [M, K]
+  int ldo;
+  int M, K;
+};
+
 int tk_launch_tail(TailArgs a, hipStream_t st);
+int tk_wide_rows();  // block tile of the many-row GEMM
+int tk_wide_cols();
+int tk_launch_gemm_wide(GemmArgs a, hipStream_t st);
+int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st);
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st);
 int tk_launch_pack(const void* w0, const void* w1, void* out, int N, int K, int interleave, hipStream_t st);
 int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st);
