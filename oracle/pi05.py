@@ -57,6 +57,11 @@ class PI05Shape:
     num_steps: int = 10
     min_period: float = 4e-3
     max_period: float = 4.0
+    # drift tiers of the vision tower (tybok/policies/pi05/engine.py:196-230):
+    #   vit_mlp_dtype: fc1 / gelu / fc2 run in that dtype, cast at the boundary (vision.py:79-87);
+    #   vit_lowp_attn: q/k/v and out_proj run in bf16 too, attention scores and softmax in fp32.
+    vit_mlp_dtype: torch.dtype | None = None
+    vit_lowp_attn: bool = False
 
 
 def fp8_linear_names(shape: PI05Shape, llm_mlp: bool, expert_mlp: bool) -> frozenset:
@@ -77,17 +82,31 @@ def embed_image(w: Weights, shape: PI05Shape, image: torch.Tensor) -> torch.Tens
     x = x.flatten(2).transpose(1, 2)
     x = x + w[VIS + "embeddings.position_embedding.weight"][None]
     hd = shape.vis_hidden // shape.vis_heads
+    mdt = shape.vit_mlp_dtype
+
+    def lowp(name, t, dt):  # Linear with weights and bias converted to dt (vision.py:223-235)
+        return F.linear(t.to(dt), w[name + ".weight"].to(dt), w[name + ".bias"].to(dt))
+
     for i in range(shape.vis_layers):
         p = f"{VIS}encoder.layers.{i}."
         h = F.layer_norm(x, (shape.vis_hidden,), w[p + "layer_norm1.weight"], w[p + "layer_norm1.bias"], EPS)
-        q = w.linear(p + "self_attn.q_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
-        k = w.linear(p + "self_attn.k_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
-        v = w.linear(p + "self_attn.v_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
-        a = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, scale=hd**-0.5, is_causal=False)
-        a = a.transpose(1, 2).contiguous().reshape(b, -1, shape.vis_hidden)
-        x = x + w.linear(p + "self_attn.out_proj", a)
+        if shape.vit_lowp_attn:
+            q, k, v = (lowp(p + f"self_attn.{n}_proj", h, torch.bfloat16).view(b, -1, shape.vis_heads, hd).transpose(1, 2) for n in "qkv")
+            probs = torch.softmax(torch.matmul(q.float(), k.float().transpose(2, 3)) * hd**-0.5, dim=-1)
+            a = torch.matmul(probs, v.float()).to(torch.bfloat16).transpose(1, 2).reshape(b, -1, shape.vis_hidden)
+            x = x + lowp(p + "self_attn.out_proj", a, torch.bfloat16).float()
+        else:
+            q = w.linear(p + "self_attn.q_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
+            k = w.linear(p + "self_attn.k_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
+            v = w.linear(p + "self_attn.v_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
+            a = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, scale=hd**-0.5, is_causal=False)
+            a = a.transpose(1, 2).contiguous().reshape(b, -1, shape.vis_hidden)
+            x = x + w.linear(p + "self_attn.out_proj", a)
         h = F.layer_norm(x, (shape.vis_hidden,), w[p + "layer_norm2.weight"], w[p + "layer_norm2.bias"], EPS)
-        x = x + w.linear(p + "mlp.fc2", F.gelu(w.linear(p + "mlp.fc1", h), approximate="tanh"))
+        if mdt is not None:
+            x = x + lowp(p + "mlp.fc2", F.gelu(lowp(p + "mlp.fc1", h, mdt), approximate="tanh"), mdt).float()
+        else:
+            x = x + w.linear(p + "mlp.fc2", F.gelu(w.linear(p + "mlp.fc1", h), approximate="tanh"))
     x = F.layer_norm(x, (shape.vis_hidden,), w[VIS + "post_layernorm.weight"], w[VIS + "post_layernorm.bias"], EPS)
     return w.linear(PROJ, x)
 

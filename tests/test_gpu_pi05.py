@@ -18,12 +18,12 @@ from oracle.smolvla import Weights  # noqa: E402
 pytestmark = pytest.mark.gpu
 
 
-def _shape(cfg) -> O.PI05Shape:
-    return O.PI05Shape(depth=cfg.paligemma_dims["depth"], vis_layers=cfg.vision_layers, num_steps=cfg.num_steps)
+def _shape(cfg, **vit) -> O.PI05Shape:
+    return O.PI05Shape(depth=cfg.paligemma_dims["depth"], vis_layers=cfg.vision_layers, num_steps=cfg.num_steps, **vit)
 
 
-def _oracle_chunk(cfg, sd, inp, llm_fp8, exp_fp8):
-    shape = _shape(cfg)
+def _oracle_chunk(cfg, sd, inp, llm_fp8, exp_fp8, **vit):
+    shape = _shape(cfg, **vit)
     w = Weights(sd, O.fp8_linear_names(shape, llm_fp8, exp_fp8))
     with torch.no_grad():
         return O.sample_actions(w, shape, [i * 2.0 - 1.0 for i in inp["images"]], inp["img_masks"], inp["lang_tokens"], inp["lang_masks"], inp["noise"])
@@ -48,19 +48,22 @@ TIERS = [
     dict(fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True),
     dict(fused_expert=False, fp8_expert_mlp=False, fp8_llm_mlp=False, fused_prefill=True),
     dict(fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True, fused_prefill=True),
+    dict(fused_expert=False, fp8_expert_mlp=False, fp8_llm_mlp=False, vit_mlp_dtype=torch.float16),
+    dict(fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True, fused_prefill=True, vit_mlp_dtype=torch.bfloat16, vit_lowp_attn=True),
 ]
 
 
-@pytest.mark.parametrize("tiers", TIERS, ids=["eager", "attn", "full", "prefill", "full+prefill"])
+@pytest.mark.parametrize("tiers", TIERS, ids=["eager", "attn", "full", "prefill", "full+prefill", "vit-mlp-fp16", "everything"])
 def test_small_model_chunk_matches_oracle(tiers):
     cfg, sd, inp = cases.pi05_build(cases.PI05_CASES["small"])
-    want = _oracle_chunk(cfg, sd, inp, tiers["fp8_llm_mlp"], tiers["fp8_expert_mlp"])
+    vit = {k: v for k, v in tiers.items() if k.startswith("vit_")}
+    want = _oracle_chunk(cfg, sd, inp, tiers["fp8_llm_mlp"], tiers["fp8_expert_mlp"], **vit)
     got = _gpu_chunk(cfg, sd, inp, **tiers)
     err = float((got - want).abs().max())
     print(f"pi05 small {tiers}: max|err| = {err:.4g}, |chunk|max = {float(want.abs().max()):.3g}")
     assert torch.isfinite(got).all()
     assert err <= 1e-2 * max(1.0, float(want.abs().max()))
-    if not any(tiers.values()):
+    if not any(tiers.values()):  # all tiers off: also the committed golden chunk
         gold = torch.from_numpy(np.load(os.path.join(HERE, "golden", "pi05_small.npz"))["chunk"])[None]
         assert float((got - gold).abs().max()) <= 1e-2 * max(1.0, float(gold.abs().max()))
 
@@ -80,6 +83,27 @@ def test_zero_noise_chunk_within_bound():
     assert err <= 1e-2
 
 
+@pytest.mark.parametrize("vit", [dict(vit_mlp_dtype=torch.bfloat16), dict(vit_mlp_dtype=torch.float16), dict(vit_mlp_dtype=torch.bfloat16, vit_lowp_attn=True)])
+def test_vision_tower_drift_tiers_match_their_oracle(vit):
+    # the low-precision vision tiers against the oracle's restatement of the same tier, and against the
+    # fp32 tower (they are drift tiers: close, not equal)
+    from tybok_amd.policies.pi05.model import PI05Model
+
+    cfg, sd, inp = cases.pi05_build(cases.PI05_CASES["small"])
+    img = inp["images"][0] * 2.0 - 1.0
+    w = Weights(sd, frozenset())
+    with torch.no_grad():
+        want = O.embed_image(w, _shape(cfg, **vit), img)
+        full = O.embed_image(w, _shape(cfg), img)
+    with torch.inference_mode():
+        got = PI05Model(cfg, sd, "cuda", **vit).embed_image(img.cuda()).cpu()
+    scale = float(full.abs().max())
+    err, drift = float((got - want).abs().max()), float((want - full).abs().max())
+    print(f"pi05 vision {vit}: max|err| vs tier oracle {err:.4g}, tier drift vs fp32 {drift:.4g}, |emb|max {scale:.3g}")
+    assert err <= 2e-2 * max(1.0, scale)
+    assert drift <= 5e-2 * max(1.0, scale)
+
+
 @pytest.fixture(scope="module")
 def ckpt(tmp_path_factory):
     from tybok_amd.policies.synthetic import write_pi05_checkpoint
@@ -90,7 +114,7 @@ def ckpt(tmp_path_factory):
 def test_engine_api_and_graph_equals_eager(ckpt):
     from tybok_amd.registry import create_engine
 
-    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_flash_attn=True)
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_flash_attn=True, tl_fused_vit=True)
     eager = create_engine(ckpt, device="cuda", graph=False, warmup=False, **flags)
     graph = create_engine(ckpt, device="cuda", graph=True, warmup=True, **flags)
     assert graph.graph_enabled and list(graph._graph_runner.keys()) == [(2, 200)]
@@ -110,3 +134,6 @@ def test_engine_api_and_graph_equals_eager(ckpt):
         create_engine(ckpt, device="cuda", warmup=False, pad_free=True)
     with pytest.raises(NotImplementedError):
         create_engine(ckpt, device="cuda", warmup=False, rtc_config={"enabled": True})
+    with pytest.raises(ValueError):
+        create_engine(ckpt, device="cuda", warmup=False, vit_mlp_dtype="fp8")
+    assert create_engine(ckpt, device="cuda", warmup=False, vit_mlp_dtype="fp16").model.vit_mlp_dtype == torch.float16

@@ -10,9 +10,12 @@ flags wired to the HIP kernels:
 * ``tl_llm_flash_attn``   VLM prefill layers on the fused launches (norm + q|k|v + RoPE, attention
                           under the pad mask, o_proj + residual), K/V cache written by the projection
 
-The prefix-side tiers (``tl_fused_vit``, ``vit_mlp_dtype``, ``pad_free``,
-``skip_empty_images``), ``compile_model`` and Real-Time Chunking are not implemented here and are
-rejected when requested.
+* ``vit_mlp_dtype``       SigLIP fc1 / gelu / fc2 in fp16 or bf16, everything else fp32 (drift tier)
+* ``tl_fused_vit``        every linear of the SigLIP tower in bf16, scores / softmax / norms /
+                          residuals fp32 (drift tier; owns the MLP precision)
+
+``pad_free``, ``skip_empty_images``, ``compile_model`` and Real-Time Chunking are not implemented
+here and are rejected when requested.
 """
 
 from __future__ import annotations
@@ -69,8 +72,6 @@ class PI05Engine(PolicyEngine):
     _UNSUPPORTED_FLAGS = {
         "tl_llm_fused_attn": False,
         "tl_vit_oproj": False,
-        "tl_fused_vit": False,
-        "vit_mlp_dtype": None,
         "skip_empty_images": False,
         "pad_free": False,
         "pack_qkv": False,
@@ -118,8 +119,7 @@ class PI05Engine(PolicyEngine):
         reject_unsupported_flags(type(self), "pi05", kwargs)
         reject_unsupported_flags(
             type(self), "pi05",
-            dict(tl_fused_vit=tl_fused_vit, vit_mlp_dtype=vit_mlp_dtype,
-                 skip_empty_images=skip_empty_images, pad_free=pad_free),
+            dict(skip_empty_images=skip_empty_images, pad_free=pad_free),
         )  # fmt: skip
         if sampler != "euler":
             raise ValueError(f"sampler {sampler!r} not supported for pi05 (only 'euler')")
@@ -155,13 +155,24 @@ class PI05Engine(PolicyEngine):
             sd = random_state_dict(self.config, seed=int(self.config.random_init.get("seed", 0)))
         else:
             sd = load_state_dict(checkpoint_dir, {n: s for n, s, _, _ in parameter_inventory(self.config)}, remap=_KEY_REMAP)
+        # vision drift tiers (tybok/policies/pi05/engine.py:196-230): --vit-mlp-dtype converts fc1 / fc2 only;
+        # --tl-fused-vit runs every linear of the tower in bf16 (scores and softmax stay fp32) and owns
+        # the MLP precision, so --vit-mlp-dtype is inert under it
+        if vit_mlp_dtype not in (None, "fp16", "bf16"):
+            raise ValueError(f"--vit-mlp-dtype must be 'fp16' or 'bf16', got {vit_mlp_dtype!r}")
+        self.tl_fused_vit = bool(tl_fused_vit)
+        self.vit_mlp_dtype = None
+        if self.tl_fused_vit:
+            self.vit_mlp_dtype = torch.bfloat16
+        elif vit_mlp_dtype is not None:
+            self.vit_mlp_dtype = torch.float16 if vit_mlp_dtype == "fp16" else torch.bfloat16
         self.tl_fused_expert = bool(tl_fused_expert)
         self.tl_fp8_llm_mlp = bool(tl_fp8_llm_mlp)
         self.tl_fp8_expert_mlp = bool(tl_fp8_expert_mlp)
         self.model = PI05Model(
             self.config, sd, self.device,
             fused_expert=self.tl_fused_expert, fp8_expert_mlp=self.tl_fp8_expert_mlp, fp8_llm_mlp=self.tl_fp8_llm_mlp,
-            fused_prefill=bool(tl_llm_flash_attn),
+            fused_prefill=bool(tl_llm_flash_attn), vit_mlp_dtype=self.vit_mlp_dtype, vit_lowp_attn=self.tl_fused_vit,
         )  # fmt: skip
         del sd
 

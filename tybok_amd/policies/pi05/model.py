@@ -77,8 +77,12 @@ class PI05Model:
         fp8_expert_mlp: bool = False,
         fp8_llm_mlp: bool = False,
         fused_prefill: bool = False,
+        vit_mlp_dtype: torch.dtype | None = None,
+        vit_lowp_attn: bool = False,
     ):
         self.cfg = cfg
+        self.vit_mlp_dtype = vit_mlp_dtype
+        self.vit_lowp_attn = bool(vit_lowp_attn)
         self.device = torch.device(device)
         self.fused_expert = bool(fused_expert)
         self.fp8_expert_mlp = bool(fp8_expert_mlp)
@@ -130,6 +134,19 @@ class PI05Model:
             ]
         self.embed_scale = torch.tensor(self.vd["width"] ** 0.5, dtype=BF16, device=self.device)
         self.patch_w = self.p[VIS + "embeddings.patch_embedding.weight"].reshape(cfg.vision_hidden, -1)
+        # low-precision copies of the vision tower's linears (the drift tiers convert weights and bias)
+        self.vis_lowp: dict[str, tuple[torch.Tensor, torch.Tensor]] = {}
+        for i in range(cfg.vision_layers):
+            lp = f"{VIS}encoder.layers.{i}."
+            if self.vit_mlp_dtype is not None:
+                for n in ("mlp.fc1", "mlp.fc2"):
+                    self.vis_lowp[lp + n] = (self.p[lp + n + ".weight"].to(self.vit_mlp_dtype), self.p[lp + n + ".bias"].to(self.vit_mlp_dtype))
+            if self.vit_lowp_attn:
+                self.vis_lowp[lp + "self_attn.qkv"] = (
+                    torch.cat([self.p[lp + f"self_attn.{n}_proj.weight"] for n in "qkv"], dim=0).to(BF16),
+                    torch.cat([self.p[lp + f"self_attn.{n}_proj.bias"] for n in "qkv"], dim=0).to(BF16),
+                )
+                self.vis_lowp[lp + "self_attn.out_proj"] = (self.p[lp + "self_attn.out_proj.weight"].to(BF16), self.p[lp + "self_attn.out_proj.bias"].to(BF16))
         self.set_num_steps(cfg.num_steps)
 
     def lin(self, name: str, x: torch.Tensor) -> torch.Tensor:
@@ -181,14 +198,26 @@ class PI05Model:
         for i in range(cfg.vision_layers):
             lp = f"{VIS}encoder.layers.{i}."
             h = F.layer_norm(x, (vh,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], EPS)
-            q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
-            k = self.lin(lp + "self_attn.k_proj", h).view(b, -1, heads, hd).transpose(1, 2)
-            v = self.lin(lp + "self_attn.v_proj", h).view(b, -1, heads, hd).transpose(1, 2)
-            att = torch.softmax(torch.matmul(q, k.transpose(2, 3)) * hd**-0.5, dim=-1)
-            a = torch.matmul(att, v).transpose(1, 2).reshape(b, -1, vh)
-            x = x + self.lin(lp + "self_attn.out_proj", a)
+            if self.vit_lowp_attn:
+                # bf16 projections (one packed q|k|v GEMM), fp32 scores / softmax / P.V
+                qkv = F.linear(h.to(BF16), *self.vis_lowp[lp + "self_attn.qkv"]).view(b, -1, 3, heads, hd).permute(2, 0, 3, 1, 4).float()
+                att = torch.softmax(torch.matmul(qkv[0], qkv[1].transpose(2, 3)) * hd**-0.5, dim=-1)
+                a = torch.matmul(att, qkv[2]).to(BF16).transpose(1, 2).reshape(b, -1, vh)
+                x = x + F.linear(a, *self.vis_lowp[lp + "self_attn.out_proj"]).float()
+            else:
+                q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
+                k = self.lin(lp + "self_attn.k_proj", h).view(b, -1, heads, hd).transpose(1, 2)
+                v = self.lin(lp + "self_attn.v_proj", h).view(b, -1, heads, hd).transpose(1, 2)
+                att = torch.softmax(torch.matmul(q, k.transpose(2, 3)) * hd**-0.5, dim=-1)
+                a = torch.matmul(att, v).transpose(1, 2).reshape(b, -1, vh)
+                x = x + self.lin(lp + "self_attn.out_proj", a)
             h = F.layer_norm(x, (vh,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS)
-            x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
+            if self.vit_mlp_dtype is not None:
+                # MLP-only low precision: fc1, gelu and fc2 in that dtype, cast at the boundary
+                m = F.gelu(F.linear(h.to(self.vit_mlp_dtype), *self.vis_lowp[lp + "mlp.fc1"]), approximate="tanh")
+                x = x + F.linear(m, *self.vis_lowp[lp + "mlp.fc2"]).float()
+            else:
+                x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
         x = F.layer_norm(x, (vh,), p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], EPS)
         return self.lin(PROJ, x)
 
