@@ -67,8 +67,13 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   constexpr int DS = D / 16;                 // k steps of Q.K^T
   constexpr int PL = SPLIT ? 2 : 1;          // operand planes (hi, lo)
   constexpr int PF = (NWV > 4 || D > 128) ? 1 : 2;  // key tiles in flight per wave
-  __shared__ __align__(16) f32x4 red[2][kNW][4][64];
+  // D = 256: the query tile (the same for every wave of the block) lives in LDS instead of 64
+  // registers per lane -- with it in registers the kernel spills to scratch
+  constexpr bool QLDS = D >= 256;
+  constexpr int QPITCH = D * 2 + 16;         // bytes; 16-byte operand reads of 32 rows stay conflict-free
+  __shared__ __align__(16) f32x4 red[DT][kNW][4][64];  // every wave's partial output tiles, exchanged at once
   __shared__ float st_m[kNW][32], st_l[kNW][32];
+  __shared__ __align__(16) unsigned char qs[QLDS ? 32 * QPITCH : 16];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keeps tile indices scalar
@@ -143,12 +148,22 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   };
 
   // ---- Q as B operand, resident in registers; the first tiles' loads go out with it ----
-  bf16x8 qf[DS];
+  bf16x8 qf[QLDS ? 1 : DS];
   Stage stg[PF];
-  {
+  constexpr int QPT = QLDS ? 32 * (D / 8) / (kNW * 64) : 1;  // 16-byte pieces of the query tile per thread
+  i32x4 qraw[QPT];
+  if (QLDS) {
+#pragma unroll
+    for (int i = 0; i < QPT; ++i) {
+      const int p = threadIdx.x + i * kNW * 64;
+      int row = mtile * 32 + p / (D / 8);
+      if (row > a.M - 1) row = a.M - 1;
+      qraw[i] = *(const i32x4*)(a.q + (size_t)row * a.q_sm + (size_t)h * a.q_sh + (p % (D / 8)) * 8);
+    }
+  } else {
     const u16* qp = a.q + (size_t)(q_ok ? qi : a.M - 1) * a.q_sm + (size_t)h * a.q_sh + 8 * half;
 #pragma unroll
-    for (int s = 0; s < DS; ++s) qf[s] = as_bf16x8(*(const i32x4*)(qp + 16 * s));
+    for (int s = 0; s < DS; ++s) qf[QLDS ? 0 : s] = as_bf16x8(*(const i32x4*)(qp + 16 * s));
   }
   // tiles of this wave: t_lo + wave + kNW * i, i < nt_w; indices past the end are clamped to a valid
   // tile so that every prefetch is unconditional (never processed)
@@ -159,6 +174,15 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   };
 #pragma unroll
   for (int p = 0; p < PF; ++p) load(stg[p], tile_of(p));
+  if (QLDS) {
+#pragma unroll
+    for (int i = 0; i < QPT; ++i) {
+      const int p = threadIdx.x + i * kNW * 64;
+      *(i32x4*)(qs + (p / (D / 8)) * QPITCH + (p % (D / 8)) * 16) = qraw[i];
+    }
+    __syncthreads();
+  }
+  TA_MARK(1);
 
   f32x16 o[DT];
 #pragma unroll
@@ -178,7 +202,10 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
 #pragma unroll
     for (int s = 0; s < DS; ++s)
 #pragma unroll
-      for (int pl = 0; pl < PL; ++pl) sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(st.k[pl][s]), qf[s], sT, 0, 0, 0);
+      for (int pl = 0; pl < PL; ++pl) {
+        const bf16x8 qv = QLDS ? as_bf16x8(*(const i32x4*)(qs + l32 * QPITCH + (16 * s + 8 * half) * 2)) : qf[QLDS ? 0 : s];
+        sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(st.k[pl][s]), qv, sT, 0, 0, 0);
+      }
 
     // ---- scale, mask, online softmax (one query column per lane) ----
     // Register i of this lane holds key kl(i) = 16*(i/8) + 8*half + i%8 of the tile.  Visibility and
@@ -266,21 +293,30 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   };
 
   {
-    // software pipeline over this wave's tiles: the steady-state loop has no branch (precise
-    // wait counts), the tail (< 2*PF tiles) uses wave-uniform conditions
-    int i = 0;
-    for (; i + 2 * PF <= nt_w; i += PF) {
-#pragma unroll
-      for (int p = 0; p < PF; ++p) {
-        process(stg[p], tile_of(i + p));
-        load(stg[p], tile_of(i + p + PF));
+    if (D > 128) {
+      // one tile in flight and one copy of the tile code: with the pipelined form below the
+      // register allocator spills this head size to scratch
+      for (int i = 0; i < nt_w; ++i) {
+        process(stg[0], tile_of(i));
+        if (i + 1 < nt_w) load(stg[0], tile_of(i + 1));
       }
-    }
+    } else {
+      // software pipeline over this wave's tiles: the steady-state loop has no branch (precise
+      // wait counts), the tail (< 2*PF tiles) uses wave-uniform conditions
+      int i = 0;
+      for (; i + 2 * PF <= nt_w; i += PF) {
 #pragma unroll
-    for (int q = 0; q < 2 * PF - 1; ++q) {
-      if (i + q < nt_w) {
-        process(stg[q % PF], tile_of(i + q));
-        if (i + q + PF < nt_w) load(stg[q % PF], tile_of(i + q + PF));
+        for (int p = 0; p < PF; ++p) {
+          process(stg[p], tile_of(i + p));
+          load(stg[p], tile_of(i + p + PF));
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < 2 * PF - 1; ++q) {
+        if (i + q < nt_w) {
+          process(stg[q % PF], tile_of(i + q));
+          if (i + q + PF < nt_w) load(stg[q % PF], tile_of(i + q + PF));
+        }
       }
     }
   }
@@ -299,31 +335,33 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   float ew[kNW];
   float bm = -INFINITY, bl = 0.f;  // block-level (m, l) of this lane's query
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) {
+  for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
       f32x4 v = {o[dt][4 * gq], o[dt][4 * gq + 1], o[dt][4 * gq + 2], o[dt][4 * gq + 3]};
-      red[dt & 1][wave][gq][lane] = v;
+      red[dt][wave][gq][lane] = v;
     }
-    __syncthreads();
-    if (dt == 0) {
-      float mw[kNW];
+  __syncthreads();
+  {
+    float mw[kNW];
 #pragma unroll
-      for (int w = 0; w < kNW; ++w) {
-        mw[w] = st_m[w][l32];
-        bm = fmaxf(bm, mw[w]);
-      }
-#pragma unroll
-      for (int w = 0; w < kNW; ++w) {
-        ew[w] = (mw[w] == -INFINITY) ? 0.f : __expf(mw[w] - bm);
-        bl += st_l[w][l32] * ew[w];
-      }
+    for (int w = 0; w < kNW; ++w) {
+      mw[w] = st_m[w][l32];
+      bm = fmaxf(bm, mw[w]);
     }
+#pragma unroll
+    for (int w = 0; w < kNW; ++w) {
+      ew[w] = (mw[w] == -INFINITY) ? 0.f : __expf(mw[w] - bm);
+      bl += st_l[w][l32] * ew[w];
+    }
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
     if (owner) {
-      sum = red[dt & 1][0][wg][lane] * ew[0];
+      sum = red[dt][0][wg][lane] * ew[0];
 #pragma unroll
-      for (int w = 1; w < kNW; ++w) sum += red[dt & 1][w][wg][lane] * ew[w];
+      for (int w = 1; w < kNW; ++w) sum += red[dt][w][wg][lane] * ew[w];
     }
     own[dt] = sum;
   }
@@ -369,8 +407,10 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   if (!s_last || !owner) return;
   if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
-  constexpr int MAXS = 8;  // the host never asks for more kv splits
+  constexpr int MAXS = D > 128 ? 7 : 8;  // the host never asks for more kv splits
   const float* pblk = a.partial + (size_t)blk_lin * a.kv_splits * PSTRIDE;
+  // every read of the hand-off goes out before the first one is consumed (the read-back costs round
+  // trips, not bandwidth): the statistics first, then the partial tiles in batches of DTB d tiles
   float ms[MAXS], ls[MAXS], es[MAXS];
 #pragma unroll
   for (int s = 0; s < MAXS; ++s) {
@@ -378,6 +418,21 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
     ms[s] = ld_agent(pblk + (size_t)sc * PSTRIDE + l32);
     ls[s] = ld_agent(pblk + (size_t)sc * PSTRIDE + 32 + l32);
   }
+  constexpr int DTB = DT >= 4 ? 4 : DT;
+  unsigned long long raw[DTB][MAXS][2];
+  auto fetch = [&](int d0) {
+#pragma unroll
+    for (int dd = 0; dd < DTB; ++dd)
+#pragma unroll
+      for (int s = 0; s < MAXS; ++s) {
+        const int sc = s < a.kv_splits ? s : a.kv_splits - 1;
+        const unsigned long long* src = (const unsigned long long*)(pblk + (size_t)sc * PSTRIDE + 64) +
+                                        (size_t)(d0 + dd) * 512 + ((size_t)wave * 64 + lane) * 2;
+        raw[dd][s][0] = ld_agent64(src);
+        raw[dd][s][1] = ld_agent64(src + 1);
+      }
+  };
+  fetch(0);
   float mt = -INFINITY;
 #pragma unroll
   for (int s = 0; s < MAXS; ++s)
@@ -390,34 +445,25 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   }
   TA_MARK(5);
   const float inv = 1.0f / lt;
-  // several d tiles' partials in flight together: the read-back costs round trips, not bandwidth
-  constexpr int DTB = DT >= 4 ? 4 : DT;
 #pragma unroll
   for (int d0 = 0; d0 < DT; d0 += DTB) {
-    unsigned long long raw[DTB][MAXS][2];
-#pragma unroll
-    for (int dd = 0; dd < DTB; ++dd)
-#pragma unroll
-      for (int s = 0; s < MAXS; ++s) {
-        const int sc = s < a.kv_splits ? s : a.kv_splits - 1;
-        const unsigned long long* src = (const unsigned long long*)(pblk + (size_t)sc * PSTRIDE + 64) +
-                                        (size_t)(d0 + dd) * 512 + ((size_t)wave * 64 + lane) * 2;
-        raw[dd][s][0] = ld_agent64(src);
-        raw[dd][s][1] = ld_agent64(src + 1);
-      }
+    f32x4 acc[DTB];
 #pragma unroll
     for (int dd = 0; dd < DTB; ++dd) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      acc[dd] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < MAXS; ++s) {
         if (s < a.kv_splits) {
           f32x4 v = {__uint_as_float((unsigned)raw[dd][s][0]), __uint_as_float((unsigned)(raw[dd][s][0] >> 32)),
                      __uint_as_float((unsigned)raw[dd][s][1]), __uint_as_float((unsigned)(raw[dd][s][1] >> 32))};
-          acc += v * es[s];
+          acc[dd] += v * es[s];
         }
       }
-      if (q_ok) *(i32x2*)(op + (d0 + dd) * 32) = pack_bf16x4(acc * inv);
     }
+    if (d0 + DTB < DT) fetch(d0 + DTB);  // the next batch is on its way while this one is stored
+#pragma unroll
+    for (int dd = 0; dd < DTB; ++dd)
+      if (q_ok) *(i32x2*)(op + (d0 + dd) * 32) = pack_bf16x4(acc[dd] * inv);
   }
   TA_MARK(6);
 }

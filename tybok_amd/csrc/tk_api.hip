@@ -2,6 +2,7 @@
 // Host-side argument checks, launch geometry, workspace carving.  No allocation, no sync.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "../../include/tybok_hip.h"
@@ -137,7 +138,10 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
 
   const int cus = device_cus();
   const bool has_norm = e.norm_w || e.ada_scale;
-  if (!e.w16 && !rope && !e.x_f32 && a.vec && M > 64 &&
+  // (from 256 rows on, or when its 128 x 256 tiles already fill the device; below that the skinny
+  // kernel's finer blocks and K splits win)
+  const int wide_blocks = ((a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols()) * ((M + tk_wide_rows() - 1) / tk_wide_rows());
+  if (!e.w16 && !rope && !e.x_f32 && a.vec && (M >= 256 || (M > 64 && wide_blocks >= cus)) &&
       (!has_norm || (ws && ws_bytes >= kNormOff + (size_t)M * K * 2 && (size_t)M * K * 2 <= kNormBytes))) {
     // many rows: MFMA-bound kernel with a 128 x 256 block tile
     if (has_norm) {
@@ -158,7 +162,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
       a.norm_w = nullptr;
       a.ada_scale = a.ada_shift = nullptr;
     }
-    const int blocks0 = ((a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols()) * ((M + tk_wide_rows() - 1) / tk_wide_rows());
+    const int blocks0 = wide_blocks;
     int ks = split_k;
     if (ks <= 0) {
       // fill the device once; a split keeps at least 16 k tiles and its partials must fit
@@ -475,9 +479,15 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   const int waves = tk_attn_waves(D, split ? 1 : 0, ntiles);
   int splits = (ntiles + waves - 1) / waves;
   if (splits < 1) splits = 1;
-  if (splits > 8) splits = 8;
+  if (splits > (D > 128 ? 7 : 8)) splits = D > 128 ? 7 : 8;
   // many query tiles already fill the device: keep whole key ranges in one block (no partials)
   while (splits > 1 && H * mtiles * splits > 2 * device_cus()) --splits;
+#ifdef TK_PHASE_TIMING
+  if (const char* ev = getenv("TK_ATTN_SPLITS")) {  // development aid, never in the shipped build
+    const int v = atoi(ev);
+    if (v >= 1 && v <= 8 && D == 256) splits = v;
+  }
+#endif
   a.kv_splits = splits;
   a.tile_q = ntiles / splits;
   a.tile_r = ntiles % splits;
