@@ -88,6 +88,41 @@ def gemm_launch_us(m: int, k: int, n: int, launches: int = 100, reps: int = 10, 
     return e0.elapsed_time(e1) * 1e3 / (reps * launches)
 
 
+def ffn_launch_us(m: int, k: int, i: int, launches: int = 10, reps: int = 5) -> float:
+    """Average duration (us) of one fp8-weight GeGLU FFN (gate/up + down) at many rows: the VLM prefill shape."""
+    import torch
+
+    from oracle.inputs import ffn_case
+    from tybok_amd import ops as tk
+
+    x, wg8, sg, wu8, su, wd8, sd = ffn_case(m, k, i, seed=0)
+    wgu = tk.pack_fp8_gate_up(wg8.cuda(), sg, wu8.cuda(), su)
+    wd = tk.pack_fp8_weight(wd8.cuda(), sd)
+    xc = x.cuda()
+    out = torch.empty(m, k, dtype=torch.bfloat16, device="cuda")
+    ws = tk.Workspace()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(3):
+            tk.fp8w_gated_ffn(xc, wgu, wd, "gelu_tanh", out=out, ws=ws)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
+        for _ in range(launches):
+            tk.fp8w_gated_ffn(xc, wgu, wd, "gelu_tanh", out=out, ws=ws)
+    spin_up(60.0)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * launches)
+
+
 def attn_launch_us(launches: int = 100, reps: int = 10) -> float:
     """Average duration (us) of one action-expert attention launch (50 queries, 241 prefix + 50
     own keys, 15/5 heads of 64, causal suffix) inside a replayed graph."""
@@ -195,6 +230,7 @@ def main() -> None:
     ap.add_argument("--gemm-only", action="store_true", help="only the roofline GEMM loop plus a plain copy of known size (for rocprofv3 runs)")
     ap.add_argument("--gemm-shape", type=int, nargs=3, metavar=("M", "K", "N"), default=(50, 2048, 16384), help="shape of the --gemm-only loop")
     ap.add_argument("--attn-only", action="store_true", help="only the action-expert attention loop (for rocprofv3 runs)")
+    ap.add_argument("--ffn-only", action="store_true", help="only the many-row (M=712) fp8 GeGLU FFN loop (for rocprofv3 runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is batch-1 and single-device (--gpus must be 1)")
@@ -217,6 +253,11 @@ def main() -> None:
         gm, gk, gn = args.gemm_shape
         us = gemm_launch_us(gm, gk, gn, launches=20, reps=args.steps)
         print(json.dumps({"gemm_only": {"M": gm, "K": gk, "N": gn, "us": round(us, 2), "GBps": round(bytes_gemm(gm, gk, gn) / us / 1e3, 1)}}), flush=True)
+        return
+    if args.ffn_only:
+        spin_up()
+        us = ffn_launch_us(712, 2048, 16384, launches=5, reps=args.steps)
+        print(json.dumps({"ffn_only": {"M": 712, "K": 2048, "I": 16384, "us": round(us, 1), "TFLOPs": round(6.0 * 712 * 2048 * 16384 / us / 1e6, 1)}}), flush=True)
         return
     if args.attn_only:
         spin_up()
@@ -247,6 +288,7 @@ def main() -> None:
         ckpt5 = write_pi05_checkpoint(os.path.join(tmp, "pi05"), cameras=2, seed=0)
         flags5 = {k: v for k, v in flags.items() if k not in ("tl_llm_fused_attn", "tl_vit_oproj")}  # SmolVLA-only tiers
         flags5["tl_llm_flash_attn"] = True  # pi0.5's name for the fused prefill
+        flags5["tl_fused_vit"] = True  # SigLIP linears in bf16 (the reference's drift tier of the same name)
         eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **flags5)
         frame5 = device_frame(eng5, 2)
         s5, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
@@ -279,6 +321,17 @@ def main() -> None:
         with open(traffic_file, encoding="utf-8") as f:
             roofline["traffic"] = json.load(f).get("hbm_bytes_per_launch")
 
+    # ---- many-row (prefill) FFN: MFMA-bound, priced against the dense bf16 peak ----
+    fm, fk, fi = 712, 2048, 16384
+    f_us = ffn_launch_us(fm, fk, fi)
+    f_tflops = 6.0 * fm * fk * fi / f_us / 1e6
+    prefill_ffn = {
+        "shape": {"M": fm, "K": fk, "I": fi},
+        "us": round(f_us, 1),
+        "TFLOPs": round(f_tflops, 1),
+        "frac_of_bf16_mfma_peak": round(f_tflops / 2500.0, 4),
+    }
+
     cpu = None if args.skip_cpu else cpu_baseline_smolvla(3)
 
     p50 = float(np.percentile(samples3, 50))
@@ -304,7 +357,9 @@ def main() -> None:
         "smolvla_2cam_p50_ms": round(float(np.percentile(samples2, 50)), 3),
         "smolvla_3cam_host_inputs_p50_ms": round(float(np.percentile(samples_host, 50)), 3),
         "pi05_2cam_p50_ms": None if pi05_p50 is None else round(pi05_p50, 3),
+        "pi05_tiers": "tl_fused_expert, tl_fp8_expert_mlp, tl_fp8_llm_mlp, tl_llm_flash_attn, tl_fused_vit",
         "gemm_sweep_M50": sweep,
+        "pi05_prefill_ffn_M712": prefill_ffn,
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
