@@ -146,6 +146,8 @@ class SmolVLAEngine(PolicyEngine):
             self.config, sd, self.device,
             fused_expert=self.tl_fused_expert, fp8_expert_mlp=self.tl_fp8_expert_mlp, fp8_llm_mlp=self.tl_fp8_llm_mlp,
             fused_prefill=self.tl_llm_fused_attn, fused_vit=self.tl_vit_oproj,
+            # graph mode only, like the reference (smolvla/engine.py:229-237); needs both fused tiers
+            overlap=bool(overlap) and bool(graph) and str(self.device).startswith("cuda"),
         )  # fmt: skip
         del sd
 
@@ -162,7 +164,7 @@ class SmolVLAEngine(PolicyEngine):
 
         self.graph_requested = bool(graph)
         self.graph_enabled = self.graph_requested and str(self.device).startswith("cuda")
-        self.overlap = False  # prefill x step-0 two-stream overlap is not implemented; accepted, inert
+        self.overlap = self.model.overlap  # step 0 of the Euler loop hidden inside the prefill (two streams)
         self._sess = CaptureSession(self.device)
         self._graph_runner = GraphRunner(self._capture_graph, self.device, label="smolvla graph", logger=log)
         self._graph_fallback_warned = False

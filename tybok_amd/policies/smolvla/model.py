@@ -104,6 +104,7 @@ class SmolVLAModel:
         fp8_llm_mlp: bool = False,
         fused_prefill: bool = False,
         fused_vit: bool = False,
+        overlap: bool = False,
     ):
         assert cfg.vlm_config is not None
         self.cfg = cfg
@@ -126,6 +127,12 @@ class SmolVLAModel:
         self.vlm_mlp = [GatedMLP(state_dict, f"{TXT}layers.{i}.mlp.", self.device, self.fp8_llm_mlp) for i in range(self.num_layers)]
         self.exp_mlp = [GatedMLP(state_dict, f"{EXP}layers.{i}.mlp.", self.device, self.fp8_expert_mlp) for i in range(cfg.n_expert_layers)]
         self.ws = tk.default_workspace(self.device) if self.use_hip else None
+        # prefill x step-0 overlap (flow_matching.py:455-531): step-0 expert layer i runs on a second
+        # stream as soon as prefill layer i has produced its K/V.  Kernels that may run at the same
+        # time must not share split-K partials / counters: the side stream has its own workspace.
+        self.overlap = bool(overlap) and self.fused_prefill and self.fused_expert
+        self.side_stream = torch.cuda.Stream(self.device) if self.overlap else None
+        self.ws_side = tk.Workspace(self.device) if self.overlap else None
         if self.fused_prefill:
             self.vlm_qkv, self.vlm_o = self._pack_attention_weights(TXT, lambda i: False)
         if self.fused_vit:
@@ -306,52 +313,65 @@ class SmolVLAModel:
             hidden = self._layer_tail(lp, self.vlm_mlp[i], att, hidden)
         return keys, values
 
-    def prefill_fused(self, embs, pad_masks, att_masks):
-        """VLM prefill on the fused launches (per layer: norm + q|k|v + RoPE, attention under the
-        2-D prefix mask, o_proj + residual, gated FFN) -> ``(K, V, V^T)``: K / V are ``[layers, 1, P,
-        G, D]`` views of the per-layer projection outputs, V^T ``[layers, G, D, P rounded up to 32]``
-        is the attention kernel's value layout (written by the projection epilogue)."""
+    def _prefill_setup(self, embs, pad_masks, att_masks) -> dict:
+        """Per-request operands of the fused prefill: 2-D visibility bytes, positions, output buffers."""
         p_len = embs.shape[1]
         p_pad = (p_len + 31) // 32 * 32
-        h_q, h_kv, d = self.heads, self.kv_heads, self.head_dim
-        nq, nkv = h_q * d, h_kv * d
+        nq, nkv = self.heads * self.head_dim, self.kv_heads * self.head_dim
         mask2d = torch.zeros(p_len, p_pad, dtype=torch.uint8, device=self.device)
         mask2d[:, :p_len] = self.make_att_2d_masks(pad_masks, att_masks)[0]
         pos32 = (torch.cumsum(pad_masks, dim=1) - 1)[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
         qkv_all = torch.empty(self.num_layers, p_len, nq + 2 * nkv, dtype=BF16, device=self.device)
         vt_all = torch.zeros(self.num_layers, nkv, p_pad, dtype=BF16, device=self.device)
+        return dict(p_len=p_len, p_pad=p_pad, mask2d=mask2d, pos32=pos32, qkv_all=qkv_all, vt_all=vt_all)
+
+    def _prefill_layer_fused(self, i: int, hidden: torch.Tensor, c: dict) -> torch.Tensor:
+        """One VLM layer on the fused launches: norm + q|k|v + RoPE, attention under the 2-D prefix
+        mask, o_proj + residual, gated FFN.  Fills ``qkv_all[i]`` / ``vt_all[i]`` (the layer's K/V cache)."""
+        h_q, h_kv, d = self.heads, self.kv_heads, self.head_dim
+        nq, nkv = h_q * d, h_kv * d
+        p_len, p_pad = c["p_len"], c["p_pad"]
+        lp = f"{TXT}layers.{i}."
+        qkv = tk.bf16w_linear(
+            hidden, self.vlm_qkv[i], norm_w=self.p[lp + "input_layernorm.weight"], eps=self.eps, rope=self.rope_tables,
+            rope_pos=c["pos32"], rope_cols=nq + nkv, vt_out=c["vt_all"][i], vt_col0=nq + nkv, out=c["qkv_all"][i], ws=self.ws,
+        )  # fmt: skip
+        cache = tk.PrefixKV(qkv[:, nq : nq + nkv].view(p_len, h_kv, d), c["vt_all"][i].view(h_kv, d, p_pad))
+        att = tk.expert_attn(qkv[:, :nq].view(p_len, h_q, d), cache, None, None, tk.MASK_NONE, mask2d=c["mask2d"], ws=self.ws)
+        out = tk.bf16w_linear(att, self.vlm_o[i], resid=hidden, ws=self.ws)
+        mlp = self.vlm_mlp[i]
+        post_w = self.p[lp + "post_attention_layernorm.weight"]
+        if mlp.fp8:
+            return tk.fp8w_gated_ffn(out, mlp.wgu, mlp.wd, mlp.act, resid=out, norm_w=post_w, eps=self.eps, ws=self.ws)
+        return mlp(rms_norm(out, post_w, self.eps)[None], out[None])[0]
+
+    def _prefill_views(self, c: dict):
+        """``(K, V, V^T)`` of the fused prefill: K / V ``[layers, 1, P, G, D]`` views of the projection
+        outputs, V^T ``[layers, G, D, P rounded up to 32]`` (the attention kernel's value layout)."""
+        h_kv, d = self.kv_heads, self.head_dim
+        nq, nkv = self.heads * d, h_kv * d
+        keys = c["qkv_all"][:, None, :, nq : nq + nkv].unflatten(-1, (h_kv, d))
+        values = c["qkv_all"][:, None, :, nq + nkv :].unflatten(-1, (h_kv, d))
+        return keys, values, c["vt_all"].view(self.num_layers, h_kv, d, c["p_pad"])
+
+    def prefill_fused(self, embs, pad_masks, att_masks):
+        """VLM prefill on the fused launches -> ``(K, V, V^T)`` (see ``_prefill_views``)."""
+        c = self._prefill_setup(embs, pad_masks, att_masks)
         hidden = embs[0]
         for i in range(self.num_layers):
-            lp = f"{TXT}layers.{i}."
-            qkv = tk.bf16w_linear(
-                hidden, self.vlm_qkv[i], norm_w=self.p[lp + "input_layernorm.weight"], eps=self.eps, rope=self.rope_tables,
-                rope_pos=pos32, rope_cols=nq + nkv, vt_out=vt_all[i], vt_col0=nq + nkv, out=qkv_all[i], ws=self.ws,
-            )  # fmt: skip
-            cache = tk.PrefixKV(qkv[:, nq : nq + nkv].view(p_len, h_kv, d), vt_all[i].view(h_kv, d, p_pad))
-            att = tk.expert_attn(qkv[:, :nq].view(p_len, h_q, d), cache, None, None, tk.MASK_NONE, mask2d=mask2d, ws=self.ws)
-            out = tk.bf16w_linear(att, self.vlm_o[i], resid=hidden, ws=self.ws)
-            mlp = self.vlm_mlp[i]
-            post_w = self.p[lp + "post_attention_layernorm.weight"]
-            if mlp.fp8:
-                hidden = tk.fp8w_gated_ffn(out, mlp.wgu, mlp.wd, mlp.act, resid=out, norm_w=post_w, eps=self.eps, ws=self.ws)
-            else:
-                hidden = mlp(rms_norm(out, post_w, self.eps)[None], out[None])[0]
-        keys = qkv_all[:, None, :, nq : nq + nkv].unflatten(-1, (h_kv, d))
-        values = qkv_all[:, None, :, nq + nkv :].unflatten(-1, (h_kv, d))
-        return keys, values, vt_all.view(self.num_layers, h_kv, d, p_pad)
+            hidden = self._prefill_layer_fused(i, hidden, c)
+        return self._prefill_views(c)
+
+    def _expert_prefix_kv_layer(self, i: int, keys_i, values_i):
+        lp = f"{EXP}layers.{i}.self_attn."
+        b, length = keys_i.shape[0], keys_i.shape[1]
+        ek = self.lin(lp + "k_proj", keys_i.float().reshape(b, length, -1)).view(b, length, -1, self.head_dim)
+        ev = self.lin(lp + "v_proj", values_i.float().reshape(b, length, -1)).view(b, length, -1, self.head_dim)
+        return ek, ev
 
     def expert_prefix_kv(self, keys, values):
         """fp32 expert K/V projections of the prefix for the cross layers (flow_matching.py:553-578)."""
-        out = {}
-        for i in range(self.num_layers):
-            if not self.cfg.is_cross_layer(i):
-                continue
-            lp = f"{EXP}layers.{i}.self_attn."
-            b, length = keys.shape[1], keys.shape[2]
-            ek = self.lin(lp + "k_proj", keys[i].float().reshape(b, length, -1)).view(b, length, -1, self.head_dim)
-            ev = self.lin(lp + "v_proj", values[i].float().reshape(b, length, -1)).view(b, length, -1, self.head_dim)
-            out[i] = (ek, ev)
-        return out
+        return {i: self._expert_prefix_kv_layer(i, keys[i], values[i]) for i in range(self.num_layers) if self.cfg.is_cross_layer(i)}
 
     # ------------------------------------------------------------------ denoising
     def embed_suffix(self, x_t: torch.Tensor, time_emb: torch.Tensor) -> torch.Tensor:
@@ -381,33 +401,35 @@ class SmolVLAModel:
                 caches.append(tk.prepare_prefix_kv(keys[i, 0], values[i, 0]))
         return caches
 
-    def _denoise_step_fused(self, prefix_pad, caches, hidden, pos32, pos0_32):
-        """Expert stack on the fused launches; ``hidden [S, E]`` fp32 in, bf16 out."""
+    def _denoise_layer_fused(self, i: int, hidden: torch.Tensor, cache, pad, pos32, pos0_32, ws) -> torch.Tensor:
+        """Expert layer ``i`` on the fused launches (``hidden [S, E]``: fp32 into layer 0, bf16 after)."""
         h_q, h_kv, d = self.heads, self.kv_heads, self.head_dim
         nq, nkv = h_q * d, h_kv * d
         s = hidden.shape[0]
-        pad = prefix_pad[0]
+        lp = f"{EXP}layers.{i}."
+        cross = self.cfg.is_cross_layer(i)
+        qkv = tk.bf16w_linear(
+            hidden, self.exp_qkv[i], norm_w=self.p[lp + "input_layernorm.weight"], eps=self.eps, rope=self.rope_tables,
+            rope_pos=pos0_32 if cross else pos32, rope_cols=nq if cross else nq + nkv,
+            vt_out=None if cross else self.vt_suf.view(nkv, -1), vt_col0=nq + nkv, ws=ws,
+        )  # fmt: skip
+        q = qkv[:, :nq].view(s, h_q, d)
+        if cross:
+            att = tk.expert_attn(q, cache, None, pad, tk.MASK_NONE, ws=ws)
+        else:
+            suffix = tk.SuffixKV(qkv[:, nq : nq + nkv].view(s, h_kv, d), self.vt_suf)
+            att = tk.expert_attn(q, cache, suffix, pad, tk.MASK_CAUSAL, ws=ws)
+        out = tk.bf16w_linear(att, self.exp_o[i], resid=hidden, ws=ws)
+        mlp = self.exp_mlp[i]
+        post_w = self.p[lp + "post_attention_layernorm.weight"]
+        if mlp.fp8:
+            return tk.fp8w_gated_ffn(out, mlp.wgu, mlp.wd, mlp.act, resid=out, norm_w=post_w, eps=self.eps, ws=ws)
+        return mlp(rms_norm(out, post_w, self.eps)[None], out[None])[0]
+
+    def _denoise_step_fused(self, prefix_pad, caches, hidden, pos32, pos0_32):
+        """Expert stack on the fused launches; ``hidden [S, E]`` fp32 in, bf16 out."""
         for i in range(self.num_layers):
-            lp = f"{EXP}layers.{i}."
-            cross = self.cfg.is_cross_layer(i)
-            qkv = tk.bf16w_linear(
-                hidden, self.exp_qkv[i], norm_w=self.p[lp + "input_layernorm.weight"], eps=self.eps, rope=self.rope_tables,
-                rope_pos=pos0_32 if cross else pos32, rope_cols=nq if cross else nq + nkv,
-                vt_out=None if cross else self.vt_suf.view(nkv, -1), vt_col0=nq + nkv, ws=self.ws,
-            )  # fmt: skip
-            q = qkv[:, :nq].view(s, h_q, d)
-            if cross:
-                att = tk.expert_attn(q, caches[i], None, pad, tk.MASK_NONE, ws=self.ws)
-            else:
-                suffix = tk.SuffixKV(qkv[:, nq : nq + nkv].view(s, h_kv, d), self.vt_suf)
-                att = tk.expert_attn(q, caches[i], suffix, pad, tk.MASK_CAUSAL, ws=self.ws)
-            out = tk.bf16w_linear(att, self.exp_o[i], resid=hidden, ws=self.ws)
-            mlp = self.exp_mlp[i]
-            post_w = self.p[lp + "post_attention_layernorm.weight"]
-            if mlp.fp8:
-                hidden = tk.fp8w_gated_ffn(out, mlp.wgu, mlp.wd, mlp.act, resid=out, norm_w=post_w, eps=self.eps, ws=self.ws)
-            else:
-                hidden = mlp(rms_norm(out, post_w, self.eps)[None], out[None])[0]
+            hidden = self._denoise_layer_fused(i, hidden, caches[i], prefix_pad[0], pos32, pos0_32, self.ws)
         return hidden
 
     def fused_euler_step(self, prefix_pad, caches, x_t, step: int, positions, dt: float) -> torch.Tensor:
@@ -456,7 +478,49 @@ class SmolVLAModel:
         out = rms_norm(hidden, self.p[EXP + "norm.weight"], self.eps)
         return self.lin("action_out_proj", out.to(torch.float32))
 
+    def _sample_actions_overlapped(self, embs, pads, att, noise) -> torch.Tensor:
+        """Same result as the sequential core, bit for bit, with step 0 of the Euler loop hidden inside
+        the prefill: the main stream runs prefill layer i and records an event; the side stream waits
+        for it, builds layer i's attention cache (cross layers: the fp32 expert K/V projection) and
+        runs step-0 expert layer i.  Both are chains of small latency-bound launches that leave most
+        of the device idle, so they overlap almost completely.  The streams join before step 1."""
+        main, side = torch.cuda.current_stream(), self.side_stream
+        dt = -1.0 / self.num_steps
+        positions = tuple(t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32) for t in self.suffix_positions(pads, noise.shape[1]))
+        c = self._prefill_setup(embs, pads, att)
+        keys, values, vt = self._prefill_views(c)
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            h = F.silu(F.linear(noise[0], self.suffix_w, self.suffix_b[0]))
+            hid_s = F.linear(h, self.p["action_time_mlp_out.weight"], self.p["action_time_mlp_out.bias"])
+        hidden = embs[0]
+        caches: list = [None] * self.num_layers
+        for i in range(self.num_layers):
+            hidden = self._prefill_layer_fused(i, hidden, c)
+            done = torch.cuda.Event()
+            done.record(main)
+            with torch.cuda.stream(side):
+                side.wait_event(done)
+                if self.cfg.is_cross_layer(i):
+                    ek, ev = self._expert_prefix_kv_layer(i, keys[i], values[i])
+                    caches[i] = tk.prepare_prefix_kv(ek[0], ev[0])
+                else:
+                    caches[i] = tk.PrefixKV(keys[i, 0], vt[i])
+                hid_s = self._denoise_layer_fused(i, hid_s, caches[i], pads[0], positions[0], positions[1], self.ws_side)
+        with torch.cuda.stream(side):
+            _, x_new = tk.expert_tail(
+                hid_s, self.p["action_out_proj.weight"], self.p["action_out_proj.bias"], norm_w=self.p[EXP + "norm.weight"],
+                eps=self.eps, x_t=noise[0], dt=dt,
+            )  # fmt: skip
+        main.wait_stream(side)
+        x_t = x_new[None]
+        for step in range(1, self.num_steps):
+            x_t = self.fused_euler_step(pads, caches, x_t, step, positions, dt)
+        return x_t
+
     def sample_actions_core(self, embs, pads, att, noise, trace: dict | None = None) -> torch.Tensor:
+        if self.overlap and trace is None and embs.shape[0] == 1 and noise.shape[0] == 1 and noise.dtype == torch.float32 and noise.is_contiguous():
+            return self._sample_actions_overlapped(embs, pads, att, noise)
         vt = None
         if self.fused_prefill and embs.shape[0] == 1:
             keys, values, vt = self.prefill_fused(embs, pads, att)
