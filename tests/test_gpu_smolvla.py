@@ -153,3 +153,50 @@ def test_engine_rejects_flags_it_does_not_implement(ckpt):
         create_engine(ckpt, device="cuda", warmup=False, compile_model=True)
     with pytest.raises(ValueError):
         create_engine(ckpt, device="cuda", warmup=False, sampler="heun")
+
+
+def test_validate_against_an_oracle_dump(ckpt, tmp_path):
+    # `engine.validate(reference_dir)` (smolvla/engine.py:655-752): the dump directory is written here by
+    # the CPU oracle -- frame, preprocessed batch, prefix embedding, per-layer prefix K/V, one velocity
+    # evaluation at t = 0.5, the zero-noise chunk -- and every component must agree.
+    from tybok_amd.policies.smolvla.weights import random_state_dict
+    from tybok_amd.registry import create_engine
+
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_fused_attn=True, tl_vit_oproj=True)
+    eng = create_engine(ckpt, device="cuda", graph=True, graph_cameras=(3,), warmup=True, **flags)
+    cfg = eng.config
+    frame = eng._profile_frame(cameras=3, seed=11)
+    with torch.inference_mode():
+        batch = {k: v.cpu() for k, v in eng._batch_from_frame(frame).items() if isinstance(v, torch.Tensor)}
+        images01 = [batch[k] for k in cfg.image_features]
+        state = eng.prepare_state(batch)
+    shape = O.SmolVLAShape(num_vlm_layers=cfg.num_vlm_layers, vis_layers=cfg.vlm_config.vision_config.num_hidden_layers, num_steps=cfg.num_steps)
+    w = O.Weights(random_state_dict(cfg, seed=5), O.fp8_linear_names(shape, True, True))
+    tokens, lang_masks = batch["observation.language.tokens"], batch["observation.language.attention_mask"]
+    masks = [torch.ones(1, dtype=torch.bool)] * 3
+    with torch.no_grad():
+        images = O.prepare_images(images01)
+        embs, pads, att = O.embed_prefix(w, shape, images, masks, tokens, lang_masks, state)
+        kv = O.prefill(w, shape, embs, pads, att)
+        v_t = O.denoise_step(w, shape, pads, kv, O.expert_prefix_kv(w, shape, kv), torch.zeros(1, 50, 32), 0.5)
+        chunk = O.sample_actions(w, shape, images, masks, tokens, lang_masks, state, torch.zeros(1, 50, 32))[:, :, :6]
+    post = eng.unnormalizer.unnormalize(chunk.cuda(), "action", "ACTION").cpu()
+    d = str(tmp_path)
+    torch.save({k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in frame.items()}, os.path.join(d, "frame.pt"))
+    torch.save(batch, os.path.join(d, "batch.pt"))
+    torch.save({"embs": embs, "pad_masks": pads, "att_masks": att}, os.path.join(d, "prefix.pt"))
+    torch.save({f"layer{i}": {"keys": k, "values": v} for i, (k, v) in enumerate(kv)}, os.path.join(d, "prefix_kv.pt"))
+    torch.save({"v_t": v_t}, os.path.join(d, "denoise.pt"))
+    torch.save({"chunk": chunk, "chunk_post": post}, os.path.join(d, "chunk.pt"))
+    errors = eng.validate(d)
+    worst = {k: v for k, v in errors.items() if k.endswith(".max")}
+    print("validate:", {k: round(v, 5) for k, v in sorted(worst.items(), key=lambda kv: -kv[1])[:6]})
+    assert {"prefix.embs.max", "prefix_kv.layer0.keys.max", "denoise.v_t.max", "chunk.max", "chunk_post.max"} <= set(errors)
+    assert errors["prefix.pad_masks.max"] == 0 and errors["prefix.att_masks.max"] == 0
+    assert all(v == 0 for k, v in errors.items() if k.startswith("batch.") and k.endswith(".max"))
+    assert errors["prefix.embs.max"] <= 2e-2 * max(1.0, float(embs.abs().max()))
+    assert max(v for k, v in worst.items() if k.startswith("prefix_kv.")) <= 5e-2 * max(1.0, max(float(k.abs().max()) for k, _ in kv))
+    # one velocity evaluation carries the per-step bf16 noise undamped (the chunk integrates ten of them with dt = 0.1)
+    assert errors["denoise.v_t.max"] <= 5e-2 * max(1.0, float(v_t.abs().max())) and errors["chunk.max"] <= 1.25e-2
+    with pytest.raises(FileNotFoundError):
+        eng.validate(os.path.join(d, "nowhere"))

@@ -102,19 +102,31 @@ class SyntheticTokenizer:
 
 
 def load_state_dict(checkpoint_dir: str, wanted: dict[str, tuple], remap: dict[str, str] | None = None) -> dict[str, torch.Tensor]:
-    """Read every ``*.safetensors`` of the checkpoint (processor statistics aside) and return the
-    tensors whose names (minus a leading ``model.``) are in ``wanted``; raises if one is missing."""
+    """Read the checkpoint's ``*.safetensors`` (processor statistics aside) and return the tensors
+    whose names (minus a leading ``model.``) are in ``wanted``; raises if one is missing.
+
+    A file that contains ``*.scale_weight`` keys is a self-contained fp8 file: when one is present,
+    only fp8 files are read (docs/fastWAM_weight_quantization.md:9), and the ``<module>.scale_weight``
+    of every wanted fp8 ``<module>.weight`` is returned beside it."""
     from safetensors import safe_open
 
+    from ..fp8_checkpoint import SCALE_SUFFIX, fp8_files
+
+    files = fp8_files(checkpoint_dir) or [
+        f for f in sorted(glob.glob(os.path.join(checkpoint_dir, "*.safetensors"))) if "processor" not in os.path.basename(f)
+    ]
     out: dict[str, torch.Tensor] = {}
-    for file in sorted(glob.glob(os.path.join(checkpoint_dir, "*.safetensors"))):
-        if "processor" in os.path.basename(file):
-            continue
+    for file in files:
         with safe_open(file, "pt", "cpu") as f:
             for name in f.keys():
                 key = (remap or {}).get(name, name)
                 for cand in (key, key[len("model.") :] if key.startswith("model.") else None):
+                    if cand is None:
+                        continue
                     if cand in wanted:
+                        out[cand] = f.get_tensor(name)
+                        break
+                    if cand.endswith(SCALE_SUFFIX) and cand[: -len(SCALE_SUFFIX)] + ".weight" in wanted:
                         out[cand] = f.get_tensor(name)
                         break
     missing = [k for k in wanted if k not in out]

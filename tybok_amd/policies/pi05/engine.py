@@ -151,7 +151,7 @@ class PI05Engine(PolicyEngine):
         else:
             raise FileNotFoundError("no tokenizer.json: pass --tokenizer-dir")
 
-        if self.config.random_init is not None:
+        if self.config.random_init is not None and self.config.random_init.get("weights") != "files":
             sd = random_state_dict(self.config, seed=int(self.config.random_init.get("seed", 0)))
         else:
             sd = load_state_dict(checkpoint_dir, {n: s for n, s, _, _ in parameter_inventory(self.config)}, remap=_KEY_REMAP)

@@ -129,7 +129,7 @@ class SmolVLAEngine(PolicyEngine):
         else:
             raise FileNotFoundError(f"no tokenizer.json under {tok_dir}")
 
-        if self.config.random_init is not None:
+        if self.config.random_init is not None and self.config.random_init.get("weights") != "files":
             sd = random_state_dict(self.config, seed=int(self.config.random_init.get("seed", 0)))
         else:
             sd = load_state_dict(checkpoint_dir, {n: s for n, s, _, _ in parameter_inventory(self.config)})
@@ -210,21 +210,72 @@ class SmolVLAEngine(PolicyEngine):
         action = self._action_queue.popleft()
         return self.unnormalizer.unnormalize(action, ACTION, "ACTION").cpu().numpy()[0]
 
+    @torch.inference_mode()
     def validate(self, reference_dir: str) -> dict[str, float]:
-        """Max/mean-abs errors of the full zero-noise chunk against ``chunk.pt`` of a reference dump
-        (``frame.pt`` + ``chunk.pt``: tybok/policies/smolvla/engine.py:668-673, 738-752)."""
+        """Per-component max / mean-abs errors against a reference dump, keyed like the reference's
+        report (tybok/policies/smolvla/engine.py:655-752): ``batch.*``, ``prefix.{embs,pad_masks,
+        att_masks}``, ``prefix_kv.layer<i>.{keys,values}``, ``denoise.v_t`` (zero ``x_t``, t = 0.5),
+        ``chunk`` (zero noise, through the graph when enabled) and ``chunk_post``.  ``frame.pt`` and
+        ``chunk.pt`` are required, the other dump files are compared when present.  Dumps are read
+        with ``weights_only=True``: tensors and plain containers only."""
 
-        def load(name: str):
+        def load(name: str, required: bool = False):
             path = os.path.join(reference_dir, name)
             if not os.path.exists(path):
-                raise FileNotFoundError(f"reference dump {path} missing")
+                if required:
+                    raise FileNotFoundError(f"reference dump {path} missing")
+                return None
             return torch.load(path, weights_only=True)
 
-        frame, ref = load("frame.pt"), load("chunk.pt")
-        noise = torch.zeros(1, self.config.chunk_size, self.config.action_feature_shape[0])
-        chunk = torch.from_numpy(self.predict_action_chunk(frame, noise=noise))
-        diff = (chunk - ref["chunk_post"].float().cpu().reshape(chunk.shape)).abs()
-        return {"chunk_post.max": float(diff.max()), "chunk_post.mean": float(diff.mean())}
+        frame, ref_chunk = load("frame.pt", True), load("chunk.pt", True)
+        ref_batch, ref_prefix, ref_kv, ref_denoise = load("batch.pt"), load("prefix.pt"), load("prefix_kv.pt"), load("denoise.pt")
+        errors: dict[str, float] = {}
+
+        def max_err(name: str, a: torch.Tensor, b: torch.Tensor) -> None:
+            a, b = a.detach().float().cpu(), b.detach().float().cpu()
+            if a.shape != b.shape:
+                raise AssertionError(f"{name}: shape mismatch {tuple(a.shape)} vs {tuple(b.shape)}")
+            diff = (a - b).abs()
+            errors[name + ".max"] = float(diff.max())
+            errors[name + ".mean"] = float(diff.mean())
+
+        batch = self._batch_from_frame(frame)
+        if ref_batch is not None:
+            for key in [OBS_STATE, OBS_LANGUAGE_TOKENS, OBS_LANGUAGE_ATTENTION_MASK] + [k for k in ref_batch if k.startswith("observation.images.")]:
+                if key in batch and key in ref_batch:
+                    max_err(f"batch.{key}", batch[key], ref_batch[key])
+        images, img_masks = self.prepare_images(batch)
+        state = self.prepare_state(batch)
+        tokens, lang_masks = batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK]
+        m = self.model
+        embs, pads, att = m.embed_prefix(images, img_masks, tokens, lang_masks, state)
+        if ref_prefix is not None:
+            max_err("prefix.embs", embs, ref_prefix["embs"])
+            max_err("prefix.pad_masks", pads, ref_prefix["pad_masks"])
+            max_err("prefix.att_masks", att, ref_prefix["att_masks"])
+        if ref_kv is not None or ref_denoise is not None:
+            if m.fused_prefill and embs.shape[0] == 1:
+                keys, values, _ = m.prefill_fused(embs, pads, att)
+            else:
+                keys, values = m.prefill(embs, pads, att)
+            if ref_kv is not None:
+                for i in range(self.config.num_vlm_layers):
+                    max_err(f"prefix_kv.layer{i}.keys", keys[i], ref_kv[f"layer{i}"]["keys"])
+                    max_err(f"prefix_kv.layer{i}.values", values[i], ref_kv[f"layer{i}"]["values"])
+            if ref_denoise is not None:
+                from .model import sinusoidal_time_embedding
+
+                x_t = torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, device=self.device)
+                te = sinusoidal_time_embedding(torch.tensor([0.5]), self.config.expert_hidden_size, self.config.min_period, self.config.max_period)
+                v_t = m.denoise_step(pads, keys, values, m.expert_prefix_kv(keys, values), x_t, te.float().to(self.device))
+                max_err("denoise.v_t", v_t, ref_denoise["v_t"])
+        noise = torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, device=self.device)
+        chunk = self._infer(batch, noise)[:, :, : self.config.action_feature_shape[0]]
+        if "chunk" in ref_chunk:
+            max_err("chunk", chunk, ref_chunk["chunk"].reshape(chunk.shape))
+        post = self.unnormalizer.unnormalize(chunk, ACTION, "ACTION")
+        max_err("chunk_post", post, ref_chunk["chunk_post"].reshape(post.shape))
+        return errors
 
     # ------------------------------------------------------------------ request plumbing
     def _resolve_alias(self, camera_alias: dict[str, str] | None) -> dict[str, str]:

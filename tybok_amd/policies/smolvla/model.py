@@ -27,6 +27,7 @@ import torch
 import torch.nn.functional as F  # noqa: N812
 
 from ... import ops as tk
+from ...fp8_checkpoint import SCALE_SUFFIX, dequantize_entry
 from ...quant import quantize_weight_rows
 from .config import SmolVLAConfig
 from .weights import CONNECTOR, EXP, TXT, VIS
@@ -70,15 +71,23 @@ class GatedMLP:
     def __init__(self, sd: dict, prefix: str, device, fp8: bool, act: str = "silu"):
         self.act = act
         self.fp8 = fp8
-        wg, wu, wd = (sd[prefix + n + ".weight"] for n in ("gate_proj", "up_proj", "down_proj"))
+        names = [prefix + n + ".weight" for n in ("gate_proj", "up_proj", "down_proj")]
+
+        def codes_and_scale(name: str):
+            # an fp8 checkpoint stores the e4m3fn codes with their row scales: used as they are
+            w = sd[name]
+            if w.dtype == torch.float8_e4m3fn:
+                return w.to(device), sd[name[: -len(".weight")] + SCALE_SUFFIX].to(device=device, dtype=torch.float32)
+            return quantize_weight_rows(w.to(device))
+
         if fp8:
-            g8, sg = quantize_weight_rows(wg.to(device))
-            u8, su = quantize_weight_rows(wu.to(device))
-            d8, sdn = quantize_weight_rows(wd.to(device))
+            (g8, sg), (u8, su), (d8, sdn) = (codes_and_scale(n) for n in names)
             self.wgu = tk.pack_fp8_gate_up(g8, sg, u8, su)
             self.wd = tk.pack_fp8_weight(d8, sdn)
         else:
-            self.wg, self.wu, self.wdn = wg.to(device), wu.to(device), wd.to(device)
+            self.wg, self.wu, self.wdn = (
+                (dequantize_entry(sd, n) if sd[n].dtype == torch.float8_e4m3fn else sd[n]).to(device) for n in names
+            )
 
     def __call__(self, x: torch.Tensor, resid: torch.Tensor) -> torch.Tensor:
         """``down(act(gate(x)) * up(x)) + resid`` for ``x [B, L, hidden]`` bf16 (in-place add semantics)."""

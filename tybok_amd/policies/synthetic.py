@@ -49,3 +49,30 @@ def write_pi05_checkpoint(path: str, cameras: int = 2, seed: int = 0, depth: int
     with open(os.path.join(path, "config.json"), "w", encoding="utf-8") as f:
         json.dump(cfg, f, indent=1)
     return path
+
+
+def write_weight_files(path: str) -> str:
+    """Materialise the random-init weights of a synthetic checkpoint as ``model.safetensors`` and
+    switch its config to read weights from files (``random_init.weights = "files"``; tokenizer and
+    normalisation statistics stay synthetic).  Lets the file loaders -- including the fp8 checkpoint
+    format -- run without a downloaded model."""
+    from safetensors.torch import save_file
+
+    with open(os.path.join(path, "config.json"), encoding="utf-8") as f:
+        cfg = json.load(f)
+    seed = int(cfg["random_init"]["seed"])
+    if cfg["type"] == "smolvla":
+        from .smolvla.config import SmolVLAConfig
+        from .smolvla.weights import random_state_dict
+
+        sd = random_state_dict(SmolVLAConfig.from_pretrained(path), seed=seed)
+    else:
+        from .pi05.config import PI05Config
+        from .pi05.weights import random_state_dict
+
+        sd = random_state_dict(PI05Config.from_pretrained(path), seed=seed)
+    save_file({k: v.contiguous() for k, v in sd.items()}, os.path.join(path, "model.safetensors"))
+    cfg["random_init"]["weights"] = "files"
+    with open(os.path.join(path, "config.json"), "w", encoding="utf-8") as f:
+        json.dump(cfg, f, indent=1)
+    return path

@@ -19,7 +19,11 @@ def quantize_weight_rows(w: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     if w.dim() != 2:
         raise ValueError("expected a 2-D [out, in] weight")
     wf = w.detach().to(torch.float32)
-    scale = (wf.abs().amax(dim=1, keepdim=True) / FP8_MAX).clamp_min(1e-12)
+    # tensor / tensor: a true fp32 division on every device (dividing by a Python scalar is turned into
+    # a multiplication by 1/448 on the GPU, one ulp off for some rows -- the codes of a checkpoint
+    # quantised offline on the CPU and at load time on the GPU would then differ)
+    amax = wf.abs().amax(dim=1, keepdim=True)
+    scale = torch.div(amax, torch.full_like(amax, FP8_MAX)).clamp_min(1e-12)
     w8 = (wf / scale).to(torch.float8_e4m3fn).contiguous()
     return w8, scale.squeeze(1).contiguous()
 
