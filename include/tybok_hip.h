@@ -211,7 +211,7 @@ int tk_attn_prepare_kv(const void* k, const void* v, int kv_dtype, int sl, int s
  *   mask_mode: TK_MASK_*; q head h reads kv head h / (H / G).
  *   logits_bf16: 0 = fp32 logits (SmolVLA); 1 = logits rounded to bf16 before the softmax and
  *           masked with the additive -2.3819763e38 (pi0.5).
- *   D in {64, 128, 256}; masked logits use finfo(float32).min, so a fully masked row is uniform.
+ *   D in {64, 96, 128, 256}; masked logits use finfo(float32).min, so a fully masked row is uniform.
  *   out:    8-byte aligned, out_sm a multiple of 4.
  */
 int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const void* k_pre_lo, int pre_sl, int pre_sh,
@@ -225,10 +225,13 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
  * operands of tk_expert_attn (K [P, G, D]; V^T [G, D, >= P rounded up to 32], zero padded), with
  * element strides q_sb / k_sb / vt_sb / out_sb between problems.  logits_bf16 = 1 rounds q.K^T to
  * bf16 before the fp32 scale and softmax, as a bf16 matmul followed by `.float() * scale` does
- * (tybok/policies/smolvla/models/vision.py:197-257). */
+ * (tybok/policies/smolvla/models/vision.py:197-257).  scale > 0 replaces D^-0.5: a head whose true
+ * size is not supported (SigLIP-So400m: 72) is padded with zero columns to the next D and passes
+ * 72^-0.5 (tybok/policies/pi05/models/vision.py:52-66); scale = 0 keeps the default. */
 int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const void* k, long long k_sb, int k_sl, int k_sh,
                     const void* vt, long long vt_sb, int vt_sd, int vt_sh, void* out, long long out_sb, int out_sm, int B,
-                    int M, int P, int H, int G, int D, int logits_bf16, void* ws, size_t ws_bytes, void* stream);
+                    int M, int P, int H, int G, int D, int logits_bf16, float scale, void* ws, size_t ws_bytes,
+                    void* stream);
 
 /* ---- tail of a denoising step ---------------------------------------------------------------- */
 /* Final norm of the expert hidden state + fp32 action projection + Euler update in one launch:

@@ -59,7 +59,8 @@ class PI05Shape:
     max_period: float = 4.0
     # drift tiers of the vision tower (tybok/policies/pi05/engine.py:196-230):
     #   vit_mlp_dtype: fc1 / gelu / fc2 run in that dtype, cast at the boundary (vision.py:79-87);
-    #   vit_lowp_attn: q/k/v and out_proj run in bf16 too, attention scores and softmax in fp32.
+    #   vit_lowp_attn: q/k/v and out_proj run in bf16 too; attention scores and softmax in fp32, the
+    #                  probabilities rounded to bf16 for P.V (fp32 accumulate, bf16 result).
     vit_mlp_dtype: torch.dtype | None = None
     vit_lowp_attn: bool = False
 
@@ -92,8 +93,8 @@ def embed_image(w: Weights, shape: PI05Shape, image: torch.Tensor) -> torch.Tens
         h = F.layer_norm(x, (shape.vis_hidden,), w[p + "layer_norm1.weight"], w[p + "layer_norm1.bias"], EPS)
         if shape.vit_lowp_attn:
             q, k, v = (lowp(p + f"self_attn.{n}_proj", h, torch.bfloat16).view(b, -1, shape.vis_heads, hd).transpose(1, 2) for n in "qkv")
-            probs = torch.softmax(torch.matmul(q.float(), k.float().transpose(2, 3)) * hd**-0.5, dim=-1)
-            a = torch.matmul(probs, v.float()).to(torch.bfloat16).transpose(1, 2).reshape(b, -1, shape.vis_hidden)
+            probs = torch.softmax(torch.matmul(q.float(), k.float().transpose(2, 3)) * hd**-0.5, dim=-1).to(torch.bfloat16)
+            a = torch.matmul(probs.float(), v.float()).to(torch.bfloat16).transpose(1, 2).reshape(b, -1, shape.vis_hidden)
             x = x + lowp(p + "self_attn.out_proj", a, torch.bfloat16).float()
         else:
             q = w.linear(p + "self_attn.q_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)

@@ -240,6 +240,21 @@ def test_batched_vision_attention(tk):
     _close(got, want, "batched vision attention")
 
 
+def test_batched_attention_padded_head_with_explicit_scale(tk):
+    # SigLIP-So400m heads are 72 wide: run as 96-wide heads whose last 24 columns are zero, with the
+    # logit scale of the true size; the padded output columns must come back as zeros
+    b, length, heads, hd, hp = 2, 256, 16, 72, 96
+    g = torch.Generator().manual_seed(31)
+    q, k, v = (torch.randn(b, length, heads, hd, generator=g).to(torch.bfloat16) for _ in range(3))
+    pad = lambda t: torch.nn.functional.pad(t, (0, hp - hd))  # noqa: E731
+    vt = pad(v).permute(0, 2, 3, 1).contiguous()
+    got = tk.batched_attn(pad(q).cuda(), pad(k).cuda(), vt.cuda(), scale=hd**-0.5).cpu().view(b, length, heads, hp)
+    assert torch.count_nonzero(got[..., hd:]) == 0
+    probs = torch.softmax(torch.einsum("blhd,bmhd->bhlm", q.float(), k.float()) * hd**-0.5, dim=-1).to(torch.bfloat16)
+    want = torch.einsum("bhlm,bmhd->blhd", probs.float(), v.float()).to(torch.bfloat16)
+    _close(got[..., :hd], want, "padded-head batched attention")
+
+
 def test_gated_residual_epilogue(tk):
     # pi0.5 AdaRMS gated residual: y = resid + bf16(ffn(x) * gate)
     x, wg8, sg, wu8, su, wd8, sd = ffn_case(50, 1024, 4096, seed=3)

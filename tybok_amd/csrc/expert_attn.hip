@@ -542,6 +542,7 @@ int tk_launch_attn(AttnArgs a, int D, int waves, hipStream_t st) {
     if (waves == 8) return launch_attn<64, false, 8>(a, st);
     return launch_attn<64, false, 4>(a, st);
   }
+  if (D == 96) return launch_attn<96, false, 4>(a, st);
   if (D == 128) return launch_attn<128, false, 4>(a, st);
   if (D == 256) return launch_attn<256, false, 4>(a, st);
   return -1;

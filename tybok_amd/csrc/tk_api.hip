@@ -411,10 +411,11 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
                    const void* vt_pre, const void* vt_pre_lo, int pre_vt_sd, int pre_vt_sh, const void* k_suf, int suf_sl,
                    int suf_sh, const void* vt_suf, int suf_vt_sd, int suf_vt_sh, const void* pad, const void* mask2d,
                    int mask_ld, void* out, int out_sm, int M, int P, int S, int H, int G, int D, int mask_mode,
-                   int logits_bf16, void* ws, size_t ws_bytes, void* stream) {
+                   int logits_bf16, float scale, void* ws, size_t ws_bytes, void* stream) {
   if (M <= 0 || P < 0 || S < 0 || P + S <= 0 || H <= 0 || G <= 0 || H % G)
     return fail(TK_EINVAL, "attn: bad shape M=%d P=%d S=%d H=%d G=%d", M, P, S, H, G);
-  if (D != 64 && D != 128 && D != 256) return fail(TK_EINVAL, "attn: head_dim %d not in {64,128,256}", D);
+  if (D != 64 && D != 96 && D != 128 && D != 256) return fail(TK_EINVAL, "attn: head_dim %d not in {64,96,128,256}", D);
+  if (!(scale >= 0.f)) return fail(TK_EINVAL, "attn: negative or NaN scale");
   const bool split = k_pre_lo != nullptr || vt_pre_lo != nullptr;
   if (split && (!k_pre_lo || !vt_pre_lo)) return fail(TK_EINVAL, "attn: hi/lo planes need both K and V^T low planes");
   if (split && (S != 0 || D != 64))
@@ -470,7 +471,7 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   a.G = G;
   a.mask_mode = mask_mode;
   a.logits_bf16 = logits_bf16;
-  a.scale = 1.0f / sqrtf((float)D);
+  a.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
 
   const int ntiles = (P + 31) / 32 + (S + 31) / 32;
   const int mtiles = ((M + 31) / 32) * (batch > 0 ? batch : 1);
@@ -515,17 +516,17 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
                    int logits_bf16, void* ws, size_t ws_bytes, void* stream) {
   return attn_impl(0, 0, 0, 0, 0, q, q_sm, q_sh, k_pre, k_pre_lo, pre_sl, pre_sh, vt_pre, vt_pre_lo, pre_vt_sd, pre_vt_sh, k_suf,
                    suf_sl, suf_sh, vt_suf, suf_vt_sd, suf_vt_sh, pad, mask2d, mask_ld, out, out_sm, M, P, S, H, G, D, mask_mode,
-                   logits_bf16, ws, ws_bytes, stream);
+                   logits_bf16, 0.f, ws, ws_bytes, stream);
 }
 
 int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const void* k, long long k_sb, int k_sl, int k_sh,
                     const void* vt, long long vt_sb, int vt_sd, int vt_sh, void* out, long long out_sb, int out_sm, int B,
-                    int M, int P, int H, int G, int D, int logits_bf16, void* ws, size_t ws_bytes, void* stream) {
+                    int M, int P, int H, int G, int D, int logits_bf16, float scale, void* ws, size_t ws_bytes, void* stream) {
   if (B <= 0) return fail(TK_EINVAL, "batched_attn: B=%d", B);
   if (q_sb % 8 || k_sb % 8 || vt_sb % 8 || out_sb % 4) return fail(TK_EINVAL, "batched_attn: batch strides must keep 16-byte alignment");
   return attn_impl(B, q_sb, k_sb, vt_sb, out_sb, q, q_sm, q_sh, k, nullptr, k_sl, k_sh, vt, nullptr, vt_sd, vt_sh, nullptr, 0, 0,
-                   nullptr, 0, 0, nullptr, nullptr, 0, out, out_sm, M, P, 0, H, G, D, TK_MASK_NONE, logits_bf16, ws, ws_bytes,
-                   stream);
+                   nullptr, 0, 0, nullptr, nullptr, 0, out, out_sm, M, P, 0, H, G, D, TK_MASK_NONE, logits_bf16, scale, ws,
+                   ws_bytes, stream);
 }
 
 int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps,

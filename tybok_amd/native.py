@@ -63,7 +63,7 @@ SIGNATURES: dict[str, tuple] = {
     "tk_batched_attn": (
         c_int,
         [c_void_p, c_longlong, c_int, c_int, c_void_p, c_longlong, c_int, c_int, c_void_p, c_longlong, c_int, c_int,
-         c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
+         c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
     "tk_expert_attn": (
         c_int,

@@ -472,12 +472,14 @@ def batched_attn(
     vt: torch.Tensor,
     *,
     logits_bf16: bool = False,
+    scale: float | None = None,
     out: torch.Tensor | None = None,
     ws: Workspace | None = None,
 ) -> torch.Tensor:
     """``B`` independent unmasked attentions: ``q [B, M, H, D]``, ``k [B, P, G, D]`` (views with a
     contiguous head dim), ``vt [B, G, D, >= P rounded up to 32]`` (V transposed, zero padded) ->
-    bf16 ``[B, M, H*D]``."""
+    bf16 ``[B, M, H*D]``.  ``scale`` multiplies the logits (default ``D ** -0.5``; a head padded with
+    zero columns up to a supported ``D`` passes the scale of its true size)."""
     lib = native.lib()
     bf = torch.bfloat16
     if q.dtype != bf or k.dtype != bf or vt.dtype != bf or q.dim() != 4 or k.dim() != 4 or vt.dim() != 4:
@@ -494,7 +496,7 @@ def batched_attn(
     rc = lib.tk_batched_attn(
         q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), k.data_ptr(), k.stride(0), k.stride(1), k.stride(2) if g > 1 else 0,
         vt.data_ptr(), vt.stride(0), vt.stride(2), vt.stride(1) if g > 1 else 0, out.data_ptr(), out.stride(0), out.stride(1),
-        b, m, p, h, g, d, int(logits_bf16), ws.ptr, ws.nbytes, _stream(),
+        b, m, p, h, g, d, int(logits_bf16), float(scale or 0.0), ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip
     native.check(rc, "tk_batched_attn")
     return out

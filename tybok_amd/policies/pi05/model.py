@@ -88,7 +88,7 @@ class PI05Model:
         self.fp8_expert_mlp = bool(fp8_expert_mlp)
         self.fp8_llm_mlp = bool(fp8_llm_mlp)
         self.fused_prefill = bool(fused_prefill)
-        self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp or self.fused_prefill
+        self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp or self.fused_prefill or self.vit_lowp_attn
         if self.use_hip and self.device.type != "cuda":
             raise RuntimeError("the fused / fp8 tiers run HIP kernels and need a GPU device")
         self.vd, self.ed = cfg.paligemma_dims, cfg.expert_dims
@@ -136,17 +136,34 @@ class PI05Model:
         self.patch_w = self.p[VIS + "embeddings.patch_embedding.weight"].reshape(cfg.vision_hidden, -1)
         # low-precision copies of the vision tower's linears (the drift tiers convert weights and bias)
         self.vis_lowp: dict[str, tuple[torch.Tensor, torch.Tensor]] = {}
+        # head size the attention kernel runs: the smallest supported one that holds the tower's heads
+        self.vis_head_pad = next((d for d in (64, 96, 128, 256) if d >= cfg.vision_hidden // cfg.vision_heads), 0)
+        if self.vit_lowp_attn and not self.vis_head_pad:
+            raise ValueError("vision heads wider than 256 are not supported by the attention kernel")
         for i in range(cfg.vision_layers):
             lp = f"{VIS}encoder.layers.{i}."
             if self.vit_mlp_dtype is not None:
                 for n in ("mlp.fc1", "mlp.fc2"):
                     self.vis_lowp[lp + n] = (self.p[lp + n + ".weight"].to(self.vit_mlp_dtype), self.p[lp + n + ".bias"].to(self.vit_mlp_dtype))
             if self.vit_lowp_attn:
+                # q|k|v as one bf16 GEMM whose output is already the attention kernel's layout: every
+                # head padded with zero rows from 72 to 96 columns (zero q/k columns add nothing to the
+                # scores, zero value columns give zero outputs that out_proj's zero columns ignore)
+                heads, hd, hp = cfg.vision_heads, cfg.vision_hidden // cfg.vision_heads, self.vis_head_pad
+
+                def pad_rows(t: torch.Tensor) -> torch.Tensor:  # [heads * hd, ...] -> [heads * hp, ...]
+                    out = torch.zeros(heads, hp, *t.shape[1:], dtype=t.dtype, device=t.device)
+                    out[:, :hd] = t.view(heads, hd, *t.shape[1:])
+                    return out.view(heads * hp, *t.shape[1:])
+
                 self.vis_lowp[lp + "self_attn.qkv"] = (
-                    torch.cat([self.p[lp + f"self_attn.{n}_proj.weight"] for n in "qkv"], dim=0).to(BF16),
-                    torch.cat([self.p[lp + f"self_attn.{n}_proj.bias"] for n in "qkv"], dim=0).to(BF16),
+                    torch.cat([pad_rows(self.p[lp + f"self_attn.{n}_proj.weight"]) for n in "qkv"], dim=0).to(BF16).contiguous(),
+                    torch.cat([pad_rows(self.p[lp + f"self_attn.{n}_proj.bias"]) for n in "qkv"], dim=0).to(BF16).contiguous(),
                 )
-                self.vis_lowp[lp + "self_attn.out_proj"] = (self.p[lp + "self_attn.out_proj.weight"].to(BF16), self.p[lp + "self_attn.out_proj.bias"].to(BF16))
+                self.vis_lowp[lp + "self_attn.out_proj"] = (
+                    pad_rows(self.p[lp + "self_attn.out_proj.weight"].t().contiguous()).t().to(BF16).contiguous(),
+                    self.p[lp + "self_attn.out_proj.bias"].to(BF16),
+                )
         self.set_num_steps(cfg.num_steps)
 
     def lin(self, name: str, x: torch.Tensor) -> torch.Tensor:
@@ -199,10 +216,12 @@ class PI05Model:
             lp = f"{VIS}encoder.layers.{i}."
             h = F.layer_norm(x, (vh,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], EPS)
             if self.vit_lowp_attn:
-                # bf16 projections (one packed q|k|v GEMM), fp32 scores / softmax / P.V
-                qkv = F.linear(h.to(BF16), *self.vis_lowp[lp + "self_attn.qkv"]).view(b, -1, 3, heads, hd).permute(2, 0, 3, 1, 4).float()
-                att = torch.softmax(torch.matmul(qkv[0], qkv[1].transpose(2, 3)) * hd**-0.5, dim=-1)
-                a = torch.matmul(att, qkv[2]).to(BF16).transpose(1, 2).reshape(b, -1, vh)
+                # bf16 projections (one packed q|k|v GEMM), then the HIP attention, one problem per image:
+                # fp32 scores and softmax, probabilities rounded to bf16 for P.V (fp32 accumulate)
+                hp = self.vis_head_pad
+                qkv = F.linear(h.to(BF16), *self.vis_lowp[lp + "self_attn.qkv"]).view(b, -1, 3, heads, hp)
+                vt = qkv[:, :, 2].permute(0, 2, 3, 1).contiguous()
+                a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, scale=hd**-0.5, ws=self.ws)
                 x = x + F.linear(a, *self.vis_lowp[lp + "self_attn.out_proj"]).float()
             else:
                 q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
