@@ -528,6 +528,8 @@ int tk_attn_waves(int D, int split_planes, int ntiles) {
   if (D != 64) return 4;
   if (ntiles <= 8 && ntiles > 4) return 8;
   if (!split_planes && ntiles <= 12 && ntiles > 8) return 12;
+  // long key ranges (vision tower: 32 tiles): two waves per SIMD hide more of the per-tile latency
+  if (!split_planes && ntiles > 12) return 8;
   return 4;
 }
 
