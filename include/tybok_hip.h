@@ -220,6 +220,19 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
                    const void* mask2d, int mask_ld, void* out, int out_sm, int M, int P, int S, int H, int G, int D,
                    int mask_mode, int logits_bf16, void* ws, size_t ws_bytes, void* stream);
 
+/* Expert K/V projection of the cached VLM prefix for the cross-attention layers, straight into the
+ * attention kernel's fp32 operand layout (bf16 hi + lo planes):
+ *   ek = float(k) . wk^T, ev = float(v) . wv^T with fp32 weights and fp32 accumulation, then
+ *   k_hi / k_lo [P, N] and vt_hi / vt_lo [N, vt_ld] (V transposed, keys contiguous, zero filled
+ *   from P to P rounded up to 32) -- N = kv_heads * head_dim.
+ * Replaces `_compute_expert_prefix_kv` + the cache fill: two `.float()` casts, two fp32 linears
+ * and tk_attn_prepare_kv (tybok/policies/smolvla/models/flow_matching.py:553-578,
+ * tybok/policies/smolvla/models/expert.py:35-39).
+ *   k, v: bf16 [P, KV] rows with element stride sl (a multiple of 8), 16-byte aligned; wk, wv: fp32
+ *   [N, KV]; N a multiple of 32, KV of 16; k_hi / k_lo 8-byte aligned; vt_ld >= P rounded up to 32. */
+int tk_expert_kv_project(const void* k, const void* v, int sl, int P, int KV, const void* wk, const void* wv, int N,
+                         void* k_hi, void* k_lo, void* vt_hi, void* vt_lo, int vt_ld, void* stream);
+
 /* B independent unmasked attentions in one launch (the vision tower's self-attention, one problem
  * per camera image): out[b][M, H*D] = softmax(q[b].K[b]^T * D^-0.5) . V[b].  Layouts as the prefix
  * operands of tk_expert_attn (K [P, G, D]; V^T [G, D, >= P rounded up to 32], zero padded), with

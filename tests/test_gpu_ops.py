@@ -255,6 +255,34 @@ def test_batched_attention_padded_head_with_explicit_scale(tk):
     _close(got[..., :hd], want, "padded-head batched attention")
 
 
+@pytest.mark.parametrize("p,kv,n,d", [(241, 320, 320, 64), (177, 320, 320, 64), (40, 96, 128, 64), (33, 208, 64, 64)])
+def test_expert_kv_projection_into_attention_planes(tk, p, kv, n, d):
+    # float(K) @ Wk^T / float(V) @ Wv^T in fp32, delivered as the attention kernel's hi + lo planes:
+    # hi + lo must reproduce the fp32 projection to ~2^-16, the padded V^T keys must be zero, and the
+    # attention over the planes must equal the attention over the torch projection
+    g = torch.Generator().manual_seed(41)
+    wide = torch.randn(p, 4 * kv, generator=g).to(torch.bfloat16).cuda()  # rows strided like a q|k|v buffer
+    k, v = wide[:, 2 * kv : 3 * kv], wide[:, 3 * kv :]
+    wk, wv = (torch.randn(n, kv, generator=g) * kv**-0.5).cuda(), (torch.randn(n, kv, generator=g) * kv**-0.5).cuda()
+    cache = tk.project_prefix_kv(k, v, wk, wv, d)
+    ek = (k.float().cpu().double() @ wk.cpu().double().T).float()
+    ev = (v.float().cpu().double() @ wv.cpu().double().T).float()
+    got_k = (cache.k.float() + cache.k_lo.float()).cpu().reshape(p, n)
+    got_vt = (cache.vt.float() + cache.vt_lo.float()).cpu()
+    assert float((got_k - ek).abs().max()) <= 3e-5 * max(1.0, float(ek.abs().max()))
+    assert float((got_vt[:, :, :p].reshape(n, p).T - ev).abs().max()) <= 3e-5 * max(1.0, float(ev.abs().max()))
+    assert torch.count_nonzero(got_vt[:, :, p:]) == 0
+    # same bits on a second call (fixed accumulation order)
+    again = tk.project_prefix_kv(k, v, wk, wv, d)
+    assert torch.equal(again.k, cache.k) and torch.equal(again.k_lo, cache.k_lo) and torch.equal(again.vt_lo, cache.vt_lo)
+    heads = n // d
+    q = torch.randn(50, heads * 3, d, generator=g).to(torch.bfloat16).cuda()
+    ref_cache = tk.prepare_prefix_kv(ek.view(p, heads, d).cuda(), ev.view(p, heads, d).cuda())
+    a = tk.expert_attn(q, cache, None, None, tk.MASK_NONE)
+    b = tk.expert_attn(q, ref_cache, None, None, tk.MASK_NONE)
+    _close(a, b.cpu(), "attention over projected planes")
+
+
 def test_gated_residual_epilogue(tk):
     # pi0.5 AdaRMS gated residual: y = resid + bf16(ffn(x) * gate)
     x, wg8, sg, wu8, su, wd8, sd = ffn_case(50, 1024, 4096, seed=3)

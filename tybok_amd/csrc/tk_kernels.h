@@ -92,6 +92,20 @@ struct KvPrepArgs {
   int ld;
 };
 
+struct KvProjArgs {
+  const unsigned short* k;  // bf16 [P, KV] rows (element stride sl)
+  const unsigned short* v;
+  int sl;
+  const float* wk;  // fp32 [N, KV]
+  const float* wv;
+  int P, KV, N;
+  unsigned short* k_hi;  // [P, N]
+  unsigned short* k_lo;
+  unsigned short* vt_hi;  // [N, ld], ld >= P rounded up to 32
+  unsigned short* vt_lo;
+  int ld;
+};
+
 struct TailArgs {
   const unsigned short* x;  // bf16 [M, K]
   int ldx;
@@ -121,6 +135,7 @@ struct NormRowsArgs {
 };
 
 int tk_launch_tail(TailArgs a, hipStream_t st);
+int tk_launch_kv_proj(KvProjArgs a, hipStream_t st);
 int tk_wide_rows();  // block tile of the many-row GEMM
 int tk_wide_cols();
 int tk_launch_gemm_wide(GemmArgs a, hipStream_t st);

@@ -392,6 +392,30 @@ def prepare_prefix_kv(k: torch.Tensor, v: torch.Tensor) -> PrefixKV:
     return PrefixKV(k, vt)
 
 
+def project_prefix_kv(k: torch.Tensor, v: torch.Tensor, wk: torch.Tensor, wv: torch.Tensor, d: int) -> PrefixKV:
+    """fp32 expert K/V projection of a cached prefix, straight into the attention operand layout:
+    ``k, v [P, KV]`` bf16 rows (views with a contiguous last dim and the same row stride), ``wk, wv
+    [N, KV]`` fp32 -> :class:`PrefixKV` of ``float(k) @ wk.T`` / ``float(v) @ wv.T`` as bf16 hi + lo
+    planes (``[P, N/d, d]`` and ``[N/d, d, P rounded up to 32]``).  One launch."""
+    lib = native.lib()
+    bf = torch.bfloat16
+    if k.dtype != bf or v.dtype != bf or wk.dtype != torch.float32 or wv.dtype != torch.float32:
+        raise TypeError("project_prefix_kv: k, v bf16 and wk, wv fp32")
+    p, kv = k.shape
+    n = wk.shape[0]
+    if v.shape != k.shape or wk.shape != (n, kv) or wv.shape != (n, kv) or n % d or k.stride(1) != 1 or v.stride(1) != 1 or k.stride(0) != v.stride(0):
+        raise ValueError("project_prefix_kv: k, v [P, KV] with equal row strides; wk, wv [N, KV]; N a multiple of d")
+    wk, wv = wk.contiguous(), wv.contiguous()
+    g = n // d
+    opts = dict(dtype=bf, device=k.device)
+    k_hi, k_lo = torch.empty(p, g, d, **opts), torch.empty(p, g, d, **opts)
+    vt_hi, vt_lo = torch.empty(g, d, _pad32(p), **opts), torch.empty(g, d, _pad32(p), **opts)
+    rc = lib.tk_expert_kv_project(k.data_ptr(), v.data_ptr(), k.stride(0), p, kv, wk.data_ptr(), wv.data_ptr(), n, k_hi.data_ptr(),
+                                  k_lo.data_ptr(), vt_hi.data_ptr(), vt_lo.data_ptr(), vt_hi.shape[2], _stream())  # fmt: skip
+    native.check(rc, "tk_expert_kv_project")
+    return PrefixKV(k_hi, vt_hi, k_lo, vt_lo)
+
+
 def expert_attn(
     q: torch.Tensor,
     prefix: PrefixKV | None,

@@ -395,6 +395,12 @@ class SmolVLAModel:
         pos0 = pos - pos.min(dim=1, keepdim=True).values
         return pos, pos0
 
+    def _cross_cache(self, i: int, keys_i: torch.Tensor, values_i: torch.Tensor):
+        """Cross layer ``i``: fp32 expert K/V projection of the prefix ``[P, G, D]`` views, written as the
+        attention kernel's hi + lo planes by one launch."""
+        lp = f"{EXP}layers.{i}.self_attn."
+        return tk.project_prefix_kv(keys_i.flatten(1), values_i.flatten(1), self.p[lp + "k_proj.weight"], self.p[lp + "v_proj.weight"], self.head_dim)
+
     def attention_caches(self, keys, values, ekv, vt=None) -> list:
         """Per-layer prefix K/V in the attention kernel's layout, once per request: V transposed
         (self layers, bf16 cache; ``vt`` when the prefill already produced it) or K and V^T split
@@ -402,6 +408,9 @@ class SmolVLAModel:
         caches = []
         for i in range(self.num_layers):
             if self.cfg.is_cross_layer(i):
+                if ekv is None:  # projection and operand layout in one launch
+                    caches.append(self._cross_cache(i, keys[i, 0], values[i, 0]))
+                    continue
                 ek, ev = ekv[i]
                 caches.append(tk.prepare_prefix_kv(ek[0], ev[0]))
             elif vt is not None:
@@ -511,8 +520,7 @@ class SmolVLAModel:
             with torch.cuda.stream(side):
                 side.wait_event(done)
                 if self.cfg.is_cross_layer(i):
-                    ek, ev = self._expert_prefix_kv_layer(i, keys[i], values[i])
-                    caches[i] = tk.prepare_prefix_kv(ek[0], ev[0])
+                    caches[i] = self._cross_cache(i, keys[i, 0], values[i, 0])
                 else:
                     caches[i] = tk.PrefixKV(keys[i, 0], vt[i])
                 hid_s = self._denoise_layer_fused(i, hid_s, caches[i], pads[0], positions[0], positions[1], self.ws_side)
@@ -535,7 +543,9 @@ class SmolVLAModel:
             keys, values, vt = self.prefill_fused(embs, pads, att)
         else:
             keys, values = self.prefill(embs, pads, att)
-        ekv = self.expert_prefix_kv(keys, values)
+        fused = self.fused_expert and noise.shape[0] == 1
+        # the fused tier projects the cross layers' K/V inside attention_caches (one launch per layer)
+        ekv = None if fused and trace is None else self.expert_prefix_kv(keys, values)
         if trace is not None:
             trace.update(prefix_embs=embs, pad_masks=pads, keys=keys, values=values, ekv=ekv)
         dt = -1.0 / self.num_steps
