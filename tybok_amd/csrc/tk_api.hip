@@ -206,8 +206,9 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   if (ks <= 0) {
     // Launch-cost model (microseconds, measured per phase on MI355X): the k loop costs about
     // 0.35 per block round (NW k tiles) with a floor of one memory round trip; splitting K adds a
-    // partial write, an arrival count and a partial read-back (about 2 + 0.05 per split) and only
-    // pays while the grid still fits the device twice over.
+    // partial write, an arrival count and a read-back that the finishing block issues four splits at
+    // a time (about 1.2 + 0.9 per batch of four) and only pays while the grid still fits the device
+    // twice over.
     ks = 1;
     if (blocks0 < cus) {
       float best = 1e30f;
@@ -215,7 +216,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
         const int rounds = (a.KT + c * NW - 1) / (c * NW);
         float t = rounds * 0.35f;
         if (t < 1.0f) t = 1.0f;
-        if (c > 1) t += 2.0f + 0.05f * c;
+        if (c > 1) t += 1.2f + 0.9f * (float)((c + 3) / 4);
         if (t < best - 1e-3f) {
           best = t;
           ks = c;
