@@ -233,6 +233,21 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
 int tk_expert_kv_project(const void* k, const void* v, int sl, int P, int KV, const void* wk, const void* wv, int N,
                          void* k_hi, void* k_lo, void* vt_hi, void* vt_lo, int vt_ld, void* stream);
 
+/* Cross-attention layer of the action expert with the query projection inside the attention launch:
+ *   q = rope(bf16(RMSNorm(x) . Wq^T)) per head (bf16(w * bf16(x * rstd)) norm, fp32 half-split rotary
+ *   embedding with table rows rope_pos[m]), then attention over the fp32 (hi + lo planes) expert
+ *   prefix K/V under the prefix pad mask.  Replaces `triton_cross_attn` (norm + q projection + RoPE
+ *   + attention in one kernel: tybok/policies/smolvla/models/triton_attn.py:791-855; call site
+ *   vlm_with_expert.py:275-297) and equals tk_bf16w_linear (norm + q + RoPE) followed by tk_expert_attn.
+ *   x: bf16 [M, K] (row pitch ldx), K a multiple of 8 and at most 768; norm_w bf16 [K];
+ *   wq_packed: tk_pack_bf16_weight of the [H*D, K] q weight with rope_half = D/2;
+ *   D = 64; P at most 256 (8 key tiles: one block covers the prefix); K/V layouts, pad, out as tk_expert_attn. */
+int tk_expert_cross_attn_fused(const void* x, int ldx, const void* norm_w, float norm_eps, const void* wq_packed, int K,
+                               const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions,
+                               const void* k_hi, const void* k_lo, int pre_sl, int pre_sh, const void* vt_hi,
+                               const void* vt_lo, int pre_vt_sd, int pre_vt_sh, const void* pad, void* out, int out_sm,
+                               int M, int P, int H, int G, int D, void* stream);
+
 /* B independent unmasked attentions in one launch (the vision tower's self-attention, one problem
  * per camera image): out[b][M, H*D] = softmax(q[b].K[b]^T * D^-0.5) . V[b].  Layouts as the prefix
  * operands of tk_expert_attn (K [P, G, D]; V^T [G, D, >= P rounded up to 32], zero padded), with

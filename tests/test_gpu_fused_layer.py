@@ -238,3 +238,51 @@ def test_step_tail_norm_projection_euler(tk, adaptive):
     assert float((x_new.cpu() - x_want).abs().max()) < 2e-4, "Euler update differs"
     v_only, none = tk.expert_tail(x.cuda(), w.cuda(), b.cuda(), **kw)
     assert none is None and torch.equal(v_only, v)
+
+
+@pytest.mark.parametrize("m,p,k", [(50, 241, 720), (50, 177, 720), (7, 33, 96), (33, 256, 768)])
+def test_cross_layer_in_one_launch(tk, m, p, k):
+    # norm + q projection + RoPE inside the attention launch (SmolVLA cross layers: 15 / 5 heads of 64,
+    # fp32 expert K/V as hi + lo planes, prefix pad mask) against projecting first and attending afterwards,
+    # and against the CPU oracle's composition
+    heads, kv_heads, d, eps = 15, 5, 64, 1e-5
+    g = torch.Generator().manual_seed(51)
+    x = (torch.randn(m, k, generator=g) * 1.7).to(BF16)
+    norm_w = (1.0 + 0.2 * torch.randn(k, generator=g)).to(BF16)
+    wq = (torch.randn(heads * d, k, generator=g) * k**-0.5).to(BF16)
+    ek, ev = torch.randn(p, kv_heads, d, generator=g), torch.randn(p, kv_heads, d, generator=g)
+    pad = torch.rand(p, generator=g) > 0.2
+    pad[0] = True
+    pos = torch.randint(0, 300, (m,), generator=g, dtype=torch.int32)
+    rope = _tables(tk, 512, d // 2)
+    pw = tk.pack_bf16_weight(wq.cuda(), rope_half=d // 2)
+    cache = tk.prepare_prefix_kv(ek.cuda(), ev.cuda())
+    fused = tk.cross_attn_fused(x.cuda(), pw, norm_w.cuda(), eps, rope, pos.cuda(), cache, pad.cuda())
+    q = tk.bf16w_linear(x.cuda(), pw, norm_w=norm_w.cuda(), eps=eps, rope=rope, rope_pos=pos.cuda(), rope_cols=heads * d)
+    two = tk.expert_attn(q.view(m, heads, d), cache, None, pad.cuda(), tk.MASK_NONE)
+    _close(fused, two.cpu(), f"fused cross layer vs two launches M={m} P={p}")
+    same = (fused == two).float().mean().item()
+    assert same > 0.9, f"only {same:.1%} of the outputs agree bit for bit with the two-launch path"
+    assert torch.equal(fused, tk.cross_attn_fused(x.cuda(), pw, norm_w.cuda(), eps, rope, pos.cuda(), cache, pad.cuda()))
+    # oracle: RMSNorm -> q -> half-split RoPE -> eager attention over the fp32 K/V under the pad mask
+    h = oops.rms_norm_llama(x, norm_w, eps)
+    qo = oops.rope_half_split(F.linear(h, wq).view(1, m, heads, d), pos[None].long())
+    want = oops.eager_attention(pad[None, None, :].expand(1, m, p), qo, ek[None], ev[None])[0]
+    _close(fused, want, f"fused cross layer vs oracle M={m} P={p}")
+
+
+def test_cross_layer_in_one_launch_rejects_what_it_cannot_run(tk):
+    g = torch.Generator().manual_seed(52)
+    rope = _tables(tk, 64, 32)
+    x = torch.randn(8, 96, generator=g).to(BF16).cuda()
+    nw = torch.ones(96, dtype=BF16, device="cuda")
+    pw = tk.pack_bf16_weight(torch.randn(128, 96, generator=g).to(BF16).cuda(), rope_half=32)
+    pos = torch.zeros(8, dtype=torch.int32, device="cuda")
+    ok = tk.prepare_prefix_kv(torch.randn(40, 2, 64, generator=g).cuda(), torch.randn(40, 2, 64, generator=g).cuda())
+    with pytest.raises(ValueError):  # bf16 K/V: no lo planes
+        bf = tk.prepare_prefix_kv(torch.randn(40, 2, 64, generator=g).to(BF16).cuda(), torch.randn(40, 2, 64, generator=g).to(BF16).cuda())
+        tk.cross_attn_fused(x, pw, nw, 1e-5, rope, pos, bf, None)
+    with pytest.raises(RuntimeError, match="8 key tiles"):
+        big = tk.prepare_prefix_kv(torch.randn(300, 2, 64, generator=g).cuda(), torch.randn(300, 2, 64, generator=g).cuda())
+        tk.cross_attn_fused(x, pw, nw, 1e-5, rope, pos, big, None)
+    assert tk.cross_attn_fused(x, pw, nw, 1e-5, rope, pos, ok, None).shape == (8, 128)

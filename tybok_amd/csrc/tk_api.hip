@@ -465,6 +465,7 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   if (out_sm < H * D || out_sm % 4 || !aligned8(out)) return fail(TK_EINVAL, "attn: out_sm=%d must be >= H*D, a multiple of 4, out 8-byte aligned", out_sm);
 
   AttnArgs a;
+  memset(&a, 0, sizeof(a));
   a.q = (const u16*)q;
   a.q_sm = q_sm;
   a.q_sh = q_sh;
@@ -545,6 +546,61 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
   return attn_impl(0, 0, 0, 0, 0, q, q_sm, q_sh, k_pre, k_pre_lo, pre_sl, pre_sh, vt_pre, vt_pre_lo, pre_vt_sd, pre_vt_sh, k_suf,
                    suf_sl, suf_sh, vt_suf, suf_vt_sd, suf_vt_sh, pad, mask2d, mask_ld, out, out_sm, M, P, S, H, G, D, mask_mode,
                    logits_bf16, 0.f, ws, ws_bytes, stream);
+}
+
+int tk_expert_cross_attn_fused(const void* x, int ldx, const void* norm_w, float norm_eps, const void* wq_packed, int K,
+                               const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions,
+                               const void* k_hi, const void* k_lo, int pre_sl, int pre_sh, const void* vt_hi,
+                               const void* vt_lo, int pre_vt_sd, int pre_vt_sh, const void* pad, void* out, int out_sm,
+                               int M, int P, int H, int G, int D, void* stream) {
+  if (M <= 0 || P <= 0 || H <= 0 || G <= 0 || H % G) return fail(TK_EINVAL, "cross_attn_fused: bad shape M=%d P=%d H=%d G=%d", M, P, H, G);
+  if (D != 64) return fail(TK_EINVAL, "cross_attn_fused: head_dim %d (built for 64)", D);
+  if ((P + 31) / 32 > 8) return fail(TK_EINVAL, "cross_attn_fused: P=%d needs more than 8 key tiles (one block of 8 waves covers the prefix)", P);
+  if (K <= 0 || K % 8 || K > 768 || ldx < K || ldx % 8) return fail(TK_EINVAL, "cross_attn_fused: K=%d must be a multiple of 8, at most 768, ldx=%d >= K and a multiple of 8", K, ldx);
+  if (!x || !norm_w || !wq_packed || !rope_pos || !rope_cos || !rope_sin || rope_positions <= 0 || !k_hi || !k_lo || !vt_hi || !vt_lo || !out)
+    return fail(TK_EINVAL, "cross_attn_fused: null pointer");
+  if (pre_sl % 8 || pre_sh % 8 || pre_vt_sd % 8 || pre_vt_sh % 8) return fail(TK_EINVAL, "cross_attn_fused: strides must be multiples of 8 elements");
+  if (!aligned16(x) || !aligned16(norm_w) || !aligned16(wq_packed) || !aligned16(rope_cos) || !aligned16(rope_sin) || !aligned16(k_hi) ||
+      !aligned16(k_lo) || !aligned16(vt_hi) || !aligned16(vt_lo))
+    return fail(TK_EINVAL, "cross_attn_fused: operands must be 16-byte aligned");
+  if (pre_vt_sd < ((P + 31) / 32) * 32) return fail(TK_EINVAL, "cross_attn_fused: a V^T row must hold P rounded up to 32 keys (zero padded)");
+  if (out_sm < H * D || out_sm % 4 || !aligned8(out)) return fail(TK_EINVAL, "cross_attn_fused: out_sm=%d must be >= H*D, a multiple of 4, out 8-byte aligned", out_sm);
+  AttnArgs a;
+  memset(&a, 0, sizeof(a));
+  a.q = (const u16*)x;  // never read as queries; keeps the kernel's dummy operand address valid
+  a.k_pre = (const u16*)k_hi;
+  a.k_pre_lo = (const u16*)k_lo;
+  a.vt_pre = (const u16*)vt_hi;
+  a.vt_pre_lo = (const u16*)vt_lo;
+  a.pre_sl = pre_sl;
+  a.pre_sh = pre_sh;
+  a.pre_vt_sd = pre_vt_sd;
+  a.pre_vt_sh = pre_vt_sh;
+  a.pad = (const uint8_t*)pad;
+  a.out = (u16*)out;
+  a.out_sm = out_sm;
+  a.M = M;
+  a.P = P;
+  a.H = H;
+  a.G = G;
+  a.mask_mode = TK_MASK_NONE;
+  a.scale = 1.0f / sqrtf((float)D);
+  a.kv_splits = 1;
+  a.tile_q = (P + 31) / 32;
+  a.gqa_mul = (65536 + H / G - 1) / (H / G);
+  a.qp_x = (const u16*)x;
+  a.qp_ldx = ldx;
+  a.qp_norm_w = (const u16*)norm_w;
+  a.qp_eps = norm_eps;
+  a.qp_w = (const uint8_t*)wq_packed;
+  a.qp_K = K;
+  a.qp_KT = (K + 31) / 32;
+  a.qp_rope_pos = (const int*)rope_pos;
+  a.qp_cos = (const float*)rope_cos;
+  a.qp_sin = (const float*)rope_sin;
+  a.qp_positions = rope_positions;
+  if (tk_launch_attn_qproj(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "cross_attn_fused: launch failed (%s)", hipGetErrorString(hipGetLastError()));
+  return TK_OK;
 }
 
 int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const void* k, long long k_sb, int k_sl, int k_sh,

@@ -77,6 +77,19 @@ struct AttnArgs {
   float* partial;
   int* counters;
   float scale;
+  // in-kernel query projection (cross layers; nullptr / 0 otherwise): hidden rows bf16 [M, qp_ldx],
+  // RMSNorm weight bf16 [qp_K], packed bf16 q weight (rotary pair order, tiles of 2 KiB, qp_KT k
+  // tiles per n tile), rotary tables fp32 [qp_positions, D/2] and int32 positions [M]
+  const unsigned short* qp_x;
+  int qp_ldx;
+  const unsigned short* qp_norm_w;
+  float qp_eps;
+  const uint8_t* qp_w;
+  int qp_K, qp_KT;
+  const int* qp_rope_pos;
+  const float* qp_cos;
+  const float* qp_sin;
+  int qp_positions;
 };
 
 struct KvPrepArgs {
@@ -147,4 +160,5 @@ int tk_launch_fill_zero(int* p, int n, hipStream_t st);
 int tk_launch_decode_fp8(float* out, hipStream_t st);
 int tk_attn_waves(int D, int split_planes, int ntiles);
 int tk_launch_attn(AttnArgs a, int D, int waves, hipStream_t st);
+int tk_launch_attn_qproj(AttnArgs a, hipStream_t st);
 int tk_launch_kv_prepare(KvPrepArgs p, hipStream_t st);

@@ -490,6 +490,60 @@ def expert_attn(
     return out
 
 
+CROSS_FUSED_MAX_K = 768    # widest hidden size the in-kernel q projection stages
+CROSS_FUSED_MAX_P = 256    # 8 key tiles: one block of 8 waves covers the prefix
+
+
+def cross_attn_fused(
+    x: torch.Tensor,
+    wq: PackedBf16Weight,
+    norm_w: torch.Tensor,
+    eps: float,
+    rope: RopeTables,
+    rope_pos: torch.Tensor,
+    prefix: PrefixKV,
+    prefix_pad: torch.Tensor | None,
+    *,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Cross layer in one launch: ``q = rope(RMSNorm(x) @ Wq^T)`` computed per head inside the
+    attention kernel, then attention over the fp32 (hi + lo planes) prefix ``K/V`` under the pad
+    mask.  ``x [M, K]`` bf16 (``K <= 768``), ``wq`` packed with ``rope_half = 32`` (head size 64),
+    ``prefix`` from :func:`project_prefix_kv` / :func:`prepare_prefix_kv` of fp32 tensors with at most
+    256 keys.  Returns bf16 ``[M, H*64]``; equals :func:`bf16w_linear` + :func:`expert_attn`."""
+    lib = native.lib()
+    bf = torch.bfloat16
+    if x.dtype != bf or x.dim() != 2 or x.stride(1) != 1 or norm_w.dtype != bf:
+        raise TypeError("cross_attn_fused: x [M, K] and norm_w must be bf16, x rows contiguous")
+    m, k = x.shape
+    if wq.k != k or norm_w.numel() != k or wq.rope_half != 32 or wq.n % 64:
+        raise ValueError("cross_attn_fused: wq must be the [H*64, K] q weight packed with rope_half=32")
+    if prefix.k_lo is None or prefix.vt_lo is None:
+        raise ValueError("cross_attn_fused: the prefix must carry hi + lo planes (fp32 expert K/V)")
+    h, d = wq.n // 64, 64
+    p, g = prefix.k.shape[0], prefix.k.shape[1]
+    if prefix.k.shape[2] != d or prefix.k_lo.stride() != prefix.k.stride() or prefix.vt_lo.stride() != prefix.vt.stride():
+        raise ValueError("cross_attn_fused: prefix planes must be [P, G, 64] / [G, 64, >= P rounded up to 32] with mirrored layouts")
+    if rope_pos.dtype != torch.int32 or rope_pos.numel() != m or not rope_pos.is_contiguous():
+        raise ValueError("cross_attn_fused: rope_pos must be a contiguous int32 [M]")
+    pad = None
+    if prefix_pad is not None:
+        pad = prefix_pad.view(torch.uint8) if prefix_pad.dtype == torch.bool else prefix_pad
+        if pad.dtype != torch.uint8 or pad.numel() != p or not pad.is_contiguous():
+            raise ValueError("prefix_pad must be a contiguous uint8/bool [P]")
+    if out is None:
+        out = torch.empty(m, h * d, dtype=bf, device=x.device)
+    pre_sl, pre_sh = _eff_strides(prefix.k)
+    rc = lib.tk_expert_cross_attn_fused(
+        x.data_ptr(), x.stride(0), norm_w.data_ptr(), float(eps), wq.data.data_ptr(), k, rope_pos.data_ptr(), rope.cos.data_ptr(),
+        rope.sin.data_ptr(), rope.cos.shape[0], prefix.k.data_ptr(), prefix.k_lo.data_ptr(), pre_sl, pre_sh, prefix.vt.data_ptr(),
+        prefix.vt_lo.data_ptr(), prefix.vt.stride(1), prefix.vt.stride(0) if g > 1 else 0, _ptr(pad), out.data_ptr(), out.stride(0),
+        m, p, h, g, d, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_expert_cross_attn_fused")
+    return out
+
+
 def batched_attn(
     q: torch.Tensor,
     k: torch.Tensor,

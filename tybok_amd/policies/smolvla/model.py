@@ -139,6 +139,7 @@ class SmolVLAModel:
         # prefill x step-0 overlap (flow_matching.py:455-531): step-0 expert layer i runs on a second
         # stream as soon as prefill layer i has produced its K/V.  Kernels that may run at the same
         # time must not share split-K partials / counters: the side stream has its own workspace.
+        self.fuse_cross_q = True  # cross layers: q projection inside the attention launch (tk.cross_attn_fused)
         self.overlap = bool(overlap) and self.fused_prefill and self.fused_expert
         self.side_stream = torch.cuda.Stream(self.device) if self.overlap else None
         self.ws_side = tk.Workspace(self.device) if self.overlap else None
@@ -419,6 +420,14 @@ class SmolVLAModel:
                 caches.append(tk.prepare_prefix_kv(keys[i, 0], values[i, 0]))
         return caches
 
+    def _cross_fusable(self, hidden: torch.Tensor, cache) -> bool:
+        """The one-launch cross layer applies: bf16 hidden rows, head size 64, fp32 (hi + lo) prefix planes
+        that one block covers."""
+        return (
+            self.fuse_cross_q and hidden.dtype == BF16 and self.head_dim == 64 and hidden.shape[1] <= tk.CROSS_FUSED_MAX_K
+            and cache.k_lo is not None and cache.k.shape[0] <= tk.CROSS_FUSED_MAX_P
+        )  # fmt: skip
+
     def _denoise_layer_fused(self, i: int, hidden: torch.Tensor, cache, pad, pos32, pos0_32, ws) -> torch.Tensor:
         """Expert layer ``i`` on the fused launches (``hidden [S, E]``: fp32 into layer 0, bf16 after)."""
         h_q, h_kv, d = self.heads, self.kv_heads, self.head_dim
@@ -426,17 +435,22 @@ class SmolVLAModel:
         s = hidden.shape[0]
         lp = f"{EXP}layers.{i}."
         cross = self.cfg.is_cross_layer(i)
-        qkv = tk.bf16w_linear(
-            hidden, self.exp_qkv[i], norm_w=self.p[lp + "input_layernorm.weight"], eps=self.eps, rope=self.rope_tables,
-            rope_pos=pos0_32 if cross else pos32, rope_cols=nq if cross else nq + nkv,
-            vt_out=None if cross else self.vt_suf.view(nkv, -1), vt_col0=nq + nkv, ws=ws,
-        )  # fmt: skip
-        q = qkv[:, :nq].view(s, h_q, d)
-        if cross:
-            att = tk.expert_attn(q, cache, None, pad, tk.MASK_NONE, ws=ws)
+        norm_w = self.p[lp + "input_layernorm.weight"]
+        if cross and self._cross_fusable(hidden, cache):
+            # norm + q projection + RoPE inside the attention launch
+            att = tk.cross_attn_fused(hidden, self.exp_qkv[i], norm_w, self.eps, self.rope_tables, pos0_32, cache, pad)
         else:
-            suffix = tk.SuffixKV(qkv[:, nq : nq + nkv].view(s, h_kv, d), self.vt_suf)
-            att = tk.expert_attn(q, cache, suffix, pad, tk.MASK_CAUSAL, ws=ws)
+            qkv = tk.bf16w_linear(
+                hidden, self.exp_qkv[i], norm_w=norm_w, eps=self.eps, rope=self.rope_tables,
+                rope_pos=pos0_32 if cross else pos32, rope_cols=nq if cross else nq + nkv,
+                vt_out=None if cross else self.vt_suf.view(nkv, -1), vt_col0=nq + nkv, ws=ws,
+            )  # fmt: skip
+            q = qkv[:, :nq].view(s, h_q, d)
+            if cross:
+                att = tk.expert_attn(q, cache, None, pad, tk.MASK_NONE, ws=ws)
+            else:
+                suffix = tk.SuffixKV(qkv[:, nq : nq + nkv].view(s, h_kv, d), self.vt_suf)
+                att = tk.expert_attn(q, cache, suffix, pad, tk.MASK_CAUSAL, ws=ws)
         out = tk.bf16w_linear(att, self.exp_o[i], resid=hidden, ws=ws)
         mlp = self.exp_mlp[i]
         post_w = self.p[lp + "post_attention_layernorm.weight"]
