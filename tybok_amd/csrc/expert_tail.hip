@@ -15,7 +15,7 @@ namespace {
 constexpr int kThreads = 256;
 
 __global__ __launch_bounds__(kThreads) void expert_tail_kernel(TailArgs a) {
-  extern __shared__ float hrow[];  // [K] normalised row, as fp32 values of bf16 numbers
+  extern __shared__ __align__(16) float hrow[];  // [K] normalised row, as fp32 values of bf16 numbers
   __shared__ float red[kThreads / 64];
   __shared__ float part[kThreads];
   const int m = blockIdx.x;
@@ -54,9 +54,20 @@ __global__ __launch_bounds__(kThreads) void expert_tail_kernel(TailArgs a) {
   const int slices = kThreads / a.N;  // host guarantees N divides kThreads and N <= kThreads
   const int n = tid / slices, sl = tid % slices;
   const float* w = a.w + (size_t)n * a.K;
-  float acc = 0.f;
-  for (int k = sl; k < a.K; k += slices) acc = fmaf(hrow[k], w[k], acc);
-  part[tid] = acc;
+  // 16-byte pieces: the slices of an output read consecutive pieces, each thread several in flight
+  // (K is a multiple of 4: checked by the host)
+  float acc0 = 0.f, acc1 = 0.f;
+  const int pieces = a.K / 4;
+#pragma unroll 8
+  for (int p = sl; p < pieces; p += slices) {
+    const f32x4 wv = *(const f32x4*)(w + 4 * p);
+    const f32x4 hv = *(const f32x4*)(hrow + 4 * p);
+    acc0 = fmaf(hv[0], wv[0], acc0);
+    acc1 = fmaf(hv[1], wv[1], acc1);
+    acc0 = fmaf(hv[2], wv[2], acc0);
+    acc1 = fmaf(hv[3], wv[3], acc1);
+  }
+  part[tid] = acc0 + acc1;
   __syncthreads();
   if (sl == 0) {
     float v = 0.f;

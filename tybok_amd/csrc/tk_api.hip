@@ -618,7 +618,8 @@ int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_s
                    void* stream) {
   if (M <= 0 || N <= 0 || K <= 0 || ldx < K) return fail(TK_EINVAL, "tail: bad shape M=%d N=%d K=%d ldx=%d", M, N, K, ldx);
   if (N > 256 || 256 % N) return fail(TK_EINVAL, "tail: N=%d must divide 256", N);
-  if (K > 16384) return fail(TK_EINVAL, "tail: K=%d too large for the row buffer", K);
+  if (K > 16384 || K % 4) return fail(TK_EINVAL, "tail: K=%d must be a multiple of 4 and at most 16384", K);
+  if (!aligned16(w)) return fail(TK_EINVAL, "tail: w must be 16-byte aligned");
   if (!x || !w || (!norm_w && !(ada_scale && ada_shift)) || (norm_w && (ada_scale || ada_shift)))
     return fail(TK_EINVAL, "tail: needs x, w and exactly one of norm_w or ada_scale + ada_shift");
   if (x_out && !x_t) return fail(TK_EINVAL, "tail: x_out needs x_t");
