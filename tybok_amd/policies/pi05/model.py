@@ -329,7 +329,7 @@ class PI05Model:
         g = self.vt_suf.shape[0]
         nq, nkv = heads * d, g * d
         s = hidden.shape[0]
-        pos32 = pos[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
+        pos32 = pos if pos.dtype == torch.int32 else pos[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
         pad = prefix_pad[0]
         for i in range(self.ed["depth"]):
             (sc_in, sh_in, gate_in), (sc_post, sh_post, gate_post) = self.mods_split[step][i]
@@ -404,6 +404,21 @@ class PI05Model:
         x_t = noise
         if caches is None or not self.fused_expert:
             caches = self.attention_caches(kv) if self.fused_expert else None
+        if self.fused_expert and x_t.shape[0] == 1 and x_t.dtype == torch.float32 and x_t.is_contiguous() and all(m.fp8 for m in self.exp_mlp):
+            # fused loop: positions once per request, Euler update inside the step's last launch
+            s = x_t.shape[1]
+            if self.vt_suf is None or self.vt_suf.shape[2] < (s + 31) // 32 * 32:
+                self.vt_suf = torch.zeros(kv[0][0].shape[1], self.head_dim, (s + 31) // 32 * 32, dtype=BF16, device=self.device)
+            pos32 = (pads.sum(dim=-1)[:, None] + torch.arange(s, device=self.device)[None, :])[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
+            for step in range(self.num_steps):
+                hidden = self.lin("action_in_proj", x_t)[0].to(BF16)
+                hidden = self._denoise_layers_fused(pads, caches, hidden, pos32, step)
+                _, x_new = tk.expert_tail(
+                    hidden, self.p["action_out_proj.weight"], self.p["action_out_proj.bias"], ada=self.final_split[step], eps=EPS,
+                    x_t=x_t[0], dt=dt,
+                )  # fmt: skip
+                x_t = x_new[None]
+            return x_t
         for step in range(self.num_steps):
             x_t = x_t + dt * self.denoise_step(pads, kv, x_t, step, caches)
         return x_t
