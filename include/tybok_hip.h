@@ -261,6 +261,16 @@ int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const voi
                     int M, int P, int H, int G, int D, int logits_bf16, float scale, void* ws, size_t ws_bytes,
                     void* stream);
 
+/* ---- vision tower glue ------------------------------------------------------------------------ */
+/* LayerNorm of token rows with the cast to the GEMM input type folded in:
+ *   y[m, :] = bf16((x[m, :] - mean) * rstd * w + b), statistics in fp32 (biased variance).
+ * Replaces `layer_norm1/2(x)` (+ the `.to(bf16)` of the low-precision tiers) in the encoder layers
+ * (tybok/policies/pi05/models/vision.py:115-170, tybok/policies/smolvla/models/vision.py:197-257).
+ *   x: fp32 or bf16 [M, K] (x_dtype, element pitch ldx); w, b: [K] of the same type (wb_dtype);
+ *   y: bf16 [M, K] (pitch ldy); K a multiple of 8, at most 2048; pitches multiples of 8; 16-byte aligned. */
+int tk_layer_norm(const void* x, int ldx, int x_dtype, const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy,
+                  int M, int K, void* stream);
+
 /* ---- tail of a denoising step ---------------------------------------------------------------- */
 /* Final norm of the expert hidden state + fp32 action projection + Euler update in one launch:
  *   h = norm(x) (bf16 row; norm_w: Llama RMSNorm bf16(w * bf16(x * rstd)); or ada_scale / ada_shift:

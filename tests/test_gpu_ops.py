@@ -283,6 +283,25 @@ def test_expert_kv_projection_into_attention_planes(tk, p, kv, n, d):
     _close(a, b.cpu(), "attention over projected planes")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,k", [(512, 1152), (3072, 768), (5, 8), (131, 2048)])
+def test_layer_norm_with_folded_cast(tk, dtype, m, k):
+    # F.layer_norm in fp32 statistics, result rounded once to bf16 -- for fp32 rows (pi0.5 tower, followed
+    # by .to(bf16) in the reference's low-precision tiers) and bf16 rows (SmolVLA tower)
+    g = torch.Generator().manual_seed(61)
+    x = (torch.randn(m, k, generator=g) * 3.0 + 0.5).to(dtype)
+    w, b = (1.0 + 0.3 * torch.randn(k, generator=g)).to(dtype), (0.2 * torch.randn(k, generator=g)).to(dtype)
+    want = torch.nn.functional.layer_norm(x.float(), (k,), w.float(), b.float(), 1e-6).to(torch.bfloat16)
+    got = tk.layer_norm(x.cuda(), w.cuda(), b.cuda(), 1e-6)
+    assert got.dtype == torch.bfloat16 and got.shape == x.shape
+    diff = (got.float().cpu() - want.float()).abs()
+    ulp = want.float().abs().clamp_min(2.0**-6) * 2.0**-7  # one bf16 step at the value's magnitude
+    assert bool((diff <= ulp).all()), f"max |err| {float(diff.max()):.4g}: more than one bf16 step from the fp32 LayerNorm"
+    assert float((diff > 0).float().mean()) < 0.02, "more than 2% of the outputs differ from the fp32 LayerNorm rounded once"
+    with pytest.raises(TypeError):
+        tk.layer_norm(x.cuda(), w.float().cuda(), b.half().cuda(), 1e-6)
+
+
 def test_gated_residual_epilogue(tk):
     # pi0.5 AdaRMS gated residual: y = resid + bf16(ffn(x) * gate)
     x, wg8, sg, wu8, su, wd8, sd = ffn_case(50, 1024, 4096, seed=3)

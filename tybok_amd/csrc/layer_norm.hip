@@ -1,0 +1,106 @@
+// LayerNorm of the vision towers' token rows with the cast to the GEMM input type folded in:
+//   y[m, :] = bf16((x[m, :] - mean) * rstd * w + b),   mean / biased variance / rstd in fp32
+// for fp32 rows with fp32 parameters (SigLIP tower of pi0.5: F.layer_norm(x) followed by .to(bf16),
+// tybok/policies/pi05/models/vision.py:115-170) or bf16 rows with bf16 parameters (SmolVLA's tower,
+// which torch normalises in fp32 and rounds once: tybok/policies/smolvla/models/vision.py:197-257).
+// One wave per row, the row stays in registers between the mean, variance and output passes; sums
+// by wave shuffles in a fixed order.
+#include "tk_common.h"
+#include "tk_kernels.h"
+
+namespace {
+
+constexpr int PMAX = 4;  // 8-element pieces per lane: rows up to 64 * 8 * PMAX = 2048 columns
+
+template <bool XF32, bool WF32>
+__global__ __launch_bounds__(256) void layer_norm_kernel(LayerNormArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.M) return;
+  const int pieces = a.K / 8;
+  float v[PMAX][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < PMAX; ++i) {
+    const int p = lane + 64 * i;
+    if (p < pieces) {
+      if (XF32) {
+        const f32x4* src = (const f32x4*)((const float*)a.x + (size_t)row * a.ldx + 8 * p);
+        const f32x4 lo = src[0], hi = src[1];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { v[i][e] = lo[e]; v[i][4 + e] = hi[e]; }
+      } else {
+        union { i32x4 q; unsigned u[4]; } xu;
+        xu.q = *(const i32x4*)((const u16*)a.x + (size_t)row * a.ldx + 8 * p);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[i][2 * e] = __uint_as_float(xu.u[e] << 16);
+          v[i][2 * e + 1] = __uint_as_float(xu.u[e] & 0xffff0000u);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum += v[i][e];
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+  const float mean = sum / (float)a.K;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < PMAX; ++i)
+    if (lane + 64 * i < pieces) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = v[i][e] - mean;
+        sq = fmaf(d, d, sq);
+      }
+    }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
+  const float rstd = rsqrtf(sq / (float)a.K + a.eps);
+#pragma unroll
+  for (int i = 0; i < PMAX; ++i) {
+    const int p = lane + 64 * i;
+    if (p < pieces) {
+      float w[8], b[8];
+      if (WF32) {
+        const f32x4* wp = (const f32x4*)((const float*)a.w + 8 * p);
+        const f32x4* bp = (const f32x4*)((const float*)a.b + 8 * p);
+        const f32x4 w0 = wp[0], w1 = wp[1], b0 = bp[0], b1 = bp[1];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { w[e] = w0[e]; w[4 + e] = w1[e]; b[e] = b0[e]; b[4 + e] = b1[e]; }
+      } else {
+        union { i32x4 q; unsigned u[4]; } wu, bu;
+        wu.q = *(const i32x4*)((const u16*)a.w + 8 * p);
+        bu.q = *(const i32x4*)((const u16*)a.b + 8 * p);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          w[2 * e] = __uint_as_float(wu.u[e] << 16);
+          w[2 * e + 1] = __uint_as_float(wu.u[e] & 0xffff0000u);
+          b[2 * e] = __uint_as_float(bu.u[e] << 16);
+          b[2 * e + 1] = __uint_as_float(bu.u[e] & 0xffff0000u);
+        }
+      }
+      union { i32x4 q; unsigned u[4]; } o4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        o4.u[e] = pack_bf16x2((v[i][2 * e] - mean) * rstd * w[2 * e] + b[2 * e], (v[i][2 * e + 1] - mean) * rstd * w[2 * e + 1] + b[2 * e + 1]);
+      *(i32x4*)(a.y + (size_t)row * a.ldy + 8 * p) = o4.q;
+    }
+  }
+}
+
+}  // namespace
+
+int tk_layer_norm_max_k() { return 64 * 8 * PMAX; }
+
+int tk_launch_layer_norm(LayerNormArgs a, hipStream_t st) {
+  dim3 grid((a.M + 3) / 4);
+  if (a.x_f32 && a.wb_f32)
+    hipLaunchKernelGGL((layer_norm_kernel<true, true>), grid, dim3(256), 0, st, a);
+  else if (!a.x_f32 && !a.wb_f32)
+    hipLaunchKernelGGL((layer_norm_kernel<false, false>), grid, dim3(256), 0, st, a);
+  else
+    return -1;
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}

@@ -644,6 +644,28 @@ int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_s
   return TK_OK;
 }
 
+int tk_layer_norm(const void* x, int ldx, int x_dtype, const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy,
+                  int M, int K, void* stream) {
+  if (M <= 0 || K <= 0 || K % 8 || K > tk_layer_norm_max_k()) return fail(TK_EINVAL, "layer_norm: K=%d must be a multiple of 8, at most %d", K, tk_layer_norm_max_k());
+  if ((x_dtype != TK_BF16 && x_dtype != TK_F32) || x_dtype != wb_dtype) return fail(TK_EINVAL, "layer_norm: rows and parameters must both be bf16 or both fp32");
+  if (!x || !w || !b || !y || ldx < K || ldy < K || ldx % 8 || ldy % 8) return fail(TK_EINVAL, "layer_norm: null pointer or row pitch not a multiple of 8 >= K");
+  if (!aligned16(x) || !aligned16(w) || !aligned16(b) || !aligned16(y)) return fail(TK_EINVAL, "layer_norm: operands must be 16-byte aligned");
+  LayerNormArgs a;
+  a.x = x;
+  a.ldx = ldx;
+  a.x_f32 = x_dtype == TK_F32;
+  a.w = w;
+  a.b = b;
+  a.wb_f32 = wb_dtype == TK_F32;
+  a.eps = eps;
+  a.y = (u16*)y;
+  a.ldy = ldy;
+  a.M = M;
+  a.K = K;
+  if (tk_launch_layer_norm(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "layer_norm: launch failed");
+  return TK_OK;
+}
+
 int tk_debug_decode_fp8(void* out_f32, void* stream) {
   if (!out_f32) return fail(TK_EINVAL, "decode: null pointer");
   if (tk_launch_decode_fp8((float*)out_f32, (hipStream_t)stream)) return fail(TK_ELAUNCH, "decode: launch failed");

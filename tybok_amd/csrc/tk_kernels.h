@@ -119,6 +119,18 @@ struct KvProjArgs {
   int ld;
 };
 
+struct LayerNormArgs {
+  const void* x;  // fp32 (x_f32) or bf16 [M, K] rows, element pitch ldx
+  int ldx, x_f32;
+  const void* w;  // fp32 (wb_f32) or bf16 [K]
+  const void* b;
+  int wb_f32;
+  float eps;
+  unsigned short* y;  // bf16 [M, K], element pitch ldy
+  int ldy;
+  int M, K;
+};
+
 struct TailArgs {
   const unsigned short* x;  // bf16 [M, K]
   int ldx;
@@ -149,6 +161,8 @@ struct NormRowsArgs {
 
 int tk_launch_tail(TailArgs a, hipStream_t st);
 int tk_launch_kv_proj(KvProjArgs a, hipStream_t st);
+int tk_layer_norm_max_k();
+int tk_launch_layer_norm(LayerNormArgs a, hipStream_t st);
 int tk_wide_rows();  // block tile of the many-row GEMM
 int tk_wide_cols();
 int tk_launch_gemm_wide(GemmArgs a, hipStream_t st);

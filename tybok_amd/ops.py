@@ -640,6 +640,24 @@ def expert_tail(
     return v, x_new
 
 
+def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) -> torch.Tensor:
+    """``bf16(LayerNorm(x) * w + b)`` over the last dim of ``x [..., K]`` (fp32 with fp32 parameters, or
+    bf16 with bf16 parameters; contiguous rows), statistics in fp32.  One launch, bf16 result."""
+    lib = native.lib()
+    if x.dtype not in (torch.float32, torch.bfloat16) or w.dtype != x.dtype or b.dtype != x.dtype:
+        raise TypeError("layer_norm: x, w, b must all be fp32 or all bf16")
+    k = x.shape[-1]
+    x2 = x.reshape(-1, k)
+    if x2.stride(1) != 1 or w.numel() != k or b.numel() != k:
+        raise ValueError("layer_norm: rows must be contiguous and w, b hold K values")
+    y = torch.empty(x2.shape, dtype=torch.bfloat16, device=x.device)
+    dt = _F32 if x.dtype == torch.float32 else _BF16
+    rc = lib.tk_layer_norm(x2.data_ptr(), x2.stride(0), dt, w.contiguous().data_ptr(), b.contiguous().data_ptr(), dt, float(eps),
+                           y.data_ptr(), y.stride(0), x2.shape[0], k, _stream())  # fmt: skip
+    native.check(rc, "tk_layer_norm")
+    return y.view(x.shape)
+
+
 def decode_fp8_table(device: torch.device | str = "cuda") -> torch.Tensor:
     """Values of all 256 e4m3fn codes as the device's conversion instruction decodes them."""
     out = torch.empty(256, dtype=torch.float32, device=device)

@@ -214,28 +214,35 @@ class PI05Model:
         hd = vh // heads
         for i in range(cfg.vision_layers):
             lp = f"{VIS}encoder.layers.{i}."
-            h = F.layer_norm(x, (vh,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], EPS)
             if self.vit_lowp_attn:
-                # bf16 projections (one packed q|k|v GEMM), then the HIP attention, one problem per image:
-                # fp32 scores and softmax, probabilities rounded to bf16 for P.V (fp32 accumulate)
+                # LayerNorm + cast in one launch, bf16 projections (one packed q|k|v GEMM), then the HIP
+                # attention, one problem per image: fp32 scores and softmax, probabilities rounded to bf16
+                # for P.V (fp32 accumulate)
                 hp = self.vis_head_pad
-                qkv = F.linear(h.to(BF16), *self.vis_lowp[lp + "self_attn.qkv"]).view(b, -1, 3, heads, hp)
+                h = tk.layer_norm(x, p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], EPS)
+                qkv = F.linear(h, *self.vis_lowp[lp + "self_attn.qkv"]).view(b, -1, 3, heads, hp)
                 vt = qkv[:, :, 2].permute(0, 2, 3, 1).contiguous()
                 a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, scale=hd**-0.5, ws=self.ws)
-                x = x + F.linear(a, *self.vis_lowp[lp + "self_attn.out_proj"]).float()
+                x = x + F.linear(a, *self.vis_lowp[lp + "self_attn.out_proj"])  # fp32 + bf16: promoted inside the add
             else:
+                h = F.layer_norm(x, (vh,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], EPS)
                 q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
                 k = self.lin(lp + "self_attn.k_proj", h).view(b, -1, heads, hd).transpose(1, 2)
                 v = self.lin(lp + "self_attn.v_proj", h).view(b, -1, heads, hd).transpose(1, 2)
                 att = torch.softmax(torch.matmul(q, k.transpose(2, 3)) * hd**-0.5, dim=-1)
                 a = torch.matmul(att, v).transpose(1, 2).reshape(b, -1, vh)
                 x = x + self.lin(lp + "self_attn.out_proj", a)
-            h = F.layer_norm(x, (vh,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS)
             if self.vit_mlp_dtype is not None:
-                # MLP-only low precision: fc1, gelu and fc2 in that dtype, cast at the boundary
-                m = F.gelu(F.linear(h.to(self.vit_mlp_dtype), *self.vis_lowp[lp + "mlp.fc1"]), approximate="tanh")
-                x = x + F.linear(m, *self.vis_lowp[lp + "mlp.fc2"]).float()
+                # MLP-only low precision: fc1, gelu and fc2 in that dtype, cast at the boundary (for bf16 on a
+                # GPU the LayerNorm and the cast are one launch)
+                if self.vit_mlp_dtype == BF16 and x.is_cuda:
+                    h = tk.layer_norm(x, p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS)
+                else:
+                    h = F.layer_norm(x, (vh,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS).to(self.vit_mlp_dtype)
+                m = F.gelu(F.linear(h, *self.vis_lowp[lp + "mlp.fc1"]), approximate="tanh")
+                x = x + F.linear(m, *self.vis_lowp[lp + "mlp.fc2"])  # fp32 + low precision: promoted inside the add
             else:
+                h = F.layer_norm(x, (vh,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS)
                 x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
         x = F.layer_norm(x, (vh,), p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], EPS)
         return self.lin(PROJ, x)

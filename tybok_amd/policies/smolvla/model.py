@@ -239,8 +239,8 @@ class SmolVLAModel:
         hd = v.hidden_size // heads
         for i in range(v.num_hidden_layers):
             lp = f"{VIS}encoder.layers.{i}."
-            h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], v.layer_norm_eps)
             if self.fused_vit:
+                h = tk.layer_norm(x, p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], v.layer_norm_eps)
                 # packed q|k|v GEMM, then the HIP attention (one problem per camera): q.K^T rounded to
                 # bf16 before the fp32 scale and softmax, exactly what the bf16 matmul below produces
                 w_qkv, b_qkv = self.vis_qkv[i]
@@ -248,9 +248,10 @@ class SmolVLAModel:
                 vt = qkv[:, :, 2].permute(0, 2, 3, 1).contiguous()
                 a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, ws=self.ws)
                 x = x + self.lin(lp + "self_attn.out_proj", a)
-                h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
+                h = tk.layer_norm(x, p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
                 x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
                 continue
+            h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], v.layer_norm_eps)
             q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
             k = self.lin(lp + "self_attn.k_proj", h).view(b, -1, heads, hd).transpose(1, 2)
             val = self.lin(lp + "self_attn.v_proj", h).view(b, -1, heads, hd).transpose(1, 2)
