@@ -137,3 +137,55 @@ def test_engine_api_and_graph_equals_eager(ckpt):
     with pytest.raises(ValueError):
         create_engine(ckpt, device="cuda", warmup=False, vit_mlp_dtype="fp8")
     assert create_engine(ckpt, device="cuda", warmup=False, vit_mlp_dtype="fp16").model.vit_mlp_dtype == torch.float16
+
+
+def test_validate_against_an_oracle_dump(ckpt, tmp_path):
+    # `engine.validate(reference_dir)` (pi05/engine.py:740-857): the dump directory is written here by the CPU
+    # oracle -- frame, preprocessed batch, prefix embedding, per-layer prefix K/V, one velocity evaluation at
+    # t = 0.5 (off this checkpoint's 3-step Euler grid), the zero-noise chunk -- and every component must agree.
+    from tybok_amd.policies.pi05.weights import random_state_dict
+    from tybok_amd.registry import create_engine
+
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_flash_attn=True)
+    eng = create_engine(ckpt, device="cuda", graph=True, warmup=True, **flags)
+    cfg = eng.config
+    frame = eng._profile_frame(seed=12)
+    with torch.inference_mode():
+        batch = {k: v.cpu() for k, v in eng._batch_from_frame(frame).items() if isinstance(v, torch.Tensor)}
+        images, masks = eng.prepare_images(batch)
+    shape = _shape(cfg)
+    w = Weights(random_state_dict(cfg, seed=6), O.fp8_linear_names(shape, True, True))
+    tokens, lang_masks = batch["observation.language.tokens"], batch["observation.language.attention_mask"]
+    a_dim = cfg.action_feature_shape[0]
+    with torch.no_grad():
+        embs, pads, att = O.embed_prefix(w, shape, images, masks, tokens, lang_masks)
+        kv = O.prefill(w, shape, embs, pads, att)
+        zeros = torch.zeros(1, cfg.chunk_size, cfg.max_action_dim)
+        v_t = O.denoise_step(w, shape, pads, kv, zeros, 0.5)
+        chunk = O.sample_actions(w, shape, images, masks, tokens, lang_masks, zeros)[:, :, :a_dim]
+    post = eng.unnormalizer.unnormalize(chunk.cuda(), "action", "ACTION").cpu()
+    d = str(tmp_path)
+    torch.save({k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in frame.items()}, os.path.join(d, "frame.pt"))
+    torch.save(batch, os.path.join(d, "batch.pt"))
+    torch.save({"embs": embs, "pad_masks": pads, "att_masks": att}, os.path.join(d, "prefix.pt"))
+    torch.save({f"layer{i}": {"keys": k, "values": v} for i, (k, v) in enumerate(kv)}, os.path.join(d, "prefix_kv.pt"))
+    torch.save({"v_t": v_t}, os.path.join(d, "denoise.pt"))
+    torch.save({"chunk": chunk, "chunk_post": post}, os.path.join(d, "chunk.pt"))
+    errors = eng.validate(d)
+    worst = {k: v for k, v in errors.items() if k.endswith(".max")}
+    print("pi05 validate:", {k: round(v, 5) for k, v in sorted(worst.items(), key=lambda kv: -kv[1])[:6]})
+    assert {"prefix.embs.max", "prefix_kv.layer0.keys.max", "prefix_kv.layer1.values.max", "denoise.v_t.max", "chunk.max", "chunk_post.max"} <= set(errors)
+    assert errors["prefix.pad_masks.max"] == 0 and errors["prefix.att_masks.max"] == 0
+    assert all(v == 0 for k, v in errors.items() if k.startswith("batch.") and k.endswith(".max"))
+    assert errors["prefix.embs.max"] <= 2e-2 * max(1.0, float(embs.abs().max()))
+    assert max(v for k, v in worst.items() if k.startswith("prefix_kv.")) <= 5e-2 * max(1.0, max(float(k.abs().max()) for k, _ in kv))
+    # this checkpoint integrates 3 Euler steps (dt = 1/3), so a velocity evaluation's bf16 noise enters the chunk
+    # three times less damped than on the 10-step grid the 1e-2 bound is stated for
+    assert errors["denoise.v_t.max"] <= 5e-2 * max(1.0, float(v_t.abs().max())) and errors["chunk.max"] <= 1.5e-2
+    # the step tables are untouched by the off-grid evaluation: the next request is bit-identical
+    noise = torch.zeros(1, cfg.chunk_size, a_dim)
+    first = eng.predict_action_chunk(frame, noise=noise)
+    eng.validate(d)
+    assert np.array_equal(first, eng.predict_action_chunk(frame, noise=noise))
+    with pytest.raises(FileNotFoundError):
+        eng.validate(os.path.join(d, "nowhere"))

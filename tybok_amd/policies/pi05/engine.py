@@ -246,18 +246,65 @@ class PI05Engine(PolicyEngine):
         action = self._action_queue.popleft()
         return self.unnormalizer.unnormalize(action, ACTION, "ACTION").cpu().numpy()[0]
 
+    @torch.inference_mode()
     def validate(self, reference_dir: str) -> dict[str, float]:
-        def load(name: str):
+        """Per-component max / mean-abs errors against a reference dump, keyed like the reference's
+        report (tybok/policies/pi05/engine.py:740-857): ``batch.*``, ``prefix.{embs,pad_masks,att_masks}``,
+        ``prefix_kv.layer<i>.{keys,values}``, ``denoise.v_t`` (zero ``x_t``, t = 0.5), ``chunk`` (zero
+        noise, through the graph when enabled) and ``chunk_post``.  ``frame.pt`` and ``chunk.pt`` are
+        required, the other dump files are compared when present.  Dumps are read with
+        ``weights_only=True``: tensors and plain containers only."""
+
+        def load(name: str, required: bool = False):
             path = os.path.join(reference_dir, name)
             if not os.path.exists(path):
-                raise FileNotFoundError(f"reference dump {path} missing")
+                if required:
+                    raise FileNotFoundError(f"reference dump {path} missing")
+                return None
             return torch.load(path, weights_only=True)
 
-        frame, ref = load("frame.pt"), load("chunk.pt")
-        noise = torch.zeros(1, self.config.chunk_size, self.config.action_feature_shape[0])
-        chunk = torch.from_numpy(self.predict_action_chunk(frame, noise=noise))
-        diff = (chunk - ref["chunk_post"].float().cpu().reshape(chunk.shape)).abs()
-        return {"chunk_post.max": float(diff.max()), "chunk_post.mean": float(diff.mean())}
+        frame, ref_chunk = load("frame.pt", True), load("chunk.pt", True)
+        ref_batch, ref_prefix, ref_kv, ref_denoise = load("batch.pt"), load("prefix.pt"), load("prefix_kv.pt"), load("denoise.pt")
+        errors: dict[str, float] = {}
+
+        def max_err(name: str, a: torch.Tensor, b: torch.Tensor) -> None:
+            a, b = a.detach().float().cpu(), b.detach().float().cpu()
+            if a.shape != b.shape:
+                raise AssertionError(f"{name}: shape mismatch {tuple(a.shape)} vs {tuple(b.shape)}")
+            diff = (a - b).abs()
+            errors[name + ".max"] = float(diff.max())
+            errors[name + ".mean"] = float(diff.mean())
+
+        batch = self._batch_from_frame(frame)
+        if ref_batch is not None:
+            for key in [OBS_STATE, OBS_LANGUAGE_TOKENS, OBS_LANGUAGE_ATTENTION_MASK] + [k for k in ref_batch if k.startswith("observation.images.")]:
+                if key in batch and key in ref_batch:
+                    max_err(f"batch.{key}", batch[key], ref_batch[key])
+        images, img_masks = self.prepare_images(batch)
+        tokens, masks = batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK]
+        m = self.model
+        embs, pads = m.embed_prefix(images, img_masks, tokens, masks)
+        if ref_prefix is not None:
+            max_err("prefix.embs", embs, ref_prefix["embs"])
+            max_err("prefix.pad_masks", pads, ref_prefix["pad_masks"])
+            if "att_masks" in ref_prefix:  # every prefix token attends to every valid one: all zeros
+                max_err("prefix.att_masks", torch.zeros_like(pads), ref_prefix["att_masks"])
+        if ref_kv is not None or ref_denoise is not None:
+            kv = m.prefill_fused(embs, pads)[0] if m.fused_prefill and embs.shape[0] == 1 else m.prefill(embs, pads)
+            if ref_kv is not None:
+                for i, (k, v) in enumerate(kv):
+                    max_err(f"prefix_kv.layer{i}.keys", k, ref_kv[f"layer{i}"]["keys"])
+                    max_err(f"prefix_kv.layer{i}.values", v, ref_kv[f"layer{i}"]["values"])
+            if ref_denoise is not None:
+                x_t = torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, device=self.device)
+                max_err("denoise.v_t", m.velocity_at(pads, kv, x_t, 0.5), ref_denoise["v_t"])
+        noise = torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, device=self.device)
+        chunk = self._infer(batch, noise)[:, :, : self.config.action_feature_shape[0]]
+        if "chunk" in ref_chunk:
+            max_err("chunk", chunk, ref_chunk["chunk"].reshape(chunk.shape))
+        post = self.unnormalizer.unnormalize(chunk, ACTION, "ACTION")
+        max_err("chunk_post", post, ref_chunk["chunk_post"].reshape(post.shape))
+        return errors
 
     # ------------------------------------------------------------------ request plumbing
     def _batch_from_frame(self, frame: dict[str, Any]) -> dict[str, torch.Tensor]:

@@ -169,33 +169,49 @@ class PI05Model:
     def lin(self, name: str, x: torch.Tensor) -> torch.Tensor:
         return F.linear(x, self.p[name + ".weight"], self.p.get(name + ".bias"))
 
+    def _modulations_at(self, t: float):
+        """AdaRMS modulations of every expert norm at flow time ``t``: per layer ``(input, post_attention)``
+        raw ``[1, 3W]`` rows, the final norm's row, and the same split into contiguous (scale fp32, shift
+        fp32, gate bf16) vectors for the fused launches (flow_matching.py:505-556)."""
+        tt = torch.tensor(float(t), dtype=torch.float32).expand(1)
+        te = sinusoidal_time_embedding(tt, self.ed["width"], self.cfg.min_period, self.cfg.max_period).float().to(self.device)
+        cond = F.silu(self.lin("time_mlp_out", F.silu(self.lin("time_mlp_in", te))))
+        mods = [
+            (self.lin(f"{EXP}layers.{i}.input_layernorm.dense", cond), self.lin(f"{EXP}layers.{i}.post_attention_layernorm.dense", cond))
+            for i in range(self.ed["depth"])
+        ]
+        final = self.lin(EXP + "norm.dense", cond)
+        w = self.ed["width"]
+
+        def split(mod: torch.Tensor):
+            m = mod.reshape(-1).float()
+            return m[:w].contiguous(), m[w : 2 * w].contiguous(), m[2 * w :].to(BF16).contiguous()
+
+        return mods, final, [(split(a), split(b)) for a, b in mods], split(final)[:2]
+
     def set_num_steps(self, n: int) -> None:
         """Per-step AdaRMS modulations of every expert norm (computed on the device, once)."""
         self.num_steps = int(n)
         dt = -1.0 / self.num_steps
-        self.mods: list[list[tuple[torch.Tensor, torch.Tensor]]] = []
-        self.final_mods: list[torch.Tensor] = []
+        self.mods, self.final_mods, self.mods_split, self.final_split = [], [], [], []
         with torch.inference_mode():
             for step in range(self.num_steps):
-                t = torch.tensor(1.0 + step * dt, dtype=torch.float32).expand(1)
-                te = sinusoidal_time_embedding(t, self.ed["width"], self.cfg.min_period, self.cfg.max_period).float().to(self.device)
-                cond = F.silu(self.lin("time_mlp_out", F.silu(self.lin("time_mlp_in", te))))
-                self.mods.append(
-                    [
-                        (self.lin(f"{EXP}layers.{i}.input_layernorm.dense", cond), self.lin(f"{EXP}layers.{i}.post_attention_layernorm.dense", cond))
-                        for i in range(self.ed["depth"])
-                    ]
-                )
-                self.final_mods.append(self.lin(EXP + "norm.dense", cond))
-            # (scale, shift, gate) of every modulation as separate contiguous vectors for the fused launches
-            w = self.ed["width"]
+                mods, final, mods_split, final_split = self._modulations_at(1.0 + step * dt)
+                self.mods.append(mods)
+                self.final_mods.append(final)
+                self.mods_split.append(mods_split)
+                self.final_split.append(final_split)
 
-            def split(mod: torch.Tensor):
-                m = mod.reshape(-1).float()
-                return m[:w].contiguous(), m[w : 2 * w].contiguous(), m[2 * w :].to(BF16).contiguous()
-
-            self.mods_split = [[(split(a), split(b)) for a, b in step] for step in self.mods]
-            self.final_split = [split(m)[:2] for m in self.final_mods]
+    def velocity_at(self, prefix_pad, kv, x_t, t: float) -> torch.Tensor:
+        """One velocity evaluation at an arbitrary flow time (the per-step tables hold only the Euler
+        grid): used by the engine's ``validate`` for the reference's t = 0.5 probe."""
+        saved = self.mods, self.final_mods, self.mods_split, self.final_split
+        mods, final, mods_split, final_split = self._modulations_at(t)
+        self.mods, self.final_mods, self.mods_split, self.final_split = [mods], [final], [mods_split], [final_split]
+        try:
+            return self.denoise_step(prefix_pad, kv, x_t, 0)
+        finally:
+            self.mods, self.final_mods, self.mods_split, self.final_split = saved
 
     def rope_tables(self, pos: torch.Tensor, dtype) -> tuple[torch.Tensor, torch.Tensor]:
         return self.rope_cos[pos].to(dtype), self.rope_sin[pos].to(dtype)
