@@ -261,6 +261,16 @@ int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const voi
                     int M, int P, int H, int G, int D, int logits_bf16, float scale, void* ws, size_t ws_bytes,
                     void* stream);
 
+/* V^T for tk_batched_attn from the projection output, one launch for all problems:
+ *   v:  bf16 [B, P, G, D], element strides (v_sb, v_sl, v_sh), d contiguous (a view into a packed
+ *       q|k|v buffer is fine);  vt: bf16 [B, G, D, vt_keys], element strides (vt_sb, vt_sh, vt_sd),
+ *       keys contiguous, vt_keys >= P rounded up to 32, zero filled from P on (up to the end of the
+ *       last 64-key tile or vt_keys).  D in {64, 96}; all strides multiples of 8 elements.
+ * Replaces the `v.transpose(1, 2)` operand of the towers' `attn @ v`
+ * (tybok/policies/smolvla/models/vision.py:197-257, tybok/policies/pi05/models/vision.py:115-170). */
+int tk_batched_transpose_v(const void* v, long long v_sb, int v_sl, int v_sh, void* vt, long long vt_sb, int vt_sh,
+                           int vt_sd, int vt_keys, int B, int P, int G, int D, void* stream);
+
 /* ---- vision tower glue ------------------------------------------------------------------------ */
 /* LayerNorm of token rows with the cast to the GEMM input type folded in:
  *   y[m, :] = bf16((x[m, :] - mean) * rstd * w + b), statistics in fp32 (biased variance).

@@ -240,6 +240,43 @@ def test_batched_vision_attention(tk):
     _close(got, want, "batched vision attention")
 
 
+@pytest.mark.parametrize("b,m,p,h,g,d", [(3, 1024, 1024, 12, 12, 64), (2, 200, 200, 4, 4, 64), (1, 130, 300, 6, 2, 64), (2, 160, 160, 3, 3, 96), (1, 128, 129, 2, 1, 96)])
+def test_tower_attention_ragged_shapes(tk, b, m, p, h, g, d):
+    # the many-query path (128 queries per block, keys in stages of 64): full SmolVLA tower shape, query and
+    # key counts that end inside a tile / a stage, grouped heads, both head sizes; zero-padded V^T keys
+    gen = torch.Generator().manual_seed(17)
+    q = torch.randn(b, m, h, d, generator=gen).to(torch.bfloat16)
+    k = torch.randn(b, p, g, d, generator=gen).to(torch.bfloat16)
+    v = torch.randn(b, p, g, d, generator=gen).to(torch.bfloat16)
+    rep = h // g
+    kk, vv = k.repeat_interleave(rep, dim=2).float(), v.repeat_interleave(rep, dim=2).float()
+    logits = torch.einsum("bmhd,bphd->bhmp", q.float(), kk).to(torch.bfloat16).float() * d**-0.5
+    probs = torch.softmax(logits, dim=-1).to(torch.bfloat16).float()
+    want = torch.einsum("bhmp,bphd->bmhd", probs, vv).to(torch.bfloat16).reshape(b, m, h * d)
+    p_pad = (p + 31) // 32 * 32
+    vt = torch.zeros(b, g, d, p_pad, dtype=torch.bfloat16)
+    vt[..., :p] = v.permute(0, 2, 3, 1)
+    got = tk.batched_attn(q.cuda(), k.cuda(), vt.cuda(), logits_bf16=True)
+    again = tk.batched_attn(q.cuda(), k.cuda(), vt.cuda(), logits_bf16=True)
+    assert torch.equal(got, again)
+    _close(got, want, f"tower attention B={b} M={m} P={p} H={h} G={g} D={d}")
+
+
+@pytest.mark.parametrize("b,p,g,d", [(3, 1024, 12, 64), (2, 256, 16, 96), (1, 200, 3, 64), (2, 33, 2, 96)])
+def test_batched_value_transpose(tk, b, p, g, d):
+    # V^T operand straight from a packed q|k|v buffer: exact copy, zero padding keys
+    gen = torch.Generator().manual_seed(23)
+    qkv = torch.randn(b, p, 3, g, d, generator=gen).to(torch.bfloat16).cuda()
+    p_pad = (p + 31) // 32 * 32
+    out = torch.full((b, g, d, p_pad + 8), 7.0, dtype=torch.bfloat16, device="cuda")[..., :p_pad]  # rows longer than the operand
+    got = tk.transpose_v(qkv[:, :, 2], out=out)
+    assert torch.equal(got[..., :p], qkv[:, :, 2].permute(0, 2, 3, 1))
+    assert torch.count_nonzero(got[..., p:]) == 0
+    assert torch.equal(tk.transpose_v(qkv[:, :, 2]), got)
+    with pytest.raises(RuntimeError):
+        tk.transpose_v(torch.zeros(1, 64, 2, 128, dtype=torch.bfloat16, device="cuda"))
+
+
 def test_batched_attention_padded_head_with_explicit_scale(tk):
     # SigLIP-So400m heads are 72 wide: run as 96-wide heads whose last 24 columns are zero, with the
     # logit scale of the true size; the padded output columns must come back as zeros

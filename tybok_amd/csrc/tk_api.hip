@@ -297,6 +297,7 @@ int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void
                       int resid_dtype, const void* gate, int M, int K, int I, int act, void* ws, size_t ws_bytes,
                       void* stream) {
   if (act != TK_ACT_SILU && act != TK_ACT_GELU_TANH) return fail(TK_EINVAL, "ffn: unknown activation %d", act);
+  if (M <= 0 || K <= 0 || I <= 0) return fail(TK_EINVAL, "ffn: non-positive shape M=%d K=%d I=%d", M, K, I);
   if (!sg || !su || !sd) return fail(TK_EINVAL, "ffn: null scale pointer");
   if (I % 32) return fail(TK_EINVAL, "ffn: I=%d must be a multiple of 32", I);
   if (!ws) return fail(TK_EWORKSPACE, "ffn: needs a workspace");
@@ -364,6 +365,7 @@ int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float nor
                            const void* resid, int ldr, int resid_dtype, const void* gate, int M, int K, int I, int act,
                            void* ws, size_t ws_bytes, void* stream) {
   if (act != TK_ACT_SILU && act != TK_ACT_GELU_TANH) return fail(TK_EINVAL, "ffn: unknown activation %d", act);
+  if (M <= 0 || K <= 0 || I <= 0) return fail(TK_EINVAL, "ffn: non-positive shape M=%d K=%d I=%d", M, K, I);
   if (!sg || !su || !sd || (!norm_w && !ada_scale)) return fail(TK_EINVAL, "ffn: null scale or norm pointer");
   if (I % 32) return fail(TK_EINVAL, "ffn: I=%d must be a multiple of 32", I);
   if (!ws) return fail(TK_EWORKSPACE, "ffn: needs a workspace");
@@ -502,6 +504,13 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   a.logits_bf16 = logits_bf16;
   a.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
 
+  if (batch > 0 && !split && S == 0 && !mask2d && !pad && (D == 64 || D == 96) && P >= 128 && M >= 128) {
+    // vision towers: many query tiles over a long key range -- K / V^T staged through LDS once per 128 queries
+    a.gqa_mul = (65536 + H / G - 1) / (H / G);
+    int rc = tk_launch_tower_attn(a, D, (hipStream_t)stream);
+    if (rc) return fail(TK_ELAUNCH, "attn: launch failed (%s)", hipGetErrorString(hipGetLastError()));
+    return TK_OK;
+  }
   const int ntiles = (P + 31) / 32 + (S + 31) / 32;
   const int mtiles = ((M + 31) / 32) * (batch > 0 ? batch : 1);
   // one 32-key tile per wave: split the keys over blocks of four waves (at most 8 splits, beyond
@@ -613,12 +622,38 @@ int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const voi
                    ws_bytes, stream);
 }
 
+int tk_batched_transpose_v(const void* v, long long v_sb, int v_sl, int v_sh, void* vt, long long vt_sb, int vt_sh, int vt_sd,
+                           int vt_keys, int B, int P, int G, int D, void* stream) {
+  if (B <= 0 || P <= 0 || G <= 0) return fail(TK_EINVAL, "transpose_v: bad shape B=%d P=%d G=%d", B, P, G);
+  if (D != 64 && D != 96) return fail(TK_EINVAL, "transpose_v: head_dim %d not in {64, 96}", D);
+  if (!v || !vt || !aligned16(v) || !aligned16(vt)) return fail(TK_EINVAL, "transpose_v: null or unaligned pointer");
+  if (v_sb % 8 || v_sl % 8 || v_sh % 8 || vt_sb % 8 || vt_sh % 8 || vt_sd % 8 || vt_keys % 8)
+    return fail(TK_EINVAL, "transpose_v: strides must be multiples of 8 elements");
+  if (vt_keys < ((P + 31) / 32) * 32 || vt_sd < vt_keys) return fail(TK_EINVAL, "transpose_v: a V^T row must hold P rounded up to 32 keys (vt_keys=%d, vt_sd=%d)", vt_keys, vt_sd);
+  TransposeVArgs a;
+  a.v = (const u16*)v;
+  a.v_sb = v_sb;
+  a.v_sl = v_sl;
+  a.v_sh = v_sh;
+  a.vt = (u16*)vt;
+  a.vt_sb = vt_sb;
+  a.vt_sh = vt_sh;
+  a.vt_sd = vt_sd;
+  a.ld = vt_keys;
+  a.B = B;
+  a.P = P;
+  a.G = G;
+  if (tk_launch_transpose_v(a, D, (hipStream_t)stream)) return fail(TK_ELAUNCH, "transpose_v: launch failed");
+  return TK_OK;
+}
+
 int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps,
                    const void* w, const void* bias, void* v_out, const void* x_t, void* x_out, float dt, int M, int N, int K,
                    void* stream) {
   if (M <= 0 || N <= 0 || K <= 0 || ldx < K) return fail(TK_EINVAL, "tail: bad shape M=%d N=%d K=%d ldx=%d", M, N, K, ldx);
   if (N > 256 || 256 % N) return fail(TK_EINVAL, "tail: N=%d must divide 256", N);
-  if (K > 16384 || K % 4) return fail(TK_EINVAL, "tail: K=%d must be a multiple of 4 and at most 16384", K);
+  // (the normalised row lives in LDS as fp32: 32 KiB at the limit)
+  if (K > 8192 || K % 4) return fail(TK_EINVAL, "tail: K=%d must be a multiple of 4 and at most 8192", K);
   if (!aligned16(w)) return fail(TK_EINVAL, "tail: w must be 16-byte aligned");
   if (!x || !w || (!norm_w && !(ada_scale && ada_shift)) || (norm_w && (ada_scale || ada_shift)))
     return fail(TK_EINVAL, "tail: needs x, w and exactly one of norm_w or ada_scale + ada_shift");

@@ -172,6 +172,19 @@ int tk_launch_pack(const void* w0, const void* w1, void* out, int N, int K, int 
 int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st);
 int tk_launch_fill_zero(int* p, int n, hipStream_t st);
 int tk_launch_decode_fp8(float* out, hipStream_t st);
+struct TransposeVArgs {
+  const unsigned short* v;  // bf16 [B, P, G, D], element strides (v_sb, v_sl, v_sh), d contiguous
+  long long v_sb;
+  int v_sl, v_sh;
+  unsigned short* vt;  // bf16 [B, G, D, ld], element strides (vt_sb, vt_sh, vt_sd), keys contiguous
+  long long vt_sb;
+  int vt_sh, vt_sd;
+  int ld;  // keys a V^T row can hold (a multiple of 8)
+  int B, P, G;
+};
+int tk_launch_transpose_v(TransposeVArgs a, int D, hipStream_t st);
+// vision-tower self-attention (batched, unmasked, prefix-only, head size 64 / 96): 128 queries per block
+int tk_launch_tower_attn(AttnArgs a, int D, hipStream_t st);
 int tk_attn_waves(int D, int split_planes, int ntiles);
 int tk_launch_attn(AttnArgs a, int D, int waves, hipStream_t st);
 int tk_launch_attn_qproj(AttnArgs a, hipStream_t st);

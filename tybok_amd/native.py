@@ -75,6 +75,10 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_longlong, c_int, c_int, c_void_p, c_longlong, c_int, c_int, c_void_p, c_longlong, c_int, c_int,
          c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
+    "tk_batched_transpose_v": (
+        c_int,
+        [c_void_p, c_longlong, c_int, c_int, c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    ),  # fmt: skip
     "tk_expert_attn": (
         c_int,
         [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int,

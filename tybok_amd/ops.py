@@ -580,6 +580,26 @@ def batched_attn(
     return out
 
 
+def transpose_v(v: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``v [B, P, G, D]`` bf16 (a view with a contiguous head dim, e.g. into a packed q|k|v buffer) ->
+    ``vt [B, G, D, P rounded up to 32]`` with zero-filled padding keys: the V^T operand of
+    :func:`batched_attn`, one launch for all problems.  ``D`` in {64, 96}."""
+    lib = native.lib()
+    if v.dtype != torch.bfloat16 or v.dim() != 4 or v.stride(3) != 1:
+        raise TypeError("v must be a 4-D bf16 tensor with a contiguous head dim")
+    b, p, g, d = v.shape
+    if out is None:
+        out = torch.empty(b, g, d, _pad32(p), dtype=torch.bfloat16, device=v.device)
+    if out.shape[:3] != (b, g, d) or out.shape[3] < _pad32(p) or out.stride(3) != 1 or out.dtype != torch.bfloat16:
+        raise ValueError("out must be bf16 [B, G, D, >= P rounded up to 32] with contiguous keys")
+    rc = lib.tk_batched_transpose_v(
+        v.data_ptr(), v.stride(0), v.stride(1), v.stride(2), out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+        out.shape[3], b, p, g, d, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_batched_transpose_v")
+    return out
+
+
 def expert_attn_plain(
     q: torch.Tensor,
     k_pre: torch.Tensor | None,

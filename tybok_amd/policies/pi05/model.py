@@ -237,7 +237,7 @@ class PI05Model:
                 hp = self.vis_head_pad
                 h = tk.layer_norm(x, p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], EPS)
                 qkv = F.linear(h, *self.vis_lowp[lp + "self_attn.qkv"]).view(b, -1, 3, heads, hp)
-                vt = qkv[:, :, 2].permute(0, 2, 3, 1).contiguous()
+                vt = tk.transpose_v(qkv[:, :, 2]) if hp in (64, 96) else qkv[:, :, 2].permute(0, 2, 3, 1).contiguous()
                 a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, scale=hd**-0.5, ws=self.ws)
                 x = x + F.linear(a, *self.vis_lowp[lp + "self_attn.out_proj"])  # fp32 + bf16: promoted inside the add
             else:

@@ -245,7 +245,7 @@ class SmolVLAModel:
                 # bf16 before the fp32 scale and softmax, exactly what the bf16 matmul below produces
                 w_qkv, b_qkv = self.vis_qkv[i]
                 qkv = F.linear(h, w_qkv, b_qkv).view(b, -1, 3, heads, hd)
-                vt = qkv[:, :, 2].permute(0, 2, 3, 1).contiguous()
+                vt = tk.transpose_v(qkv[:, :, 2])
                 a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, ws=self.ws)
                 x = x + self.lin(lp + "self_attn.out_proj", a)
                 h = tk.layer_norm(x, p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
