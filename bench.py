@@ -159,6 +159,39 @@ def attn_launch_us(launches: int = 100, reps: int = 10) -> float:
     return e0.elapsed_time(e1) * 1e3 / (reps * launches)
 
 
+def tower_attn_launch_us(cameras: int = 3, tokens: int = 1024, heads: int = 12, d: int = 64, launches: int = 20, reps: int = 10) -> float:
+    """Average duration (us) of one vision-tower attention launch (SmolVLA tower: one 1024-token problem
+    per camera, 12 heads of 64, bf16-rounded logits) inside a replayed graph."""
+    import torch
+
+    from tybok_amd import ops as tk
+
+    g = torch.Generator().manual_seed(0)
+    qkv = torch.randn(cameras, tokens, 3, heads, d, generator=g).to(torch.bfloat16).cuda()
+    vt = tk.transpose_v(qkv[:, :, 2])
+    out = torch.empty(cameras, tokens, heads * d, dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(3):
+            tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, out=out)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
+        for _ in range(launches):
+            tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, out=out)
+    spin_up(60.0)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * launches)
+
+
 def device_frame(engine, cameras: int, seed: int = 0) -> dict:
     """Synthetic observation (uint8-valued images / 255, random state) already on the GPU."""
     import torch
@@ -230,6 +263,7 @@ def main() -> None:
     ap.add_argument("--gemm-only", action="store_true", help="only the roofline GEMM loop plus a plain copy of known size (for rocprofv3 runs)")
     ap.add_argument("--gemm-shape", type=int, nargs=3, metavar=("M", "K", "N"), default=(50, 2048, 16384), help="shape of the --gemm-only loop")
     ap.add_argument("--attn-only", action="store_true", help="only the action-expert attention loop (for rocprofv3 runs)")
+    ap.add_argument("--tower-attn-only", action="store_true", help="only the vision-tower attention loop, 3 cameras x 1024 tokens (for rocprofv3 runs)")
     ap.add_argument("--ffn-only", action="store_true", help="only the many-row (M=712) fp8 GeGLU FFN loop (for rocprofv3 runs)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -258,6 +292,12 @@ def main() -> None:
         spin_up()
         us = ffn_launch_us(712, 2048, 16384, launches=5, reps=args.steps)
         print(json.dumps({"ffn_only": {"M": 712, "K": 2048, "I": 16384, "us": round(us, 1), "TFLOPs": round(6.0 * 712 * 2048 * 16384 / us / 1e6, 1)}}), flush=True)
+        return
+    if args.tower_attn_only:
+        spin_up()
+        us = tower_attn_launch_us(launches=20, reps=args.steps)
+        flops = 4.0 * 3 * 12 * 1024 * 1024 * 64
+        print(json.dumps({"tower_attn_only": {"B": 3, "M": 1024, "P": 1024, "H": 12, "D": 64, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1)}}), flush=True)
         return
     if args.attn_only:
         spin_up()
