@@ -56,3 +56,80 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(native, "_LIB_PATH", "/nonexistent/libtybok_hip.so")
     with pytest.raises(RuntimeError, match="no CPU or torch fallback"):
         native.lib()
+
+
+P = 0x10000  # a 16-byte aligned stand-in for device pointers: every call below is rejected before any launch
+
+
+def _cases():
+    """(entry point, arguments, error code, fragment of tk_last_error()) -- one row per validation rule."""
+    gemm = lambda **kw: _args(  # noqa: E731
+        dict(x=P, ldx=2048, w=P, scale=P, y=P, ldy=16384, resid=None, ldr=0, rdt=0, gate=None, M=50, N=16384, K=2048, split=0, ws=None, wsb=0, st=None), kw
+    )
+    ffn = lambda **kw: _args(  # noqa: E731
+        dict(x=P, ldx=720, wgu=P, sg=P, su=P, wd=P, sd=P, y=P, ldy=720, resid=None, ldr=0, rdt=0, gate=None, M=50, K=720, I=2048, act=0, ws=P, wsb=1 << 27, st=None), kw
+    )
+    attn = lambda **kw: _args(  # noqa: E731
+        dict(q=P, q_sm=960, q_sh=64, k=P, k_lo=None, sl=320, sh=64, vt=P, vt_lo=None, vsd=256, vsh=64 * 256, ks=None, ssl=0, ssh=0, vts=None, svsd=0, svsh=0,
+             pad=None, m2=None, mld=0, out=P, osm=960, M=50, Pk=241, S=0, H=15, G=5, D=64, mode=0, lb=0, ws=None, wsb=0, st=None), kw
+    )  # fmt: skip
+    tail = lambda **kw: _args(  # noqa: E731
+        dict(x=P, ldx=720, nw=P, asc=None, ash=None, eps=1e-6, w=P, b=None, v=P, xt=None, xo=None, dt=0.0, M=50, N=32, K=720, st=None), kw
+    )
+    ln = lambda **kw: _args(dict(x=P, ldx=768, xdt=0, w=P, b=P, wdt=0, eps=1e-6, y=P, ldy=768, M=64, K=768, st=None), kw)  # noqa: E731
+    tv = lambda **kw: _args(dict(v=P, sb=1 << 20, sl=2304, sh=64, vt=P, tsb=1 << 20, tsh=65536, tsd=1024, keys=1024, B=3, Pk=1024, G=12, D=64, st=None), kw)  # noqa: E731
+    return [
+        ("tk_fp8w_gemm", gemm(K=2040), -1, "multiple of 16"),
+        ("tk_fp8w_gemm", gemm(ldx=1024), -1, "ldx"),
+        ("tk_fp8w_gemm", gemm(x=P + 2), -1, "16-byte aligned"),
+        ("tk_fp8w_gemm", gemm(y=None), -1, "null pointer"),
+        ("tk_fp8w_gemm", gemm(M=0), -1, "non-positive"),
+        ("tk_fp8w_gemm", gemm(resid=P, ldr=8), -1, "ldr"),
+        ("tk_fp8w_gemm", gemm(resid=P, ldr=16384, rdt=5), -1, "resid_dtype"),
+        ("tk_fp8w_gemm", gemm(N=720, K=16384, ldx=16384, ldy=720, split=8), -2, "needs a workspace"),
+        ("tk_fp8w_gated_ffn", ffn(act=7), -1, "unknown activation"),
+        ("tk_fp8w_gated_ffn", ffn(I=2000), -1, "multiple of 32"),
+        ("tk_fp8w_gated_ffn", ffn(ws=None), -2, "needs a workspace"),
+        ("tk_fp8w_gated_ffn", ffn(M=100000, I=16384), -2, "intermediate"),
+        ("tk_fp8w_gated_ffn", ffn(M=-3), -1, "non-positive"),
+        ("tk_expert_attn", attn(D=80), -1, "head_dim"),
+        ("tk_expert_attn", attn(G=4), -1, "bad shape"),
+        ("tk_expert_attn", attn(sl=324), -1, "multiples of 8"),
+        ("tk_expert_attn", attn(S=50, ks=P, vts=P, ssl=320, ssh=64, svsd=64, svsh=4096), -1, "suffix mask mode"),
+        ("tk_expert_attn", attn(vsd=224), -1, "rounded up to 32"),
+        ("tk_expert_attn", attn(k_lo=P), -1, "both K and V^T low planes"),
+        ("tk_expert_attn", attn(osm=900), -1, "out_sm"),
+        ("tk_expert_attn", attn(mode=3), -1, "mask_mode"),
+        ("tk_expert_tail", tail(N=48), -1, "divide 256"),
+        ("tk_expert_tail", tail(K=8200, ldx=8200), -1, "at most 8192"),
+        ("tk_expert_tail", tail(asc=P, ash=P), -1, "exactly one"),
+        ("tk_expert_tail", tail(v=None), -1, "no output"),
+        ("tk_layer_norm", ln(K=4096, ldx=4096, ldy=4096), -1, "at most"),
+        ("tk_layer_norm", ln(wdt=1), -1, "both"),
+        ("tk_layer_norm", ln(ldy=760), -1, "row pitch"),
+        ("tk_batched_transpose_v", tv(D=128), -1, "head_dim"),
+        ("tk_batched_transpose_v", tv(keys=1000), -1, "rounded up to 32"),
+        ("tk_batched_transpose_v", tv(sl=2300), -1, "multiples of 8"),
+    ]
+
+
+def _args(defaults, overrides):
+    unknown = set(overrides) - set(defaults)
+    assert not unknown, unknown
+    return list({**defaults, **overrides}.values())
+
+
+@pytest.mark.parametrize("name,args,code,fragment", _cases(), ids=lambda v: v if isinstance(v, str) and v.startswith("tk_") else None)
+def test_arguments_are_checked_on_the_host(name, args, code, fragment):
+    # every entry point validates shapes, strides, alignment and workspace before it launches anything: a bad
+    # call returns the documented error code and says why, with or without a GPU in the machine
+    from tybok_amd import native
+
+    if not os.path.exists(native.library_path()):
+        pytest.skip("libtybok_hip.so not built")
+    lib = native.lib()
+    assert len(args) == len(native.SIGNATURES[name][1])
+    rc = getattr(lib, name)(*args)
+    message = lib.tk_last_error().decode()
+    assert rc == code, f"{name}: rc {rc}, message {message!r}"
+    assert fragment in message, message
