@@ -272,6 +272,23 @@ int tk_batched_transpose_v(const void* v, long long v_sb, int v_sl, int v_sh, vo
                            int vt_sd, int vt_keys, int B, int P, int G, int D, void* stream);
 
 /* ---- vision tower glue ------------------------------------------------------------------------ */
+/* RMSNorm of bf16 rows into a bf16 buffer, for projections that run as a plain library GEMM (many
+ * rows): y[m, :] = bf16(norm_w * bf16(x * rstd))  (Llama RMSNorm, norm_w bf16 [K]) or
+ * bf16((x * rstd) * (1 + ada_scale) + ada_shift)  (Gemma / adaptive RMSNorm, fp32 [K] vectors; a
+ * plain Gemma norm passes its weight as ada_scale and zeros as ada_shift) -- the prologues of
+ * tk_bf16w_linear / tk_fp8w_norm_gated_ffn as a launch of their own
+ * (tybok/policies/smolvla/models/layers.py:23-58, tybok/policies/pi05/models/layers.py:51-84). */
+int tk_rms_norm_rows(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps,
+                     void* y, int ldy, int M, int K, void* stream);
+
+/* Rotary embedding in place on the columns < rope_cols of a bf16 projection output y [M, ldy] (heads
+ * of 2 * rope_half columns, pairs (i, i + rope_half)); positions int32 [M] clamped into the fp32
+ * tables [rope_positions, rope_half]; rope_bf16 selects pi0.5's bf16 arithmetic -- the rotary
+ * epilogue of tk_bf16w_linear as a launch of its own
+ * (tybok/policies/smolvla/models/rope.py:51-73, tybok/policies/pi05/models/layers.py:101-128). */
+int tk_rope_rows(void* y, int ldy, const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions,
+                 int rope_cols, int rope_half, int rope_bf16, int M, void* stream);
+
 /* LayerNorm of token rows with the cast to the GEMM input type folded in:
  *   y[m, :] = bf16((x[m, :] - mean) * rstd * w + b), statistics in fp32 (biased variance).
  * Replaces `layer_norm1/2(x)` (+ the `.to(bf16)` of the low-precision tiers) in the encoder layers

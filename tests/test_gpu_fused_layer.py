@@ -286,3 +286,52 @@ def test_cross_layer_in_one_launch_rejects_what_it_cannot_run(tk):
         big = tk.prepare_prefix_kv(torch.randn(300, 2, 64, generator=g).cuda(), torch.randn(300, 2, 64, generator=g).cuda())
         tk.cross_attn_fused(x, pw, nw, 1e-5, rope, pos, big, None)
     assert tk.cross_attn_fused(x, pw, nw, 1e-5, rope, pos, ok, None).shape == (8, 128)
+
+
+@pytest.mark.parametrize("bf16_math", [False, True])
+@pytest.mark.parametrize("m,k,heads,kv_heads,d", [(300, 256, 4, 1, 64), (712, 2048, 8, 1, 256), (7, 96, 2, 2, 32)])
+def test_norm_and_rotary_as_launches_of_their_own_equal_the_fused_projection(tk, m, k, heads, kv_heads, d, bf16_math):
+    # many-row prefills run the q|k|v projection as a library GEMM between tk_rms_norm_rows and tk_rope_rows:
+    # the two kernels must reproduce the fused projection's prologue / epilogue bit for bit on the same GEMM output
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(m, k, generator=g).to(BF16).cuda()
+    scale = (0.3 * torch.randn(k, generator=g)).cuda()
+    shift = (0.1 * torch.randn(k, generator=g)).cuda()
+    w = torch.randn(k, generator=g).to(BF16).cuda()
+    xf = x.float()
+    rstd = torch.rsqrt(xf.square().mean(-1, keepdim=True) + 1e-6)
+    want_ada = ((xf * rstd) * (1.0 + scale) + shift).to(BF16)
+    want_llama = (w.float() * (xf * rstd).to(BF16).float()).to(BF16)
+    got_ada = tk.rms_norm_rows(x, ada=(scale, shift), eps=1e-6)
+    got_llama = tk.rms_norm_rows(x, norm_w=w, eps=1e-6)
+    for got, want in ((got_ada, want_ada), (got_llama, want_llama)):
+        diff = (got.float() - want.float()).abs()
+        assert bool((diff <= want.float().abs().clamp_min(2.0**-6) * 2.0**-7).all())  # one bf16 step (rstd differs in its last bit)
+        assert float((diff > 0).float().mean()) < 0.02
+    # rotary: same table, same arithmetic as the projection epilogue -> compare on an identity-like path
+    nq, nkv = heads * d, kv_heads * d
+    half = d // 2
+    pos = torch.randint(0, 60, (m,), generator=g).to(torch.int32).cuda()
+    inv = 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float32) / half))
+    ang = torch.arange(64, dtype=torch.float32)[:, None] * inv[None, :]
+    cos, sin = ang.cos(), ang.sin()
+    if bf16_math:
+        cos, sin = cos.to(BF16).float(), sin.to(BF16).float()
+    tables = tk.RopeTables(cos.contiguous().cuda(), sin.contiguous().cuda())
+    y = torch.randn(m, nq + 2 * nkv, generator=g).to(BF16).cuda()
+    ref = y.clone().float().cpu()
+    c, s_ = cos[pos.cpu().long()], sin[pos.cpu().long()]  # [m, half]
+    for h in range(heads + kv_heads):
+        a, b = ref[:, h * d : h * d + half].clone(), ref[:, h * d + half : (h + 1) * d].clone()
+        if bf16_math:
+            r = lambda t: t.to(BF16).float()  # noqa: E731
+            ref[:, h * d : h * d + half] = r(r(a * c) - r(b * s_))
+            ref[:, h * d + half : (h + 1) * d] = r(r(b * c) + r(a * s_))
+        else:
+            ref[:, h * d : h * d + half] = (a * c - b * s_).to(BF16).float()
+            ref[:, h * d + half : (h + 1) * d] = (b * c + a * s_).to(BF16).float()
+    out = tk.rope_rows(y, tables, pos, nq + nkv, rope_bf16=bf16_math)
+    assert out.data_ptr() == y.data_ptr()
+    assert torch.equal(out.float().cpu(), ref), f"max diff {float((out.float().cpu() - ref).abs().max())}"
+    with pytest.raises(RuntimeError):
+        tk.rope_rows(y, tables, pos, nq + nkv + 8)

@@ -274,8 +274,8 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         // separately rounded products, as an elementwise fp32 implementation computes them
-        ra[j] = __fsub_rn(__fmul_rn(va[j], cs[j]), __fmul_rn(vb[j], sn[j]));
-        rb[j] = __fadd_rn(__fmul_rn(vb[j], cs[j]), __fmul_rn(va[j], sn[j]));
+        ra[j] = sub_rn(mul_rn(va[j], cs[j]), mul_rn(vb[j], sn[j]));
+        rb[j] = add_rn(mul_rn(vb[j], cs[j]), mul_rn(va[j], sn[j]));
       }
       *(i32x2*)(qs + l32 * QPITCH + fi * 2) = pack_bf16x4(ra);
       *(i32x2*)(qs + l32 * QPITCH + (D / 2 + fi) * 2) = pack_bf16x4(rb);

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kThreads) void expert_tail_kernel(TailArgs a) {
     float h;
     if (a.ada_scale) {
       // adaptive: bf16((x * rstd) * (1 + scale) + shift), fp32 steps rounded separately
-      h = round_bf16(__fadd_rn(__fmul_rn(__fmul_rn(f, rstd), __fadd_rn(1.0f, a.ada_scale[k])), a.ada_shift[k]));
+      h = round_bf16(add_rn(mul_rn(mul_rn(f, rstd), add_rn(1.0f, a.ada_scale[k])), a.ada_shift[k]));
     } else {
       // Llama RMSNorm on a bf16 row: bf16(w * bf16(x * rstd))
       h = round_bf16(bf16_bits_to_f32(a.norm_w[k]) * round_bf16(f * rstd));
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kThreads) void expert_tail_kernel(TailArgs a) {
     for (int j = 0; j < slices; ++j) v += part[tid + j];
     if (a.bias) v += a.bias[n];
     if (a.v_out) a.v_out[(size_t)m * a.N + n] = v;
-    if (a.x_out) a.x_out[(size_t)m * a.N + n] = __fadd_rn(a.x_t[(size_t)m * a.N + n], __fmul_rn(a.dt, v));
+    if (a.x_out) a.x_out[(size_t)m * a.N + n] = add_rn(a.x_t[(size_t)m * a.N + n], mul_rn(a.dt, v));
   }
 }
 

@@ -200,8 +200,8 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
         for (int e = 0; e < 4; ++e) {
           // separately rounded fp32 operations, as the elementwise reference computes them
           const float x0 = __uint_as_float(xu.u[e] << 16), x1 = __uint_as_float(xu.u[e] & 0xffff0000u);
-          const float y0 = __fadd_rn(__fmul_rn(__fmul_rn(x0, my_rstd[i]), __fadd_rn(1.0f, sc.f[2 * e])), sh.f[2 * e]);
-          const float y1 = __fadd_rn(__fmul_rn(__fmul_rn(x1, my_rstd[i]), __fadd_rn(1.0f, sc.f[2 * e + 1])), sh.f[2 * e + 1]);
+          const float y0 = add_rn(mul_rn(mul_rn(x0, my_rstd[i]), add_rn(1.0f, sc.f[2 * e])), sh.f[2 * e]);
+          const float y1 = add_rn(mul_rn(mul_rn(x1, my_rstd[i]), add_rn(1.0f, sc.f[2 * e + 1])), sh.f[2 * e + 1]);
           o.u[e] = pack_bf16x2(y0, y1);
         }
         out = o.v;
@@ -560,8 +560,8 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               // separately rounded products, as an elementwise fp32 implementation computes them
-              ra[j] = __fsub_rn(__fmul_rn(va[j], cs[j]), __fmul_rn(vb[j], sn[j]));
-              rb[j] = __fadd_rn(__fmul_rn(vb[j], cs[j]), __fmul_rn(va[j], sn[j]));
+              ra[j] = sub_rn(mul_rn(va[j], cs[j]), mul_rn(vb[j], sn[j]));
+              rb[j] = add_rn(mul_rn(vb[j], cs[j]), mul_rn(va[j], sn[j]));
             }
           }
           va = ra;

@@ -358,8 +358,8 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(NormRowsArgs a) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float x0 = __uint_as_float(xu.u[e] << 16), x1 = __uint_as_float(xu.u[e] & 0xffff0000u);
-        const float y0 = __fadd_rn(__fmul_rn(__fmul_rn(x0, rstd), __fadd_rn(1.0f, sc.f[2 * e])), sh.f[2 * e]);
-        const float y1 = __fadd_rn(__fmul_rn(__fmul_rn(x1, rstd), __fadd_rn(1.0f, sc.f[2 * e + 1])), sh.f[2 * e + 1]);
+        const float y0 = add_rn(mul_rn(mul_rn(x0, rstd), add_rn(1.0f, sc.f[2 * e])), sh.f[2 * e]);
+        const float y1 = add_rn(mul_rn(mul_rn(x1, rstd), add_rn(1.0f, sc.f[2 * e + 1])), sh.f[2 * e + 1]);
         o.u[e] = pack_bf16x2(y0, y1);
       }
     } else {

@@ -679,6 +679,51 @@ int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_s
   return TK_OK;
 }
 
+int tk_rms_norm_rows(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps, void* y,
+                     int ldy, int M, int K, void* stream) {
+  if (M <= 0 || K <= 0 || K % 8) return fail(TK_EINVAL, "rms_norm_rows: bad shape M=%d K=%d (K a multiple of 8)", M, K);
+  if (!x || !y || ldx < K || ldy < K || ldx % 8 || ldy % 8) return fail(TK_EINVAL, "rms_norm_rows: null pointer or row pitch not a multiple of 8 >= K");
+  if ((norm_w != nullptr) == (ada_scale != nullptr) || (ada_scale != nullptr) != (ada_shift != nullptr))
+    return fail(TK_EINVAL, "rms_norm_rows: needs exactly one of norm_w or ada_scale + ada_shift");
+  if (!aligned16(x) || !aligned16(y) || !aligned16(norm_w) || !aligned16(ada_scale) || !aligned16(ada_shift))
+    return fail(TK_EINVAL, "rms_norm_rows: operands must be 16-byte aligned");
+  NormRowsArgs a;
+  a.x = (const u16*)x;
+  a.ldx = ldx;
+  a.norm_w = (const u16*)norm_w;
+  a.ada_scale = (const float*)ada_scale;
+  a.ada_shift = (const float*)ada_shift;
+  a.eps = eps;
+  a.out = (u16*)y;
+  a.ldo = ldy;
+  a.M = M;
+  a.K = K;
+  if (tk_launch_norm_rows(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "rms_norm_rows: launch failed");
+  return TK_OK;
+}
+
+int tk_rope_rows(void* y, int ldy, const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions,
+                 int rope_cols, int rope_half, int rope_bf16, int M, void* stream) {
+  if (M <= 0 || rope_cols <= 0 || rope_half < 8 || rope_half % 8 || rope_cols % (2 * rope_half))
+    return fail(TK_EINVAL, "rope_rows: bad shape M=%d rope_cols=%d rope_half=%d (half a multiple of 8, cols of the head size)", M, rope_cols, rope_half);
+  if (!y || !rope_pos || !rope_cos || !rope_sin || rope_positions <= 0) return fail(TK_EINVAL, "rope_rows: null pointer or empty table");
+  if (ldy < rope_cols || ldy % 8 || !aligned16(y) || !aligned16(rope_cos) || !aligned16(rope_sin))
+    return fail(TK_EINVAL, "rope_rows: ldy=%d must be >= rope_cols and a multiple of 8; y and the tables 16-byte aligned", ldy);
+  RopeRowsArgs a;
+  a.y = (u16*)y;
+  a.ldy = ldy;
+  a.pos = (const int*)rope_pos;
+  a.cos = (const float*)rope_cos;
+  a.sin = (const float*)rope_sin;
+  a.positions = rope_positions;
+  a.rope_cols = rope_cols;
+  a.half = rope_half;
+  a.bf16_math = rope_bf16;
+  a.M = M;
+  if (tk_launch_rope_rows(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "rope_rows: launch failed");
+  return TK_OK;
+}
+
 int tk_layer_norm(const void* x, int ldx, int x_dtype, const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy,
                   int M, int K, void* stream) {
   if (M <= 0 || K <= 0 || K % 8 || K > tk_layer_norm_max_k()) return fail(TK_EINVAL, "layer_norm: K=%d must be a multiple of 8, at most %d", K, tk_layer_norm_max_k());

@@ -39,6 +39,21 @@ __device__ __forceinline__ f32x4 unpack_bf16x4(i32x2 r) {
              __uint_as_float((unsigned)r[1] << 16), __uint_as_float((unsigned)r[1] & 0xffff0000u)};
   return v;
 }
+// Products, sums and differences that round on their own, as separate elementwise launches of the
+// reference round them: without the pragma the compiler is free to fuse `a * b + c` into one fma
+// (the __f*_rn intrinsics are plain operators to it).
+__device__ __forceinline__ float mul_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
+__device__ __forceinline__ float add_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a + b;
+}
+__device__ __forceinline__ float sub_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a - b;
+}
 __device__ __forceinline__ float round_bf16(float f) { return __uint_as_float(pack_bf16x2(f, 0.f) << 16); }
 
 // 4 e4m3fn bytes (one dword) -> 4 bf16 (exact: every e4m3 value is a bf16 value).

@@ -159,6 +159,17 @@ struct NormRowsArgs {
   int M, K;
 };
 
+struct RopeRowsArgs {
+  unsigned short* y;  // bf16 [M, ldy], rotated in place in columns < rope_cols
+  int ldy;
+  const int* pos;  // int32 [M], clamped into the table
+  const float* cos;  // fp32 [positions, half]
+  const float* sin;
+  int positions, rope_cols, half, bf16_math;
+  int M;
+};
+int tk_launch_rope_rows(RopeRowsArgs a, hipStream_t st);
+int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st);
 int tk_launch_tail(TailArgs a, hipStream_t st);
 int tk_launch_kv_proj(KvProjArgs a, hipStream_t st);
 int tk_layer_norm_max_k();

@@ -678,6 +678,46 @@ def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) ->
     return y.view(x.shape)
 
 
+def rms_norm_rows(x: torch.Tensor, *, norm_w: torch.Tensor | None = None, ada: tuple[torch.Tensor, torch.Tensor] | None = None, eps: float) -> torch.Tensor:
+    """RMSNorm of bf16 rows ``x [M, K]`` into a new bf16 tensor: Llama (``norm_w`` bf16 ``[K]``) or
+    Gemma / adaptive (``ada = (scale, shift)`` fp32 ``[K]``: ``(x * rstd) * (1 + scale) + shift``).  The
+    norm prologue of the fused projections as one launch, for projections that run as a library GEMM."""
+    lib = native.lib()
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or x.stride(1) != 1:
+        raise TypeError("rms_norm_rows: x must be a 2-D bf16 tensor with contiguous rows")
+    if (norm_w is None) == (ada is None):
+        raise ValueError("rms_norm_rows: exactly one of norm_w and ada")
+    m, k = x.shape
+    if norm_w is not None and (norm_w.dtype != torch.bfloat16 or norm_w.numel() != k):
+        raise TypeError("rms_norm_rows: norm_w must be bf16 [K]")
+    if ada is not None and any(t.dtype != torch.float32 or t.numel() != k or not t.is_contiguous() for t in ada):
+        raise TypeError("rms_norm_rows: ada scale / shift must be contiguous fp32 [K]")
+    y = torch.empty(m, k, dtype=torch.bfloat16, device=x.device)
+    rc = lib.tk_rms_norm_rows(
+        x.data_ptr(), x.stride(0), norm_w.contiguous().data_ptr() if norm_w is not None else None,
+        ada[0].data_ptr() if ada is not None else None, ada[1].data_ptr() if ada is not None else None, float(eps),
+        y.data_ptr(), y.stride(0), m, k, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_rms_norm_rows")
+    return y
+
+
+def rope_rows(y: torch.Tensor, rope: RopeTables, rope_pos: torch.Tensor, rope_cols: int, *, rope_bf16: bool = False) -> torch.Tensor:
+    """Rotary embedding in place on the first ``rope_cols`` columns of a bf16 projection output
+    ``y [M, N]`` (heads of ``2 * rope.half`` columns), int32 positions ``[M]``.  Returns ``y``."""
+    lib = native.lib()
+    if y.dtype != torch.bfloat16 or y.dim() != 2 or y.stride(1) != 1:
+        raise TypeError("rope_rows: y must be a 2-D bf16 tensor with contiguous rows")
+    if rope_pos.dtype != torch.int32 or rope_pos.numel() != y.shape[0] or not rope_pos.is_contiguous():
+        raise TypeError("rope_rows: positions must be contiguous int32 [M]")
+    if rope_cols > y.shape[1]:
+        raise ValueError("rope_rows: rope_cols exceeds the row width")
+    rc = lib.tk_rope_rows(y.data_ptr(), y.stride(0), rope_pos.data_ptr(), rope.cos.data_ptr(), rope.sin.data_ptr(), rope.positions,
+                          int(rope_cols), rope.half, int(rope_bf16), y.shape[0], _stream())  # fmt: skip
+    native.check(rc, "tk_rope_rows")
+    return y
+
+
 def decode_fp8_table(device: torch.device | str = "cuda") -> torch.Tensor:
     """Values of all 256 e4m3fn codes as the device's conversion instruction decodes them."""
     out = torch.empty(256, dtype=torch.float32, device=device)

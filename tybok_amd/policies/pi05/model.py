@@ -126,6 +126,12 @@ class PI05Model:
             self.exp_qkv, self.exp_o = pack_stack(EXP, self.ed["depth"])
         if self.fused_prefill:
             self.vlm_qkv, self.vlm_o = pack_stack(VLM, self.depth)
+            # the same q|k|v weights row-major, for prefixes long enough that the projection is a plain
+            # many-row GEMM (library call) followed by the rotary kernel
+            self.vlm_qkv_plain = [
+                torch.cat([self.p[f"{VLM}layers.{i}.self_attn.{n}_proj.weight"] for n in "qkv"], dim=0).to(BF16).contiguous()
+                for i in range(self.depth)
+            ]
             # Gemma RMSNorm x * rstd * (1 + w) is the adaptive norm with scale = w and shift = 0
             zeros = torch.zeros(self.vd["width"], dtype=torch.float32, device=self.device)
             self.vlm_norms = [
@@ -320,12 +326,19 @@ class PI05Model:
         vt_all = torch.zeros(self.depth, nkv, p_pad, dtype=BF16, device=self.device)
         hidden = embs[0].to(BF16)
         kv, caches = [], []
+        many_rows = p_len >= 256 and nkv % 64 == 0
         for i in range(self.depth):
             norm_in, norm_post = self.vlm_norms[i]
-            qkv = tk.bf16w_linear(
-                hidden, self.vlm_qkv[i], ada=norm_in, eps=EPS, rope=self.rope_tables_hip, rope_pos=pos32, rope_cols=nq + nkv,
-                rope_bf16=True, vt_out=vt_all[i], vt_col0=nq + nkv, out=qkv_all[i], ws=self.ws,
-            )  # fmt: skip
+            if many_rows:
+                # norm, library GEMM, rotary embedding in place, V^T through the tiled transpose
+                qkv = torch.matmul(tk.rms_norm_rows(hidden, ada=norm_in, eps=EPS), self.vlm_qkv_plain[i].t(), out=qkv_all[i])
+                tk.rope_rows(qkv, self.rope_tables_hip, pos32, nq + nkv, rope_bf16=True)
+                tk.transpose_v(qkv[:, nq + nkv :].view(1, p_len, nkv // 64, 64), out=vt_all[i].view(1, nkv // 64, 64, p_pad))
+            else:
+                qkv = tk.bf16w_linear(
+                    hidden, self.vlm_qkv[i], ada=norm_in, eps=EPS, rope=self.rope_tables_hip, rope_pos=pos32, rope_cols=nq + nkv,
+                    rope_bf16=True, vt_out=vt_all[i], vt_col0=nq + nkv, out=qkv_all[i], ws=self.ws,
+                )  # fmt: skip
             k = qkv[:, nq : nq + nkv].view(p_len, g, d)
             cache = tk.PrefixKV(k, vt_all[i].view(g, d, p_pad))
             att = tk.expert_attn(qkv[:, :nq].view(p_len, heads, d), cache, None, None, tk.MASK_NONE, mask2d=mask2d, logits_bf16=True, ws=self.ws)
