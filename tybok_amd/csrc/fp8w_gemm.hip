@@ -40,9 +40,6 @@ namespace {
 // LDS-only barrier: waits for this wave's LDS traffic, not for the global prefetch queue
 // (a full __syncthreads() would drain vmcnt and serialise the weight stream every round).
 __device__ __forceinline__ void lds_barrier() {
-#ifdef TK_EXP_NOBARRIER
-  return;
-#endif
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -151,9 +148,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     i32x4 nw[PRO ? XPT : 1][ADA ? 4 : 1];  // norm weights of the piece's 8 columns (ADA: fp32 scale, shift)
   };
   auto xload = [&](XFrag& f, int r) {
-#ifdef TK_EXP_NOX
-    if (r > 0) return;
-#endif
     const int k0 = (kt_lo + r * RKT) * 32;
 #pragma unroll
     for (int i = 0; i < XPT; ++i) {
@@ -648,6 +642,10 @@ __global__ void decode_fp8_kernel(float* out) {
   out[c] = bf16_bits_to_f32((u16)(cv.u & 0xffff));
 }
 
+// Pipeline depth (block rounds in flight) and k tiles per wave and round.  Measured on MI355X: 4 rounds
+// cover the weight stream's latency at the 33.5 MB shapes; two k tiles per wave and round halve the
+// barriers but lengthen every small launch of the denoise loop (request +0.8 ms).  Overridable at
+// compile time for tuning runs.
 #ifndef TK_EXP_PF
 #define TK_EXP_PF 4
 #endif
