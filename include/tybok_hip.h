@@ -298,6 +298,14 @@ int tk_rope_rows(void* y, int ldy, const void* rope_pos, const void* rope_cos, c
 int tk_layer_norm(const void* x, int ldx, int x_dtype, const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy,
                   int M, int K, void* stream);
 
+/* The residual add that closes a tower branch and the LayerNorm that opens the next one, in one
+ * launch: xsum = x + r (r bf16 [M, K]: the branch's last linear; the sum in x's type -- fp32 rows:
+ * x + float(r); bf16 rows: rounded once -- and xsum may be x itself), y = bf16(LayerNorm(xsum) * w + b).
+ * Other arguments as tk_layer_norm (`hidden = residual + hidden; hidden = layer_norm(hidden)`,
+ * tybok/policies/smolvla/models/vision.py:197-257, tybok/policies/pi05/models/vision.py:115-170). */
+int tk_add_layer_norm(const void* x, int ldx, int x_dtype, const void* r, int ldr, void* xsum, int ldxs, const void* w,
+                      const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream);
+
 /* ---- tail of a denoising step ---------------------------------------------------------------- */
 /* Final norm of the expert hidden state + fp32 action projection + Euler update in one launch:
  *   h = norm(x) (bf16 row; norm_w: Llama RMSNorm bf16(w * bf16(x * rstd)); or ada_scale / ada_shift:

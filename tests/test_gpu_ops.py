@@ -339,6 +339,26 @@ def test_layer_norm_with_folded_cast(tk, dtype, m, k):
         tk.layer_norm(x.cuda(), w.float().cuda(), b.half().cuda(), 1e-6)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,k", [(512, 1152), (3072, 768), (5, 8)])
+def test_residual_add_and_layer_norm_in_one_launch(tk, dtype, m, k):
+    # x += r (the sum in x's type: exact for fp32 rows, rounded once for bf16 rows), then the LayerNorm of the sum
+    g = torch.Generator().manual_seed(62)
+    x = (torch.randn(m, k, generator=g) * 2.0).to(dtype)
+    r = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w, b = (1.0 + 0.3 * torch.randn(k, generator=g)).to(dtype), (0.2 * torch.randn(k, generator=g)).to(dtype)
+    want_sum = x + r  # torch promotes bf16 to fp32 for fp32 x; bf16 + bf16 rounds once
+    assert want_sum.dtype == dtype
+    want = torch.nn.functional.layer_norm(want_sum.float(), (k,), w.float(), b.float(), 1e-6).to(torch.bfloat16)
+    xd = x.cuda()
+    got_x, got = tk.add_layer_norm(xd, r.cuda(), w.cuda(), b.cuda(), 1e-6)
+    assert got_x.data_ptr() == xd.data_ptr() and torch.equal(got_x.cpu(), want_sum)
+    diff = (got.float().cpu() - want.float()).abs()
+    assert bool((diff <= want.float().abs().clamp_min(2.0**-6) * 2.0**-7).all())
+    assert float((diff > 0).float().mean()) < 0.02
+    assert torch.equal(got, tk.layer_norm(got_x, w.cuda(), b.cuda(), 1e-6))  # same kernel arithmetic after the add
+
+
 def test_gated_residual_epilogue(tk):
     # pi0.5 AdaRMS gated residual: y = resid + bf16(ffn(x) * gate)
     x, wg8, sg, wu8, su, wd8, sd = ffn_case(50, 1024, 4096, seed=3)

@@ -12,7 +12,10 @@ namespace {
 
 constexpr int PMAX = 4;  // 8-element pieces per lane: rows up to 64 * 8 * PMAX = 2048 columns
 
-template <bool XF32, bool WF32>
+// ADD: the rows are x + r first (r bf16: the output of the linear that closes a residual branch), the
+// sum is written back in x's type (fp32: x + float(r); bf16: rounded once, as torch's bf16 add) and
+// normalised -- the residual add and the next LayerNorm of a tower layer in one launch.
+template <bool XF32, bool WF32, bool ADD>
 __global__ __launch_bounds__(256) void layer_norm_kernel(LayerNormArgs a) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -36,6 +39,30 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(LayerNormArgs a) {
         for (int e = 0; e < 4; ++e) {
           v[i][2 * e] = __uint_as_float(xu.u[e] << 16);
           v[i][2 * e + 1] = __uint_as_float(xu.u[e] & 0xffff0000u);
+        }
+      }
+      if (ADD) {
+        union { i32x4 q; unsigned u[4]; } ru;
+        ru.q = *(const i32x4*)(a.r + (size_t)row * a.ldr + 8 * p);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[i][2 * e] += __uint_as_float(ru.u[e] << 16);
+          v[i][2 * e + 1] += __uint_as_float(ru.u[e] & 0xffff0000u);
+        }
+        if (XF32) {
+          f32x4* dst = (f32x4*)((float*)a.xsum + (size_t)row * a.ldxs + 8 * p);
+          const f32x4 lo = {v[i][0], v[i][1], v[i][2], v[i][3]}, hi = {v[i][4], v[i][5], v[i][6], v[i][7]};
+          dst[0] = lo;
+          dst[1] = hi;
+        } else {
+          union { i32x4 q; unsigned u[4]; } su;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            su.u[e] = pack_bf16x2(v[i][2 * e], v[i][2 * e + 1]);
+            v[i][2 * e] = __uint_as_float(su.u[e] << 16);
+            v[i][2 * e + 1] = __uint_as_float(su.u[e] & 0xffff0000u);
+          }
+          *(i32x4*)((u16*)a.xsum + (size_t)row * a.ldxs + 8 * p) = su.q;
         }
       }
 #pragma unroll
@@ -96,11 +123,19 @@ int tk_layer_norm_max_k() { return 64 * 8 * PMAX; }
 
 int tk_launch_layer_norm(LayerNormArgs a, hipStream_t st) {
   dim3 grid((a.M + 3) / 4);
-  if (a.x_f32 && a.wb_f32)
-    hipLaunchKernelGGL((layer_norm_kernel<true, true>), grid, dim3(256), 0, st, a);
-  else if (!a.x_f32 && !a.wb_f32)
-    hipLaunchKernelGGL((layer_norm_kernel<false, false>), grid, dim3(256), 0, st, a);
-  else
+  const bool add = a.r != nullptr;
+  if (a.x_f32 && a.wb_f32) {
+    if (add)
+      hipLaunchKernelGGL((layer_norm_kernel<true, true, true>), grid, dim3(256), 0, st, a);
+    else
+      hipLaunchKernelGGL((layer_norm_kernel<true, true, false>), grid, dim3(256), 0, st, a);
+  } else if (!a.x_f32 && !a.wb_f32) {
+    if (add)
+      hipLaunchKernelGGL((layer_norm_kernel<false, false, true>), grid, dim3(256), 0, st, a);
+    else
+      hipLaunchKernelGGL((layer_norm_kernel<false, false, false>), grid, dim3(256), 0, st, a);
+  } else {
     return -1;
+  }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }

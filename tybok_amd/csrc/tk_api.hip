@@ -724,12 +724,14 @@ int tk_rope_rows(void* y, int ldy, const void* rope_pos, const void* rope_cos, c
   return TK_OK;
 }
 
-int tk_layer_norm(const void* x, int ldx, int x_dtype, const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy,
-                  int M, int K, void* stream) {
-  if (M <= 0 || K <= 0 || K % 8 || K > tk_layer_norm_max_k()) return fail(TK_EINVAL, "layer_norm: K=%d must be a multiple of 8, at most %d", K, tk_layer_norm_max_k());
-  if ((x_dtype != TK_BF16 && x_dtype != TK_F32) || x_dtype != wb_dtype) return fail(TK_EINVAL, "layer_norm: rows and parameters must both be bf16 or both fp32");
-  if (!x || !w || !b || !y || ldx < K || ldy < K || ldx % 8 || ldy % 8) return fail(TK_EINVAL, "layer_norm: null pointer or row pitch not a multiple of 8 >= K");
-  if (!aligned16(x) || !aligned16(w) || !aligned16(b) || !aligned16(y)) return fail(TK_EINVAL, "layer_norm: operands must be 16-byte aligned");
+static int layer_norm_impl(const char* who, const void* x, int ldx, int x_dtype, const void* r, int ldr, void* xsum, int ldxs,
+                           const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream) {
+  if (M <= 0 || K <= 0 || K % 8 || K > tk_layer_norm_max_k()) return fail(TK_EINVAL, "%s: K=%d must be a multiple of 8, at most %d", who, K, tk_layer_norm_max_k());
+  if ((x_dtype != TK_BF16 && x_dtype != TK_F32) || x_dtype != wb_dtype) return fail(TK_EINVAL, "%s: rows and parameters must both be bf16 or both fp32", who);
+  if (!x || !w || !b || !y || ldx < K || ldy < K || ldx % 8 || ldy % 8) return fail(TK_EINVAL, "%s: null pointer or row pitch not a multiple of 8 >= K", who);
+  if (!aligned16(x) || !aligned16(w) || !aligned16(b) || !aligned16(y)) return fail(TK_EINVAL, "%s: operands must be 16-byte aligned", who);
+  if (r && (!xsum || ldr < K || ldxs < K || ldr % 8 || ldxs % 8 || !aligned16(r) || !aligned16(xsum)))
+    return fail(TK_EINVAL, "%s: the residual branch and the sum need 16-byte aligned pointers and row pitches that are multiples of 8 >= K", who);
   LayerNormArgs a;
   a.x = x;
   a.ldx = ldx;
@@ -742,8 +744,23 @@ int tk_layer_norm(const void* x, int ldx, int x_dtype, const void* w, const void
   a.ldy = ldy;
   a.M = M;
   a.K = K;
-  if (tk_launch_layer_norm(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "layer_norm: launch failed");
+  a.r = (const u16*)r;
+  a.ldr = ldr;
+  a.xsum = xsum;
+  a.ldxs = ldxs;
+  if (tk_launch_layer_norm(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "%s: launch failed", who);
   return TK_OK;
+}
+
+int tk_layer_norm(const void* x, int ldx, int x_dtype, const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy,
+                  int M, int K, void* stream) {
+  return layer_norm_impl("layer_norm", x, ldx, x_dtype, nullptr, 0, nullptr, 0, w, b, wb_dtype, eps, y, ldy, M, K, stream);
+}
+
+int tk_add_layer_norm(const void* x, int ldx, int x_dtype, const void* r, int ldr, void* xsum, int ldxs, const void* w,
+                      const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream) {
+  if (!r) return fail(TK_EINVAL, "add_layer_norm: null residual branch");
+  return layer_norm_impl("add_layer_norm", x, ldx, x_dtype, r, ldr, xsum, ldxs, w, b, wb_dtype, eps, y, ldy, M, K, stream);
 }
 
 int tk_debug_decode_fp8(void* out_f32, void* stream) {

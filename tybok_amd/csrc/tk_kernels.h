@@ -129,6 +129,12 @@ struct LayerNormArgs {
   unsigned short* y;  // bf16 [M, K], element pitch ldy
   int ldy;
   int M, K;
+  // optional residual branch: rows are x + r (r bf16, pitch ldr), the sum goes to xsum in x's type
+  // (pitch ldxs; may be x itself)
+  const unsigned short* r;
+  int ldr;
+  void* xsum;
+  int ldxs;
 };
 
 struct TailArgs {

@@ -678,6 +678,28 @@ def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) ->
     return y.view(x.shape)
 
 
+def add_layer_norm(x: torch.Tensor, r: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) -> tuple[torch.Tensor, torch.Tensor]:
+    """``x += r`` in place (``r`` bf16: the linear that closes a residual branch; fp32 ``x`` takes
+    ``float(r)``, bf16 ``x`` rounds the sum once) and ``bf16(LayerNorm(x) * w + b)`` of the sum, one launch.
+    Returns ``(x, normalised)``; ``x`` must own contiguous rows."""
+    lib = native.lib()
+    if x.dtype not in (torch.float32, torch.bfloat16) or w.dtype != x.dtype or b.dtype != x.dtype or r.dtype != torch.bfloat16:
+        raise TypeError("add_layer_norm: x, w, b all fp32 or all bf16; r bf16")
+    k = x.shape[-1]
+    if r.shape != x.shape or not x.is_contiguous() or w.numel() != k or b.numel() != k:
+        raise ValueError("add_layer_norm: r must have x's shape, x contiguous, w and b hold K values")
+    x2, r2 = x.view(-1, k), r.reshape(-1, k)
+    if r2.stride(1) != 1:
+        r2 = r2.contiguous()
+    y = torch.empty(x2.shape, dtype=torch.bfloat16, device=x.device)
+    dt = _F32 if x.dtype == torch.float32 else _BF16
+    rc = lib.tk_add_layer_norm(x2.data_ptr(), x2.stride(0), dt, r2.data_ptr(), r2.stride(0), x2.data_ptr(), x2.stride(0),
+                               w.contiguous().data_ptr(), b.contiguous().data_ptr(), dt, float(eps), y.data_ptr(), y.stride(0),
+                               x2.shape[0], k, _stream())  # fmt: skip
+    native.check(rc, "tk_add_layer_norm")
+    return x, y.view(x.shape)
+
+
 def rms_norm_rows(x: torch.Tensor, *, norm_w: torch.Tensor | None = None, ada: tuple[torch.Tensor, torch.Tensor] | None = None, eps: float) -> torch.Tensor:
     """RMSNorm of bf16 rows ``x [M, K]`` into a new bf16 tensor: Llama (``norm_w`` bf16 ``[K]``) or
     Gemma / adaptive (``ada = (scale, shift)`` fp32 ``[K]``: ``(x * rstd) * (1 + scale) + shift``).  The

@@ -234,6 +234,8 @@ class PI05Model:
         x = x + p[VIS + "embeddings.position_embedding.weight"][None]
         vh, heads = cfg.vision_hidden, cfg.vision_heads
         hd = vh // heads
+        if self.vit_lowp_attn and self.vit_mlp_dtype == BF16 and x.is_cuda and self.vis_head_pad in (64, 96):
+            return self._tower_bf16_linears(x.contiguous())
         for i in range(cfg.vision_layers):
             lp = f"{VIS}encoder.layers.{i}."
             if self.vit_lowp_attn:
@@ -266,6 +268,28 @@ class PI05Model:
             else:
                 h = F.layer_norm(x, (vh,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS)
                 x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
+        x = F.layer_norm(x, (vh,), p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], EPS)
+        return self.lin(PROJ, x)
+
+    def _tower_bf16_linears(self, x: torch.Tensor) -> torch.Tensor:
+        """The tower with every linear in bf16 (both low-precision tiers on): fp32 residual stream updated
+        in place, each residual add in the launch of the LayerNorm that follows it, attention on the HIP
+        kernel (fp32 scores and softmax, probabilities rounded to bf16 for P.V)."""
+        cfg, p = self.cfg, self.p
+        b, vh, heads, hp = x.shape[0], cfg.vision_hidden, cfg.vision_heads, self.vis_head_pad
+        hd = vh // heads
+        ln = lambda i, n: (p[f"{VIS}encoder.layers.{i}.layer_norm{n}.weight"], p[f"{VIS}encoder.layers.{i}.layer_norm{n}.bias"])  # noqa: E731
+        h = tk.layer_norm(x, *ln(0, 1), EPS)
+        for i in range(cfg.vision_layers):
+            lp = f"{VIS}encoder.layers.{i}."
+            qkv = F.linear(h, *self.vis_lowp[lp + "self_attn.qkv"]).view(b, -1, 3, heads, hp)
+            a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], tk.transpose_v(qkv[:, :, 2]), scale=hd**-0.5, ws=self.ws)
+            x, h = tk.add_layer_norm(x, F.linear(a, *self.vis_lowp[lp + "self_attn.out_proj"]), *ln(i, 2), EPS)
+            m = F.linear(F.gelu(F.linear(h, *self.vis_lowp[lp + "mlp.fc1"]), approximate="tanh"), *self.vis_lowp[lp + "mlp.fc2"])
+            if i + 1 < cfg.vision_layers:
+                x, h = tk.add_layer_norm(x, m, *ln(i + 1, 1), EPS)
+            else:
+                x = x + m
         x = F.layer_norm(x, (vh,), p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], EPS)
         return self.lin(PROJ, x)
 

@@ -240,16 +240,22 @@ class SmolVLAModel:
         for i in range(v.num_hidden_layers):
             lp = f"{VIS}encoder.layers.{i}."
             if self.fused_vit:
-                h = tk.layer_norm(x, p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], v.layer_norm_eps)
+                # each residual add runs in the launch of the LayerNorm that follows it (x is updated in place)
+                if i == 0:
+                    h = tk.layer_norm(x, p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], v.layer_norm_eps)
                 # packed q|k|v GEMM, then the HIP attention (one problem per camera): q.K^T rounded to
                 # bf16 before the fp32 scale and softmax, exactly what the bf16 matmul below produces
                 w_qkv, b_qkv = self.vis_qkv[i]
                 qkv = F.linear(h, w_qkv, b_qkv).view(b, -1, 3, heads, hd)
                 vt = tk.transpose_v(qkv[:, :, 2])
                 a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, ws=self.ws)
-                x = x + self.lin(lp + "self_attn.out_proj", a)
-                h = tk.layer_norm(x, p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
-                x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
+                x, h = tk.add_layer_norm(x, self.lin(lp + "self_attn.out_proj", a), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
+                m = self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
+                if i + 1 < v.num_hidden_layers:
+                    nx = f"{VIS}encoder.layers.{i + 1}."
+                    x, h = tk.add_layer_norm(x, m, p[nx + "layer_norm1.weight"], p[nx + "layer_norm1.bias"], v.layer_norm_eps)
+                else:
+                    x = x + m
                 continue
             h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], v.layer_norm_eps)
             q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
