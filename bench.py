@@ -372,6 +372,15 @@ def main() -> None:
         "frac_of_bf16_mfma_peak": round(f_tflops / 2500.0, 4),
     }
 
+    # ---- the single-op configurations at the action-chunk shape: latency-bound launches ----
+    c1_us = ffn_launch_us(50, 720, 2048, launches=50, reps=10)
+    c1_bytes = 3 * 720 * 2048 + 4 * (2 * 2048 + 720) + 2 * 50 * 720 * 2  # fp8 weights, fp32 scales, bf16 in / out
+    ops_small = {
+        "ffn_M50_K720_I2048": {"us": round(c1_us, 2), "GBps": round(c1_bytes / c1_us / 1e3, 1), "launches": 2},
+        "expert_attn_M50_P241_S50_H15_G5_D64": {"us": round(attn_launch_us(launches=50, reps=10), 2)},
+        "tower_attn_B3_M1024_H12_D64": {"us": round(tower_attn_launch_us(launches=20, reps=10), 2)},
+    }
+
     cpu = None if args.skip_cpu else cpu_baseline_smolvla(3)
 
     p50 = float(np.percentile(samples3, 50))
@@ -399,6 +408,7 @@ def main() -> None:
         "pi05_2cam_p50_ms": None if pi05_p50 is None else round(pi05_p50, 3),
         "pi05_tiers": "tl_fused_expert, tl_fp8_expert_mlp, tl_fp8_llm_mlp, tl_llm_flash_attn, tl_fused_vit",
         "gemm_sweep_M50": sweep,
+        "ops_action_chunk_shape": ops_small,
         "pi05_prefill_ffn_M712": prefill_ffn,
         "roofline": roofline,
         "cpu_baseline": cpu,
