@@ -1,18 +1,18 @@
-"""Model-agnostic engine interface, API-compatible with the reference's ``tybok/base.py``.
+"""The engine interface the serving side of tybok programs against.
 
-The gateway / worker layers of the reference only depend on this interface
-(``PolicyEngine.{describe, select_action, predict_action_chunk, validate, profile}``:
-tybok/base.py:50-235), so a backend registered under the same name with the same constructor
-keywords is a drop-in.  ``compile_region`` (torch.compile plumbing) has no counterpart here: the
-HIP tiers replace it, and ``compile_model=True`` is rejected by the backends.
+The reference's gateway and worker only touch ``PolicyEngine.{describe, select_action,
+predict_action_chunk, validate, profile, make_frame}`` (tybok/base.py:50-235); a backend registered
+under the same model name, with the same constructor keywords and the same return types, is a
+drop-in for them.  The reference's ``compile_region`` (torch.compile plumbing) has no counterpart: the
+HIP tiers take its place and the backends reject ``compile_model=True``.
 """
 
 from __future__ import annotations
 
+import abc
 import logging
 import time
-from abc import ABC, abstractmethod
-from collections.abc import Mapping
+from collections.abc import Mapping, Sequence
 from typing import Any
 
 import numpy as np
@@ -20,8 +20,31 @@ import torch
 
 log = logging.getLogger("tybok.engine")
 
+_IMAGE_PREFIX = "observation.images."
+_CHANNEL_COUNTS = (1, 3, 4)
 
-class PolicyEngine(ABC):
+
+def _resolve_device(device: str) -> str:
+    return ("cuda" if torch.cuda.is_available() else "cpu") if device == "auto" else device
+
+
+def _as_chw_float(name: str, image: Any) -> torch.Tensor:
+    """One camera image as a contiguous fp32 ``(C, H, W)`` tensor; ``(H, W, C)`` input is transposed."""
+    if isinstance(image, np.ndarray):
+        image = torch.from_numpy(image)
+    if not isinstance(image, torch.Tensor):
+        raise TypeError(f"image {name} must be a tensor or ndarray")
+    channels_last = image.ndim == 3 and image.shape[0] not in _CHANNEL_COUNTS
+    return (image.permute(2, 0, 1) if channels_last else image).float().contiguous()
+
+
+def _as_state(state: Any) -> torch.Tensor:
+    if isinstance(state, torch.Tensor):
+        return state.float().contiguous()
+    return torch.from_numpy(np.asarray(state, dtype=np.float32)).contiguous()
+
+
+class PolicyEngine(abc.ABC):
     """Base class of the policy backends (inference only)."""
 
     config: Any
@@ -30,116 +53,99 @@ class PolicyEngine(ABC):
 
     def __init__(self, checkpoint_dir: str, device: str = "auto", **kwargs):
         self.checkpoint_dir = checkpoint_dir
-        if device == "auto":
-            device = "cuda" if torch.cuda.is_available() else "cpu"
-        self.device = device
-        self.compiled_regions: list[str] = []
-        if isinstance(device, str) and device.startswith("cuda"):
-            dev = torch.device(device)
-            if dev.index is not None:
-                torch.cuda.set_device(dev)
+        self.device = _resolve_device(device)
+        self.compiled_regions: list[str] = []  # kept for callers that report it; always empty here
+        if str(self.device).startswith("cuda") and torch.device(self.device).index is not None:
+            torch.cuda.set_device(torch.device(self.device))
 
-    # ------------------------------------------------------------------ interface
-    @abstractmethod
+    # ------------------------------------------------------------------ what a backend implements
+    @abc.abstractmethod
     def describe(self) -> dict[str, Any]:
         """``{"model_type", "cameras", "resize": [W, H], "action_dim", "chunk_size", ...}``."""
 
-    @abstractmethod
+    @abc.abstractmethod
     def select_action(self, frame: dict[str, Any], noise: torch.Tensor | None = None) -> np.ndarray:
-        """One action ``(action_dim,)`` for one observation frame."""
+        """The next action ``(action_dim,)`` for one observation frame."""
 
-    @abstractmethod
+    @abc.abstractmethod
     def predict_action_chunk(self, frame: dict[str, Any], noise: torch.Tensor | None = None) -> np.ndarray:
-        """Full chunk ``(chunk_size, action_dim)`` for one observation frame."""
+        """A whole chunk ``(chunk_size, action_dim)`` for one observation frame."""
 
-    @abstractmethod
+    @abc.abstractmethod
     def validate(self, reference_dir: str) -> dict[str, float]:
-        """Score this backend against a reference dump directory."""
+        """Per-component errors of this backend against a dump directory of the reference."""
 
     def supports_rtc(self) -> bool:
         return False
 
-    # ------------------------------------------------------------------ shared helpers
-    def make_frame(
-        self,
-        images: Mapping[str, torch.Tensor | np.ndarray],
-        state: torch.Tensor | np.ndarray | list,
-        task: str,
-    ) -> dict[str, Any]:
-        """Raw frame dict: ``(C,H,W)`` fp32 images in [0,1] under ``observation.images.<cam>``,
-        a 1-D fp32 ``observation.state`` and the ``task`` string."""
-        frame: dict[str, Any] = {}
-        for key, img in images.items():
-            if isinstance(img, np.ndarray):
-                img = torch.from_numpy(img)
-            if not torch.is_tensor(img):
-                raise TypeError(f"image {key} must be a tensor or ndarray")
-            if img.ndim == 3 and img.shape[0] not in (1, 3, 4):
-                img = img.permute(2, 0, 1)  # HWC -> CHW
-            frame[f"observation.images.{key}"] = img.float().contiguous()
-        if isinstance(state, (list, tuple)):
-            state = np.asarray(state, dtype=np.float32)
-        if isinstance(state, np.ndarray):
-            state = torch.from_numpy(state.astype(np.float32))
-        frame["observation.state"] = state.float().contiguous()
+    # ------------------------------------------------------------------ frames
+    def make_frame(self, images: Mapping[str, torch.Tensor | np.ndarray], state: torch.Tensor | np.ndarray | Sequence[float], task: str) -> dict[str, Any]:
+        """The raw frame dict of a request: fp32 ``(C, H, W)`` images in [0, 1] under
+        ``observation.images.<camera>``, a 1-D fp32 ``observation.state`` and the ``task`` string."""
+        frame: dict[str, Any] = {_IMAGE_PREFIX + name: _as_chw_float(name, image) for name, image in images.items()}
+        frame["observation.state"] = _as_state(state)
         frame["task"] = task
         return frame
 
-    def _warmup(self) -> None:
-        """One dummy inference so lazy initialisation does not land on the first request."""
-        spec = self.describe()
-        t0 = time.perf_counter()
-        images = {cam: torch.zeros(3, spec["resize"][1], spec["resize"][0]) for cam in spec["cameras"]}
-        frame = self.make_frame(images, torch.zeros(8), "warmup")
-        self.predict_action_chunk(frame)
-        if str(self.device).startswith("cuda"):
-            torch.cuda.synchronize()
-        log.info(f"warmup done in {time.perf_counter() - t0:.1f}s")
+    def _camera_names(self, cameras: int | None) -> list[str]:
+        names = [c.split(_IMAGE_PREFIX)[-1] for c in self.describe()["cameras"]]
+        return names if cameras is None else names[:cameras]
 
     def _profile_frame(self, cameras: int | None = None, seed: int = 0) -> dict[str, Any]:
-        """Synthetic frame: random images for the configured (or requested) cameras + random state."""
-        spec = self.describe()
-        g = torch.Generator().manual_seed(seed)
-        cams = spec["cameras"] if cameras is None else spec["cameras"][:cameras]
-        images = {
-            cam.split("observation.images.")[-1]: torch.rand(3, spec["resize"][1], spec["resize"][0], generator=g)
-            for cam in cams
-        }
-        state = torch.rand(int(getattr(self.config, "proprio_dim", None) or 8), generator=g)
-        return self.make_frame(images, state, "profile")
+        """A seeded synthetic frame: uniform images for the configured (or the first ``cameras``)
+        cameras, drawn in camera order, then a uniform state -- the draw order of the reference, whose
+        tests feed ``_profile_frame(seed=...)`` to the engines they compare."""
+        width, height = self.describe()["resize"]
+        rng = torch.Generator().manual_seed(seed)
+        images = {}
+        for name in self._camera_names(cameras):
+            images[name] = torch.rand(3, height, width, generator=rng)
+        state_dim = int(getattr(self.config, "proprio_dim", None) or 8)
+        return self.make_frame(images, torch.rand(state_dim, generator=rng), "profile")
+
+    # ------------------------------------------------------------------ start-up and timing
+    def _sync(self) -> None:
+        if str(self.device).startswith("cuda") and torch.cuda.is_available():
+            torch.cuda.synchronize()
+
+    def _warmup(self) -> None:
+        """One inference on an all-zero frame, so lazy initialisation never lands on a request."""
+        width, height = self.describe()["resize"]
+        started = time.perf_counter()
+        blank = {name: torch.zeros(3, height, width) for name in self._camera_names(None)}
+        self.predict_action_chunk(self.make_frame(blank, torch.zeros(8), "warmup"))
+        self._sync()
+        log.info("warmup done in %.1fs", time.perf_counter() - started)
 
     def profile(self, iters: int = 5, warmup: int = 3, cameras: int | None = None, seed: int = 0) -> dict[str, Any]:
-        """Wall-time latency of :meth:`predict_action_chunk` on a synthetic frame, engine as configured."""
+        """Wall-clock latency of :meth:`predict_action_chunk` on a synthetic frame, engine as configured."""
         frame = self._profile_frame(cameras, seed)
         for _ in range(warmup):
             self.predict_action_chunk(frame)
-        cuda = str(self.device).startswith("cuda") and torch.cuda.is_available()
-        if cuda:
-            torch.cuda.synchronize()
-        samples = []
-        for _ in range(iters):
-            t0 = time.perf_counter()
+        self._sync()
+        wall_ms = np.empty(iters, dtype=np.float64)
+        for i in range(iters):
+            started = time.perf_counter()
             self.predict_action_chunk(frame)
-            if cuda:
-                torch.cuda.synchronize()
-            samples.append((time.perf_counter() - t0) * 1e3)
+            self._sync()
+            wall_ms[i] = (time.perf_counter() - started) * 1e3
         spec = self.describe()
-        cams = spec["cameras"] if cameras is None else spec["cameras"][:cameras]
         report: dict[str, Any] = {
-            "wall_ms": float(np.mean(samples)),
-            "p50_ms": float(np.percentile(samples, 50)),
-            "p95_ms": float(np.percentile(samples, 95)),
+            "wall_ms": float(wall_ms.mean()),
+            "p50_ms": float(np.percentile(wall_ms, 50)),
+            "p95_ms": float(np.percentile(wall_ms, 95)),
             "iters": iters,
-            "cameras": len(cams),
+            "cameras": len(self._camera_names(cameras)),
             "spec": spec,
             "phases": self._profile_phases(iters=iters, warmup=warmup, cameras=cameras, seed=seed),
         }
-        path = "hip-graph" if getattr(self, "graph_enabled", False) else "eager"
         logging.getLogger(f"tybok.{spec.get('model_type')}").info(
-            f"profile: device={self.device} path={path} cameras={report['cameras']} iters={iters} "
-            f"wall {report['wall_ms']:.2f} ms/iter (p50 {report['p50_ms']:.2f}, p95 {report['p95_ms']:.2f})"
-        )
+            "profile: device=%s path=%s cameras=%d iters=%d wall %.2f ms/iter (p50 %.2f, p95 %.2f)",
+            self.device, "hip-graph" if getattr(self, "graph_enabled", False) else "eager", report["cameras"], iters,
+            report["wall_ms"], report["p50_ms"], report["p95_ms"],
+        )  # fmt: skip
         return report
 
     def _profile_phases(self, iters: int = 5, warmup: int = 3, cameras: int | None = None, seed: int = 0) -> dict[str, float]:
+        """Per-phase timings a backend may add to :meth:`profile`'s report."""
         return {}

@@ -1,31 +1,30 @@
-"""hipGraph plumbing shared by the backends, with the reference's contract
-(tybok/graph.py:60-251): graph keys start with the number of image inputs, warm-up on a side
-stream before capture, lazy capture on first sight, startup pre-capture that tolerates a failing
-key, and input copies on a dedicated stream joined by one event before the replay.
+"""hipGraph plumbing shared by the two backends.
 
-On PyTorch-ROCm ``torch.cuda.CUDAGraph`` is a hipGraph; the HIP kernels of this package are
-launched on torch's current stream, so stream capture records them like any torch op.
+Behaviour follows the reference's helper of the same name (tybok/graph.py:60-251): a captured graph
+is looked up by a key whose first element is the number of image inputs; a shape is run eagerly a
+few times on a forked stream before it is recorded; shapes named at start-up are recorded then and a
+shape that fails to record is reported and left to the eager path; any other shape is recorded the
+first time a request needs it; per request the inputs are copied into the graph's static tensors on
+a stream of their own and the replay waits for that stream through one event.
+
+On PyTorch-ROCm ``torch.cuda.CUDAGraph`` is a hipGraph, and this package's HIP kernels are launched
+on torch's current stream, so stream capture records them exactly like torch's own launches.
 """
 
 from __future__ import annotations
 
-import contextlib
 import logging
-from collections.abc import Callable, Hashable, Iterable
+from collections.abc import Callable, Hashable, Iterable, Iterator
+from contextlib import contextmanager
 from typing import Any
 
 import torch
 
-log = logging.getLogger("tybok.graph")
-
-GRAPH_CAMERAS_HELP = (
-    "comma-separated image counts to pre-capture at startup, e.g. '2,3' "
-    "(default: the configured image count; other counts are captured lazily)"
-)
+_LOG = logging.getLogger("tybok.graph")
 
 
 def camera_counts(graph_cameras: Iterable[int] | None, *, default: int, max_images: int) -> tuple[int, ...]:
-    """Image counts to pre-capture: the valid, de-duplicated, sorted entries of ``--graph-cameras``,
+    """Image counts to record at start-up: the valid, de-duplicated, sorted entries of ``--graph-cameras``,
     else the (clamped) configured count."""
     hi = max(1, int(max_images))
     counts = sorted({int(n) for n in (graph_cameras or ()) if 1 <= int(n) <= hi})
@@ -33,105 +32,130 @@ def camera_counts(graph_cameras: Iterable[int] | None, *, default: int, max_imag
 
 
 class CaptureSession:
-    """Warm-up (side stream, joined back) + capture, both under ``inference_mode``."""
+    """Turns a zero-argument callable into a replayable graph: eager passes first, then the recording."""
 
     def __init__(self, device: str | torch.device, warmup_iters: int = 3):
         self.device = torch.device(device)
-        self.warmup_iters = int(warmup_iters)
+        self.warmup_iters = max(0, int(warmup_iters))
 
     def prime(self, fn: Callable[[], Any], iters: int | None = None) -> None:
-        iters = self.warmup_iters if iters is None else int(iters)
-        main = torch.cuda.current_stream(self.device)
-        side = torch.cuda.Stream(device=self.device)
-        side.wait_stream(main)
-        with torch.inference_mode(), torch.cuda.stream(side):
-            for _ in range(iters):
+        """Eager passes on a stream forked from the current one (lazy initialisation, workspace and
+        allocator warm-up happen here, outside any recording); the current stream waits for them."""
+        current = torch.cuda.current_stream(self.device)
+        fork = torch.cuda.Stream(device=self.device)
+        fork.wait_stream(current)
+        with torch.inference_mode(), torch.cuda.stream(fork):
+            for _ in range(self.warmup_iters if iters is None else max(0, int(iters))):
                 fn()
-        main.wait_stream(side)
+        current.wait_stream(fork)
 
-    @staticmethod
-    def capture(fn: Callable[[], Any]) -> torch.cuda.CUDAGraph:
-        graph = torch.cuda.CUDAGraph()
-        with torch.inference_mode(), torch.cuda.graph(graph):
+    def capture(self, fn: Callable[[], Any]) -> torch.cuda.CUDAGraph:
+        recorded = torch.cuda.CUDAGraph()
+        with torch.inference_mode(), torch.cuda.graph(recorded):
             fn()
-        return graph
+        return recorded
 
     def prime_and_capture(self, fn: Callable[[], Any]) -> torch.cuda.CUDAGraph:
         self.prime(fn)
         return self.capture(fn)
 
-    def sync(self) -> None:
-        torch.cuda.synchronize()
+
+class StaticCall:
+    """One recorded call ``output <- fn(**inputs)``: the static tensors it reads (by keyword; a value
+    may be a list of tensors), the static tensor it writes, and the graph that replays it."""
+
+    def __init__(self, output: torch.Tensor, **inputs: Any):
+        self.inputs = inputs
+        self.output = output
+        self.graph: torch.cuda.CUDAGraph | None = None
+
+    def record(self, session: CaptureSession, fn: Callable[..., torch.Tensor]) -> "StaticCall":
+        def body() -> None:
+            self.output.copy_(fn(**self.inputs))
+
+        self.graph = session.prime_and_capture(body)
+        torch.cuda.synchronize()  # a failed recording surfaces here, not at the first request
+        return self
+
+    def store(self, **values: Any) -> None:
+        """Copy a request's values into the static tensors of the same names (on the current stream)."""
+        for name, value in values.items():
+            slot = self.inputs[name]
+            if isinstance(slot, (list, tuple)):
+                if len(value) != len(slot):
+                    raise ValueError(f"{name}: {len(value)} tensors for {len(slot)} static slots")
+                for dst, src in zip(slot, value):
+                    dst.copy_(src)
+            else:
+                slot.copy_(value)
+
+    def replay(self) -> torch.Tensor:
+        """Run the graph; the result is copied out so the next replay cannot overwrite it."""
+        if self.graph is None:
+            raise RuntimeError("replay() before record()")
+        self.graph.replay()
+        return self.output.clone()
 
 
 class GraphRunner:
-    """``key -> entry`` registry plus the per-request copy/replay primitives."""
+    """Recorded shapes by key, and the two-stream hand-over of a request's inputs.
 
-    def __init__(self, capture_fn: Callable[[Hashable, Any], Any], device, *, label: str = "graph", logger=None):
+    ``record(key, request)`` is the backend's function that builds static tensors for ``key``, records
+    the graph and returns whatever the backend wants to keep for replays (an "entry")."""
+
+    def __init__(self, record: Callable[[Hashable, Any], Any], device, *, label: str = "graph", logger: logging.Logger | None = None):
         self.device = torch.device(device)
         self.label = label
-        self._capture_fn = capture_fn
-        self._log = logger or log
-        self._entries: dict[Hashable, Any] = {}
-        self.copy_stream: torch.cuda.Stream | None = None
-        self.ev_in: torch.cuda.Event | None = None
+        self._record = record
+        self._log = logger if logger is not None else _LOG
+        self._shapes: dict[Hashable, Any] = {}
+        self._input_stream: torch.cuda.Stream | None = None
+        self._inputs_ready: torch.cuda.Event | None = None
 
-    def __bool__(self) -> bool:
-        return bool(self._entries)
-
-    def __contains__(self, key: Hashable) -> bool:
-        return key in self._entries
-
-    def __len__(self) -> int:
-        return len(self._entries)
+    # -- recorded shapes ------------------------------------------------------------------------
+    def __bool__(self) -> bool:  # "is there anything to replay"
+        return len(self._shapes) > 0
 
     def keys(self):
-        return self._entries.keys()
+        return self._shapes.keys()
 
-    @property
-    def entries(self) -> dict[Hashable, Any]:
-        return self._entries
-
-    def get(self, key: Hashable, default: Any = None) -> Any:
-        return self._entries.get(key, default)
-
-    def set(self, key: Hashable, entry: Any) -> None:
-        self._entries[key] = entry
-
-    def clear(self) -> None:
-        self._entries.clear()
+    def forget(self) -> None:
+        """Drop every recorded shape (the backend is going back to the eager path)."""
+        self._shapes.clear()
 
     def entry(self, key: Hashable, request: Any = None) -> Any:
-        got = self._entries.get(key)
-        if got is None:
-            got = self._capture_fn(key, request)
-            self._entries[key] = got
-        return got
+        """The entry of ``key``, recording it now if this is the first request of that shape."""
+        if key not in self._shapes:
+            self._shapes[key] = self._record(key, request)
+        return self._shapes[key]
 
     def precapture(self, keys: Iterable[Hashable]) -> bool:
-        """Capture ``keys`` now; True if at least one succeeded (a failing key is logged and skipped)."""
-        ok = False
+        """Record every key of ``keys`` that can be recorded; False if none could."""
+        recorded = 0
         for key in keys:
             try:
-                self.set(key, self._capture_fn(key, None))
-                ok = True
-            except Exception as e:  # noqa: BLE001 - a failed shape is a result, not a crash
-                self._log.warning(f"{self.label} capture for {key} failed ({e}); that shape falls back to eager")
-        return ok
+                self._shapes[key] = self._record(key, None)
+            except Exception as exc:  # noqa: BLE001 - the shape simply stays on the eager path
+                self._log.warning("%s: recording %s failed (%s); requests of that shape run eagerly", self.label, key, exc)
+            else:
+                recorded += 1
+        return recorded > 0
 
-    @contextlib.contextmanager
-    def copy_inputs(self):
-        """Fork the main stream into the copy stream for the input copies (joined by :meth:`wait_inputs`)."""
-        if self.copy_stream is None:
-            self.copy_stream = torch.cuda.Stream(device=self.device)
-            self.ev_in = torch.cuda.Event()
-        main = torch.cuda.current_stream(self.device)
-        with torch.cuda.stream(self.copy_stream):
-            self.copy_stream.wait_stream(main)
-            yield self.copy_stream
-            assert self.ev_in is not None
-            self.ev_in.record(self.copy_stream)
+    # -- inputs of one request ------------------------------------------------------------------
+    @contextmanager
+    def copy_inputs(self) -> Iterator[torch.cuda.Stream]:
+        """Inside the block, copies into the static tensors run on the input stream (ordered after
+        everything already queued on the current stream); leaving it marks the inputs ready."""
+        if self._input_stream is None:
+            self._input_stream = torch.cuda.Stream(device=self.device)
+            self._inputs_ready = torch.cuda.Event()
+        self._input_stream.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(self._input_stream):
+            yield self._input_stream
+            self._inputs_ready.record(self._input_stream)
 
     def wait_inputs(self) -> None:
-        assert self.ev_in is not None, "copy_inputs() must run before wait_inputs()"
-        torch.cuda.current_stream(self.device).wait_event(self.ev_in)
+        """Order the current stream (the replay) after the copies of the last :meth:`copy_inputs` block."""
+        if self._inputs_ready is None:
+            raise RuntimeError("wait_inputs() called before any copy_inputs() block")
+        torch.cuda.current_stream(self.device).wait_event(self._inputs_ready)

@@ -10,6 +10,7 @@ import glob
 import hashlib
 import os
 from dataclasses import dataclass, field
+from typing import Any
 
 import torch
 
@@ -133,3 +134,53 @@ def load_state_dict(checkpoint_dir: str, wanted: dict[str, tuple], remap: dict[s
     if missing:
         raise FileNotFoundError(f"{len(missing)} parameters missing from {checkpoint_dir} (e.g. {missing[0]})")
     return out
+
+
+# ---------------------------------------------------------------------- validate() plumbing
+DUMP_FILES = ("frame.pt", "batch.pt", "prefix.pt", "prefix_kv.pt", "denoise.pt", "chunk.pt")
+REQUIRED_DUMP_FILES = ("frame.pt", "chunk.pt")
+
+
+def load_reference_dump(reference_dir: str) -> dict[str, Any]:
+    """The files of a ``validate`` dump directory by stem (``frame``, ``batch``, ``prefix``, ``prefix_kv``,
+    ``denoise``, ``chunk``; the layout of tybok/policies/smolvla/engine.py:668-673).  ``frame`` and
+    ``chunk`` must exist, a missing optional file maps to ``None``.  Files are read with
+    ``weights_only=True``: tensors and plain containers, nothing executable."""
+    dump: dict[str, Any] = {}
+    for name in DUMP_FILES:
+        path = os.path.join(reference_dir, name)
+        if os.path.exists(path):
+            dump[name[:-3]] = torch.load(path, weights_only=True)
+        elif name in REQUIRED_DUMP_FILES:
+            raise FileNotFoundError(f"reference dump {path} missing")
+        else:
+            dump[name[:-3]] = None
+    return dump
+
+
+class ErrorReport(dict):
+    """``{"<component>.max": ..., "<component>.mean": ...}`` -- the keys of the reference's validation report."""
+
+    def compare(self, component: str, got: torch.Tensor, want: torch.Tensor) -> None:
+        got, want = got.detach().float().cpu(), want.detach().float().cpu()
+        if got.shape != want.shape:
+            raise AssertionError(f"{component}: shape mismatch {tuple(got.shape)} vs {tuple(want.shape)}")
+        distance = (got - want).abs()
+        self[f"{component}.max"] = float(distance.max())
+        self[f"{component}.mean"] = float(distance.mean())
+
+    def compare_batch(self, batch: dict[str, torch.Tensor], want: dict[str, Any] | None, keys: tuple[str, ...]) -> None:
+        """The preprocessed request: the named keys plus every camera image of the dump."""
+        if want is None:
+            return
+        for key in (*keys, *(k for k in want if k.startswith("observation.images."))):
+            if key in batch and key in want:
+                self.compare(f"batch.{key}", batch[key], want[key])
+
+    def compare_prefix_kv(self, kv, want: dict[str, Any] | None) -> None:
+        """``kv``: per layer ``(keys, values)``; the dump holds ``layer<i>: {"keys", "values"}``."""
+        if want is None:
+            return
+        for i, (keys, values) in enumerate(kv):
+            self.compare(f"prefix_kv.layer{i}.keys", keys, want[f"layer{i}"]["keys"])
+            self.compare(f"prefix_kv.layer{i}.values", values, want[f"layer{i}"]["values"])

@@ -30,7 +30,7 @@ import torch
 import torch.nn.functional as F  # noqa: N812
 
 from ...base import PolicyEngine
-from ...graph import CaptureSession, GraphRunner
+from ...graph import CaptureSession, GraphRunner, StaticCall
 from ...image_utils import resize_with_pad_center
 from ...registry import register, reject_unsupported_flags
 from ..common import (
@@ -38,9 +38,11 @@ from ..common import (
     OBS_LANGUAGE_ATTENTION_MASK,
     OBS_LANGUAGE_TOKENS,
     OBS_STATE,
+    ErrorReport,
     FileTokenizer,
     SyntheticTokenizer,
     load_normalizer,
+    load_reference_dump,
     load_state_dict,
     load_unnormalizer,
 )
@@ -206,7 +208,7 @@ class PI05Engine(PolicyEngine):
             if not self._graph_runner.precapture([key]):
                 log.warning("graph capture failed; falling back to eager")
                 self.graph_enabled = False
-                self._graph_runner.clear()
+                self._graph_runner.forget()
         if profile:
             try:
                 self.profile()
@@ -252,59 +254,31 @@ class PI05Engine(PolicyEngine):
         report (tybok/policies/pi05/engine.py:740-857): ``batch.*``, ``prefix.{embs,pad_masks,att_masks}``,
         ``prefix_kv.layer<i>.{keys,values}``, ``denoise.v_t`` (zero ``x_t``, t = 0.5), ``chunk`` (zero
         noise, through the graph when enabled) and ``chunk_post``.  ``frame.pt`` and ``chunk.pt`` are
-        required, the other dump files are compared when present.  Dumps are read with
-        ``weights_only=True``: tensors and plain containers only."""
-
-        def load(name: str, required: bool = False):
-            path = os.path.join(reference_dir, name)
-            if not os.path.exists(path):
-                if required:
-                    raise FileNotFoundError(f"reference dump {path} missing")
-                return None
-            return torch.load(path, weights_only=True)
-
-        frame, ref_chunk = load("frame.pt", True), load("chunk.pt", True)
-        ref_batch, ref_prefix, ref_kv, ref_denoise = load("batch.pt"), load("prefix.pt"), load("prefix_kv.pt"), load("denoise.pt")
-        errors: dict[str, float] = {}
-
-        def max_err(name: str, a: torch.Tensor, b: torch.Tensor) -> None:
-            a, b = a.detach().float().cpu(), b.detach().float().cpu()
-            if a.shape != b.shape:
-                raise AssertionError(f"{name}: shape mismatch {tuple(a.shape)} vs {tuple(b.shape)}")
-            diff = (a - b).abs()
-            errors[name + ".max"] = float(diff.max())
-            errors[name + ".mean"] = float(diff.mean())
-
-        batch = self._batch_from_frame(frame)
-        if ref_batch is not None:
-            for key in [OBS_STATE, OBS_LANGUAGE_TOKENS, OBS_LANGUAGE_ATTENTION_MASK] + [k for k in ref_batch if k.startswith("observation.images.")]:
-                if key in batch and key in ref_batch:
-                    max_err(f"batch.{key}", batch[key], ref_batch[key])
+        required, the other dump files are compared when present."""
+        dump = load_reference_dump(reference_dir)
+        report = ErrorReport()
+        cfg, m = self.config, self.model
+        batch = self._batch_from_frame(dump["frame"])
+        report.compare_batch(batch, dump["batch"], (OBS_STATE, OBS_LANGUAGE_TOKENS, OBS_LANGUAGE_ATTENTION_MASK))
         images, img_masks = self.prepare_images(batch)
-        tokens, masks = batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK]
-        m = self.model
-        embs, pads = m.embed_prefix(images, img_masks, tokens, masks)
-        if ref_prefix is not None:
-            max_err("prefix.embs", embs, ref_prefix["embs"])
-            max_err("prefix.pad_masks", pads, ref_prefix["pad_masks"])
-            if "att_masks" in ref_prefix:  # every prefix token attends to every valid one: all zeros
-                max_err("prefix.att_masks", torch.zeros_like(pads), ref_prefix["att_masks"])
-        if ref_kv is not None or ref_denoise is not None:
+        embs, pads = m.embed_prefix(images, img_masks, batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK])
+        if dump["prefix"] is not None:
+            report.compare("prefix.embs", embs, dump["prefix"]["embs"])
+            report.compare("prefix.pad_masks", pads, dump["prefix"]["pad_masks"])
+            if "att_masks" in dump["prefix"]:  # every prefix token attends to every valid one: all zeros
+                report.compare("prefix.att_masks", torch.zeros_like(pads), dump["prefix"]["att_masks"])
+        if dump["prefix_kv"] is not None or dump["denoise"] is not None:
             kv = m.prefill_fused(embs, pads)[0] if m.fused_prefill and embs.shape[0] == 1 else m.prefill(embs, pads)
-            if ref_kv is not None:
-                for i, (k, v) in enumerate(kv):
-                    max_err(f"prefix_kv.layer{i}.keys", k, ref_kv[f"layer{i}"]["keys"])
-                    max_err(f"prefix_kv.layer{i}.values", v, ref_kv[f"layer{i}"]["values"])
-            if ref_denoise is not None:
-                x_t = torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, device=self.device)
-                max_err("denoise.v_t", m.velocity_at(pads, kv, x_t, 0.5), ref_denoise["v_t"])
-        noise = torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, device=self.device)
-        chunk = self._infer(batch, noise)[:, :, : self.config.action_feature_shape[0]]
-        if "chunk" in ref_chunk:
-            max_err("chunk", chunk, ref_chunk["chunk"].reshape(chunk.shape))
+            report.compare_prefix_kv(kv, dump["prefix_kv"])
+            if dump["denoise"] is not None:
+                x_t = torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, device=self.device)
+                report.compare("denoise.v_t", m.velocity_at(pads, kv, x_t, 0.5), dump["denoise"]["v_t"])
+        chunk = self._infer(batch, torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, device=self.device))[:, :, : cfg.action_feature_shape[0]]
+        if "chunk" in dump["chunk"]:
+            report.compare("chunk", chunk, dump["chunk"]["chunk"].reshape(chunk.shape))
         post = self.unnormalizer.unnormalize(chunk, ACTION, "ACTION")
-        max_err("chunk_post", post, ref_chunk["chunk_post"].reshape(post.shape))
-        return errors
+        report.compare("chunk_post", post, dump["chunk"]["chunk_post"].reshape(post.shape))
+        return report
 
     # ------------------------------------------------------------------ request plumbing
     def _batch_from_frame(self, frame: dict[str, Any]) -> dict[str, torch.Tensor]:
@@ -369,41 +343,32 @@ class PI05Engine(PolicyEngine):
         return self.model.sample_actions(images, img_masks, tokens, masks, noise)
 
     # ------------------------------------------------------------------ hipGraph path
-    def _capture_graph(self, key, request=None) -> dict[str, Any]:
-        """One graph of the whole inference core for ``key = (n_cams, lang_len)`` (engine.py:542-606)."""
+    def _capture_graph(self, key, request=None) -> StaticCall:
+        """Record the whole inference core once for ``key = (n_cams, lang_len)`` (the reference records the
+        same unit: tybok/policies/pi05/engine.py:542-606).  Static tensors are named after the keyword
+        arguments of ``PI05Model.sample_actions``."""
+        cfg, dev = self.config, self.device
         n_cams, lang_len = int(key[0]), int(key[1])
-        h, w = self.config.image_resolution
-        dev = self.device
-        static: dict[str, Any] = {
-            "images": [torch.zeros(1, 3, h, w, dtype=torch.float32, device=dev) for _ in range(n_cams)],
-            "img_masks": [torch.ones(1, dtype=torch.bool, device=dev) for _ in range(n_cams)],
-            "tokens": torch.zeros(1, lang_len, dtype=torch.int64, device=dev),
-            "masks": torch.ones(1, lang_len, dtype=torch.bool, device=dev),
-            "noise": torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, dtype=torch.float32, device=dev),
-            "out": torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, dtype=torch.float32, device=dev),
-        }
-        model = self.model
+        height, width = cfg.image_resolution
+        f32 = dict(dtype=torch.float32, device=dev)
+        call = StaticCall(
+            torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, **f32),
+            images=[torch.zeros(1, 3, height, width, **f32) for _ in range(n_cams)],
+            img_masks=[torch.ones(1, dtype=torch.bool, device=dev) for _ in range(n_cams)],
+            tokens=torch.zeros(1, lang_len, dtype=torch.int64, device=dev),
+            masks=torch.ones(1, lang_len, dtype=torch.bool, device=dev),
+            noise=torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, **f32),
+        )
+        log.info(f"capturing one graph for {n_cams} camera(s), lang={lang_len}, steps={cfg.num_steps}")
+        return call.record(self._sess, self.model.sample_actions)
 
-        def core() -> None:
-            static["out"].copy_(model.sample_actions(static["images"], static["img_masks"], static["tokens"], static["masks"], static["noise"]))
-
-        log.info(f"capturing one graph for {n_cams} camera(s), lang={lang_len}, steps={self.config.num_steps}")
-        graph = self._sess.prime_and_capture(core)
-        self._sess.sync()
-        return {"graph": graph, "statics": static}
-
-    def _run_graph(self, entry, images, img_masks, tokens, masks, noise) -> torch.Tensor:
-        static = entry["statics"]
+    def _run_graph(self, call: StaticCall, images, img_masks, tokens, masks, noise) -> torch.Tensor:
+        """The request's tensors go into the static ones on the input stream, then the replay."""
         with self._graph_runner.copy_inputs():
-            for i, (img, mask) in enumerate(zip(images, img_masks)):
-                static["images"][i].copy_(img)
-                static["img_masks"][i].copy_(mask)
-            static["tokens"].copy_(tokens)
-            static["masks"].copy_(masks)
+            call.store(images=images, img_masks=img_masks, tokens=tokens, masks=masks)
             if noise is None:
-                self._sample_noise(out=static["noise"])
+                self._sample_noise(out=call.inputs["noise"])  # drawn outside the graph, from the engine's generator
             else:
-                static["noise"].copy_(noise)
+                call.store(noise=noise)
         self._graph_runner.wait_inputs()
-        entry["graph"].replay()
-        return static["out"].clone()
+        return call.replay()

@@ -28,7 +28,7 @@ import torch
 import torch.nn.functional as F  # noqa: N812
 
 from ...base import PolicyEngine
-from ...graph import CaptureSession, GraphRunner, camera_counts
+from ...graph import CaptureSession, GraphRunner, StaticCall, camera_counts
 from ...image_utils import resize_with_pad
 from ...registry import register
 from ..common import (
@@ -36,9 +36,11 @@ from ..common import (
     OBS_LANGUAGE_ATTENTION_MASK,
     OBS_LANGUAGE_TOKENS,
     OBS_STATE,
+    ErrorReport,
     FileTokenizer,
     SyntheticTokenizer,
     load_normalizer,
+    load_reference_dump,
     load_state_dict,
     load_unnormalizer,
 )
@@ -177,7 +179,7 @@ class SmolVLAEngine(PolicyEngine):
             if not self._graph_runner.precapture([(n,) for n in counts]):
                 log.warning("graph capture failed for all requested camera counts; falling back to eager mode")
                 self.graph_enabled = False
-                self._graph_runner.clear()
+                self._graph_runner.forget()
         if profile:
             try:
                 self.profile()
@@ -216,66 +218,34 @@ class SmolVLAEngine(PolicyEngine):
         report (tybok/policies/smolvla/engine.py:655-752): ``batch.*``, ``prefix.{embs,pad_masks,
         att_masks}``, ``prefix_kv.layer<i>.{keys,values}``, ``denoise.v_t`` (zero ``x_t``, t = 0.5),
         ``chunk`` (zero noise, through the graph when enabled) and ``chunk_post``.  ``frame.pt`` and
-        ``chunk.pt`` are required, the other dump files are compared when present.  Dumps are read
-        with ``weights_only=True``: tensors and plain containers only."""
-
-        def load(name: str, required: bool = False):
-            path = os.path.join(reference_dir, name)
-            if not os.path.exists(path):
-                if required:
-                    raise FileNotFoundError(f"reference dump {path} missing")
-                return None
-            return torch.load(path, weights_only=True)
-
-        frame, ref_chunk = load("frame.pt", True), load("chunk.pt", True)
-        ref_batch, ref_prefix, ref_kv, ref_denoise = load("batch.pt"), load("prefix.pt"), load("prefix_kv.pt"), load("denoise.pt")
-        errors: dict[str, float] = {}
-
-        def max_err(name: str, a: torch.Tensor, b: torch.Tensor) -> None:
-            a, b = a.detach().float().cpu(), b.detach().float().cpu()
-            if a.shape != b.shape:
-                raise AssertionError(f"{name}: shape mismatch {tuple(a.shape)} vs {tuple(b.shape)}")
-            diff = (a - b).abs()
-            errors[name + ".max"] = float(diff.max())
-            errors[name + ".mean"] = float(diff.mean())
-
-        batch = self._batch_from_frame(frame)
-        if ref_batch is not None:
-            for key in [OBS_STATE, OBS_LANGUAGE_TOKENS, OBS_LANGUAGE_ATTENTION_MASK] + [k for k in ref_batch if k.startswith("observation.images.")]:
-                if key in batch and key in ref_batch:
-                    max_err(f"batch.{key}", batch[key], ref_batch[key])
+        ``chunk.pt`` are required, the other dump files are compared when present."""
+        dump = load_reference_dump(reference_dir)
+        report = ErrorReport()
+        cfg, m = self.config, self.model
+        batch = self._batch_from_frame(dump["frame"])
+        report.compare_batch(batch, dump["batch"], (OBS_STATE, OBS_LANGUAGE_TOKENS, OBS_LANGUAGE_ATTENTION_MASK))
         images, img_masks = self.prepare_images(batch)
-        state = self.prepare_state(batch)
-        tokens, lang_masks = batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK]
-        m = self.model
-        embs, pads, att = m.embed_prefix(images, img_masks, tokens, lang_masks, state)
-        if ref_prefix is not None:
-            max_err("prefix.embs", embs, ref_prefix["embs"])
-            max_err("prefix.pad_masks", pads, ref_prefix["pad_masks"])
-            max_err("prefix.att_masks", att, ref_prefix["att_masks"])
-        if ref_kv is not None or ref_denoise is not None:
-            if m.fused_prefill and embs.shape[0] == 1:
-                keys, values, _ = m.prefill_fused(embs, pads, att)
-            else:
-                keys, values = m.prefill(embs, pads, att)
-            if ref_kv is not None:
-                for i in range(self.config.num_vlm_layers):
-                    max_err(f"prefix_kv.layer{i}.keys", keys[i], ref_kv[f"layer{i}"]["keys"])
-                    max_err(f"prefix_kv.layer{i}.values", values[i], ref_kv[f"layer{i}"]["values"])
-            if ref_denoise is not None:
+        embs, pads, att = m.embed_prefix(images, img_masks, batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK], self.prepare_state(batch))
+        if dump["prefix"] is not None:
+            for name, got in (("embs", embs), ("pad_masks", pads), ("att_masks", att)):
+                report.compare(f"prefix.{name}", got, dump["prefix"][name])
+        if dump["prefix_kv"] is not None or dump["denoise"] is not None:
+            fused = m.fused_prefill and embs.shape[0] == 1
+            keys, values = m.prefill_fused(embs, pads, att)[:2] if fused else m.prefill(embs, pads, att)
+            report.compare_prefix_kv(list(zip(keys, values))[: cfg.num_vlm_layers], dump["prefix_kv"])
+            if dump["denoise"] is not None:
                 from .model import sinusoidal_time_embedding
 
-                x_t = torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, device=self.device)
-                te = sinusoidal_time_embedding(torch.tensor([0.5]), self.config.expert_hidden_size, self.config.min_period, self.config.max_period)
+                x_t = torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, device=self.device)
+                te = sinusoidal_time_embedding(torch.tensor([0.5]), cfg.expert_hidden_size, cfg.min_period, cfg.max_period)
                 v_t = m.denoise_step(pads, keys, values, m.expert_prefix_kv(keys, values), x_t, te.float().to(self.device))
-                max_err("denoise.v_t", v_t, ref_denoise["v_t"])
-        noise = torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, device=self.device)
-        chunk = self._infer(batch, noise)[:, :, : self.config.action_feature_shape[0]]
-        if "chunk" in ref_chunk:
-            max_err("chunk", chunk, ref_chunk["chunk"].reshape(chunk.shape))
+                report.compare("denoise.v_t", v_t, dump["denoise"]["v_t"])
+        chunk = self._infer(batch, torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, device=self.device))[:, :, : cfg.action_feature_shape[0]]
+        if "chunk" in dump["chunk"]:
+            report.compare("chunk", chunk, dump["chunk"]["chunk"].reshape(chunk.shape))
         post = self.unnormalizer.unnormalize(chunk, ACTION, "ACTION")
-        max_err("chunk_post", post, ref_chunk["chunk_post"].reshape(post.shape))
-        return errors
+        report.compare("chunk_post", post, dump["chunk"]["chunk_post"].reshape(post.shape))
+        return report
 
     # ------------------------------------------------------------------ request plumbing
     def _resolve_alias(self, camera_alias: dict[str, str] | None) -> dict[str, str]:
@@ -367,48 +337,32 @@ class SmolVLAEngine(PolicyEngine):
     def _prefix_len_for(self, n_cams: int) -> int:
         return n_cams * self.config.vlm_config.image_seq_len + self.config.tokenizer_max_length + 1
 
-    def _capture_graph(self, key, request=None) -> dict[str, Any]:
-        """One graph of the whole inference core for ``key = (n_cams,)`` (engine.py:408-472)."""
-        n_cams = int(key[0])
-        w, h = self.config.resize_imgs_with_padding
-        dev = self.device
-        static: dict[str, Any] = {
-            "images": [torch.zeros(1, 3, h, w, dtype=torch.float32, device=dev) for _ in range(n_cams)],
-            "img_masks": [torch.ones(1, dtype=torch.bool, device=dev) for _ in range(n_cams)],
-            "lang_tokens": torch.zeros(1, self.config.tokenizer_max_length, dtype=torch.long, device=dev),
-            "lang_masks": torch.ones(1, self.config.tokenizer_max_length, dtype=torch.bool, device=dev),
-            "state": torch.zeros(1, self.config.max_state_dim, dtype=torch.float32, device=dev),
-            "noise": torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, dtype=torch.float32, device=dev),
-            "out": torch.zeros(1, self.config.chunk_size, self.config.max_action_dim, dtype=torch.float32, device=dev),
-        }
-        model = self.model
+    def _capture_graph(self, key, request=None) -> StaticCall:
+        """Record the whole inference core once for ``key = (n_cams,)`` (the reference records the same
+        unit: tybok/policies/smolvla/engine.py:408-472).  Static tensors are named after the keyword
+        arguments of ``SmolVLAModel.sample_actions``."""
+        cfg, dev, n_cams = self.config, self.device, int(key[0])
+        width, height = cfg.resize_imgs_with_padding
+        f32 = dict(dtype=torch.float32, device=dev)
+        call = StaticCall(
+            torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, **f32),
+            images=[torch.zeros(1, 3, height, width, **f32) for _ in range(n_cams)],
+            img_masks=[torch.ones(1, dtype=torch.bool, device=dev) for _ in range(n_cams)],
+            lang_tokens=torch.zeros(1, cfg.tokenizer_max_length, dtype=torch.long, device=dev),
+            lang_masks=torch.ones(1, cfg.tokenizer_max_length, dtype=torch.bool, device=dev),
+            state=torch.zeros(1, cfg.max_state_dim, **f32),
+            noise=torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, **f32),
+        )
+        log.info(f"capturing one graph for {n_cams} camera(s) (prefix_len={self._prefix_len_for(n_cams)}, steps={cfg.num_steps})")
+        return call.record(self._sess, self.model.sample_actions)
 
-        def core() -> None:
-            static["out"].copy_(
-                model.sample_actions(
-                    static["images"], static["img_masks"], static["lang_tokens"], static["lang_masks"], static["state"], static["noise"]
-                )
-            )
-
-        log.info(f"capturing one graph for {n_cams} camera(s) (prefix_len={self._prefix_len_for(n_cams)}, steps={self.config.num_steps})")
-        graph = self._sess.prime_and_capture(core)
-        self._sess.sync()
-        return {"graph": graph, "statics": static}
-
-    def _run_graph(self, entry, images, img_masks, tokens, lang_masks, state, noise) -> torch.Tensor:
-        """Copy the request into the static buffers (copy stream), replay, return a copy of the output."""
-        static = entry["statics"]
+    def _run_graph(self, call: StaticCall, images, img_masks, tokens, lang_masks, state, noise) -> torch.Tensor:
+        """The request's tensors go into the static ones on the input stream, then the replay."""
         with self._graph_runner.copy_inputs():
-            for i, (img, mask) in enumerate(zip(images, img_masks)):
-                static["images"][i].copy_(img)
-                static["img_masks"][i].copy_(mask)
-            static["lang_tokens"].copy_(tokens)
-            static["lang_masks"].copy_(lang_masks)
-            static["state"].copy_(state)
+            call.store(images=images, img_masks=img_masks, lang_tokens=tokens, lang_masks=lang_masks, state=state)
             if noise is None:
-                self._sample_noise(out=static["noise"])  # noise is drawn outside the graph
+                self._sample_noise(out=call.inputs["noise"])  # drawn outside the graph, from the engine's generator
             else:
-                static["noise"].copy_(noise)
+                call.store(noise=noise)
         self._graph_runner.wait_inputs()
-        entry["graph"].replay()
-        return static["out"].clone()
+        return call.replay()
