@@ -12,11 +12,14 @@ from __future__ import annotations
 import abc
 import logging
 import time
+from collections import deque
 from collections.abc import Mapping, Sequence
 from typing import Any
 
 import numpy as np
 import torch
+
+from .graph import CaptureSession, GraphRunner
 
 log = logging.getLogger("tybok.engine")
 
@@ -149,3 +152,64 @@ class PolicyEngine(abc.ABC):
     def _profile_phases(self, iters: int = 5, warmup: int = 3, cameras: int | None = None, seed: int = 0) -> dict[str, float]:
         """Per-phase timings a backend may add to :meth:`profile`'s report."""
         return {}
+
+
+class ChunkRuntime:
+    """What the two flow-matching backends share once their model is built: the seeded noise source,
+    the queue ``select_action`` drains, recorded shapes, and the order of the start-up steps.  A backend
+    provides ``_infer(batch, noise)``, ``_batch_from_frame(frame)``, ``_capture_graph(key, request)``, an
+    ``unnormalizer`` and a ``config`` with ``chunk_size``, ``n_action_steps``, ``max_action_dim`` and
+    ``action_feature_shape``."""
+
+    def _init_sampling(self, seed: int | None) -> None:
+        self.seed = seed
+        self._noise_gen = None if seed is None else torch.Generator(device=self.device).manual_seed(int(seed))
+        self._action_queue: deque[torch.Tensor] = deque(maxlen=self.config.n_action_steps)
+
+    def _init_graphs(self, graph: bool, label: str, logger: logging.Logger) -> None:
+        self.graph_requested = bool(graph)
+        self.graph_enabled = self.graph_requested and str(self.device).startswith("cuda")
+        self._sess = CaptureSession(self.device)
+        self._graph_runner = GraphRunner(self._capture_graph, self.device, label=label, logger=logger)
+
+    def _start(self, *, warmup: bool, graph_keys: Sequence[Any], profile: bool, logger: logging.Logger) -> None:
+        """Start-up in the reference's order: one warm-up inference, the shapes named on the command
+        line recorded (none recordable: back to eager, loudly), an optional latency report."""
+        if warmup:
+            self._warmup()
+        if self.graph_enabled and not self._graph_runner.precapture(list(graph_keys)):
+            logger.warning("no requested shape could be recorded as a graph; running eagerly")
+            self.graph_enabled = False
+            self._graph_runner.forget()
+        if profile:
+            try:
+                self.profile()
+            except Exception as exc:  # noqa: BLE001 - a diagnostic must not stop the server from starting
+                logger.warning("profile failed: %s", exc)
+
+    # ------------------------------------------------------------------ noise and outputs
+    def _sample_noise(self, out: torch.Tensor | None = None) -> torch.Tensor:
+        shape = (1, self.config.chunk_size, self.config.max_action_dim)
+        return torch.normal(0.0, 1.0, size=shape, dtype=torch.float32, device=self.device, generator=self._noise_gen, out=out)
+
+    def _prepare_noise(self, noise: torch.Tensor | None) -> torch.Tensor | None:
+        """A caller's noise on the device in fp32, zero-padded to the model's action width."""
+        if noise is None:
+            return None
+        noise = noise.to(self.device, dtype=torch.float32)
+        missing = self.config.max_action_dim - noise.shape[-1]
+        return torch.nn.functional.pad(noise, (0, missing)) if missing else noise
+
+    def _robot_actions(self, frame: dict[str, Any], noise: torch.Tensor | None) -> torch.Tensor:
+        """Normalised actions ``[1, chunk, action_dim]`` of one request (the padded columns dropped)."""
+        actions = self._infer(self._batch_from_frame(frame), self._prepare_noise(noise))
+        return actions[:, :, : self.config.action_feature_shape[0]]
+
+    def _to_robot_units(self, actions: torch.Tensor) -> np.ndarray:
+        return self.unnormalizer.unnormalize(actions, "action", "ACTION").cpu().numpy()[0]
+
+    def _next_queued_action(self, frame: dict[str, Any], noise: torch.Tensor | None) -> np.ndarray:
+        """``select_action``: infer a chunk only when the queue of the previous one is empty."""
+        if not self._action_queue:
+            self._action_queue.extend(self._robot_actions(frame, noise).transpose(0, 1)[: self.config.n_action_steps])
+        return self._to_robot_units(self._action_queue.popleft())

@@ -22,15 +22,13 @@ from __future__ import annotations
 
 import logging
 import os
-from collections import deque
 from typing import Any
 
 import numpy as np
 import torch
-import torch.nn.functional as F  # noqa: N812
 
-from ...base import PolicyEngine
-from ...graph import CaptureSession, GraphRunner, StaticCall
+from ...base import ChunkRuntime, PolicyEngine
+from ...graph import StaticCall
 from ...image_utils import resize_with_pad_center
 from ...registry import register, reject_unsupported_flags
 from ..common import (
@@ -70,7 +68,7 @@ def build_prompt(task: str, normalized_state: torch.Tensor) -> str:
 
 
 @register("pi05")
-class PI05Engine(PolicyEngine):
+class PI05Engine(ChunkRuntime, PolicyEngine):
     _UNSUPPORTED_FLAGS = {
         "tl_llm_fused_attn": False,
         "tl_vit_oproj": False,
@@ -189,31 +187,12 @@ class PI05Engine(PolicyEngine):
                 raise ValueError(f"camera_alias target {dst!r} is not an expected image feature")
             self.camera_alias[s] = d
 
-        self.seed = seed
-        self._noise_gen: torch.Generator | None = None
-        if seed is not None:
-            self._noise_gen = torch.Generator(device=self.device).manual_seed(int(seed))
-        self._action_queue: deque[torch.Tensor] = deque(maxlen=self.config.n_action_steps)
+        self._init_sampling(seed)
         self.rtc_processor = None
-
-        self.graph_requested = bool(graph)
-        self.graph_enabled = self.graph_requested and str(self.device).startswith("cuda")
+        self._init_graphs(graph, "pi05 graph", log)
         self.overlap = False  # prefill x step-0 two-stream overlap is not implemented; accepted, inert
-        self._sess = CaptureSession(self.device)
-        self._graph_runner = GraphRunner(self._capture_graph, self.device, label="pi05 graph", logger=log)
-        if warmup:
-            self._warmup()
-        if self.graph_enabled:
-            key = (len(self.config.image_features), self.config.tokenizer_max_length)
-            if not self._graph_runner.precapture([key]):
-                log.warning("graph capture failed; falling back to eager")
-                self.graph_enabled = False
-                self._graph_runner.forget()
-        if profile:
-            try:
-                self.profile()
-            except Exception as e:  # noqa: BLE001 - never fail startup on a diagnostic
-                log.warning(f"profile failed: {e}")
+        key = (len(self.config.image_features), self.config.tokenizer_max_length)
+        self._start(warmup=warmup, graph_keys=[key], profile=profile, logger=log)
 
     # ------------------------------------------------------------------ API
     def supports_rtc(self) -> bool:
@@ -234,19 +213,13 @@ class PI05Engine(PolicyEngine):
     def predict_action_chunk(self, frame: dict[str, Any], noise: torch.Tensor | None = None, *, return_normalized: bool = False, **rtc: Any) -> Any:
         if any(v is not None for v in rtc.values()):
             raise NotImplementedError("Real-Time Chunking guidance arguments are not supported by this backend")
-        batch = self._batch_from_frame(frame)
-        actions = self._infer(batch, self._prepare_noise(noise))[:, :, : self.config.action_feature_shape[0]]
-        chunk = self.unnormalizer.unnormalize(actions, ACTION, "ACTION").cpu().numpy()[0]
+        actions = self._robot_actions(frame, noise)
+        chunk = self._to_robot_units(actions)
         return (chunk, actions.cpu().numpy()[0]) if return_normalized else chunk
 
     @torch.inference_mode()
     def select_action(self, frame: dict[str, Any], noise: torch.Tensor | None = None) -> np.ndarray:
-        if not self._action_queue:
-            batch = self._batch_from_frame(frame)
-            actions = self._infer(batch, self._prepare_noise(noise))[:, : self.config.n_action_steps, : self.config.action_feature_shape[0]]
-            self._action_queue.extend(actions.transpose(0, 1))
-        action = self._action_queue.popleft()
-        return self.unnormalizer.unnormalize(action, ACTION, "ACTION").cpu().numpy()[0]
+        return self._next_queued_action(frame, noise)
 
     @torch.inference_mode()
     def validate(self, reference_dir: str) -> dict[str, float]:
@@ -304,14 +277,6 @@ class PI05Engine(PolicyEngine):
             batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK] = self.tokenizer.encode_task(prompt)
         return {k: v.to(self.device) for k, v in batch.items()}
 
-    def _prepare_noise(self, noise: torch.Tensor | None) -> torch.Tensor | None:
-        if noise is None:
-            return None
-        noise = noise.to(self.device, dtype=torch.float32)
-        if noise.shape[-1] != self.config.max_action_dim:
-            noise = F.pad(noise, (0, self.config.max_action_dim - noise.shape[-1]))
-        return noise
-
     def prepare_images(self, batch: dict[str, torch.Tensor]):
         """Centre-padded resize to 224x224, [0,1] -> [-1,1]; missing slots become -1 images with a zero mask (policy.py:170-234)."""
         h, w = self.config.image_resolution
@@ -327,10 +292,6 @@ class PI05Engine(PolicyEngine):
             images.append(torch.ones_like(images[-1]) * -1)
             masks.append(torch.zeros_like(masks[-1]))
         return images, masks
-
-    def _sample_noise(self, out: torch.Tensor | None = None) -> torch.Tensor:
-        shape = (1, self.config.chunk_size, self.config.max_action_dim)
-        return torch.normal(0.0, 1.0, size=shape, dtype=torch.float32, device=self.device, generator=self._noise_gen, out=out)
 
     def _infer(self, batch: dict[str, torch.Tensor], noise: torch.Tensor | None) -> torch.Tensor:
         images, img_masks = self.prepare_images(batch)

@@ -20,15 +20,14 @@ from __future__ import annotations
 
 import logging
 import os
-from collections import deque
 from typing import Any
 
 import numpy as np
 import torch
 import torch.nn.functional as F  # noqa: N812
 
-from ...base import PolicyEngine
-from ...graph import CaptureSession, GraphRunner, StaticCall, camera_counts
+from ...base import ChunkRuntime, PolicyEngine
+from ...graph import StaticCall, camera_counts
 from ...image_utils import resize_with_pad
 from ...registry import register
 from ..common import (
@@ -52,7 +51,7 @@ log = logging.getLogger("tybok.smolvla")
 
 
 @register("smolvla")
-class SmolVLAEngine(PolicyEngine):
+class SmolVLAEngine(ChunkRuntime, PolicyEngine):
     # flags owned by other backends or not implemented here: inert default -> accepted, else rejected
     _UNSUPPORTED_FLAGS = {
         "tl_fused_vit": False,
@@ -158,33 +157,13 @@ class SmolVLAEngine(PolicyEngine):
         self.unnormalizer = load_unnormalizer(checkpoint_dir, norm_map)
         self.camera_alias = self._resolve_alias(camera_alias)
 
-        self.seed = seed
-        self._noise_gen: torch.Generator | None = None
-        if seed is not None:
-            self._noise_gen = torch.Generator(device=self.device).manual_seed(int(seed))
-        self._action_queue: deque[torch.Tensor] = deque(maxlen=self.config.n_action_steps)
-
-        self.graph_requested = bool(graph)
-        self.graph_enabled = self.graph_requested and str(self.device).startswith("cuda")
+        self._init_sampling(seed)
+        self._init_graphs(graph, "smolvla graph", log)
         self.overlap = self.model.overlap  # step 0 of the Euler loop hidden inside the prefill (two streams)
-        self._sess = CaptureSession(self.device)
-        self._graph_runner = GraphRunner(self._capture_graph, self.device, label="smolvla graph", logger=log)
         self._graph_fallback_warned = False
-
-        if warmup:
-            self._warmup()
-        if self.graph_enabled:
-            max_cams = len(self.config.image_features)
-            counts = camera_counts(graph_cameras, default=max_cams, max_images=max_cams)
-            if not self._graph_runner.precapture([(n,) for n in counts]):
-                log.warning("graph capture failed for all requested camera counts; falling back to eager mode")
-                self.graph_enabled = False
-                self._graph_runner.forget()
-        if profile:
-            try:
-                self.profile()
-            except Exception as e:  # noqa: BLE001 - never fail startup on a diagnostic
-                log.warning(f"profile failed: {e}")
+        cameras = len(self.config.image_features)
+        keys = [(n,) for n in camera_counts(graph_cameras, default=cameras, max_images=cameras)]
+        self._start(warmup=warmup, graph_keys=keys, profile=profile, logger=log)
 
     # ------------------------------------------------------------------ API
     def describe(self) -> dict[str, Any]:
@@ -198,19 +177,11 @@ class SmolVLAEngine(PolicyEngine):
 
     @torch.inference_mode()
     def predict_action_chunk(self, frame: dict[str, Any], noise: torch.Tensor | None = None) -> np.ndarray:
-        batch = self._batch_from_frame(frame)
-        actions = self._infer(batch, self._prepare_noise(noise))
-        actions = actions[:, :, : self.config.action_feature_shape[0]]
-        return self.unnormalizer.unnormalize(actions, ACTION, "ACTION").cpu().numpy()[0]
+        return self._to_robot_units(self._robot_actions(frame, noise))
 
     @torch.inference_mode()
     def select_action(self, frame: dict[str, Any], noise: torch.Tensor | None = None) -> np.ndarray:
-        if not self._action_queue:
-            batch = self._batch_from_frame(frame)
-            actions = self._infer(batch, self._prepare_noise(noise))[:, :, : self.config.action_feature_shape[0]]
-            self._action_queue.extend(actions.transpose(0, 1)[: self.config.n_action_steps])
-        action = self._action_queue.popleft()
-        return self.unnormalizer.unnormalize(action, ACTION, "ACTION").cpu().numpy()[0]
+        return self._next_queued_action(frame, noise)
 
     @torch.inference_mode()
     def validate(self, reference_dir: str) -> dict[str, float]:
@@ -280,14 +251,6 @@ class SmolVLAEngine(PolicyEngine):
             batch[OBS_STATE] = self.normalizer.normalize(batch[OBS_STATE], OBS_STATE, "STATE")
         return batch
 
-    def _prepare_noise(self, noise: torch.Tensor | None) -> torch.Tensor | None:
-        if noise is None:
-            return None
-        noise = noise.to(self.device, dtype=torch.float32)
-        if noise.shape[-1] != self.config.max_action_dim:
-            noise = F.pad(noise, (0, self.config.max_action_dim - noise.shape[-1]))
-        return noise
-
     def prepare_images(self, batch: dict[str, torch.Tensor]):
         """Resize (left/top pad) to the model resolution, [0,1] -> [-1,1]; masks all true (policy.py:117-163)."""
         w, h = self.config.resize_imgs_with_padding
@@ -310,10 +273,6 @@ class SmolVLAEngine(PolicyEngine):
         if state.shape[-1] < self.config.max_state_dim:
             state = F.pad(state, (0, self.config.max_state_dim - state.shape[-1]))
         return state
-
-    def _sample_noise(self, out: torch.Tensor | None = None) -> torch.Tensor:
-        shape = (1, self.config.chunk_size, self.config.max_action_dim)
-        return torch.normal(0.0, 1.0, size=shape, dtype=torch.float32, device=self.device, generator=self._noise_gen, out=out)
 
     def _infer(self, batch: dict[str, torch.Tensor], noise: torch.Tensor | None) -> torch.Tensor:
         images, img_masks = self.prepare_images(batch)
