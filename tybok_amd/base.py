@@ -211,5 +211,6 @@ class ChunkRuntime:
     def _next_queued_action(self, frame: dict[str, Any], noise: torch.Tensor | None) -> np.ndarray:
         """``select_action``: infer a chunk only when the queue of the previous one is empty."""
         if not self._action_queue:
-            self._action_queue.extend(self._robot_actions(frame, noise).transpose(0, 1)[: self.config.n_action_steps])
+            # (the queue outlives this request: it gets its own copy, not a view of a graph's static output)
+            self._action_queue.extend(self._robot_actions(frame, noise).transpose(0, 1)[: self.config.n_action_steps].clone())
         return self._to_robot_units(self._action_queue.popleft())

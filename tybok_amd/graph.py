@@ -89,12 +89,26 @@ class StaticCall:
             else:
                 slot.copy_(value)
 
-    def replay(self) -> torch.Tensor:
-        """Run the graph; the result is copied out so the next replay cannot overwrite it."""
+    def store_owned(self, **values: Any) -> None:
+        """:meth:`store` for tensors the backend owns and never changes in place (cached token ids, all-true
+        masks): a value that is the very object stored last time is not copied again."""
+        if not hasattr(self, "_last_owned"):
+            self._last_owned: dict[str, Any] = {}
+        for name, value in values.items():
+            objects = tuple(value) if isinstance(value, (list, tuple)) else (value,)
+            last = self._last_owned.get(name, ())
+            if len(last) != len(objects) or any(a is not b for a, b in zip(last, objects)):
+                self.store(**{name: value})
+                self._last_owned[name] = objects
+
+    def replay(self, *, copy: bool = True) -> torch.Tensor:
+        """Run the graph.  By default the result is copied out so that the next replay cannot overwrite
+        it; ``copy=False`` returns the static tensor itself, for callers that finish with it (or copy it)
+        before they replay again."""
         if self.graph is None:
             raise RuntimeError("replay() before record()")
         self.graph.replay()
-        return self.output.clone()
+        return self.output.clone() if copy else self.output
 
 
 class GraphRunner:

@@ -158,6 +158,8 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
         self.camera_alias = self._resolve_alias(camera_alias)
 
         self._init_sampling(seed)
+        self._token_cache: dict[str, tuple[torch.Tensor, torch.Tensor]] = {}
+        self._mask_cache: dict[tuple[int, bool], torch.Tensor] = {}
         self._init_graphs(graph, "smolvla graph", log)
         self.overlap = self.model.overlap  # step 0 of the Euler loop hidden inside the prefill (two streams)
         self._graph_fallback_warned = False
@@ -245,28 +247,59 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
             task = frame.get("task", "")
             if isinstance(task, str) and not task.endswith("\n"):
                 task = f"{task}\n"
-            batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK] = self.tokenizer.encode_task(task)
+            batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK] = self._task_tokens(task)
         batch = {k: v.to(self.device) for k, v in batch.items()}
         if OBS_STATE in batch:
             batch[OBS_STATE] = self.normalizer.normalize(batch[OBS_STATE], OBS_STATE, "STATE")
         return batch
 
-    def prepare_images(self, batch: dict[str, torch.Tensor]):
-        """Resize (left/top pad) to the model resolution, [0,1] -> [-1,1]; masks all true (policy.py:117-163)."""
+    def _task_tokens(self, task: str) -> tuple[torch.Tensor, torch.Tensor]:
+        """Token ids and mask of a task string, on the device; the last few tasks are kept (a robot
+        repeats its task every request), so the tokenizer and two host-to-device copies run once per task."""
+        hit = self._token_cache.get(task)
+        if hit is None:
+            ids, mask = self.tokenizer.encode_task(task)
+            hit = (ids.to(self.device), mask.to(self.device))
+            if len(self._token_cache) >= 8:
+                self._token_cache.pop(next(iter(self._token_cache)))
+            self._token_cache[task] = hit
+        return hit
+
+    def _mask(self, batch_size: int, value: bool) -> torch.Tensor:
+        """A cached all-true / all-false image mask (never written to)."""
+        key = (batch_size, value)
+        if key not in self._mask_cache:
+            self._mask_cache[key] = torch.full((batch_size,), value, dtype=torch.bool, device=self.device)
+        return self._mask_cache[key]
+
+    def prepare_images01(self, batch: dict[str, torch.Tensor]):
+        """Camera images resized (left/top pad) to the model resolution, still in [0, 1], and their
+        masks; configured cameras the frame lacks become black-after-scaling images with a false mask,
+        up to ``empty_cameras`` of them (policy.py:117-163)."""
         w, h = self.config.resize_imgs_with_padding
         present = [k for k in self.config.image_features if k in batch]
         if not present:
             raise ValueError(f"All image features are missing from the batch (expected {self.config.image_features})")
-        images, masks = [], []
-        for key in present:
-            img = resize_with_pad(batch[key], h, w, pad_value=0) * 2.0 - 1.0
-            images.append(img)
-            masks.append(torch.ones(img.shape[0], dtype=torch.bool, device=img.device))
-        missing = [k for k in self.config.image_features if k not in batch]
-        for _ in range(min(len(missing), self.config.empty_cameras)):
-            images.append(torch.ones_like(images[-1]) * -1)
-            masks.append(torch.zeros_like(masks[-1]))
+        images = [resize_with_pad(batch[key], h, w, pad_value=0) for key in present]
+        masks = [self._mask(img.shape[0], True) for img in images]
+        missing = len(self.config.image_features) - len(present)
+        for _ in range(min(missing, self.config.empty_cameras)):
+            images.append(torch.zeros_like(images[-1]))  # 0 * 2 - 1 = -1: the reference's filler value
+            masks.append(self._mask(images[-1].shape[0], False))
         return images, masks
+
+    @staticmethod
+    def _to_model_range(images01):
+        return [img * 2.0 - 1.0 for img in images01]
+
+    def prepare_images(self, batch: dict[str, torch.Tensor]):
+        """:meth:`prepare_images01` scaled to the tower's [-1, 1] input range."""
+        images01, masks = self.prepare_images01(batch)
+        return self._to_model_range(images01), masks
+
+    def _core(self, images01, img_masks, lang_tokens, lang_masks, state, noise) -> torch.Tensor:
+        """The unit a graph records: input scaling and the whole model."""
+        return self.model.sample_actions(self._to_model_range(images01), img_masks, lang_tokens, lang_masks, state, noise)
 
     def prepare_state(self, batch: dict[str, torch.Tensor]) -> torch.Tensor:
         state = batch[OBS_STATE]
@@ -275,7 +308,7 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
         return state
 
     def _infer(self, batch: dict[str, torch.Tensor], noise: torch.Tensor | None) -> torch.Tensor:
-        images, img_masks = self.prepare_images(batch)
+        images, img_masks = self.prepare_images01(batch)
         state = self.prepare_state(batch)
         tokens, lang_masks = batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK]
         if self.graph_enabled and self._graph_runner:
@@ -290,7 +323,7 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
                 return self._run_graph(entry, images, img_masks, tokens, lang_masks, state, noise)
         if noise is None:
             noise = self._sample_noise()
-        return self.model.sample_actions(images, img_masks, tokens, lang_masks, state, noise)
+        return self._core(images, img_masks, tokens, lang_masks, state, noise)
 
     # ------------------------------------------------------------------ hipGraph path
     def _prefix_len_for(self, n_cams: int) -> int:
@@ -305,7 +338,7 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
         f32 = dict(dtype=torch.float32, device=dev)
         call = StaticCall(
             torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, **f32),
-            images=[torch.zeros(1, 3, height, width, **f32) for _ in range(n_cams)],
+            images01=[torch.zeros(1, 3, height, width, **f32) for _ in range(n_cams)],
             img_masks=[torch.ones(1, dtype=torch.bool, device=dev) for _ in range(n_cams)],
             lang_tokens=torch.zeros(1, cfg.tokenizer_max_length, dtype=torch.long, device=dev),
             lang_masks=torch.ones(1, cfg.tokenizer_max_length, dtype=torch.bool, device=dev),
@@ -313,15 +346,19 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
             noise=torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, **f32),
         )
         log.info(f"capturing one graph for {n_cams} camera(s) (prefix_len={self._prefix_len_for(n_cams)}, steps={cfg.num_steps})")
-        return call.record(self._sess, self.model.sample_actions)
+        return call.record(self._sess, self._core)
 
-    def _run_graph(self, call: StaticCall, images, img_masks, tokens, lang_masks, state, noise) -> torch.Tensor:
-        """The request's tensors go into the static ones on the input stream, then the replay."""
+    def _run_graph(self, call: StaticCall, images01, img_masks, tokens, lang_masks, state, noise) -> torch.Tensor:
+        """The request's tensors go into the static ones on the input stream (one copy per camera and
+        one for the state; token ids and masks only when they are not the cached objects stored last
+        time), then the replay.  Returns the graph's static output: every caller is done with it, or has
+        copied it, before the next request replays."""
         with self._graph_runner.copy_inputs():
-            call.store(images=images, img_masks=img_masks, lang_tokens=tokens, lang_masks=lang_masks, state=state)
+            call.store(images01=images01, state=state)
+            call.store_owned(lang_tokens=tokens, lang_masks=lang_masks, img_masks=img_masks)
             if noise is None:
                 self._sample_noise(out=call.inputs["noise"])  # drawn outside the graph, from the engine's generator
             else:
                 call.store(noise=noise)
         self._graph_runner.wait_inputs()
-        return call.replay()
+        return call.replay(copy=False)
