@@ -4,8 +4,8 @@ Behaviour follows the reference's helper of the same name (tybok/graph.py:60-251
 is looked up by a key whose first element is the number of image inputs; a shape is run eagerly a
 few times on a forked stream before it is recorded; shapes named at start-up are recorded then and a
 shape that fails to record is reported and left to the eager path; any other shape is recorded the
-first time a request needs it; per request the inputs are copied into the graph's static tensors on
-a stream of their own and the replay waits for that stream through one event.
+first time a request needs it; per request the inputs are copied into the graph's static tensors
+(optionally on a stream of their own that the replay waits for through one event, as the reference does).
 
 On PyTorch-ROCm ``torch.cuda.CUDAGraph`` is a hipGraph, and this package's HIP kernels are launched
 on torch's current stream, so stream capture records them exactly like torch's own launches.
@@ -117,9 +117,17 @@ class GraphRunner:
     ``record(key, request)`` is the backend's function that builds static tensors for ``key``, records
     the graph and returns whatever the backend wants to keep for replays (an "entry")."""
 
-    def __init__(self, record: Callable[[Hashable, Any], Any], device, *, label: str = "graph", logger: logging.Logger | None = None):
+    def __init__(
+        self, record: Callable[[Hashable, Any], Any], device, *, label: str = "graph", logger: logging.Logger | None = None,
+        input_stream: bool = False,
+    ):  # fmt: skip
         self.device = torch.device(device)
         self.label = label
+        # The reference copies a request's inputs on a stream of their own and joins it to the replay with
+        # one event.  The engine API is synchronous (one request at a time, the result returned to the
+        # host), so nothing can overlap with those copies; on this stack the fork / join costs 0.1 ms per
+        # request, and the copies run on the current stream unless ``input_stream`` asks for the other way.
+        self.use_input_stream = bool(input_stream)
         self._record = record
         self._log = logger if logger is not None else _LOG
         self._shapes: dict[Hashable, Any] = {}
@@ -160,6 +168,9 @@ class GraphRunner:
     def copy_inputs(self) -> Iterator[torch.cuda.Stream]:
         """Inside the block, copies into the static tensors run on the input stream (ordered after
         everything already queued on the current stream); leaving it marks the inputs ready."""
+        if not self.use_input_stream:
+            yield torch.cuda.current_stream(self.device)
+            return
         if self._input_stream is None:
             self._input_stream = torch.cuda.Stream(device=self.device)
             self._inputs_ready = torch.cuda.Event()
@@ -170,6 +181,8 @@ class GraphRunner:
 
     def wait_inputs(self) -> None:
         """Order the current stream (the replay) after the copies of the last :meth:`copy_inputs` block."""
+        if not self.use_input_stream:
+            return
         if self._inputs_ready is None:
             raise RuntimeError("wait_inputs() called before any copy_inputs() block")
         torch.cuda.current_stream(self.device).wait_event(self._inputs_ready)
