@@ -148,6 +148,36 @@ def test_engine_api_graph_equals_eager_and_camera_keys(ckpt):
     assert not np.array_equal(c1, c2)
 
 
+def test_graph_requests_with_changing_task_noise_and_host_inputs(ckpt):
+    # the graph path caches task tokens / masks and reuses static tensors: alternating tasks, an implicit-noise
+    # request between explicit ones, host-resident frames and a queue drained across requests must all give
+    # what the eager engine gives
+    from tybok_amd.registry import create_engine
+
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_fused_attn=True, tl_vit_oproj=True)
+    eager = create_engine(ckpt, device="cuda", graph=False, warmup=False, **flags)
+    graph = create_engine(ckpt, device="cuda", graph=True, graph_cameras=(3,), warmup=True, seed=9, **flags)
+    noise = torch.zeros(1, 50, 6)
+    frames = []
+    for seed, task in ((1, "pick up the cube"), (2, "open the drawer"), (3, "pick up the cube")):
+        f = eager._profile_frame(cameras=3, seed=seed)
+        f["task"] = task
+        frames.append(f)
+    want = [eager.predict_action_chunk(f, noise=noise) for f in frames]
+    assert not np.array_equal(want[0], want[1])
+    for f, w in zip(frames, want):
+        assert np.array_equal(graph.predict_action_chunk(f, noise=noise), w)
+    graph.predict_action_chunk(frames[0])  # implicit noise fills every padded action column of the static tensor
+    assert np.array_equal(graph.predict_action_chunk(frames[1], noise=noise), want[1])
+    on_device = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in frames[2].items()}
+    assert np.array_equal(graph.predict_action_chunk(on_device, noise=noise.cuda()), want[2])
+    # select_action keeps the chunk of its first request while other requests replay the graph in between
+    first = graph.select_action(frames[0], noise=noise)
+    graph.predict_action_chunk(frames[1], noise=noise)
+    second = graph.select_action(frames[1], noise=noise)  # still from the queue filled by frames[0]
+    assert np.array_equal(first, want[0][0]) and np.array_equal(second, want[0][1])
+
+
 def test_engine_rejects_flags_it_does_not_implement(ckpt):
     from tybok_amd.registry import create_engine
 
