@@ -133,3 +133,17 @@ def test_arguments_are_checked_on_the_host(name, args, code, fragment):
     message = lib.tk_last_error().decode()
     assert rc == code, f"{name}: rc {rc}, message {message!r}"
     assert fragment in message, message
+
+
+@pytest.mark.parametrize("compiler,flags", [("gcc", ["-std=c99", "-x", "c"]), ("g++", ["-std=c++17", "-x", "c++"])])
+def test_header_is_plain_c_and_cxx(tmp_path, compiler, flags):
+    # the boundary is a C ABI: the header must be usable from C (cgo, ctypes generators, C hosts) and from C++
+    import shutil
+    import subprocess
+
+    if shutil.which(compiler) is None:
+        pytest.skip(f"{compiler} not installed")
+    src = tmp_path / "use_header.c"
+    src.write_text(f'#include "{HEADER}"\nint main(void) {{ return tk_version() > 0 && TK_OK == 0 ? 0 : 1; }}\n')
+    done = subprocess.run([compiler, *flags, "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", str(src)], capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr
