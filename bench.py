@@ -240,16 +240,26 @@ def cpu_baseline_smolvla(cameras: int) -> dict:
     state = torch.zeros(1, shape.max_state_dim)
     noise = torch.zeros(1, shape.chunk, shape.max_action_dim)
     masks = [torch.ones(1, dtype=torch.bool)] * cameras
-    t0 = time.perf_counter()
-    with torch.no_grad():
-        O.sample_actions(w, shape, O.prepare_images(images), masks, tokens, torch.ones(1, shape.tok_len, dtype=torch.bool), state, noise)
-    ms = (time.perf_counter() - t0) * 1e3
+    lang_masks = torch.ones(1, shape.tok_len, dtype=torch.bool)
+
+    def request() -> float:
+        t0 = time.perf_counter()
+        with torch.no_grad():
+            O.sample_actions(w, shape, O.prepare_images(images), masks, tokens, lang_masks, state, noise)
+        return (time.perf_counter() - t0) * 1e3
+
+    request()  # warm-up (thread pool, allocator)
+    # a bounded sample: requests until about 12 s of CPU work have been spent, at least 3, at most 20
+    samples, budget_ms = [], 12_000.0
+    while len(samples) < 3 or (sum(samples) < budget_ms and len(samples) < 20):
+        samples.append(request())
     return {
-        "value": round(ms, 1),
+        "value": round(float(np.percentile(samples, 50)), 1),
         "unit": "ms",
         "cores": int(torch.get_num_threads()),
         "kind": "port",
-        "sample": f"1 predict_action_chunk of the same SmolVLA-shaped workload ({cameras} cameras, 10 steps, fp8 MLP weights), CPU oracle, no warm-up",
+        "sample": f"p50 of {len(samples)} predict_action_chunk requests of the same SmolVLA-shaped workload ({cameras} cameras, 10 steps, "
+        f"fp8 MLP weights) through the CPU oracle after one warm-up ({sum(samples) / 1e3:.1f} s of CPU work)",
     }
 
 
