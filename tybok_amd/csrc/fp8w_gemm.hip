@@ -665,15 +665,15 @@ int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st) {
   const int epi = a.s1 != nullptr ? 1 : (a.rope_pos != nullptr ? 2 : 0);
   const int pro = a.ada_scale != nullptr ? 3 : (a.norm_w == nullptr ? 0 : (a.x_f32 ? 2 : 1));
   if (a.w16) {
-    // bf16-weight linears of the expert layers (M > 32 only: the action chunk)
-    if (MT != 2 || NT != 2) return -1;
+    // bf16-weight linears of the expert / VLM layers: two-tile strips, 32- or 64-row blocks
+    if (NT != 2) return -1;
     if (epi == 2) {
-      if (pro == 1) return launch<2, 2, 2, true, 1>(a, grid, st);
-      if (pro == 2) return launch<2, 2, 2, true, 2>(a, grid, st);
-      if (pro == 3) return launch<2, 2, 2, true, 3>(a, grid, st);
-      return launch<2, 2, 2, true, 0>(a, grid, st);
+      if (pro == 1) return MT == 1 ? launch<1, 2, 2, true, 1>(a, grid, st) : launch<2, 2, 2, true, 1>(a, grid, st);
+      if (pro == 2) return MT == 1 ? launch<1, 2, 2, true, 2>(a, grid, st) : launch<2, 2, 2, true, 2>(a, grid, st);
+      if (pro == 3) return MT == 1 ? launch<1, 2, 2, true, 3>(a, grid, st) : launch<2, 2, 2, true, 3>(a, grid, st);
+      return MT == 1 ? launch<1, 2, 2, true, 0>(a, grid, st) : launch<2, 2, 2, true, 0>(a, grid, st);
     }
-    if (epi == 0 && pro == 0) return launch<2, 2, 0, true, 0>(a, grid, st);
+    if (epi == 0 && pro == 0) return MT == 1 ? launch<1, 2, 0, true, 0>(a, grid, st) : launch<2, 2, 0, true, 0>(a, grid, st);
     return -1;
   }
   if (epi == 2 || pro == 2) return -1;

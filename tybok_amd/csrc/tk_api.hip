@@ -192,9 +192,14 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
     return TK_OK;
   }
   int MT = M <= 32 ? 1 : 2;
+  // The action chunk (33..64 rows) over a small weight matrix is a latency-bound launch: two blocks
+  // of 32 rows per strip halve each block's staging, normalisation and product work and put twice
+  // as many CUs on it (measured: FFN at K=720 12.6 -> 10.0 us, with the norm prologue 15.7 -> 12.6 us);
+  // the weights are then read twice, which only a large matrix notices (the 33.5 MB shapes lose 5 %).
+  if (M > 32 && M <= 64 && (size_t)a.ntiles * 32 * a.KT * 32 * (e.w16 ? 2 : 1) <= (16u << 20)) MT = 1;
   int NT = 2;
   if (e.w16) {
-    MT = 2;  // the bf16-weight kernels exist for the action-chunk tile shape only
+    // (the bf16-weight kernels are built with two-tile strips only)
   } else if (!gated && ((a.ntiles + 1) / 2) * ((M + 32 * MT - 1) / (32 * MT)) < cus / 2) {
     NT = 1;  // few columns: finer strips
   }
