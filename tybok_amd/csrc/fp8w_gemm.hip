@@ -665,8 +665,11 @@ int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st) {
   const int epi = a.s1 != nullptr ? 1 : (a.rope_pos != nullptr ? 2 : 0);
   const int pro = a.ada_scale != nullptr ? 3 : (a.norm_w == nullptr ? 0 : (a.x_f32 ? 2 : 1));
   if (a.w16) {
-    // bf16-weight linears of the expert / VLM layers: two-tile strips, 32- or 64-row blocks
-    if (NT != 2) return -1;
+    // bf16-weight linears of the expert / VLM layers: 32- or 64-row blocks; one-tile strips for the plain epilogue only
+    if (NT == 1) {
+      if (epi != 0 || pro != 0) return -1;
+      return MT == 1 ? launch<1, 1, 0, true, 0>(a, grid, st) : launch<2, 1, 0, true, 0>(a, grid, st);
+    }
     if (epi == 2) {
       if (pro == 1) return MT == 1 ? launch<1, 2, 2, true, 1>(a, grid, st) : launch<2, 2, 2, true, 1>(a, grid, st);
       if (pro == 2) return MT == 1 ? launch<1, 2, 2, true, 2>(a, grid, st) : launch<2, 2, 2, true, 2>(a, grid, st);

@@ -198,10 +198,8 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   // the weights are then read twice, which only a large matrix notices (the 33.5 MB shapes lose 5 %).
   if (M > 32 && M <= 64 && (size_t)a.ntiles * 32 * a.KT * 32 * (e.w16 ? 2 : 1) <= (16u << 20)) MT = 1;
   int NT = 2;
-  if (e.w16) {
-    // (the bf16-weight kernels are built with two-tile strips only)
-  } else if (!gated && ((a.ntiles + 1) / 2) * ((M + 32 * MT - 1) / (32 * MT)) < cus / 2) {
-    NT = 1;  // few columns: finer strips
+  if (!gated && !rope && ((a.ntiles + 1) / 2) * ((M + 32 * MT - 1) / (32 * MT)) < cus / 2) {
+    NT = 1;  // few columns: finer strips (the paired epilogues need both tiles of a strip in one wave)
   }
   const int mblocks = (M + 32 * MT - 1) / (32 * MT);
   const int strips = (a.ntiles + NT - 1) / NT;
@@ -209,19 +207,21 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   const int NW = 4;
   int ks = split_k;
   if (ks <= 0) {
-    // Launch-cost model (microseconds, measured per phase on MI355X): the k loop costs about
-    // 0.35 per block round (NW k tiles) with a floor of one memory round trip; splitting K adds a
-    // partial write, an arrival count and a read-back that the finishing block issues four splits at
-    // a time (about 1.2 + 0.9 per batch of four) and only pays while the grid still fits the device
-    // twice over.
+    // Launch-cost model (microseconds, fitted to graph-replayed launches on MI355X): the k loop costs
+    // 0.35 per block round (NW k tiles) for 64-row blocks, 0.20 (fp8) / 0.27 (bf16 weights) for 32-row
+    // blocks, with a floor of one memory round trip; splitting K adds a partial write, an arrival
+    // count and a read-back that grows with the number of splits and steps up with every batch of four
+    // the finishing block has in flight (1.1 + 0.4 c + 1.0 per further batch), and only pays while the
+    // grid still fits the device twice over.
     ks = 1;
     if (blocks0 < cus) {
+      const float per_round = MT == 1 ? (e.w16 ? 0.27f : 0.20f) : 0.35f;
       float best = 1e30f;
       for (int c = 1; c <= 64 && c * NW <= a.KT && (c == 1 || blocks0 * c <= 2 * cus); ++c) {
         const int rounds = (a.KT + c * NW - 1) / (c * NW);
-        float t = rounds * 0.35f;
+        float t = rounds * per_round;
         if (t < 1.0f) t = 1.0f;
-        if (c > 1) t += 1.2f + 0.9f * (float)((c + 3) / 4);
+        if (c > 1) t += 1.1f + 0.4f * (float)c + 1.0f * (float)((c + 3) / 4 - 1);
         if (t < best - 1e-3f) {
           best = t;
           ks = c;
