@@ -76,7 +76,8 @@ __global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kerne
   constexpr int KT = kStageKeys / 32;   // key tiles per stage
   constexpr int KP = L::KP, VP = L::VP, KBYTES = L::KBYTES, VBYTES = L::VBYTES;
   constexpr int KCH = D / 8;            // 16-byte chunks per K row
-  constexpr int NLD = D / 32;           // chunks per thread and stage, K and V^T alike (64*D/8 / 256)
+  constexpr int NLD = kStageKeys * KCH / kGroupThreads;  // 16-byte chunks per thread and stage, K and V^T alike
+  static_assert(kStageKeys * KCH % kGroupThreads == 0, "a stage must divide evenly over the group's threads");
   extern __shared__ __align__(16) unsigned char lds_all[];
 
   const int tid = threadIdx.x;
