@@ -208,14 +208,14 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   int ks = split_k;
   if (ks <= 0) {
     // Launch-cost model (microseconds, fitted to graph-replayed launches on MI355X): the k loop costs
-    // 0.35 per block round (NW k tiles) for 64-row blocks, 0.20 (fp8) / 0.27 (bf16 weights) for 32-row
-    // blocks, with a floor of one memory round trip; splitting K adds a partial write, an arrival
+    // 0.35 per block round (NW k tiles) for 64-row blocks, 0.20 for 32-row blocks (0.27 with two bf16
+    // weight tiles per wave and round), with a floor of one memory round trip; splitting K adds a partial write, an arrival
     // count and a read-back that grows with the number of splits and steps up with every batch of four
     // the finishing block has in flight (1.1 + 0.4 c + 1.0 per further batch), and only pays while the
     // grid still fits the device twice over.
     ks = 1;
     if (blocks0 < cus) {
-      const float per_round = MT == 1 ? (e.w16 ? 0.27f : 0.20f) : 0.35f;
+      const float per_round = MT == 1 ? (e.w16 && NT == 2 ? 0.27f : 0.20f) : 0.35f;
       float best = 1e30f;
       for (int c = 1; c <= 64 && c * NW <= a.KT && (c == 1 || blocks0 * c <= 2 * cus); ++c) {
         const int rounds = (a.KT + c * NW - 1) / (c * NW);
