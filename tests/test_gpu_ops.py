@@ -375,3 +375,24 @@ def test_gated_residual_epilogue(tk):
     want = resid + oops.lin_fp8w(h, wd8, sd) * gate
     got = tk.fp8w_gemm(h.cuda(), pw, resid=resid.cuda(), gate=gate.cuda())
     _close(got, want, "gemm gated residual")
+
+
+@pytest.mark.parametrize("m,k,n", [(3072, 768, 3072), (512, 1152, 4304), (7, 64, 96)])
+def test_linear_gelu_tanh_is_the_tanh_form_of_the_two_launch_op(tk, m, k, n):
+    """The vision towers' fc1 + GELU as one library GEMM (activation in the epilogue) against the two-launch
+    form of the reference (vision.py: ``gelu_pytorch_tanh(fc1(x))``) on the CPU, and -- on the rows where the
+    tanh and the erf form differ most -- against both closed forms in fp64: it has to be the tanh one."""
+    g = torch.Generator().manual_seed(m + n)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) * 1.5 * k**-0.5).to(torch.bfloat16)
+    b = torch.randn(n, generator=g).to(torch.bfloat16)
+    got = tk.linear_gelu_tanh(x.cuda(), w.cuda(), b.cuda())
+    want = torch.nn.functional.gelu(torch.nn.functional.linear(x, w, b), approximate="tanh")
+    _close(got, want, f"linear_gelu_tanh {m}x{k}->{n}")
+    z = x.double() @ w.double().t() + b.double()
+    sel = (z.abs() > 1.0) & (z.abs() < 3.0)
+    if int(sel.sum()) > 100_000:
+        err_tanh = (got.cpu().double() - torch.nn.functional.gelu(z, approximate="tanh"))[sel]
+        err_erf = (got.cpu().double() - torch.nn.functional.gelu(z))[sel]
+        # the two forms differ by 2.2e-5 on average over this range; rounding noise averages out
+        assert abs(float(err_tanh.mean())) < 6e-6 < abs(float(err_erf.mean()))

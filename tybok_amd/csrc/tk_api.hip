@@ -197,6 +197,12 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   // as many CUs on it (measured: FFN at K=720 12.6 -> 10.0 us, with the norm prologue 15.7 -> 12.6 us);
   // the weights are then read twice, which only a large matrix notices (the 33.5 MB shapes lose 5 %).
   if (M > 32 && M <= 64 && (size_t)a.ntiles * 32 * a.KT * 32 * (e.w16 ? 2 : 1) <= (16u << 20)) MT = 1;
+#ifdef TK_PHASE_TIMING
+  if (const char* ev = getenv("TK_GEMM_MT")) {  // development aid, never in the shipped build
+    const int v = atoi(ev);
+    if ((v == 1 || v == 2) && M > 32) MT = v;
+  }
+#endif
   int NT = 2;
   if (!gated && !rope && ((a.ntiles + 1) / 2) * ((M + 32 * MT - 1) / (32 * MT)) < cus / 2) {
     NT = 1;  // few columns: finer strips (the paired epilogues need both tiles of a strip in one wave)

@@ -580,6 +580,17 @@ def batched_attn(
     return out
 
 
+def linear_gelu_tanh(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """``gelu_tanh(x @ weight^T + bias)`` for bf16 operands on the GPU as ONE library GEMM with the bias and the
+    activation in its epilogue (the vision towers' fc1: 32 us instead of 46 us as GEMM + elementwise launch at
+    3072 x 768 -> 3072).  The epilogue evaluates the tanh form on the fp32 accumulator, so the one difference
+    from ``F.gelu(F.linear(...), approximate="tanh")`` is that the pre-activation is not rounded to bf16 first."""
+    if not (x.is_cuda and x.dtype == weight.dtype == bias.dtype == torch.bfloat16):
+        raise TypeError("linear_gelu_tanh: bf16 CUDA operands only")
+    y = torch._addmm_activation(bias, x.reshape(-1, x.shape[-1]), weight.t(), use_gelu=True)
+    return y.view(*x.shape[:-1], weight.shape[0])
+
+
 def transpose_v(v: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Tensor:
     """``v [B, P, G, D]`` bf16 (a view with a contiguous head dim, e.g. into a packed q|k|v buffer) ->
     ``vt [B, G, D, P rounded up to 32]`` with zero-filled padding keys: the V^T operand of

@@ -263,7 +263,10 @@ class PI05Model:
                     h = tk.layer_norm(x, p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS)
                 else:
                     h = F.layer_norm(x, (vh,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS).to(self.vit_mlp_dtype)
-                m = F.gelu(F.linear(h, *self.vis_lowp[lp + "mlp.fc1"]), approximate="tanh")
+                if self.vit_mlp_dtype == BF16 and x.is_cuda:
+                    m = tk.linear_gelu_tanh(h, *self.vis_lowp[lp + "mlp.fc1"])
+                else:
+                    m = F.gelu(F.linear(h, *self.vis_lowp[lp + "mlp.fc1"]), approximate="tanh")
                 x = x + F.linear(m, *self.vis_lowp[lp + "mlp.fc2"])  # fp32 + low precision: promoted inside the add
             else:
                 h = F.layer_norm(x, (vh,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS)
@@ -285,7 +288,7 @@ class PI05Model:
             qkv = F.linear(h, *self.vis_lowp[lp + "self_attn.qkv"]).view(b, -1, 3, heads, hp)
             a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], tk.transpose_v(qkv[:, :, 2]), scale=hd**-0.5, ws=self.ws)
             x, h = tk.add_layer_norm(x, F.linear(a, *self.vis_lowp[lp + "self_attn.out_proj"]), *ln(i, 2), EPS)
-            m = F.linear(F.gelu(F.linear(h, *self.vis_lowp[lp + "mlp.fc1"]), approximate="tanh"), *self.vis_lowp[lp + "mlp.fc2"])
+            m = F.linear(tk.linear_gelu_tanh(h, *self.vis_lowp[lp + "mlp.fc1"]), *self.vis_lowp[lp + "mlp.fc2"])
             if i + 1 < cfg.vision_layers:
                 x, h = tk.add_layer_norm(x, m, *ln(i + 1, 1), EPS)
             else:

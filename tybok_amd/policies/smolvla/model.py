@@ -250,7 +250,7 @@ class SmolVLAModel:
                 vt = tk.transpose_v(qkv[:, :, 2])
                 a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, ws=self.ws)
                 x, h = tk.add_layer_norm(x, self.lin(lp + "self_attn.out_proj", a), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
-                m = self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
+                m = self.lin(lp + "mlp.fc2", tk.linear_gelu_tanh(h, p[lp + "mlp.fc1.weight"], p[lp + "mlp.fc1.bias"]))
                 if i + 1 < v.num_hidden_layers:
                     nx = f"{VIS}encoder.layers.{i + 1}."
                     x, h = tk.add_layer_norm(x, m, p[nx + "layer_norm1.weight"], p[nx + "layer_norm1.bias"], v.layer_norm_eps)
