@@ -157,6 +157,12 @@ ATTN_CASES = [
     (50, 712, 8, 1, 256, oops.MASK_BIDIR, True),    # pi0.5 expert
     (7, 5, 4, 2, 64, oops.MASK_CAUSAL, False),      # tiny, ragged
     (33, 95, 4, 4, 128, oops.MASK_BIDIR, False),
+    # 256-wide heads take the kernel that cuts the two products along different axes (8 key tiles per block)
+    (50, 712, 8, 1, 256, oops.MASK_CAUSAL, False),  # 4 key splits, causal suffix, fp32 logits
+    (7, 5, 4, 2, 256, oops.MASK_CAUSAL, True),      # one block of two key tiles: six idle waves
+    (50, 230, 8, 1, 256, oops.MASK_BIDIR, True),    # 2 splits of 5 tiles
+    (33, 1900, 2, 2, 256, oops.MASK_BIDIR, False),  # 8 splits, the most one launch takes
+    (40, 2100, 2, 1, 256, oops.MASK_BIDIR, True),   # beyond that: the general kernel
 ]
 
 
@@ -197,8 +203,9 @@ def test_attention_strided_kv_cache_views(tk):
     _close(got, want, "attn head-major prefix")
 
 
-def test_attention_fully_masked_prefix_is_uniform(tk):
-    q, k_pre, v_pre, _, _ = attn_case(50, 64, 15, 5, 64, seed=3)
+@pytest.mark.parametrize("h,g,d", [(15, 5, 64), (8, 1, 256)])
+def test_attention_fully_masked_prefix_is_uniform(tk, h, g, d):
+    q, k_pre, v_pre, _, _ = attn_case(50, 64, h, g, d, seed=3)
     none = torch.zeros(64, dtype=torch.bool)
     want = oops.expert_attention(q, k_pre, v_pre, None, None, none, oops.MASK_NONE)
     got = tk.expert_attn_plain(q.cuda(), k_pre.cuda(), v_pre.cuda(), None, None, none.cuda(), oops.MASK_NONE)

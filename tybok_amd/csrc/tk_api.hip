@@ -532,10 +532,21 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   if (splits > (D > 128 ? 7 : 8)) splits = D > 128 ? 7 : 8;
   // many query tiles already fill the device: keep whole key ranges in one block (no partials)
   while (splits > 1 && H * mtiles * splits > 2 * device_cus()) --splits;
+  // 256-wide heads, few query tiles (the pi0.5 action expert): blocks of 8 waves that cut the two
+  // products along different axes and cover 8 key tiles each
+  bool d256 = false;
+  if (D == 256 && !split && !mask2d && batch == 0 && ntiles <= tk_attn_d256_max_tiles()) {
+    const int per = tk_attn_d256_tiles_per_block();
+    const int sp = (ntiles + per - 1) / per;
+    if (H * mtiles * sp <= 2 * device_cus()) {
+      d256 = true;
+      splits = sp;
+    }
+  }
 #ifdef TK_PHASE_TIMING
   if (const char* ev = getenv("TK_ATTN_SPLITS")) {  // development aid, never in the shipped build
     const int v = atoi(ev);
-    if (v >= 1 && v <= 8 && D == 256) splits = v;
+    if (v >= 1 && v <= 8 && D == 256 && !d256) splits = v;
   }
 #endif
   a.kv_splits = splits;
@@ -553,7 +564,7 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
     a.partial = (float*)((char*)ws + kPartialOff);
     a.counters = (int*)ws;
   }
-  int rc = tk_launch_attn(a, D, waves, (hipStream_t)stream);
+  int rc = d256 ? tk_launch_attn_d256(a, (hipStream_t)stream) : tk_launch_attn(a, D, waves, (hipStream_t)stream);
   if (rc) return fail(TK_ELAUNCH, "attn: launch failed (%s)", hipGetErrorString(hipGetLastError()));
   return TK_OK;
 }
