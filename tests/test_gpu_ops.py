@@ -157,12 +157,12 @@ ATTN_CASES = [
     (50, 712, 8, 1, 256, oops.MASK_BIDIR, True),    # pi0.5 expert
     (7, 5, 4, 2, 64, oops.MASK_CAUSAL, False),      # tiny, ragged
     (33, 95, 4, 4, 128, oops.MASK_BIDIR, False),
-    # 256-wide heads take the kernel that cuts the two products along different axes (8 key tiles per block)
+    # 256-wide heads take the kernel that cuts the two products along different axes (rounds of 8 key tiles)
     (50, 712, 8, 1, 256, oops.MASK_CAUSAL, False),  # 4 key splits, causal suffix, fp32 logits
     (7, 5, 4, 2, 256, oops.MASK_CAUSAL, True),      # one block of two key tiles: six idle waves
     (50, 230, 8, 1, 256, oops.MASK_BIDIR, True),    # 2 splits of 5 tiles
-    (33, 1900, 2, 2, 256, oops.MASK_BIDIR, False),  # 8 splits, the most one launch takes
-    (40, 2100, 2, 1, 256, oops.MASK_BIDIR, True),   # beyond that: the general kernel
+    (33, 1900, 2, 2, 256, oops.MASK_BIDIR, False),  # 8 splits (the most) of one round each
+    (40, 2100, 2, 1, 256, oops.MASK_BIDIR, True),   # 8 splits of two rounds (8 + 1 tiles; the suffix in the last)
 ]
 
 
@@ -212,7 +212,7 @@ def test_attention_fully_masked_prefix_is_uniform(tk, h, g, d):
     _close(got, want, "attn fully masked")
 
 
-@pytest.mark.parametrize("p,h,g,d", [(241, 15, 5, 64), (177, 15, 5, 64), (40, 4, 2, 128), (1024, 12, 12, 64)])
+@pytest.mark.parametrize("p,h,g,d", [(241, 15, 5, 64), (177, 15, 5, 64), (40, 4, 2, 128), (1024, 12, 12, 64), (712, 8, 1, 256), (90, 4, 2, 256), (1000, 16, 2, 256)])
 def test_prefill_attention_with_2d_mask(tk, p, h, g, d):
     # the VLM prefill: every token is a query, keys are the same tokens, visibility from the
     # block-causal 2-D mask (image/language tokens see each other, the state token sees all) & padding

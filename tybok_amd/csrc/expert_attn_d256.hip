@@ -12,8 +12,10 @@
 // Each wave requests everything it will read -- its Q tile, its K tile and the V^T rows of its 32
 // output columns for the whole key range -- before the first MFMA, keeps one accumulator tile, and the
 // eight waves finish (or hand to the last-arriving block of a key split) disjoint slices of the output.
-// A block covers at most 8 key tiles; longer key ranges are split over blocks (fixed-order merge of
-// the fp32 partials by the last-arriving block, as in the other attention kernel).
+// A block walks its key range in rounds of 8 key tiles (online softmax across rounds: one rescale of the
+// accumulator tile per round).  Few query tiles (the denoise step): the key range is split over blocks
+// of one round each, and the last-arriving block merges the fp32 partials in split order, as in the
+// other attention kernel.  Many query tiles (the prefill): one block per query tile and head, no hand-off.
 #include <math.h>
 #include "tk_common.h"
 #include "tk_kernels.h"
@@ -84,18 +86,29 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
   const int g = (h * a.gqa_mul) >> 16;
   const int tp = (a.P + 31) >> 5;  // prefix tiles; suffix tiles follow
   const int t_lo = split * a.tile_q + (split < a.tile_r ? split : a.tile_r);
-  const int nt = a.tile_q + (split < a.tile_r ? 1 : 0);  // key tiles of this block, 1..kWaves
+  const int ntb = a.tile_q + (split < a.tile_r ? 1 : 0);  // key tiles of this block, in rounds of kWaves
   const int qi = mtile * 32 + l32;
   const bool q_ok = qi < a.M;
-  const bool active = wave < nt;  // this wave has a key tile of its own
   unsigned char* const mine = lds + (1 + wave) * kTileBytes;
+  const int tid = threadIdx.x;
+
+  // running softmax base / sum of this lane's query (the same in every wave) and this wave's slice of O^T
+  float bm = -INFINITY, bl = 0.f;
+  f32x16 o;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) o[i] = 0.f;
 
   TA_MARK(0);
+  for (int r_lo = 0; r_lo < ntb; r_lo += kWaves) {
+  const int nt = ntb - r_lo < kWaves ? ntb - r_lo : kWaves;  // key tiles of this round, 1..kWaves
+  const int rt_lo = t_lo + r_lo;
+  const bool active = wave < nt;  // this wave has a key tile of its own
+  // (a further round: every wave must be past its reads of the last round's P^T, which the Q tile overwrites)
+  if (r_lo > 0) lds_only_barrier();
   // ---- every load, back to back, as whole 512-byte rows (lane -> consecutive 16-byte chunks): Q by the
   // block, K (32 keys x 256 d) and V^T (this wave's 32 d rows x the block's 256 keys) per wave.  Read
   // straight into operand registers instead (one row per lane), every load instruction would touch
   // 32 cache lines for 1 KiB, and the CU's 8 waves x 48 such loads are bound by its tag-lookup rate. ----
-  const int tid = threadIdx.x;
   i32x4 qreg[2], kreg[16], vreg[16];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
@@ -104,7 +117,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
     if (m > a.M - 1) m = a.M - 1;  // rows past M are never stored
     qreg[i] = *(const i32x4*)(a.q + (size_t)m * a.q_sm + (size_t)h * a.q_sh + col * 8);
   }
-  const int t = t_lo + (active ? wave : nt - 1);  // idle waves read a valid tile and drop it
+  const int t = rt_lo + (active ? wave : nt - 1);  // idle waves read a valid tile and drop it
   const bool pre = t < tp;
   const int tt = pre ? t : t - tp;
   const int len = pre ? a.P : a.S;
@@ -120,16 +133,22 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
     }
   }
   // per-key visibility of the prefix (always requested, from a harmless address when unused)
-  const bool use_pad = pre && a.pad != nullptr;
+  const bool use_pad = pre && a.mask2d == nullptr && a.pad != nullptr;
   const int key = tt * 32 + l32;
   const int padv = *((use_pad && key < a.P) ? a.pad + key : (const uint8_t*)a.q);
   const int pad_ok = use_pad ? (key < a.P ? padv : 0) : 1;
+  // per-(query, key) visibility bytes of the tile (prefill): eight consecutive keys per word, the keys of
+  // this lane's registers 0..7 and 8..15
+  const bool use_m2 = pre && a.mask2d != nullptr;
+  const uint8_t* mp = use_m2 ? a.mask2d + (size_t)(q_ok ? qi : a.M - 1) * a.mask_ld + tt * 32 + 8 * half : (const uint8_t*)a.q;
+  const unsigned long long m2lo = *(const unsigned long long*)mp;
+  const unsigned long long m2hi = *(const unsigned long long*)(mp + (use_m2 ? 16 : 8));
   {
     // chunk col of a staged V^T row: key tile col / 4 of the block (tiles past the range: a valid
     // address, P^T is zero there), keys 8 * (col % 4) .. + 7 of that tile
     const int col = lane & 31;
     const int j = col >> 2;
-    const int tj = t_lo + (j < nt ? j : nt - 1);
+    const int tj = rt_lo + (j < nt ? j : nt - 1);
     const bool pj = tj < tp;
     const int ttj = pj ? tj : tj - tp;
     const size_t vsd = pj ? a.pre_vt_sd : a.suf_vt_sd;
@@ -160,18 +179,21 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
     *(i32x4*)(mine + key_of_row(c >> 5) * kPitch + (c & 31) * 16) = kreg[i];  // MFMA row r holds key key_of_row(r)
   }
   lds_only_barrier();  // the Q tile is complete (the K tile is this wave's own)
-  {
-    // every operand read goes out before the first product waits for one
-    i32x4 ka[DS], qb[DS];
+  // operand reads in two batches of 8 k steps, each batch out before its first product waits for one
+  // (all 16 at once would not leave registers for the V^T rows still held for the second product)
 #pragma unroll
-    for (int s = 0; s < DS; ++s) {
-      const int off = l32 * kPitch + (16 * s + 8 * half) * 2;
+  for (int s0 = 0; s0 < DS; s0 += 8) {
+    i32x4 ka[8], qb[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int off = l32 * kPitch + (16 * (s0 + s) + 8 * half) * 2;
       ka[s] = *(const i32x4*)(mine + off);
       qb[s] = *(const i32x4*)(qs + off);
     }
     __builtin_amdgcn_sched_barrier(0);  // (the scheduler would pair each read with its product again)
 #pragma unroll
-    for (int s = 0; s < DS; ++s) sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(ka[s]), as_bf16x8(qb[s]), sT, 0, 0, 0);
+    for (int s = 0; s < 8; ++s) sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(ka[s]), as_bf16x8(qb[s]), sT, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // ---- scale and mask.  Register i of this lane holds key 16*(i/8) + 8*half + i%8 of the tile;
@@ -192,6 +214,10 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
         const unsigned ch = c >= 24 ? 0xffu : (c > 16 ? (1u << (c - 16)) - 1u : 0u);
         vbits = cl | (ch << 8);
       }
+    } else if (a.mask2d) {
+      // one byte (0 or 1) per key: gather bit 0 of the 8 bytes of each word
+      const unsigned long long gather = 0x0102040810204080ull, ones = 0x0101010101010101ull;
+      vbits = (unsigned)(((m2lo & ones) * gather) >> 56) | ((unsigned)(((m2hi & ones) * gather) >> 56) << 8);
     } else {
       const unsigned pmask = (unsigned)__ballot(pad_ok != 0);  // lanes 0..31: keys of this tile
       vbits = ((pmask >> (8 * half)) & 0xffu) | (((pmask >> (16 + 8 * half)) & 0xffu) << 8);
@@ -214,13 +240,16 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
   tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
   if (half == 0) st_m[wave][l32] = tmax;
   lds_only_barrier();
-  float bm = st_m[0][l32];
+  float m_new = bm;
 #pragma unroll
-  for (int w = 1; w < kWaves; ++w) bm = fmaxf(bm, st_m[w][l32]);
+  for (int w = 0; w < kWaves; ++w) m_new = fmaxf(m_new, st_m[w][l32]);
+  // every round has a key in range, so m_new is finite; the first round's alpha is exp(-inf) = 0
+  const float alpha = __expf(bm - m_new);
+  bm = m_new;
   float lsum = 0.f;
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
-    p[i] = __expf(p[i] - bm);  // every block has a key in range: bm is finite; out-of-range keys give 0
+    p[i] = __expf(p[i] - bm);  // out-of-range keys give 0
     lsum += p[i];
   }
   lsum += __shfl_xor(lsum, 32);
@@ -234,15 +263,17 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
     *(i32x4*)(mine + (c >> 5) * kPitch + (c & 31) * 16) = vreg[i];  // over this wave's K tile, which it has consumed
   }
   lds_only_barrier();
-  float bl = st_l[0][l32];
+  {
+    float rl = st_l[0][l32];
 #pragma unroll
-  for (int w = 1; w < kWaves; ++w) bl += st_l[w][l32];
+    for (int w = 1; w < kWaves; ++w) rl += st_l[w][l32];
+    bl = bl * alpha + rl;
+  }
 
   TA_MARK(2);
-  // ---- O^T rows [32w, 32w + 32) += V^T . P^T over every key tile ----
-  f32x16 o;
+  // ---- O^T rows [32w, 32w + 32) += V^T . P^T over every key tile of the round ----
 #pragma unroll
-  for (int i = 0; i < 16; ++i) o[i] = 0.f;
+  for (int i = 0; i < 16; ++i) o[i] *= alpha;  // all of a lane's registers belong to its one query
   {
     i32x4 va[kWaves][2], pb[kWaves][2];
 #pragma unroll
@@ -258,6 +289,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
 #pragma unroll
       for (int s = 0; s < 2; ++s) o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(va[j][s]), as_bf16x8(pb[j][s]), o, 0, 0, 0);
   }
+  }  // rounds
 
   TA_MARK(3);
   // this lane's output: query qi, columns 32w + 8g4 + 4*half + 0..3 for the four register groups g4
@@ -356,13 +388,13 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
 
 }  // namespace
 
-int tk_attn_d256_max_tiles() { return kWaves * kMaxSplits; }
+int tk_attn_d256_max_splits() { return kMaxSplits; }
 int tk_attn_d256_tiles_per_block() { return kWaves; }
 
-// a.kv_splits blocks of at most 8 key tiles each; no hi/lo planes, no per-(query, key) mask, one problem
+// a.kv_splits blocks per (head, query tile), each over its share of the key tiles; no hi/lo planes, one problem
 int tk_launch_attn_d256(AttnArgs a, hipStream_t st) {
-  if (a.k_pre_lo || a.mask2d || a.batch > 0 || a.kv_splits < 1 || a.kv_splits > kMaxSplits) return -1;
-  if (a.tile_q + (a.tile_r ? 1 : 0) > kWaves || a.tile_q < 1) return -1;
+  if (a.k_pre_lo || a.batch > 0 || a.kv_splits < 1 || a.kv_splits > kMaxSplits) return -1;
+  if (a.tile_q < 1) return -1;
   // more LDS than a launch gets by default: raise the kernel's limit once per process
   static int raised = 0;
   if (!raised) {

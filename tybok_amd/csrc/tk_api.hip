@@ -532,16 +532,19 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   if (splits > (D > 128 ? 7 : 8)) splits = D > 128 ? 7 : 8;
   // many query tiles already fill the device: keep whole key ranges in one block (no partials)
   while (splits > 1 && H * mtiles * splits > 2 * device_cus()) --splits;
-  // 256-wide heads, few query tiles (the pi0.5 action expert): blocks of 8 waves that cut the two
-  // products along different axes and cover 8 key tiles each
+  // 256-wide heads (pi0.5): blocks of 8 waves that cut the two products along different axes and walk the
+  // keys 8 tiles at a time; one round per block while that leaves the device room, else several
   bool d256 = false;
-  if (D == 256 && !split && !mask2d && batch == 0 && ntiles <= tk_attn_d256_max_tiles()) {
+  if (D == 256 && !split && batch == 0) {
     const int per = tk_attn_d256_tiles_per_block();
-    const int sp = (ntiles + per - 1) / per;
-    if (H * mtiles * sp <= 2 * device_cus()) {
-      d256 = true;
-      splits = sp;
-    }
+    int sp = (ntiles + per - 1) / per;
+    if (sp > tk_attn_d256_max_splits()) sp = tk_attn_d256_max_splits();
+    if (H * mtiles * 2 >= device_cus()) sp = 1;  // the query tiles alone fill half the device: no hand-off
+    while (sp > 1 && H * mtiles * sp > 2 * device_cus()) --sp;
+    const size_t need = (size_t)H * mtiles * sp * (64 + (size_t)(D / 32) * 1024) * 4;
+    if (sp > 1 && !(ws && H * mtiles <= kMaxCounters && need <= kPartialBytes && ws_bytes >= kPartialOff + need)) sp = 1;
+    d256 = true;
+    splits = sp;
   }
 #ifdef TK_PHASE_TIMING
   if (const char* ev = getenv("TK_ATTN_SPLITS")) {  // development aid, never in the shipped build

@@ -204,9 +204,9 @@ int tk_launch_transpose_v(TransposeVArgs a, int D, hipStream_t st);
 int tk_launch_tower_attn(AttnArgs a, int D, hipStream_t st);
 int tk_attn_waves(int D, int split_planes, int ntiles);
 int tk_launch_attn(AttnArgs a, int D, int waves, hipStream_t st);
-// 256-wide heads: blocks of 8 waves over at most 8 key tiles each (a.kv_splits blocks per query tile)
+// 256-wide heads: blocks of 8 waves that walk their share of the key tiles 8 at a time (a.kv_splits blocks per query tile)
 int tk_launch_attn_d256(AttnArgs a, hipStream_t st);
-int tk_attn_d256_max_tiles();
+int tk_attn_d256_max_splits();
 int tk_attn_d256_tiles_per_block();
 int tk_launch_attn_qproj(AttnArgs a, hipStream_t st);
 int tk_launch_kv_prepare(KvPrepArgs p, hipStream_t st);
