@@ -1,0 +1,249 @@
+// Action-expert attention for 64-wide heads when one block covers the whole key range (the SmolVLA
+// self layers: 50 queries, 15 heads over 5 K/V heads, ~290 keys = 10 key tiles), same operands and
+// masks as expert_attn.hip.
+//
+// One wave per 32-key tile computes S^T = K . Q^T for its tile and the tile's softmax terms against
+// the block-wide maximum (one exchange of the tile maxima through LDS).  Q, K and V^T are read as whole
+// rows with coalesced 16-byte loads and staged through LDS into MFMA operand order.  Instead of every wave also multiplying its probabilities with its V tile and
+// the block then merging one partial output per wave (8 KiB each through LDS, summed by four owner
+// waves -- the longest phase of that kernel), the waves park their P^T tiles in LDS as ready-made B
+// operands (2 KiB each) and D/32 waves compute the whole O^T = V^T . P^T, one 32-row slice each, from
+// V^T rows they requested at the very start: no partial outputs, no merge.
+#include <math.h>
+#include "tk_common.h"
+#include "tk_kernels.h"
+
+namespace {
+
+constexpr float kF32Min = -3.4028234663852886e38f;  // finfo(float32).min
+constexpr float kOpenpiMask = -2.3819763e38f;       // additive mask of the pi0.5 path
+
+// K row held by MFMA row r of a key tile (bits 2 and 3 of r swapped): accumulator registers 8s..8s+7
+// of a lane are then eight consecutive keys, one 16-byte chunk of a V^T row and of the P^T operand
+__device__ __forceinline__ int key_of_row(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
+
+__device__ __forceinline__ i32x4 pack8(const float* v) {
+  i32x4 r = {(int)pack_bf16x2(v[0], v[1]), (int)pack_bf16x2(v[2], v[3]), (int)pack_bf16x2(v[4], v[5]), (int)pack_bf16x2(v[6], v[7])};
+  return r;
+}
+
+__device__ __forceinline__ void lds_only_barrier() {
+  // waits for LDS traffic only: the V^T loads stay in flight across it
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// NWV waves, at most NWV key tiles (prefix tiles, then suffix tiles); grid (head, query tile)
+template <int D, int NWV>
+__global__ __launch_bounds__(NWV * 64) void expert_attn_px_kernel(AttnArgs a) {
+  constexpr int DS = D / 16;  // k steps of Q.K^T
+  constexpr int DT = D / 32;  // 32-row slices of O^T = waves of the second product
+  static_assert(DT <= NWV, "one wave per output slice");
+  constexpr int RCH = D / 8;            // 16-byte chunks of a Q or K row
+  constexpr int KCH = 32 * RCH / 64;    // chunks of a K tile per lane
+  constexpr int VCH = D * 4 / 64;       // chunks of the block's V^T (D rows x NWV tiles x 4) per thread
+  constexpr int QPITCH = D * 2 + 16;    // staged Q / K rows: 16-byte operand reads of 32 rows stay conflict-free
+  constexpr int VPITCH = NWV * 64 + 16; // staged V^T rows (NWV tiles x 32 keys)
+  __shared__ float st_m[NWV][32], st_l[NWV][32];
+  __shared__ __align__(16) i32x4 pt[NWV][2][64];  // P^T of every key tile as B operands [tile][k step][lane]
+  __shared__ __align__(16) unsigned char qs[32 * QPITCH];
+  __shared__ __align__(16) unsigned char kst[NWV][32 * QPITCH];
+  __shared__ __align__(16) unsigned char vs[D * VPITCH];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int half = lane >> 5;
+  const int l32 = lane & 31;
+  const int h = blockIdx.x;
+  const int mtile = blockIdx.y;
+  const int g = (h * a.gqa_mul) >> 16;
+  const int tp = (a.P + 31) >> 5;  // prefix tiles; suffix tiles follow
+  const int nt = tp + ((a.S + 31) >> 5);
+  const int qi = mtile * 32 + l32;
+  const bool q_ok = qi < a.M;
+  const bool active = wave < nt;  // this wave has a key tile of its own
+  unsigned char* const ks = kst[wave];
+
+  // ---- every load up front, as whole rows (lane -> consecutive 16-byte chunks) staged through LDS:
+  // read straight into operand registers (one row per lane) every load instruction touches 32 cache
+  // lines for 1 KiB, and a block's 12 waves x 12 such loads are bound by the CU's tag-lookup rate ----
+  const int tid = threadIdx.x;
+  const int t = active ? wave : nt - 1;  // idle waves read a valid tile and drop it
+  const bool pre = t < tp;
+  const int tt = pre ? t : t - tp;
+  const int len = pre ? a.P : a.S;
+  i32x4 qreg, kreg[KCH], vreg[VCH];
+  {
+    // Q tile: 32 rows x D, one chunk per thread of the first waves
+    const int c = tid < 32 * RCH ? tid : 0, row = c / RCH, col = c % RCH;
+    int m = mtile * 32 + row;
+    if (m > a.M - 1) m = a.M - 1;  // rows past M are never stored
+    qreg = *(const i32x4*)(a.q + (size_t)m * a.q_sm + (size_t)h * a.q_sh + col * 8);
+  }
+  {
+    const u16* kb = (pre ? a.k_pre : a.k_suf) + (size_t)g * (pre ? a.pre_sh : a.suf_sh);
+    const size_t ksl = pre ? a.pre_sl : a.suf_sl;
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = lane + 64 * i, row = c / RCH, col = c % RCH;
+      int kr = tt * 32 + row;
+      if (kr > len - 1) kr = len - 1;  // masked below; keeps the address valid and the value finite
+      kreg[i] = *(const i32x4*)(kb + (size_t)kr * ksl + col * 8);
+    }
+  }
+  // per-key visibility of the prefix (always requested, from a harmless address when unused)
+  const bool use_pad = pre && a.pad != nullptr;
+  const int key = tt * 32 + l32;
+  const int padv = *((use_pad && key < a.P) ? a.pad + key : (const uint8_t*)a.q);
+  const int pad_ok = use_pad ? (key < a.P ? padv : 0) : 1;
+  // V^T: D rows x (NWV key tiles x 4 chunks), dealt to all threads; tiles past the range read a valid
+  // tile (their P^T is zero)
+#pragma unroll
+  for (int i = 0; i < VCH; ++i) {
+    const int c = tid + i * NWV * 64, row = c / (NWV * 4), col = c % (NWV * 4);
+    const int j = col >> 2;
+    const int tj = j < nt ? j : nt - 1;
+    const bool pj = tj < tp;
+    const int ttj = pj ? tj : tj - tp;
+    const u16* vb = (pj ? a.vt_pre : a.vt_suf) + (size_t)g * (pj ? a.pre_vt_sh : a.suf_vt_sh) + (size_t)row * (pj ? a.pre_vt_sd : a.suf_vt_sd);
+    vreg[i] = *(const i32x4*)(vb + ttj * 32 + (col & 3) * 8);
+  }
+  // keep the V^T requests above the first product: sunk below it they would leave a round trip later
+  __builtin_amdgcn_sched_barrier(0);
+
+  if (tid < 32 * RCH) *(i32x4*)(qs + (tid / RCH) * QPITCH + (tid % RCH) * 16) = qreg;
+#pragma unroll
+  for (int i = 0; i < KCH; ++i) {
+    const int c = lane + 64 * i;
+    *(i32x4*)(ks + key_of_row(c / RCH) * QPITCH + (c % RCH) * 16) = kreg[i];  // MFMA row r holds key key_of_row(r)
+  }
+  lds_only_barrier();  // the Q tile is complete (the K tile is this wave's own)
+
+  // ---- S^T tile = K . Q^T (one query column per lane) ----
+  f32x16 sT;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) sT[i] = 0.f;
+  {
+    i32x4 ka[DS], qb[DS];
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+      const int off = l32 * QPITCH + (16 * s + 8 * half) * 2;
+      ka[s] = *(const i32x4*)(ks + off);
+      qb[s] = *(const i32x4*)(qs + off);
+    }
+#pragma unroll
+    for (int s = 0; s < DS; ++s) sT = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(ka[s]), as_bf16x8(qb[s]), sT, 0, 0, 0);
+  }
+
+  // ---- scale and mask.  Register i of this lane holds key 16*(i/8) + 8*half + i%8 of the tile;
+  // visibility and range become two 16-bit masks (bit i = register i) ----
+  unsigned vbits, ibits;
+  {
+    const int k0 = tt * 32 + 8 * half;
+    const int left = len - k0;
+    const unsigned lo8 = left >= 8 ? 0xffu : (left > 0 ? (1u << left) - 1u : 0u);
+    const unsigned hi8 = left >= 24 ? 0xffu : (left > 16 ? (1u << (left - 16)) - 1u : 0u);
+    ibits = active ? (lo8 | (hi8 << 8)) : 0u;
+    if (!pre) {
+      if (a.mask_mode == 1) {
+        vbits = 0xffffu;
+      } else {  // causal among the suffix tokens: key <= query
+        const int c = qi - k0 + 1;
+        const unsigned cl = c >= 8 ? 0xffu : (c > 0 ? (1u << c) - 1u : 0u);
+        const unsigned ch = c >= 24 ? 0xffu : (c > 16 ? (1u << (c - 16)) - 1u : 0u);
+        vbits = cl | (ch << 8);
+      }
+    } else {
+      const unsigned pmask = (unsigned)__ballot(pad_ok != 0);  // lanes 0..31: keys of this tile
+      vbits = ((pmask >> (8 * half)) & 0xffu) | (((pmask >> (16 + 8 * half)) & 0xffu) << 8);
+    }
+  }
+  const bool lb = a.logits_bf16 != 0;
+  float p[16];
+  float tmax = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    float sv = sT[i];
+    sv = lb ? round_bf16(sv) : sv;
+    sv *= a.scale;
+    const float masked = lb ? sv + kOpenpiMask : kF32Min;
+    sv = (vbits >> i) & 1u ? sv : masked;
+    sv = (ibits >> i) & 1u ? sv : -INFINITY;
+    p[i] = sv;
+    tmax = fmaxf(tmax, sv);
+  }
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+  if (half == 0) st_m[wave][l32] = tmax;
+  lds_only_barrier();
+  float bm = st_m[0][l32];  // tile 0 always has a key in range: finite
+#pragma unroll
+  for (int w = 1; w < NWV; ++w) bm = fmaxf(bm, st_m[w][l32]);
+  float lsum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    p[i] = __expf(p[i] - bm);  // out-of-range keys give 0
+    lsum += p[i];
+  }
+  lsum += __shfl_xor(lsum, 32);
+  if (half == 0) st_l[wave][l32] = lsum;
+  pt[wave][0][lane] = pack8(p);
+  pt[wave][1][lane] = pack8(p + 8);
+#pragma unroll
+  for (int i = 0; i < VCH; ++i) {
+    const int c = tid + i * NWV * 64;
+    *(i32x4*)(vs + (c / (NWV * 4)) * VPITCH + (c % (NWV * 4)) * 16) = vreg[i];
+  }
+  lds_only_barrier();
+  if (wave >= DT) return;
+
+  // ---- O^T rows [32w, 32w + 32) = V^T . P^T over every key tile ----
+  float bl = st_l[0][l32];
+#pragma unroll
+  for (int w = 1; w < NWV; ++w) bl += st_l[w][l32];
+  i32x4 pb[NWV][2], vf[NWV][2];
+#pragma unroll
+  for (int j = 0; j < NWV; ++j)
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      pb[j][s] = pt[j][s][lane];
+      vf[j][s] = *(const i32x4*)(vs + (32 * wave + l32) * VPITCH + (32 * j + 16 * s + 8 * half) * 2);
+    }
+  f32x16 o;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) o[i] = 0.f;
+#pragma unroll
+  for (int j = 0; j < NWV; ++j)
+#pragma unroll
+    for (int s = 0; s < 2; ++s) o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[j][s]), as_bf16x8(pb[j][s]), o, 0, 0, 0);
+
+  // this lane's output: query qi, columns 32w + 8g4 + 4*half + 0..3 for the four register groups g4
+  if (q_ok) {
+    u16* op = a.out + (size_t)qi * a.out_sm + (size_t)h * D + 32 * wave + 4 * half;
+    const float inv = 1.0f / bl;
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      const f32x4 v = {o[4 * g4], o[4 * g4 + 1], o[4 * g4 + 2], o[4 * g4 + 3]};
+      *(i32x2*)(op + 8 * g4) = pack_bf16x4(v * inv);
+    }
+  }
+}
+
+template <int NWV>
+int launch_px(const AttnArgs& a, hipStream_t st) {
+  hipLaunchKernelGGL((expert_attn_px_kernel<64, NWV>), dim3(a.H, (a.M + 31) / 32), dim3(NWV * 64), 0, st, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+}  // namespace
+
+int tk_attn_px_max_tiles() { return 12; }
+
+// head size 64, bf16 K/V (no hi/lo planes), no per-(query, key) mask, one problem, at most 12 key tiles
+int tk_launch_attn_px(AttnArgs a, int D, hipStream_t st) {
+  const int nt = (a.P + 31) / 32 + (a.S + 31) / 32;
+  if (D != 64 || a.k_pre_lo || a.mask2d || a.batch > 0 || nt < 1 || nt > 12) return -1;
+  if (nt <= 4) return launch_px<4>(a, st);
+  if (nt <= 8) return launch_px<8>(a, st);
+  return launch_px<12>(a, st);
+}

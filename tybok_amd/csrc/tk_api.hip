@@ -546,10 +546,13 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
     d256 = true;
     splits = sp;
   }
+  // 64-wide heads, whole key range in one block (the SmolVLA self layers)
+  const bool px = D == 64 && !split && !mask2d && batch == 0 && ntiles <= tk_attn_px_max_tiles();
+  if (px) splits = 1;
 #ifdef TK_PHASE_TIMING
   if (const char* ev = getenv("TK_ATTN_SPLITS")) {  // development aid, never in the shipped build
     const int v = atoi(ev);
-    if (v >= 1 && v <= 8 && D == 256 && !d256) splits = v;
+    if (v >= 1 && v <= 8 && D == 256 && !d256 && !px) splits = v;
   }
 #endif
   a.kv_splits = splits;
@@ -567,7 +570,7 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
     a.partial = (float*)((char*)ws + kPartialOff);
     a.counters = (int*)ws;
   }
-  int rc = d256 ? tk_launch_attn_d256(a, (hipStream_t)stream) : tk_launch_attn(a, D, waves, (hipStream_t)stream);
+  int rc = d256 ? tk_launch_attn_d256(a, (hipStream_t)stream) : px ? tk_launch_attn_px(a, D, (hipStream_t)stream) : tk_launch_attn(a, D, waves, (hipStream_t)stream);
   if (rc) return fail(TK_ELAUNCH, "attn: launch failed (%s)", hipGetErrorString(hipGetLastError()));
   return TK_OK;
 }

@@ -208,5 +208,9 @@ int tk_launch_attn(AttnArgs a, int D, int waves, hipStream_t st);
 int tk_launch_attn_d256(AttnArgs a, hipStream_t st);
 int tk_attn_d256_max_splits();
 int tk_attn_d256_tiles_per_block();
+// 64-wide heads, whole key range (at most tk_attn_px_max_tiles() tiles) in one block: probabilities exchanged
+// between the waves instead of partial outputs
+int tk_launch_attn_px(AttnArgs a, int D, hipStream_t st);
+int tk_attn_px_max_tiles();
 int tk_launch_attn_qproj(AttnArgs a, hipStream_t st);
 int tk_launch_kv_prepare(KvPrepArgs p, hipStream_t st);
