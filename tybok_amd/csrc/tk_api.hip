@@ -636,7 +636,7 @@ int tk_expert_cross_attn_fused(const void* x, int ldx, const void* norm_w, float
   a.qp_cos = (const float*)rope_cos;
   a.qp_sin = (const float*)rope_sin;
   a.qp_positions = rope_positions;
-  if (tk_launch_attn_qproj(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "cross_attn_fused: launch failed (%s)", hipGetErrorString(hipGetLastError()));
+  if (tk_launch_attn_cross_px(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "cross_attn_fused: launch failed (%s)", hipGetErrorString(hipGetLastError()));
   return TK_OK;
 }
 
