@@ -13,6 +13,7 @@
 namespace {
 
 constexpr int kThreads = 256;
+constexpr int kHeld = 32;  // weight pieces per thread held in registers (K = 1024 with 32 outputs)
 
 __global__ __launch_bounds__(kThreads) void expert_tail_kernel(TailArgs a) {
   extern __shared__ __align__(16) float hrow[];  // [K] normalised row, as fp32 values of bf16 numbers
@@ -21,6 +22,26 @@ __global__ __launch_bounds__(kThreads) void expert_tail_kernel(TailArgs a) {
   const int m = blockIdx.x;
   const int tid = threadIdx.x;
   const u16* x = a.x + (size_t)m * a.ldx;
+
+  // thread -> (output n, k slice): slices of an output are consecutive threads
+  const int slices = kThreads / a.N;  // host guarantees N divides kThreads and N <= kThreads
+  const int n = tid / slices, sl = tid % slices;
+  const float* w = a.w + (size_t)n * a.K;
+  const int pieces = a.K / 4;  // 16-byte pieces of a weight row (K is a multiple of 4: checked by the host)
+  // The weights, the bias and x_t depend on nothing computed here: requested before the row statistics,
+  // they arrive during the first round trip instead of starting three more after it.  The slices of an
+  // output read consecutive pieces; the first kHeld pieces of a thread are held in registers.
+  f32x4 wreg[kHeld];
+#pragma unroll
+  for (int i = 0; i < kHeld; ++i) {
+    const int p = sl + i * slices;
+    const f32x4 wv = *(const f32x4*)(w + 4 * (p < pieces ? p : 0));
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    wreg[i] = p < pieces ? wv : zero;
+  }
+  const size_t oidx = (size_t)m * a.N + n;
+  const float bias_n = a.bias ? a.bias[n] : 0.f;
+  const float xt_n = a.x_out ? a.x_t[oidx] : 0.f;
 
   float ss = 0.f;
   for (int k = tid; k < a.K; k += kThreads) {
@@ -50,16 +71,18 @@ __global__ __launch_bounds__(kThreads) void expert_tail_kernel(TailArgs a) {
   }
   __syncthreads();
 
-  // thread -> (output n, k slice): slices of an output are consecutive threads
-  const int slices = kThreads / a.N;  // host guarantees N divides kThreads and N <= kThreads
-  const int n = tid / slices, sl = tid % slices;
-  const float* w = a.w + (size_t)n * a.K;
-  // 16-byte pieces: the slices of an output read consecutive pieces, each thread several in flight
-  // (K is a multiple of 4: checked by the host)
   float acc0 = 0.f, acc1 = 0.f;
-  const int pieces = a.K / 4;
+#pragma unroll
+  for (int i = 0; i < kHeld; ++i) {
+    const int p = sl + i * slices;
+    const f32x4 hv = *(const f32x4*)(hrow + 4 * (p < pieces ? p : 0));  // (a piece past the row meets zero weights)
+    acc0 = fmaf(hv[0], wreg[i][0], acc0);
+    acc1 = fmaf(hv[1], wreg[i][1], acc1);
+    acc0 = fmaf(hv[2], wreg[i][2], acc0);
+    acc1 = fmaf(hv[3], wreg[i][3], acc1);
+  }
 #pragma unroll 8
-  for (int p = sl; p < pieces; p += slices) {
+  for (int p = sl + kHeld * slices; p < pieces; p += slices) {  // rows wider than the held pieces cover
     const f32x4 wv = *(const f32x4*)(w + 4 * p);
     const f32x4 hv = *(const f32x4*)(hrow + 4 * p);
     acc0 = fmaf(hv[0], wv[0], acc0);
@@ -72,9 +95,9 @@ __global__ __launch_bounds__(kThreads) void expert_tail_kernel(TailArgs a) {
   if (sl == 0) {
     float v = 0.f;
     for (int j = 0; j < slices; ++j) v += part[tid + j];
-    if (a.bias) v += a.bias[n];
-    if (a.v_out) a.v_out[(size_t)m * a.N + n] = v;
-    if (a.x_out) a.x_out[(size_t)m * a.N + n] = add_rn(a.x_t[(size_t)m * a.N + n], mul_rn(a.dt, v));
+    if (a.bias) v += bias_n;
+    if (a.v_out) a.v_out[oidx] = v;
+    if (a.x_out) a.x_out[oidx] = add_rn(xt_n, mul_rn(a.dt, v));
   }
 }
 
