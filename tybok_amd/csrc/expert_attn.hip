@@ -60,21 +60,7 @@ __device__ __forceinline__ bf16x8 pack_bf16x8(const float* v) {
 // NWV waves per block, one 32-key tile each per pass.  With few key tiles (the action expert:
 // 8-10) a block of 8 or 12 waves covers the whole key range, so the waves merge through LDS only and
 // the global partial hand-off between kv splits (two more round trips) is not needed.
-//
-// QPROJ (cross layers of the action expert): the block computes its own query tile first --
-// RMSNorm of the 32 hidden rows, projection with this head's 64 columns of the packed bf16 q weight
-// (k tiles dealt to the waves, fixed-order reduction through LDS), rotary embedding -- and leaves it
-// in LDS for Q.K^T, while the loads of the first key tiles are already in flight.  One launch and
-// one round trip less per layer than projecting first and attending afterwards.
-__device__ __forceinline__ void lds_only_barrier() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-constexpr int kQpMaxK = 768;  // widest hidden size the in-kernel projection stages (SmolVLA expert: 720)
-
-template <int D, bool SPLIT, int NWV, bool QPROJ = false>
+template <int D, bool SPLIT, int NWV>
 __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   constexpr int kNW = NWV;
   constexpr int DT = D / 32;                 // d tiles of the output
@@ -83,14 +69,11 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   constexpr int PF = (NWV > 4 || D > 128) ? 1 : 2;  // key tiles in flight per wave
   // D = 256: the query tile (the same for every wave of the block) lives in LDS instead of 64
   // registers per lane -- with it in registers the kernel spills to scratch
-  constexpr bool QLDS = D >= 256 || QPROJ;
+  constexpr bool QLDS = D >= 256;
   constexpr int QPITCH = D * 2 + 16;         // bytes; 16-byte operand reads of 32 rows stay conflict-free
   __shared__ __align__(16) f32x4 red[DT][kNW][4][64];  // every wave's partial output tiles, exchanged at once
   __shared__ float st_m[kNW][32], st_l[kNW][32];
   __shared__ __align__(16) unsigned char qs[QLDS ? 32 * QPITCH : 16];
-  constexpr int XPITCH = kQpMaxK * 2 + 16;   // staged hidden rows (bf16): conflict-free 16-byte operand reads
-  __shared__ __align__(16) unsigned char xs[QPROJ ? 32 * XPITCH : 16];
-  static_assert(!QPROJ || D == 64, "the in-kernel projection is built for 64-wide heads (two 32-column tiles = one rotary pair)");
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keeps tile indices scalar
@@ -174,115 +157,8 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   // ---- Q as B operand, resident in registers (or LDS); the first tiles' loads go out with it ----
   bf16x8 qf[QLDS ? 1 : DS];
   Stage stg[PF];
-  if (QPROJ) {
-#pragma unroll
-    for (int p = 0; p < PF; ++p) load(stg[p], tile_of(p));
-    // this wave's weight tiles of the head's strip (packed n tiles 2h, 2h+1): k tiles wave, wave + kNW, ...
-    constexpr int KPW = (kQpMaxK / 32 + kNW - 1) / kNW;
-    const uint8_t* wq = a.qp_w + ((size_t)(2 * h) * a.qp_KT) * 2048 + lane * 16;
-    i32x4 wfr[KPW][2][2];
-#pragma unroll
-    for (int i = 0; i < KPW; ++i) {
-      int kt = wave + kNW * i;
-      if (kt > a.qp_KT - 1) kt = a.qp_KT - 1;
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int c = 0; c < 2; ++c) wfr[i][nt][c] = *(const i32x4*)(wq + ((size_t)nt * a.qp_KT + kt) * 2048 + c * 1024);
-    }
-    // 1 / rms of the block's 32 hidden rows: TPR threads per row
-    constexpr int TPR = kNW * 2;
-    const int xr = threadIdx.x / TPR, xq = threadIdx.x % TPR;
-    const int xm = mtile * 32 + xr;
-    const u16* xrow = a.qp_x + (size_t)(xm < a.M ? xm : a.M - 1) * a.qp_ldx;
-    const int npieces = a.qp_K / 8;
-    float ss0 = 0.f, ss1 = 0.f;
-    for (int p = xq; p < npieces; p += TPR) {
-      union { i32x4 v; bf16x2 hh[4]; } xu;
-      xu.v = *(const i32x4*)(xrow + 8 * p);
-      ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[0], xu.hh[0], ss0, false);
-      ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[1], xu.hh[1], ss1, false);
-      ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[2], xu.hh[2], ss0, false);
-      ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[3], xu.hh[3], ss1, false);
-    }
-    float ss = ss0 + ss1;
-#pragma unroll
-    for (int o2 = TPR / 2; o2 > 0; o2 >>= 1) ss += __shfl_xor(ss, o2);
-    const float rstd = rsqrtf(ss / (float)a.qp_K + a.qp_eps);
-    // normalised rows into LDS as bf16(w * bf16(x * rstd)); columns from K to the end of the last k tile are zero
-    const int kpieces = a.qp_KT * 4;
-    for (int p = xq; p < kpieces; p += TPR) {
-      union { i32x4 v; unsigned u[4]; } xu, nw, o4;
-      o4.v = i32x4{0, 0, 0, 0};
-      if (p < npieces) {
-        xu.v = *(const i32x4*)(xrow + 8 * p);
-        nw.v = *(const i32x4*)(a.qp_norm_w + 8 * p);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const unsigned u = pack_bf16x2(__uint_as_float(xu.u[e] << 16) * rstd, __uint_as_float(xu.u[e] & 0xffff0000u) * rstd);
-          o4.u[e] = pack_bf16x2(__uint_as_float(nw.u[e] << 16) * __uint_as_float(u << 16),
-                                __uint_as_float(nw.u[e] & 0xffff0000u) * __uint_as_float(u & 0xffff0000u));
-        }
-      }
-      *(i32x4*)(xs + xr * XPITCH + p * 16) = o4.v;
-    }
-    lds_only_barrier();
-    f32x16 qacc[2];
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) qacc[nt][i] = 0.f;
-#pragma unroll
-    for (int i = 0; i < KPW; ++i) {
-      const int kt = wave + kNW * i;
-      if (kt < a.qp_KT) {  // wave-uniform
-        const i32x4* xp = (const i32x4*)(xs + l32 * XPITCH + (kt * 32 + 16 * half) * 2);
-        const i32x4 xa0 = xp[0], xa1 = xp[1];
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-          qacc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(wfr[i][nt][0]), as_bf16x8(xa0), qacc[nt], 0, 0, 0);
-          qacc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(wfr[i][nt][1]), as_bf16x8(xa1), qacc[nt], 0, 0, 0);
-        }
-      }
-    }
-    // fixed-order reduction over the waves; waves 0..3 own register group w (query row l32, four
-    // consecutive columns 8w + 4*half .. of both tiles = a rotary pair (c, c + 32))
-    static_assert(!QPROJ || DT == 2, "the wave exchange buffer holds two tiles");
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int gq = 0; gq < 4; ++gq) {
-        f32x4 v = {qacc[nt][4 * gq], qacc[nt][4 * gq + 1], qacc[nt][4 * gq + 2], qacc[nt][4 * gq + 3]};
-        red[QPROJ ? nt : 0][wave][gq][lane] = v;
-      }
-    lds_only_barrier();
-    if (wave < 4) {
-      f32x4 sum[2];
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
-        sum[nt] = red[QPROJ ? nt : 0][0][wave][lane];
-#pragma unroll
-        for (int w = 1; w < kNW; ++w) sum[nt] += red[QPROJ ? nt : 0][w][wave][lane];
-      }
-      const int fi = 8 * wave + 4 * half;  // first of this lane's four columns within the half head
-      int pos = a.qp_rope_pos[qi < a.M ? qi : a.M - 1];
-      pos = pos < 0 ? 0 : (pos > a.qp_positions - 1 ? a.qp_positions - 1 : pos);
-      const f32x4 cs = *(const f32x4*)(a.qp_cos + (size_t)pos * (D / 2) + fi);
-      const f32x4 sn = *(const f32x4*)(a.qp_sin + (size_t)pos * (D / 2) + fi);
-      const f32x4 va = unpack_bf16x4(pack_bf16x4(sum[0])), vb = unpack_bf16x4(pack_bf16x4(sum[1]));
-      f32x4 ra, rb;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // separately rounded products, as an elementwise fp32 implementation computes them
-        ra[j] = sub_rn(mul_rn(va[j], cs[j]), mul_rn(vb[j], sn[j]));
-        rb[j] = add_rn(mul_rn(vb[j], cs[j]), mul_rn(va[j], sn[j]));
-      }
-      *(i32x2*)(qs + l32 * QPITCH + fi * 2) = pack_bf16x4(ra);
-      *(i32x2*)(qs + l32 * QPITCH + (D / 2 + fi) * 2) = pack_bf16x4(rb);
-    }
-    lds_only_barrier();  // q tile complete; `red` is free again for the merge below
-  } else {
-  constexpr int QPT = (QLDS && !QPROJ) ? 32 * (D / 8) / (kNW * 64) : 1;  // 16-byte pieces of the query tile per thread
+  {
+  constexpr int QPT = QLDS ? 32 * (D / 8) / (kNW * 64) : 1;  // 16-byte pieces of the query tile per thread
   i32x4 qraw[QPT];
   if (QLDS) {
 #pragma unroll
@@ -647,18 +523,7 @@ int launch_attn(const AttnArgs& a, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
-int launch_attn_q(const AttnArgs& a, hipStream_t st) {
-  dim3 grid(a.H, (a.M + 31) / 32, 1);
-  hipLaunchKernelGGL((expert_attn_kernel<64, true, 8, true>), grid, dim3(8 * 64), 0, st, a);
-  return hipGetLastError() == hipSuccess ? 0 : -3;
-}
-
 }  // namespace
-
-int tk_launch_attn_qproj(AttnArgs a, hipStream_t st) {
-  // cross layers: fp32 (hi + lo) prefix K/V, head size 64, the whole key range in one block of 8 waves
-  return launch_attn_q(a, st);
-}
 
 int tk_attn_waves(int D, int split_planes, int ntiles) {
   // a block of 8 or 12 waves when that covers every key tile (D = 64 only: register budget)

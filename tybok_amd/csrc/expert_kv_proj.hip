@@ -19,7 +19,7 @@
 
 namespace {
 
-constexpr int JB = 5;  // k steps (of 16 input columns) whose loads are in flight together
+constexpr int JB = 10;  // k steps (of 16 input columns) whose loads are in flight together (KV = 320: two batches)
 
 __global__ __launch_bounds__(256) void expert_kv_proj_kernel(KvProjArgs a) {
   const int lane = threadIdx.x & 63;

@@ -213,5 +213,4 @@ int tk_attn_d256_tiles_per_block();
 int tk_launch_attn_px(AttnArgs a, int D, hipStream_t st);
 int tk_attn_px_max_tiles();
 int tk_launch_attn_cross_px(AttnArgs a, hipStream_t st);
-int tk_launch_attn_qproj(AttnArgs a, hipStream_t st);
 int tk_launch_kv_prepare(KvPrepArgs p, hipStream_t st);
