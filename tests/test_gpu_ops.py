@@ -403,3 +403,20 @@ def test_linear_gelu_tanh_is_the_tanh_form_of_the_two_launch_op(tk, m, k, n):
         err_erf = (got.cpu().double() - torch.nn.functional.gelu(z))[sel]
         # the two forms differ by 2.2e-5 on average over this range; rounding noise averages out
         assert abs(float(err_tanh.mean())) < 6e-6 < abs(float(err_erf.mean()))
+
+
+@pytest.mark.parametrize("h,g,d,mode", [(15, 5, 64, oops.MASK_CAUSAL), (8, 1, 256, oops.MASK_BIDIR), (4, 2, 128, oops.MASK_CAUSAL)])
+def test_attention_over_the_suffix_alone_and_with_whole_key_tiles_masked(tk, h, g, d, mode):
+    # no prefix at all (the first tile is then a suffix tile), and a prefix whose pad mask removes two whole
+    # 32-key tiles plus a ragged remainder: a masked tile must contribute exactly nothing
+    q, k_pre, v_pre, k_suf, v_suf = attn_case(50, 200, h, g, d, seed=9)
+    bl = d == 256
+    want = oops.expert_attention(q, k_pre[:0], v_pre[:0], k_suf, v_suf, torch.ones(0, dtype=torch.bool), mode, bf16_logits=bl)
+    got = tk.expert_attn_plain(q.cuda(), None, None, k_suf.cuda(), v_suf.cuda(), None, mode, logits_bf16=bl)
+    _close(got, want, f"suffix-only attention D={d}")
+    pad = torch.ones(200, dtype=torch.bool)
+    pad[32:96] = False
+    pad[190:] = False
+    want = oops.expert_attention(q, k_pre, v_pre, k_suf, v_suf, pad, mode, bf16_logits=bl)
+    got = tk.expert_attn_plain(q.cuda(), k_pre.cuda(), v_pre.cuda(), k_suf.cuda(), v_suf.cuda(), pad.cuda(), mode, logits_bf16=bl)
+    _close(got, want, f"attention with whole key tiles masked D={d}")
