@@ -93,10 +93,16 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_px_kernel(AttnArgs a) {
     }
   }
   // per-key visibility of the prefix (always requested, from a harmless address when unused)
-  const bool use_pad = pre && a.pad != nullptr;
+  const bool use_pad = pre && a.mask2d == nullptr && a.pad != nullptr;
   const int key = tt * 32 + l32;
   const int padv = *((use_pad && key < a.P) ? a.pad + key : (const uint8_t*)a.q);
   const int pad_ok = use_pad ? (key < a.P ? padv : 0) : 1;
+  // per-(query, key) visibility bytes of the tile (prefill): eight consecutive keys per word, the keys of
+  // this lane's registers 0..7 and 8..15
+  const bool use_m2 = pre && a.mask2d != nullptr;
+  const uint8_t* mp = use_m2 ? a.mask2d + (size_t)(q_ok ? qi : a.M - 1) * a.mask_ld + tt * 32 + 8 * half : (const uint8_t*)a.q;
+  const unsigned long long m2lo = *(const unsigned long long*)mp;
+  const unsigned long long m2hi = *(const unsigned long long*)(mp + (use_m2 ? 16 : 8));
   // V^T: D rows x (NWV key tiles x 4 chunks), dealt to all threads; tiles past the range read a valid
   // tile (their P^T is zero)
 #pragma unroll
@@ -154,6 +160,10 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_px_kernel(AttnArgs a) {
         const unsigned ch = c >= 24 ? 0xffu : (c > 16 ? (1u << (c - 16)) - 1u : 0u);
         vbits = cl | (ch << 8);
       }
+    } else if (a.mask2d) {
+      // one byte (0 or 1) per key: gather bit 0 of the 8 bytes of each word
+      const unsigned long long gather = 0x0102040810204080ull, ones = 0x0101010101010101ull;
+      vbits = (unsigned)(((m2lo & ones) * gather) >> 56) | ((unsigned)(((m2hi & ones) * gather) >> 56) << 8);
     } else {
       const unsigned pmask = (unsigned)__ballot(pad_ok != 0);  // lanes 0..31: keys of this tile
       vbits = ((pmask >> (8 * half)) & 0xffu) | (((pmask >> (16 + 8 * half)) & 0xffu) << 8);
@@ -540,10 +550,10 @@ int launch_px(const AttnArgs& a, hipStream_t st) {
 
 int tk_attn_px_max_tiles() { return 12; }
 
-// head size 64, bf16 K/V (no hi/lo planes), no per-(query, key) mask, one problem, at most 12 key tiles
+// head size 64, bf16 K/V (no hi/lo planes), one problem, at most 12 key tiles
 int tk_launch_attn_px(AttnArgs a, int D, hipStream_t st) {
   const int nt = (a.P + 31) / 32 + (a.S + 31) / 32;
-  if (D != 64 || a.k_pre_lo || a.mask2d || a.batch > 0 || nt < 1 || nt > 12) return -1;
+  if (D != 64 || a.k_pre_lo || a.batch > 0 || nt < 1 || nt > 12) return -1;
   if (nt <= 4) return launch_px<4>(a, st);
   if (nt <= 8) return launch_px<8>(a, st);
   return launch_px<12>(a, st);

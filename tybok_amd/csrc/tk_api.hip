@@ -546,8 +546,8 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
     d256 = true;
     splits = sp;
   }
-  // 64-wide heads, whole key range in one block (the SmolVLA self layers)
-  const bool px = D == 64 && !split && !mask2d && batch == 0 && ntiles <= tk_attn_px_max_tiles();
+  // 64-wide heads, whole key range in one block (the SmolVLA self layers and prefill)
+  const bool px = D == 64 && !split && batch == 0 && ntiles <= tk_attn_px_max_tiles();
   if (px) splits = 1;
 #ifdef TK_PHASE_TIMING
   if (const char* ev = getenv("TK_ATTN_SPLITS")) {  // development aid, never in the shipped build
