@@ -275,6 +275,7 @@ def main() -> None:
     ap.add_argument("--attn-only", action="store_true", help="only the action-expert attention loop (for rocprofv3 runs)")
     ap.add_argument("--tower-attn-only", action="store_true", help="only the vision-tower attention loop, 3 cameras x 1024 tokens (for rocprofv3 runs)")
     ap.add_argument("--ffn-only", action="store_true", help="only the many-row (M=712) fp8 GeGLU FFN loop (for rocprofv3 runs)")
+    ap.add_argument("--request-only", choices=("smolvla", "pi05"), help="only the requests of one model, all tiers, graph replay (for rocprofv3 runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is batch-1 and single-device (--gpus must be 1)")
@@ -316,6 +317,18 @@ def main() -> None:
         return
     flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_fused_attn=True, tl_vit_oproj=True)
     tmp = tempfile.mkdtemp(prefix="tybok_bench_")
+    if args.request_only:
+        if args.request_only == "smolvla":
+            eng = create_engine(write_smolvla_checkpoint(os.path.join(tmp, "smolvla"), cameras=3, seed=0), device="cuda", graph=True, graph_cameras=(3,), warmup=True, **flags)
+            cams, dim = 3, 6
+        else:
+            flags5 = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_flash_attn=True, tl_fused_vit=True)
+            eng = create_engine(write_pi05_checkpoint(os.path.join(tmp, "pi05"), cameras=2, seed=0), device="cuda", graph=True, warmup=True, **flags5)
+            cams, dim = 2, 7
+        spin_up()
+        samples, _ = time_requests(eng, device_frame(eng, cams), torch.zeros(1, 50, dim, device="cuda"), args.steps, args.warmup)
+        print(json.dumps({"request_only": {"model": args.request_only, "cameras": cams, "requests": args.steps, "p50_ms": round(float(np.percentile(samples, 50)), 3)}}), flush=True)
+        return
 
     # ---- SmolVLA-shaped chunk (headline) ----
     ckpt = write_smolvla_checkpoint(os.path.join(tmp, "smolvla"), cameras=3, seed=0)

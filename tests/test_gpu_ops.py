@@ -212,7 +212,7 @@ def test_attention_fully_masked_prefix_is_uniform(tk, h, g, d):
     _close(got, want, "attn fully masked")
 
 
-@pytest.mark.parametrize("p,h,g,d", [(241, 15, 5, 64), (177, 15, 5, 64), (40, 4, 2, 128), (1024, 12, 12, 64), (712, 8, 1, 256), (90, 4, 2, 256), (1000, 16, 2, 256)])
+@pytest.mark.parametrize("p,h,g,d", [(241, 15, 5, 64), (177, 15, 5, 64), (100, 15, 5, 64), (384, 6, 2, 64), (385, 6, 2, 64), (40, 4, 2, 128), (1024, 12, 12, 64), (712, 8, 1, 256), (90, 4, 2, 256), (1000, 16, 2, 256)])
 def test_prefill_attention_with_2d_mask(tk, p, h, g, d):
     # the VLM prefill: every token is a query, keys are the same tokens, visibility from the
     # block-causal 2-D mask (image/language tokens see each other, the state token sees all) & padding
