@@ -52,7 +52,9 @@ __device__ __forceinline__ void lds_barrier() {
 //      bf16 activations: bf16((x * rstd) * (1 + scale[k]) + shift[k]) in fp32 -- applied while the
 //      activations are staged into LDS, with the reference's rounding points:
 //      bf16 input: bf16(w * bf16(x * rstd));  fp32 input: bf16(w * (x * rstd)).
-template <int MT, int NT, int NW, int EPI, int PF, int TPW, bool W16, int PRO>
+//  NR: number of block rounds when the host knows it (every block walks the same number of k tiles), else 0:
+//      with a constant count the pipeline below is straight-line code -- no tail conditions, exact wait counts.
+template <int MT, int NT, int NW, int EPI, int PF, int TPW, bool W16, int PRO, int NR = 0>
 __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   constexpr bool GATED = EPI == 1;
   constexpr bool PAIRED = EPI != 0;  // both n tiles of a pair are finished by the same wave
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   // division: a 64-bit divide here costs some 300 scalar instructions before the first load)
   const int kt_lo = split * a.kt_q + (split < a.kt_r ? split : a.kt_r);
   const int kt_hi = kt_lo + a.kt_q + (split < a.kt_r ? 1 : 0);
-  const int nrounds = (kt_hi - kt_lo + RKT - 1) / RKT;
+  const int nrounds = NR > 0 ? NR : (kt_hi - kt_lo + RKT - 1) / RKT;
   const int k_end = kt_hi * 32 < a.K ? kt_hi * 32 : a.K;  // first activation column this block must not use
 
   // weight tile streams of this wave; a strip may hang over the last n tile: clamp to a valid
@@ -652,10 +654,22 @@ __global__ void decode_fp8_kernel(float* out) {
 #ifndef TK_EXP_TPW
 #define TK_EXP_TPW 1
 #endif
+template <int MT, int NT, int EPI, bool W16, int PRO, int NR>
+int launch_nr(const GemmArgs& a, dim3 grid, hipStream_t st) {
+  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, TK_EXP_PF, TK_EXP_TPW, W16, PRO, NR>), grid, dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
 template <int MT, int NT, int EPI, bool W16, int PRO>
 int launch(const GemmArgs& a, dim3 grid, hipStream_t st) {
-  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, TK_EXP_PF, TK_EXP_TPW, W16, PRO>), grid, dim3(256), 0, st, a);
-  return hipGetLastError() == hipSuccess ? 0 : -3;
+  // the action chunk's launches (32-row blocks, every block the same number of k tiles) at the round counts
+  // of the two models' expert layers: K = 720 -> 6, 960 / 1024 -> 8, 2048 -> 16, 4096 in four splits -> 8
+  if (MT == 1 && a.kt_r == 0) {
+    const int nr = (a.kt_q + 4 * TK_EXP_TPW - 1) / (4 * TK_EXP_TPW);
+    if (nr == 6) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 6 : 0>(a, grid, st);
+    if (nr == 8) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 8 : 0>(a, grid, st);
+    if (nr == 16) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 16 : 0>(a, grid, st);
+  }
+  return launch_nr<MT, NT, EPI, W16, PRO, 0>(a, grid, st);
 }
 
 }  // namespace
