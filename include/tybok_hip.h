@@ -98,6 +98,24 @@ int tk_fp8w_gemm(const void* x, int ldx, const void* w_packed, const void* scale
                  const void* resid, int ldr, int resid_dtype, const void* gate, int M, int N, int K, int split_k,
                  void* ws, size_t ws_bytes, void* stream);
 
+/* tk_fp8w_gemm for callers that cannot allocate or carry a workspace (code under graph capture that
+ * owns no buffers, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference, whose native layer always receives caller-owned scratch.  Arguments and results as
+ * tk_fp8w_gemm (same kernels, same bits), without `ws`: the split-K partials and arrival counters live
+ * in an array inside the library's device image -- tk_static_scratch_bytes() bytes (64 KiB of counters
+ * + 8 MiB of partials) that each GPU the library runs on holds until the process ends.
+ *   Limits: M <= 64 (the action chunk); an explicit split_k whose partials exceed the 8 MiB is
+ *   rejected with TK_EWORKSPACE; split_k = 0 never chooses more than fits.
+ *   The first call on a device looks the array's address up (make it outside stream capture).  No
+ *   call allocates, frees or synchronises.  All calls on one GPU share the one array: calls that
+ *   may overlap in time (two streams, two threads) race -- serialise them or use tk_fp8w_gemm with
+ *   one workspace per stream.  The counters a split launch uses are cleared by a fill kernel
+ *   right before it, so a call does not depend on what the previous one left behind. */
+int tk_fp8w_gemm_static(const void* x, int ldx, const void* w_packed, const void* scale, void* y, int ldy,
+                        const void* resid, int ldr, int resid_dtype, const void* gate, int M, int N, int K,
+                        int split_k, void* stream);
+size_t tk_static_scratch_bytes(void);
+
 /* ---- fused gated FFN ----------------------------------------------------------------------- */
 /* y[M, K] = down( act(gate(x)) * up(x) ) with fp8 weights, bf16 in/out:
  *   g = bf16(x.Wg^T * sg), u = bf16(x.Wu^T * su), h = bf16(bf16(act(g)) * u), y = bf16(h.Wd^T * sd)

@@ -31,6 +31,17 @@ constexpr size_t kHiddenOff = kNormOff + kNormBytes;
 constexpr size_t kHiddenBytes = TK_WS_TOTAL_BYTES - kHiddenOff;  // FFN [M, I] bf16 intermediate
 constexpr int kMaxCounters = (int)(kCounterBytes / 4);
 
+// Scratch of tk_fp8w_gemm_static (callers that cannot allocate): arrival counters followed by split-K
+// partials, the head of the workspace layout above at a modest size.  Every device the library runs on
+// holds its own copy until the process ends.  In host code the array's NAME is only a handle: the
+// device address comes from hipGetSymbolAddress (static_scratch() below), once per device.
+constexpr size_t kStaticPartialBytes = 8ull << 20;
+constexpr size_t kStaticBytes = kCounterBytes + kStaticPartialBytes;
+constexpr int kStaticMaxRows = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` per device ordinal, nullptr = not looked up yet
+
 bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 bool aligned8(const void* p) { return (((uintptr_t)p) & 7) == 0; }
 
@@ -43,6 +54,22 @@ int device_cus() {
     g_cus = n;
   }
   return g_cus;
+}
+
+// Device address of this device's copy of `scratch` (looked up on the first call per device, with that
+// device current; concurrent first calls would store the same value twice).
+int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(TK_ELAUNCH, "static scratch: no current device (or ordinal >= %d)", kMaxDevices);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    const hipError_t rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (rc != hipSuccess || !p) return fail(TK_ELAUNCH, "static scratch: hipGetSymbolAddress failed (%s)", hipGetErrorString(rc));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return TK_OK;
 }
 
 // Optional pieces of a GEMM launch beyond y = bf16((x . W^T) * scale).
@@ -59,6 +86,7 @@ struct GemmExtra {
   int rope_positions = 0, rope_cols = 0, rope_half = 0, rope_bf16 = 0;
   void* vt = nullptr;  // transposed copy of the columns >= vt_col0 (rotary epilogue)
   int vt_col0 = 0, vt_ld = 0;
+  int clear_counters = 0;  // zero the arrival counters a split launch uses right before it (shared static scratch)
 };
 
 // One GEMM launch (plain, gated or rotary).  `N` is the logical output width.
@@ -223,7 +251,9 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
     if (blocks0 < cus) {
       const float per_round = MT == 1 ? (e.w16 && NT == 2 ? 0.27f : 0.20f) : 0.35f;
       float best = 1e30f;
-      for (int c = 1; c <= 64 && c * NW <= a.KT && (c == 1 || blocks0 * c <= 2 * cus); ++c) {
+      // (an automatic choice never asks for more partial space than the workspace holds)
+      const size_t cap = !ws || ws_bytes <= kPartialOff ? 0 : (ws_bytes - kPartialOff < kPartialBytes ? ws_bytes - kPartialOff : kPartialBytes);
+      for (int c = 1; c <= 64 && c * NW <= a.KT && (c == 1 || (blocks0 * c <= 2 * cus && (size_t)blocks0 * c * MT * NT * 4096 <= cap && blocks0 <= kMaxCounters)); ++c) {
         const int rounds = (a.KT + c * NW - 1) / (c * NW);
         float t = rounds * per_round;
         if (t < 1.0f) t = 1.0f;
@@ -249,6 +279,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
       return fail(TK_EWORKSPACE, "gemm: workspace too small (need %zu partial bytes, %d counters)", need, blocks0);
     a.partial = (float*)((char*)ws + kPartialOff);
     a.counters = (int*)ws;
+    if (e.clear_counters && tk_launch_fill_zero(a.counters, blocks0, st)) return fail(TK_ELAUNCH, "gemm: counter fill launch failed");
   }
   int rc = tk_launch_gemm(a, MT, NT, mblocks, st);
   if (rc == -1) return fail(TK_EINVAL, "gemm: this combination of weight type, prologue and epilogue is not built");
@@ -302,6 +333,22 @@ int tk_fp8w_gemm(const void* x, int ldx, const void* w_packed, const void* scale
   return gemm_common(x, ldx, w_packed, (const float*)scale, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, N, K,
                      split_k, 0, ws, ws_bytes, (hipStream_t)stream);
 }
+
+int tk_fp8w_gemm_static(const void* x, int ldx, const void* w_packed, const void* scale, void* y, int ldy,
+                        const void* resid, int ldr, int resid_dtype, const void* gate, int M, int N, int K, int split_k,
+                        void* stream) {
+  if (M > kStaticMaxRows)
+    return fail(TK_EINVAL, "gemm_static: M=%d exceeds the %d rows this entry point is built for (use tk_fp8w_gemm with a workspace)",
+                M, kStaticMaxRows);
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  GemmExtra e;
+  e.clear_counters = 1;
+  return gemm_common(x, ldx, w_packed, (const float*)scale, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, N, K, split_k,
+                     0, ws, kStaticBytes, (hipStream_t)stream, e);
+}
+
+size_t tk_static_scratch_bytes(void) { return kStaticBytes; }
 
 int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void* sg, const void* su,
                       const void* wd_packed, const void* sd, void* y, int ldy, const void* resid, int ldr,

@@ -32,6 +32,12 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
          c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
+    "tk_fp8w_gemm_static": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
+         c_int, c_void_p],
+    ),  # fmt: skip
+    "tk_static_scratch_bytes": (c_size_t, []),
     "tk_fp8w_gated_ffn": (
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
