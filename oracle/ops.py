@@ -17,7 +17,7 @@ BF16 = torch.bfloat16
 # --------------------------------------------------------------------------- #
 # fp8-weight linear and gated FFN
 # --------------------------------------------------------------------------- #
-def lin_fp8w(x: torch.Tensor, w8: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+def lin_fp8w(x: torch.Tensor, w8: torch.Tensor, scale: torch.Tensor, out_dtype: torch.dtype = BF16) -> torch.Tensor:
     """``bf16((x.float() @ W8.float().T) * scale[None, :])`` -- weight-only fp8 linear.
 
     The per-output-channel scale multiplies the fp32 accumulator, as every fp8 kernel of the
@@ -25,7 +25,7 @@ def lin_fp8w(x: torch.Tensor, w8: torch.Tensor, scale: torch.Tensor) -> torch.Te
     tybok/policies/fastwam/models/fp8_linear.py:70); activations stay bf16 (no ``a_scale``).
     """
     acc = x.float() @ w8.float().t()
-    return (acc * scale.float()[None, :]).to(BF16)
+    return (acc * scale.float()[None, :]).to(out_dtype)
 
 
 def lin_fp8w_f64(x: torch.Tensor, w8: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:

@@ -120,7 +120,7 @@ def embed_prefix(w: Weights, shape: PI05Shape, images, img_masks, tokens, masks)
         embs.append(e)
         pads.append(m[:, None].expand(e.shape[0], e.shape[1]))
     lang = F.embedding(tokens, w[VLM + "embed_tokens.weight"])
-    lang = lang * torch.tensor(shape.vlm_width**0.5, dtype=lang.dtype)  # bf16-rounded sqrt(width)
+    lang = lang * torch.tensor(shape.vlm_width**0.5, dtype=BF16).to(lang.dtype)  # bf16-rounded sqrt(width)
     embs.append(lang)
     pads.append(masks)
     embs = torch.cat(embs, dim=1)
@@ -152,7 +152,7 @@ def prefill(w: Weights, shape: PI05Shape, embs, pad_masks, att_masks):
     mask = ops.make_att_2d_masks(pad_masks, att_masks)
     add = torch.where(mask[:, None], 0.0, ops.OPENPI_MASK_VALUE)
     pos = torch.cumsum(pad_masks, dim=1) - 1
-    hidden = embs.to(BF16)
+    hidden = embs.to(w.act_dtype)
     cos, sin = ops.gemma_rope_cos_sin(shape.head_dim, pos, hidden.dtype)
     kv = []
     for i in range(shape.depth):
@@ -176,7 +176,7 @@ def adarms_cond(w: Weights, shape: PI05Shape, time: float) -> torch.Tensor:
 def denoise_step(w: Weights, shape: PI05Shape, prefix_pad, kv, x_t, time: float):
     """One velocity evaluation fp32 ``[1, chunk, max_action_dim]`` (flow_matching.py:505-556)."""
     cond = adarms_cond(w, shape, time)
-    hidden = w.linear("action_in_proj", x_t).to(BF16)
+    hidden = w.linear("action_in_proj", x_t).to(w.act_dtype)
     s = hidden.shape[1]
     mask = ops.suffix_mask(prefix_pad[0], s, s, ops.MASK_BIDIR)
     add = torch.where(mask[:, None], 0.0, ops.OPENPI_MASK_VALUE)

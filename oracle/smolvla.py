@@ -87,6 +87,16 @@ class Weights:
     sd: dict
     fp8_names: frozenset = frozenset()
     _q: dict = field(default_factory=dict)
+    # bf16 = the reference's dtypes.  float32 = the same weight VALUES (bf16-rounded, fp8 codes) with every
+    # activation kept in fp32: the yardstick that tells rounding noise of a bf16 execution order from error.
+    act_dtype: torch.dtype = BF16
+
+    def __post_init__(self):
+        if self.act_dtype != BF16:
+            self.sd_quant = self.sd  # quantisation starts from the stored (bf16) weights in either mode
+            self.sd = {k: (v.to(self.act_dtype) if v.is_floating_point() else v) for k, v in self.sd.items()}
+        else:
+            self.sd_quant = self.sd
 
     def __getitem__(self, name: str) -> torch.Tensor:
         return self.sd[name]
@@ -98,9 +108,9 @@ class Weights:
         if prefix in self.fp8_names:
             q = self._q.get(prefix)
             if q is None:
-                q = ofp8.quantize_weight_rows(w)
+                q = ofp8.quantize_weight_rows(self.sd_quant[prefix + ".weight"])
                 self._q[prefix] = q
-            y = ops.lin_fp8w(x.reshape(-1, x.shape[-1]), q[0], q[1]).reshape(*x.shape[:-1], w.shape[0])
+            y = ops.lin_fp8w(x.reshape(-1, x.shape[-1]), q[0], q[1], self.act_dtype).reshape(*x.shape[:-1], w.shape[0])
             return y if b is None else y + b
         return F.linear(x, w, b)
 
@@ -137,7 +147,7 @@ def _vision_position_ids(shape: SmolVLAShape, n_h: int, n_w: int) -> torch.Tenso
 
 def embed_image(w: Weights, shape: SmolVLAShape, image: torch.Tensor) -> torch.Tensor:
     """``[1, 3, H, W]`` in [-1, 1] -> ``[1, 64, hidden]`` bf16 (vision.py:197-257)."""
-    x = image.to(BF16)
+    x = image.to(w.act_dtype)
     x = F.conv2d(x, w[VIS + "embeddings.patch_embedding.weight"], w[VIS + "embeddings.patch_embedding.bias"], stride=shape.patch)
     b = x.shape[0]
     n_h, n_w = x.shape[2], x.shape[3]
@@ -181,7 +191,7 @@ def embed_prefix(w: Weights, shape: SmolVLAShape, images, img_masks, lang_tokens
     embs, pads, att = [], [], []
     for img, m in zip(images, img_masks):
         e = embed_image(w, shape, img)
-        e = e * torch.tensor(e.shape[-1] ** 0.5, dtype=e.dtype)  # bf16-rounded sqrt(hidden)
+        e = e * torch.tensor(e.shape[-1] ** 0.5, dtype=BF16).to(e.dtype)  # bf16-rounded sqrt(hidden)
         embs.append(e)
         pads.append(m[:, None].expand(e.shape[0], e.shape[1]))
         att += [0] * e.shape[1]
@@ -202,7 +212,7 @@ def embed_prefix(w: Weights, shape: SmolVLAShape, images, img_masks, lang_tokens
 
 def _layer_tail(w: Weights, shape: SmolVLAShape, prefix: str, att_out: torch.Tensor, hidden: torch.Tensor) -> torch.Tensor:
     """o_proj, first residual (in-place add), post norm, MLP, second residual (vlm_with_expert.py:370-410)."""
-    out = w.linear(prefix + "self_attn.o_proj", att_out.to(BF16))
+    out = w.linear(prefix + "self_attn.o_proj", att_out.to(w.act_dtype))
     out += hidden  # bf16 += (fp32|bf16): fp32 math, bf16 result
     after_first = out.clone()
     h = ops.rms_norm_llama(out, w[prefix + "post_attention_layernorm.weight"], shape.rms_eps)
@@ -222,7 +232,7 @@ def prefill(w: Weights, shape: SmolVLAShape, embs, pad_masks, att_masks):
     b, length = embs.shape[0], embs.shape[1]
     for i in range(shape.num_vlm_layers):
         p = f"{TXT}layers.{i}."
-        h = ops.rms_norm_llama(hidden, w[p + "input_layernorm.weight"], shape.rms_eps).to(BF16)
+        h = ops.rms_norm_llama(hidden, w[p + "input_layernorm.weight"], shape.rms_eps).to(w.act_dtype)
         q = w.linear(p + "self_attn.q_proj", h).view(b, length, -1, shape.head_dim)
         k = w.linear(p + "self_attn.k_proj", h).view(b, length, -1, shape.head_dim)
         v = w.linear(p + "self_attn.v_proj", h).view(b, length, -1, shape.head_dim)
@@ -273,7 +283,7 @@ def denoise_step(w: Weights, shape: SmolVLAShape, prefix_pad, kv, ekv, x_t, time
         p = f"{EXP}layers.{i}."
         h = ops.rms_norm_llama(hidden, w[p + "input_layernorm.weight"], shape.rms_eps)
         if not shape.is_cross(i):
-            h = h.to(BF16)
+            h = h.to(w.act_dtype)
             q = w.linear(p + "self_attn.q_proj", h).view(b, s, -1, shape.head_dim)
             k = w.linear(p + "self_attn.k_proj", h).view(b, s, -1, shape.head_dim)
             v = w.linear(p + "self_attn.v_proj", h).view(b, s, -1, shape.head_dim)
@@ -283,7 +293,7 @@ def denoise_step(w: Weights, shape: SmolVLAShape, prefix_pad, kv, ekv, x_t, time
             vv = torch.cat([kv[i][1], v], dim=1)
             att = ops.eager_attention(full_mask, q, kk, vv)
         else:
-            q = w.linear(p + "self_attn.q_proj", h.to(BF16)).view(b, s, -1, shape.head_dim)
+            q = w.linear(p + "self_attn.q_proj", h.to(w.act_dtype)).view(b, s, -1, shape.head_dim)
             q = ops.rope_half_split(q, pos - pos.min(dim=1, keepdim=True).values)
             att = ops.eager_attention(full_mask[:, :, :p_len], q, ekv[i][0], ekv[i][1])
         hidden = _layer_tail(w, shape, p, att, hidden)

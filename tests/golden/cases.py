@@ -16,6 +16,8 @@ SMOLVLA_CASES = {
 PI05_CASES = {
     # reduced depth: 3 VLM/expert layers, 2 vision layers, 2 cameras, padded language tail, 3 steps
     "small": dict(depth=3, vision_layers=2, cameras=2, num_steps=3, seed=12, noise="randn", lang_pad=60),
+    # full depth (config 5 of the benchmark): 18 + 18 layers, 27 vision layers, 2 cameras, 200 tokens, 10 steps, zero noise
+    "full": dict(depth=18, vision_layers=27, cameras=2, num_steps=10, seed=0, noise="zeros", lang_pad=0),
 }
 
 

@@ -2,7 +2,7 @@
 
 Run ONCE in the build container (the reference is not available elsewhere):
 
-    python tests/golden/make_golden.py [smolvla|pi05|all]
+    python tests/golden/make_golden.py [smolvla|pi05|all] [case]
 
 For each case the reference's eager model classes (``/root/reference/tybok/policies/<model>/models``)
 are constructed on the CPU from plain config dataclasses (no checkpoint, no tokenizer), loaded with
@@ -139,6 +139,8 @@ def pi05_case(name: str) -> dict:
         out["v_t_half"] = v_half[0].float().numpy()
         chunk = model.sample_actions(images, inputs["img_masks"], inputs["lang_tokens"], inputs["lang_masks"], noise=inputs["noise"])
         out["chunk"] = chunk[0].float().numpy()
+    if name == "full":  # full depth: the chunk and the probe velocity only (small fixture)
+        out = {k: out[k] for k in ("chunk", "v_t_half")}
     return out
 
 
@@ -150,7 +152,10 @@ def main() -> None:
         jobs += [("smolvla", n) for n in cases.SMOLVLA_CASES]
     if which in ("pi05", "all"):
         jobs += [("pi05", n) for n in cases.PI05_CASES]
+    only = sys.argv[2] if len(sys.argv) > 2 else None  # optional: one case name
     for model, name in jobs:
+        if only and name != only:
+            continue
         t0 = time.time()
         out = smolvla_case(name) if model == "smolvla" else pi05_case(name)
         path = os.path.join(HERE, f"{model}_{name}.npz")

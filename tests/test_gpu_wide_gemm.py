@@ -121,20 +121,27 @@ def test_many_row_norm_gated_ffn(tk, adaptive):
     assert mism < 0.02, f"fused norm differs from norm-then-FFN on {mism:.1%} of the outputs"
 
 
-def test_prefill_size_ffn_linearity_and_row_independence(tk):
-    # pi0.5 prefill size (M=712, K=2048, I=16384): too slow for the CPU oracle in a unit test, so use
+def test_prefill_size_ffn_matches_oracle_and_rows_are_independent(tk):
+    # pi0.5 prefill size (M=712, K=2048, I=16384; `make_fp8_mlp_forward`,
+    # tybok/policies/pi05/models/triton_prefill_mlp.py:145-166) against the CPU oracle at full size, plus
     # what the mathematics fixes: an output row depends on its own input row only (shuffling the rows
-    # shuffles the result bit-exactly, whatever block / wave / tile a row lands in), and the first 64
-    # rows must match the skinny kernel, which the oracle pins.
+    # shuffles the result bit-exactly, whatever block / wave / tile a row lands in).
     m, k, i = 712, 2048, 16384
     x, wg8, sg, wu8, su, wd8, sd = ffn_case(m, k, i, seed=8)
     wgu = tk.pack_fp8_gate_up(wg8.cuda(), sg, wu8.cuda(), su)
     wd = tk.pack_fp8_weight(wd8.cuda(), sd)
     xc = x.cuda()
     y = tk.fp8w_gated_ffn(xc, wgu, wd, "gelu_tanh")
+    want = oops.gated_ffn(x, wg8, sg, wu8, su, wd8, sd, "gelu_tanh")
+    _close(y, want, "prefill-size ffn (712, 2048, 16384) vs oracle")
+    # the two linears on their own at this size (`w8a8_gemm` shapes, weight-only semantics)
+    g = tk.fp8w_gemm(xc, tk.pack_fp8_weight(wg8.cuda(), sg))
+    _close(g, oops.lin_fp8w(x, wg8, sg), "prefill-size gate projection (712, 2048 -> 16384) vs oracle")
+    h = (oops.act_fn("gelu_tanh", oops.lin_fp8w(x, wg8, sg)) * oops.lin_fp8w(x, wu8, su)).to(BF16)
+    d = tk.fp8w_gemm(h.cuda(), wd)
+    _close(d, oops.lin_fp8w(h, wd8, sd), "prefill-size down projection (712, 16384 -> 2048) vs oracle")
     perm = torch.randperm(m, generator=torch.Generator().manual_seed(9)).cuda()
     yp = tk.fp8w_gated_ffn(xc[perm].contiguous(), wgu, wd, "gelu_tanh")
     assert torch.equal(yp, y[perm]), "rows must not depend on their position in the batch"
     skinny = tk.fp8w_gated_ffn(xc[:64].contiguous(), wgu, wd, "gelu_tanh")
     _close(y[:64], skinny.cpu(), "prefill-size ffn vs skinny kernel rows")
-    assert torch.isfinite(y.float()).all()

@@ -24,7 +24,7 @@ def _maxdiff(a, b) -> float:
     return float(np.abs(np.asarray(a, dtype=np.float64) - np.asarray(b, dtype=np.float64)).max())
 
 
-@pytest.mark.parametrize("name", ["small"])
+@pytest.mark.parametrize("name", ["small", "full"])
 def test_oracle_matches_reference_golden(name):
     gold = np.load(os.path.join(HERE, "golden", f"pi05_{name}.npz"))
     cfg, sd, inp = cases.pi05_build(cases.PI05_CASES[name])
@@ -37,10 +37,11 @@ def test_oracle_matches_reference_golden(name):
         x0 = torch.zeros(1, shape.chunk, shape.max_action_dim)
         v_half = O.denoise_step(w, shape, trace["pad_masks"], trace["kv"], x0, 0.5)
     embs = trace["prefix_embs"]
-    assert _maxdiff(embs[0, :4].float().numpy(), gold["prefix_embs_head"]) <= 1e-6
-    assert _maxdiff(embs[0, -8:, :64].float().numpy(), gold["prefix_embs_tail"]) == 0.0
-    assert _maxdiff(trace["kv"][0][0][0, 0, ::32].float().numpy(), gold["k_first"]) <= 1e-6
-    assert _maxdiff(trace["kv"][-1][1][0, 0, ::32].float().numpy(), gold["v_last"]) <= 1e-6
+    if "prefix_embs_head" in gold:  # the full-depth fixture stores the chunk and the probe velocity only
+        assert _maxdiff(embs[0, :4].float().numpy(), gold["prefix_embs_head"]) <= 1e-6
+        assert _maxdiff(embs[0, -8:, :64].float().numpy(), gold["prefix_embs_tail"]) == 0.0
+        assert _maxdiff(trace["kv"][0][0][0, 0, ::32].float().numpy(), gold["k_first"]) <= 1e-6
+        assert _maxdiff(trace["kv"][-1][1][0, 0, ::32].float().numpy(), gold["v_last"]) <= 1e-6
     assert _maxdiff(v_half[0].numpy(), gold["v_t_half"]) <= 1e-5
     assert _maxdiff(chunk[0].numpy(), gold["chunk"]) <= 1e-5
     assert float(np.abs(gold["chunk"]).max()) > 0.1
