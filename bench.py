@@ -88,6 +88,46 @@ def gemm_launch_us(m: int, k: int, n: int, launches: int = 100, reps: int = 10, 
     return e0.elapsed_time(e1) * 1e3 / (reps * launches)
 
 
+def stream_read_us(window_bytes: int, blocks: int = 1024, launches: int = 100, reps: int = 10) -> float:
+    """Average duration (us) of one plain streaming read of ``window_bytes`` (16 bytes per lane, nothing
+    computed) inside a replayed graph whose launches rotate through > 1 GB of distinct windows: what one
+    dependent launch of a weight-streaming GEMM's size can pull from cold HBM on this device."""
+    import torch
+
+    from tybok_amd import native
+
+    lib = native.lib()
+    window_bytes -= window_bytes % (blocks * 4096)
+    copies = max(2, int(1.1e9 // window_bytes))
+    buf = torch.full((copies * window_bytes,), 1, dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.Stream()
+
+    def launch(i: int) -> None:
+        rc = lib.tk_debug_stream_read(buf.data_ptr() + (i % copies) * window_bytes, window_bytes, blocks, sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        native.check(rc, "tk_debug_stream_read")
+
+    with torch.cuda.stream(stream):
+        for i in range(3):
+            launch(i)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
+        for i in range(launches):
+            launch(i)
+    spin_up(60.0)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * launches)
+
+
 def ffn_launch_us(m: int, k: int, i: int, launches: int = 10, reps: int = 5) -> float:
     """Average duration (us) of one fp8-weight GeGLU FFN (gate/up + down) at many rows: the VLM prefill shape."""
     import torch
@@ -297,7 +337,9 @@ def main() -> None:
         spin_up()
         gm, gk, gn = args.gemm_shape
         us = gemm_launch_us(gm, gk, gn, launches=20, reps=args.steps)
-        print(json.dumps({"gemm_only": {"M": gm, "K": gk, "N": gn, "us": round(us, 2), "GBps": round(bytes_gemm(gm, gk, gn) / us / 1e3, 1)}}), flush=True)
+        sc = stream_read_us(gk * gn, launches=20, reps=args.steps)
+        print(json.dumps({"gemm_only": {"M": gm, "K": gk, "N": gn, "us": round(us, 2), "GBps": round(bytes_gemm(gm, gk, gn) / us / 1e3, 1),
+                                        "stream_read_us": round(sc, 2), "stream_read_GBps": round(gk * gn / sc / 1e3, 1)}}), flush=True)  # fmt: skip
         return
     if args.ffn_only:
         spin_up()
@@ -379,6 +421,20 @@ def main() -> None:
         "bytes_per_launch": bytes_gemm(50, rk, rn),
         "us_per_launch": r_us,
     }
+    # the box's own ceiling for one dependent launch of this size: a plain streaming read of a cold window
+    # as large as the GEMM's weight matrix, timed the same way
+    sc_us = stream_read_us(rk * rn)
+    sc_gbps = rk * rn / sc_us / 1e3
+    roofline["stream_ceiling"] = {
+        "what": "plain 16-byte-per-lane read of a cold 32 MiB window per launch, graph of back-to-back launches",
+        "us_per_launch": round(sc_us, 2),
+        "GBps": round(sc_gbps, 1),
+        "frac_of_peak": round(sc_gbps / HBM_PEAK_GBS, 4),
+    }
+    roofline["frac_of_stream_ceiling"] = round(achieved / sc_gbps, 4)
+    k2, n2 = 16384, 2048
+    a2 = sweep[f"K{k2}_N{n2}"]["GBps"]
+    roofline["other_33MB_shape"] = {"kernel": "fp8w_gemm_kernel (M=50, K=16384, N=2048, cold weights)", "achieved": a2, "frac": round(a2 / HBM_PEAK_GBS, 4), "frac_of_stream_ceiling": round(a2 / sc_gbps, 4)}
     traffic_file = os.path.join(ROOT, "profiles", "fp8w_gemm_traffic.json")
     if os.path.exists(traffic_file):
         with open(traffic_file, encoding="utf-8") as f:

@@ -343,6 +343,12 @@ int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_s
  * (the weight path of the GEMM); used to assert the OCP (not FNUZ) flavour on the box. */
 int tk_debug_decode_fp8(void* out_f32, void* stream);
 
+/* Reads `bytes` of device memory at `src` with a plain streaming kernel (16 bytes per lane, `blocks`
+ * blocks of 256 threads, bytes a multiple of blocks * 4096) and discards them: the yardstick for the
+ * weight-streaming launches -- what one dependent launch of that size can pull from HBM on this device.
+ * `sink` (int32, may be NULL) is never written for real data.  No counterpart in the reference. */
+int tk_debug_stream_read(const void* src, size_t bytes, int blocks, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

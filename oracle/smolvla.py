@@ -301,8 +301,8 @@ def denoise_step(w: Weights, shape: SmolVLAShape, prefix_pad, kv, ekv, x_t, time
     return w.linear("action_out_proj", out.to(torch.float32))
 
 
-def sample_actions(w: Weights, shape: SmolVLAShape, images, img_masks, lang_tokens, lang_masks, state, noise, trace: dict | None = None):
-    """Full inference: prefix embed, prefill, expert prefix KV, Euler loop -> ``[1, chunk, max_action_dim]`` fp32."""
+def sample_actions(w: Weights, shape: SmolVLAShape, images, img_masks, lang_tokens, lang_masks, state, noise, trace: dict | None = None, sampler: str = "euler"):
+    """Full inference: prefix embed, prefill, expert prefix KV, Euler (or Heun) loop -> ``[1, chunk, max_action_dim]`` fp32."""
     embs, pads, att = embed_prefix(w, shape, images, img_masks, lang_tokens, lang_masks, state)
     kv = prefill(w, shape, embs, pads, att)
     ekv = expert_prefix_kv(w, shape, kv)
@@ -314,8 +314,13 @@ def sample_actions(w: Weights, shape: SmolVLAShape, images, img_masks, lang_toke
     dt = -1.0 / shape.num_steps
     x_t = noise
     for step in range(shape.num_steps):
-        v_t = denoise_step(w, shape, pads, kv, ekv, x_t, 1.0 + step * dt)
+        t = 1.0 + step * dt
+        v_t = denoise_step(w, shape, pads, kv, ekv, x_t, t)
         if trace is not None and step == 0:
             trace["v0"] = v_t
-        x_t = x_t + dt * v_t
+        if sampler == "heun":  # corrector evaluation at t + dt (flow_matching.py:596-625)
+            v_1 = denoise_step(w, shape, pads, kv, ekv, x_t + dt * v_t, t + dt)
+            x_t = x_t + (dt * 0.5) * (v_t + v_1)
+        else:
+            x_t = x_t + dt * v_t
     return x_t

@@ -11,6 +11,8 @@ SMOLVLA_CASES = {
     "small": dict(num_vlm_layers=4, vision_layers=2, cameras=2, num_steps=3, seed=11, noise="randn", lang_pad=8),
     # full depth (config 4 of the benchmark): 16 + 16 layers, 12 vision layers, 3 cameras, 10 steps, zero noise
     "full": dict(num_vlm_layers=16, vision_layers=12, cameras=3, num_steps=10, seed=0, noise="zeros", lang_pad=0),
+    # the Heun sampler (predictor + corrector evaluation per step) on the reduced-depth model; chunk only
+    "small_heun": dict(num_vlm_layers=4, vision_layers=2, cameras=2, num_steps=3, seed=11, noise="randn", lang_pad=8, sampler="heun"),
 }
 
 PI05_CASES = {
@@ -30,6 +32,7 @@ def smolvla_build(case: dict):
         num_steps=case["num_steps"],
         vlm_config=VLMConfig(text_config=TextConfig(), vision_config=VisionConfig(num_hidden_layers=case["vision_layers"])),
         image_features=[f"observation.images.camera{i + 1}" for i in range(case["cameras"])],
+        sampler=case.get("sampler", "euler"),
     )
     sd = random_state_dict(cfg, seed=case["seed"])
     return cfg, sd, smolvla_inputs(cfg, case)

@@ -62,6 +62,7 @@ def smolvla_case(name: str) -> dict:
     ref_cfg = rcfg.SmolVLAConfig(
         num_vlm_layers=cfg.num_vlm_layers,
         num_steps=cfg.num_steps,
+        sampler=cfg.sampler,
         vlm_config=rcfg.VLMConfig(
             text_config=rcfg.TextConfig(), vision_config=rcfg.VisionConfig(num_hidden_layers=vis.num_hidden_layers)
         ),
@@ -94,6 +95,8 @@ def smolvla_case(name: str) -> dict:
         out["v_t_half"] = v_half[0].float().numpy()
         chunk = model.sample_actions(images, inputs["img_masks"], inputs["lang_tokens"], inputs["lang_masks"], inputs["state"], noise=inputs["noise"])
         out["chunk"] = chunk[0].float().numpy()
+    if cfg.sampler != "euler":  # everything before the loop is the Euler case's: keep the chunk only
+        out = {"chunk": out["chunk"]}
     return out
 
 

@@ -155,7 +155,7 @@ def test_engine_api_graph_equals_eager_and_camera_keys(ckpt):
 
     flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_fused_attn=True, tl_vit_oproj=True)
     eager = create_engine(ckpt, device="cuda", graph=False, warmup=False, **flags)
-    graph = create_engine(ckpt, device="cuda", graph=True, graph_cameras=(2, 3), warmup=True, seed=3, **flags)
+    graph = create_engine(ckpt, device="cuda", graph=True, graph_cameras=(2, 3), warmup=True, seed=3, overlap=True, **flags)
     assert graph.graph_enabled and sorted(graph._graph_runner.keys()) == [(2,), (3,)]
     # graph mode hides step 0 inside the prefill on a second stream; the eager engine is sequential:
     # the comparisons below are therefore also overlapped == sequential, bit for bit
@@ -205,6 +205,18 @@ def test_graph_requests_with_changing_task_noise_and_host_inputs(ckpt):
     assert np.array_equal(graph.predict_action_chunk(frames[1], noise=noise), want[1])
     on_device = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in frames[2].items()}
     assert np.array_equal(graph.predict_action_chunk(on_device, noise=noise.cuda()), want[2])
+    # a frame that carries its own token tensors on the device and changes them in place between requests:
+    # the replay must see the new ids (such tensors are copied every time, unlike the engine's cached ones)
+    ids1, mask1 = (t.clone() for t in graph._task_tokens("open the drawer\n"))
+    ids0, _ = graph._task_tokens("pick up the cube\n")
+    own = dict(on_device)
+    own.pop("task")
+    own["observation.language.tokens"], own["observation.language.attention_mask"] = ids1, mask1
+    first = graph.predict_action_chunk(own, noise=noise.cuda())
+    ids1.copy_(ids0)
+    second = graph.predict_action_chunk(own, noise=noise.cuda())
+    own_eager = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in own.items()}
+    assert not np.array_equal(first, second) and np.array_equal(second, eager.predict_action_chunk(own_eager, noise=noise.cuda()))
     # select_action keeps the chunk of its first request while other requests replay the graph in between
     first = graph.select_action(frames[0], noise=noise)
     graph.predict_action_chunk(frames[1], noise=noise)
@@ -220,7 +232,42 @@ def test_engine_rejects_flags_it_does_not_implement(ckpt):
     with pytest.raises(NotImplementedError):
         create_engine(ckpt, device="cuda", warmup=False, compile_model=True)
     with pytest.raises(ValueError):
-        create_engine(ckpt, device="cuda", warmup=False, sampler="heun")
+        create_engine(ckpt, device="cuda", warmup=False, sampler="rk4")
+
+
+@pytest.mark.parametrize("tiers", [dict(fused_expert=False, fp8_expert_mlp=False, fp8_llm_mlp=False), dict(FP8, fused_prefill=True, fused_vit=True)], ids=["eager", "all"])
+def test_heun_sampler_matches_oracle_and_reference_golden(tiers):
+    # sampler="heun": two velocity evaluations per step, x <- x + dt/2 (v0 + v1)
+    # (tybok/policies/smolvla/models/flow_matching.py:583-644); reduced depth, random noise
+    cfg, sd, inp = cases.smolvla_build(cases.SMOLVLA_CASES["small_heun"])
+    assert cfg.sampler == "heun"
+    shape = O.SmolVLAShape(num_vlm_layers=cfg.num_vlm_layers, vis_layers=cfg.vlm_config.vision_config.num_hidden_layers, num_steps=cfg.num_steps)
+    w = O.Weights(sd, O.fp8_linear_names(shape, tiers["fp8_llm_mlp"], tiers["fp8_expert_mlp"]))
+    with torch.no_grad():
+        want = O.sample_actions(w, shape, O.prepare_images(inp["images"]), inp["img_masks"], inp["lang_tokens"], inp["lang_masks"], inp["state"], inp["noise"], sampler="heun")
+    got = _gpu_chunk(cfg, sd, inp, **tiers)
+    err = float((got - want).abs().max())
+    print(f"heun {sorted(k for k, v in tiers.items() if v)}: max|err| = {err:.4g}, |chunk|max = {float(want.abs().max()):.3g}")
+    assert err <= 1e-2 * max(1.0, float(want.abs().max()))
+    if not any(tiers.values()):
+        gold = torch.from_numpy(np.load(os.path.join(HERE, "golden", "smolvla_small_heun.npz"))["chunk"])[None]
+        assert float((got - gold).abs().max()) <= 1e-2 * max(1.0, float(gold.abs().max()))
+
+
+def test_engine_heun_graph_equals_eager(ckpt):
+    from tybok_amd.registry import create_engine
+
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_fused_attn=True, tl_vit_oproj=True)
+    eager = create_engine(ckpt, device="cuda", graph=False, warmup=False, sampler="heun", **flags)
+    graph = create_engine(ckpt, device="cuda", graph=True, graph_cameras=(3,), warmup=True, sampler="heun", overlap=True, **flags)
+    euler = create_engine(ckpt, device="cuda", graph=False, warmup=False, **flags)
+    assert not graph.overlap  # Heun keeps the sequential path
+    frame = eager._profile_frame(cameras=3, seed=4)
+    noise = torch.zeros(1, 50, 6)
+    a = eager.predict_action_chunk(frame, noise=noise)
+    for _ in range(2):
+        assert np.array_equal(a, graph.predict_action_chunk(frame, noise=noise))
+    assert not np.array_equal(a, euler.predict_action_chunk(frame, noise=noise))
 
 
 def test_validate_against_an_oracle_dump(ckpt, tmp_path):

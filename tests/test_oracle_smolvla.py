@@ -57,3 +57,16 @@ def test_oracle_matches_reference_golden(name):
     assert _maxdiff(v_half[0].numpy(), gold["v_t_half"]) <= 1e-5
     assert _maxdiff(chunk[0].numpy(), gold["chunk"]) <= 1e-5
     assert float(np.abs(gold["chunk"]).max()) > 0.1  # the case is not degenerate
+
+
+def test_oracle_heun_sampler_matches_reference_golden():
+    # predictor + corrector evaluation per step (tybok/policies/smolvla/models/flow_matching.py:596-625)
+    case = cases.SMOLVLA_CASES["small_heun"]
+    gold = np.load(os.path.join(HERE, "golden", "smolvla_small_heun.npz"))
+    cfg, sd, inp = cases.smolvla_build(case)
+    with torch.no_grad():
+        args = (O.Weights(sd), _shape(cfg), O.prepare_images(inp["images"]), inp["img_masks"], inp["lang_tokens"], inp["lang_masks"], inp["state"], inp["noise"])
+        chunk = O.sample_actions(*args, sampler="heun")
+        euler = O.sample_actions(*args)
+    assert _maxdiff(chunk[0].numpy(), gold["chunk"]) <= 1e-5
+    assert _maxdiff(euler[0].numpy(), gold["chunk"]) > 1e-3  # the corrector changes the result: the fixture pins it

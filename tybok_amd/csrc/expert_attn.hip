@@ -25,22 +25,6 @@
 #include "tk_common.h"
 #include "tk_kernels.h"
 
-#ifdef TK_PHASE_TIMING
-// development aid (never built into the shipped library): per-block phase timestamps
-__device__ long long tk_attn_stamps[8 * 8192];
-#define TA_MARK(i)                                                                   \
-  do {                                                                               \
-    if (threadIdx.x == 0) {                                                          \
-      const int b_ = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x; \
-      if (b_ < 8192) tk_attn_stamps[b_ * 8 + (i)] = wall_clock64();                  \
-    }                                                                                \
-  } while (0)
-extern "C" int tk_debug_read_attn_phases(void* host_out) {
-  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(tk_attn_stamps), sizeof(long long) * 8 * 8192);
-}
-#else
-#define TA_MARK(i)
-#endif
 
 namespace {
 
@@ -100,7 +84,6 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   a.vt_pre += bi * a.vt_sb;
   a.out += bi * a.out_sb;
   const int g = (h * a.gqa_mul) >> 16;       // h / (H / G) without a runtime divide
-  TA_MARK(0);
   const int tp = (a.P + 31) >> 5;            // prefix tiles; suffix tiles follow
   const int t_lo = split * a.tile_q + (split < a.tile_r ? split : a.tile_r);
   const int t_hi = t_lo + a.tile_q + (split < a.tile_r ? 1 : 0);
@@ -184,7 +167,6 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
     __syncthreads();
   }
   }
-  TA_MARK(1);
 
   f32x16 o[DT];
 #pragma unroll
@@ -322,8 +304,6 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
       }
     }
   }
-
-  TA_MARK(2);
   // ---- merge the four waves in fixed order (LDS) ----
   if (half == 0) {
     st_m[wave][l32] = m_run;
@@ -367,8 +347,6 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
     }
     own[dt] = sum;
   }
-
-  TA_MARK(3);
   // this lane's output: query qi, columns d0 .. d0+3 of every d tile
   u16* op = a.out + (size_t)(q_ok ? qi : 0) * a.out_sm + (size_t)h * D + 8 * wg + 4 * half;
   if (a.kv_splits == 1) {
@@ -405,7 +383,6 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
     s_last = (old == a.kv_splits - 1);
   }
   __syncthreads();
-  TA_MARK(4);
   if (!s_last || !owner) return;
   if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
@@ -445,7 +422,6 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
     es[s] = (s < a.kv_splits && ms[s] != -INFINITY) ? __expf(ms[s] - mt) : 0.f;
     if (s < a.kv_splits) lt += ls[s] * es[s];
   }
-  TA_MARK(5);
   const float inv = 1.0f / lt;
 #pragma unroll
   for (int d0 = 0; d0 < DT; d0 += DTB) {
@@ -467,7 +443,6 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
     for (int dd = 0; dd < DTB; ++dd)
       if (q_ok) *(i32x2*)(op + (d0 + dd) * 32) = pack_bf16x4(acc[dd] * inv);
   }
-  TA_MARK(6);
 }
 
 // Lays a [L, G, D] K/V pair out for the attention kernel: V transposed to [G, D, ld] (keys

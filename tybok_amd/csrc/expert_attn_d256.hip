@@ -20,22 +20,6 @@
 #include "tk_common.h"
 #include "tk_kernels.h"
 
-#ifdef TK_PHASE_TIMING
-// development aid (never built into the shipped library): per-block phase timestamps
-__device__ long long tk_attn256_stamps[8 * 8192];
-#define TA_MARK(i)                                                                   \
-  do {                                                                               \
-    if (threadIdx.x == 0) {                                                          \
-      const int b_ = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x; \
-      if (b_ < 8192) tk_attn256_stamps[b_ * 8 + (i)] = wall_clock64();               \
-    }                                                                                \
-  } while (0)
-extern "C" int tk_debug_read_attn256_phases(void* host_out) {
-  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(tk_attn256_stamps), sizeof(long long) * 8 * 8192);
-}
-#else
-#define TA_MARK(i)
-#endif
 
 namespace {
 
@@ -97,8 +81,6 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
   f32x16 o;
 #pragma unroll
   for (int i = 0; i < 16; ++i) o[i] = 0.f;
-
-  TA_MARK(0);
   for (int r_lo = 0; r_lo < ntb; r_lo += kWaves) {
   const int nt = ntb - r_lo < kWaves ? ntb - r_lo : kWaves;  // key tiles of this round, 1..kWaves
   const int rt_lo = t_lo + r_lo;
@@ -162,8 +144,6 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
   // keep the V^T requests here: sunk below the first product (to save registers) they would leave only
   // after Q and K have arrived, one memory round trip later
   __builtin_amdgcn_sched_barrier(0);
-
-  TA_MARK(1);
   // ---- S^T tile = K . Q^T (one query column per lane) ----
   f32x16 sT;
 #pragma unroll
@@ -269,8 +249,6 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
     for (int w = 1; w < kWaves; ++w) rl += st_l[w][l32];
     bl = bl * alpha + rl;
   }
-
-  TA_MARK(2);
   // ---- O^T rows [32w, 32w + 32) += V^T . P^T over every key tile of the round ----
 #pragma unroll
   for (int i = 0; i < 16; ++i) o[i] *= alpha;  // all of a lane's registers belong to its one query
@@ -290,8 +268,6 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
       for (int s = 0; s < 2; ++s) o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(va[j][s]), as_bf16x8(pb[j][s]), o, 0, 0, 0);
   }
   }  // rounds
-
-  TA_MARK(3);
   // this lane's output: query qi, columns 32w + 8g4 + 4*half + 0..3 for the four register groups g4
   u16* op = a.out + (size_t)(q_ok ? qi : 0) * a.out_sm + (size_t)h * kD + 32 * wave + 4 * half;
   if (a.kv_splits == 1) {
@@ -330,7 +306,6 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
     s_last = (old == a.kv_splits - 1);
   }
   __syncthreads();
-  TA_MARK(4);
   if (!s_last) return;
   if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
@@ -358,7 +333,6 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
       }
     }
   }
-  TA_MARK(5);
   float mt = -INFINITY;
 #pragma unroll
   for (int s = 0; s < kMaxSplits; ++s)
@@ -383,7 +357,6 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
     }
     if (q_ok) *(i32x2*)(op + 8 * g4) = pack_bf16x4(acc * inv);
   }
-  TA_MARK(6);
 }
 
 }  // namespace

@@ -18,22 +18,6 @@
 #include "tk_common.h"
 #include "tk_kernels.h"
 
-#ifdef TK_PHASE_TIMING
-// development aid (never built into the shipped library): per-block phase timestamps
-__device__ long long tk_phase_stamps[8 * 8192];
-#define TK_MARK(i)                                                                                       \
-  do {                                                                                                   \
-    if (threadIdx.x == 0) {                                                                              \
-      const int b_ = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;                     \
-      if (b_ < 8192) tk_phase_stamps[b_ * 8 + (i)] = wall_clock64();                                     \
-    }                                                                                                    \
-  } while (0)
-extern "C" int tk_debug_read_phases(void* host_out) {
-  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(tk_phase_stamps), sizeof(long long) * 8 * 8192);
-}
-#else
-#define TK_MARK(i)
-#endif
 
 namespace {
 
@@ -84,8 +68,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   const int mblock = blockIdx.z;
   const int half = lane >> 5;
   const int l32 = lane & 31;
-
-  TK_MARK(0);
   // k tiles of this split: KT = ksplit * kt_q + kt_r, the first kt_r splits take one more (host-side
   // division: a 64-bit divide here costs some 300 scalar instructions before the first load)
   const int kt_lo = split * a.kt_q + (split < a.kt_r ? split : a.kt_r);
@@ -282,7 +264,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     xload(xbuf[p], p);
     wload(wbuf[p], p);
   }
-  TK_MARK(1);
   if (PRO) {
     // per-row 1/rms over the whole K (every block needs it for its rows, whatever its k range)
     constexpr int TPR = NW * 64 / ROWS;  // threads per row
@@ -318,7 +299,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 #pragma unroll
     for (int i = 0; i < XPT; ++i) my_rstd[i] = rstd_s[xrow[i]];
   }
-  TK_MARK(2);
   if (nrounds > 0) {
     int it = 0;
     for (; it + 2 * PF <= nrounds; it += PF) {
@@ -349,7 +329,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     }
   }
   __syncthreads();  // staging buffers are dead; the reduction reuses the LDS
-  TK_MARK(3);
 
   // The accumulators hold C^T tiles: lane l of a tile owns activation row m = l % 32 and, in
   // register i, output column n = 8*(i/4) + 4*(l/32) + i%4 -- register group g = i/4 is four
@@ -422,7 +401,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   }
 
   // ---- K-split reduction through global partials; the last-arriving block finishes ----
-  TK_MARK(4);
   const int blk_lin = mblock * gridDim.x + strip;
   if (a.ksplit > 1) {
     // partial layout: [(block, split)][tile][group][lane][4 floats], written and read as 8-byte
@@ -443,7 +421,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       s_last = (old == a.ksplit - 1);
     }
     __syncthreads();
-    TK_MARK(5);
     if (!s_last) return;
     if (threadIdx.x == 0)  // leave the counter ready for the next launch
       __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -479,7 +456,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   }
 
   // ---- epilogue: this lane finishes row m (per m tile), columns n0 .. n0+3 of each n tile ----
-  TK_MARK(6);
   if (EPI == 0) {
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
@@ -579,7 +555,6 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       }
     }
   }
-  TK_MARK(7);
 }
 
 __global__ void pack_kernel(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1, uint8_t* __restrict__ out,
@@ -645,18 +620,13 @@ __global__ void decode_fp8_kernel(float* out) {
 }
 
 // Pipeline depth (block rounds in flight) and k tiles per wave and round.  Measured on MI355X: 4 rounds
-// cover the weight stream's latency at the 33.5 MB shapes; two k tiles per wave and round halve the
-// barriers but lengthen every small launch of the denoise loop (request +0.8 ms).  Overridable at
-// compile time for tuning runs.
-#ifndef TK_EXP_PF
-#define TK_EXP_PF 4
-#endif
-#ifndef TK_EXP_TPW
-#define TK_EXP_TPW 1
-#endif
+// cover the weight stream's latency at the 33.5 MB shapes (2, 6 and 8 are no faster); two k tiles per
+// wave and round halve the barriers but lengthen every small launch of the denoise loop.
+constexpr int kPF = 4;
+constexpr int kTPW = 1;
 template <int MT, int NT, int EPI, bool W16, int PRO, int NR>
 int launch_nr(const GemmArgs& a, dim3 grid, hipStream_t st) {
-  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, TK_EXP_PF, TK_EXP_TPW, W16, PRO, NR>), grid, dim3(256), 0, st, a);
+  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, kPF, kTPW, W16, PRO, NR>), grid, dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 template <int MT, int NT, int EPI, bool W16, int PRO>
@@ -664,7 +634,7 @@ int launch(const GemmArgs& a, dim3 grid, hipStream_t st) {
   // the action chunk's launches (32-row blocks, every block the same number of k tiles) at the round counts
   // of the two models' expert layers: K = 720 -> 6, 960 / 1024 -> 8, 2048 -> 16, 4096 in four splits -> 8
   if (MT == 1 && a.kt_r == 0) {
-    const int nr = (a.kt_q + 4 * TK_EXP_TPW - 1) / (4 * TK_EXP_TPW);
+    const int nr = (a.kt_q + 4 * kTPW - 1) / (4 * kTPW);
     if (nr == 6) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 6 : 0>(a, grid, st);
     if (nr == 8) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 8 : 0>(a, grid, st);
     if (nr == 16) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 16 : 0>(a, grid, st);

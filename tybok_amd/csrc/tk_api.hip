@@ -225,12 +225,6 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   // as many CUs on it (measured: FFN at K=720 12.6 -> 10.0 us, with the norm prologue 15.7 -> 12.6 us);
   // the weights are then read twice, which only a large matrix notices (the 33.5 MB shapes lose 5 %).
   if (M > 32 && M <= 64 && (size_t)a.ntiles * 32 * a.KT * 32 * (e.w16 ? 2 : 1) <= (16u << 20)) MT = 1;
-#ifdef TK_PHASE_TIMING
-  if (const char* ev = getenv("TK_GEMM_MT")) {  // development aid, never in the shipped build
-    const int v = atoi(ev);
-    if ((v == 1 || v == 2) && M > 32) MT = v;
-  }
-#endif
   int NT = 2;
   if (!gated && !rope && ((a.ntiles + 1) / 2) * ((M + 32 * MT - 1) / (32 * MT)) < cus / 2) {
     NT = 1;  // few columns: finer strips (the paired epilogues need both tiles of a strip in one wave)
@@ -596,12 +590,6 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   // 64-wide heads, whole key range in one block (the SmolVLA self layers and prefill)
   const bool px = D == 64 && !split && batch == 0 && ntiles <= tk_attn_px_max_tiles();
   if (px) splits = 1;
-#ifdef TK_PHASE_TIMING
-  if (const char* ev = getenv("TK_ATTN_SPLITS")) {  // development aid, never in the shipped build
-    const int v = atoi(ev);
-    if (v >= 1 && v <= 8 && D == 256 && !d256 && !px) splits = v;
-  }
-#endif
   a.kv_splits = splits;
   a.tile_q = ntiles / splits;
   a.tile_r = ntiles % splits;
@@ -836,6 +824,13 @@ int tk_add_layer_norm(const void* x, int ldx, int x_dtype, const void* r, int ld
                       const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream) {
   if (!r) return fail(TK_EINVAL, "add_layer_norm: null residual branch");
   return layer_norm_impl("add_layer_norm", x, ldx, x_dtype, r, ldr, xsum, ldxs, w, b, wb_dtype, eps, y, ldy, M, K, stream);
+}
+
+int tk_debug_stream_read(const void* src, size_t bytes, int blocks, void* sink, void* stream) {
+  if (!src || !aligned16(src) || blocks <= 0 || blocks > 65536) return fail(TK_EINVAL, "stream_read: null or unaligned source, or blocks=%d out of range", blocks);
+  if (bytes == 0 || bytes % ((size_t)blocks * 4096)) return fail(TK_EINVAL, "stream_read: bytes=%zu must be a positive multiple of blocks * 4096", bytes);
+  if (tk_launch_stream_read(src, bytes, blocks, (int*)sink, (hipStream_t)stream)) return fail(TK_ELAUNCH, "stream_read: launch failed");
+  return TK_OK;
 }
 
 int tk_debug_decode_fp8(void* out_f32, void* stream) {

@@ -189,6 +189,8 @@ int tk_launch_pack(const void* w0, const void* w1, void* out, int N, int K, int 
 int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st);
 int tk_launch_fill_zero(int* p, int n, hipStream_t st);
 int tk_launch_decode_fp8(float* out, hipStream_t st);
+// plain 16-byte-per-lane read of `bytes` (a multiple of blocks * 4096) by `blocks` blocks of 256 threads
+int tk_launch_stream_read(const void* src, size_t bytes, int blocks, int* sink, hipStream_t st);
 struct TransposeVArgs {
   const unsigned short* v;  // bf16 [B, P, G, D], element strides (v_sb, v_sl, v_sh), d contiguous
   long long v_sb;

@@ -101,6 +101,12 @@ class StaticCall:
                 self.store(**{name: value})
                 self._last_owned[name] = objects
 
+    def forget_owned(self, *names: str) -> None:
+        """The static tensors ``names`` were overwritten by a plain :meth:`store`: the next
+        :meth:`store_owned` of those names copies again."""
+        for name in names:
+            getattr(self, "_last_owned", {}).pop(name, None)
+
     def replay(self, *, copy: bool = True) -> torch.Tensor:
         """Run the graph.  By default the result is copied out so that the next replay cannot overwrite
         it; ``copy=False`` returns the static tensor itself, for callers that finish with it (or copy it)

@@ -11,10 +11,7 @@ import ctypes
 import os
 from ctypes import c_char_p, c_float, c_int, c_longlong, c_size_t, c_void_p
 
-# TYBOK_HIP_LIB points at an alternative build of the same ABI (kernel experiments); default in-tree.
-_LIB_PATH = os.environ.get("TYBOK_HIP_LIB") or os.path.join(
-    os.path.dirname(os.path.abspath(__file__)), "_lib", "libtybok_hip.so"
-)
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libtybok_hip.so")
 _lib: ctypes.CDLL | None = None
 
 # name -> (restype, argtypes); mirrors include/tybok_hip.h one to one
@@ -98,6 +95,7 @@ SIGNATURES: dict[str, tuple] = {
          c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
     "tk_debug_decode_fp8": (c_int, [c_void_p, c_void_p]),
+    "tk_debug_stream_read": (c_int, [c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
 }
 
 

@@ -47,6 +47,10 @@ _default_ws: dict[int, Workspace] = {}
 
 
 def default_workspace(device: torch.device | str | None = None) -> Workspace:
+    """The per-device workspace used when a call passes none.  It serves launches that are ordered one
+    after the other (one stream, or streams joined by events / graph capture of a single stream): the
+    split hand-offs keep counters and partials in it, so code that runs kernels on two streams AT THE
+    SAME TIME must give the second stream a :class:`Workspace` of its own (the SmolVLA overlap path does)."""
     dev = torch.device(device if device is not None else "cuda")
     idx = dev.index if dev.index is not None else torch.cuda.current_device()
     ws = _default_ws.get(idx)

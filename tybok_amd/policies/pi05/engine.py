@@ -191,6 +191,8 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
         self.rtc_processor = None
         self._init_graphs(graph, "pi05 graph", log)
         self.overlap = False  # prefill x step-0 two-stream overlap is not implemented; accepted, inert
+        if overlap and graph:
+            log.info("overlap requested: the prefill x step-0 overlap is not built for pi0.5 here; requests run sequentially (engine.overlap is False)")
         key = (len(self.config.image_features), self.config.tokenizer_max_length)
         self._start(warmup=warmup, graph_keys=[key], profile=profile, logger=log)
 

@@ -86,7 +86,7 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
         sampler: str = "euler",
         cache_expert_prefix_kv: bool = True,
         profile: bool = False,
-        overlap: bool = True,
+        overlap: bool = False,
         camera_alias: dict[str, str] | None = None,
         tl_llm_fused_attn: bool = False,
         tl_vit_oproj: bool = False,
@@ -95,8 +95,8 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
         tl_fp8_expert_mlp: bool = False,
     ):
         super().__init__(checkpoint_dir, device=device)
-        if sampler != "euler":
-            raise ValueError(f"unknown sampler {sampler!r} (this backend implements 'euler')")
+        if sampler not in ("euler", "heun"):
+            raise ValueError(f"unknown sampler {sampler!r} (expected 'euler' or 'heun')")
         if compile_model:
             raise NotImplementedError("--compile is not supported by this backend (the HIP tiers replace it)")
         self.compile_model = False
@@ -108,6 +108,7 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
             )
         if num_steps is not None:
             self.config.num_steps = int(num_steps)
+        self.config.sampler = sampler  # Heun keeps the sequential path: no prefill x step-0 overlap (reference engine :229-237)
         self.config.cache_expert_prefix_kv = bool(cache_expert_prefix_kv)
         hip_flags = [
             n
@@ -148,7 +149,7 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
             fused_expert=self.tl_fused_expert, fp8_expert_mlp=self.tl_fp8_expert_mlp, fp8_llm_mlp=self.tl_fp8_llm_mlp,
             fused_prefill=self.tl_llm_fused_attn, fused_vit=self.tl_vit_oproj,
             # graph mode only, like the reference (smolvla/engine.py:229-237); needs both fused tiers
-            overlap=bool(overlap) and bool(graph) and str(self.device).startswith("cuda"),
+            overlap=bool(overlap) and bool(graph) and sampler == "euler" and str(self.device).startswith("cuda"),
         )  # fmt: skip
         del sd
 
@@ -355,7 +356,14 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
         copied it, before the next request replays."""
         with self._graph_runner.copy_inputs():
             call.store(images01=images01, state=state)
-            call.store_owned(lang_tokens=tokens, lang_masks=lang_masks, img_masks=img_masks)
+            call.store_owned(img_masks=img_masks)  # always the engine's cached all-true / all-false masks
+            # token ids and masks: skipped only when they are the engine's own cached pair for the task; a
+            # frame that carries its own token tensors may change them in place between requests
+            if any(tokens is t and lang_masks is m for t, m in self._token_cache.values()):
+                call.store_owned(lang_tokens=tokens, lang_masks=lang_masks)
+            else:
+                call.store(lang_tokens=tokens, lang_masks=lang_masks)
+                call.forget_owned("lang_tokens", "lang_masks")
             if noise is None:
                 self._sample_noise(out=call.inputs["noise"])  # drawn outside the graph, from the engine's generator
             else:

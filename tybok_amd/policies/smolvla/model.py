@@ -176,9 +176,13 @@ class SmolVLAModel:
     def set_num_steps(self, n: int) -> None:
         self.num_steps = int(n)
         dt = -1.0 / self.num_steps
+        # Euler: one velocity evaluation per step at t = 1 + step * dt.  Heun: two, at t and t + dt
+        # (entries 2 * step and 2 * step + 1: tybok/policies/smolvla/models/flow_matching.py:583-644).
+        heun = getattr(self.cfg, "sampler", "euler") == "heun"
+        times = [1.0 + step * dt + (dt if second else 0.0) for step in range(self.num_steps) for second in ((False, True) if heun else (False,))]
         embs = []
-        for step in range(self.num_steps):
-            t = torch.tensor(1.0 + step * dt, dtype=torch.float32).expand(1)
+        for time in times:
+            t = torch.tensor(time, dtype=torch.float32).expand(1)
             embs.append(sinusoidal_time_embedding(t, self.cfg.expert_hidden_size, self.cfg.min_period, self.cfg.max_period).float())
         self.time_embs = [e.to(self.device) for e in embs]
         if getattr(self, "fused_expert", False):
@@ -471,18 +475,19 @@ class SmolVLAModel:
             hidden = self._denoise_layer_fused(i, hidden, caches[i], prefix_pad[0], pos32, pos0_32, self.ws)
         return hidden
 
-    def fused_euler_step(self, prefix_pad, caches, x_t, step: int, positions, dt: float) -> torch.Tensor:
-        """One Euler step on the fused launches: folded suffix embedding, expert stack, then final
-        norm + action projection + ``x_t + dt * v_t`` in one launch.  ``x_t [1, chunk, A]`` fp32."""
+    def fused_euler_step(self, prefix_pad, caches, x_t, step: int, positions, dt: float, want_v: bool = False):
+        """One velocity evaluation on the fused launches (time entry ``step``): folded suffix embedding, expert
+        stack, then final norm + action projection + ``x_t + dt * v_t`` in one launch.  ``x_t [1, chunk, A]``
+        fp32.  Returns the updated ``x``; with ``want_v`` the pair ``(v_t, x_t + dt * v_t)``."""
         pos32, pos0_32 = positions
         h = F.silu(F.linear(x_t[0], self.suffix_w, self.suffix_b[step]))
         hidden = F.linear(h, self.p["action_time_mlp_out.weight"], self.p["action_time_mlp_out.bias"])
         hidden = self._denoise_step_fused(prefix_pad, caches, hidden, pos32, pos0_32)
-        _, x_new = tk.expert_tail(
+        v, x_new = tk.expert_tail(
             hidden, self.p["action_out_proj.weight"], self.p["action_out_proj.bias"], norm_w=self.p[EXP + "norm.weight"],
-            eps=self.eps, x_t=x_t[0], dt=dt,
+            eps=self.eps, x_t=x_t[0], dt=dt, want_v=want_v,
         )  # fmt: skip
-        return x_new[None]
+        return (v[None], x_new[None]) if want_v else x_new[None]
 
     def denoise_step(self, prefix_pad, keys, values, ekv, x_t, time_emb, positions=None, caches=None):
         """Velocity ``v_t`` fp32 ``[1, chunk, max_action_dim]`` (flow_matching.py:316-350)."""
@@ -557,7 +562,7 @@ class SmolVLAModel:
         return x_t
 
     def sample_actions_core(self, embs, pads, att, noise, trace: dict | None = None) -> torch.Tensor:
-        if self.overlap and trace is None and embs.shape[0] == 1 and noise.shape[0] == 1 and noise.dtype == torch.float32 and noise.is_contiguous():
+        if self.overlap and getattr(self.cfg, "sampler", "euler") == "euler" and trace is None and embs.shape[0] == 1 and noise.shape[0] == 1 and noise.dtype == torch.float32 and noise.is_contiguous():
             return self._sample_actions_overlapped(embs, pads, att, noise)
         vt = None
         if self.fused_prefill and embs.shape[0] == 1:
@@ -576,6 +581,18 @@ class SmolVLAModel:
             positions = tuple(t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32) for t in positions)
         caches = self.attention_caches(keys, values, ekv, vt) if self.fused_expert and noise.shape[0] == 1 else None
         fused_loop = caches is not None and x_t.dtype == torch.float32 and x_t.is_contiguous()
+        if getattr(self.cfg, "sampler", "euler") == "heun":
+            # predictor at t, corrector at t + dt, then x <- x + (dt / 2) (v0 + v1)
+            # (tybok/policies/smolvla/models/flow_matching.py:596-625)
+            for step in range(self.num_steps):
+                if fused_loop:
+                    v0, x_pred = self.fused_euler_step(pads, caches, x_t, 2 * step, positions, dt, want_v=True)
+                    v1, _ = self.fused_euler_step(pads, caches, x_pred, 2 * step + 1, positions, dt, want_v=True)
+                else:
+                    v0 = self.denoise_step(pads, keys, values, ekv, x_t, self.time_embs[2 * step], positions, caches)
+                    v1 = self.denoise_step(pads, keys, values, ekv, x_t + dt * v0, self.time_embs[2 * step + 1], positions, caches)
+                x_t = x_t + (dt * 0.5) * (v0 + v1)
+            return x_t
         for step in range(self.num_steps):
             if fused_loop:
                 x_t = self.fused_euler_step(pads, caches, x_t, step, positions, dt)
