@@ -15,6 +15,8 @@
 //     loads need no masking: a zero activation column cancels whatever tile was read.
 //   * Reductions are fixed-order: waves through LDS (w = 0..NW-1), K splits through an fp32
 //     partial buffer summed by the last-arriving block in split order (no float atomics).
+#include <type_traits>
+
 #include "tk_common.h"
 #include "tk_kernels.h"
 
@@ -157,12 +159,16 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   float my_rstd[XPT];
 #pragma unroll
   for (int i = 0; i < XPT; ++i) my_rstd[i] = 1.f;
-  auto xstore = [&](const XFrag& f, int r, int b) {
+  // MASKED: zero the columns past the block's k range.  Only a block's LAST round can reach past it (the
+  // rounds before cover whole k tiles below kt_hi, and only the last k tile of the matrix is partial), so
+  // every other round stages without the per-element selects -- they sit on each round's critical path.
+  auto xstore = [&](const XFrag& f, int r, int b, auto masked_c) {
+    constexpr bool MASKED = decltype(masked_c)::value;
     const int k0 = (kt_lo + r * RKT) * 32;
     const i32x4 z = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < XPT; ++i) {
-      const bool ok = (k0 + xcol[i]) < k_end;
+      const bool ok = !MASKED || (k0 + xcol[i]) < k_end;
       i32x4 out;
       if (PRO == 0) {
         out = f.v[i][0];
@@ -305,7 +311,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 #pragma unroll
       for (int p = 0; p < PF; ++p) {
         const int r = it + p;
-        xstore(xbuf[p], r, r & 1);
+        xstore(xbuf[p], r, r & 1, std::false_type{});
         lds_barrier();
         compute(wbuf[p], r & 1);
         xload(xbuf[p], r + PF);
@@ -318,7 +324,8 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     for (int q = 0; q < 2 * PF - 1; ++q) {
       if (q < rem) {  // block-uniform
         const int r = it + q;
-        xstore(xbuf[q % PF], r, r & 1);
+        if (q == rem - 1) xstore(xbuf[q % PF], r, r & 1, std::true_type{});  // block-uniform
+        else xstore(xbuf[q % PF], r, r & 1, std::false_type{});
         lds_barrier();
         compute(wbuf[q % PF], r & 1);
         if (q + PF < rem) {
