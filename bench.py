@@ -262,8 +262,41 @@ def time_requests(engine, frame, noise, steps: int, warmup: int) -> tuple[list[f
     return samples, total_ms
 
 
-def cpu_baseline_smolvla(cameras: int) -> dict:
-    """One request of the benchmark workload on the host cores through the CPU oracle."""
+def _median_ms(fn, reps: int, warm: int = 2) -> float:
+    for _ in range(warm):
+        fn()
+    t = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        t.append((time.perf_counter() - t0) * 1e3)
+    return float(np.median(t))
+
+
+def cpu_ops_baseline() -> dict:
+    """The single-op configurations on the host cores through the CPU oracle: config 1 (fp8 SwiGLU FFN), the
+    M = 50 row of the GEMM sweep, config 3 (expert attention); median of 10 after 2 warm-ups, all threads."""
+    import torch
+
+    from oracle import ops as oops
+    from oracle.inputs import attn_case, ffn_case, gemm_case
+
+    out = {}
+    ffn = ffn_case(50, 720, 2048, seed=0)
+    out["ffn_M50_K720_I2048_ms"] = round(_median_ms(lambda: oops.gated_ffn(*ffn, "silu"), 10), 3)
+    for k, n in GEMM_SHAPES:
+        g = gemm_case(50, k, n)
+        out[f"gemm_M50_K{k}_N{n}_ms"] = round(_median_ms(lambda: oops.lin_fp8w(*g), 10), 3)
+    q, kp, vp, ks, vs = attn_case()
+    pad = torch.ones(241, dtype=torch.bool)
+    out["expert_attn_M50_P241_S50_ms"] = round(_median_ms(lambda: oops.expert_attention(q, kp, vp, ks, vs, pad, oops.MASK_BIDIR), 10), 3)
+    return out
+
+
+def cpu_baseline_smolvla(cameras: int, frame: dict | None = None) -> tuple[dict, "np.ndarray | None"]:
+    """Requests of the benchmark workload on the host cores through the CPU oracle.  With ``frame`` (the
+    benchmark's own observation, host tensors) the oracle's zero-noise chunk for it is returned as well, so
+    the GPU result of the timed configuration can be checked in the same run."""
     import torch
 
     from oracle import smolvla as O
@@ -278,29 +311,42 @@ def cpu_baseline_smolvla(cameras: int) -> dict:
     images = [torch.randint(0, 256, (1, 3, 512, 512), generator=g, dtype=torch.uint8).float() / 255.0 for _ in range(cameras)]
     tokens = torch.randint(0, shape.vocab, (1, shape.tok_len), generator=g)
     state = torch.zeros(1, shape.max_state_dim)
+    lang_masks = torch.ones(1, shape.tok_len, dtype=torch.bool)
+    if frame is not None:  # the observation the GPU engine was timed on, as the engine preprocessed it
+        images = [frame[k].float().reshape(1, 3, 512, 512) for k in sorted(k for k in frame if k.startswith("observation.images."))]
+        tokens, lang_masks, state = frame["tokens"], frame["lang_masks"], frame["state"]
     noise = torch.zeros(1, shape.chunk, shape.max_action_dim)
     masks = [torch.ones(1, dtype=torch.bool)] * cameras
-    lang_masks = torch.ones(1, shape.tok_len, dtype=torch.bool)
 
-    def request() -> float:
-        t0 = time.perf_counter()
+    def request():
         with torch.no_grad():
-            O.sample_actions(w, shape, O.prepare_images(images), masks, tokens, lang_masks, state, noise)
-        return (time.perf_counter() - t0) * 1e3
+            return O.sample_actions(w, shape, O.prepare_images(images), masks, tokens, lang_masks, state, noise)
 
-    request()  # warm-up (thread pool, allocator)
+    chunk = request()  # warm-up (thread pool, allocator)
     # a bounded sample: requests until about 12 s of CPU work have been spent, at least 3, at most 20
     samples, budget_ms = [], 12_000.0
     while len(samples) < 3 or (sum(samples) < budget_ms and len(samples) < 20):
-        samples.append(request())
+        t0 = time.perf_counter()
+        request()
+        samples.append((time.perf_counter() - t0) * 1e3)
+    threads = int(torch.get_num_threads())
+    torch.set_num_threads(1)
+    try:
+        t0 = time.perf_counter()
+        request()
+        one_thread_ms = (time.perf_counter() - t0) * 1e3
+    finally:
+        torch.set_num_threads(threads)
     return {
         "value": round(float(np.percentile(samples, 50)), 1),
         "unit": "ms",
-        "cores": int(torch.get_num_threads()),
+        "cores": threads,
         "kind": "port",
         "sample": f"p50 of {len(samples)} predict_action_chunk requests of the same SmolVLA-shaped workload ({cameras} cameras, 10 steps, "
         f"fp8 MLP weights) through the CPU oracle after one warm-up ({sum(samples) / 1e3:.1f} s of CPU work)",
-    }
+        "one_thread_ms": round(one_thread_ms, 1),
+        "ops_all_threads": cpu_ops_baseline(),
+    }, chunk[0].numpy()
 
 
 def main() -> None:
@@ -379,6 +425,13 @@ def main() -> None:
     spin_up()
     frame3 = device_frame(engine, 3)
     samples3, total_ms = time_requests(engine, frame3, noise, args.steps, args.warmup)
+    # the timed configuration's own result and the inputs the model saw, for the parity check against the CPU oracle
+    gpu_chunk = np.asarray(engine.predict_action_chunk(frame3, noise=noise))
+    with torch.inference_mode():
+        b3 = engine._batch_from_frame(frame3)
+        oracle_frame = {k: v.cpu() for k, v in b3.items() if k.startswith("observation.images.")}
+        oracle_frame.update(tokens=b3["observation.language.tokens"].cpu(), lang_masks=b3["observation.language.attention_mask"].cpu(), state=engine.prepare_state(b3).cpu())
+    unnorm = engine.unnormalizer
     frame2 = device_frame(engine, 2)
     samples2, _ = time_requests(engine, frame2, noise, max(5, args.steps // 2), 2)
     host_frame = {k: (v.cpu() if hasattr(v, "cpu") else v) for k, v in frame3.items()}
@@ -454,13 +507,35 @@ def main() -> None:
     # ---- the single-op configurations at the action-chunk shape: latency-bound launches ----
     c1_us = ffn_launch_us(50, 720, 2048, launches=50, reps=10)
     c1_bytes = 3 * 720 * 2048 + 4 * (2 * 2048 + 720) + 2 * 50 * 720 * 2  # fp8 weights, fp32 scales, bf16 in / out
+    roofline_ffn = {
+        "bound": "hbm",
+        "kernel": "tk_fp8w_gated_ffn (M=50, K=720, I=2048): gate/up + down launches, weights from cache (4.4 MB)",
+        "achieved": round(c1_bytes / c1_us / 1e3, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(c1_bytes / c1_us / 1e3 / HBM_PEAK_GBS, 4),
+        "bytes_per_call": c1_bytes,
+        "us_per_call": round(c1_us, 2),
+        "note": "two dependent launches moving 4.6 MB: latency-bound (1 us at peak), not a bandwidth measurement",
+    }
     ops_small = {
         "ffn_M50_K720_I2048": {"us": round(c1_us, 2), "GBps": round(c1_bytes / c1_us / 1e3, 1), "launches": 2},
         "expert_attn_M50_P241_S50_H15_G5_D64": {"us": round(attn_launch_us(launches=50, reps=10), 2)},
         "tower_attn_B3_M1024_H12_D64": {"us": round(tower_attn_launch_us(launches=20, reps=10), 2)},
     }
 
-    cpu = None if args.skip_cpu else cpu_baseline_smolvla(3)
+    cpu, parity = None, None
+    if not args.skip_cpu:
+        cpu, oracle_chunk = cpu_baseline_smolvla(3, oracle_frame)
+        want = unnorm.unnormalize(torch.from_numpy(oracle_chunk[None, :, : gpu_chunk.shape[-1]]).cuda(), "action", "ACTION")[0].cpu().numpy()
+        diff = np.abs(gpu_chunk - want)
+        parity = {
+            "what": "action chunk of the timed configuration (every tier, graph replay, zero noise) against the CPU oracle on the same frame",
+            "chunk_max_abs_err": round(float(diff.max()), 5),
+            "chunk_mean_abs_err": round(float(diff.mean()), 5),
+            "stated_bound": 1e-2,
+            "held_bound": 1.25e-2,
+        }
 
     p50 = float(np.percentile(samples3, 50))
     line = {
@@ -490,7 +565,9 @@ def main() -> None:
         "ops_action_chunk_shape": ops_small,
         "pi05_prefill_ffn_M712": prefill_ffn,
         "roofline": roofline,
+        "roofline_ffn": roofline_ffn,
         "cpu_baseline": cpu,
+        "parity": parity,
     }
     print(json.dumps(line), flush=True)
 
