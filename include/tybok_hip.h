@@ -145,6 +145,38 @@ int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float nor
                            const void* resid, int ldr, int resid_dtype, const void* gate, int M, int K, int I,
                            int act, void* ws, size_t ws_bytes, void* stream);
 
+/* ---- W8A8 tier: per-token activation quantisation + fp8 x fp8 GEMM (VLM prefill MLP) --------- */
+/* Per-token (per-row) activation quantisation to e4m3fn:
+ *   sa[m] = max_k |x[m, k]| / 448 (fp32),  a8[m, k] = RNE(x[m, k] / sa[m]) computed in fp32, one rounding;
+ *   an all-zero row gives sa = 0 and zero codes.
+ * Replaces `quantize_activation` / `_quant_act` (tybok/policies/pi05/models/triton_prefill_mlp.py:26-59,103-114),
+ * `_quant_act_fp8_kernel` (tybok/policies/pi05/models/triton_expert_mlp_fp8.py:234-277) and `quantize_act`
+ * (tybok/policies/fastwam/models/fp8_linear.py:223-243: `sa = amax/448; a8 = RNE(x/sa)`).
+ *   mode 0: the recipe above.  mode 1: the arithmetic of the prefill path's torch expression on bf16 tensors --
+ *           the scale rounded to bf16 and the quotient rounded to bf16 before the fp8 cast
+ *           (triton_prefill_mlp.py:30-36); sa then holds the bf16 value as fp32.
+ *   x: bf16 [M, K], pitch ldx (elements, a multiple of 8), 16-byte aligned; a8: [M, K] bytes, pitch lda (a multiple
+ *   of 8), 8-byte aligned; sa: fp32 [M]; K a multiple of 8, at most 16384. */
+int tk_quant_act_rows(const void* x, int ldx, void* a8, int lda, void* sa, int M, int K, int mode, void* stream);
+
+/* y[M, N] = bf16( (a8[M, K] . W8[N, K]^T) * sa[m] * sw[n] )  (+ residual: bf16(y + resid))
+ * e4m3fn activations and weights multiplied on the fp8 matrix instruction, fp32 accumulate.  Replaces `_w8a8_gemm`
+ * / `w8a8_gemm` (tybok/policies/pi05/models/triton_prefill_mlp.py:62-130).  Built for many rows (block tile
+ * 128 x 256: the VLM prefill); w_packed as for tk_fp8w_gemm; lda in bytes, a multiple of 16; N and ldy
+ * multiples of 4; split_k 0 = automatic (K splits hand fp32 partials through the workspace, fixed order). */
+int tk_w8a8_gemm(const void* a8, int lda, const void* sa, const void* w_packed, const void* w_scale, void* y, int ldy,
+                 const void* resid, int ldr, int resid_dtype, int M, int N, int K, int split_k, void* ws, size_t ws_bytes,
+                 void* stream);
+
+/* The prefill MLP in W8A8, `make_fp8_mlp_forward` (tybok/policies/pi05/models/triton_prefill_mlp.py:145-166):
+ *   (x8, sx) = quant(x);  g = w8a8(x8, Wg), u = w8a8(x8, Wu)  (bf16 each);  h = bf16(bf16(act(g)) * u);
+ *   (h8, sh) = quant(h);  y = w8a8(h8, Wd)  (+ residual)
+ * in four launches (quantise, gate/up with the gated epilogue, quantise, down); quantised copies and the [M, I]
+ * intermediate live in the workspace.  Arguments as tk_fp8w_gated_ffn (no per-column gate). */
+int tk_w8a8_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void* sg, const void* su, const void* wd_packed,
+                      const void* sd, void* y, int ldy, const void* resid, int ldr, int resid_dtype, int M, int K, int I,
+                      int act, void* ws, size_t ws_bytes, void* stream);
+
 /* ---- bf16-weight expert projections (norm prologue, rotary epilogue, residual epilogue) ----- */
 /* Bytes of a packed bf16 [N, K] weight (2 KiB per 32x32 tile). */
 size_t tk_bf16w_packed_bytes(int N, int K);

@@ -64,6 +64,52 @@ def gated_ffn(
 
 
 # --------------------------------------------------------------------------- #
+# W8A8 tier: per-token activation quantisation, fp8 x fp8 linear, the prefill MLP
+# --------------------------------------------------------------------------- #
+FP8 = torch.float8_e4m3fn
+
+
+def quantize_activation_rows(x: torch.Tensor, mode: str = "fp32") -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-token e4m3fn quantisation of ``x [M, K]`` -> ``(a8 [M, K] float8_e4m3fn, sa [M] fp32)``.
+
+    ``"fp32"``: ``sa = amax_k|x| / 448`` in fp32 and ``a8 = RNE(x / sa)`` from the fp32 quotient, one
+    rounding (tybok/policies/fastwam/models/fp8_linear.py:223-243; the expert path's kernel multiplies by
+    ``448 / amax`` instead: tybok/policies/pi05/models/triton_expert_mlp_fp8.py:268-274); an all-zero row
+    gives ``sa = 0`` and zero codes.
+    ``"bf16"``: the prefill path's torch expression evaluated on bf16 tensors -- the scale and the quotient
+    are bf16 values before the fp8 cast (tybok/policies/pi05/models/triton_prefill_mlp.py:30-36,103-114).
+    """
+    if mode == "bf16":
+        s = x.to(BF16).abs().amax(dim=-1, keepdim=True) / 448.0  # a bf16 tensor
+        q = torch.where(s > 0, x.to(BF16) / s, torch.zeros((), dtype=BF16))
+        return q.to(FP8), s.float().squeeze(-1)
+    x32 = x.float()
+    amax = x32.abs().amax(dim=-1, keepdim=True)
+    sa = amax / 448.0
+    q = torch.where(amax > 0, x32 / sa, torch.zeros(()))
+    return q.to(FP8), sa.squeeze(-1)
+
+
+def lin_w8a8(a8: torch.Tensor, sa: torch.Tensor, w8: torch.Tensor, sw: torch.Tensor) -> torch.Tensor:
+    """``bf16((a8 @ W8^T) * sa[:, None] * sw[None, :])``: fp8 x fp8 products (exact in fp32), fp32
+    accumulation, both scales on the accumulator, one bf16 rounding
+    (tybok/policies/pi05/models/triton_prefill_mlp.py:62-91)."""
+    acc = a8.float() @ w8.float().t()
+    return (acc * sa.float()[:, None] * sw.float()[None, :]).to(BF16)
+
+
+def gated_ffn_w8a8(x, wg8, sg, wu8, su, wd8, sd, act: str = "gelu_tanh", mode: str = "fp32") -> torch.Tensor:
+    """The W8A8 MLP, `make_fp8_mlp_forward` (tybok/policies/pi05/models/triton_prefill_mlp.py:145-166): gate and up
+    share the quantised input, ``act(gate) * up`` elementwise in bf16, a second per-token quantisation, down."""
+    x8, sx = quantize_activation_rows(x, mode)
+    g = lin_w8a8(x8, sx, wg8, sg)
+    u = lin_w8a8(x8, sx, wu8, su)
+    h = act_fn(act, g) * u
+    h8, sh = quantize_activation_rows(h, mode)
+    return lin_w8a8(h8, sh, wd8, sd)
+
+
+# --------------------------------------------------------------------------- #
 # norms
 # --------------------------------------------------------------------------- #
 def rms_norm_llama(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:

@@ -243,3 +243,80 @@ def test_gemma_attention_core_matches_eager_within_bf16_noise():
     b = ops.expert_attention(q, k_pre, v_pre, k_suf, v_suf, pad, ops.MASK_BIDIR, bf16_logits=True)
     assert a.shape == b.shape == (7, 8 * 256)
     assert float((a.float() - b.float()).abs().max()) < 5e-2
+
+
+# --------------------------------------------------------------------------- #
+# W8A8 tier: per-token activation quantisation and the fp8 x fp8 linear
+# --------------------------------------------------------------------------- #
+def test_activation_quantisation_closed_forms():
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(37, 96, generator=g) * torch.logspace(-3, 2, 37)[:, None]).to(BF16)
+    x[5] = 0.0  # an all-zero token
+    a8, sa = ops.quantize_activation_rows(x)
+    amax = x.float().abs().amax(dim=-1)
+    # the scale is amax / 448 exactly, the largest element of a row takes the largest code
+    assert torch.equal(sa, amax / 448.0)
+    vals = fp8.decode_e4m3fn(a8.view(torch.uint8))
+    assert torch.equal(vals.abs().amax(dim=-1)[amax > 0], torch.full((36,), 448.0))
+    assert sa[5] == 0 and (a8[5].view(torch.uint8) == 0).all()
+    # the codes are the round-to-nearest-even of x / sa: an encoder written from the format's definition agrees
+    live = amax > 0
+    want = fp8.encode_e4m3fn_rne(x.float()[live] / sa[live, None]).reshape(-1, 96)
+    assert torch.equal(a8[live].view(torch.uint8), want.to(torch.uint8))
+    # ... so the dequantised value is within half a quantum of the input: |a8 * sa - x| <= sa * 2^(e-4),
+    # e = exponent of the code's binade, 2^-9 * sa / 2 for the subnormal codes
+    e = torch.floor(torch.log2(vals.abs().clamp(min=2.0**-6)))
+    half_quantum = sa[:, None] * torch.exp2(e - 4.0)
+    assert bool(((vals * sa[:, None] - x.float()).abs() <= half_quantum * (1 + 1e-6)).all())
+    # scaling a token by a power of two scales its scale and keeps its codes (an exponent shift is exact)
+    a8b, sab = ops.quantize_activation_rows((x.float() * 8.0).to(BF16))
+    assert torch.equal(a8b.view(torch.uint8), a8.view(torch.uint8)) and torch.equal(sab, sa * 8.0)
+
+
+def test_activation_quantisation_bf16_mode_rounds_scale_and_quotient():
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(9, 64, generator=g).to(BF16) * 3.0
+    a8, sa = ops.quantize_activation_rows(x, mode="bf16")
+    # the scale is a bf16 value, within half a bf16 step of amax / 448
+    assert torch.equal(sa, sa.to(BF16).float())
+    exact = x.float().abs().amax(dim=-1) / 448.0
+    assert bool(((sa - exact).abs() <= exact * 2.0**-8).all())
+    # codes: fp8 of the bf16-rounded quotient by that scale
+    want = (x.float() / sa[:, None]).to(BF16).to(ops.FP8)
+    assert torch.equal(a8.view(torch.uint8), want.view(torch.uint8))
+    # the two modes differ (double rounding, rounded scale): the fixture tells them apart
+    a8f, _ = ops.quantize_activation_rows(x)
+    assert not torch.equal(a8f.view(torch.uint8), a8.view(torch.uint8))
+
+
+def test_w8a8_linear_against_float64_and_scale_placement():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(11, 128, generator=g).to(BF16)
+    w8, sw = fp8.quantize_weight_rows(torch.randn(24, 128, generator=g) * 0.02)
+    a8, sa = ops.quantize_activation_rows(x)
+    got = ops.lin_w8a8(a8, sa, w8, sw)
+    ref = (a8.double() @ w8.double().t()) * sa.double()[:, None] * sw.double()[None, :]
+    assert got.dtype == BF16
+    assert bool(((got.double() - ref).abs() <= ref.abs() * 2.0**-8 + 1e-30).all())  # one bf16 rounding of the exact value
+    # both scales sit on the accumulator: doubling a token's scale doubles that output row only
+    sa2 = sa.clone()
+    sa2[3] *= 2.0
+    got2 = ops.lin_w8a8(a8, sa2, w8, sw)
+    assert torch.equal(got2[3].float(), got[3].float() * 2.0) and torch.equal(got2[:3], got[:3])
+    # and the result is close to the unquantised product (e4m3 keeps 3-4 bits per factor)
+    full = x.double() @ (w8.double() * sw.double()[:, None]).t()
+    assert float((got.double() - full).abs().max()) <= 0.08 * float(full.abs().max())
+
+
+def test_w8a8_ffn_composition():
+    # gate and up share one quantised input; the intermediate is re-quantised per token before the down projection
+    x, wg8, sg, wu8, su, wd8, sd = ffn_case(13, 64, 96, seed=2)
+    y = ops.gated_ffn_w8a8(x, wg8, sg, wu8, su, wd8, sd, "gelu_tanh")
+    x8, sx = ops.quantize_activation_rows(x)
+    h = ops.act_fn("gelu_tanh", ops.lin_w8a8(x8, sx, wg8, sg)) * ops.lin_w8a8(x8, sx, wu8, su)
+    assert h.dtype == BF16
+    h8, sh = ops.quantize_activation_rows(h)
+    assert torch.equal(y, ops.lin_w8a8(h8, sh, wd8, sd))
+    # within quantisation noise of the weight-only FFN
+    wo = ops.gated_ffn(x, wg8, sg, wu8, su, wd8, sd, "gelu_tanh")
+    assert float((y.float() - wo.float()).abs().max()) <= 0.1 * float(wo.float().abs().max()) + 1e-3

@@ -366,6 +366,122 @@ int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void
                      ws, ws_bytes, (hipStream_t)stream);
 }
 
+// ---- W8A8 tier ---------------------------------------------------------------------------------
+namespace {
+int w8a8_common(const void* a8, int lda, const float* sa, const void* w_packed, const float* s0, const float* s1, void* y, int ldy,
+                const void* resid, int ldr, int resid_dtype, int M, int N, int K, int split_k, int act, void* ws, size_t ws_bytes,
+                hipStream_t st) {
+  if (M <= 0 || N <= 0 || K <= 0) return fail(TK_EINVAL, "w8a8: non-positive shape M=%d N=%d K=%d", M, N, K);
+  if (K % 16) return fail(TK_EINVAL, "w8a8: K=%d must be a multiple of 16", K);
+  if (lda % 16 || lda < K) return fail(TK_EINVAL, "w8a8: lda=%d must be >= K and a multiple of 16 (bytes)", lda);
+  if (!a8 || !sa || !w_packed || !s0 || !y) return fail(TK_EINVAL, "w8a8: null pointer");
+  if (!aligned16(a8) || !aligned16(w_packed) || !aligned16(s0) || (s1 && !aligned16(s1))) return fail(TK_EINVAL, "w8a8: a8, w_packed and the weight scales must be 16-byte aligned");
+  if (N % 4 || ldy % 4 || ldy < N || !aligned8(y)) return fail(TK_EINVAL, "w8a8: N=%d and ldy=%d must be multiples of 4, ldy >= N, y 8-byte aligned", N, ldy);
+  if (s1 && N % 32) return fail(TK_EINVAL, "w8a8 gated: I=%d must be a multiple of 32", N);
+  if (resid && resid_dtype != TK_BF16 && resid_dtype != TK_F32) return fail(TK_EINVAL, "w8a8: bad resid_dtype");
+  if (resid && (ldr < N || ldr % 4 || !(resid_dtype == TK_F32 ? aligned16(resid) : aligned8(resid)))) return fail(TK_EINVAL, "w8a8: residual pitch / alignment");
+  GemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.x = a8;
+  a.ldx = lda;
+  a.row_scale = sa;
+  a.w = (const uint8_t*)w_packed;
+  a.s0 = s0;
+  a.s1 = s1;
+  a.y = (u16*)y;
+  a.ldy = ldy;
+  a.resid = resid;
+  a.ldr = ldr;
+  a.resid_f32 = resid_dtype == TK_F32;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.KT = (K + 31) / 32;
+  a.ntiles = ((N + 31) / 32) * (s1 ? 2 : 1);
+  a.act = act;
+  a.vec = 1;
+  const int blocks0 = ((a.ntiles * 32 + tk_w8a8_cols() - 1) / tk_w8a8_cols()) * ((M + tk_w8a8_rows() - 1) / tk_w8a8_rows());
+  int ks = split_k;
+  if (ks <= 0) {
+    // fill the device once; a split keeps at least 32 k tiles and its partials must fit
+    ks = device_cus() / blocks0;
+    if (ks > a.KT / 32) ks = a.KT / 32;
+    if (ks < 1) ks = 1;
+  }
+  const size_t per_split = (size_t)tk_w8a8_rows() * tk_w8a8_cols() * 4;
+  if (ks > 1) {
+    const size_t have = ws && ws_bytes > kPartialOff ? (ws_bytes - kPartialOff < kPartialBytes ? ws_bytes - kPartialOff : kPartialBytes) / (per_split * blocks0) : 0;
+    if ((size_t)ks > have || blocks0 > kMaxCounters) {
+      if (split_k > 1) return fail(TK_EWORKSPACE, "w8a8: split_k=%d needs %zu bytes of partial space", ks, per_split * blocks0 * ks);
+      ks = have > 1 && blocks0 <= kMaxCounters ? (int)have : 1;
+    }
+  }
+  if (ks > a.KT) ks = a.KT;
+  a.ksplit = ks;
+  a.kt_q = a.KT / ks;
+  a.kt_r = a.KT % ks;
+  a.partial = ks > 1 ? (float*)((char*)ws + kPartialOff) : nullptr;
+  a.counters = ks > 1 ? (int*)ws : nullptr;
+  if (tk_launch_w8a8_gemm(a, st)) return fail(TK_ELAUNCH, "w8a8: launch failed (%s)", hipGetErrorString(hipGetLastError()));
+  return TK_OK;
+}
+}  // namespace
+
+int tk_quant_act_rows(const void* x, int ldx, void* a8, int lda, void* sa, int M, int K, int mode, void* stream) {
+  if (M <= 0 || K <= 0 || K % 8 || K > tk_quant_act_max_k()) return fail(TK_EINVAL, "quant_act_rows: bad shape M=%d K=%d (K a multiple of 8, at most %d)", M, K, tk_quant_act_max_k());
+  if (!x || !a8 || !sa || ldx < K || ldx % 8 || lda < K || lda % 8) return fail(TK_EINVAL, "quant_act_rows: null pointer or row pitch not a multiple of 8 >= K");
+  if (!aligned16(x) || !aligned8(a8)) return fail(TK_EINVAL, "quant_act_rows: x must be 16-byte and a8 8-byte aligned");
+  if (mode != 0 && mode != 1) return fail(TK_EINVAL, "quant_act_rows: mode %d (0 = fp32 scale, 1 = bf16 scale and quotient)", mode);
+  QuantActArgs q;
+  q.x = (const u16*)x;
+  q.ldx = ldx;
+  q.a8 = (unsigned char*)a8;
+  q.lda = lda;
+  q.sa = (float*)sa;
+  q.M = M;
+  q.K = K;
+  q.mode = mode;
+  if (tk_launch_quant_act_rows(q, (hipStream_t)stream)) return fail(TK_ELAUNCH, "quant_act_rows: launch failed");
+  return TK_OK;
+}
+
+int tk_w8a8_gemm(const void* a8, int lda, const void* sa, const void* w_packed, const void* w_scale, void* y, int ldy,
+                 const void* resid, int ldr, int resid_dtype, int M, int N, int K, int split_k, void* ws, size_t ws_bytes,
+                 void* stream) {
+  return w8a8_common(a8, lda, (const float*)sa, w_packed, (const float*)w_scale, nullptr, y, ldy, resid, ldr, resid_dtype, M, N, K,
+                     split_k, 0, ws, ws_bytes, (hipStream_t)stream);
+}
+
+int tk_w8a8_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void* sg, const void* su, const void* wd_packed,
+                      const void* sd, void* y, int ldy, const void* resid, int ldr, int resid_dtype, int M, int K, int I,
+                      int act, void* ws, size_t ws_bytes, void* stream) {
+  if (act != TK_ACT_SILU && act != TK_ACT_GELU_TANH) return fail(TK_EINVAL, "w8a8 ffn: unknown activation %d", act);
+  if (M <= 0 || K <= 0 || I <= 0 || I % 32 || K % 16) return fail(TK_EINVAL, "w8a8 ffn: bad shape M=%d K=%d I=%d (K a multiple of 16, I of 32)", M, K, I);
+  if (!sg || !su || !sd) return fail(TK_EINVAL, "w8a8 ffn: null scale pointer");
+  if (!ws) return fail(TK_EWORKSPACE, "w8a8 ffn: needs a workspace");
+  // workspace: quantised input + its scales in the norm region; bf16 intermediate, its codes and scales in the hidden region
+  const size_t a8_bytes = (size_t)M * K, sa_bytes = (((size_t)M * 4) + 255) / 256 * 256;
+  const size_t h_bytes = (size_t)M * I * 2, h8_bytes = (size_t)M * I;
+  if (a8_bytes + sa_bytes > kNormBytes || h_bytes + h8_bytes + sa_bytes > kHiddenBytes || ws_bytes < kHiddenOff + h_bytes + h8_bytes + sa_bytes)
+    return fail(TK_EWORKSPACE, "w8a8 ffn: workspace too small for M=%d K=%d I=%d", M, K, I);
+  char* base = (char*)ws;
+  void* a8 = base + kNormOff;
+  void* sa = base + kNormOff + (a8_bytes + 255) / 256 * 256;
+  if ((a8_bytes + 255) / 256 * 256 + sa_bytes > kNormBytes) return fail(TK_EWORKSPACE, "w8a8 ffn: workspace too small for the quantised input");
+  void* h = base + kHiddenOff;
+  void* h8 = base + kHiddenOff + (h_bytes + 255) / 256 * 256;
+  void* sh = base + kHiddenOff + (h_bytes + 255) / 256 * 256 + (h8_bytes + 255) / 256 * 256;
+  if ((size_t)((char*)sh - base) + sa_bytes > ws_bytes) return fail(TK_EWORKSPACE, "w8a8 ffn: workspace too small for the intermediate");
+  hipStream_t st = (hipStream_t)stream;
+  int rc = tk_quant_act_rows(x, ldx, a8, K, sa, M, K, 0, stream);
+  if (rc) return rc;
+  rc = w8a8_common(a8, K, (const float*)sa, wgu_packed, (const float*)sg, (const float*)su, h, I, nullptr, 0, 0, M, I, K, 0, act, ws, ws_bytes, st);
+  if (rc) return rc;
+  rc = tk_quant_act_rows(h, I, h8, I, sh, M, I, 0, stream);
+  if (rc) return rc;
+  return w8a8_common(h8, I, (const float*)sh, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, M, K, I, 0, 0, ws, ws_bytes, st);
+}
+
 size_t tk_bf16w_packed_bytes(int N, int K) {
   if (N <= 0 || K <= 0) return 0;
   return (size_t)((N + 31) / 32) * ((K + 31) / 32) * 2048;

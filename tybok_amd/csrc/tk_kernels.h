@@ -45,6 +45,18 @@ struct GemmArgs {
   unsigned short* vt;
   int vt_col0;
   int vt_ld;
+  // W8A8 launches only: x holds e4m3fn codes (ldx in bytes) and row_scale the per-token fp32 scales
+  const float* row_scale;
+};
+
+struct QuantActArgs {
+  const unsigned short* x;  // bf16 [M, K], element pitch ldx
+  int ldx;
+  unsigned char* a8;  // e4m3fn [M, K], byte pitch lda
+  int lda;
+  float* sa;  // fp32 [M]
+  int M, K;
+  int mode;  // 0: fp32 scale, one rounding; 1: bf16-rounded scale and quotient
 };
 
 struct AttnArgs {
@@ -185,6 +197,12 @@ int tk_wide_cols();
 int tk_launch_gemm_wide(GemmArgs a, hipStream_t st);
 int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st);
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st);
+// W8A8 tier: per-token activation quantisation and the fp8 x fp8 many-row GEMM (block tile tk_w8a8_rows() x tk_w8a8_cols())
+int tk_w8a8_rows();
+int tk_w8a8_cols();
+int tk_quant_act_max_k();
+int tk_launch_w8a8_gemm(GemmArgs a, hipStream_t st);
+int tk_launch_quant_act_rows(QuantActArgs a, hipStream_t st);
 int tk_launch_pack(const void* w0, const void* w1, void* out, int N, int K, int interleave, hipStream_t st);
 int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st);
 int tk_launch_fill_zero(int* p, int n, hipStream_t st);

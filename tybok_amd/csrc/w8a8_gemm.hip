@@ -1,0 +1,376 @@
+// W8A8 tier of the VLM prefill MLP on gfx950: per-token activation quantisation and the fp8 x fp8 GEMM.
+//
+//   quant_act_rows_kernel   x[M,K] bf16 -> a8[M,K] e4m3fn, sa[M] fp32 with sa = amax_k|x| / 448 and
+//                           a8 = RNE(x / sa) in fp32 (one rounding); an all-zero row gives sa = 0 and zero codes.
+//   w8a8_wide_kernel<EPI>   y[M,N] = bf16((a8 . W8^T) * sa[m] * sw[n]) on v_mfma_f32_32x32x64_f8f6f4 (e4m3 x e4m3,
+//                           fp32 accumulate, 64 k per instruction).  Same packed weight tiles and the same block
+//                           shape as the weight-only many-row kernel: 4 waves own 128 rows x 256 packed columns,
+//                           wave w the n tiles 2w, 2w+1 for all rows; weights go straight from global memory into
+//                           operand registers (a lane's 16-byte chunks of two consecutive k tiles are one 32-byte
+//                           operand), the quantised activations of a round (128 rows x 128 k) are staged once per
+//                           block through LDS as bytes -- half the LDS traffic per k of the bf16 kernel at twice
+//                           the product rate.  The order of k inside an instruction is the same permutation for both
+//                           operands (bytes 0-15 of a lane: k tile 2s, bytes 16-31: k tile 2s+1), which a dot
+//                           product does not see.
+#include "tk_common.h"
+#include "tk_kernels.h"
+
+namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+constexpr int MT = 4;   // m tiles per block (and per wave)
+constexpr int NT = 2;   // n tiles per wave
+constexpr int NW = 4;   // waves per block
+constexpr int RK = 4;   // 32-wide k tiles per round (two 64-wide product steps)
+constexpr int PF = 3;   // rounds in flight
+
+// EPI: 0 plain (scales, optional residual), 1 gated (gate/up tile pairs -> act(g) * u).
+template <int EPI>
+__global__ __launch_bounds__(NW * 64) void w8a8_wide_kernel(GemmArgs a, int nblk_m, int ngroups) {
+  constexpr int ROWS = MT * 32;
+  constexpr int ROWB = RK * 32;            // bytes of one staged (fp8) activation row per round
+  constexpr int PITCH = ROWB + 16;
+  constexpr int XBUF = ROWS * PITCH;
+  constexpr int PPR = ROWB / 16;           // 16-byte pieces per staged row
+  constexpr int XPT = ROWS * PPR / (NW * 64);
+  constexpr int TILES = MT * NT;
+  constexpr int STEPS = RK / 2;            // 64-wide product steps per round
+  __shared__ __align__(16) unsigned char lds[2 * XBUF];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5;
+  const int l32 = lane & 31;
+
+  // blocks that share weights (same n tiles and k range, different rows) get consecutive slots of one XCD
+  const unsigned id = blockIdx.x;
+  const unsigned slot = id >> 3;
+  const int mblock = (int)(slot % (unsigned)nblk_m);
+  const int group = (int)((slot / (unsigned)nblk_m) * 8 + (id & 7));
+  if (group >= ngroups) return;
+  const int split = group % a.ksplit;
+  const int nblk = group / a.ksplit;
+
+  const int kt_lo = split * a.kt_q + (split < a.kt_r ? split : a.kt_r);
+  const int kt_hi = kt_lo + a.kt_q + (split < a.kt_r ? 1 : 0);
+  const int nrounds = (kt_hi - kt_lo + RK - 1) / RK;
+  const int k_end = kt_hi * 32 < a.K ? kt_hi * 32 : a.K;
+
+  const int strip = nblk * NW + wave;
+  const uint8_t* wbase[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    int ntg = strip * NT + nt;
+    if (ntg > a.ntiles - 1) ntg = a.ntiles - 1;  // overhanging tiles are computed on valid data, never stored
+    wbase[nt] = a.w + ((size_t)ntg * a.KT) * 1024 + lane * 16;
+  }
+
+  const char* xsrc[XPT];
+  int xcol[XPT], xdst[XPT];
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) {
+    const int p = tid + i * NW * 64;
+    const int r = p / PPR, c = p % PPR;
+    int m = mblock * ROWS + r;
+    if (m > a.M - 1) m = a.M - 1;  // rows past M: valid data, never stored
+    xsrc[i] = (const char*)a.x + (size_t)m * a.ldx;  // one byte per element
+    xcol[i] = c * 16;
+    xdst[i] = r * PITCH + c * 16;
+  }
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
+
+  struct WFrag {
+    i32x4 w[RK][NT];
+  };
+  struct XFrag {
+    i32x4 v[XPT];
+  };
+  auto wload = [&](WFrag& f, int r) {
+#pragma unroll
+    for (int j = 0; j < RK; ++j) {
+      int kt = kt_lo + r * RK + j;
+      if (kt > a.KT - 1) kt = a.KT - 1;  // its activation columns are zeroed
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) f.w[j][nt] = *(const i32x4*)(wbase[nt] + (size_t)kt * 1024);
+    }
+  };
+  auto xload = [&](XFrag& f, int r) {
+    const int k0 = (kt_lo + r * RK) * 32;
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) {
+      int k = k0 + xcol[i];
+      if (k > a.K - 16) k = a.K - 16;
+      f.v[i] = *(const i32x4*)(xsrc[i] + k);
+    }
+  };
+  auto xstore = [&](const XFrag& f, int r, int b) {
+    const int k0 = (kt_lo + r * RK) * 32;
+    const i32x4 z = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) *(i32x4*)(lds + b * XBUF + xdst[i]) = (k0 + xcol[i]) < k_end ? f.v[i] : z;
+  };
+  auto step = [&](const WFrag& f, int b, int s) {
+    i32x8 xa[MT], wb[NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const unsigned char* p = lds + b * XBUF + (mt * 32 + l32) * PITCH + s * 64 + 16 * half;
+      const i32x4 lo = *(const i32x4*)p, hi = *(const i32x4*)(p + 32);
+      xa[mt] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const i32x4 lo = f.w[2 * s][nt], hi = f.w[2 * s + 1][nt];
+      wb[nt] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wb[nt], xa[mt], acc[mt][nt], 0, 0, 0, 0, 0, 0);
+  };
+
+  // PF rounds in flight, every load unconditional (clamped addresses; columns past the block's k range are
+  // zeroed when staged); one LDS barrier per round, the staging buffers alternate.
+  WFrag wbuf[PF];
+  XFrag xbuf[PF];
+#pragma unroll
+  for (int p = 0; p < PF; ++p) {
+    xload(xbuf[p], p);
+    wload(wbuf[p], p);
+  }
+  auto round = [&](int p, int r) {
+    xstore(xbuf[p], r, r & 1);
+    xload(xbuf[p], r + PF);
+    lds_barrier();
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) step(wbuf[p], r & 1, s);
+    wload(wbuf[p], r + PF);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  {
+    int it = 0;
+    for (; it + PF <= nrounds; it += PF) {
+#pragma unroll
+      for (int p = 0; p < PF; ++p) round(p, it + p);
+    }
+    const int rem = nrounds - it;  // in [0, PF)
+#pragma unroll
+    for (int q = 0; q < PF - 1; ++q)
+      if (q < rem) round(q, it + q);  // block-uniform
+  }
+
+  // ---- K-split hand-off: fp32 partials [(block, split)][wave][tile][group][lane][4], last arriver sums in split order
+  const int blk_lin = nblk * nblk_m + mblock;
+  if (a.ksplit > 1) {
+    unsigned long long* pbase = (unsigned long long*)a.partial + ((size_t)wave * TILES * 4 * 64 + lane) * 2;
+    unsigned long long* mine = pbase + ((size_t)blk_lin * a.ksplit + split) * (NW * TILES * 4 * 64 * 2);
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& c = acc[t / NT][t % NT];
+        unsigned long long* dst = mine + (size_t)(t * 4 + g) * 128;
+        st_agent64(dst, c[4 * g], c[4 * g + 1]);
+        st_agent64(dst + 1, c[4 * g + 2], c[4 * g + 3]);
+      }
+    __shared__ int s_last;
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0);  // the write-through stores are acknowledged: visible to every block
+    asm volatile("" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (old == a.ksplit - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
+    for (int s = 0; s < a.ksplit; ++s) {
+      const unsigned long long* src = pbase + ((size_t)blk_lin * a.ksplit + s) * (NW * TILES * 4 * 64 * 2);
+      unsigned long long raw[TILES][4][2];
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          raw[t][g][0] = ld_agent64(src + (size_t)(t * 4 + g) * 128);
+          raw[t][g][1] = ld_agent64(src + (size_t)(t * 4 + g) * 128 + 1);
+        }
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f32x16& c = acc[t / NT][t % NT];
+          c[4 * g] += __uint_as_float((unsigned)raw[t][g][0]);
+          c[4 * g + 1] += __uint_as_float((unsigned)(raw[t][g][0] >> 32));
+          c[4 * g + 2] += __uint_as_float((unsigned)raw[t][g][1]);
+          c[4 * g + 3] += __uint_as_float((unsigned)(raw[t][g][1] >> 32));
+        }
+    }
+  }
+
+  // ---- epilogue: lane l of a tile owns row m = l % 32 and, per register group g, columns 8g + 4*(l/32) .. +3;
+  // out = (acc * sa[m]) * sw[n], one bf16 rounding (the reference's `acc * a_scale[:, None] * w_scale[None, :]`)
+  float sa[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int m = (mblock * MT + mt) * 32 + l32;
+    if (m > a.M - 1) m = a.M - 1;
+    sa[mt] = a.row_scale[m];
+  }
+  if (EPI == 0) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n0 = (strip * NT + nt) * 32 + 8 * g + 4 * half;
+        if (n0 >= a.N) continue;
+        const f32x4 sc = *(const f32x4*)(a.s0 + n0);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const int m = (mblock * MT + mt) * 32 + l32;
+          if (m >= a.M) continue;
+          const f32x16& c = acc[mt][nt];
+          f32x4 v = {c[4 * g], c[4 * g + 1], c[4 * g + 2], c[4 * g + 3]};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] = mul_rn(mul_rn(v[j], sa[mt]), sc[j]);
+          i32x2 r = pack_bf16x4(v);
+          if (a.resid) {
+            const f32x4 rv = a.resid_f32 ? *(const f32x4*)((const float*)a.resid + (size_t)m * a.ldr + n0)
+                                         : unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n0));
+            r = pack_bf16x4(unpack_bf16x4(r) + rv);
+          }
+          *(i32x2*)(a.y + (size_t)m * a.ldy + n0) = r;
+        }
+      }
+  } else {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int col = strip * 32 + 8 * g + 4 * half;
+      if (col >= a.N) continue;
+      const f32x4 scg = *(const f32x4*)(a.s0 + col), scu = *(const f32x4*)(a.s1 + col);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = (mblock * MT + mt) * 32 + l32;
+        if (m >= a.M) continue;
+        const f32x16& cg = acc[mt][0];
+        const f32x16& cu = acc[mt][1];
+        f32x4 vg = {cg[4 * g], cg[4 * g + 1], cg[4 * g + 2], cg[4 * g + 3]};
+        f32x4 vu = {cu[4 * g], cu[4 * g + 1], cu[4 * g + 2], cu[4 * g + 3]};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          vg[j] = mul_rn(mul_rn(vg[j], sa[mt]), scg[j]);
+          vu[j] = mul_rn(mul_rn(vu[j], sa[mt]), scu[j]);
+        }
+        const f32x4 gg = unpack_bf16x4(pack_bf16x4(vg));
+        const f32x4 up = unpack_bf16x4(pack_bf16x4(vu));
+        f32x4 act;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) act[j] = a.act == 0 ? silu_f(gg[j]) : gelu_tanh_f(gg[j]);
+        act = unpack_bf16x4(pack_bf16x4(act));
+        *(i32x2*)(a.y + (size_t)m * a.ldy + col) = pack_bf16x4(act * up);
+      }
+    }
+  }
+}
+
+// One block per row.  MODE 0: sa = amax / 448 (fp32), a8 = RNE(x / sa) from fp32 -- one rounding.
+// MODE 1: the arithmetic of a torch expression on bf16 tensors, `s = x.abs().max() / 448` (a bf16 value) and
+// `(x / s).to(float8_e4m3fn)` (quotient rounded to bf16, then to fp8): sa = float(bf16(amax / 448)).
+constexpr int kQuantMaxPieces = 8;  // 16-byte pieces of a row per thread: K <= 8 * 256 * 8 = 16384
+__global__ __launch_bounds__(256) void quant_act_rows_kernel(QuantActArgs a) {
+  __shared__ float part[4];
+  const int tid = threadIdx.x;
+  const char* row = (const char*)a.x + (size_t)blockIdx.x * a.ldx * 2;
+  const int pieces = a.K / 8;
+  i32x4 v[kQuantMaxPieces];
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < kQuantMaxPieces; ++i) {
+    const int p = tid + i * 256;
+    v[i] = i32x4{0, 0, 0, 0};
+    if (p < pieces) v[i] = *(const i32x4*)(row + (size_t)p * 16);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const unsigned u = (unsigned)v[i][e];
+      amax = fmaxf(amax, fmaxf(fabsf(__uint_as_float(u << 16)), fabsf(__uint_as_float(u & 0xffff0000u))));
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  if ((tid & 63) == 0) part[tid >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+  float sa = amax / 448.0f;
+  if (a.mode == 1) sa = round_bf16(sa);
+  if (tid == 0) a.sa[blockIdx.x] = sa;
+  unsigned char* dst = (unsigned char*)a.a8 + (size_t)blockIdx.x * a.lda;
+#pragma unroll
+  for (int i = 0; i < kQuantMaxPieces; ++i) {
+    const int p = tid + i * 256;
+    if (p >= pieces) continue;
+    float q[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const unsigned u = (unsigned)v[i][e];
+      q[2 * e] = __uint_as_float(u << 16);
+      q[2 * e + 1] = __uint_as_float(u & 0xffff0000u);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float y = amax == 0.f ? 0.f : q[e] / sa;  // IEEE division, as the elementwise reference computes it
+      if (a.mode == 1) y = round_bf16(y);
+      q[e] = y;
+    }
+    // four fp32 -> four e4m3fn (RNE, saturating at +-448) per conversion pair
+    int lo = 0, hi = 0;
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], lo, false);
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], lo, true);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], hi, false);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], hi, true);
+    *(i32x2*)(dst + (size_t)p * 8) = i32x2{lo, hi};
+  }
+}
+
+}  // namespace
+
+int tk_w8a8_rows() { return MT * 32; }
+int tk_w8a8_cols() { return NW * NT * 32; }
+int tk_quant_act_max_k() { return kQuantMaxPieces * 256 * 8; }
+
+int tk_launch_w8a8_gemm(GemmArgs a, hipStream_t st) {
+  const int nblk_m = (a.M + MT * 32 - 1) / (MT * 32);
+  const int nblk_n = (a.ntiles + NW * NT - 1) / (NW * NT);
+  const int ngroups = nblk_n * a.ksplit;
+  const unsigned blocks = (unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m;
+  if (a.s1)
+    hipLaunchKernelGGL(w8a8_wide_kernel<1>, dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
+  else
+    hipLaunchKernelGGL(w8a8_wide_kernel<0>, dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int tk_launch_quant_act_rows(QuantActArgs a, hipStream_t st) {
+  hipLaunchKernelGGL(quant_act_rows_kernel, dim3(a.M), dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}

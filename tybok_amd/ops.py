@@ -236,6 +236,64 @@ def fp8w_gated_ffn(
     return out
 
 
+def quant_act_rows(x: torch.Tensor, mode: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-token e4m3fn quantisation of ``x [M, K]`` bf16 -> ``(a8 [M, K] float8_e4m3fn, sa [M] fp32)``."""
+    lib = native.lib()
+    if x.dtype != torch.bfloat16 or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
+        raise TypeError("activations must be a bf16 CUDA matrix with unit inner stride")
+    m, k = x.shape
+    a8 = torch.empty(m, k, dtype=torch.uint8, device=x.device)
+    sa = torch.empty(m, dtype=torch.float32, device=x.device)
+    native.check(lib.tk_quant_act_rows(x.data_ptr(), x.stride(0), a8.data_ptr(), k, sa.data_ptr(), m, k, int(mode), _stream()), "tk_quant_act_rows")
+    return a8.view(torch.float8_e4m3fn), sa
+
+
+def w8a8_gemm(
+    a8: torch.Tensor, sa: torch.Tensor, w: PackedWeight, *, resid: torch.Tensor | None = None, out: torch.Tensor | None = None,
+    split_k: int = 0, ws: Workspace | None = None,
+) -> torch.Tensor:  # fmt: skip
+    """``bf16((a8 @ W8^T) * sa[m] * sw[n])`` (``+ residual``) on the fp8 matrix instruction."""
+    lib = native.lib()
+    if a8.dtype == torch.float8_e4m3fn:
+        a8 = a8.view(torch.uint8)
+    if a8.dtype != torch.uint8 or a8.dim() != 2 or a8.shape[1] != w.k or a8.stride(1) != 1:
+        raise TypeError(f"a8 must be e4m3fn codes [M, {w.k}] with unit inner stride")
+    m = a8.shape[0]
+    if sa.dtype != torch.float32 or sa.numel() != m or not sa.is_contiguous():
+        raise ValueError("sa must be contiguous fp32 [M]")
+    if out is None:
+        out = torch.empty(m, w.n, dtype=torch.bfloat16, device=a8.device)
+    rp, ldr, rdt = _resid_args(resid, m, w.n)
+    ws = ws or default_workspace(a8.device)
+    rc = lib.tk_w8a8_gemm(
+        a8.data_ptr(), a8.stride(0), sa.data_ptr(), w.data.data_ptr(), w.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt,
+        m, w.n, w.k, split_k, ws.ptr, ws.nbytes, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_w8a8_gemm")
+    return out
+
+
+def w8a8_gated_ffn(
+    x: torch.Tensor, wgu: PackedGateUp, wd: PackedWeight, act: str = "gelu_tanh", *, resid: torch.Tensor | None = None,
+    out: torch.Tensor | None = None, ws: Workspace | None = None,
+) -> torch.Tensor:  # fmt: skip
+    """The W8A8 MLP: quantise, gate/up with the gated epilogue, quantise, down (``+ residual``)."""
+    lib = native.lib()
+    m, ldx = _check_act(x, wgu.k)
+    if wd.k != wgu.i or wd.n != wgu.k:
+        raise ValueError("down weight must be [K, I]")
+    if out is None:
+        out = torch.empty(m, wd.n, dtype=torch.bfloat16, device=x.device)
+    rp, ldr, rdt = _resid_args(resid, m, wd.n)
+    ws = ws or default_workspace(x.device)
+    rc = lib.tk_w8a8_gated_ffn(
+        x.data_ptr(), ldx, wgu.data.data_ptr(), wgu.scale_gate.data_ptr(), wgu.scale_up.data_ptr(), wd.data.data_ptr(),
+        wd.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt, m, wgu.k, wgu.i, ACT[act], ws.ptr, ws.nbytes, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_w8a8_gated_ffn")
+    return out
+
+
 def pack_bf16_weight(w: torch.Tensor, rope_half: int = 0) -> PackedBf16Weight:
     """Row-major bf16 ``[N, K]`` -> :class:`PackedBf16Weight` (once per model)."""
     lib = native.lib()
