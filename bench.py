@@ -128,7 +128,7 @@ def stream_read_us(window_bytes: int, blocks: int = 1024, launches: int = 100, r
     return e0.elapsed_time(e1) * 1e3 / (reps * launches)
 
 
-def ffn_launch_us(m: int, k: int, i: int, launches: int = 10, reps: int = 5) -> float:
+def ffn_launch_us(m: int, k: int, i: int, launches: int = 10, reps: int = 5, w8a8: bool = False) -> float:
     """Average duration (us) of one fp8-weight GeGLU FFN (gate/up + down) at many rows: the VLM prefill shape."""
     import torch
 
@@ -142,14 +142,15 @@ def ffn_launch_us(m: int, k: int, i: int, launches: int = 10, reps: int = 5) -> 
     out = torch.empty(m, k, dtype=torch.bfloat16, device="cuda")
     ws = tk.Workspace()
     stream = torch.cuda.Stream()
+    ffn = tk.w8a8_gated_ffn if w8a8 else tk.fp8w_gated_ffn
     with torch.cuda.stream(stream):
         for _ in range(3):
-            tk.fp8w_gated_ffn(xc, wgu, wd, "gelu_tanh", out=out, ws=ws)
+            ffn(xc, wgu, wd, "gelu_tanh", out=out, ws=ws)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
         for _ in range(launches):
-            tk.fp8w_gated_ffn(xc, wgu, wd, "gelu_tanh", out=out, ws=ws)
+            ffn(xc, wgu, wd, "gelu_tanh", out=out, ws=ws)
     spin_up(60.0)
     for _ in range(3):
         graph.replay()
@@ -361,6 +362,7 @@ def main() -> None:
     ap.add_argument("--attn-only", action="store_true", help="only the action-expert attention loop (for rocprofv3 runs)")
     ap.add_argument("--tower-attn-only", action="store_true", help="only the vision-tower attention loop, 3 cameras x 1024 tokens (for rocprofv3 runs)")
     ap.add_argument("--ffn-only", action="store_true", help="only the many-row (M=712) fp8 GeGLU FFN loop (for rocprofv3 runs)")
+    ap.add_argument("--w8a8", action="store_true", help="with --ffn-only: the W8A8 FFN (fp8 x fp8 matrix instruction) instead of the weight-only one")
     ap.add_argument("--request-only", choices=("smolvla", "pi05"), help="only the requests of one model, all tiers, graph replay (for rocprofv3 runs)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -389,8 +391,8 @@ def main() -> None:
         return
     if args.ffn_only:
         spin_up()
-        us = ffn_launch_us(712, 2048, 16384, launches=5, reps=args.steps)
-        print(json.dumps({"ffn_only": {"M": 712, "K": 2048, "I": 16384, "us": round(us, 1), "TFLOPs": round(6.0 * 712 * 2048 * 16384 / us / 1e6, 1)}}), flush=True)
+        us = ffn_launch_us(712, 2048, 16384, launches=5, reps=args.steps, w8a8=args.w8a8)
+        print(json.dumps({"ffn_only": {"M": 712, "K": 2048, "I": 16384, "w8a8": bool(args.w8a8), "us": round(us, 1), "TFLOPs": round(6.0 * 712 * 2048 * 16384 / us / 1e6, 1)}}), flush=True)
         return
     if args.tower_attn_only:
         spin_up()
@@ -441,7 +443,7 @@ def main() -> None:
     torch.cuda.empty_cache()
 
     # ---- pi0.5-shaped chunk ----
-    pi05_p50 = None
+    pi05_p50 = pi05_w8a8_p50 = None
     if not args.skip_pi05:
         ckpt5 = write_pi05_checkpoint(os.path.join(tmp, "pi05"), cameras=2, seed=0)
         flags5 = {k: v for k, v in flags.items() if k not in ("tl_llm_fused_attn", "tl_vit_oproj")}  # SmolVLA-only tiers
@@ -451,6 +453,13 @@ def main() -> None:
         frame5 = device_frame(eng5, 2)
         s5, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
         pi05_p50 = float(np.percentile(s5, 50))
+        del eng5
+        torch.cuda.empty_cache()
+        # the same request with the VLM MLP in W8A8 (activations quantised per token, fp8 x fp8 products): the
+        # arithmetic of the reference's own --tl-fp8-llm-mlp tier; an opt-in drift tier here
+        eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **{**flags5, "tl_fp8_llm_mlp": "w8a8"})
+        s5w, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
+        pi05_w8a8_p50 = float(np.percentile(s5w, 50))
         del eng5
         torch.cuda.empty_cache()
 
@@ -497,11 +506,15 @@ def main() -> None:
     fm, fk, fi = 712, 2048, 16384
     f_us = ffn_launch_us(fm, fk, fi)
     f_tflops = 6.0 * fm * fk * fi / f_us / 1e6
+    f8_us = ffn_launch_us(fm, fk, fi, w8a8=True)
+    f8_tflops = 6.0 * fm * fk * fi / f8_us / 1e6
     prefill_ffn = {
         "shape": {"M": fm, "K": fk, "I": fi},
         "us": round(f_us, 1),
         "TFLOPs": round(f_tflops, 1),
         "frac_of_bf16_mfma_peak": round(f_tflops / 2500.0, 4),
+        "w8a8": {"us": round(f8_us, 1), "TFLOPs": round(f8_tflops, 1), "frac_of_fp8_mfma_peak": round(f8_tflops / 5000.0, 4),
+                 "what": "quantise + gate/up + quantise + down, fp8 x fp8 matrix instruction"},
     }
 
     # ---- the single-op configurations at the action-chunk shape: latency-bound launches ----
@@ -561,6 +574,7 @@ def main() -> None:
         "smolvla_3cam_host_inputs_p50_ms": round(float(np.percentile(samples_host, 50)), 3),
         "pi05_2cam_p50_ms": None if pi05_p50 is None else round(pi05_p50, 3),
         "pi05_tiers": "tl_fused_expert, tl_fp8_expert_mlp, tl_fp8_llm_mlp, tl_llm_flash_attn, tl_fused_vit",
+        "pi05_2cam_w8a8_prefill_p50_ms": None if pi05_w8a8_p50 is None else round(pi05_w8a8_p50, 3),
         "gemm_sweep_M50": sweep,
         "ops_action_chunk_shape": ops_small,
         "pi05_prefill_ffn_M712": prefill_ffn,

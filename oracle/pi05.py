@@ -63,6 +63,9 @@ class PI05Shape:
     #                  probabilities rounded to bf16 for P.V (fp32 accumulate, bf16 result).
     vit_mlp_dtype: torch.dtype | None = None
     vit_lowp_attn: bool = False
+    # W8A8 tier of the VLM MLP (tybok/policies/pi05/models/triton_prefill_mlp.py:145-166): activations quantised
+    # per token as well; only with the VLM MLP's weights in fp8 (``fp8_linear_names(..., llm_mlp=True, ...)``)
+    llm_w8a8: bool = False
 
 
 def fp8_linear_names(shape: PI05Shape, llm_mlp: bool, expert_mlp: bool) -> frozenset:
@@ -147,6 +150,13 @@ def _mlp(w: Weights, prefix: str, x):
     return w.linear(prefix + "down_proj", F.gelu(w.linear(prefix + "gate_proj", x), approximate="tanh") * w.linear(prefix + "up_proj", x))
 
 
+def _mlp_w8a8(w: Weights, prefix: str, x):
+    """The W8A8 forward of one GeGLU MLP: both operands of every product in e4m3fn."""
+    q = [w.quantised(prefix + n) for n in ("gate_proj", "up_proj", "down_proj")]
+    y = ops.gated_ffn_w8a8(x.reshape(-1, x.shape[-1]), *q[0], *q[1], *q[2], "gelu_tanh")
+    return y.reshape(*x.shape[:-1], y.shape[-1])
+
+
 def prefill(w: Weights, shape: PI05Shape, embs, pad_masks, att_masks):
     """VLM prefill -> per-layer post-RoPE ``(K, V)`` bf16 ``[1, G, P, D]``."""
     mask = ops.make_att_2d_masks(pad_masks, att_masks)
@@ -162,7 +172,7 @@ def prefill(w: Weights, shape: PI05Shape, embs, pad_masks, att_masks):
         kv.append((k, v))
         hidden = hidden + a
         h, _ = ops.gemma_rms_norm(hidden, EPS, weight=w[p + "post_attention_layernorm.weight"])
-        hidden = hidden + _mlp(w, p + "mlp.", h)
+        hidden = hidden + (_mlp_w8a8(w, p + "mlp.", h) if shape.llm_w8a8 else _mlp(w, p + "mlp.", h))
     return kv
 
 

@@ -101,15 +101,20 @@ class Weights:
     def __getitem__(self, name: str) -> torch.Tensor:
         return self.sd[name]
 
+    def quantised(self, prefix: str) -> tuple[torch.Tensor, torch.Tensor]:
+        """``(W8, scale)`` of the linear named ``prefix`` (quantised once from the stored weights)."""
+        q = self._q.get(prefix)
+        if q is None:
+            q = ofp8.quantize_weight_rows(self.sd_quant[prefix + ".weight"])
+            self._q[prefix] = q
+        return q
+
     def linear(self, prefix: str, x: torch.Tensor) -> torch.Tensor:
         """``nn.Linear`` named ``prefix`` applied to ``x`` (bias if the state dict has one)."""
         w = self.sd[prefix + ".weight"]
         b = self.sd.get(prefix + ".bias")
         if prefix in self.fp8_names:
-            q = self._q.get(prefix)
-            if q is None:
-                q = ofp8.quantize_weight_rows(self.sd_quant[prefix + ".weight"])
-                self._q[prefix] = q
+            q = self.quantised(prefix)
             y = ops.lin_fp8w(x.reshape(-1, x.shape[-1]), q[0], q[1], self.act_dtype).reshape(*x.shape[:-1], w.shape[0])
             return y if b is None else y + b
         return F.linear(x, w, b)

@@ -68,6 +68,22 @@ def test_small_model_chunk_matches_oracle(tiers):
         assert float((got - gold).abs().max()) <= 1e-2 * max(1.0, float(gold.abs().max()))
 
 
+def test_w8a8_prefill_tier_matches_its_oracle():
+    # tl_fp8_llm_mlp="w8a8": VLM MLP with per-token quantised activations on the fp8 matrix instruction, against
+    # the oracle's restatement of `make_fp8_mlp_forward` (tybok/policies/pi05/models/triton_prefill_mlp.py:145-166);
+    # a drift tier like the reference's: also reported against the weight-only result
+    cfg, sd, inp = cases.pi05_build(cases.PI05_CASES["small"])
+    want = _oracle_chunk(cfg, sd, inp, True, True, llm_w8a8=True)
+    base = _oracle_chunk(cfg, sd, inp, True, True)
+    for fused in (False, True):
+        got = _gpu_chunk(cfg, sd, inp, fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True, fp8_llm_act=True, fused_prefill=fused)
+        err, drift = float((got - want).abs().max()), float((want - base).abs().max())
+        print(f"pi05 small W8A8 prefill (fused_prefill={fused}): max|err| vs W8A8 oracle {err:.4g}; W8A8 vs weight-only oracle {drift:.4g}; |chunk|max {float(want.abs().max()):.3g}")
+        assert torch.isfinite(got).all()
+        assert err <= 1.5e-2 * max(1.0, float(want.abs().max()))
+    assert drift <= 5e-2 * max(1.0, float(base.abs().max()))  # the reference's acceptance bound for its fp8 tiers
+
+
 def test_zero_noise_chunk_within_bound():
     # zero noise, full fp8 path, reduced depth (full depth: the full_depth tests below)
     case = dict(cases.PI05_CASES["small"], noise="zeros", depth=4, num_steps=10, seed=21)

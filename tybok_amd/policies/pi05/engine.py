@@ -168,10 +168,13 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
             self.vit_mlp_dtype = torch.float16 if vit_mlp_dtype == "fp16" else torch.bfloat16
         self.tl_fused_expert = bool(tl_fused_expert)
         self.tl_fp8_llm_mlp = bool(tl_fp8_llm_mlp)
+        # tl_fp8_llm_mlp="w8a8": the reference tier's own arithmetic -- activations quantised per token, fp8 x fp8
+        # products (True keeps the activations in bf16: weight-only)
+        self.fp8_llm_act = isinstance(tl_fp8_llm_mlp, str) and tl_fp8_llm_mlp.lower() == "w8a8"
         self.tl_fp8_expert_mlp = bool(tl_fp8_expert_mlp)
         self.model = PI05Model(
             self.config, sd, self.device,
-            fused_expert=self.tl_fused_expert, fp8_expert_mlp=self.tl_fp8_expert_mlp, fp8_llm_mlp=self.tl_fp8_llm_mlp,
+            fused_expert=self.tl_fused_expert, fp8_expert_mlp=self.tl_fp8_expert_mlp, fp8_llm_mlp=self.tl_fp8_llm_mlp, fp8_llm_act=self.fp8_llm_act,
             fused_prefill=bool(tl_llm_flash_attn), vit_mlp_dtype=self.vit_mlp_dtype, vit_lowp_attn=self.tl_fused_vit,
         )  # fmt: skip
         del sd

@@ -76,6 +76,7 @@ class PI05Model:
         fused_expert: bool = False,
         fp8_expert_mlp: bool = False,
         fp8_llm_mlp: bool = False,
+        fp8_llm_act: bool = False,
         fused_prefill: bool = False,
         vit_mlp_dtype: torch.dtype | None = None,
         vit_lowp_attn: bool = False,
@@ -87,6 +88,9 @@ class PI05Model:
         self.fused_expert = bool(fused_expert)
         self.fp8_expert_mlp = bool(fp8_expert_mlp)
         self.fp8_llm_mlp = bool(fp8_llm_mlp)
+        # W8A8: the VLM MLP's activations are quantised per token as well and the products run on the fp8 matrix
+        # instruction -- what the reference's fp8 prefill tier computes (tybok/policies/pi05/models/triton_prefill_mlp.py:145-166)
+        self.fp8_llm_act = bool(fp8_llm_act) and self.fp8_llm_mlp
         self.fused_prefill = bool(fused_prefill)
         self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp or self.fused_prefill or self.vit_lowp_attn
         if self.use_hip and self.device.type != "cuda":
@@ -96,7 +100,7 @@ class PI05Model:
         self.head_dim = self.vd["head_dim"]
         mlp_keys = tuple(f".mlp.{p}_proj.weight" for p in ("gate", "up", "down"))
         self.p = {k: v.to(self.device) for k, v in state_dict.items() if not k.endswith(mlp_keys)}
-        self.vlm_mlp = [GatedMLP(state_dict, f"{VLM}layers.{i}.mlp.", self.device, self.fp8_llm_mlp, act="gelu_tanh") for i in range(self.depth)]
+        self.vlm_mlp = [GatedMLP(state_dict, f"{VLM}layers.{i}.mlp.", self.device, self.fp8_llm_mlp, act="gelu_tanh", w8a8=self.fp8_llm_act) for i in range(self.depth)]
         self.exp_mlp = [GatedMLP(state_dict, f"{EXP}layers.{i}.mlp.", self.device, self.fp8_expert_mlp, act="gelu_tanh") for i in range(self.ed["depth"])]
         self.ws = tk.default_workspace(self.device) if self.use_hip else None
         self.vt_suf = None  # zero-padded V^T of the action tokens, allocated on first use
@@ -371,7 +375,10 @@ class PI05Model:
             att = tk.expert_attn(qkv[:, :nq].view(p_len, heads, d), cache, None, None, tk.MASK_NONE, mask2d=mask2d, logits_bf16=True, ws=self.ws)
             out = tk.bf16w_linear(att, self.vlm_o[i], resid=hidden, ws=self.ws)
             mlp = self.vlm_mlp[i]
-            if mlp.fp8:
+            if mlp.w8a8:
+                normed = tk.rms_norm_rows(out, ada=norm_post, eps=EPS)
+                hidden = tk.w8a8_gated_ffn(normed, mlp.wgu, mlp.wd, "gelu_tanh", resid=out, ws=self.ws)
+            elif mlp.fp8:
                 hidden = tk.fp8w_gated_ffn(out, mlp.wgu, mlp.wd, "gelu_tanh", resid=out, ada=norm_post, eps=EPS, ws=self.ws)
             else:
                 h, _ = gemma_norm(out[None], weight=self.p[f"{VLM}layers.{i}.post_attention_layernorm.weight"])

@@ -68,9 +68,10 @@ def eager_attention(mask: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: tor
 class GatedMLP:
     """gate/up/down of one decoder layer: bf16 torch linears, or fp8 weights on the HIP kernel."""
 
-    def __init__(self, sd: dict, prefix: str, device, fp8: bool, act: str = "silu"):
+    def __init__(self, sd: dict, prefix: str, device, fp8: bool, act: str = "silu", w8a8: bool = False):
         self.act = act
         self.fp8 = fp8
+        self.w8a8 = bool(w8a8) and fp8  # activations quantised per token too (the W8A8 tier)
         names = [prefix + n + ".weight" for n in ("gate_proj", "up_proj", "down_proj")]
 
         def codes_and_scale(name: str):
@@ -93,7 +94,8 @@ class GatedMLP:
         """``down(act(gate(x)) * up(x)) + resid`` for ``x [B, L, hidden]`` bf16 (in-place add semantics)."""
         if self.fp8:
             b, length, hidden = x.shape
-            y = tk.fp8w_gated_ffn(x.reshape(b * length, hidden), self.wgu, self.wd, self.act, resid=resid.reshape(b * length, hidden))
+            ffn = tk.w8a8_gated_ffn if self.w8a8 else tk.fp8w_gated_ffn
+            y = ffn(x.reshape(b * length, hidden), self.wgu, self.wd, self.act, resid=resid.reshape(b * length, hidden))
             return y.view(b, length, hidden)
         a = F.silu(F.linear(x, self.wg)) if self.act == "silu" else F.gelu(F.linear(x, self.wg), approximate="tanh")
         out = F.linear(a * F.linear(x, self.wu), self.wdn)
