@@ -63,6 +63,26 @@ def test_w8a8_gemm_matches_oracle(tk, m, k, n):
     _close(got, want, f"w8a8 gemm M={m} K={k} N={n}")
 
 
+@pytest.mark.parametrize("resid_dtype", [None, torch.float32, BF16])
+@pytest.mark.parametrize("m,k,n", [(385, 96, 260), (300, 256, 36)])
+def test_w8a8_gemm_row_segment_stores_respect_n_and_the_pitch(tk, m, k, n, resid_dtype):
+    # 16-byte row segment stores into a column slice of a wider buffer: the tail segment is cut to N, nothing
+    # past N is written, and both residual types go through the coalesced path
+    x, w8, sw = gemm_case(m, k, n)
+    a8, sa = oops.quantize_activation_rows(x)
+    want = oops.lin_w8a8(a8, sa, w8, sw)
+    pitch = (n + 15) // 8 * 8
+    buf = torch.full((m, pitch), 7.0, dtype=BF16, device="cuda")
+    resid = None
+    if resid_dtype is not None:
+        r = torch.randn(m, pitch, generator=torch.Generator().manual_seed(3)).to(resid_dtype)
+        want = (want.float() + r[:, :n].float()).to(BF16)
+        resid = r.cuda()[:, :n]
+    tk.w8a8_gemm(a8.cuda(), sa.cuda(), tk.pack_fp8_weight(w8.cuda(), sw.cuda()), resid=resid, out=buf[:, :n])
+    _close(buf[:, :n], want, f"w8a8 gemm M={m} K={k} N={n} pitch={pitch}")
+    assert bool((buf[:, n:] == 7.0).all()), "wrote past N"
+
+
 def test_w8a8_gemm_exact_on_small_integers(tk):
     # integer-valued codes and power-of-two scales: every product and sum is exact in fp32, whatever the order --
     # a wrong pairing of k between the two operands of the matrix instruction cannot hide behind a tolerance

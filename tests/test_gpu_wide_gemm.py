@@ -39,6 +39,26 @@ def test_many_row_gemm(tk, m, k, n):
     _close(got, oops.lin_fp8w(x, w8, s), f"gemm M={m} K={k} N={n}")
 
 
+@pytest.mark.parametrize("resid_dtype", [None, torch.float32, BF16])
+@pytest.mark.parametrize("m,k,n", [(385, 96, 260), (300, 256, 36), (257, 128, 1000)])
+def test_many_row_gemm_row_segment_stores_respect_n_and_the_pitch(tk, m, k, n, resid_dtype):
+    # output and residual are column slices of wider 16-byte aligned buffers (pitch % 8 == 0): the kernel stores
+    # 16-byte row segments, the last one of a row cut to N; the columns past N must keep their sentinel
+    x, w8, s = gemm_case(m, k, n)
+    pw = tk.pack_fp8_weight(w8.cuda(), s.cuda())
+    pitch = (n + 15) // 8 * 8
+    buf = torch.full((m, pitch), 7.0, dtype=BF16, device="cuda")
+    want = oops.lin_fp8w(x, w8, s)
+    resid = None
+    if resid_dtype is not None:
+        r = torch.randn(m, pitch, generator=torch.Generator().manual_seed(3)).to(resid_dtype)
+        want = (want.float() + r[:, :n].float()).to(BF16)
+        resid = r.cuda()[:, :n]
+    tk.fp8w_gemm(x.cuda(), pw, resid=resid, out=buf[:, :n])
+    _close(buf[:, :n], want, f"gemm M={m} K={k} N={n} pitch={pitch}")
+    assert bool((buf[:, n:] == 7.0).all()), "wrote past N"
+
+
 def test_many_row_gemm_matches_skinny_kernel_rows(tk):
     # the same rows through the skinny kernel (M <= 64 per call) must give the same bits: both
     # kernels accumulate a row's k tiles in ascending order within a wave ... but split K over waves

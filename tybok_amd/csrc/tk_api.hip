@@ -140,6 +140,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   a.act = act;
   a.vec = N % 4 == 0 && ldy % 4 == 0 && aligned8(y) && (e.w16 || aligned16(s0)) && (!gate || aligned8(gate)) &&
           (!resid || (ldr % 4 == 0 && (resid_dtype == TK_F32 ? aligned16(resid) : aligned8(resid))));
+  a.vec16 = ldy % 8 == 0 && aligned16(y) && (!resid || (aligned16(resid) && ldr % (resid_dtype == TK_F32 ? 4 : 8) == 0));
   if ((gated || rope) && (ldy % 4 || !aligned8(y) || (gated && (!aligned16(s0) || !aligned16(s1)))))
     return fail(TK_EINVAL, "gemm: this epilogue needs ldy %% 4 == 0, an 8-byte aligned y and 16-byte aligned scales");
   if (rope && (!aligned16(e.rope_cos) || !aligned16(e.rope_sin)))
@@ -400,6 +401,7 @@ int w8a8_common(const void* a8, int lda, const float* sa, const void* w_packed, 
   a.ntiles = ((N + 31) / 32) * (s1 ? 2 : 1);
   a.act = act;
   a.vec = 1;
+  a.vec16 = ldy % 8 == 0 && aligned16(y) && (!resid || (aligned16(resid) && ldr % (resid_dtype == TK_F32 ? 4 : 8) == 0));
   const int blocks0 = ((a.ntiles * 32 + tk_w8a8_cols() - 1) / tk_w8a8_cols()) * ((M + tk_w8a8_rows() - 1) / tk_w8a8_rows());
   int ks = split_k;
   if (ks <= 0) {

@@ -47,6 +47,9 @@ struct GemmArgs {
   int vt_ld;
   // W8A8 launches only: x holds e4m3fn codes (ldx in bytes) and row_scale the per-token fp32 scales
   const float* row_scale;
+  // many-row kernels: y (and the residual) allow 16-byte row-contiguous accesses (pitches multiples of 8
+  // elements, 16-byte aligned pointers): the epilogue stores whole row segments through LDS
+  int vec16;
 };
 
 struct QuantActArgs {

@@ -124,28 +124,40 @@ __global__ __launch_bounds__(NW * 64) void w8a8_wide_kernel(GemmArgs a, int nblk
 #pragma unroll
     for (int i = 0; i < XPT; ++i) *(i32x4*)(lds + b * XBUF + xdst[i]) = (k0 + xcol[i]) < k_end ? f.v[i] : z;
   };
-  auto step = [&](const WFrag& f, int b, int s) {
-    i32x8 xa[MT], wb[NT];
+  // operands of a whole round (two 64-wide steps x four m tiles): requested together right after the round's
+  // barrier, so the matrix instructions that follow wait for the first pair only and the rest streams in behind
+  i32x8 xa[STEPS][MT];
+  auto xread = [&](int b) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const unsigned char* p = lds + b * XBUF + (mt * 32 + l32) * PITCH + s * 64 + 16 * half;
-      const i32x4 lo = *(const i32x4*)p, hi = *(const i32x4*)(p + 32);
-      xa[mt] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const unsigned char* p = lds + b * XBUF + (mt * 32 + l32) * PITCH + s * 64 + 16 * half;
+        const i32x4 lo = *(const i32x4*)p, hi = *(const i32x4*)(p + 32);
+        xa[s][mt] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+  };
+  auto mma = [&](const WFrag& f) {
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      i32x8 wb[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const i32x4 lo = f.w[2 * s][nt], hi = f.w[2 * s + 1][nt];
+        wb[nt] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wb[nt], xa[s][mt], acc[mt][nt], 0, 0, 0, 0, 0, 0);
     }
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const i32x4 lo = f.w[2 * s][nt], hi = f.w[2 * s + 1][nt];
-      wb[nt] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wb[nt], xa[mt], acc[mt][nt], 0, 0, 0, 0, 0, 0);
   };
 
   // PF rounds in flight, every load unconditional (clamped addresses; columns past the block's k range are
-  // zeroed when staged); one LDS barrier per round, the staging buffers alternate.
+  // zeroed when staged).  Round r: its operands are requested from LDS, then round r+1 is staged into the other
+  // buffer (every wave has passed barrier r, i.e. holds round r-1's operands in registers) and the next global
+  // loads go out -- all of it under the 16 matrix instructions of round r; one barrier per round.
   WFrag wbuf[PF];
   XFrag xbuf[PF];
 #pragma unroll
@@ -153,13 +165,19 @@ __global__ __launch_bounds__(NW * 64) void w8a8_wide_kernel(GemmArgs a, int nblk
     xload(xbuf[p], p);
     wload(wbuf[p], p);
   }
+  xstore(xbuf[0], 0, 0);
+  xload(xbuf[0], PF);
+  lds_barrier();
   auto round = [&](int p, int r) {
-    xstore(xbuf[p], r, r & 1);
-    xload(xbuf[p], r + PF);
-    lds_barrier();
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) step(wbuf[p], r & 1, s);
+    const int pn = (p + 1) % PF;
+    xread(r & 1);
+    __builtin_amdgcn_sched_barrier(0);
+    xstore(xbuf[pn], r + 1, (r + 1) & 1);
+    xload(xbuf[pn], r + 1 + PF);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(wbuf[p]);
     wload(wbuf[p], r + PF);
+    lds_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
   {
@@ -237,6 +255,100 @@ __global__ __launch_bounds__(NW * 64) void w8a8_wide_kernel(GemmArgs a, int nblk
     int m = (mblock * MT + mt) * 32 + l32;
     if (m > a.M - 1) m = a.M - 1;
     sa[mt] = a.row_scale[m];
+  }
+  if (a.vec16) {
+    // Coalesced stores: a lane holds, per tile, row l % 32 and four 4-column pieces 16 bytes apart -- stored as
+    // they are, one instruction would touch 32 rows with 16 bytes each.  Each wave therefore passes its 32 rows of
+    // an m tile through a private LDS tile (a wave's LDS instructions execute in order, so it needs no barrier of its own) and stores
+    // them as 16-byte chunks of consecutive columns, whole 64- or 128-byte segments of a row per 4 or 8 lanes.
+    constexpr int COLS = EPI == 0 ? NT * 32 : 32;       // output columns of a wave per row
+    constexpr int EP = COLS * 2 + 16;                   // LDS row pitch (bytes)
+    constexpr int LPR = COLS / 8;                       // lanes (16-byte chunks) per row
+    constexpr int RPI = 64 / LPR;                       // rows per store instruction
+    static_assert(NW * 32 * EP <= 2 * XBUF, "the staging buffers hold every wave's tile");
+    lds_barrier();  // every wave has left the staged activations behind
+    unsigned char* wl = lds + wave * 32 * EP;
+    const int ncol0 = EPI == 0 ? strip * NT * 32 : strip * 32;  // first output column of this wave
+    f32x4 sc0[EPI == 0 ? NT : 1][4], sc1[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      if (EPI == 0) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          int n0 = (strip * NT + nt) * 32 + 8 * g + 4 * half;
+          if (n0 > a.N - 4) n0 = a.N - 4;  // columns past N are never stored
+          sc0[EPI == 0 ? nt : 0][g] = *(const f32x4*)(a.s0 + n0);
+        }
+      } else {
+        int col = strip * 32 + 8 * g + 4 * half;
+        if (col > a.N - 4) col = a.N - 4;
+        sc0[0][g] = *(const f32x4*)(a.s0 + col);
+        sc1[g] = *(const f32x4*)(a.s1 + col);
+      }
+    }
+    const int lrow = lane / LPR, lchunk = lane % LPR;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        if (EPI == 0) {
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            const f32x16& c = acc[mt][nt];
+            f32x4 v = {c[4 * g], c[4 * g + 1], c[4 * g + 2], c[4 * g + 3]};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = mul_rn(mul_rn(v[j], sa[mt]), sc0[EPI == 0 ? nt : 0][g][j]);
+            *(i32x2*)(wl + l32 * EP + (nt * 32 + 8 * g + 4 * half) * 2) = pack_bf16x4(v);
+          }
+        } else {
+          const f32x16& cg = acc[mt][0];
+          const f32x16& cu = acc[mt][1];
+          f32x4 vg = {cg[4 * g], cg[4 * g + 1], cg[4 * g + 2], cg[4 * g + 3]};
+          f32x4 vu = {cu[4 * g], cu[4 * g + 1], cu[4 * g + 2], cu[4 * g + 3]};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            vg[j] = mul_rn(mul_rn(vg[j], sa[mt]), sc0[0][g][j]);
+            vu[j] = mul_rn(mul_rn(vu[j], sa[mt]), sc1[g][j]);
+          }
+          const f32x4 gg = unpack_bf16x4(pack_bf16x4(vg));
+          const f32x4 up = unpack_bf16x4(pack_bf16x4(vu));
+          f32x4 act;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) act[j] = a.act == 0 ? silu_f(gg[j]) : gelu_tanh_f(gg[j]);
+          act = unpack_bf16x4(pack_bf16x4(act));
+          *(i32x2*)(wl + l32 * EP + (8 * g + 4 * half) * 2) = pack_bf16x4(act * up);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 32 / RPI; ++j) {
+        const int row = j * RPI + lrow;
+        const int m = (mblock * MT + mt) * 32 + row;
+        const int n = ncol0 + lchunk * 8;
+        i32x4 t = *(const i32x4*)(wl + row * EP + lchunk * 16);
+        if (m >= a.M || n >= a.N) continue;
+        if (EPI == 0 && a.resid) {
+          // bf16(y + resid) on the bf16-rounded product, as the scattered path computes it
+          f32x4 r0, r1 = {0.f, 0.f, 0.f, 0.f};
+          if (a.resid_f32) {
+            const f32x4* rp = (const f32x4*)((const float*)a.resid + (size_t)m * a.ldr + n);
+            r0 = rp[0];
+            if (n + 8 <= a.N) r1 = rp[1];
+          } else if (n + 8 <= a.N) {
+            const i32x4 rr = *(const i32x4*)((const u16*)a.resid + (size_t)m * a.ldr + n);
+            r0 = unpack_bf16x4(i32x2{rr[0], rr[1]});
+            r1 = unpack_bf16x4(i32x2{rr[2], rr[3]});
+          } else {
+            r0 = unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n));
+          }
+          const i32x2 lo = pack_bf16x4(unpack_bf16x4(i32x2{t[0], t[1]}) + r0), hi = pack_bf16x4(unpack_bf16x4(i32x2{t[2], t[3]}) + r1);
+          t = i32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+        u16* dst = a.y + (size_t)m * a.ldy + n;
+        if (n + 8 <= a.N) *(i32x4*)dst = t;
+        else *(i32x2*)dst = i32x2{t[0], t[1]};  // N % 8 == 4: the row's last four columns
+      }
+    }
+    return;
   }
   if (EPI == 0) {
 #pragma unroll
