@@ -225,6 +225,26 @@ int tk_bf16w_linear(const void* x, int ldx, int x_dtype, const void* w_packed, c
                     int vt_col0, int vt_ld, void* y, int ldy, const void* resid, int ldr, int resid_dtype,
                     const void* gate, int M, int N, int K, int split_k, void* ws, size_t ws_bytes, void* stream);
 
+/* y[M, N] (bf16) = bf16( resid + act( bf16( x[M, K] . W[N, K]^T + bias[N] ) ) ): the linears of the vision towers
+ * (q|k|v, out_proj, fc1 + GELU, fc2) and any other bf16 linear over hundreds of rows, on the many-row MFMA kernel.
+ * Replaces the reference's fused tower kernels' GEMM parts (`triton_vision_qkv`, `triton_vision_out_proj`,
+ * `triton_vision_mlp`, tybok/policies/pi05/models/vision.py:116-173; SmolVLA: the bf16 `nn.Linear`s of
+ * tybok/policies/smolvla/models/vision.py:197-257).
+ *   x:     bf16 [M, K], pitch ldx (elements, a multiple of 8; K a multiple of 16; 16-byte aligned).
+ *   w_packed: tk_pack_bf16_weight(..., rope_half = 0).
+ *   bias:  bf16 [N] or NULL.
+ *   act:   0 none; 1 tanh GELU of the bf16-rounded linear output (`gelu(linear(x))` on bf16 tensors,
+ *          tybok/policies/pi05/models/vision.py:79-87); 2 tanh GELU of the fp32 pre-activation (the reference's fused
+ *          MLP keeps fc1's output in fp32 through the GELU, vision.py:259-273).
+ *   resid: optional bf16 or fp32 [M, N] (resid_dtype TK_BF16 / TK_F32), added to the bf16-rounded result.
+ *   y:     bf16 [M, N], pitch ldy (a multiple of 8, 16-byte aligned); N a multiple of 4.
+ *   tile:  0 = chosen from the shape; 42, 41, 32, 31, 22, 21, 12, 11 = (32-row tiles per block, 32-column tiles per
+ *          wave of a 4-wave block).
+ *   split_k: 0 = automatic; > 1 needs the workspace (fp32 partials, summed in split order: bit-deterministic). */
+int tk_bf16w_dense(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy,
+                   const void* resid, int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws,
+                   size_t ws_bytes, void* stream);
+
 /* ---- action-expert attention over the cached prefix ------------------------------------------ */
 /* Lays one layer's prefix K/V out for tk_expert_attn, once per request (the counterpart of the
  * reference filling its static per-layer prefix cache after the VLM prefill,

@@ -1,0 +1,116 @@
+"""bf16-weight many-row linear (bias / GELU / residual epilogues) against plain torch fp32 arithmetic on the same
+bf16 operands, with the rounding points of ``F.linear`` / ``F.gelu`` on bf16 tensors.  GPU only."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+
+
+@pytest.fixture(scope="module")
+def tk():
+    from tybok_amd import ops
+
+    return ops
+
+
+def _case(m, k, n, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, k, generator=g).to(BF16)
+    w = (torch.randn(n, k, generator=g) / k**0.5).to(BF16)
+    b = torch.randn(n, generator=g).to(BF16)
+    return x, w, b
+
+
+def _want(x, w, b, act=None, resid=None):
+    y = (x.double() @ w.double().t() + (0 if b is None else b.double())).float()
+    if act == "gelu_tanh":
+        y = F.gelu(y.to(BF16).float(), approximate="tanh")
+    elif act == "gelu_tanh_fp32":
+        y = F.gelu(y, approximate="tanh")
+    y = y.to(BF16)
+    if resid is not None:
+        y = (y.float() + resid.float()).to(BF16)
+    return y
+
+
+def _close(got, want, what, frac_exact=0.97):
+    got, want = got.float().cpu(), want.float()
+    err = (got - want).abs()
+    tol = 1e-2 + 2**-7 * want.abs()  # one bf16 ulp of the result (the fp32 sum order differs) plus a floor near zero
+    bad = err > tol
+    assert not bad.any(), f"{what}: {int(bad.sum())} / {bad.numel()} outside tolerance, max |err| {err.max():.4g}"
+    same = (got == want).float().mean().item()
+    assert same >= frac_exact, f"{what}: only {same:.1%} of the outputs equal the correctly rounded result"
+
+
+TILES = [0, 42, 41, 32, 31, 22, 21, 12, 11]
+
+
+@pytest.mark.parametrize("tile", TILES)
+@pytest.mark.parametrize("m,k,n", [(768, 1152, 4608), (300, 4304, 1152), (3072, 768, 768), (257, 80, 40), (1, 64, 8), (130, 208, 264)])
+def test_dense_matches_torch(tk, tile, m, k, n):
+    x, w, b = _case(m, k, n)
+    pw = tk.pack_bf16_weight(w.cuda())
+    got = tk.bf16w_dense(x.cuda(), pw, b.cuda(), tile=tile)
+    _close(got, _want(x, w, b), f"dense M={m} K={k} N={n} tile={tile}")
+    got = tk.bf16w_dense(x.cuda(), pw, None, tile=tile)
+    _close(got, _want(x, w, None), f"dense without bias M={m} K={k} N={n} tile={tile}")
+
+
+@pytest.mark.parametrize("act", ["gelu_tanh", "gelu_tanh_fp32"])
+@pytest.mark.parametrize("m,k,n", [(768, 1152, 4304), (3072, 768, 3072), (100, 64, 96)])
+def test_dense_gelu(tk, act, m, k, n):
+    x, w, b = _case(m, k, n, seed=1)
+    got = tk.bf16w_dense(x.cuda(), tk.pack_bf16_weight(w.cuda()), b.cuda(), act)
+    _close(got, _want(x, w, b, act), f"dense {act} M={m} K={k} N={n}", frac_exact=0.95)
+
+
+@pytest.mark.parametrize("resid_dtype", [torch.float32, BF16])
+@pytest.mark.parametrize("tile", [42, 31, 21, 11])
+def test_dense_residual_tail_and_pitch(tk, resid_dtype, tile):
+    # N % 8 == 4, output and residual are column slices of wider buffers; nothing past N may be written
+    m, k, n = 385, 96, 260
+    x, w, b = _case(m, k, n, seed=2)
+    pitch = 272
+    r = torch.randn(m, pitch, generator=torch.Generator().manual_seed(3)).to(resid_dtype)
+    buf = torch.full((m, pitch), 7.0, dtype=BF16, device="cuda")
+    tk.bf16w_dense(x.cuda(), tk.pack_bf16_weight(w.cuda()), b.cuda(), resid=r.cuda()[:, :n], out=buf[:, :n], tile=tile)
+    _close(buf[:, :n], _want(x, w, b, resid=r[:, :n]), "dense + residual")
+    assert bool((buf[:, n:] == 7.0).all()), "wrote past N"
+
+
+@pytest.mark.parametrize("split", [2, 3, 5])
+def test_dense_split_k_is_deterministic(tk, split):
+    x, w, b = _case(300, 4304, 256, seed=4)
+    pw = tk.pack_bf16_weight(w.cuda())
+    xc, bc = x.cuda(), b.cuda()
+    first = tk.bf16w_dense(xc, pw, bc, split_k=split)
+    again = tk.bf16w_dense(xc, pw, bc, split_k=split)
+    assert torch.equal(first, again)
+    _close(first, _want(x, w, b), f"split {split}")
+
+
+def test_dense_exact_on_small_integers(tk):
+    # integer operands: every product and partial sum is exact in fp32 whatever the order, so a wrong pairing of k
+    # between the two MFMA operands or a misplaced output column cannot hide behind a tolerance
+    g = torch.Generator().manual_seed(5)
+    m, k, n = 200, 144, 104
+    x = torch.randint(-4, 5, (m, k), generator=g).to(BF16)
+    w = torch.randint(-3, 4, (n, k), generator=g).to(BF16)
+    b = torch.randint(-8, 9, (n,), generator=g).to(BF16)
+    want = (x.float() @ w.float().t() + b.float()).to(BF16)
+    for tile in TILES:
+        got = tk.bf16w_dense(x.cuda(), tk.pack_bf16_weight(w.cuda()), b.cuda(), tile=tile)
+        assert torch.equal(got.cpu(), want), f"tile {tile}"
+
+
+def test_dense_rejects_bad_arguments(tk):
+    x, w, b = _case(64, 64, 64)
+    pw = tk.pack_bf16_weight(w.cuda())
+    with pytest.raises(RuntimeError):
+        tk.bf16w_dense(x.cuda(), pw, b.cuda(), tile=33)
+    with pytest.raises(ValueError):
+        tk.bf16w_dense(x.cuda()[:, :32], pw, b.cuda())

@@ -1,0 +1,355 @@
+// bf16-weight GEMM for many rows with bias / GELU / residual epilogues on gfx950: the linears of the vision
+// towers (q|k|v, out_proj, fc1, fc2 over 256 .. 1024 patches per camera) and the bf16 projections of the VLM
+// prefill.
+//
+//   y[M, N] = bf16( resid + act( bf16( x[M, K] . W[N, K]^T + bias[N] ) ) )
+//
+// Operands: x bf16 row-major; W in the 2 KiB tile order of tk_pack_bf16_weight (tile (nt, kt): two 1 KiB chunks,
+// chunk c of lane l = 8 bf16 of column nt*32 + l%32 at k = 32*kt + 16*(l/32) + 8*c), so a weight operand of
+// v_mfma_f32_32x32x16_bf16 is one coalesced 16-byte load per lane straight into registers.
+//   * a block of 4 waves owns MT*32 rows x 4*NT*32 columns and a range of k tiles; wave w owns n tiles
+//     w*NT .. w*NT+NT-1 for all rows;
+//   * the activations of a round (MT*32 rows x 64 columns) are staged once per block through LDS with whole
+//     128-byte lines per row, double buffered, one LDS barrier per round;
+//   * blocks that share weights (same n tiles and k range, different rows) get consecutive slots of ONE XCD, so
+//     a weight tile comes from HBM once and from that XCD's L2 afterwards;
+//   * K splits hand fp32 partials through the workspace; the last-arriving block sums them in split order:
+//     bit-deterministic;
+//   * the epilogue passes each wave's 32-row slices through a private LDS tile and stores 16-byte row segments.
+// Tile shapes (MT, NT) from (4, 2) = 128 x 256, one block per CU, down to (1, 1) = 32 x 128 with four blocks per
+// CU: the host picks the one whose blocks are all resident at once and load the CUs evenly (co-resident blocks
+// overlap each other's first loads and epilogue, a second generation of blocks would pay both again).
+#include "tk_common.h"
+#include "tk_kernels.h"
+
+namespace {
+
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+constexpr int NW = 4;  // waves per block
+constexpr int RK = 2;  // k tiles (of 32) per round
+
+template <int MT, int NT, int PF, int OCC>
+__global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, int nblk_m, int ngroups) {
+  constexpr int ROWS = MT * 32;
+  constexpr int ROWB = RK * 64;     // bytes of one staged activation row per round
+  constexpr int PITCH = ROWB + 16;  // conflict-free 16-byte operand reads, 16-byte aligned
+  constexpr int XBUF = ROWS * PITCH;
+  constexpr int PPR = ROWB / 16;    // 16-byte pieces per staged row
+  constexpr int XPT = ROWS * PPR / (NW * 64);
+  constexpr int TILES = MT * NT;
+  static_assert(RK == 2 && PF % 2 == 0, "a round is two phases; buffer parity follows the pipeline slot");
+  // epilogue: each wave's 32 x (NT*32) bf16 slice passes through a private LDS tile in the staging buffers' space
+  constexpr int COLS = NT * 32;      // output columns of a wave per row
+  constexpr int EP = COLS * 2 + 16;  // LDS row pitch (bytes)
+  constexpr int LPR = COLS / 8;      // lanes (16-byte chunks) per row
+  constexpr int RPI = 64 / LPR;      // rows per store instruction
+  constexpr int LDSB = 2 * XBUF > NW * 32 * EP ? 2 * XBUF : NW * 32 * EP;
+  __shared__ __align__(16) unsigned char lds[LDSB];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5;
+  const int l32 = lane & 31;
+
+  // slot s of XCD x (blocks are dealt to the 8 XCDs round-robin) -> group (s / nblk_m) * 8 + x, m block
+  // s % nblk_m: the nblk_m blocks of a group (same weights) run back to back on one XCD
+  const unsigned id = blockIdx.x;
+  const unsigned slot = id >> 3;
+  const int mblock = (int)(slot % (unsigned)nblk_m);
+  const int group = (int)((slot / (unsigned)nblk_m) * 8 + (id & 7));
+  if (group >= ngroups) return;
+  const int split = group % a.ksplit;
+  const int nblk = group / a.ksplit;
+
+  const int kt_lo = split * a.kt_q + (split < a.kt_r ? split : a.kt_r);
+  const int kt_hi = kt_lo + a.kt_q + (split < a.kt_r ? 1 : 0);
+  const int nrounds = (kt_hi - kt_lo + RK - 1) / RK;
+  const int k_end = kt_hi * 32 < a.K ? kt_hi * 32 : a.K;
+
+  const int strip = nblk * NW + wave;  // this wave's NT packed n tiles
+  const uint8_t* wbase[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    int ntg = strip * NT + nt;
+    if (ntg > a.ntiles - 1) ntg = a.ntiles - 1;  // overhanging tiles are computed on valid data, never stored
+    wbase[nt] = a.w + ((size_t)ntg * a.KT) * 2048 + lane * 16;
+  }
+
+  const char* xsrc[XPT];
+  int xcol[XPT], xdst[XPT];
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) {
+    const int p = tid + i * NW * 64;
+    const int r = p / PPR, c = p % PPR;
+    int m = mblock * ROWS + r;
+    if (m > a.M - 1) m = a.M - 1;  // rows past M: valid data, never stored
+    xsrc[i] = (const char*)a.x + (size_t)m * a.ldx * 2;
+    xcol[i] = c * 8;
+    xdst[i] = r * PITCH + c * 16;
+  }
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
+
+  struct WFrag {
+    i32x4 w[RK][NT][2];
+  };
+  struct XFrag {
+    i32x4 v[XPT];
+  };
+  auto wload = [&](WFrag& f, int r, int j) {  // k tile j of round r
+    int kt = kt_lo + r * RK + j;
+    if (kt > a.KT - 1) kt = a.KT - 1;  // its activation columns are zeroed
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const uint8_t* p = wbase[nt] + (size_t)kt * 2048;
+      f.w[j][nt][0] = *(const i32x4*)p;
+      f.w[j][nt][1] = *(const i32x4*)(p + 1024);
+    }
+  };
+  auto xload = [&](XFrag& f, int r) {
+    const int k0 = (kt_lo + r * RK) * 32;
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) {
+      int k = k0 + xcol[i];
+      if (k > a.K - 8) k = a.K - 8;
+      f.v[i] = *(const i32x4*)(xsrc[i] + (size_t)k * 2);
+    }
+  };
+  auto xstore = [&](const XFrag& f, int r, int b) {
+    const int k0 = (kt_lo + r * RK) * 32;
+    const i32x4 z = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) *(i32x4*)(lds + b * XBUF + xdst[i]) = (k0 + xcol[i]) < k_end ? f.v[i] : z;
+  };
+  // Operand fragments of two k tiles: while the MFMAs of one k tile run, the LDS reads of the next are issued.
+  i32x4 xa[2][MT][2];
+  auto xread = [&](int set, int b, int j) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const i32x4* p = (const i32x4*)(lds + b * XBUF + (mt * 32 + l32) * PITCH + (j * 32 + 16 * half) * 2);
+      xa[set][mt][0] = p[0];
+      xa[set][mt][1] = p[1];
+    }
+  };
+  auto mma = [&](int set, const WFrag& f, int j) {
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(f.w[j][nt][h2]), as_bf16x8(xa[set][mt][h2]), acc[mt][nt], 0, 0, 0);
+  };
+  // scheduling hint for a phase of 2*MT*NT MFMAs and 2*MT LDS reads: spread the reads between the MFMAs
+  // instead of waiting for each read right before its MFMA
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2 * MT; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
+    }
+  };
+
+  // PF rounds in flight; every load is unconditional (clamped addresses; columns past the block's k range are
+  // zeroed when staged), so the loop bodies have no branch and the compiler keeps precise wait counts.  Round r:
+  // phase A multiplies k tile 0 while k tile 1's operands are fetched from LDS, then refills k tile 0's weight
+  // registers for round r+PF; phase B stages round r+1 into the other LDS buffer, passes the round's only
+  // barrier (a wave can write buffer b for round r+2 only after every wave has passed the barrier of round r+1,
+  // i.e. has its round-r operands in registers), fetches round r+1's first operands and multiplies k tile 1.
+  WFrag wbuf[PF];
+  XFrag xbuf[PF];
+#pragma unroll
+  for (int p = 0; p < PF; ++p) {
+    xload(xbuf[p], p);
+    wload(wbuf[p], p, 0);
+    wload(wbuf[p], p, 1);
+  }
+  xstore(xbuf[0], 0, 0);
+  xload(xbuf[0], PF);
+  lds_barrier();
+  xread(0, 0, 0);
+  auto round = [&](int p, int r) {
+    const int b = p & 1;  // == r & 1: rounds advance PF at a time
+    const int pn = (p + 1) % PF;
+    __builtin_amdgcn_sched_barrier(0);
+    xread(1, b, 1);
+    mma(0, wbuf[p], 0);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    wload(wbuf[p], r + PF, 0);
+    xstore(xbuf[pn], r + 1, b ^ 1);
+    xload(xbuf[pn], r + 1 + PF);
+    lds_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    xread(0, b ^ 1, 0);
+    mma(1, wbuf[p], 1);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    wload(wbuf[p], r + PF, 1);
+  };
+  {
+    int it = 0;
+    for (; it + PF <= nrounds; it += PF) {
+#pragma unroll
+      for (int p = 0; p < PF; ++p) round(p, it + p);
+    }
+    const int rem = nrounds - it;  // in [0, PF)
+#pragma unroll
+    for (int q = 0; q < PF - 1; ++q)
+      if (q < rem) round(q, it + q);  // block-uniform
+  }
+
+  // ---- K-split hand-off: fp32 partials [(block, split)][wave][tile][group][lane][4] ----
+  const int blk_lin = nblk * nblk_m + mblock;
+  if (a.ksplit > 1) {
+    unsigned long long* pbase = (unsigned long long*)a.partial + ((size_t)wave * TILES * 4 * 64 + lane) * 2;
+    unsigned long long* mine = pbase + ((size_t)blk_lin * a.ksplit + split) * (NW * TILES * 4 * 64 * 2);
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& c = acc[t / NT][t % NT];
+        unsigned long long* dst = mine + (size_t)(t * 4 + g) * 128;
+        st_agent64(dst, c[4 * g], c[4 * g + 1]);
+        st_agent64(dst + 1, c[4 * g + 2], c[4 * g + 3]);
+      }
+    __shared__ int s_last;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (old == a.ksplit - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
+    for (int s = 0; s < a.ksplit; ++s) {  // split order, whoever arrived last
+      const unsigned long long* src = pbase + ((size_t)blk_lin * a.ksplit + s) * (NW * TILES * 4 * 64 * 2);
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) {
+        unsigned long long raw[4][2];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          raw[g][0] = ld_agent64(src + (size_t)(t * 4 + g) * 128);
+          raw[g][1] = ld_agent64(src + (size_t)(t * 4 + g) * 128 + 1);
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f32x16& c = acc[t / NT][t % NT];
+          c[4 * g] += __uint_as_float((unsigned)raw[g][0]);
+          c[4 * g + 1] += __uint_as_float((unsigned)(raw[g][0] >> 32));
+          c[4 * g + 2] += __uint_as_float((unsigned)raw[g][1]);
+          c[4 * g + 3] += __uint_as_float((unsigned)(raw[g][1] >> 32));
+        }
+      }
+    }
+  }
+
+  // ---- epilogue: lane l of a tile owns row m = l % 32 and, per register group g, four consecutive columns
+  // 8g + 4*(l/32) .. +3 (the accumulators hold C^T).  Stored as they are, one instruction would touch 32 rows with
+  // 8 bytes each; each wave therefore passes its 32 rows of an m tile through a private LDS tile (a wave's LDS
+  // instructions execute in order, so it needs no barrier of its own) and stores 16-byte chunks of consecutive
+  // columns: whole row segments of NT*64 bytes per 4*NT lanes. ----
+  lds_barrier();  // every wave has left the staged activations behind
+  unsigned char* wl = lds + wave * 32 * EP;
+  const int ncol0 = strip * COLS;  // first output column of this wave
+  f32x4 bias[NT][4];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      int n0 = ncol0 + nt * 32 + 8 * g + 4 * half;
+      if (n0 > a.N - 4) n0 = a.N - 4;  // columns past N are never stored
+      bias[nt][g] = a.bias ? unpack_bf16x4(*(const i32x2*)(a.bias + n0)) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  const int lrow = lane / LPR, lchunk = lane % LPR;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& c = acc[mt][nt];
+        f32x4 v = {c[4 * g], c[4 * g + 1], c[4 * g + 2], c[4 * g + 3]};
+        v = v + bias[nt][g];
+        if (a.act == 1) v = unpack_bf16x4(pack_bf16x4(v));  // the linear's bf16 output, then the activation on it
+        if (a.act) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] = gelu_tanh_f(v[j]);
+        }
+        *(i32x2*)(wl + l32 * EP + (nt * 32 + 8 * g + 4 * half) * 2) = pack_bf16x4(v);
+      }
+#pragma unroll
+    for (int j = 0; j < 32 / RPI; ++j) {
+      const int row = j * RPI + lrow;
+      const int m = (mblock * MT + mt) * 32 + row;
+      const int n = ncol0 + lchunk * 8;
+      i32x4 t = *(const i32x4*)(wl + row * EP + lchunk * 16);
+      if (m >= a.M || n >= a.N) continue;
+      if (a.resid) {
+        f32x4 r0, r1 = {0.f, 0.f, 0.f, 0.f};
+        if (a.resid_f32) {
+          const f32x4* rp = (const f32x4*)((const float*)a.resid + (size_t)m * a.ldr + n);
+          r0 = rp[0];
+          if (n + 8 <= a.N) r1 = rp[1];
+        } else if (n + 8 <= a.N) {
+          const i32x4 rr = *(const i32x4*)((const u16*)a.resid + (size_t)m * a.ldr + n);
+          r0 = unpack_bf16x4(i32x2{rr[0], rr[1]});
+          r1 = unpack_bf16x4(i32x2{rr[2], rr[3]});
+        } else {
+          r0 = unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n));
+        }
+        const i32x2 lo = pack_bf16x4(unpack_bf16x4(i32x2{t[0], t[1]}) + r0), hi = pack_bf16x4(unpack_bf16x4(i32x2{t[2], t[3]}) + r1);
+        t = i32x4{lo[0], lo[1], hi[0], hi[1]};
+      }
+      u16* dst = a.y + (size_t)m * a.ldy + n;
+      if (n + 8 <= a.N) *(i32x4*)dst = t;
+      else *(i32x2*)dst = i32x2{t[0], t[1]};  // N % 8 == 4: the row's last four columns
+    }
+  }
+}
+
+template <int MT, int NT, int PF, int OCC>
+int launch(const GemmArgs& a, hipStream_t st) {
+  const int nblk_m = (a.M + MT * 32 - 1) / (MT * 32);
+  const int nblk_n = (a.ntiles + NW * NT - 1) / (NW * NT);
+  const int ngroups = nblk_n * a.ksplit;
+  const unsigned blocks = (unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m;
+  hipLaunchKernelGGL((bf16w_wide_kernel<MT, NT, PF, OCC>), dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+}  // namespace
+
+// tile = 10 * MT + NT
+int tk_launch_bf16w_wide(const GemmArgs& a, int tile, hipStream_t st) {
+  switch (tile) {
+    case 42: return launch<4, 2, 4, 1>(a, st);
+    case 41: return launch<4, 1, 2, 2>(a, st);
+    case 32: return launch<3, 2, 2, 2>(a, st);
+    case 31: return launch<3, 1, 2, 3>(a, st);
+    case 22: return launch<2, 2, 2, 2>(a, st);
+    case 21: return launch<2, 1, 2, 4>(a, st);
+    case 12: return launch<1, 2, 2, 4>(a, st);
+    case 11: return launch<1, 1, 2, 4>(a, st);
+  }
+  return -1;
+}

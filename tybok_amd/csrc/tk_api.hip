@@ -429,6 +429,109 @@ int w8a8_common(const void* a8, int lda, const float* sa, const void* w_packed, 
 }
 }  // namespace
 
+// ---- bf16-weight linears with bias / GELU / residual epilogues (vision towers) ---------------------------------
+namespace {
+struct DenseTile {
+  int id, rows, cols;
+  int occ;  // blocks of this shape that fit one CU (registers)
+};
+constexpr DenseTile kDenseTiles[] = {{42, 128, 256, 1}, {41, 128, 128, 2}, {32, 96, 256, 2}, {31, 96, 128, 3},
+                                     {22, 64, 256, 2},  {21, 64, 128, 4},  {12, 32, 256, 4}, {11, 32, 128, 4}};
+
+// Estimated duration (us) of a launch with this tile and K split; the constants are fitted to timings of the
+// vision towers' and the prefill's shapes.  Blocks that are resident together share a CU's matrix pipes and
+// overlap each other's first loads and epilogues; every further generation of blocks pays those again.  A wave
+// issues (rows/32) * (cols/128) MFMAs per 16 columns of k (18.8 ns each under full load, half of that rate
+// reached), and a block loads (rows + cols) * 128 bytes per 64 columns of k at about 60 KiB/us per CU.
+float dense_cost(const DenseTile& t, int M, int N, int KT, int ks, int cus) {
+  const long long blocks = (long long)((M + t.rows - 1) / t.rows) * ((N + t.cols - 1) / t.cols) * ks;
+  const float kt = (float)((KT + ks - 1) / ks);
+  const float mfma_us = (float)(t.rows / 32) * (float)(t.cols / 128) * 2.f * kt * 0.0188f / 0.5f;
+  const float load_us = 0.5f * kt * (float)(t.rows + t.cols) * 0.125f / 60.f;
+  const float tile_us = mfma_us > load_us ? mfma_us : load_us;
+  const float fixed_us = 4.f + (t.occ == 1 ? 3.f : 0.f);  // one wave per SIMD hides nothing
+  float us = 0.f;
+  long long left = blocks;
+  while (left > 0) {
+    const long long gen = left < (long long)cus * t.occ ? left : (long long)cus * t.occ;
+    us += fixed_us + (float)((gen + cus - 1) / cus) * tile_us;
+    left -= gen;
+  }
+  if (ks > 1) us += 1.5f + (float)blocks * (float)(t.rows * t.cols) * 8.f / 4e6f;  // fp32 partials out and back in
+  return us;
+}
+}  // namespace
+
+int tk_bf16w_dense(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy, const void* resid,
+                   int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws, size_t ws_bytes, void* stream) {
+  if (M <= 0 || N <= 0 || K <= 0) return fail(TK_EINVAL, "bf16w_dense: non-positive shape M=%d N=%d K=%d", M, N, K);
+  if (K % 16 || ldx % 8 || ldx < K) return fail(TK_EINVAL, "bf16w_dense: K=%d must be a multiple of 16 and ldx=%d a multiple of 8 >= K", K, ldx);
+  if (!x || !w_packed || !y) return fail(TK_EINVAL, "bf16w_dense: null pointer");
+  if (!aligned16(x) || !aligned16(w_packed) || !aligned16(y) || (bias && !aligned8(bias)))
+    return fail(TK_EINVAL, "bf16w_dense: x, w_packed and y must be 16-byte aligned, bias 8-byte aligned");
+  if (N % 4 || ldy % 8 || ldy < N) return fail(TK_EINVAL, "bf16w_dense: N=%d must be a multiple of 4 and ldy=%d a multiple of 8 >= N", N, ldy);
+  if (act < 0 || act > 2) return fail(TK_EINVAL, "bf16w_dense: act=%d (0 none, 1 tanh-GELU of the bf16 output, 2 tanh-GELU in fp32)", act);
+  if (resid && resid_dtype != TK_BF16 && resid_dtype != TK_F32) return fail(TK_EINVAL, "bf16w_dense: bad resid_dtype");
+  if (resid && (ldr < N || ldr % (resid_dtype == TK_F32 ? 4 : 8) || !aligned16(resid)))
+    return fail(TK_EINVAL, "bf16w_dense: residual must be 16-byte aligned with a pitch >= N that keeps rows 16-byte aligned");
+  GemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.x = x;
+  a.ldx = ldx;
+  a.w16 = 1;
+  a.w = (const uint8_t*)w_packed;
+  a.bias = (const u16*)bias;
+  a.y = (u16*)y;
+  a.ldy = ldy;
+  a.resid = resid;
+  a.ldr = ldr;
+  a.resid_f32 = resid_dtype == TK_F32;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.KT = (K + 31) / 32;
+  a.ntiles = (N + 31) / 32;
+  a.act = act;
+  a.vec = a.vec16 = 1;
+  const int cus = device_cus();
+  const DenseTile* best = nullptr;
+  int ks = split_k > 0 ? split_k : 1;
+  float best_cost = 0.f;
+  for (const DenseTile& t : kDenseTiles) {
+    if (tile && t.id != tile) continue;
+    const int blocks0 = ((M + t.rows - 1) / t.rows) * ((N + t.cols - 1) / t.cols);
+    int k1 = 1;
+    if (split_k > 0) {
+      k1 = split_k;
+    } else {
+      // few blocks and a long K: split, keeping at least 32 k tiles per split
+      k1 = cus / blocks0;
+      if (k1 > a.KT / 32) k1 = a.KT / 32;
+      if (k1 < 1) k1 = 1;
+    }
+    const float c = dense_cost(t, M, N, a.KT, k1, cus);
+    if (!best || c < best_cost) best = &t, best_cost = c, ks = k1;
+  }
+  if (!best) return fail(TK_EINVAL, "bf16w_dense: tile=%d (0 = automatic, or 42, 41, 32, 31, 22, 21, 12, 11)", tile);
+  const int blocks0 = ((M + best->rows - 1) / best->rows) * ((N + best->cols - 1) / best->cols);
+  const size_t per_split = (size_t)best->rows * best->cols * 4;
+  if (ks > 1) {
+    const size_t have = ws && ws_bytes > kPartialOff ? (ws_bytes - kPartialOff < kPartialBytes ? ws_bytes - kPartialOff : kPartialBytes) / (per_split * blocks0) : 0;
+    if ((size_t)ks > have || blocks0 > kMaxCounters) {
+      if (split_k > 1) return fail(TK_EWORKSPACE, "bf16w_dense: split_k=%d needs %zu bytes of partial space", ks, per_split * blocks0 * ks);
+      ks = have > 1 && blocks0 <= kMaxCounters ? (int)have : 1;
+    }
+  }
+  if (ks > a.KT) ks = a.KT;
+  a.ksplit = ks;
+  a.kt_q = a.KT / ks;
+  a.kt_r = a.KT % ks;
+  a.partial = ks > 1 ? (float*)((char*)ws + kPartialOff) : nullptr;
+  a.counters = ks > 1 ? (int*)ws : nullptr;
+  if (tk_launch_bf16w_wide(a, best->id, (hipStream_t)stream)) return fail(TK_ELAUNCH, "bf16w_dense: launch failed (%s)", hipGetErrorString(hipGetLastError()));
+  return TK_OK;
+}
+
 int tk_quant_act_rows(const void* x, int ldx, void* a8, int lda, void* sa, int M, int K, int mode, void* stream) {
   if (M <= 0 || K <= 0 || K % 8 || K > tk_quant_act_max_k()) return fail(TK_EINVAL, "quant_act_rows: bad shape M=%d K=%d (K a multiple of 8, at most %d)", M, K, tk_quant_act_max_k());
   if (!x || !a8 || !sa || ldx < K || ldx % 8 || lda < K || lda % 8) return fail(TK_EINVAL, "quant_act_rows: null pointer or row pitch not a multiple of 8 >= K");

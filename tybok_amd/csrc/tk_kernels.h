@@ -50,6 +50,9 @@ struct GemmArgs {
   // many-row kernels: y (and the residual) allow 16-byte row-contiguous accesses (pitches multiples of 8
   // elements, 16-byte aligned pointers): the epilogue stores whole row segments through LDS
   int vec16;
+  // bf16-weight many-row kernel only: bf16 [N] bias added to the accumulator, or nullptr; there act is
+  // 0 none, 1 tanh-GELU of the bf16-rounded pre-activation, 2 tanh-GELU of the fp32 pre-activation
+  const unsigned short* bias;
 };
 
 struct QuantActArgs {
@@ -210,6 +213,8 @@ int tk_launch_pack(const void* w0, const void* w1, void* out, int N, int K, int 
 int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st);
 int tk_launch_fill_zero(int* p, int n, hipStream_t st);
 int tk_launch_decode_fp8(float* out, hipStream_t st);
+// tile = 10 * (m tiles per block) + (n tiles per wave): 42, 41, 32, 31, 22, 21, 12 or 11
+int tk_launch_bf16w_wide(const GemmArgs& a, int tile, hipStream_t st);
 // plain 16-byte-per-lane read of `bytes` (a multiple of blocks * 4096) by `blocks` blocks of 256 threads
 int tk_launch_stream_read(const void* src, size_t bytes, int blocks, int* sink, hipStream_t st);
 struct TransposeVArgs {

@@ -64,6 +64,11 @@ SIGNATURES: dict[str, tuple] = {
          c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
          c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
+    "tk_bf16w_dense": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+         c_int, c_void_p, c_size_t, c_void_p],
+    ),  # fmt: skip
     "tk_attn_prepare_kv": (
         c_int,
         [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,

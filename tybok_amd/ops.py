@@ -306,6 +306,45 @@ def pack_bf16_weight(w: torch.Tensor, rope_half: int = 0) -> PackedBf16Weight:
     return PackedBf16Weight(out, n, k, rope_half)
 
 
+_DENSE_ACTS = {None: 0, "none": 0, "gelu_tanh": 1, "gelu_tanh_fp32": 2}
+
+
+def bf16w_dense(
+    x: torch.Tensor,
+    w: PackedBf16Weight,
+    bias: torch.Tensor | None = None,
+    act: str | None = None,
+    *,
+    resid: torch.Tensor | None = None,
+    out: torch.Tensor | None = None,
+    tile: int = 0,
+    split_k: int = 0,
+    ws: Workspace | None = None,
+) -> torch.Tensor:
+    """``bf16(resid + act(bf16(x @ W^T + bias)))`` for ``x [M, K]`` bf16 and a packed bf16 weight: the linears of the
+    vision towers on the many-row MFMA kernel.  ``act``: ``"gelu_tanh"`` applies the tanh GELU to the bf16-rounded
+    linear output (what ``gelu(linear(x))`` on bf16 tensors computes), ``"gelu_tanh_fp32"`` to the fp32 one (a GEMM
+    with the activation in its epilogue).  ``tile`` picks the block tile (0 = by shape)."""
+    lib = native.lib()
+    if w.rope_half:
+        raise ValueError("bf16w_dense takes weights packed in natural tile order (rope_half = 0)")
+    m, ldx = _check_act(x, w.k)
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != w.n or not bias.is_contiguous() or bias.device != x.device):
+        raise ValueError(f"bias must be a contiguous bf16 vector of {w.n} elements on the activations' device")
+    if out is None:
+        out = torch.empty(m, w.n, dtype=torch.bfloat16, device=x.device)
+    if out.dtype != torch.bfloat16 or out.shape != (m, w.n) or out.stride(1) != 1:
+        raise ValueError("out must be bf16 [M, N] with unit inner stride")
+    rp, ldr, rdt = _resid_args(resid, m, w.n)
+    ws = ws or default_workspace(x.device)
+    rc = lib.tk_bf16w_dense(
+        x.data_ptr(), ldx, w.data.data_ptr(), None if bias is None else bias.data_ptr(), _DENSE_ACTS[act], out.data_ptr(),
+        out.stride(0), rp, ldr, rdt, m, w.n, w.k, tile, split_k, ws.ptr, ws.nbytes, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_bf16w_dense")
+    return out
+
+
 def _norm_ptr(norm_w: torch.Tensor | None, k: int) -> int | None:
     if norm_w is None:
         return None

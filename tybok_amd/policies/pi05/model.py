@@ -174,6 +174,12 @@ class PI05Model:
                     pad_rows(self.p[lp + "self_attn.out_proj.weight"].t().contiguous()).t().to(BF16).contiguous(),
                     self.p[lp + "self_attn.out_proj.bias"].to(BF16),
                 )
+        # with both low-precision tiers in bf16 every linear of the tower runs on the many-row MFMA kernel: the
+        # same weights in its tile order (shapes it does not take -- K % 16, N % 8 -- stay on the library GEMM)
+        self.vis_dense: dict[str, tuple] = {}
+        if self.vit_lowp_attn and self.vit_mlp_dtype == BF16 and self.device.type == "cuda" and self.vis_head_pad in (64, 96):
+            if all(w.shape[1] % 16 == 0 and w.shape[0] % 8 == 0 for w, _ in self.vis_lowp.values()):
+                self.vis_dense = {n: (tk.pack_bf16_weight(w), b.contiguous()) for n, (w, b) in self.vis_lowp.items()}
         self.set_num_steps(cfg.num_steps)
 
     def lin(self, name: str, x: torch.Tensor) -> torch.Tensor:
@@ -287,12 +293,22 @@ class PI05Model:
         hd = vh // heads
         ln = lambda i, n: (p[f"{VIS}encoder.layers.{i}.layer_norm{n}.weight"], p[f"{VIS}encoder.layers.{i}.layer_norm{n}.bias"])  # noqa: E731
         h = tk.layer_norm(x, *ln(0, 1), EPS)
+
+        def dense(name: str, t: torch.Tensor, act: str | None = None) -> torch.Tensor:
+            if self.vis_dense:
+                w, bias = self.vis_dense[name]
+                return tk.bf16w_dense(t.reshape(-1, t.shape[-1]), w, bias, act, ws=self.ws).view(*t.shape[:-1], w.n)
+            if act:  # library GEMM with the activation in its epilogue
+                return tk.linear_gelu_tanh(t, *self.vis_lowp[name])
+            return F.linear(t, *self.vis_lowp[name])
+
         for i in range(cfg.vision_layers):
             lp = f"{VIS}encoder.layers.{i}."
-            qkv = F.linear(h, *self.vis_lowp[lp + "self_attn.qkv"]).view(b, -1, 3, heads, hp)
+            qkv = dense(lp + "self_attn.qkv", h).view(b, -1, 3, heads, hp)
             a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], tk.transpose_v(qkv[:, :, 2]), scale=hd**-0.5, ws=self.ws)
-            x, h = tk.add_layer_norm(x, F.linear(a, *self.vis_lowp[lp + "self_attn.out_proj"]), *ln(i, 2), EPS)
-            m = F.linear(tk.linear_gelu_tanh(h, *self.vis_lowp[lp + "mlp.fc1"]), *self.vis_lowp[lp + "mlp.fc2"])
+            x, h = tk.add_layer_norm(x, dense(lp + "self_attn.out_proj", a), *ln(i, 2), EPS)
+            # fc1's GELU on the bf16-rounded linear output: the eager tier's gelu(fc1(h)) on bf16 tensors (vision.py:79-87)
+            m = dense(lp + "mlp.fc2", dense(lp + "mlp.fc1", h, "gelu_tanh"))
             if i + 1 < cfg.vision_layers:
                 x, h = tk.add_layer_norm(x, m, *ln(i + 1, 1), EPS)
             else:

@@ -149,12 +149,19 @@ class SmolVLAModel:
             self.vlm_qkv, self.vlm_o = self._pack_attention_weights(TXT, lambda i: False)
         if self.fused_vit:
             # vision q|k|v as one projection (one GEMM over all cameras' patches instead of three)
+            # and every linear of the tower in the tile order of the many-row MFMA kernel
             self.vis_qkv = []
+            self.vis_dense: dict[str, tuple] = {}
             for i in range(cfg.vlm_config.vision_config.num_hidden_layers):
-                lp = f"{VIS}encoder.layers.{i}.self_attn."
-                w = torch.cat([self.p[lp + n + "_proj.weight"] for n in "qkv"], dim=0).contiguous()
-                b = torch.cat([self.p[lp + n + "_proj.bias"] for n in "qkv"], dim=0).contiguous()
-                self.vis_qkv.append((w, b))
+                lp = f"{VIS}encoder.layers.{i}."
+                w = torch.cat([self.p[lp + "self_attn." + n + "_proj.weight"] for n in "qkv"], dim=0).contiguous()
+                b = torch.cat([self.p[lp + "self_attn." + n + "_proj.bias"] for n in "qkv"], dim=0).contiguous()
+                self.vis_qkv.append((tk.pack_bf16_weight(w), b))
+                for n in ("self_attn.out_proj", "mlp.fc1", "mlp.fc2"):
+                    self.vis_dense[lp + n] = (tk.pack_bf16_weight(self.p[lp + n + ".weight"]), self.p[lp + n + ".bias"].contiguous())
+            pw = self.p[VIS + "embeddings.patch_embedding.weight"]
+            self.vis_dense["patch"] = (tk.pack_bf16_weight(pw.reshape(pw.shape[0], -1).contiguous()), self.p[VIS + "embeddings.patch_embedding.bias"].contiguous())
+            self.vis_dense["connector"] = (tk.pack_bf16_weight(self.p[CONNECTOR + ".weight"]), self.p.get(CONNECTOR + ".bias"))
         if self.fused_expert:
             self._pack_expert_projections()
             # V^T of the action tokens [G, D, chunk rounded up to 32]; the projection kernel writes
@@ -239,7 +246,10 @@ class SmolVLAModel:
         n_h, n_w = image.shape[2] // ps, image.shape[3] // ps
         # non-overlapping patch convolution as one GEMM over unfolded patches
         x = image.to(BF16).view(b, 3, n_h, ps, n_w, ps).permute(0, 2, 4, 1, 3, 5).reshape(b, n_h * n_w, 3 * ps * ps)
-        x = F.linear(x, self.patch_w, p[VIS + "embeddings.patch_embedding.bias"])
+        if self.fused_vit:
+            x = self._dense("patch", x)
+        else:
+            x = F.linear(x, self.patch_w, p[VIS + "embeddings.patch_embedding.bias"])
         x = x + p[VIS + "embeddings.position_embedding.weight"][self.vis_pos][None]
         heads = v.num_attention_heads
         hd = v.hidden_size // heads
@@ -252,11 +262,12 @@ class SmolVLAModel:
                 # packed q|k|v GEMM, then the HIP attention (one problem per camera): q.K^T rounded to
                 # bf16 before the fp32 scale and softmax, exactly what the bf16 matmul below produces
                 w_qkv, b_qkv = self.vis_qkv[i]
-                qkv = F.linear(h, w_qkv, b_qkv).view(b, -1, 3, heads, hd)
+                qkv = tk.bf16w_dense(h.view(-1, h.shape[-1]), w_qkv, b_qkv, ws=self.ws).view(b, -1, 3, heads, hd)
                 vt = tk.transpose_v(qkv[:, :, 2])
                 a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, ws=self.ws)
-                x, h = tk.add_layer_norm(x, self.lin(lp + "self_attn.out_proj", a), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
-                m = self.lin(lp + "mlp.fc2", tk.linear_gelu_tanh(h, p[lp + "mlp.fc1.weight"], p[lp + "mlp.fc1.bias"]))
+                x, h = tk.add_layer_norm(x, self._dense(lp + "self_attn.out_proj", a), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
+                # fc1's GELU on the bf16-rounded linear output, as gelu(linear(h)) on bf16 tensors computes it
+                m = self._dense(lp + "mlp.fc2", self._dense(lp + "mlp.fc1", h, "gelu_tanh"))
                 if i + 1 < v.num_hidden_layers:
                     nx = f"{VIS}encoder.layers.{i + 1}."
                     x, h = tk.add_layer_norm(x, m, p[nx + "layer_norm1.weight"], p[nx + "layer_norm1.bias"], v.layer_norm_eps)
@@ -278,7 +289,12 @@ class SmolVLAModel:
         side = int(seq**0.5)
         x = x.view(b, side, side, dim).view(b, side, side // s, dim * s).permute(0, 2, 1, 3)
         x = x.reshape(b, side // s, side // s, dim * s * s).permute(0, 2, 1, 3).reshape(b, seq // (s * s), dim * s * s)
-        return self.lin(CONNECTOR, x)
+        return self._dense("connector", x.contiguous()) if self.fused_vit else self.lin(CONNECTOR, x)
+
+    def _dense(self, name: str, x: torch.Tensor, act: str | None = None) -> torch.Tensor:
+        """A linear of the vision tower on the many-row MFMA kernel; ``x [..., K]`` bf16 -> ``[..., N]`` bf16."""
+        w, bias = self.vis_dense[name]
+        return tk.bf16w_dense(x.reshape(-1, x.shape[-1]), w, bias, act, ws=self.ws).view(*x.shape[:-1], w.n)
 
     def embed_prefix(self, images, img_masks, lang_tokens, lang_masks, state):
         """-> ``(embs fp32 [1,P,hidden], pad_masks bool [1,P], att_masks bool [1,P])`` (flow_matching.py:160-257)."""
