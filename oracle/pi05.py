@@ -58,9 +58,14 @@ class PI05Shape:
     min_period: float = 4e-3
     max_period: float = 4.0
     # drift tiers of the vision tower (tybok/policies/pi05/engine.py:196-230):
-    #   vit_mlp_dtype: fc1 / gelu / fc2 run in that dtype, cast at the boundary (vision.py:79-87);
+    #   vit_mlp_dtype: fc1 / gelu / fc2 run in that dtype, cast at the boundary (vision.py:79-87); pinned by a
+    #                  fixture written from the reference's own tower after set_mlp_dtype
+    #                  (tests/golden/pi05_small_vit_tiers.npz);
     #   vit_lowp_attn: q/k/v and out_proj run in bf16 too; attention scores and softmax in fp32, the
-    #                  probabilities rounded to bf16 for P.V (fp32 accumulate, bf16 result).
+    #                  probabilities rounded to bf16 for P.V (fp32 accumulate, bf16 result).  PARITY UNPINNED:
+    #                  this restates the HIP backend's own tier, not the reference's fused tower kernels
+    #                  (vision.py:116-173 run q|k|v in fp16 on Triton kernels that cannot run here); it is a
+    #                  regression check of that tier, bounded against the fp32 tower, not a parity claim.
     vit_mlp_dtype: torch.dtype | None = None
     vit_lowp_attn: bool = False
     # W8A8 tier of the VLM MLP (tybok/policies/pi05/models/triton_prefill_mlp.py:145-166): activations quantised

@@ -2,7 +2,7 @@
 
 Run ONCE in the build container (the reference is not available elsewhere):
 
-    python tests/golden/make_golden.py [smolvla|pi05|all] [case]
+    python tests/golden/make_golden.py [smolvla|pi05|pi05_vit|all] [case]
 
 For each case the reference's eager model classes (``/root/reference/tybok/policies/<model>/models``)
 are constructed on the CPU from plain config dataclasses (no checkpoint, no tokenizer), loaded with
@@ -147,6 +147,45 @@ def pi05_case(name: str) -> dict:
     return out
 
 
+def pi05_vit_tiers() -> dict:
+    """The reference's eager SigLIP tower with ``set_mlp_dtype`` (tybok/policies/pi05/models/vision.py:79-87,
+    223-235; the engine's ``--vit-mlp-dtype``, engine.py:211-230) on the small case: samples of both cameras' image
+    embeddings (tower + projector) for the fp32 tower and for the bf16 and fp16 MLP tiers."""
+    _import_reference()
+    from tybok.policies.pi05 import config as rcfg
+    from tybok.policies.pi05.models.flow_matching import PI05FlowMatching
+
+    case = cases.PI05_CASES["small"]
+    cfg, sd, inputs = cases.pi05_build(case)
+    rcfg.GEMMA_VARIANTS["golden_vlm"] = dict(cfg.paligemma_dims)
+    rcfg.GEMMA_VARIANTS["golden_expert"] = dict(cfg.expert_dims)
+    ref_cfg = rcfg.PI05Config(
+        paligemma_variant="golden_vlm", action_expert_variant="golden_expert", num_steps=cfg.num_steps,
+        tokenizer_max_length=cfg.tokenizer_max_length,
+    )  # fmt: skip
+    ref_cfg._image_features = list(cfg.image_features)
+    images = [img * 2.0 - 1.0 for img in inputs["images"]]
+    out: dict[str, np.ndarray] = {}
+    for tag, dt in (("fp32", None), ("bf16", torch.bfloat16), ("fp16", torch.float16)):
+        default = torch.get_default_dtype()
+        torch.set_default_dtype(torch.bfloat16)
+        try:
+            model = PI05FlowMatching(ref_cfg)
+        finally:
+            torch.set_default_dtype(default)
+        vt = model.paligemma_with_expert.paligemma.model.vision_tower.vision_model
+        vt.encoder.layers = vt.encoder.layers[: cfg.vision_layers]
+        model.eval()
+        _load(model, sd)
+        if dt is not None:
+            vt.set_mlp_dtype(dt)
+        with torch.inference_mode():
+            for cam, img in enumerate(images):
+                emb = model.paligemma_with_expert.embed_image(img)
+                out[f"emb_{tag}_cam{cam}"] = emb[0, ::8, ::16].float().numpy()  # 32 patches x 128 channels
+    return out
+
+
 def main() -> None:
     which = sys.argv[1] if len(sys.argv) > 1 else "all"
     torch.manual_seed(0)
@@ -155,6 +194,11 @@ def main() -> None:
         jobs += [("smolvla", n) for n in cases.SMOLVLA_CASES]
     if which in ("pi05", "all"):
         jobs += [("pi05", n) for n in cases.PI05_CASES]
+    if which in ("pi05_vit", "all"):
+        t0 = time.time()
+        path = os.path.join(HERE, "pi05_small_vit_tiers.npz")
+        np.savez_compressed(path, **pi05_vit_tiers())
+        print(f"pi05 vit tiers: wrote {path} ({os.path.getsize(path) / 1024:.0f} KiB) in {time.time() - t0:.1f}s", flush=True)
     only = sys.argv[2] if len(sys.argv) > 2 else None  # optional: one case name
     for model, name in jobs:
         if only and name != only:

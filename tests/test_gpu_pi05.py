@@ -155,6 +155,26 @@ def test_full_depth_bf16_path_matches_reference_golden(full_case):
     assert e_max <= 1.25e-2 and e_mean <= 3e-3
 
 
+@pytest.mark.parametrize("tag,vit", [("fp32", {}), ("bf16", dict(vit_mlp_dtype=torch.bfloat16)), ("fp16", dict(vit_mlp_dtype=torch.float16))])
+def test_vision_tower_mlp_tiers_against_the_reference_eager_tower(tag, vit):
+    # golden written from the reference's own tower after set_mlp_dtype (tests/golden/make_golden.py pi05_vit)
+    from tybok_amd.policies.pi05.model import PI05Model
+
+    gold = np.load(os.path.join(HERE, "golden", "pi05_small_vit_tiers.npz"))
+    cfg, sd, inp = cases.pi05_build(cases.PI05_CASES["small"])
+    model = PI05Model(cfg, sd, "cuda", **vit)
+    worst = 0.0
+    with torch.no_grad():
+        for cam, img in enumerate(inp["images"]):
+            got = model.embed_image((img * 2.0 - 1.0).cuda()).cpu()[0, ::8, ::16].numpy()
+            want = gold[f"emb_{tag}_cam{cam}"]
+            scale = float(np.abs(want).max())
+            worst = max(worst, float(np.abs(got - want).max()) / scale)
+    print(f"pi05 vision tier {tag}: max|err| vs the reference tower, relative to |emb|max: {worst:.3g}")
+    # fp32 tower: GPU fp32 GEMMs against CPU ones; low-precision MLP: one bf16 / fp16 ulp of a 2-layer tower's output
+    assert worst <= (2e-4 if tag == "fp32" else 4e-3 if tag == "fp16" else 2e-2)
+
+
 @pytest.mark.parametrize("vit", [dict(vit_mlp_dtype=torch.bfloat16), dict(vit_mlp_dtype=torch.float16), dict(vit_mlp_dtype=torch.bfloat16, vit_lowp_attn=True)])
 def test_vision_tower_drift_tiers_match_their_oracle(vit):
     # the low-precision vision tiers against the oracle's restatement of the same tier, and against the

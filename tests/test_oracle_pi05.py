@@ -45,3 +45,22 @@ def test_oracle_matches_reference_golden(name):
     assert _maxdiff(v_half[0].numpy(), gold["v_t_half"]) <= 1e-5
     assert _maxdiff(chunk[0].numpy(), gold["chunk"]) <= 1e-5
     assert float(np.abs(gold["chunk"]).max()) > 0.1
+
+
+@pytest.mark.parametrize("tag,dt", [("fp32", None), ("bf16", torch.bfloat16), ("fp16", torch.float16)])
+def test_oracle_vision_mlp_tiers_match_the_reference_eager_tower(tag, dt):
+    # the reference's own tower after set_mlp_dtype (tybok/policies/pi05/models/vision.py:79-87,223-235), written by
+    # tests/golden/make_golden.py pi05_vit: samples of both cameras' image embeddings
+    gold = np.load(os.path.join(HERE, "golden", "pi05_small_vit_tiers.npz"))
+    cfg, sd, inp = cases.pi05_build(cases.PI05_CASES["small"])
+    shape = O.PI05Shape(depth=cfg.paligemma_dims["depth"], vis_layers=cfg.vision_layers, num_steps=cfg.num_steps, vit_mlp_dtype=dt)
+    w = Weights(sd)
+    with torch.no_grad():
+        for cam, img in enumerate(inp["images"]):
+            emb = O.embed_image(w, shape, img * 2.0 - 1.0)
+            want = gold[f"emb_{tag}_cam{cam}"]
+            # same torch CPU kernels on the same operands: equal up to the summation order of a reshaped GEMM
+            assert _maxdiff(emb[0, ::8, ::16].numpy(), want) <= 2e-5 * max(1.0, float(np.abs(want).max()))
+    # the tiers are real: the low-precision fixtures differ from the fp32 one
+    assert _maxdiff(gold["emb_bf16_cam0"], gold["emb_fp32_cam0"]) > 1e-4
+    assert _maxdiff(gold["emb_fp16_cam0"], gold["emb_fp32_cam0"]) > 1e-6

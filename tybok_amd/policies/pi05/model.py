@@ -130,10 +130,10 @@ class PI05Model:
             self.exp_qkv, self.exp_o = pack_stack(EXP, self.ed["depth"])
         if self.fused_prefill:
             self.vlm_qkv, self.vlm_o = pack_stack(VLM, self.depth)
-            # the same q|k|v weights row-major, for prefixes long enough that the projection is a plain
-            # many-row GEMM (library call) followed by the rotary kernel
-            self.vlm_qkv_plain = [
-                torch.cat([self.p[f"{VLM}layers.{i}.self_attn.{n}_proj.weight"] for n in "qkv"], dim=0).to(BF16).contiguous()
+            # the same q|k|v weights in natural tile order, for prefixes long enough that the projection runs on
+            # the many-row MFMA kernel, followed by the rotary kernel
+            self.vlm_qkv_dense = [
+                tk.pack_bf16_weight(torch.cat([self.p[f"{VLM}layers.{i}.self_attn.{n}_proj.weight"] for n in "qkv"], dim=0).to(BF16).contiguous())
                 for i in range(self.depth)
             ]
             # Gemma RMSNorm x * rstd * (1 + w) is the adaptive norm with scale = w and shift = 0
@@ -377,8 +377,8 @@ class PI05Model:
         for i in range(self.depth):
             norm_in, norm_post = self.vlm_norms[i]
             if many_rows:
-                # norm, library GEMM, rotary embedding in place, V^T through the tiled transpose
-                qkv = torch.matmul(tk.rms_norm_rows(hidden, ada=norm_in, eps=EPS), self.vlm_qkv_plain[i].t(), out=qkv_all[i])
+                # norm, many-row GEMM, rotary embedding in place, V^T through the tiled transpose
+                qkv = tk.bf16w_dense(tk.rms_norm_rows(hidden, ada=norm_in, eps=EPS), self.vlm_qkv_dense[i], out=qkv_all[i], ws=self.ws)
                 tk.rope_rows(qkv, self.rope_tables_hip, pos32, nq + nkv, rope_bf16=True)
                 tk.transpose_v(qkv[:, nq + nkv :].view(1, p_len, nkv // 64, 64), out=vt_all[i].view(1, nkv // 64, 64, p_pad))
             else:
@@ -389,7 +389,10 @@ class PI05Model:
             k = qkv[:, nq : nq + nkv].view(p_len, g, d)
             cache = tk.PrefixKV(k, vt_all[i].view(g, d, p_pad))
             att = tk.expert_attn(qkv[:, :nq].view(p_len, heads, d), cache, None, None, tk.MASK_NONE, mask2d=mask2d, logits_bf16=True, ws=self.ws)
-            out = tk.bf16w_linear(att, self.vlm_o[i], resid=hidden, ws=self.ws)
+            if many_rows:
+                out = tk.bf16w_dense(att, self.vlm_o[i], resid=hidden, ws=self.ws)  # bf16(bf16(att . Wo^T) + hidden), as below
+            else:
+                out = tk.bf16w_linear(att, self.vlm_o[i], resid=hidden, ws=self.ws)
             mlp = self.vlm_mlp[i]
             if mlp.w8a8:
                 normed = tk.rms_norm_rows(out, ada=norm_post, eps=EPS)
