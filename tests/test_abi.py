@@ -78,7 +78,39 @@ def _cases():
     )
     ln = lambda **kw: _args(dict(x=P, ldx=768, xdt=0, w=P, b=P, wdt=0, eps=1e-6, y=P, ldy=768, M=64, K=768, st=None), kw)  # noqa: E731
     tv = lambda **kw: _args(dict(v=P, sb=1 << 20, sl=2304, sh=64, vt=P, tsb=1 << 20, tsh=65536, tsd=1024, keys=1024, B=3, Pk=1024, G=12, D=64, st=None), kw)  # noqa: E731
+    qa = lambda **kw: _args(dict(x=P, ldx=2048, a8=P, lda=2048, sa=P, M=712, K=2048, mode=0, st=None), kw)  # noqa: E731
+    w8 = lambda **kw: _args(  # noqa: E731
+        dict(a8=P, lda=2048, sa=P, w=P, sw=P, y=P, ldy=16384, resid=None, ldr=0, rdt=0, M=712, N=16384, K=2048, split=0, ws=None, wsb=0, st=None), kw
+    )
+    w8ffn = lambda **kw: _args(  # noqa: E731
+        dict(x=P, ldx=2048, wgu=P, sg=P, su=P, wd=P, sd=P, y=P, ldy=2048, resid=None, ldr=0, rdt=0, M=712, K=2048, I=16384, act=1, ws=P, wsb=1 << 27, st=None), kw
+    )
+    dense = lambda **kw: _args(  # noqa: E731
+        dict(x=P, ldx=768, w=P, bias=P, act=0, y=P, ldy=3072, resid=None, ldr=0, rdt=0, M=3072, N=3072, K=768, tile=0, split=0, ws=None, wsb=0, st=None), kw
+    )
+    static = lambda **kw: _args(  # noqa: E731
+        dict(x=P, ldx=2048, w=P, scale=P, y=P, ldy=16384, resid=None, ldr=0, rdt=0, gate=None, M=50, N=16384, K=2048, split=0, st=None), kw
+    )
+    sread = lambda **kw: _args(dict(src=P, bytes=1 << 25, blocks=256, sink=P, st=None), kw)  # noqa: E731
     return [
+        ("tk_quant_act_rows", qa(K=2044), -1, "multiple of 8"),
+        ("tk_quant_act_rows", qa(K=32768, ldx=32768, lda=32768), -1, "at most"),
+        ("tk_quant_act_rows", qa(mode=2), -1, "mode 2"),
+        ("tk_quant_act_rows", qa(x=P + 8), -1, "16-byte"),
+        ("tk_w8a8_gemm", w8(K=2040), -1, "multiple of 16"),
+        ("tk_w8a8_gemm", w8(lda=2000), -1, "lda"),
+        ("tk_w8a8_gemm", w8(sa=None), -1, "null pointer"),
+        ("tk_w8a8_gemm", w8(N=16382), -1, "multiples of 4"),
+        ("tk_w8a8_gemm", w8(split=4), -2, "partial space"),
+        ("tk_w8a8_gated_ffn", w8ffn(act=9), -1, "unknown activation"),
+        ("tk_bf16w_dense", dense(K=776, ldx=776), -1, "multiple of 16"),
+        ("tk_bf16w_dense", dense(ldy=3076), -1, "multiple of 8"),
+        ("tk_bf16w_dense", dense(act=3), -1, "act=3"),
+        ("tk_bf16w_dense", dense(tile=33), -1, "tile=33"),
+        ("tk_bf16w_dense", dense(resid=P, ldr=3070, rdt=0), -1, "residual"),
+        ("tk_bf16w_dense", dense(y=P + 8), -1, "16-byte aligned"),
+        ("tk_fp8w_gemm_static", static(M=65), -1, "exceeds the 64 rows"),
+        ("tk_debug_stream_read", sread(bytes=1000), -1, "multiple"),
         ("tk_fp8w_gemm", gemm(K=2040), -1, "multiple of 16"),
         ("tk_fp8w_gemm", gemm(ldx=1024), -1, "ldx"),
         ("tk_fp8w_gemm", gemm(x=P + 2), -1, "16-byte aligned"),
