@@ -233,6 +233,67 @@ def tower_attn_launch_us(cameras: int = 3, tokens: int = 1024, heads: int = 12, 
     return e0.elapsed_time(e1) * 1e3 / (reps * launches)
 
 
+def graph_launch_us(fn, launches: int = 20, reps: int = 10) -> float:
+    """Average duration (us) of one call of ``fn`` inside a replayed graph of ``launches`` back-to-back calls."""
+    import torch
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(3):
+            fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
+        for _ in range(launches):
+            fn()
+    spin_up(60.0)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * launches)
+
+
+# the four linears of a SmolVLA tower layer over 3 x 1024 patches: (name, M, K, N, activation)
+TOWER_LINEARS = (("qkv", 3072, 768, 2304, None), ("out_proj", 3072, 768, 768, None), ("fc1_gelu", 3072, 768, 3072, "gelu_tanh"), ("fc2", 3072, 3072, 768, None))
+
+
+def dense_launch_us(m: int, k: int, n: int, act: str | None, launches: int = 20, reps: int = 10) -> float:
+    """Average duration (us) of one many-row bf16 linear (bias, optional GELU) inside a replayed graph."""
+    import torch
+
+    from tybok_amd import ops as tk
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16).cuda()
+    w = tk.pack_bf16_weight((torch.randn(n, k, generator=g) / k**0.5).to(torch.bfloat16).cuda())
+    b = torch.randn(n, generator=g).to(torch.bfloat16).cuda()
+    out = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+    return graph_launch_us(lambda: tk.bf16w_dense(x, w, b, act, out=out), launches, reps)
+
+
+def attn_d256_launch_us(launches: int = 20, reps: int = 10) -> float:
+    """Average duration (us) of one pi0.5 action-expert attention launch (50 queries, 712 prefix + 50 own keys,
+    8 heads over one 256-wide K/V head, bidirectional suffix, bf16-rounded logits) inside a replayed graph."""
+    import torch
+
+    from oracle.inputs import attn_case
+    from tybok_amd import ops as tk
+
+    q, k_pre, v_pre, k_suf, v_suf = (t.cuda() for t in attn_case(50, 712, 8, 1, 256))
+    prefix = tk.prepare_prefix_kv(k_pre, v_pre)
+    vt = torch.zeros(1, 256, 64, dtype=torch.bfloat16, device="cuda")
+    vt[:, :, :50] = v_suf.permute(1, 2, 0)
+    suffix = tk.SuffixKV(k_suf, vt)
+    out = torch.empty(50, 2048, dtype=torch.bfloat16, device="cuda")
+    return graph_launch_us(lambda: tk.expert_attn(q, prefix, suffix, None, tk.MASK_BIDIR, logits_bf16=True, out=out), launches, reps)
+
+
 def device_frame(engine, cameras: int, seed: int = 0) -> dict:
     """Synthetic observation (uint8-valued images / 255, random state) already on the GPU."""
     import torch
@@ -360,6 +421,8 @@ def main() -> None:
     ap.add_argument("--gemm-only", action="store_true", help="only the roofline GEMM loop plus a plain copy of known size (for rocprofv3 runs)")
     ap.add_argument("--gemm-shape", type=int, nargs=3, metavar=("M", "K", "N"), default=(50, 2048, 16384), help="shape of the --gemm-only loop")
     ap.add_argument("--attn-only", action="store_true", help="only the action-expert attention loop (for rocprofv3 runs)")
+    ap.add_argument("--attn-d256-only", action="store_true", help="only the pi0.5 action-expert attention loop, 256-wide heads (for rocprofv3 runs)")
+    ap.add_argument("--dense-only", action="store_true", help="only the many-row bf16 linears of a SmolVLA tower layer (for rocprofv3 runs)")
     ap.add_argument("--tower-attn-only", action="store_true", help="only the vision-tower attention loop, 3 cameras x 1024 tokens (for rocprofv3 runs)")
     ap.add_argument("--ffn-only", action="store_true", help="only the many-row (M=712) fp8 GeGLU FFN loop (for rocprofv3 runs)")
     ap.add_argument("--w8a8", action="store_true", help="with --ffn-only: the W8A8 FFN (fp8 x fp8 matrix instruction) instead of the weight-only one")
@@ -393,6 +456,19 @@ def main() -> None:
         spin_up()
         us = ffn_launch_us(712, 2048, 16384, launches=5, reps=args.steps, w8a8=args.w8a8)
         print(json.dumps({"ffn_only": {"M": 712, "K": 2048, "I": 16384, "w8a8": bool(args.w8a8), "us": round(us, 1), "TFLOPs": round(6.0 * 712 * 2048 * 16384 / us / 1e6, 1)}}), flush=True)
+        return
+    if args.dense_only:
+        spin_up()
+        res = {}
+        for name, m, k, n, act in TOWER_LINEARS:
+            us = dense_launch_us(m, k, n, act, launches=10, reps=args.steps)
+            res[name] = {"M": m, "K": k, "N": n, "us": round(us, 2), "TFLOPs": round(2.0 * m * k * n / us / 1e6, 1)}
+        print(json.dumps({"dense_only": res}), flush=True)
+        return
+    if args.attn_d256_only:
+        spin_up()
+        us = attn_d256_launch_us(launches=20, reps=args.steps)
+        print(json.dumps({"attn_d256_only": {"M": 50, "P": 712, "S": 50, "H": 8, "G": 1, "D": 256, "us": round(us, 2)}}), flush=True)
         return
     if args.tower_attn_only:
         spin_up()
@@ -535,7 +611,11 @@ def main() -> None:
         "ffn_M50_K720_I2048": {"us": round(c1_us, 2), "GBps": round(c1_bytes / c1_us / 1e3, 1), "launches": 2},
         "expert_attn_M50_P241_S50_H15_G5_D64": {"us": round(attn_launch_us(launches=50, reps=10), 2)},
         "tower_attn_B3_M1024_H12_D64": {"us": round(tower_attn_launch_us(launches=20, reps=10), 2)},
+        "pi05_expert_attn_M50_P712_S50_H8_G1_D256": {"us": round(attn_d256_launch_us(launches=20, reps=10), 2)},
     }
+    for name, dm, dk, dn, dact in TOWER_LINEARS:  # the vision tower's linears on the many-row bf16 kernel
+        us = dense_launch_us(dm, dk, dn, dact, launches=10, reps=10)
+        ops_small[f"tower_{name}_M{dm}_K{dk}_N{dn}"] = {"us": round(us, 2), "TFLOPs": round(2.0 * dm * dk * dn / us / 1e6, 1)}
 
     cpu, parity = None, None
     if not args.skip_cpu:

@@ -402,7 +402,12 @@ int w8a8_common(const void* a8, int lda, const float* sa, const void* w_packed, 
   a.act = act;
   a.vec = 1;
   a.vec16 = ldy % 8 == 0 && aligned16(y) && (!resid || (aligned16(resid) && ldr % (resid_dtype == TK_F32 ? 4 : 8) == 0));
-  const int blocks0 = ((a.ntiles * 32 + tk_w8a8_cols() - 1) / tk_w8a8_cols()) * ((M + tk_w8a8_rows() - 1) / tk_w8a8_rows());
+  // 64-row blocks, two per CU, once the 128-row grid would run in several generations anyway: co-resident blocks
+  // cover each other's first loads and epilogue (gate/up at 712 rows: 73 -> 59 us); few blocks keep the 128-row tile
+  const int blocks128 = ((a.ntiles * 32 + tk_w8a8_cols() - 1) / tk_w8a8_cols()) * ((M + 127) / 128);
+  a.mtiles = blocks128 >= 2 * device_cus() ? 2 : 4;
+  const int rows = a.mtiles * 32;
+  const int blocks0 = ((a.ntiles * 32 + tk_w8a8_cols() - 1) / tk_w8a8_cols()) * ((M + rows - 1) / rows);
   int ks = split_k;
   if (ks <= 0) {
     // fill the device once; a split keeps at least 32 k tiles and its partials must fit
@@ -410,7 +415,7 @@ int w8a8_common(const void* a8, int lda, const float* sa, const void* w_packed, 
     if (ks > a.KT / 32) ks = a.KT / 32;
     if (ks < 1) ks = 1;
   }
-  const size_t per_split = (size_t)tk_w8a8_rows() * tk_w8a8_cols() * 4;
+  const size_t per_split = (size_t)rows * tk_w8a8_cols() * 4;
   if (ks > 1) {
     const size_t have = ws && ws_bytes > kPartialOff ? (ws_bytes - kPartialOff < kPartialBytes ? ws_bytes - kPartialOff : kPartialBytes) / (per_split * blocks0) : 0;
     if ((size_t)ks > have || blocks0 > kMaxCounters) {

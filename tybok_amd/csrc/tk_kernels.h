@@ -53,6 +53,8 @@ struct GemmArgs {
   // bf16-weight many-row kernel only: bf16 [N] bias added to the accumulator, or nullptr; there act is
   // 0 none, 1 tanh-GELU of the bf16-rounded pre-activation, 2 tanh-GELU of the fp32 pre-activation
   const unsigned short* bias;
+  // many-row fp8 kernels: 32-row tiles per block (2 or 4), chosen by the host
+  int mtiles;
 };
 
 struct QuantActArgs {
@@ -203,8 +205,7 @@ int tk_wide_cols();
 int tk_launch_gemm_wide(GemmArgs a, hipStream_t st);
 int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st);
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st);
-// W8A8 tier: per-token activation quantisation and the fp8 x fp8 many-row GEMM (block tile tk_w8a8_rows() x tk_w8a8_cols())
-int tk_w8a8_rows();
+// W8A8 tier: per-token activation quantisation and the fp8 x fp8 many-row GEMM (block tile 32 * mtiles x tk_w8a8_cols())
 int tk_w8a8_cols();
 int tk_quant_act_max_k();
 int tk_launch_w8a8_gemm(GemmArgs a, hipStream_t st);

@@ -25,15 +25,16 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-constexpr int MT = 4;   // m tiles per block (and per wave)
 constexpr int NT = 2;   // n tiles per wave
 constexpr int NW = 4;   // waves per block
 constexpr int RK = 4;   // 32-wide k tiles per round (two 64-wide product steps)
 constexpr int PF = 3;   // rounds in flight
 
-// EPI: 0 plain (scales, optional residual), 1 gated (gate/up tile pairs -> act(g) * u).
-template <int EPI>
-__global__ __launch_bounds__(NW * 64) void w8a8_wide_kernel(GemmArgs a, int nblk_m, int ngroups) {
+// EPI: 0 plain (scales, optional residual), 1 gated (gate/up tile pairs -> act(g) * u).  MT: 32-row tiles per block
+// (and per wave): 4 with one block per CU, 2 with two -- co-resident blocks cover each other's first loads
+// and epilogue, which weigh as much as the k loop when K is a few thousand.
+template <int EPI, int MT, int OCC>
+__global__ __launch_bounds__(NW * 64, OCC) void w8a8_wide_kernel(GemmArgs a, int nblk_m, int ngroups) {
   constexpr int ROWS = MT * 32;
   constexpr int ROWB = RK * 32;            // bytes of one staged (fp8) activation row per round
   constexpr int PITCH = ROWB + 16;
@@ -42,7 +43,8 @@ __global__ __launch_bounds__(NW * 64) void w8a8_wide_kernel(GemmArgs a, int nblk
   constexpr int XPT = ROWS * PPR / (NW * 64);
   constexpr int TILES = MT * NT;
   constexpr int STEPS = RK / 2;            // 64-wide product steps per round
-  __shared__ __align__(16) unsigned char lds[2 * XBUF];
+  constexpr int EPB = NW * 32 * ((EPI == 0 ? NT * 32 : 32) * 2 + 16);  // the epilogue's per-wave tiles
+  __shared__ __align__(16) unsigned char lds[2 * XBUF > EPB ? 2 * XBUF : EPB];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -100,85 +102,89 @@ __global__ __launch_bounds__(NW * 64) void w8a8_wide_kernel(GemmArgs a, int nblk
   struct XFrag {
     i32x4 v[XPT];
   };
-  auto wload = [&](WFrag& f, int r) {
-#pragma unroll
-    for (int j = 0; j < RK; ++j) {
-      int kt = kt_lo + r * RK + j;
-      if (kt > a.KT - 1) kt = a.KT - 1;  // its activation columns are zeroed
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) f.w[j][nt] = *(const i32x4*)(wbase[nt] + (size_t)kt * 1024);
-    }
+  // One piece of each kind of work, so that a round can deal them out between its matrix instructions: a wave
+  // cannot issue anything while it waits for the matrix pipe to take its next instruction, so whatever stands
+  // between two groups of matrix instructions in program order runs with the pipe empty.
+  auto wload1 = [&](WFrag& f, int r, int st, int q) {  // q in [0, 2*NT): k tile 2*st + q/NT of round r, n tile q%NT
+    const int j = 2 * st + q / NT, nt = q % NT;
+    int kt = kt_lo + r * RK + j;
+    if (kt > a.KT - 1) kt = a.KT - 1;  // its activation columns are zeroed
+    f.w[j][nt] = *(const i32x4*)(wbase[nt] + (size_t)kt * 1024);
   };
-  auto xload = [&](XFrag& f, int r) {
-    const int k0 = (kt_lo + r * RK) * 32;
-#pragma unroll
-    for (int i = 0; i < XPT; ++i) {
-      int k = k0 + xcol[i];
-      if (k > a.K - 16) k = a.K - 16;
-      f.v[i] = *(const i32x4*)(xsrc[i] + k);
-    }
+  auto xload1 = [&](XFrag& f, int r, int i) {
+    int k = (kt_lo + r * RK) * 32 + xcol[i];
+    if (k > a.K - 16) k = a.K - 16;
+    f.v[i] = *(const i32x4*)(xsrc[i] + k);
   };
-  auto xstore = [&](const XFrag& f, int r, int b) {
-    const int k0 = (kt_lo + r * RK) * 32;
+  auto xstore1 = [&](const XFrag& f, int r, int b, int i) {
     const i32x4 z = {0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < XPT; ++i) *(i32x4*)(lds + b * XBUF + xdst[i]) = (k0 + xcol[i]) < k_end ? f.v[i] : z;
+    *(i32x4*)(lds + b * XBUF + xdst[i]) = ((kt_lo + r * RK) * 32 + xcol[i]) < k_end ? f.v[i] : z;
   };
-  // operands of a whole round (two 64-wide steps x four m tiles): requested together right after the round's
-  // barrier, so the matrix instructions that follow wait for the first pair only and the rest streams in behind
-  i32x8 xa[STEPS][MT];
-  auto xread = [&](int b) {
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const unsigned char* p = lds + b * XBUF + (mt * 32 + l32) * PITCH + s * 64 + 16 * half;
-        const i32x4 lo = *(const i32x4*)p, hi = *(const i32x4*)(p + 32);
-        xa[s][mt] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      }
+  // operand fragments of the round's two 64-wide steps, as the 16-byte halves they are read in
+  static_assert(STEPS == 2, "a round is two phases");
+  i32x4 xa[STEPS][MT][2];
+  auto xread1 = [&](int st, int b, int u) {  // u in [0, 2*MT): half u%2 of m tile u/2
+    xa[st][u / 2][u % 2] = *(const i32x4*)(lds + b * XBUF + ((u / 2) * 32 + l32) * PITCH + st * 64 + 16 * half + 32 * (u % 2));
   };
-  auto mma = [&](const WFrag& f) {
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      i32x8 wb[NT];
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        const i32x4 lo = f.w[2 * s][nt], hi = f.w[2 * s + 1][nt];
-        wb[nt] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      }
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wb[nt], xa[s][mt], acc[mt][nt], 0, 0, 0, 0, 0, 0);
-    }
+  auto mma1 = [&](const WFrag& f, int st, int t) {  // t in [0, MT*NT): m tile t/NT, n tile t%NT
+    const int mt = t / NT, nt = t % NT;
+    const i32x4 wl = f.w[2 * st][nt], wh = f.w[2 * st + 1][nt], xl = xa[st][mt][0], xh = xa[st][mt][1];
+    const i32x8 wb = {wl[0], wl[1], wl[2], wl[3], wh[0], wh[1], wh[2], wh[3]};
+    const i32x8 xb = {xl[0], xl[1], xl[2], xl[3], xh[0], xh[1], xh[2], xh[3]};
+    acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wb, xb, acc[mt][nt], 0, 0, 0, 0, 0, 0);
   };
 
   // PF rounds in flight, every load unconditional (clamped addresses; columns past the block's k range are
-  // zeroed when staged).  Round r: its operands are requested from LDS, then round r+1 is staged into the other
-  // buffer (every wave has passed barrier r, i.e. holds round r-1's operands in registers) and the next global
-  // loads go out -- all of it under the 16 matrix instructions of round r; one barrier per round.
+  // zeroed when staged).  Round r, phase A: multiplies step 0 while step 1's operands are fetched from LDS, round
+  // r+1 is staged into the other LDS buffer and the weight registers that round r-1's step 1 has left are
+  // refilled; then the round's only barrier (a wave can write buffer b for round r+2 only after every wave has
+  // passed the barrier of round r+1, i.e. has its round-r operands in registers); phase B: fetches round r+1's
+  // first operands, multiplies step 1 and refills step 0's weight registers.  A phase never reloads registers its
+  // own matrix instructions read.  Each of a phase's MT*NT matrix instructions is followed by its share of the
+  // other work, fenced so that the order stands.
+  constexpr int SLOTS = MT * NT;
+  static_assert(SLOTS == 2 * MT && SLOTS >= 2 * NT && 2 * XPT <= SLOTS, "one operand read per slot; the other pieces fit");
   WFrag wbuf[PF];
   XFrag xbuf[PF];
 #pragma unroll
   for (int p = 0; p < PF; ++p) {
-    xload(xbuf[p], p);
-    wload(wbuf[p], p);
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) xload1(xbuf[p], p, i);
+#pragma unroll
+    for (int q = 0; q < 2 * NT; ++q) {
+      wload1(wbuf[p], p, 0, q);
+      wload1(wbuf[p], p, 1, q);
+    }
   }
-  xstore(xbuf[0], 0, 0);
-  xload(xbuf[0], PF);
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) xstore1(xbuf[0], 0, 0, i);
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) xload1(xbuf[0], PF, i);
   lds_barrier();
+#pragma unroll
+  for (int u = 0; u < 2 * MT; ++u) xread1(0, 0, u);
   auto round = [&](int p, int r) {
-    const int pn = (p + 1) % PF;
-    xread(r & 1);
+    const int b = r & 1;
+    const int pn = (p + 1) % PF, pp = (p + PF - 1) % PF;
     __builtin_amdgcn_sched_barrier(0);
-    xstore(xbuf[pn], r + 1, (r + 1) & 1);
-    xload(xbuf[pn], r + 1 + PF);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(wbuf[p]);
-    wload(wbuf[p], r + PF);
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) {
+      mma1(wbuf[p], 0, i);
+      xread1(1, b, i);
+      if (i < XPT) xstore1(xbuf[pn], r + 1, b ^ 1, i);
+      if (i >= SLOTS - XPT) xload1(xbuf[pn], r + 1 + PF, i - (SLOTS - XPT));
+      if (i < 2 * NT) wload1(wbuf[pp], r - 1 + PF, 1, i);  // the registers round r-1 finished with in its phase B
+      __builtin_amdgcn_sched_barrier(0);
+    }
     lds_barrier();
     __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) {
+      mma1(wbuf[p], 1, i);
+      xread1(0, b ^ 1, i);
+      if (i < 2 * NT) wload1(wbuf[p], r + PF, 0, i);  // step 0's registers: free since phase A
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
   {
     int it = 0;
@@ -265,7 +271,7 @@ __global__ __launch_bounds__(NW * 64) void w8a8_wide_kernel(GemmArgs a, int nblk
     constexpr int EP = COLS * 2 + 16;                   // LDS row pitch (bytes)
     constexpr int LPR = COLS / 8;                       // lanes (16-byte chunks) per row
     constexpr int RPI = 64 / LPR;                       // rows per store instruction
-    static_assert(NW * 32 * EP <= 2 * XBUF, "the staging buffers hold every wave's tile");
+    static_assert(NW * 32 * EP == EPB, "the epilogue tiles fit the LDS array");
     lds_barrier();  // every wave has left the staged activations behind
     unsigned char* wl = lds + wave * 32 * EP;
     const int ncol0 = EPI == 0 ? strip * NT * 32 : strip * 32;  // first output column of this wave
@@ -466,19 +472,27 @@ __global__ __launch_bounds__(256) void quant_act_rows_kernel(QuantActArgs a) {
 
 }  // namespace
 
-int tk_w8a8_rows() { return MT * 32; }
 int tk_w8a8_cols() { return NW * NT * 32; }
 int tk_quant_act_max_k() { return kQuantMaxPieces * 256 * 8; }
 
+// a.mtiles: 32-row tiles per block, 2 or 4
 int tk_launch_w8a8_gemm(GemmArgs a, hipStream_t st) {
-  const int nblk_m = (a.M + MT * 32 - 1) / (MT * 32);
+  if (a.mtiles != 2 && a.mtiles != 4) return -1;
+  const int nblk_m = (a.M + a.mtiles * 32 - 1) / (a.mtiles * 32);
   const int nblk_n = (a.ntiles + NW * NT - 1) / (NW * NT);
   const int ngroups = nblk_n * a.ksplit;
-  const unsigned blocks = (unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m;
-  if (a.s1)
-    hipLaunchKernelGGL(w8a8_wide_kernel<1>, dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
-  else
-    hipLaunchKernelGGL(w8a8_wide_kernel<0>, dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
+  const dim3 grid((unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m), block(NW * 64);
+  if (a.s1) {
+    if (a.mtiles == 4)
+      hipLaunchKernelGGL((w8a8_wide_kernel<1, 4, 1>), grid, block, 0, st, a, nblk_m, ngroups);
+    else
+      hipLaunchKernelGGL((w8a8_wide_kernel<1, 2, 2>), grid, block, 0, st, a, nblk_m, ngroups);
+  } else {
+    if (a.mtiles == 4)
+      hipLaunchKernelGGL((w8a8_wide_kernel<0, 4, 1>), grid, block, 0, st, a, nblk_m, ngroups);
+    else
+      hipLaunchKernelGGL((w8a8_wide_kernel<0, 2, 2>), grid, block, 0, st, a, nblk_m, ngroups);
+  }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
