@@ -108,96 +108,96 @@ __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, in
   struct XFrag {
     i32x4 v[XPT];
   };
-  auto wload = [&](WFrag& f, int r, int j) {  // k tile j of round r
+  // One piece of each kind of work, so that a round can deal them out between its matrix instructions: a wave
+  // cannot issue anything while it waits for the matrix pipe to take its next instruction, so whatever stands
+  // between two groups of matrix instructions in program order runs with the pipe empty.
+  auto wload1 = [&](WFrag& f, int r, int j, int q) {  // q in [0, 2*NT): chunk q%2 of n tile q/2, k tile j of round r
     int kt = kt_lo + r * RK + j;
     if (kt > a.KT - 1) kt = a.KT - 1;  // its activation columns are zeroed
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const uint8_t* p = wbase[nt] + (size_t)kt * 2048;
-      f.w[j][nt][0] = *(const i32x4*)p;
-      f.w[j][nt][1] = *(const i32x4*)(p + 1024);
-    }
+    f.w[j][q / 2][q % 2] = *(const i32x4*)(wbase[q / 2] + (size_t)kt * 2048 + (q % 2) * 1024);
   };
-  auto xload = [&](XFrag& f, int r) {
-    const int k0 = (kt_lo + r * RK) * 32;
-#pragma unroll
-    for (int i = 0; i < XPT; ++i) {
-      int k = k0 + xcol[i];
-      if (k > a.K - 8) k = a.K - 8;
-      f.v[i] = *(const i32x4*)(xsrc[i] + (size_t)k * 2);
-    }
+  auto xload1 = [&](XFrag& f, int r, int i) {
+    int k = (kt_lo + r * RK) * 32 + xcol[i];
+    if (k > a.K - 8) k = a.K - 8;
+    f.v[i] = *(const i32x4*)(xsrc[i] + (size_t)k * 2);
   };
-  auto xstore = [&](const XFrag& f, int r, int b) {
-    const int k0 = (kt_lo + r * RK) * 32;
+  auto xstore1 = [&](const XFrag& f, int r, int b, int i) {
     const i32x4 z = {0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < XPT; ++i) *(i32x4*)(lds + b * XBUF + xdst[i]) = (k0 + xcol[i]) < k_end ? f.v[i] : z;
+    *(i32x4*)(lds + b * XBUF + xdst[i]) = ((kt_lo + r * RK) * 32 + xcol[i]) < k_end ? f.v[i] : z;
   };
-  // Operand fragments of two k tiles: while the MFMAs of one k tile run, the LDS reads of the next are issued.
+  // operand fragments of the round's two k tiles, as the 16-byte halves (k steps of 16) they are read in
   i32x4 xa[2][MT][2];
-  auto xread = [&](int set, int b, int j) {
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const i32x4* p = (const i32x4*)(lds + b * XBUF + (mt * 32 + l32) * PITCH + (j * 32 + 16 * half) * 2);
-      xa[set][mt][0] = p[0];
-      xa[set][mt][1] = p[1];
-    }
+  auto xread1 = [&](int set, int b, int j, int u) {  // u in [0, 2*MT): k step u%2 of m tile u/2, k tile j
+    xa[set][u / 2][u % 2] = *(const i32x4*)(lds + b * XBUF + ((u / 2) * 32 + l32) * PITCH + (j * 32 + 16 * half) * 2 + 16 * (u % 2));
   };
-  auto mma = [&](int set, const WFrag& f, int j) {
-#pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(f.w[j][nt][h2]), as_bf16x8(xa[set][mt][h2]), acc[mt][nt], 0, 0, 0);
-  };
-  // scheduling hint for a phase of 2*MT*NT MFMAs and 2*MT LDS reads: spread the reads between the MFMAs
-  // instead of waiting for each read right before its MFMA
-  auto interleave = [&]() {
-#pragma unroll
-    for (int i = 0; i < 2 * MT; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);  // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
-    }
+  auto mma1 = [&](int set, const WFrag& f, int j, int t) {  // t in [0, 2*MT*NT): k step, m tile, n tile
+    const int h2 = t / (MT * NT), mt = (t / NT) % MT, nt = t % NT;
+    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(f.w[j][nt][h2]), as_bf16x8(xa[set][mt][h2]), acc[mt][nt], 0, 0, 0);
   };
 
   // PF rounds in flight; every load is unconditional (clamped addresses; columns past the block's k range are
-  // zeroed when staged), so the loop bodies have no branch and the compiler keeps precise wait counts.  Round r:
-  // phase A multiplies k tile 0 while k tile 1's operands are fetched from LDS, then refills k tile 0's weight
-  // registers for round r+PF; phase B stages round r+1 into the other LDS buffer, passes the round's only
-  // barrier (a wave can write buffer b for round r+2 only after every wave has passed the barrier of round r+1,
-  // i.e. has its round-r operands in registers), fetches round r+1's first operands and multiplies k tile 1.
+  // zeroed when staged), so the loop bodies have no branch and the compiler keeps precise wait counts.  Round r,
+  // phase A: multiplies k tile 0 while k tile 1's operands are fetched from LDS, round r+1 is staged into the
+  // other LDS buffer and the weight registers that round r-1's k tile 1 has left are refilled; then the round's
+  // only barrier (a wave can write buffer b for round r+2 only after every wave has passed the barrier of round
+  // r+1, i.e. has its round-r operands in registers); phase B: fetches round r+1's first operands, multiplies k
+  // tile 1 and refills k tile 0's weight registers.  A phase never reloads registers its own matrix instructions
+  // read.  Each of a phase's 2*MT*NT matrix instructions is followed by its share of the other work (piece j of
+  // n goes to slot j * SLOTS / n), fenced so that the order stands.
+  constexpr int SLOTS = 2 * MT * NT;
+  constexpr int HS = SLOTS / 2;  // staging: stores in the first half of phase A's slots, loads in the second
   WFrag wbuf[PF];
   XFrag xbuf[PF];
 #pragma unroll
   for (int p = 0; p < PF; ++p) {
-    xload(xbuf[p], p);
-    wload(wbuf[p], p, 0);
-    wload(wbuf[p], p, 1);
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) xload1(xbuf[p], p, i);
+#pragma unroll
+    for (int q = 0; q < 2 * NT; ++q) {
+      wload1(wbuf[p], p, 0, q);
+      wload1(wbuf[p], p, 1, q);
+    }
   }
-  xstore(xbuf[0], 0, 0);
-  xload(xbuf[0], PF);
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) xstore1(xbuf[0], 0, 0, i);
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) xload1(xbuf[0], PF, i);
   lds_barrier();
-  xread(0, 0, 0);
+#pragma unroll
+  for (int u = 0; u < 2 * MT; ++u) xread1(0, 0, 0, u);
   auto round = [&](int p, int r) {
     const int b = p & 1;  // == r & 1: rounds advance PF at a time
-    const int pn = (p + 1) % PF;
+    const int pn = (p + 1) % PF, pp = (p + PF - 1) % PF;
     __builtin_amdgcn_sched_barrier(0);
-    xread(1, b, 1);
-    mma(0, wbuf[p], 0);
-    interleave();
-    __builtin_amdgcn_sched_barrier(0);
-    wload(wbuf[p], r + PF, 0);
-    xstore(xbuf[pn], r + 1, b ^ 1);
-    xload(xbuf[pn], r + 1 + PF);
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) {
+      mma1(0, wbuf[p], 0, i);
+#pragma unroll
+      for (int u = 0; u < 2 * MT; ++u)
+        if (u * SLOTS / (2 * MT) == i) xread1(1, b, 1, u);
+#pragma unroll
+      for (int x = 0; x < XPT; ++x) {
+        if (x * HS / XPT == i) xstore1(xbuf[pn], r + 1, b ^ 1, x);
+        if (HS + x * HS / XPT == i) xload1(xbuf[pn], r + 1 + PF, x);
+      }
+#pragma unroll
+      for (int q = 0; q < 2 * NT; ++q)
+        if (q * SLOTS / (2 * NT) == i) wload1(wbuf[pp], r - 1 + PF, 1, q);  // registers round r-1 finished with in its phase B
+      __builtin_amdgcn_sched_barrier(0);
+    }
     lds_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    xread(0, b ^ 1, 0);
-    mma(1, wbuf[p], 1);
-    interleave();
-    __builtin_amdgcn_sched_barrier(0);
-    wload(wbuf[p], r + PF, 1);
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) {
+      mma1(1, wbuf[p], 1, i);
+#pragma unroll
+      for (int u = 0; u < 2 * MT; ++u)
+        if (u * SLOTS / (2 * MT) == i) xread1(0, b ^ 1, 0, u);
+#pragma unroll
+      for (int q = 0; q < 2 * NT; ++q)
+        if (q * SLOTS / (2 * NT) == i) wload1(wbuf[p], r + PF, 0, q);  // k tile 0's registers: free since phase A
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
   {
     int it = 0;
@@ -348,7 +348,7 @@ int tk_launch_bf16w_wide(const GemmArgs& a, int tile, hipStream_t st) {
     case 31: return launch<3, 1, 2, 3>(a, st);
     case 22: return launch<2, 2, 2, 2>(a, st);
     case 21: return launch<2, 1, 2, 4>(a, st);
-    case 12: return launch<1, 2, 2, 4>(a, st);
+    case 12: return launch<1, 2, 2, 3>(a, st);
     case 11: return launch<1, 1, 2, 4>(a, st);
   }
   return -1;

@@ -441,7 +441,7 @@ struct DenseTile {
   int occ;  // blocks of this shape that fit one CU (registers)
 };
 constexpr DenseTile kDenseTiles[] = {{42, 128, 256, 1}, {41, 128, 128, 2}, {32, 96, 256, 2}, {31, 96, 128, 3},
-                                     {22, 64, 256, 2},  {21, 64, 128, 4},  {12, 32, 256, 4}, {11, 32, 128, 4}};
+                                     {22, 64, 256, 2},  {21, 64, 128, 4},  {12, 32, 256, 3}, {11, 32, 128, 4}};
 
 // Estimated duration (us) of a launch with this tile and K split; the constants are fitted to timings of the
 // vision towers' and the prefill's shapes.  Blocks that are resident together share a CU's matrix pipes and
