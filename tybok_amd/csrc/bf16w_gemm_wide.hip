@@ -226,7 +226,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, in
         st_agent64(dst + 1, c[4 * g + 2], c[4 * g + 3]);
       }
     __shared__ int s_last;
-    __builtin_amdgcn_s_waitcnt(0);
+    handoff_publish();
     __syncthreads();
     if (threadIdx.x == 0) {
       int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -234,6 +234,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, in
     }
     __syncthreads();
     if (!s_last) return;
+    handoff_acquire();
     if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)

@@ -376,7 +376,7 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
     }
   }
   __shared__ int s_last;
-  __builtin_amdgcn_s_waitcnt(0);  // partials acknowledged (written through) before the count
+  handoff_publish();  // partials acknowledged (written through) before the count
   __syncthreads();
   if (threadIdx.x == 0) {
     int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -384,6 +384,7 @@ __global__ __launch_bounds__(NWV * 64) void expert_attn_kernel(AttnArgs a) {
   }
   __syncthreads();
   if (!s_last || !owner) return;
+  handoff_acquire();
   if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
   constexpr int MAXS = D > 128 ? 7 : 8;  // the host never asks for more kv splits

@@ -299,7 +299,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
       st_agent64(dst + (size_t)g4 * 128 + 1, o[4 * g4 + 2], o[4 * g4 + 3]);
     }
   }
-  __builtin_amdgcn_s_waitcnt(0);  // partials acknowledged (written through) before the count
+  handoff_publish();  // partials acknowledged (written through) before the count
   __syncthreads();
   if (threadIdx.x == 0) {
     const int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -307,6 +307,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
   }
   __syncthreads();
   if (!s_last) return;
+  handoff_acquire();
   if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
   const float* pblk = a.partial + (size_t)blk_lin * a.kv_splits * PSTRIDE;

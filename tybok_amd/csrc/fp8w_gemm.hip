@@ -421,7 +421,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     }
     // wait until the partials are acknowledged, then count this block in
     __shared__ int s_last;
-    __builtin_amdgcn_s_waitcnt(0);
+    handoff_publish();
     __syncthreads();
     if (threadIdx.x == 0) {
       int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -429,6 +429,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     }
     __syncthreads();
     if (!s_last) return;
+    handoff_acquire();
     if (threadIdx.x == 0)  // leave the counter ready for the next launch
       __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll

@@ -105,6 +105,18 @@ __device__ __forceinline__ unsigned long long ld_agent64(const unsigned long lon
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Ordering of such a hand-off.  The writer's partials are write-through stores, visible to every block once
+// the wave's memory counters have drained; handoff_publish() drains them and pins the compiler on both sides
+// (no memory access may be moved across it), and the arrival count that follows it publishes the data.  On the
+// reader's side handoff_acquire() pins the compiler between seeing the count and reading the partials (the
+// reads themselves bypass the non-coherent caches).
+__device__ __forceinline__ void handoff_publish() {
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  __builtin_amdgcn_s_waitcnt(0);
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+}
+__device__ __forceinline__ void handoff_acquire() { __atomic_signal_fence(__ATOMIC_SEQ_CST); }
+
 // C layout of v_mfma_f32_32x32x16: lane l, register i holds
 //   column = l % 32, row = 8*(i/4) + 4*(l/32) + (i%4).
 __device__ __forceinline__ int mfma32_row(int lane, int i) { return 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3); }

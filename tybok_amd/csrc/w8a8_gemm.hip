@@ -214,7 +214,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void w8a8_wide_kernel(GemmArgs a, int
       }
     __shared__ int s_last;
     asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(0);  // the write-through stores are acknowledged: visible to every block
+    handoff_publish();  // the write-through stores are acknowledged: visible to every block
     asm volatile("" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -223,6 +223,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void w8a8_wide_kernel(GemmArgs a, int
     }
     __syncthreads();
     if (!s_last) return;
+    handoff_acquire();
     if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
