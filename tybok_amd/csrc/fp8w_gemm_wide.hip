@@ -25,15 +25,15 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-constexpr int MT = 4;   // m tiles per block (and per wave)
 constexpr int NT = 2;   // n tiles per wave
 constexpr int NW = 4;   // waves per block
 constexpr int RK = 2;   // k tiles per round
-constexpr int PF = 4;   // rounds in flight (even: round r uses LDS buffer r % 2)
 
 // EPI: 0 plain (scale, optional per-column gate, optional residual), 1 gated (gate/up tile pairs).
-template <int EPI>
-__global__ __launch_bounds__(NW * 64) void fp8w_wide_kernel(GemmArgs a, int nblk_m, int ngroups) {
+// MT: 32-row tiles per block (and per wave): 4 with one block per CU, 2 with two -- co-resident blocks cover each
+// other's first loads and epilogue.  PF: rounds in flight (even: round r uses LDS buffer r % 2).
+template <int EPI, int MT, int PF, int OCC>
+__global__ __launch_bounds__(NW * 64, OCC) void fp8w_wide_kernel(GemmArgs a, int nblk_m, int ngroups) {
   constexpr int ROWS = MT * 32;
   constexpr int ROWB = RK * 64;            // bytes of one staged activation row per round
   constexpr int PITCH = ROWB + 16;         // conflict-free 16-byte operand reads, 16-byte aligned
@@ -41,7 +41,8 @@ __global__ __launch_bounds__(NW * 64) void fp8w_wide_kernel(GemmArgs a, int nblk
   constexpr int PPR = ROWB / 16;           // 16-byte pieces per staged row
   constexpr int XPT = ROWS * PPR / (NW * 64);
   constexpr int TILES = MT * NT;
-  __shared__ __align__(16) unsigned char lds[2 * XBUF];
+  constexpr int EPB = NW * 32 * ((EPI == 0 ? NT * 32 : 32) * 2 + 16);  // the epilogue's per-wave tiles
+  __shared__ __align__(16) unsigned char lds[2 * XBUF > EPB ? 2 * XBUF : EPB];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -100,107 +101,113 @@ __global__ __launch_bounds__(NW * 64) void fp8w_wide_kernel(GemmArgs a, int nblk
   struct XFrag {
     i32x4 v[XPT];
   };
-  auto wload = [&](WFrag& f, int r) {
-#pragma unroll
-    for (int j = 0; j < RK; ++j) {
-      int kt = kt_lo + r * RK + j;
-      if (kt > a.KT - 1) kt = a.KT - 1;  // its activation columns are zeroed
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) f.w[j][nt] = *(const i32x4*)(wbase[nt] + (size_t)kt * 1024);
-    }
+  // One piece of each kind of work, so that a round can deal them out between its matrix instructions: a wave
+  // cannot issue anything while it waits for the matrix pipe to take its next instruction, so whatever stands
+  // between two groups of matrix instructions in program order runs with the pipe empty.
+  auto wload1 = [&](WFrag& f, int r, int j, int nt) {  // k tile j of round r, n tile nt: one 1 KiB tile
+    int kt = kt_lo + r * RK + j;
+    if (kt > a.KT - 1) kt = a.KT - 1;  // its activation columns are zeroed
+    f.w[j][nt] = *(const i32x4*)(wbase[nt] + (size_t)kt * 1024);
   };
-  auto xload = [&](XFrag& f, int r) {
-    const int k0 = (kt_lo + r * RK) * 32;
-#pragma unroll
-    for (int i = 0; i < XPT; ++i) {
-      int k = k0 + xcol[i];
-      if (k > a.K - 8) k = a.K - 8;
-      f.v[i] = *(const i32x4*)(xsrc[i] + (size_t)k * 2);
-    }
+  auto xload1 = [&](XFrag& f, int r, int i) {
+    int k = (kt_lo + r * RK) * 32 + xcol[i];
+    if (k > a.K - 8) k = a.K - 8;
+    f.v[i] = *(const i32x4*)(xsrc[i] + (size_t)k * 2);
   };
-  auto xstore = [&](const XFrag& f, int r, int b) {
-    const int k0 = (kt_lo + r * RK) * 32;
+  auto xstore1 = [&](const XFrag& f, int r, int b, int i) {
     const i32x4 z = {0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < XPT; ++i) *(i32x4*)(lds + b * XBUF + xdst[i]) = (k0 + xcol[i]) < k_end ? f.v[i] : z;
+    *(i32x4*)(lds + b * XBUF + xdst[i]) = ((kt_lo + r * RK) * 32 + xcol[i]) < k_end ? f.v[i] : z;
   };
-  // Operand fragments and converted weights of two k tiles: while the MFMAs of one k tile run,
-  // the LDS reads and the e4m3 -> bf16 conversions of the next one are issued between them.
+  // operand fragments and converted weights of two k tiles: while the MFMAs of one k tile run, the LDS reads and
+  // the e4m3 -> bf16 conversions of the next one are issued between them
   i32x4 xa[2][MT][2];
   bf16x8 wb[2][NT][2];
-  auto xread = [&](int set, int b, int j) {
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const i32x4* p = (const i32x4*)(lds + b * XBUF + (mt * 32 + l32) * PITCH + (j * 32 + 16 * half) * 2);
-      xa[set][mt][0] = p[0];
-      xa[set][mt][1] = p[1];
-    }
+  auto xread1 = [&](int set, int b, int j, int u) {  // u in [0, 2*MT): k step u%2 of m tile u/2, k tile j
+    xa[set][u / 2][u % 2] = *(const i32x4*)(lds + b * XBUF + ((u / 2) * 32 + l32) * PITCH + (j * 32 + 16 * half) * 2 + 16 * (u % 2));
   };
-  auto wcvt = [&](int set, const WFrag& f, int j) {
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      wb[set][nt][0] = fp8x8_to_bf16x8(f.w[j][nt][0], f.w[j][nt][1]);
-      wb[set][nt][1] = fp8x8_to_bf16x8(f.w[j][nt][2], f.w[j][nt][3]);
-    }
+  auto wcvt1 = [&](int set, const WFrag& f, int j, int q) {  // q in [0, 2*NT): k step q%2 of n tile q/2
+    wb[set][q / 2][q % 2] = fp8x8_to_bf16x8(f.w[j][q / 2][2 * (q % 2)], f.w[j][q / 2][2 * (q % 2) + 1]);
   };
-  auto mma = [&](int set) {
-#pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[set][nt][h2], as_bf16x8(xa[set][mt][h2]), acc[mt][nt], 0, 0, 0);
-  };
-  // scheduling hint for a phase of 16 MFMAs, 8 LDS reads and 16 conversions: spread the reads and
-  // the conversions between the MFMAs instead of waiting for each read right before its MFMA
-  auto interleave = [&]() {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS read
-      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // VALU
-    }
+  auto mma1 = [&](int set, int t) {  // t in [0, 2*MT*NT): k step, m tile, n tile
+    const int h2 = t / (MT * NT), mt = (t / NT) % MT, nt = t % NT;
+    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[set][nt][h2], as_bf16x8(xa[set][mt][h2]), acc[mt][nt], 0, 0, 0);
   };
   static_assert(RK == 2 && PF % 2 == 0, "a round is two phases; buffer parity follows the pipeline slot");
 
-  // PF rounds in flight; every load is unconditional (clamped addresses; columns past the block's k
-  // range are zeroed when staged), so the loop bodies have no branch and the compiler keeps precise
-  // wait counts.  Round r: phase A multiplies k tile 0 while k tile 1's operands are fetched from
-  // LDS; phase B stages round r+1 into the other LDS buffer, passes the round's only barrier (a wave
-  // can write buffer b for round r+2 only after every wave has passed the barrier of round r+1, i.e.
-  // has its round-r operands in registers), fetches round r+1's first operands and multiplies k tile 1.
+  // PF rounds in flight; every load is unconditional (clamped addresses; columns past the block's k range are
+  // zeroed when staged), so the loop bodies have no branch and the compiler keeps precise wait counts.  Round r,
+  // phase A: multiplies k tile 0 while k tile 1's operands are fetched from LDS and its weights converted (their
+  // registers are refilled for round r+PF right after), and round r+1 is staged into the other LDS buffer; then
+  // the round's only barrier (a wave can write buffer b for round r+2 only after every wave has passed the barrier
+  // of round r+1, i.e. has its round-r operands in registers); phase B: fetches round r+1's first operands,
+  // converts its first weights (and refills their registers) and multiplies k tile 1.  Each of a phase's
+  // 2*MT*NT matrix instructions is followed by its share of the other work, fenced so that the order stands:
+  // reads and conversions in the first half of the slots, the loads that refill converted registers in the second.
+  constexpr int SLOTS = 2 * MT * NT;
+  constexpr int HS = SLOTS / 2;
+  static_assert(2 * MT <= SLOTS && 2 * NT <= HS && NT <= HS && XPT <= HS, "the pieces fit the slots");
   WFrag wbuf[PF];
   XFrag xbuf[PF];
 #pragma unroll
   for (int p = 0; p < PF; ++p) {
-    xload(xbuf[p], p);
-    wload(wbuf[p], p);
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) xload1(xbuf[p], p, i);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      wload1(wbuf[p], p, 0, nt);
+      wload1(wbuf[p], p, 1, nt);
+    }
   }
-  xstore(xbuf[0], 0, 0);
-  xload(xbuf[0], PF);
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) xstore1(xbuf[0], 0, 0, i);
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) xload1(xbuf[0], PF, i);
   lds_barrier();
-  xread(0, 0, 0);
-  wcvt(0, wbuf[0], 0);
+#pragma unroll
+  for (int u = 0; u < 2 * MT; ++u) xread1(0, 0, 0, u);
+#pragma unroll
+  for (int q = 0; q < 2 * NT; ++q) wcvt1(0, wbuf[0], 0, q);
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) wload1(wbuf[0], PF, 0, nt);
   auto round = [&](int p, int r) {
     const int b = p & 1;  // == r & 1: rounds advance PF at a time
     const int pn = (p + 1) % PF;
     __builtin_amdgcn_sched_barrier(0);
-    xread(1, b, 1);
-    wcvt(1, wbuf[p], 1);
-    mma(0);
-    interleave();
-    __builtin_amdgcn_sched_barrier(0);
-    wload(wbuf[p], r + PF);
-    xstore(xbuf[pn], r + 1, b ^ 1);
-    xload(xbuf[pn], r + 1 + PF);
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) {
+      mma1(0, i);
+#pragma unroll
+      for (int u = 0; u < 2 * MT; ++u)
+        if (u * SLOTS / (2 * MT) == i) xread1(1, b, 1, u);
+#pragma unroll
+      for (int q = 0; q < 2 * NT; ++q)
+        if (q * HS / (2 * NT) == i) wcvt1(1, wbuf[p], 1, q);
+#pragma unroll
+      for (int x = 0; x < XPT; ++x) {
+        if (x * HS / XPT == i) xstore1(xbuf[pn], r + 1, b ^ 1, x);
+        if (HS + x * HS / XPT == i) xload1(xbuf[pn], r + 1 + PF, x);
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        if (HS + nt * HS / NT == i) wload1(wbuf[p], r + PF, 1, nt);  // converted above
+      __builtin_amdgcn_sched_barrier(0);
+    }
     lds_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    xread(0, b ^ 1, 0);
-    wcvt(0, wbuf[pn], 0);
-    mma(1);
-    interleave();
-    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) {
+      mma1(1, i);
+#pragma unroll
+      for (int u = 0; u < 2 * MT; ++u)
+        if (u * SLOTS / (2 * MT) == i) xread1(0, b ^ 1, 0, u);
+#pragma unroll
+      for (int q = 0; q < 2 * NT; ++q)
+        if (q * HS / (2 * NT) == i) wcvt1(0, wbuf[pn], 0, q);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        if (HS + nt * HS / NT == i) wload1(wbuf[pn], r + 1 + PF, 0, nt);  // converted above
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
   {
     int it = 0;
@@ -280,7 +287,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_wide_kernel(GemmArgs a, int nblk
     constexpr int EP = COLS * 2 + 16;              // LDS row pitch (bytes)
     constexpr int LPR = COLS / 8;                  // lanes (16-byte chunks) per row
     constexpr int RPI = 64 / LPR;                  // rows per store instruction
-    static_assert(NW * 32 * EP <= 2 * XBUF, "the staging buffers hold every wave's tile");
+    static_assert(NW * 32 * EP == EPB, "the epilogue tiles fit the LDS array");
     lds_barrier();  // every wave has left the staged activations behind
     unsigned char* wl = lds + wave * 32 * EP;
     const int ncol0 = EPI == 0 ? strip * NT * 32 : strip * 32;  // first output column of this wave
@@ -470,18 +477,26 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(NormRowsArgs a) {
 
 }  // namespace
 
-int tk_wide_rows() { return MT * 32; }
 int tk_wide_cols() { return NW * NT * 32; }
 
+// a.mtiles: 32-row tiles per block, 2 or 4
 int tk_launch_gemm_wide(GemmArgs a, hipStream_t st) {
-  const int nblk_m = (a.M + MT * 32 - 1) / (MT * 32);
+  if (a.mtiles != 2 && a.mtiles != 4) return -1;
+  const int nblk_m = (a.M + a.mtiles * 32 - 1) / (a.mtiles * 32);
   const int nblk_n = (a.ntiles + NW * NT - 1) / (NW * NT);
   const int ngroups = nblk_n * a.ksplit;
-  const unsigned blocks = (unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m;
-  if (a.s1)
-    hipLaunchKernelGGL(fp8w_wide_kernel<1>, dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
-  else
-    hipLaunchKernelGGL(fp8w_wide_kernel<0>, dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
+  const dim3 grid((unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m), block(NW * 64);
+  if (a.s1) {
+    if (a.mtiles == 4)
+      hipLaunchKernelGGL((fp8w_wide_kernel<1, 4, 4, 1>), grid, block, 0, st, a, nblk_m, ngroups);
+    else
+      hipLaunchKernelGGL((fp8w_wide_kernel<1, 2, 4, 2>), grid, block, 0, st, a, nblk_m, ngroups);
+  } else {
+    if (a.mtiles == 4)
+      hipLaunchKernelGGL((fp8w_wide_kernel<0, 4, 4, 1>), grid, block, 0, st, a, nblk_m, ngroups);
+    else
+      hipLaunchKernelGGL((fp8w_wide_kernel<0, 2, 4, 2>), grid, block, 0, st, a, nblk_m, ngroups);
+  }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -169,7 +169,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   const bool has_norm = e.norm_w || e.ada_scale;
   // (from 256 rows on, or when its 128 x 256 tiles already fill the device; below that the skinny
   // kernel's finer blocks and K splits win)
-  const int wide_blocks = ((a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols()) * ((M + tk_wide_rows() - 1) / tk_wide_rows());
+  const int wide_blocks = ((a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols()) * ((M + 127) / 128);
   if (!e.w16 && !rope && !e.x_f32 && a.vec && (M >= 256 || (M > 64 && wide_blocks >= cus)) &&
       (!has_norm || (ws && ws_bytes >= kNormOff + (size_t)M * K * 2 && (size_t)M * K * 2 <= kNormBytes))) {
     // many rows: MFMA-bound kernel with a 128 x 256 block tile
@@ -191,7 +191,10 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
       a.norm_w = nullptr;
       a.ada_scale = a.ada_shift = nullptr;
     }
-    const int blocks0 = wide_blocks;
+    // 64-row blocks, two per CU, once the 128-row grid would run in several generations anyway: co-resident
+    // blocks cover each other's first loads and epilogue; few blocks keep the 128-row tile
+    a.mtiles = wide_blocks >= 2 * cus ? 2 : 4;
+    const int blocks0 = a.mtiles == 4 ? wide_blocks : ((a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols()) * ((M + 63) / 64);
     int ks = split_k;
     if (ks <= 0) {
       // fill the device once; a split keeps at least 16 k tiles and its partials must fit
@@ -199,7 +202,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
       if (ks > a.KT / 16) ks = a.KT / 16;
       if (ks < 1) ks = 1;
     }
-    const size_t per_split = (size_t)tk_wide_rows() * tk_wide_cols() * 4;
+    const size_t per_split = (size_t)a.mtiles * 32 * tk_wide_cols() * 4;
     if (ks > 1 && ws) {
       const size_t fit = kPartialBytes / (per_split * blocks0);
       const size_t have = ws_bytes > kPartialOff ? (ws_bytes - kPartialOff) / (per_split * blocks0) : 0;

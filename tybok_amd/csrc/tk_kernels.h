@@ -200,8 +200,7 @@ int tk_launch_tail(TailArgs a, hipStream_t st);
 int tk_launch_kv_proj(KvProjArgs a, hipStream_t st);
 int tk_layer_norm_max_k();
 int tk_launch_layer_norm(LayerNormArgs a, hipStream_t st);
-int tk_wide_rows();  // block tile of the many-row GEMM
-int tk_wide_cols();
+int tk_wide_cols();  // columns of the many-row GEMM's block tile (rows: 32 * GemmArgs::mtiles)
 int tk_launch_gemm_wide(GemmArgs a, hipStream_t st);
 int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st);
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st);
