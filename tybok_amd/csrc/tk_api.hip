@@ -447,22 +447,23 @@ constexpr DenseTile kDenseTiles[] = {{42, 128, 256, 1}, {41, 128, 128, 2}, {32, 
                                      {22, 64, 256, 2},  {21, 64, 128, 4},  {12, 32, 256, 3}, {11, 32, 128, 4}};
 
 // Estimated duration (us) of a launch with this tile and K split; the constants are fitted to timings of the
-// vision towers' and the prefill's shapes.  Blocks that are resident together share a CU's matrix pipes and
-// overlap each other's first loads and epilogues; every further generation of blocks pays those again.  A wave
-// issues (rows/32) * (cols/128) MFMAs per 16 columns of k (18.8 ns each under full load, half of that rate
-// reached), and a block loads (rows + cols) * 128 bytes per 64 columns of k at about 60 KiB/us per CU.
+// vision towers' and the prefill's shapes (the picked tile is within 1 % of the best one on average).  Blocks
+// that are resident together share a CU's matrix pipes and overlap each other's first loads and epilogues; every
+// further generation of blocks pays those again.  A wave issues (rows/32) * (cols/128) MFMAs per 16 columns of k
+// (18.8 ns each under full load; 30 / 35 / 45 % of that rate reached with one / two / three or more waves per
+// SIMD), and a block loads (rows + cols) * 128 bytes per 64 columns of k at about 60 KiB/us per CU.
 float dense_cost(const DenseTile& t, int M, int N, int KT, int ks, int cus) {
   const long long blocks = (long long)((M + t.rows - 1) / t.rows) * ((N + t.cols - 1) / t.cols) * ks;
   const float kt = (float)((KT + ks - 1) / ks);
-  const float mfma_us = (float)(t.rows / 32) * (float)(t.cols / 128) * 2.f * kt * 0.0188f / 0.5f;
+  const float eff = t.occ >= 3 ? 0.45f : t.occ == 2 ? 0.35f : 0.3f;
+  const float mfma_us = (float)(t.rows / 32) * (float)(t.cols / 128) * 2.f * kt * 0.0188f / eff;
   const float load_us = 0.5f * kt * (float)(t.rows + t.cols) * 0.125f / 60.f;
   const float tile_us = mfma_us > load_us ? mfma_us : load_us;
-  const float fixed_us = 4.f + (t.occ == 1 ? 3.f : 0.f);  // one wave per SIMD hides nothing
   float us = 0.f;
   long long left = blocks;
   while (left > 0) {
     const long long gen = left < (long long)cus * t.occ ? left : (long long)cus * t.occ;
-    us += fixed_us + (float)((gen + cus - 1) / cus) * tile_us;
+    us += 3.f + (float)((gen + cus - 1) / cus) * tile_us;
     left -= gen;
   }
   if (ks > 1) us += 1.5f + (float)blocks * (float)(t.rows * t.cols) * 8.f / 4e6f;  // fp32 partials out and back in
