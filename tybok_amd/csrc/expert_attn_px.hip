@@ -282,7 +282,38 @@ __global__ __launch_bounds__(kCrossWaves * 64) void expert_cross_px_kernel(AttnA
   const bool active = wave < nt;
   unsigned char* const ks = lds + (size_t)wave * 2 * kKTile;           // this wave's K tile: hi plane, then lo
 
-  // ---- K / V^T requests (whole rows, lane -> consecutive chunks), then the projection's weights ----
+  // ---- requests in the order of use (memory returns in order): the block's 32 hidden rows and the norm weight
+  // (16 threads per row, a thread's pieces requested together and kept in registers), the projection's weights,
+  // then K / V^T (whole rows, lane -> consecutive chunks) ----
+  constexpr int TPR = NWV * 2, XP = kCrossMaxK / 8 / TPR;  // threads per row, 16-byte pieces per thread
+  const int xr = tid / TPR, xq = tid % TPR;
+  const int xm = mtile * 32 + xr;
+  const u16* xrow = a.qp_x + (size_t)(xm < a.M ? xm : a.M - 1) * a.qp_ldx;
+  const int npieces = a.qp_K / 8;
+  i32x4 xpc[XP], nwp[XP];
+#pragma unroll
+  for (int i = 0; i < XP; ++i) {
+    const int p = xq + TPR * i;
+    const int pc = p < npieces ? p : npieces - 1;  // past the row: a valid piece, not used
+    xpc[i] = *(const i32x4*)(xrow + 8 * pc);
+    nwp[i] = *(const i32x4*)(a.qp_norm_w + 8 * pc);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // this wave's weight tiles of the head's strip (packed n tiles 2h, 2h+1): k tiles wave, wave + 8, wave + 16
+  constexpr int KPW = (kCrossMaxK / 32 + NWV - 1) / NWV;
+  i32x4 wfr[KPW][2][2];
+  {
+    const uint8_t* wq = a.qp_w + ((size_t)(2 * h) * a.qp_KT) * 2048 + lane * 16;
+#pragma unroll
+    for (int i = 0; i < KPW; ++i) {
+      int kt = wave + NWV * i;
+      if (kt > a.qp_KT - 1) kt = a.qp_KT - 1;
+#pragma unroll
+      for (int n2 = 0; n2 < 2; ++n2)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) wfr[i][n2][c] = *(const i32x4*)(wq + ((size_t)n2 * a.qp_KT + kt) * 2048 + c * 1024);
+    }
+  }
   const int tt = active ? wave : nt - 1;  // idle waves read a valid tile and drop it
   i32x4 kreg[2][4], vreg[2][4];
   {
@@ -309,59 +340,46 @@ __global__ __launch_bounds__(kCrossWaves * 64) void expert_cross_px_kernel(AttnA
     vreg[0][i] = *(const i32x4*)(a.vt_pre + off);
     vreg[1][i] = *(const i32x4*)(a.vt_pre_lo + off);
   }
-  // this wave's weight tiles of the head's strip (packed n tiles 2h, 2h+1): k tiles wave, wave + 8, wave + 16
-  constexpr int KPW = (kCrossMaxK / 32 + NWV - 1) / NWV;
-  i32x4 wfr[KPW][2][2];
-  {
-    const uint8_t* wq = a.qp_w + ((size_t)(2 * h) * a.qp_KT) * 2048 + lane * 16;
-#pragma unroll
-    for (int i = 0; i < KPW; ++i) {
-      int kt = wave + NWV * i;
-      if (kt > a.qp_KT - 1) kt = a.qp_KT - 1;
-#pragma unroll
-      for (int n2 = 0; n2 < 2; ++n2)
-#pragma unroll
-        for (int c = 0; c < 2; ++c) wfr[i][n2][c] = *(const i32x4*)(wq + ((size_t)n2 * a.qp_KT + kt) * 2048 + c * 1024);
-    }
-  }
   __builtin_amdgcn_sched_barrier(0);
 
-  // ---- the query tile: 1 / rms of the block's 32 hidden rows (16 threads per row), normalised rows
-  // into LDS as bf16(w * bf16(x * rstd)), columns from K to the end of the last k tile zero ----
+  // ---- the query tile: 1 / rms of its rows, normalised rows into LDS as bf16(w * bf16(x * rstd)), columns from K
+  // to the end of the last k tile zero ----
   {
-    constexpr int TPR = NWV * 2;
-    const int xr = tid / TPR, xq = tid % TPR;
-    const int xm = mtile * 32 + xr;
-    const u16* xrow = a.qp_x + (size_t)(xm < a.M ? xm : a.M - 1) * a.qp_ldx;
-    const int npieces = a.qp_K / 8;
     float ss0 = 0.f, ss1 = 0.f;
-    for (int p = xq; p < npieces; p += TPR) {
-      union { i32x4 v; bf16x2 hh[4]; } xu;
-      xu.v = *(const i32x4*)(xrow + 8 * p);
-      ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[0], xu.hh[0], ss0, false);
-      ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[1], xu.hh[1], ss1, false);
-      ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[2], xu.hh[2], ss0, false);
-      ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[3], xu.hh[3], ss1, false);
+#pragma unroll
+    for (int i = 0; i < XP; ++i) {
+      if (xq + TPR * i < npieces) {
+        union { i32x4 v; bf16x2 hh[4]; } xu;
+        xu.v = xpc[i];
+        ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[0], xu.hh[0], ss0, false);
+        ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[1], xu.hh[1], ss1, false);
+        ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[2], xu.hh[2], ss0, false);
+        ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.hh[3], xu.hh[3], ss1, false);
+      }
     }
     float ss = ss0 + ss1;
 #pragma unroll
     for (int o2 = TPR / 2; o2 > 0; o2 >>= 1) ss += __shfl_xor(ss, o2);
     const float rstd = rsqrtf(ss / (float)a.qp_K + a.qp_eps);
     const int kpieces = a.qp_KT * 4;
-    for (int p = xq; p < kpieces; p += TPR) {
-      union { i32x4 v; unsigned u[4]; } xu, nw, o4;
-      o4.v = i32x4{0, 0, 0, 0};
-      if (p < npieces) {
-        xu.v = *(const i32x4*)(xrow + 8 * p);
-        nw.v = *(const i32x4*)(a.qp_norm_w + 8 * p);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const unsigned u = pack_bf16x2(__uint_as_float(xu.u[e] << 16) * rstd, __uint_as_float(xu.u[e] & 0xffff0000u) * rstd);
-          o4.u[e] = pack_bf16x2(__uint_as_float(nw.u[e] << 16) * __uint_as_float(u << 16),
-                                __uint_as_float(nw.u[e] & 0xffff0000u) * __uint_as_float(u & 0xffff0000u));
+    for (int i = 0; i < XP; ++i) {
+      const int p = xq + TPR * i;
+      if (p < kpieces) {
+        union { i32x4 v; unsigned u[4]; } xu, nw, o4;
+        o4.v = i32x4{0, 0, 0, 0};
+        if (p < npieces) {
+          xu.v = xpc[i];
+          nw.v = nwp[i];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const unsigned u = pack_bf16x2(__uint_as_float(xu.u[e] << 16) * rstd, __uint_as_float(xu.u[e] & 0xffff0000u) * rstd);
+            o4.u[e] = pack_bf16x2(__uint_as_float(nw.u[e] << 16) * __uint_as_float(u << 16),
+                                  __uint_as_float(nw.u[e] & 0xffff0000u) * __uint_as_float(u & 0xffff0000u));
+          }
         }
+        *(i32x4*)(xs + xr * kXPitch + p * 16) = o4.v;
       }
-      *(i32x4*)(xs + xr * kXPitch + p * 16) = o4.v;
     }
   }
   lds_only_barrier();
