@@ -43,6 +43,10 @@ __device__ __forceinline__ void lds_barrier() {
 template <int MT, int NT, int NW, int EPI, int PF, int TPW, bool W16, int PRO, int NR = 0>
 __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   constexpr bool GATED = EPI == 1;
+  // every round of the block in flight from the start (PF == NR) with the bf16 RMSNorm prologue: the staged pieces
+  // stay in registers until the row statistics are known, so the statistics come from them -- no second pass over
+  // the rows.  The host picks this only when a block walks the whole K (no K split).
+  constexpr bool FULL = PRO == 1 && NR > 0 && PF == NR;
   constexpr bool PAIRED = EPI != 0;  // both n tiles of a pair are finished by the same wave
   constexpr bool XF32 = PRO == 2;
   constexpr int TILES = MT * NT;
@@ -265,12 +269,42 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   // valid tiles: a branch here would make the compiler's wait-count analysis assume, at the head
   // of the steady-state loop, that the first stage's loads might be the youngest in flight, and
   // drain the whole queue once per pass)
+  if (FULL) {
+    // the activations first: memory returns in order, and the statistics below need every piece of the rows
 #pragma unroll
-  for (int p = 0; p < PF; ++p) {
-    xload(xbuf[p], p);
-    wload(wbuf[p], p);
+    for (int p = 0; p < PF; ++p) xload(xbuf[p], p);
+#pragma unroll
+    for (int p = 0; p < PF; ++p) wload(wbuf[p], p);
+  } else {
+#pragma unroll
+    for (int p = 0; p < PF; ++p) {
+      xload(xbuf[p], p);
+      wload(wbuf[p], p);
+    }
   }
-  if (PRO) {
+  if (FULL) {
+    // piece i of every round belongs to row xrow[i]; the PPR threads that share a row are consecutive lanes
+    static_assert(!FULL || (PPR == 16 && !XF32), "the row's pieces sit in 16 consecutive lanes");
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) {
+      float ss0 = 0.f, ss1 = 0.f;
+#pragma unroll
+      for (int p = 0; p < PF; ++p) {
+        if (p * RKT * 32 + xcol[i] < a.K) {  // pieces past K hold a repeated piece of the row
+          union { i32x4 v; bf16x2 h[4]; } xu;
+          xu.v = xbuf[p].v[i][0];
+          ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[0], xu.h[0], ss0, false);
+          ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[1], xu.h[1], ss1, false);
+          ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[2], xu.h[2], ss0, false);
+          ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[3], xu.h[3], ss1, false);
+        }
+      }
+      float ss = ss0 + ss1;
+#pragma unroll
+      for (int o = PPR / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+      my_rstd[i] = rsqrtf(ss / (float)a.K + a.norm_eps);
+    }
+  } else if (PRO) {
     // per-row 1/rms over the whole K (every block needs it for its rows, whatever its k range)
     constexpr int TPR = NW * 64 / ROWS;  // threads per row
     const int r = tid / TPR, q = tid % TPR;
@@ -634,7 +668,14 @@ constexpr int kPF = 4;
 constexpr int kTPW = 1;
 template <int MT, int NT, int EPI, bool W16, int PRO, int NR>
 int launch_nr(const GemmArgs& a, dim3 grid, hipStream_t st) {
-  hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, kPF, kTPW, W16, PRO, NR>), grid, dim3(256), 0, st, a);
+  // the RMSNorm prologue over a short K that one block walks alone: all of its rounds in flight, the row
+  // statistics taken from the staged pieces (SmolVLA's expert: K = 720 -> 6 rounds, VLM: 960 -> 8)
+  constexpr bool CAN_FULL = PRO == 1 && MT == 1 && (NR == 6 || NR == 8);
+  if (CAN_FULL && a.ksplit == 1) {
+    hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, CAN_FULL ? NR : kPF, kTPW, W16, PRO, NR>), grid, dim3(256), 0, st, a);
+  } else {
+    hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, kPF, kTPW, W16, PRO, NR>), grid, dim3(256), 0, st, a);
+  }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 template <int MT, int NT, int EPI, bool W16, int PRO>
