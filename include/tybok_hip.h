@@ -390,6 +390,20 @@ int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_s
                    const void* w, const void* bias, void* v_out, const void* x_t, void* x_out, float dt, int M, int N,
                    int K, void* stream);
 
+/* tk_expert_tail plus the next denoising step's suffix embedding from the updated x, in the same launch:
+ *   emb_out[m, j] = act( sum_n x_out[m, n] * emb_w[j, n] + emb_b[j] ),  j < emb_n, fp32 arithmetic
+ * -- the first linear of `embed_suffix` applied to the action chunk: SmolVLA's `action_in_proj` folded with the
+ * action half of `action_time_mlp_in` (the time half, constant per step, folded into emb_b) and its SiLU
+ * (tybok/policies/smolvla/models/flow_matching.py:259-311); pi0.5's `action_in_proj` with the cast to bf16
+ * (tybok/policies/pi05/models/flow_matching.py:464-502).
+ *   x_t / x_out required; N must be 32 (the padded action width).
+ *   emb_w: fp32 [emb_n, N], 16-byte aligned; emb_b: fp32 [emb_n] or NULL; emb_act: 0 none, 1 SiLU;
+ *   emb_out: [M, emb_n] with row pitch emb_ld (elements), emb_dtype TK_F32 or TK_BF16 (rounded once). */
+int tk_expert_tail_embed(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps,
+                         const void* w, const void* bias, void* v_out, const void* x_t, void* x_out, float dt, int M, int N,
+                         int K, const void* emb_w, const void* emb_b, int emb_n, int emb_act, void* emb_out, int emb_ld,
+                         int emb_dtype, void* stream);
+
 /* ---- diagnostics ------------------------------------------------------------------------------- */
 /* out_f32[256] = value of every e4m3fn code as decoded by the device's conversion instruction
  * (the weight path of the GEMM); used to assert the OCP (not FNUZ) flavour on the box. */

@@ -76,6 +76,10 @@ def _cases():
     tail = lambda **kw: _args(  # noqa: E731
         dict(x=P, ldx=720, nw=P, asc=None, ash=None, eps=1e-6, w=P, b=None, v=P, xt=None, xo=None, dt=0.0, M=50, N=32, K=720, st=None), kw
     )
+    tail_e = lambda **kw: _args(  # noqa: E731
+        dict(x=P, ldx=720, nw=P, asc=None, ash=None, eps=1e-6, w=P, b=None, v=None, xt=P, xo=P, dt=-0.1, M=50, N=32, K=720,
+             ew=P, eb=None, en=720, eact=1, eo=P, eld=720, edt=1, st=None), kw
+    )  # fmt: skip
     ln = lambda **kw: _args(dict(x=P, ldx=768, xdt=0, w=P, b=P, wdt=0, eps=1e-6, y=P, ldy=768, M=64, K=768, st=None), kw)  # noqa: E731
     tv = lambda **kw: _args(dict(v=P, sb=1 << 20, sl=2304, sh=64, vt=P, tsb=1 << 20, tsh=65536, tsd=1024, keys=1024, B=3, Pk=1024, G=12, D=64, st=None), kw)  # noqa: E731
     qa = lambda **kw: _args(dict(x=P, ldx=2048, a8=P, lda=2048, sa=P, M=712, K=2048, mode=0, st=None), kw)  # noqa: E731
@@ -136,6 +140,13 @@ def _cases():
         ("tk_expert_tail", tail(K=8200, ldx=8200), -1, "at most 8192"),
         ("tk_expert_tail", tail(asc=P, ash=P), -1, "exactly one"),
         ("tk_expert_tail", tail(v=None), -1, "no output"),
+        ("tk_expert_tail_embed", tail_e(eo=None), -1, "emb_out is null"),
+        ("tk_expert_tail_embed", tail_e(xo=None, v=P), -1, "computed from x_out"),
+        ("tk_expert_tail_embed", tail_e(N=16), -1, "takes N=32 inputs"),
+        ("tk_expert_tail_embed", tail_e(ew=P + 4), -1, "16-byte aligned"),
+        ("tk_expert_tail_embed", tail_e(eld=700), -1, "bad embedding shape"),
+        ("tk_expert_tail_embed", tail_e(eact=2), -1, "emb_act=2"),
+        ("tk_expert_tail_embed", tail_e(edt=3), -1, "emb_dtype=3"),
         ("tk_layer_norm", ln(K=4096, ldx=4096, ldy=4096), -1, "at most"),
         ("tk_layer_norm", ln(wdt=1), -1, "both"),
         ("tk_layer_norm", ln(ldy=760), -1, "row pitch"),

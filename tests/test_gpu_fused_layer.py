@@ -240,6 +240,50 @@ def test_step_tail_norm_projection_euler(tk, adaptive):
     assert none is None and torch.equal(v_only, v)
 
 
+@pytest.mark.parametrize("model,m,k,j", [("smolvla", 50, 720, 720), ("pi05", 50, 1024, 1024), ("smolvla", 7, 96, 1100), ("pi05", 33, 2048, 40)])
+def test_step_tail_with_the_next_steps_embedding(tk, model, m, k, j):
+    # the tail launch also writes the first linear of the next step's suffix embedding from the updated x
+    # (flow_matching.py:259-311 with the SiLU, fp32 out; pi05 flow_matching.py:464-502, cast to bf16): against the
+    # torch expression on the tail's own x_new, and the tail's other outputs unchanged bit for bit
+    n = 32
+    g = torch.Generator().manual_seed(23)
+    x = (torch.randn(m, k, generator=g) * 2.0).to(BF16).cuda()
+    w = (torch.randn(n, k, generator=g) * k**-0.5).cuda()
+    b = torch.randn(n, generator=g).cuda()
+    x_t = torch.randn(m, n, generator=g).cuda()
+    ew = (torch.randn(j, n, generator=g) * n**-0.5).cuda()
+    eb = torch.randn(j, generator=g).cuda()
+    if model == "pi05":
+        mod = 0.3 * torch.randn(1, 3 * k, generator=g)
+        kw = dict(ada=(mod[0, :k].contiguous().cuda(), mod[0, k : 2 * k].contiguous().cuda()), eps=1e-6)
+        wide = torch.full((m, j + 8), 7.0, dtype=BF16, device="cuda")  # a row pitch wider than the rows
+        out = wide[:, :j]
+        act = "none"
+    else:
+        kw = dict(norm_w=(1.0 + 0.2 * torch.randn(k, generator=g)).to(BF16).cuda(), eps=1e-5)
+        out = torch.empty(m, j, dtype=torch.float32, device="cuda")
+        act = "silu"
+    v0, x0 = tk.expert_tail(x, w, b, x_t=x_t, dt=-0.1, want_v=True, **kw)
+    v1, x1 = tk.expert_tail(x, w, b, x_t=x_t, dt=-0.1, want_v=True, embed=(ew, eb, act, out), **kw)
+    assert torch.equal(v0, v1) and torch.equal(x0, x1)
+    want = F.linear(x1.cpu(), ew.cpu(), eb.cpu())
+    if model == "pi05":
+        # one rounding to bf16 of an fp32 sum: at most one bf16 step from the torch result where the sums differ in order
+        got = out.float().cpu()
+        assert float(((got - want.to(BF16).float()).abs() / want.abs().clamp_min(1.0)).max()) <= 2**-7
+        assert float((got != want.to(BF16).float()).float().mean()) < 0.02
+        assert torch.equal(wide[:, j:].float().cpu(), torch.full((m, 8), 7.0))
+    else:
+        want = F.silu(want)
+        assert float((out.cpu() - want).abs().max()) < 2e-5
+    # no bias
+    out2 = torch.empty(m, j, dtype=torch.float32, device="cuda")
+    tk.expert_tail(x, w, b, x_t=x_t, dt=-0.1, embed=(ew, None, "none", out2), **kw)
+    assert float((out2.cpu() - F.linear(x1.cpu(), ew.cpu())).abs().max()) < 2e-5
+    with pytest.raises(ValueError):
+        tk.expert_tail(x, w, b, embed=(ew, eb, act, out), **kw)  # no x_t: nothing to embed
+
+
 @pytest.mark.parametrize("m,p,k", [(50, 241, 720), (50, 177, 720), (7, 33, 96), (33, 256, 768)])
 def test_cross_layer_in_one_launch(tk, m, p, k):
     # norm + q projection + RoPE inside the attention launch (SmolVLA cross layers: 15 / 5 heads of 64,

@@ -940,9 +940,10 @@ int tk_batched_transpose_v(const void* v, long long v_sb, int v_sl, int v_sh, vo
   return TK_OK;
 }
 
-int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps,
-                   const void* w, const void* bias, void* v_out, const void* x_t, void* x_out, float dt, int M, int N, int K,
-                   void* stream) {
+static int tail_impl(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps,
+                     const void* w, const void* bias, void* v_out, const void* x_t, void* x_out, float dt, int M, int N, int K,
+                     const void* emb_w, const void* emb_b, int emb_n, int emb_act, void* emb_out, int emb_ld, int emb_dtype,
+                     void* stream) {
   if (M <= 0 || N <= 0 || K <= 0 || ldx < K) return fail(TK_EINVAL, "tail: bad shape M=%d N=%d K=%d ldx=%d", M, N, K, ldx);
   if (N > 256 || 256 % N) return fail(TK_EINVAL, "tail: N=%d must divide 256", N);
   // (the normalised row lives in LDS as fp32: 32 KiB at the limit)
@@ -968,8 +969,43 @@ int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_s
   a.M = M;
   a.N = N;
   a.K = K;
+  a.emb_w = nullptr;
+  a.emb_b = nullptr;
+  a.emb_out = nullptr;
+  a.emb_J = a.emb_ld = a.emb_act = a.emb_bf16 = 0;
+  if (emb_out) {
+    if (!x_out) return fail(TK_EINVAL, "tail: the embedding is computed from x_out");
+    if (N != tk_tail_embed_width()) return fail(TK_EINVAL, "tail: the embedding takes N=%d inputs, got %d", tk_tail_embed_width(), N);
+    if (!emb_w || !aligned16(emb_w)) return fail(TK_EINVAL, "tail: emb_w must be a 16-byte aligned fp32 [emb_n, N] matrix");
+    if (emb_n <= 0 || emb_ld < emb_n) return fail(TK_EINVAL, "tail: bad embedding shape emb_n=%d emb_ld=%d", emb_n, emb_ld);
+    if (emb_act != 0 && emb_act != 1) return fail(TK_EINVAL, "tail: emb_act=%d must be 0 (none) or 1 (SiLU)", emb_act);
+    if (emb_dtype != TK_BF16 && emb_dtype != TK_F32) return fail(TK_EINVAL, "tail: emb_dtype=%d", emb_dtype);
+    a.emb_w = (const float*)emb_w;
+    a.emb_b = (const float*)emb_b;
+    a.emb_out = emb_out;
+    a.emb_J = emb_n;
+    a.emb_ld = emb_ld;
+    a.emb_act = emb_act;
+    a.emb_bf16 = emb_dtype == TK_BF16;
+  }
   if (tk_launch_tail(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "tail: launch failed");
   return TK_OK;
+}
+
+int tk_expert_tail(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps,
+                   const void* w, const void* bias, void* v_out, const void* x_t, void* x_out, float dt, int M, int N, int K,
+                   void* stream) {
+  return tail_impl(x, ldx, norm_w, ada_scale, ada_shift, eps, w, bias, v_out, x_t, x_out, dt, M, N, K, nullptr, nullptr, 0, 0,
+                   nullptr, 0, 0, stream);
+}
+
+int tk_expert_tail_embed(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps,
+                         const void* w, const void* bias, void* v_out, const void* x_t, void* x_out, float dt, int M, int N,
+                         int K, const void* emb_w, const void* emb_b, int emb_n, int emb_act, void* emb_out, int emb_ld,
+                         int emb_dtype, void* stream) {
+  if (!emb_out) return fail(TK_EINVAL, "tail: emb_out is null");
+  return tail_impl(x, ldx, norm_w, ada_scale, ada_shift, eps, w, bias, v_out, x_t, x_out, dt, M, N, K, emb_w, emb_b, emb_n, emb_act,
+                   emb_out, emb_ld, emb_dtype, stream);
 }
 
 int tk_rms_norm_rows(const void* x, int ldx, const void* norm_w, const void* ada_scale, const void* ada_shift, float eps, void* y,

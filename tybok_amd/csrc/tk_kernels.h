@@ -171,6 +171,11 @@ struct TailArgs {
   float* x_out;       // fp32 [M, N] or nullptr
   float dt;
   int M, N, K;
+  // optional (with x_out, N == 32): emb_out[m, j] = act(sum_n x_out[m, n] * emb_w[j, n] + emb_b[j]), j < emb_J
+  const float* emb_w;  // fp32 [emb_J, N]
+  const float* emb_b;  // fp32 [emb_J] or nullptr
+  void* emb_out;       // fp32 or bf16 [M, emb_J], row pitch emb_ld elements
+  int emb_J, emb_ld, emb_act, emb_bf16;  // act: 0 none, 1 SiLU
 };
 
 struct NormRowsArgs {
@@ -197,6 +202,7 @@ struct RopeRowsArgs {
 int tk_launch_rope_rows(RopeRowsArgs a, hipStream_t st);
 int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st);
 int tk_launch_tail(TailArgs a, hipStream_t st);
+int tk_tail_embed_width();  // the embedding's input width the tail kernel is built for
 int tk_launch_kv_proj(KvProjArgs a, hipStream_t st);
 int tk_layer_norm_max_k();
 int tk_launch_layer_norm(LayerNormArgs a, hipStream_t st);

@@ -745,9 +745,12 @@ def expert_tail(
     x_t: torch.Tensor | None = None,
     dt: float = 0.0,
     want_v: bool = False,
+    embed: tuple[torch.Tensor, torch.Tensor | None, str, torch.Tensor] | None = None,
 ) -> tuple[torch.Tensor | None, torch.Tensor | None]:
     """Final norm of ``x [M, K]`` bf16, fp32 projection with ``w [N, K]`` (+ ``bias``), and -- with
-    ``x_t [M, N]`` -- the Euler update ``x_t + dt * v``.  Returns ``(v or None, x_new or None)``."""
+    ``x_t [M, N]`` -- the Euler update ``x_t + dt * v``.  Returns ``(v or None, x_new or None)``.
+    ``embed = (E [J, N] fp32, c [J] fp32 or None, "none" | "silu", out [M, J] fp32 or bf16)``: the same launch
+    also writes ``out = act(x_new @ E^T + c)``, the next step's suffix embedding."""
     lib = native.lib()
     if x.dtype != torch.bfloat16 or x.dim() != 2 or x.stride(1) != 1:
         raise TypeError("x must be bf16 [M, K] with unit inner stride")
@@ -764,6 +767,26 @@ def expert_tail(
         if x_t.dtype != torch.float32 or x_t.shape != (m, n) or not x_t.is_contiguous():
             raise ValueError("x_t must be contiguous fp32 [M, N]")
         x_new = torch.empty(m, n, **f32)
+    if embed is not None:
+        ew, eb, eact, eout = embed
+        if x_new is None:
+            raise ValueError("embed needs x_t")
+        if ew.dtype != torch.float32 or ew.dim() != 2 or ew.shape[1] != n or not ew.is_contiguous():
+            raise ValueError("embed weight must be contiguous fp32 [J, N]")
+        j = ew.shape[0]
+        if eb is not None and (eb.dtype != torch.float32 or eb.numel() != j or not eb.is_contiguous()):
+            raise ValueError("embed bias must be contiguous fp32 [J]")
+        if eout.dtype not in (torch.float32, torch.bfloat16) or eout.shape != (m, j) or eout.stride(1) != 1:
+            raise ValueError("embed out must be fp32 or bf16 [M, J] with unit inner stride")
+        if eact not in ("none", "silu"):
+            raise ValueError(f"embed activation {eact!r}")
+        rc = lib.tk_expert_tail_embed(
+            x.data_ptr(), x.stride(0), _norm_ptr(norm_w, k), *_ada_ptrs(ada, k), float(eps), w.data_ptr(), _ptr(bias), _ptr(v),
+            _ptr(x_t), _ptr(x_new), float(dt), m, n, k, ew.data_ptr(), _ptr(eb), j, 1 if eact == "silu" else 0, eout.data_ptr(),
+            eout.stride(0), _BF16 if eout.dtype == torch.bfloat16 else _F32, _stream(),
+        )  # fmt: skip
+        native.check(rc, "tk_expert_tail_embed")
+        return v, x_new
     rc = lib.tk_expert_tail(
         x.data_ptr(), x.stride(0), _norm_ptr(norm_w, k), *_ada_ptrs(ada, k), float(eps), w.data_ptr(), _ptr(bias), _ptr(v),
         _ptr(x_t), _ptr(x_new), float(dt), m, n, k, _stream(),

@@ -493,19 +493,34 @@ class SmolVLAModel:
             hidden = self._denoise_layer_fused(i, hidden, caches[i], prefix_pad[0], pos32, pos0_32, self.ws)
         return hidden
 
-    def fused_euler_step(self, prefix_pad, caches, x_t, step: int, positions, dt: float, want_v: bool = False):
+    def fused_euler_step(self, prefix_pad, caches, x_t, step: int, positions, dt: float, want_v: bool = False, h=None, next_step=None):
         """One velocity evaluation on the fused launches (time entry ``step``): folded suffix embedding, expert
         stack, then final norm + action projection + ``x_t + dt * v_t`` in one launch.  ``x_t [1, chunk, A]``
-        fp32.  Returns the updated ``x``; with ``want_v`` the pair ``(v_t, x_t + dt * v_t)``."""
+        fp32.  Returns the updated ``x``; with ``want_v`` the pair ``(v_t, x_t + dt * v_t)``.
+
+        ``h``: the first (folded) linear + SiLU of this step's suffix embedding when the previous step's last
+        launch already computed it.  ``next_step``: compute it for that time entry from the updated ``x`` in this
+        step's last launch; the return value is then ``(x_new, h_next)``."""
         pos32, pos0_32 = positions
-        h = F.silu(F.linear(x_t[0], self.suffix_w, self.suffix_b[step]))
+        if h is None:
+            h = F.silu(F.linear(x_t[0], self.suffix_w, self.suffix_b[step]))
         hidden = F.linear(h, self.p["action_time_mlp_out.weight"], self.p["action_time_mlp_out.bias"])
         hidden = self._denoise_step_fused(prefix_pad, caches, hidden, pos32, pos0_32)
+        h_next = None
+        if next_step is not None:
+            h_next = torch.empty(x_t.shape[1], self.suffix_w.shape[0], dtype=torch.float32, device=x_t.device)
         v, x_new = tk.expert_tail(
             hidden, self.p["action_out_proj.weight"], self.p["action_out_proj.bias"], norm_w=self.p[EXP + "norm.weight"],
             eps=self.eps, x_t=x_t[0], dt=dt, want_v=want_v,
+            embed=None if h_next is None else (self.suffix_w, self.suffix_b[next_step], "silu", h_next),
         )  # fmt: skip
+        if next_step is not None:
+            return x_new[None], h_next
         return (v[None], x_new[None]) if want_v else x_new[None]
+
+    def _fused_embed_ok(self, x_t) -> bool:
+        """The step tail can carry the next step's embedding: the padded action width it is built for."""
+        return self.suffix_w.is_contiguous() and self.suffix_w.shape[1] == 32 and x_t.shape[-1] == 32
 
     def denoise_step(self, prefix_pad, keys, values, ekv, x_t, time_emb, positions=None, caches=None):
         """Velocity ``v_t`` fp32 ``[1, chunk, max_action_dim]`` (flow_matching.py:316-350)."""
@@ -568,15 +583,20 @@ class SmolVLAModel:
                 else:
                     caches[i] = tk.PrefixKV(keys[i, 0], vt[i])
                 hid_s = self._denoise_layer_fused(i, hid_s, caches[i], pads[0], positions[0], positions[1], self.ws_side)
+        carry = self._fused_embed_ok(noise) and self.num_steps > 1
+        h = torch.empty(noise.shape[1], self.suffix_w.shape[0], dtype=torch.float32, device=noise.device) if carry else None
         with torch.cuda.stream(side):
             _, x_new = tk.expert_tail(
                 hid_s, self.p["action_out_proj.weight"], self.p["action_out_proj.bias"], norm_w=self.p[EXP + "norm.weight"],
-                eps=self.eps, x_t=noise[0], dt=dt,
+                eps=self.eps, x_t=noise[0], dt=dt, embed=(self.suffix_w, self.suffix_b[1], "silu", h) if carry else None,
             )  # fmt: skip
         main.wait_stream(side)
         x_t = x_new[None]
         for step in range(1, self.num_steps):
-            x_t = self.fused_euler_step(pads, caches, x_t, step, positions, dt)
+            if carry and step + 1 < self.num_steps:
+                x_t, h = self.fused_euler_step(pads, caches, x_t, step, positions, dt, h=h, next_step=step + 1)
+            else:
+                x_t = self.fused_euler_step(pads, caches, x_t, step, positions, dt, h=h)
         return x_t
 
     def sample_actions_core(self, embs, pads, att, noise, trace: dict | None = None) -> torch.Tensor:
@@ -611,9 +631,14 @@ class SmolVLAModel:
                     v1 = self.denoise_step(pads, keys, values, ekv, x_t + dt * v0, self.time_embs[2 * step + 1], positions, caches)
                 x_t = x_t + (dt * 0.5) * (v0 + v1)
             return x_t
+        h = None
+        carry = fused_loop and self._fused_embed_ok(x_t)
         for step in range(self.num_steps):
             if fused_loop:
-                x_t = self.fused_euler_step(pads, caches, x_t, step, positions, dt)
+                if carry and step + 1 < self.num_steps:
+                    x_t, h = self.fused_euler_step(pads, caches, x_t, step, positions, dt, h=h, next_step=step + 1)
+                else:
+                    x_t = self.fused_euler_step(pads, caches, x_t, step, positions, dt, h=h)
                 continue
             v_t = self.denoise_step(pads, keys, values, ekv, x_t, self.time_embs[step], positions, caches)
             x_t = x_t + dt * v_t
