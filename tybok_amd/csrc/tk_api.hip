@@ -229,10 +229,12 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   // as many CUs on it (measured: FFN at K=720 12.6 -> 10.0 us, with the norm prologue 15.7 -> 12.6 us);
   // the weights are then read twice, which only a large matrix notices (the 33.5 MB shapes lose 5 %).
   if (M > 32 && M <= 64 && (size_t)a.ntiles * 32 * a.KT * 32 * (e.w16 ? 2 : 1) <= (16u << 20)) MT = 1;
-  // A few hundred rows (the SmolVLA prefill: 241 / 177) with the bf16 RMSNorm prologue over a short K: 32-row
-  // blocks too -- they run the prologue that requests every round up front and takes the row statistics from
-  // the staged pieces, and there are enough of them to fill the device (measured: -3 us per launch in a request)
+  // A few hundred rows (the SmolVLA prefill: 241 / 177) over a small matrix: 32-row blocks too.  With the bf16
+  // RMSNorm prologue over a short K they run the prologue that requests every round up front and takes the row
+  // statistics from the staged pieces (-3 us per launch inside a request); the other launches gain 0.7 us from the
+  // finer blocks
   if (M > 64 && e.norm_w && !e.x_f32 && a.KT <= 32) MT = 1;
+  if (M > 64 && M <= 256 && !e.x_f32 && (size_t)a.ntiles * 32 * a.KT * 32 * (e.w16 ? 2 : 1) <= (16u << 20)) MT = 1;
   int NT = 2;
   if (!gated && !rope && ((a.ntiles + 1) / 2) * ((M + 32 * MT - 1) / (32 * MT)) < cus / 2) {
     NT = 1;  // few columns: finer strips (the paired epilogues need both tiles of a strip in one wave)
