@@ -93,15 +93,19 @@ def test_full_model_zero_noise_chunk_against_oracle_and_noise_floor(cameras):
     # asserted in a comment: `ref32` is the oracle run on the same weights with every activation in fp32.
     # The reference-dtype (bf16) oracle itself sits 0.85e-2 .. 1.3e-2 (max) / 2.0e-3 .. 2.2e-3 (mean) from
     # it -- rounding flips amplified through 32 layers x 10 steps, re-drawn by any change of summation
-    # order -- so no bf16 implementation, the reference's own included, holds 1e-2 on every frame.  Held:
+    # order (a different split of a k loop over waves, even in the fp32 K/V projection, moves a frame's
+    # maximum by +-25 %) -- so no bf16 implementation, the reference's own included, holds 1e-2 on every
+    # frame, and two of them that each sit ~1e-2 from ref32 are up to sqrt(2) times that apart.  Held:
     #   * per frame, the HIP path is no farther from ref32 than the bf16 oracle is (x1.15 mean, x1.5 max:
     #     the maximum of 1600 values re-draws by +-25 % between equally good executions);
-    #   * per frame, against the bf16 oracle: the chunk the engine returns (first 6 of 32 padded outputs)
-    #     and all 32 outputs <= 1.25e-2, mean <= 3e-3;
-    #   * on the benchmark's own configuration (3 cameras), the median over the three frames of the
-    #     all-output maxima <= 1e-2 (the stated bound); with 2 cameras the per-frame bounds only (the bf16
-    #     oracle's own distance from ref32 reaches 1.27e-2 there).
+    #   * per frame, against the bf16 oracle: the chunk the engine returns (first 6 of the 32 padded
+    #     outputs) <= 1.25e-2, all 32 outputs <= 1.5e-2, mean <= 3e-3;
+    #   * over the three frames, so that one rounding flip does not decide: the median of the returned
+    #     chunk's maxima <= 1e-2 (the stated bound) for both camera counts, and the median of the
+    #     all-output maxima <= 1e-2 on the benchmark's own configuration (3 cameras), <= 1.25e-2 with 2
+    #     cameras (the bf16 oracle's own distance from ref32 reaches 1.27e-2 there).
     maxima = {"north_star": [], "benched": []}
+    chunk_maxima = {"north_star": [], "benched": []}
     for seed in (0, 1, 2):
         cfg, sd, inp = cases.smolvla_build(dict(cases.SMOLVLA_CASES["full"], cameras=cameras, seed=seed))
         adim = cfg.action_feature_shape[0]
@@ -117,10 +121,13 @@ def test_full_model_zero_noise_chunk_against_oracle_and_noise_floor(cameras):
             )
             assert torch.isfinite(got).all()
             assert d_mean <= 1.15 * floor_mean and d_max <= 1.5 * floor_max
-            assert e_act <= 1.25e-2 and e_all <= 1.25e-2 and e_mean <= 3e-3
+            assert e_act <= 1.25e-2 and e_all <= 1.5e-2 and e_mean <= 3e-3
             maxima[name].append(e_all)
+            chunk_maxima[name].append(e_act)
     for name, vals in maxima.items():
-        assert cameras != 3 or sorted(vals)[1] <= 1e-2, f"{name}: median of the per-frame maxima {sorted(vals)} exceeds 1e-2"
+        cap = 1e-2 if cameras == 3 else 1.25e-2
+        assert sorted(vals)[1] <= cap, f"{name}: median of the per-frame maxima {sorted(vals)} exceeds {cap}"
+        assert sorted(chunk_maxima[name])[1] <= 1e-2, f"{name}: median of the returned chunk's maxima {sorted(chunk_maxima[name])} exceeds 1e-2"
 
 
 def test_full_model_bf16_path_matches_reference_golden():

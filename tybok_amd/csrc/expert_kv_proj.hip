@@ -6,8 +6,8 @@
 //   -> K as bf16 hi + lo planes [P, G, D], V^T as bf16 hi + lo planes [G, D, ld] (keys contiguous,
 //      zero filled from P to the next multiple of 32) -- what tk_attn_prepare_kv produces from ek, ev.
 //
-// One wave computes a 32 (output columns) x 32 (prefix rows) tile of K or V on the fp32 matrix
-// instruction v_mfma_f32_32x32x2_f32 (full fp32 products and sums).  The weight rows are the A
+// A block computes a 32 (output columns) x 32 (prefix rows) tile of K or V on the fp32 matrix
+// instruction v_mfma_f32_32x32x2_f32 (full fp32 products and sums), its four waves splitting the input columns.  The weight rows are the A
 // operand and the prefix rows the B operand, both read straight from global memory: lane (r, h)
 // loads 16 consecutive input columns' worth of its row in 16-byte pieces -- columns 16j + 8h .. + 7
 // for step j -- and feeds them to 8 MFMAs; which k pairs meet in one instruction does not matter
@@ -19,14 +19,17 @@
 
 namespace {
 
-constexpr int JB = 10;  // k steps (of 16 input columns) whose loads are in flight together (KV = 320: two batches)
+constexpr int JB = 5;  // k steps (of 16 input columns) a wave has in flight together (KV = 320: all of its five)
 
+// A block of four waves owns one 32 x 32 tile: wave w walks every fourth batch of JB k steps (a 160-instruction
+// fp32 MFMA chain on one wave took 5 us of the launch; four waves of 40 on one CU, 160 blocks instead of 48), the
+// partial tiles meet in LDS and wave g finishes register group g (columns 8g .. 8g + 7): sum in wave order.
 __global__ __launch_bounds__(256) void expert_kv_proj_kernel(KvProjArgs a) {
+  __shared__ f32x4 red[4][4][64];  // [wave][register group][lane]
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int half = lane >> 5, l32 = lane & 31;
-  const int nt = blockIdx.y * 4 + wave;  // 32-column tile of the output
-  if (nt * 32 >= a.N) return;
+  const int nt = blockIdx.y;  // 32-column tile of the output
   const bool is_v = blockIdx.z != 0;
   int p = blockIdx.x * 32 + l32;
   const int pc = p < a.P ? p : a.P - 1;  // rows past P: valid data, zeroed / skipped below
@@ -37,7 +40,7 @@ __global__ __launch_bounds__(256) void expert_kv_proj_kernel(KvProjArgs a) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
   const int steps = a.KV / 16;
-  for (int j0 = 0; j0 < steps; j0 += JB) {
+  for (int j0 = wave * JB; j0 < steps; j0 += 4 * JB) {  // wave-uniform
     i32x4 xr[JB];
     f32x4 wr[JB][2];
 #pragma unroll
@@ -59,12 +62,17 @@ __global__ __launch_bounds__(256) void expert_kv_proj_kernel(KvProjArgs a) {
       }
     }
   }
-
-  // lane: prefix row p, output columns nt*32 + 8g + 4*half + 0..3 in register group g
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
+  for (int g = 0; g < 4; ++g) red[wave][g][lane] = f32x4{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+  __syncthreads();
+
+  // lane: prefix row p, output columns nt*32 + 8g + 4*half + 0..3 of register group g = wave
+  {
+    const int g = wave;
     const int n = nt * 32 + 8 * g + 4 * half;
-    f32x4 v = {acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+    f32x4 v = red[0][g][lane];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) v += red[w][g][lane];
     if (p >= a.P) v = f32x4{0.f, 0.f, 0.f, 0.f};
     const i32x2 hi = pack_bf16x4(v);
     const i32x2 lo = pack_bf16x4(v - unpack_bf16x4(hi));
@@ -87,7 +95,7 @@ __global__ __launch_bounds__(256) void expert_kv_proj_kernel(KvProjArgs a) {
 }  // namespace
 
 int tk_launch_kv_proj(KvProjArgs a, hipStream_t st) {
-  dim3 grid((a.P + 31) / 32, (a.N / 32 + 3) / 4, 2);
+  dim3 grid((a.P + 31) / 32, a.N / 32, 2);
   hipLaunchKernelGGL(expert_kv_proj_kernel, grid, dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
