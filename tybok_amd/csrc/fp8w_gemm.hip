@@ -57,7 +57,8 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   constexpr int XBUF = ROWS * PITCH;          // bytes per staging buffer
   constexpr int PPR = ROWB / 16;              // 8-element pieces per row
   constexpr int XPT = ROWS * PPR / (NW * 64); // pieces per thread and round
-  constexpr int RED_BYTES = TILES * NW * 16 * 64 * 4;  // every wave's partial tiles at once
+  constexpr int RW = 4;                       // waves that reduce and finish (one per register group)
+  constexpr int RED_BYTES = TILES * RW * 16 * 64 * 4;  // four waves' partial tiles at once
   constexpr int LDS_BYTES = 2 * XBUF > RED_BYTES ? 2 * XBUF : RED_BYTES;
   constexpr int WCH = W16 ? 2 : 1;            // 16-byte operand chunks per lane, n tile and k tile
   constexpr int WTILE = W16 ? 2048 : 1024;    // bytes of one packed 32x32 tile
@@ -284,7 +285,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   }
   if (FULL) {
     // piece i of every round belongs to row xrow[i]; the PPR threads that share a row are consecutive lanes
-    static_assert(!FULL || (PPR == 16 && !XF32), "the row's pieces sit in 16 consecutive lanes");
+    static_assert(!FULL || ((PPR == 16 || PPR == 32) && !XF32), "the row's pieces sit in PPR consecutive lanes");
 #pragma unroll
     for (int i = 0; i < XPT; ++i) {
       float ss0 = 0.f, ss1 = 0.f;
@@ -375,7 +376,30 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   // register i, output column n = 8*(i/4) + 4*(l/32) + i%4 -- register group g = i/4 is four
   // consecutive columns.  From here on wave w owns group g = w of EVERY tile: all four waves take
   // part in the reductions and in the epilogue, and everything moves as 8- or 16-byte vectors.
-  static_assert(NW == 4, "one wave per register group");
+  static_assert(NW == 4 || NW == 8, "one wave per register group, or two");
+  if (NW == 8) {
+    // eight waves walked the k tiles: waves 4..7 hand their accumulators to waves 0..3 (w + 4 -> w) and leave
+    f32x4 (*fold)[RW][4][64] = (f32x4 (*)[RW][4][64])lds;  // [tile][wave - 4][group][lane]
+    if (wave >= RW) {
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          fold[t][wave - RW][g][lane] = f32x4{acc[t / NT][t % NT][4 * g], acc[t / NT][t % NT][4 * g + 1], acc[t / NT][t % NT][4 * g + 2],
+                                              acc[t / NT][t % NT][4 * g + 3]};
+    }
+    __syncthreads();
+    if (wave >= RW) return;
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 v = fold[t][wave][g][lane];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[t / NT][t % NT][4 * g + j] += v[j];
+      }
+    __syncthreads();  // (the four remaining waves) the exchange below reuses the space
+  }
   const int ng = wave * 8 + half * 4;  // first of this lane's four columns within an n tile
 
   // ---- epilogue operands: requested now, consumed after the reductions ----
@@ -421,7 +445,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   }
 
   // ---- in-block reduction over waves (fixed order w = 0..3): one exchange for all tiles ----
-  f32x4 (*red)[NW][4][64] = (f32x4 (*)[NW][4][64])lds;  // [tile][wave][group][lane]
+  f32x4 (*red)[RW][4][64] = (f32x4 (*)[RW][4][64])lds;  // [tile][wave][group][lane]
   f32x4 own[TILES];
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
@@ -437,7 +461,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   for (int t = 0; t < TILES; ++t) {
     f32x4 sum = red[t][0][wave][lane];
 #pragma unroll
-    for (int w = 1; w < NW; ++w) sum += red[t][w][wave][lane];
+    for (int w = 1; w < RW; ++w) sum += red[t][w][wave][lane];
     own[t] = sum;
   }
 
@@ -666,62 +690,77 @@ __global__ void decode_fp8_kernel(float* out) {
 // wave and round halve the barriers but lengthen every small launch of the denoise loop.
 constexpr int kPF = 4;
 constexpr int kTPW = 1;
-template <int MT, int NT, int EPI, bool W16, int PRO, int NR>
+constexpr int kPF8 = 3;  // rounds in flight of the eight-wave blocks (2 and 4 measured slower in whole requests)
+template <int MT, int NT, int EPI, bool W16, int PRO, int NR, int NW>
 int launch_nr(const GemmArgs& a, dim3 grid, hipStream_t st) {
   // the RMSNorm prologue over a short K that one block walks alone: all of its rounds in flight, the row
-  // statistics taken from the staged pieces (SmolVLA's expert: K = 720 -> 6 rounds, VLM: 960 -> 8)
-  constexpr bool CAN_FULL = PRO == 1 && MT == 1 && (NR == 6 || NR == 8);
+  // statistics taken from the staged pieces (SmolVLA's expert: K = 720, VLM: 960)
+  constexpr bool CAN_FULL = PRO == 1 && MT == 1 && NR > 0 && NR * NW <= 32;
+  constexpr int PFN = NW == 8 ? kPF8 : kPF;
   if (CAN_FULL && a.ksplit == 1) {
-    hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, CAN_FULL ? NR : kPF, kTPW, W16, PRO, NR>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, NW, EPI, CAN_FULL ? NR : PFN, kTPW, W16, PRO, NR>), grid, dim3(NW * 64), 0, st, a);
   } else {
-    hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, 4, EPI, kPF, kTPW, W16, PRO, NR>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, NW, EPI, PFN, kTPW, W16, PRO, NR>), grid, dim3(NW * 64), 0, st, a);
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 template <int MT, int NT, int EPI, bool W16, int PRO>
-int launch(const GemmArgs& a, dim3 grid, hipStream_t st) {
+int launch(const GemmArgs& a, dim3 grid, int nw, hipStream_t st) {
   // the action chunk's launches (32-row blocks, every block the same number of k tiles) at the round counts
-  // of the two models' expert layers: K = 720 -> 6, 960 / 1024 -> 8, 2048 -> 16, 4096 in four splits -> 8
+  // of the two models' expert layers.  Four waves: K = 720 -> 6, 960 / 1024 -> 8, 2048 -> 16, 4096 in four
+  // splits -> 8; eight waves: 3, 4, 8, 4
   if (MT == 1 && a.kt_r == 0) {
-    const int nr = (a.kt_q + 4 * kTPW - 1) / (4 * kTPW);
-    if (nr == 6) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 6 : 0>(a, grid, st);
-    if (nr == 8) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 8 : 0>(a, grid, st);
-    if (nr == 16) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 16 : 0>(a, grid, st);
+    const int nr = (a.kt_q + nw * kTPW - 1) / (nw * kTPW);
+    if (nw == 8) {
+      if (nr == 3) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 3 : 0, MT == 1 ? 8 : 4>(a, grid, st);
+      if (nr == 4) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 4 : 0, MT == 1 ? 8 : 4>(a, grid, st);
+      if (nr == 8) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 8 : 0, MT == 1 ? 8 : 4>(a, grid, st);
+    } else {
+      if (nr == 6) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 6 : 0, 4>(a, grid, st);
+      if (nr == 8) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 8 : 0, 4>(a, grid, st);
+      if (nr == 16) return launch_nr<MT, NT, EPI, W16, PRO, MT == 1 ? 16 : 0, 4>(a, grid, st);
+    }
   }
-  return launch_nr<MT, NT, EPI, W16, PRO, 0>(a, grid, st);
+  if (MT == 1 && nw == 8) return launch_nr<MT, NT, EPI, W16, PRO, 0, MT == 1 ? 8 : 4>(a, grid, st);
+  return launch_nr<MT, NT, EPI, W16, PRO, 0, 4>(a, grid, st);
 }
 
 }  // namespace
 
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st) {
   dim3 grid((a.ntiles + NT - 1) / NT, a.ksplit, mblocks);
+  // eight waves on a 32-row block where they pay (measured per launch and in whole requests, K = 720 .. 2048): a
+  // long k range of fp8 tiles (half the rounds) or the RMSNorm prologue (half the normalisation work per thread);
+  // elsewhere four waves are as fast or faster (one LDS exchange less)
+  const int pro_ = a.ada_scale != nullptr ? 3 : (a.norm_w == nullptr ? 0 : (a.x_f32 ? 2 : 1));
+  const int nw = (MT == 1 && ((!a.w16 && a.kt_q >= 48) || pro_ == 1)) ? 8 : 4;
   const int epi = a.s1 != nullptr ? 1 : (a.rope_pos != nullptr ? 2 : 0);
   const int pro = a.ada_scale != nullptr ? 3 : (a.norm_w == nullptr ? 0 : (a.x_f32 ? 2 : 1));
   if (a.w16) {
     // bf16-weight linears of the expert / VLM layers: 32- or 64-row blocks; one-tile strips for the plain epilogue only
     if (NT == 1) {
       if (epi != 0 || pro != 0) return -1;
-      return MT == 1 ? launch<1, 1, 0, true, 0>(a, grid, st) : launch<2, 1, 0, true, 0>(a, grid, st);
+      return MT == 1 ? launch<1, 1, 0, true, 0>(a, grid, nw, st) : launch<2, 1, 0, true, 0>(a, grid, nw, st);
     }
     if (epi == 2) {
-      if (pro == 1) return MT == 1 ? launch<1, 2, 2, true, 1>(a, grid, st) : launch<2, 2, 2, true, 1>(a, grid, st);
-      if (pro == 2) return MT == 1 ? launch<1, 2, 2, true, 2>(a, grid, st) : launch<2, 2, 2, true, 2>(a, grid, st);
-      if (pro == 3) return MT == 1 ? launch<1, 2, 2, true, 3>(a, grid, st) : launch<2, 2, 2, true, 3>(a, grid, st);
-      return MT == 1 ? launch<1, 2, 2, true, 0>(a, grid, st) : launch<2, 2, 2, true, 0>(a, grid, st);
+      if (pro == 1) return MT == 1 ? launch<1, 2, 2, true, 1>(a, grid, nw, st) : launch<2, 2, 2, true, 1>(a, grid, nw, st);
+      if (pro == 2) return MT == 1 ? launch<1, 2, 2, true, 2>(a, grid, nw, st) : launch<2, 2, 2, true, 2>(a, grid, nw, st);
+      if (pro == 3) return MT == 1 ? launch<1, 2, 2, true, 3>(a, grid, nw, st) : launch<2, 2, 2, true, 3>(a, grid, nw, st);
+      return MT == 1 ? launch<1, 2, 2, true, 0>(a, grid, nw, st) : launch<2, 2, 2, true, 0>(a, grid, nw, st);
     }
-    if (epi == 0 && pro == 0) return MT == 1 ? launch<1, 2, 0, true, 0>(a, grid, st) : launch<2, 2, 0, true, 0>(a, grid, st);
+    if (epi == 0 && pro == 0) return MT == 1 ? launch<1, 2, 0, true, 0>(a, grid, nw, st) : launch<2, 2, 0, true, 0>(a, grid, nw, st);
     return -1;
   }
   if (epi == 2 || pro == 2) return -1;
   if (epi == 1) {
     if (NT != 2) return -1;
-    if (pro == 1) return MT == 1 ? launch<1, 2, 1, false, 1>(a, grid, st) : launch<2, 2, 1, false, 1>(a, grid, st);
-    if (pro == 3) return MT == 1 ? launch<1, 2, 1, false, 3>(a, grid, st) : launch<2, 2, 1, false, 3>(a, grid, st);
-    return MT == 1 ? launch<1, 2, 1, false, 0>(a, grid, st) : launch<2, 2, 1, false, 0>(a, grid, st);
+    if (pro == 1) return MT == 1 ? launch<1, 2, 1, false, 1>(a, grid, nw, st) : launch<2, 2, 1, false, 1>(a, grid, nw, st);
+    if (pro == 3) return MT == 1 ? launch<1, 2, 1, false, 3>(a, grid, nw, st) : launch<2, 2, 1, false, 3>(a, grid, nw, st);
+    return MT == 1 ? launch<1, 2, 1, false, 0>(a, grid, nw, st) : launch<2, 2, 1, false, 0>(a, grid, nw, st);
   }
   if (pro) return -1;
-  if (NT == 1) return MT == 1 ? launch<1, 1, 0, false, 0>(a, grid, st) : launch<2, 1, 0, false, 0>(a, grid, st);
-  return MT == 1 ? launch<1, 2, 0, false, 0>(a, grid, st) : launch<2, 2, 0, false, 0>(a, grid, st);
+  if (NT == 1) return MT == 1 ? launch<1, 1, 0, false, 0>(a, grid, nw, st) : launch<2, 1, 0, false, 0>(a, grid, nw, st);
+  return MT == 1 ? launch<1, 2, 0, false, 0>(a, grid, nw, st) : launch<2, 2, 0, false, 0>(a, grid, nw, st);
 }
 
 int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st) {
