@@ -68,6 +68,9 @@ def _qkv_oracle(x, norm_w, w, pos, heads, kv_heads, d, eps):
         (50, 1024, 8, 1, 256),  # pi0.5 expert geometry
         (7, 48, 2, 1, 64),  # tiny, one ragged k tile
         (100, 720, 15, 5, 64),  # two row blocks
+        (241, 960, 15, 5, 64),  # SmolVLA prefill, 3 cameras: 32-row blocks, every round requested up front
+        (177, 960, 15, 5, 64),  # 2 cameras
+        (40, 2048, 4, 2, 64),  # a K too long for the up-front prologue: statistics in a pass of their own
     ],
 )
 def test_norm_qkv_rope(tk, m, k, heads, kv_heads, d, x_dtype):
@@ -130,7 +133,10 @@ def test_o_proj_residual(tk, m, k, n, resid_dtype):
         _close(forced, want, f"o_proj split_k={split}")
 
 
-@pytest.mark.parametrize("act,m,k,i", [("silu", 50, 720, 2048), ("gelu_tanh", 50, 1024, 4096), ("silu", 1, 720, 2048)])
+@pytest.mark.parametrize(
+    "act,m,k,i",
+    [("silu", 50, 720, 2048), ("gelu_tanh", 50, 1024, 4096), ("silu", 1, 720, 2048), ("silu", 241, 960, 2560), ("silu", 64, 720, 2048), ("silu", 33, 2048, 512)],
+)
 def test_norm_gated_ffn(tk, act, m, k, i):
     eps = 1e-5
     x, wg8, sg, wu8, su, wd8, sd = ffn_case(m, k, i, seed=14)
