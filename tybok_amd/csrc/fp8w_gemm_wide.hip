@@ -423,19 +423,38 @@ __global__ __launch_bounds__(NW * 64, OCC) void fp8w_wide_kernel(GemmArgs a, int
 
 // One block per row: out = bf16 norm of the bf16 row, with the rounding points of the skinny
 // kernel's prologues: RMSNorm bf16(w * bf16(x * rstd)); adaptive bf16((x * rstd) * (1 + scale) + shift).
+// A thread's first piece of the row and the norm's operands for it are requested together up front and stay in
+// registers (rows up to 2048 columns need nothing else): one memory round trip before the store, not three.
 __global__ __launch_bounds__(256) void norm_rows_kernel(NormRowsArgs a) {
   __shared__ float part[4];
   const int tid = threadIdx.x;
   const char* row = (const char*)a.x + (size_t)blockIdx.x * a.ldx * 2;
   const int pieces = a.K / 8;
+  const int p0 = tid < pieces ? tid : pieces - 1;  // past the row: a valid piece, not used
+  union { i32x4 v; bf16x2 h[4]; unsigned u[4]; } x0;
+  x0.v = *(const i32x4*)(row + (size_t)p0 * 16);
+  union { i32x4 v[2]; float f[8]; } sc0, sh0;
+  union { i32x4 v; unsigned u[4]; } nw0;
+  if (a.ada_scale) {
+    sc0.v[0] = *(const i32x4*)(a.ada_scale + p0 * 8);
+    sc0.v[1] = *(const i32x4*)(a.ada_scale + p0 * 8 + 4);
+    sh0.v[0] = *(const i32x4*)(a.ada_shift + p0 * 8);
+    sh0.v[1] = *(const i32x4*)(a.ada_shift + p0 * 8 + 4);
+  } else {
+    nw0.v = *(const i32x4*)(a.norm_w + p0 * 8);
+  }
   float ss0 = 0.f, ss1 = 0.f;
-  for (int p = tid; p < pieces; p += 256) {
+  auto square = [&](const bf16x2* h) {
+    ss0 = __builtin_amdgcn_fdot2_f32_bf16(h[0], h[0], ss0, false);
+    ss1 = __builtin_amdgcn_fdot2_f32_bf16(h[1], h[1], ss1, false);
+    ss0 = __builtin_amdgcn_fdot2_f32_bf16(h[2], h[2], ss0, false);
+    ss1 = __builtin_amdgcn_fdot2_f32_bf16(h[3], h[3], ss1, false);
+  };
+  if (tid < pieces) square(x0.h);
+  for (int p = tid + 256; p < pieces; p += 256) {
     union { i32x4 v; bf16x2 h[4]; } xu;
     xu.v = *(const i32x4*)(row + (size_t)p * 16);
-    ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[0], xu.h[0], ss0, false);
-    ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[1], xu.h[1], ss1, false);
-    ss0 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[2], xu.h[2], ss0, false);
-    ss1 = __builtin_amdgcn_fdot2_f32_bf16(xu.h[3], xu.h[3], ss1, false);
+    square(xu.h);
   }
   float ss = ss0 + ss1;
 #pragma unroll
@@ -445,33 +464,40 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(NormRowsArgs a) {
   ss = (part[0] + part[1]) + (part[2] + part[3]);
   const float rstd = rsqrtf(ss / (float)a.K + a.eps);
   char* dst = (char*)a.out + (size_t)blockIdx.x * a.ldo * 2;
-  for (int p = tid; p < pieces; p += 256) {
-    union { i32x4 v; unsigned u[4]; } xu, o;
+  auto norm_piece = [&](const unsigned* xu, const float* sc, const float* sh, const unsigned* nw) {
+    union { i32x4 v; unsigned u[4]; } o;
+    if (a.ada_scale) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float x0f = __uint_as_float(xu[e] << 16), x1f = __uint_as_float(xu[e] & 0xffff0000u);
+        const float y0 = add_rn(mul_rn(mul_rn(x0f, rstd), add_rn(1.0f, sc[2 * e])), sh[2 * e]);
+        const float y1 = add_rn(mul_rn(mul_rn(x1f, rstd), add_rn(1.0f, sc[2 * e + 1])), sh[2 * e + 1]);
+        o.u[e] = pack_bf16x2(y0, y1);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const unsigned u = pack_bf16x2(__uint_as_float(xu[e] << 16) * rstd, __uint_as_float(xu[e] & 0xffff0000u) * rstd);
+        o.u[e] = pack_bf16x2(__uint_as_float(nw[e] << 16) * __uint_as_float(u << 16),
+                             __uint_as_float(nw[e] & 0xffff0000u) * __uint_as_float(u & 0xffff0000u));
+      }
+    }
+    return o.v;
+  };
+  if (tid < pieces) *(i32x4*)(dst + (size_t)tid * 16) = norm_piece(x0.u, sc0.f, sh0.f, nw0.u);
+  for (int p = tid + 256; p < pieces; p += 256) {
+    union { i32x4 v; unsigned u[4]; } xu, nw;
+    union { i32x4 v[2]; float f[8]; } sc, sh;
     xu.v = *(const i32x4*)(row + (size_t)p * 16);
     if (a.ada_scale) {
-      union { i32x4 v[2]; float f[8]; } sc, sh;
       sc.v[0] = *(const i32x4*)(a.ada_scale + p * 8);
       sc.v[1] = *(const i32x4*)(a.ada_scale + p * 8 + 4);
       sh.v[0] = *(const i32x4*)(a.ada_shift + p * 8);
       sh.v[1] = *(const i32x4*)(a.ada_shift + p * 8 + 4);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float x0 = __uint_as_float(xu.u[e] << 16), x1 = __uint_as_float(xu.u[e] & 0xffff0000u);
-        const float y0 = add_rn(mul_rn(mul_rn(x0, rstd), add_rn(1.0f, sc.f[2 * e])), sh.f[2 * e]);
-        const float y1 = add_rn(mul_rn(mul_rn(x1, rstd), add_rn(1.0f, sc.f[2 * e + 1])), sh.f[2 * e + 1]);
-        o.u[e] = pack_bf16x2(y0, y1);
-      }
     } else {
-      union { i32x4 v; unsigned u[4]; } nw;
       nw.v = *(const i32x4*)(a.norm_w + p * 8);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const unsigned u = pack_bf16x2(__uint_as_float(xu.u[e] << 16) * rstd, __uint_as_float(xu.u[e] & 0xffff0000u) * rstd);
-        o.u[e] = pack_bf16x2(__uint_as_float(nw.u[e] << 16) * __uint_as_float(u << 16),
-                             __uint_as_float(nw.u[e] & 0xffff0000u) * __uint_as_float(u & 0xffff0000u));
-      }
     }
-    *(i32x4*)(dst + (size_t)p * 16) = o.v;
+    *(i32x4*)(dst + (size_t)p * 16) = norm_piece(xu.u, sc.f, sh.f, nw.u);
   }
 }
 

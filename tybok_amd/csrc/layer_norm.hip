@@ -21,6 +21,24 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(LayerNormArgs a) {
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= a.M) return;
   const int pieces = a.K / 8;
+  // the parameters of this lane's pieces are requested with the row (they depend on nothing computed here): asked
+  // for after the two reductions they would cost the launch one more memory round trip
+  i32x4 wq[PMAX][WF32 ? 2 : 1], bq[PMAX][WF32 ? 2 : 1];
+#pragma unroll
+  for (int i = 0; i < PMAX; ++i) {
+    const int p = lane + 64 * i < pieces ? lane + 64 * i : pieces - 1;
+    if (WF32) {
+      const i32x4* wp = (const i32x4*)((const float*)a.w + 8 * p);
+      const i32x4* bp = (const i32x4*)((const float*)a.b + 8 * p);
+      wq[i][0] = wp[0];
+      wq[i][WF32 ? 1 : 0] = wp[1];
+      bq[i][0] = bp[0];
+      bq[i][WF32 ? 1 : 0] = bp[1];
+    } else {
+      wq[i][0] = *(const i32x4*)((const u16*)a.w + 8 * p);
+      bq[i][0] = *(const i32x4*)((const u16*)a.b + 8 * p);
+    }
+  }
   float v[PMAX][8];
   float sum = 0.f;
 #pragma unroll
@@ -91,15 +109,17 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(LayerNormArgs a) {
     if (p < pieces) {
       float w[8], b[8];
       if (WF32) {
-        const f32x4* wp = (const f32x4*)((const float*)a.w + 8 * p);
-        const f32x4* bp = (const f32x4*)((const float*)a.b + 8 * p);
-        const f32x4 w0 = wp[0], w1 = wp[1], b0 = bp[0], b1 = bp[1];
+        union { i32x4 q[2]; float f[8]; } wu, bu;
+        wu.q[0] = wq[i][0];
+        wu.q[1] = wq[i][WF32 ? 1 : 0];
+        bu.q[0] = bq[i][0];
+        bu.q[1] = bq[i][WF32 ? 1 : 0];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { w[e] = w0[e]; w[4 + e] = w1[e]; b[e] = b0[e]; b[4 + e] = b1[e]; }
+        for (int e = 0; e < 8; ++e) { w[e] = wu.f[e]; b[e] = bu.f[e]; }
       } else {
         union { i32x4 q; unsigned u[4]; } wu, bu;
-        wu.q = *(const i32x4*)((const u16*)a.w + 8 * p);
-        bu.q = *(const i32x4*)((const u16*)a.b + 8 * p);
+        wu.q = wq[i][0];
+        bu.q = bq[i][0];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           w[2 * e] = __uint_as_float(wu.u[e] << 16);
