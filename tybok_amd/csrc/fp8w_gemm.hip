@@ -111,6 +111,16 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     xrow[i] = r;
   }
 
+  // rotary epilogue: the positions of this lane's rows, requested before anything else -- the table rows they
+  // select are requested after the k loop, and would otherwise wait a second round trip for them there
+  int rpos[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int m = (mblock * MT + mt) * 32 + l32;
+    if (m > a.M - 1) m = a.M - 1;
+    rpos[mt] = EPI == 2 ? a.rope_pos[m] : 0;
+  }
+
   f32x16 acc[MT][NT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -437,7 +447,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     for (int mt = 0; mt < MT; ++mt) {
       int m = (mblock * MT + mt) * 32 + l32;
       if (m > a.M - 1) m = a.M - 1;
-      int pos = a.rope_pos[m];
+      int pos = rpos[mt];
       pos = pos < 0 ? 0 : (pos > a.rope_positions - 1 ? a.rope_positions - 1 : pos);
       e_rv[2 * mt] = *(const f32x4*)(a.rope_cos + (size_t)pos * a.rope_half + fi);
       e_rv[2 * mt + 1] = *(const f32x4*)(a.rope_sin + (size_t)pos * a.rope_half + fi);
