@@ -282,6 +282,9 @@ __global__ __launch_bounds__(kCrossWaves * 64) void expert_cross_px_kernel(AttnA
   const bool active = wave < nt;
   unsigned char* const ks = lds + (size_t)wave * 2 * kKTile;           // this wave's K tile: hi plane, then lo
 
+  // the rotary position of this lane's query row: asked for before anything else, so that its table rows can be
+  // requested with the other operands below instead of two round trips after the projection
+  int qpos = a.qp_rope_pos[qi < a.M ? qi : a.M - 1];
   // ---- requests in the order of use (memory returns in order): the block's 32 hidden rows and the norm weight
   // (16 threads per row, a thread's pieces requested together and kept in registers), the projection's weights,
   // then K / V^T (whole rows, lane -> consecutive chunks) ----
@@ -340,6 +343,12 @@ __global__ __launch_bounds__(kCrossWaves * 64) void expert_cross_px_kernel(AttnA
     vreg[0][i] = *(const i32x4*)(a.vt_pre + off);
     vreg[1][i] = *(const i32x4*)(a.vt_pre_lo + off);
   }
+  // the rotary table rows of the query (the lanes of waves 0..3 finish the projection: four consecutive columns
+  // 8 wave + 4 half .. of both halves of the head)
+  qpos = qpos < 0 ? 0 : (qpos > a.qp_positions - 1 ? a.qp_positions - 1 : qpos);
+  const int rfi = 8 * (wave & 3) + 4 * half;
+  const f32x4 rcs = *(const f32x4*)(a.qp_cos + (size_t)qpos * (D / 2) + rfi);
+  const f32x4 rsn = *(const f32x4*)(a.qp_sin + (size_t)qpos * (D / 2) + rfi);
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- the query tile: 1 / rms of its rows, normalised rows into LDS as bf16(w * bf16(x * rstd)), columns from K
@@ -421,11 +430,8 @@ __global__ __launch_bounds__(kCrossWaves * 64) void expert_cross_px_kernel(AttnA
 #pragma unroll
       for (int w = 1; w < NWV; ++w) sum[n2] += red[n2][w][wave][lane];
     }
-    const int fi = 8 * wave + 4 * half;  // first of this lane's four columns within the half head
-    int pos = a.qp_rope_pos[qi < a.M ? qi : a.M - 1];
-    pos = pos < 0 ? 0 : (pos > a.qp_positions - 1 ? a.qp_positions - 1 : pos);
-    const f32x4 cs = *(const f32x4*)(a.qp_cos + (size_t)pos * (D / 2) + fi);
-    const f32x4 sn = *(const f32x4*)(a.qp_sin + (size_t)pos * (D / 2) + fi);
+    const int fi = rfi;  // first of this lane's four columns within the half head
+    const f32x4 cs = rcs, sn = rsn;
     const f32x4 va = unpack_bf16x4(pack_bf16x4(sum[0])), vb = unpack_bf16x4(pack_bf16x4(sum[1]));
     f32x4 ra, rb;
 #pragma unroll
