@@ -90,6 +90,10 @@ class Weights:
     # bf16 = the reference's dtypes.  float32 = the same weight VALUES (bf16-rounded, fp8 codes) with every
     # activation kept in fp32: the yardstick that tells rounding noise of a bf16 execution order from error.
     act_dtype: torch.dtype = BF16
+    # not None: every linear sums its products in another order (the K dimension of activations and weights
+    # permuted alike, seeded) -- the same arithmetic and rounding points, mathematically the same result; what
+    # differs between two such runs is what any two executions of the reference's bf16 arithmetic may differ by
+    k_order_seed: int | None = None
 
     def __post_init__(self):
         if self.act_dtype != BF16:
@@ -113,11 +117,16 @@ class Weights:
         """``nn.Linear`` named ``prefix`` applied to ``x`` (bias if the state dict has one)."""
         w = self.sd[prefix + ".weight"]
         b = self.sd.get(prefix + ".bias")
+        perm = None
+        if self.k_order_seed is not None:
+            perm = torch.randperm(w.shape[1], generator=torch.Generator().manual_seed(self.k_order_seed + w.shape[1]))
+            x = x[..., perm]
         if prefix in self.fp8_names:
             q = self.quantised(prefix)
-            y = ops.lin_fp8w(x.reshape(-1, x.shape[-1]), q[0], q[1], self.act_dtype).reshape(*x.shape[:-1], w.shape[0])
+            w8 = q[0] if perm is None else q[0][:, perm]
+            y = ops.lin_fp8w(x.reshape(-1, x.shape[-1]), w8, q[1], self.act_dtype).reshape(*x.shape[:-1], w.shape[0])
             return y if b is None else y + b
-        return F.linear(x, w, b)
+        return F.linear(x, w if perm is None else w[:, perm], b)
 
 
 def fp8_linear_names(shape: SmolVLAShape, llm_mlp: bool, expert_mlp: bool) -> frozenset:
