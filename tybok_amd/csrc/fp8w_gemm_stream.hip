@@ -1,0 +1,364 @@
+// fp8-weight GEMM for at most 64 rows over a LARGE weight matrix (the weight-streaming launches):
+//   y[M,N] = bf16((x[M,K] . W8[N,K]^T) * scale[n])  (* gate[n]) (+ resid)
+//
+// Same packed weight tiles and the same arithmetic as fp8w_gemm_kernel; what differs is the schedule.  There a
+// round is a serial chain per wave (wait for x, write LDS, barrier, read LDS, convert, multiply) and the waves
+// split the k tiles four ways, so the accumulators of all four waves meet in a 128 KiB LDS exchange after the
+// loop.  Here
+//   * a block is four waves over a 64-column strip (two n tiles) and 64 rows; wave (nt, kh) owns n tile nt and
+//     the k tiles 2*kh, 2*kh+1 of every round of four -- both row tiles, so it holds two accumulator tiles and
+//     only TWO waves ever share an output tile: after the loop each wave hands one tile to its partner
+//     (16 KiB through LDS instead of 128) and finishes the other;
+//   * the loop is software-pipelined by hand around the matrix instructions: while the eight products of round r
+//     issue, the wave stages the activations of round r+1 into LDS, reads its operands of round r+1 back,
+//     converts the weight tiles of round r+1 and requests the tiles and activations of round r+PF -- one piece
+//     of that work behind each matrix instruction, fenced so the order stands.  One LDS barrier per round, in
+//     the middle of the round's products, so nobody waits at it with an empty matrix pipe;
+//   * the round count is a template parameter: straight-line code, exact wait counts, no tail conditions.
+// Fixed summation order (k tiles in order within a wave, kh = 0 before kh = 1, K splits in split order): the
+// same inputs give the same bits on every run.
+#include "tk_common.h"
+#include "tk_kernels.h"
+
+#ifdef TK_PHASE_TIMING
+// development aid (never built into the shipped library): per-block phase timestamps, 10 ns units
+__device__ long long tk_phase_stamps_s[4 * 8 * 8192];
+extern "C" int tk_debug_read_phases_s(void* host_out) {
+  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(tk_phase_stamps_s), sizeof(long long) * 4 * 8 * 8192);
+}
+#define SMARK(i)                                                                                   \
+  do {                                                                                             \
+    if (threadIdx.x == 0) {                                                                        \
+      const int b_ = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;               \
+      if (b_ < 8192) tk_phase_stamps_s[((a.act & 3) * 8192 + b_) * 8 + (i)] = wall_clock64();      \
+    }                                                                                              \
+  } while (0)
+#else
+#define SMARK(i)
+#endif
+
+namespace {
+
+// waits for this wave's LDS traffic only, not for its global loads in flight
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+#define SLOT_END() __builtin_amdgcn_sched_barrier(0)
+
+// rounds requested once iteration r is over: PRE up front, then at most two more per iteration until PF rounds
+// are in flight (a wave cannot stage round 0 before it has issued everything in front of that in program
+// order, and the memory pipeline takes requests only as fast as it completes them)
+constexpr int stream_issued(int r, int NR, int PF, int PRE) {
+  int t = PRE + 2 * (r + 1);
+  if (t > r + 1 + PF) t = r + 1 + PF;
+  return t > NR ? NR : t;
+}
+
+// NR: rounds of four k tiles every block walks (host: KT == ksplit * 4 * NR).  PF: rounds of loads in flight.
+// PRE: rounds requested before the first one is staged.
+template <int NR, int PF, int PRE>
+__global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
+  constexpr int ROWS = 64;
+  constexpr int PITCH = 4 * 64 + 16;  // LDS row pitch (bytes) of a round's 128 staged bf16 columns
+  constexpr int XBUF = ROWS * PITCH;
+  constexpr int NBUF = 3;             // staging ring: written one round ahead, read back in the same round
+  constexpr int XPT = 4;              // 16-byte pieces per thread and round (64 rows x 16 pieces / 256 threads)
+  constexpr int XSKIP = 3;            // pieces from this index on are requested only where the wave has live rows
+  static_assert(NR >= 2 && PF >= 2 && PF <= NR && PRE >= 1 && PRE <= PF, "pipeline shape");
+  __shared__ __align__(16) unsigned char lds[NBUF * XBUF];
+  __shared__ int s_last;
+
+  SMARK(0);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nt = wave & 1, kh = wave >> 1;
+  const int half = lane >> 5, l32 = lane & 31;
+  const int strip = blockIdx.x, split = blockIdx.y;
+  const int kt_lo = split * a.kt_q;
+
+  int ntg = strip * 2 + nt;
+  if (ntg > a.ntiles - 1) ntg = a.ntiles - 1;  // a strip may hang over the last n tile: its results are not stored
+  const uint8_t* wptr = a.w + ((size_t)ntg * a.KT + kt_lo + 2 * kh) * 1024 + lane * 16;
+
+  // the activations go through a buffer resource that ends with row M-1: the pieces of rows >= M are out of range,
+  // which returns zeros and asks the memory system for nothing (every block re-reads all the activations, so the
+  // dead rows of the second row tile would otherwise cost as much as live ones)
+  const __amdgpu_buffer_rsrc_t xres =
+      __builtin_amdgcn_make_buffer_rsrc((void*)a.x, 0, (int)(((size_t)(a.M - 1) * a.ldx + a.K) * 2), 0x00020000);
+  int xoff[XPT];
+  int xdst[XPT];
+  bool xlive[XPT];  // wave-uniform: piece i of this wave covers rows 16*i + 4*wave .. +3
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) xlive[i] = 16 * i + 4 * wave < a.M;
+#pragma unroll
+  for (int i = 0; i < XPT; ++i) {
+    const int row = (tid >> 4) + 16 * i, c = tid & 15;
+    xoff[i] = row < a.M ? (int)(((size_t)row * a.ldx + (size_t)kt_lo * 32 + c * 8) * 2) : 0x7f000000;
+    xdst[i] = row * PITCH + c * 16;
+  }
+  const int rd_off = l32 * PITCH + (2 * kh * 32 + 16 * half) * 2;  // this lane's operand bytes of k tile j = 0, row tile 0
+
+  f32x16 acc[2];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[mt][i] = 0.f;
+
+  i32x4 wg[PF][2];      // raw weight tiles in flight
+  i32x4 xg[PF][XPT];    // activation pieces in flight
+  i32x4 xa[2][2][2][2]; // operands [round parity][k tile j][row tile][16-byte chunk]
+  bf16x8 wb[2][2][2];   // converted weights [round parity][k tile j][chunk]
+
+  auto load_w = [&](int r) {
+    wg[r % PF][0] = *(const i32x4*)(wptr + (size_t)r * 4096);
+    wg[r % PF][1] = *(const i32x4*)(wptr + (size_t)r * 4096 + 1024);
+  };
+  auto load_x = [&](int r) {
+#pragma unroll
+    for (int i = 0; i < XPT; ++i)
+      if (i < XSKIP || xlive[i]) xg[r % PF][i] = __builtin_amdgcn_raw_buffer_load_b128(xres, xoff[i] + r * 256, 0, 0);
+  };
+  auto stage = [&](int r) {
+#pragma unroll
+    for (int i = 0; i < XPT; ++i)
+      if (i < XSKIP || xlive[i]) *(i32x4*)(lds + (r % NBUF) * XBUF + xdst[i]) = xg[r % PF][i];
+  };
+  auto read_ops = [&](int r, int j) {
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const i32x4* p = (const i32x4*)(lds + (r % NBUF) * XBUF + mt * 32 * PITCH + rd_off + j * 64);
+      xa[r & 1][j][mt][0] = p[0];
+      xa[r & 1][j][mt][1] = p[1];
+    }
+  };
+  auto convert = [&](int r, int j) {
+    wb[r & 1][j][0] = fp8x8_to_bf16x8(wg[r % PF][j][0], wg[r % PF][j][1]);
+    wb[r & 1][j][1] = fp8x8_to_bf16x8(wg[r % PF][j][2], wg[r % PF][j][3]);
+  };
+  auto product = [&](int r, int s) {  // product s of round r: k tile j, chunk h2, row tile mt
+    const int j = s >> 2, h2 = (s >> 1) & 1, mt = s & 1;
+    acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[r & 1][j][h2], as_bf16x8(xa[r & 1][j][mt][h2]), acc[mt], 0, 0, 0);
+  };
+
+  // every load of the first PF rounds, the weights of a round in front of its activations: the weight tiles
+  // come from HBM, the activations from the L2
+#pragma unroll
+  for (int p = 0; p < PRE; ++p) {
+    load_w(p);
+    load_x(p);
+  }
+  // the column scales of the tile this wave will finish (row tile kh, n tile nt): lane l of an accumulator tile
+  // owns activation row l % 32 and, in register i, output column 8*(i/4) + 4*(l/32) + i%4 -- four groups of four
+  // consecutive columns.  Requested here, so that nothing after the loop waits for memory.
+  const int n_base = (strip * 2 + nt) * 32 + 4 * half;
+  f32x4 e_sc[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    int n0 = n_base + 8 * g;
+    if (n0 > a.N - 4) n0 = a.N - 4;  // columns past N are never stored
+    e_sc[g] = *(const f32x4*)(a.s0 + n0);  // (unconditional: a branch here would drain the load queue)
+  }
+  SMARK(1);
+  stage(0);
+  lds_barrier();
+  read_ops(0, 0);
+  read_ops(0, 1);
+  convert(0, 0);
+  convert(0, 1);
+  SMARK(2);
+
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const bool nxt = r + 1 < NR;
+    const int i0 = r == 0 ? PRE : stream_issued(r - 1, NR, PF, PRE), i1 = stream_issued(r, NR, PF, PRE);
+    SLOT_END();
+    product(r, 0);
+    if (nxt) stage(r + 1);
+    SLOT_END();
+    product(r, 1);
+    SLOT_END();
+    if (nxt) lds_barrier();
+    SLOT_END();
+    product(r, 2);
+    if (nxt) read_ops(r + 1, 0);
+    SLOT_END();
+    product(r, 3);
+    if (nxt) read_ops(r + 1, 1);
+    SLOT_END();
+    product(r, 4);
+    if (nxt) convert(r + 1, 0);
+    SLOT_END();
+    product(r, 5);
+    if (nxt) convert(r + 1, 1);
+    SLOT_END();
+    product(r, 6);
+    if (i0 < i1) {
+      load_w(i0);
+      load_x(i0);
+    }
+    SLOT_END();
+    product(r, 7);
+    if (i0 + 1 < i1) {
+      load_w(i0 + 1);
+      load_x(i0 + 1);
+    }
+    SLOT_END();
+  }
+  SMARK(3);
+
+  // ---- the optional epilogue operands (gate, residual) of this wave's tile ----
+  const int m = kh * 32 + l32;
+  const int mc = m < a.M ? m : a.M - 1;
+  f32x4 e_rv[4];
+  i32x2 e_gate[4];
+  if (a.vec && (a.gate || a.resid)) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      int n0 = n_base + 8 * g;
+      if (n0 > a.N - 4) n0 = a.N - 4;
+      if (a.gate) e_gate[g] = *(const i32x2*)(a.gate + n0);
+      if (a.resid)
+        e_rv[g] = a.resid_f32 ? *(const f32x4*)((const float*)a.resid + (size_t)mc * a.ldr + n0)
+                              : unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)mc * a.ldr + n0));
+    }
+  }
+
+  // ---- the two waves of an n tile exchange one accumulator tile each: wave (nt, kh) keeps row tile kh ----
+  lds_barrier();  // every wave is done with the staging ring
+  f32x4 (*exch)[4][64] = (f32x4 (*)[4][64])lds;  // [wave][register group][lane]
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    f32x4 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = kh ? acc[0][4 * g + j] : acc[1][4 * g + j];
+    exch[wave][g][lane] = v;
+  }
+  lds_barrier();
+  f32x4 own[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const f32x4 got = exch[wave ^ 2][g][lane];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float mine = kh ? acc[1][4 * g + j] : acc[0][4 * g + j];
+      own[g][j] = kh ? got[j] + mine : mine + got[j];  // kh = 0 first, whichever wave adds
+    }
+  }
+
+  // ---- K-split reduction through global partials; the last-arriving block finishes ----
+  const int blk_lin = strip;
+  if (a.ksplit > 1) {
+    // partial layout: [(block, split)][wave][group][lane][4 floats], 8-byte device-coherent accesses
+    // (write-through, so the hand-off needs no cache flush)
+    unsigned long long* pbase = (unsigned long long*)a.partial + ((size_t)wave * 4 * 64 + lane) * 2;
+    {
+      unsigned long long* dst = pbase + ((size_t)blk_lin * a.ksplit + split) * 2048;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        st_agent64(dst + g * 128, own[g][0], own[g][1]);
+        st_agent64(dst + g * 128 + 1, own[g][2], own[g][3]);
+      }
+    }
+    handoff_publish();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (old == a.ksplit - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    handoff_acquire();
+    if (threadIdx.x == 0)  // leave the counter ready for the next launch
+      __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) own[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int SB = 8;  // splits whose partials are in flight together
+    for (int s0 = 0; s0 < a.ksplit; s0 += SB) {
+      unsigned long long raw[SB][4][2];
+#pragma unroll
+      for (int j = 0; j < SB; ++j) {
+        const int sj = s0 + j < a.ksplit ? s0 + j : a.ksplit - 1;
+        const unsigned long long* src = pbase + ((size_t)blk_lin * a.ksplit + sj) * 2048;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          raw[j][g][0] = ld_agent64(src + g * 128);
+          raw[j][g][1] = ld_agent64(src + g * 128 + 1);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < SB; ++j) {
+        if (s0 + j < a.ksplit) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            own[g][0] += __uint_as_float((unsigned)raw[j][g][0]);
+            own[g][1] += __uint_as_float((unsigned)(raw[j][g][0] >> 32));
+            own[g][2] += __uint_as_float((unsigned)raw[j][g][1]);
+            own[g][3] += __uint_as_float((unsigned)(raw[j][g][1] >> 32));
+          }
+        }
+      }
+    }
+  }
+  SMARK(6);
+
+  // ---- epilogue: this lane finishes row m, four groups of four columns ----
+  if (m < a.M) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int n0 = n_base + 8 * g;
+      if (n0 >= a.N) continue;
+      if (a.vec) {  // N % 4 == 0 and every row pitch / pointer allows 8-byte accesses
+        i32x2 r = pack_bf16x4(own[g] * e_sc[g]);
+        if (a.gate) r = pack_bf16x4(unpack_bf16x4(r) * unpack_bf16x4(e_gate[g]));
+        if (a.resid) r = pack_bf16x4(unpack_bf16x4(r) + e_rv[g]);
+        *(i32x2*)(a.y + (size_t)m * a.ldy + n0) = r;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int n = n0 + j;
+          if (n >= a.N) continue;
+          u16 r = f32_to_bf16_bits(own[g][j] * a.s0[n]);
+          if (a.gate) r = f32_to_bf16_bits(bf16_bits_to_f32(r) * bf16_bits_to_f32(a.gate[n]));
+          if (a.resid) {
+            const float rv = a.resid_f32 ? ((const float*)a.resid)[(size_t)m * a.ldr + n]
+                                         : bf16_bits_to_f32(((const u16*)a.resid)[(size_t)m * a.ldr + n]);
+            r = f32_to_bf16_bits(bf16_bits_to_f32(r) + rv);
+          }
+          a.y[(size_t)m * a.ldy + n] = r;
+        }
+      }
+    }
+  }
+  SMARK(7);
+}
+
+// Rounds of loads in flight, and how many of them are requested before the first round is staged.  Measured on
+// MI355X at the two 33.5 MB shapes (M = 50): 4 / 4 is the fastest of 3..8 / 2..6; fewer up front start the first
+// product earlier and finish the loop later.
+constexpr int kStreamPF = 4;
+constexpr int kStreamPRE = 4;
+
+}  // namespace
+
+// Rounds per block the kernel is built for (KT == ksplit * 4 * rounds); 0-terminated.
+static const int kStreamRounds[] = {16, 8, 0};
+
+bool tk_gemm_stream_takes(const GemmArgs& a) {
+  if (a.w16 || a.s1 != nullptr || a.rope_pos != nullptr || a.norm_w != nullptr || a.ada_scale != nullptr || a.x_f32) return false;
+  if (a.M > 64 || a.M < 1 || ((size_t)a.M * a.ldx + a.K) * 2 >= 0x7f000000ull || a.N < 64 || a.K % 32 != 0 || a.kt_r != 0 || a.kt_q % 4 != 0) return false;
+  for (const int* r = kStreamRounds; *r; ++r)
+    if (a.kt_q == 4 * *r) return true;
+  return false;
+}
+
+int tk_launch_gemm_stream(GemmArgs a, hipStream_t st) {
+  if (!tk_gemm_stream_takes(a)) return -1;
+  dim3 grid((a.ntiles + 1) / 2, a.ksplit, 1);
+  if (a.kt_q == 64) hipLaunchKernelGGL((fp8w_stream_kernel<16, kStreamPF, kStreamPRE>), grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((fp8w_stream_kernel<8, kStreamPF, kStreamPRE>), grid, dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}

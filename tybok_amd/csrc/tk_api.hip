@@ -236,14 +236,27 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   if (M > 64 && e.norm_w && !e.x_f32 && a.KT <= 32) MT = 1;
   if (M > 64 && M <= 256 && !e.x_f32 && (size_t)a.ntiles * 32 * a.KT * 32 * (e.w16 ? 2 : 1) <= (16u << 20)) MT = 1;
   int NT = 2;
-  if (!gated && !rope && ((a.ntiles + 1) / 2) * ((M + 32 * MT - 1) / (32 * MT)) < cus / 2) {
+  // 33..64 rows over a large fp8 matrix with the plain epilogue: the weight-streaming schedule (two-tile strips,
+  // every block 16 or 8 rounds of four k tiles) when a K split of that size about fills the device
+  int stream_ks = 0;
+  if (MT == 2 && M <= 64 && !gated && !rope && !e.w16 && !has_norm && !e.x_f32 && K % 32 == 0 && split_k <= 0) {
+    const int strips2 = (a.ntiles + 1) / 2;
+    for (int per = 64; per >= 32 && !stream_ks; per /= 2) {
+      if (a.KT % per) continue;
+      const int c = a.KT / per;
+      const size_t need = (size_t)strips2 * c * 4 * 4096;
+      const bool fits = c == 1 || (ws && strips2 <= kMaxCounters && need <= kPartialBytes && ws_bytes >= kPartialOff + need);
+      if (fits && c <= 64 && strips2 * c >= cus / 2 && strips2 * c <= 2 * cus) stream_ks = c;
+    }
+  }
+  if (!stream_ks && !gated && !rope && ((a.ntiles + 1) / 2) * ((M + 32 * MT - 1) / (32 * MT)) < cus / 2) {
     NT = 1;  // few columns: finer strips (the paired epilogues need both tiles of a strip in one wave)
   }
   const int mblocks = (M + 32 * MT - 1) / (32 * MT);
   const int strips = (a.ntiles + NT - 1) / NT;
   const int blocks0 = strips * mblocks;
   const int NW = 4;
-  int ks = split_k;
+  int ks = stream_ks ? stream_ks : split_k;
   if (ks <= 0) {
     // Launch-cost model (microseconds, fitted to graph-replayed launches on MI355X): the k loop costs
     // 0.35 per block round (NW k tiles) for 64-row blocks, 0.20 for 32-row blocks (0.27 with two bf16
@@ -285,7 +298,9 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
     a.counters = (int*)ws;
     if (e.clear_counters && tk_launch_fill_zero(a.counters, blocks0, st)) return fail(TK_ELAUNCH, "gemm: counter fill launch failed");
   }
-  int rc = tk_launch_gemm(a, MT, NT, mblocks, st);
+  // 33..64 rows over a large fp8 matrix: the weight-streaming schedule
+  const bool stream = MT == 2 && NT == 2 && mblocks == 1 && tk_gemm_stream_takes(a);
+  int rc = stream ? tk_launch_gemm_stream(a, st) : tk_launch_gemm(a, MT, NT, mblocks, st);
   if (rc == -1) return fail(TK_EINVAL, "gemm: this combination of weight type, prologue and epilogue is not built");
   if (rc) return fail(TK_ELAUNCH, "gemm: launch failed (%s)", hipGetErrorString(hipGetLastError()));
   return TK_OK;

@@ -210,6 +210,10 @@ int tk_wide_cols();  // columns of the many-row GEMM's block tile (rows: 32 * Ge
 int tk_launch_gemm_wide(GemmArgs a, hipStream_t st);
 int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st);
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st);
+// at most 64 rows over a large fp8 matrix, plain epilogue, every block 8 or 16 rounds of four k tiles: the
+// software-pipelined kernel of fp8w_gemm_stream.hip (same grid and partial layout as tk_launch_gemm with MT = NT = 2)
+bool tk_gemm_stream_takes(const GemmArgs& a);
+int tk_launch_gemm_stream(GemmArgs a, hipStream_t st);
 // W8A8 tier: per-token activation quantisation and the fp8 x fp8 many-row GEMM (block tile 32 * mtiles x tk_w8a8_cols())
 int tk_w8a8_cols();
 int tk_quant_act_max_k();
