@@ -172,10 +172,19 @@ int tk_w8a8_gemm(const void* a8, int lda, const void* sa, const void* w_packed, 
  *   (x8, sx) = quant(x);  g = w8a8(x8, Wg), u = w8a8(x8, Wu)  (bf16 each);  h = bf16(bf16(act(g)) * u);
  *   (h8, sh) = quant(h);  y = w8a8(h8, Wd)  (+ residual)
  * in four launches (quantise, gate/up with the gated epilogue, quantise, down); quantised copies and the [M, I]
- * intermediate live in the workspace.  Arguments as tk_fp8w_gated_ffn (no per-column gate). */
+ * intermediate live in the workspace.  Arguments as tk_fp8w_gated_ffn (no per-column gate).  quant_mode is the
+ * mode of tk_quant_act_rows for both quantisations: 1 is what `quantize_activation` / `_quant_act` compute
+ * (scale and quotient rounded to bf16 before the fp8 cast, triton_prefill_mlp.py:26-59,103-114), 0 keeps the
+ * scale and the quotient in fp32 (one rounding). */
 int tk_w8a8_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void* sg, const void* su, const void* wd_packed,
                       const void* sd, void* y, int ldy, const void* resid, int ldr, int resid_dtype, int M, int K, int I,
-                      int act, void* ws, size_t ws_bytes, void* stream);
+                      int act, int quant_mode, void* ws, size_t ws_bytes, void* stream);
+
+/* Byte offsets, inside the workspace, of what tk_w8a8_gated_ffn(M, K, I) leaves behind: the bf16 [M, I] intermediate
+ * h, its e4m3fn codes h8 [M, I] and their fp32 row scales [M] -- so a caller (or a test) can check the second
+ * quantisation and the down projection on exactly the operands the library used.  No counterpart in the
+ * reference, whose forward keeps `act`, `act_q` and `act_scale` as tensors (triton_prefill_mlp.py:157-161). */
+int tk_w8a8_ffn_layout(int M, int K, int I, size_t* h_off, size_t* h8_off, size_t* sh_off);
 
 /* ---- bf16-weight expert projections (norm prologue, rotary epilogue, residual epilogue) ----- */
 /* Bytes of a packed bf16 [N, K] weight (2 KiB per 32x32 tile). */

@@ -158,7 +158,9 @@ def _mlp(w: Weights, prefix: str, x):
 def _mlp_w8a8(w: Weights, prefix: str, x):
     """The W8A8 forward of one GeGLU MLP: both operands of every product in e4m3fn."""
     q = [w.quantised(prefix + n) for n in ("gate_proj", "up_proj", "down_proj")]
-    y = ops.gated_ffn_w8a8(x.reshape(-1, x.shape[-1]), *q[0], *q[1], *q[2], "gelu_tanh")
+    # activation quantisation as `quantize_activation` computes it: scale and quotient are bf16 values
+    # (tybok/policies/pi05/models/triton_prefill_mlp.py:26-59,103-114)
+    y = ops.gated_ffn_w8a8(x.reshape(-1, x.shape[-1]), *q[0], *q[1], *q[2], "gelu_tanh", mode="bf16")
     return y.reshape(*x.shape[:-1], y.shape[-1])
 
 

@@ -87,7 +87,7 @@ def _cases():
         dict(a8=P, lda=2048, sa=P, w=P, sw=P, y=P, ldy=16384, resid=None, ldr=0, rdt=0, M=712, N=16384, K=2048, split=0, ws=None, wsb=0, st=None), kw
     )
     w8ffn = lambda **kw: _args(  # noqa: E731
-        dict(x=P, ldx=2048, wgu=P, sg=P, su=P, wd=P, sd=P, y=P, ldy=2048, resid=None, ldr=0, rdt=0, M=712, K=2048, I=16384, act=1, ws=P, wsb=1 << 27, st=None), kw
+        dict(x=P, ldx=2048, wgu=P, sg=P, su=P, wd=P, sd=P, y=P, ldy=2048, resid=None, ldr=0, rdt=0, M=712, K=2048, I=16384, act=1, qm=1, ws=P, wsb=1 << 27, st=None), kw
     )
     dense = lambda **kw: _args(  # noqa: E731
         dict(x=P, ldx=768, w=P, bias=P, act=0, y=P, ldy=3072, resid=None, ldr=0, rdt=0, M=3072, N=3072, K=768, tile=0, split=0, ws=None, wsb=0, st=None), kw
@@ -107,6 +107,7 @@ def _cases():
         ("tk_w8a8_gemm", w8(N=16382), -1, "multiples of 4"),
         ("tk_w8a8_gemm", w8(split=4), -2, "partial space"),
         ("tk_w8a8_gated_ffn", w8ffn(act=9), -1, "unknown activation"),
+        ("tk_w8a8_gated_ffn", w8ffn(qm=2), -1, "unknown quantisation mode"),
         ("tk_bf16w_dense", dense(K=776, ldx=776), -1, "multiple of 16"),
         ("tk_bf16w_dense", dense(ldy=3076), -1, "multiple of 8"),
         ("tk_bf16w_dense", dense(act=3), -1, "act=3"),

@@ -589,8 +589,9 @@ int tk_w8a8_gemm(const void* a8, int lda, const void* sa, const void* w_packed, 
 
 int tk_w8a8_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void* sg, const void* su, const void* wd_packed,
                       const void* sd, void* y, int ldy, const void* resid, int ldr, int resid_dtype, int M, int K, int I,
-                      int act, void* ws, size_t ws_bytes, void* stream) {
+                      int act, int quant_mode, void* ws, size_t ws_bytes, void* stream) {
   if (act != TK_ACT_SILU && act != TK_ACT_GELU_TANH) return fail(TK_EINVAL, "w8a8 ffn: unknown activation %d", act);
+  if (quant_mode != 0 && quant_mode != 1) return fail(TK_EINVAL, "w8a8 ffn: unknown quantisation mode %d", quant_mode);
   if (M <= 0 || K <= 0 || I <= 0 || I % 32 || K % 16) return fail(TK_EINVAL, "w8a8 ffn: bad shape M=%d K=%d I=%d (K a multiple of 16, I of 32)", M, K, I);
   if (!sg || !su || !sd) return fail(TK_EINVAL, "w8a8 ffn: null scale pointer");
   if (!ws) return fail(TK_EWORKSPACE, "w8a8 ffn: needs a workspace");
@@ -608,13 +609,22 @@ int tk_w8a8_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void
   void* sh = base + kHiddenOff + (h_bytes + 255) / 256 * 256 + (h8_bytes + 255) / 256 * 256;
   if ((size_t)((char*)sh - base) + sa_bytes > ws_bytes) return fail(TK_EWORKSPACE, "w8a8 ffn: workspace too small for the intermediate");
   hipStream_t st = (hipStream_t)stream;
-  int rc = tk_quant_act_rows(x, ldx, a8, K, sa, M, K, 0, stream);
+  int rc = tk_quant_act_rows(x, ldx, a8, K, sa, M, K, quant_mode, stream);
   if (rc) return rc;
   rc = w8a8_common(a8, K, (const float*)sa, wgu_packed, (const float*)sg, (const float*)su, h, I, nullptr, 0, 0, M, I, K, 0, act, ws, ws_bytes, st);
   if (rc) return rc;
-  rc = tk_quant_act_rows(h, I, h8, I, sh, M, I, 0, stream);
+  rc = tk_quant_act_rows(h, I, h8, I, sh, M, I, quant_mode, stream);
   if (rc) return rc;
   return w8a8_common(h8, I, (const float*)sh, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, M, K, I, 0, 0, ws, ws_bytes, st);
+}
+
+int tk_w8a8_ffn_layout(int M, int K, int I, size_t* h_off, size_t* h8_off, size_t* sh_off) {
+  if (M <= 0 || K <= 0 || I <= 0 || !h_off || !h8_off || !sh_off) return fail(TK_EINVAL, "w8a8 ffn layout: bad argument");
+  const size_t h_bytes = (size_t)M * I * 2, h8_bytes = (size_t)M * I;
+  *h_off = kHiddenOff;
+  *h8_off = kHiddenOff + (h_bytes + 255) / 256 * 256;
+  *sh_off = *h8_off + (h8_bytes + 255) / 256 * 256;
+  return TK_OK;
 }
 
 size_t tk_bf16w_packed_bytes(int N, int K) {

@@ -54,8 +54,9 @@ SIGNATURES: dict[str, tuple] = {
     "tk_w8a8_gated_ffn": (
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
-         c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
+         c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
+    "tk_w8a8_ffn_layout": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "tk_bf16w_packed_bytes": (c_size_t, [c_int, c_int]),
     "tk_pack_bf16_weight": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tk_bf16w_linear": (

@@ -275,9 +275,13 @@ def w8a8_gemm(
 
 def w8a8_gated_ffn(
     x: torch.Tensor, wgu: PackedGateUp, wd: PackedWeight, act: str = "gelu_tanh", *, resid: torch.Tensor | None = None,
-    out: torch.Tensor | None = None, ws: Workspace | None = None,
+    out: torch.Tensor | None = None, ws: Workspace | None = None, mode: str = "fp32",
 ) -> torch.Tensor:  # fmt: skip
-    """The W8A8 MLP: quantise, gate/up with the gated epilogue, quantise, down (``+ residual``)."""
+    """The W8A8 MLP: quantise, gate/up with the gated epilogue, quantise, down (``+ residual``).  ``mode``: the
+    activation quantisation of both steps, ``"bf16"`` = the reference prefill's (scale and quotient rounded to bf16,
+    tybok/policies/pi05/models/triton_prefill_mlp.py:26-59), ``"fp32"`` = one rounding."""
+    if mode not in ("fp32", "bf16"):
+        raise ValueError(f"unknown quantisation mode {mode!r}")
     lib = native.lib()
     m, ldx = _check_act(x, wgu.k)
     if wd.k != wgu.i or wd.n != wgu.k:
@@ -288,10 +292,25 @@ def w8a8_gated_ffn(
     ws = ws or default_workspace(x.device)
     rc = lib.tk_w8a8_gated_ffn(
         x.data_ptr(), ldx, wgu.data.data_ptr(), wgu.scale_gate.data_ptr(), wgu.scale_up.data_ptr(), wd.data.data_ptr(),
-        wd.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt, m, wgu.k, wgu.i, ACT[act], ws.ptr, ws.nbytes, _stream(),
+        wd.scale.data_ptr(), out.data_ptr(), out.stride(0), rp, ldr, rdt, m, wgu.k, wgu.i, ACT[act], 1 if mode == "bf16" else 0,
+        ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip
     native.check(rc, "tk_w8a8_gated_ffn")
     return out
+
+
+def w8a8_ffn_intermediates(ws: Workspace, m: int, k: int, i: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Views of what the last :func:`w8a8_gated_ffn` of this shape left in ``ws``: the bf16 intermediate ``[m, i]``,
+    its e4m3fn codes ``[m, i]`` and their fp32 row scales ``[m]``."""
+    import ctypes
+
+    offs = [ctypes.c_size_t() for _ in range(3)]
+    native.check(native.lib().tk_w8a8_ffn_layout(m, k, i, *(ctypes.addressof(o) for o in offs)), "tk_w8a8_ffn_layout")
+    h_off, h8_off, sh_off = (int(o.value) for o in offs)
+    h = ws.buf[h_off : h_off + m * i * 2].view(torch.bfloat16).view(m, i)
+    h8 = ws.buf[h8_off : h8_off + m * i].view(torch.float8_e4m3fn).view(m, i)
+    sh = ws.buf[sh_off : sh_off + m * 4].view(torch.float32)
+    return h, h8, sh
 
 
 def pack_bf16_weight(w: torch.Tensor, rope_half: int = 0) -> PackedBf16Weight:

@@ -168,8 +168,9 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
             self.vit_mlp_dtype = torch.float16 if vit_mlp_dtype == "fp16" else torch.bfloat16
         self.tl_fused_expert = bool(tl_fused_expert)
         self.tl_fp8_llm_mlp = bool(tl_fp8_llm_mlp)
-        # tl_fp8_llm_mlp="w8a8": the reference tier's own arithmetic -- activations quantised per token, fp8 x fp8
-        # products (True keeps the activations in bf16: weight-only)
+        # tl_fp8_llm_mlp="w8a8": the reference tier's arithmetic -- activations quantised per token with the scale and
+        # the quotient rounded to bf16 (triton_prefill_mlp.py:26-59), fp8 x fp8 products; True keeps the activations
+        # in bf16 (weight-only).  The weight scales stay fp32 (the reference prefill computes them in bf16)
         self.fp8_llm_act = isinstance(tl_fp8_llm_mlp, str) and tl_fp8_llm_mlp.lower() == "w8a8"
         self.tl_fp8_expert_mlp = bool(tl_fp8_expert_mlp)
         self.model = PI05Model(

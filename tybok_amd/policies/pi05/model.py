@@ -396,7 +396,7 @@ class PI05Model:
             mlp = self.vlm_mlp[i]
             if mlp.w8a8:
                 normed = tk.rms_norm_rows(out, ada=norm_post, eps=EPS)
-                hidden = tk.w8a8_gated_ffn(normed, mlp.wgu, mlp.wd, "gelu_tanh", resid=out, ws=self.ws)
+                hidden = tk.w8a8_gated_ffn(normed, mlp.wgu, mlp.wd, "gelu_tanh", resid=out, ws=self.ws, mode="bf16")
             elif mlp.fp8:
                 hidden = tk.fp8w_gated_ffn(out, mlp.wgu, mlp.wd, "gelu_tanh", resid=out, ada=norm_post, eps=EPS, ws=self.ws)
             else:
