@@ -99,18 +99,33 @@ def test_zero_noise_chunk_within_bound():
     assert err <= 1e-2
 
 
+_FULL: dict = {}
+
+
+def _full_case(seed: int):
+    """Benchmark config 5 at full depth (18 + 18 layers, 27 vision layers, 2 cameras, 200 tokens, 10 steps, zero
+    noise), weights and inputs drawn from `seed`, with the CPU oracle's chunk in the reference's dtypes ("bf16"),
+    with every activation kept in fp32 ("fp32"), and in the reference's dtypes with every linear summing its k
+    range in another order ("reordered", two runs)."""
+    if seed not in _FULL:
+        cfg, sd, inp = cases.pi05_build(dict(cases.PI05_CASES["full"], seed=seed))
+        shape = _shape(cfg)
+        out = {"reordered": []}
+        for name, kw in (("bf16", dict(act_dtype=torch.bfloat16)), ("fp32", dict(act_dtype=torch.float32)), ("r1", dict(k_order_seed=1)), ("r2", dict(k_order_seed=2))):
+            w = Weights(sd, O.fp8_linear_names(shape, True, True), **kw)
+            with torch.no_grad():
+                y = O.sample_actions(w, shape, [i * 2.0 - 1.0 for i in inp["images"]], inp["img_masks"], inp["lang_tokens"], inp["lang_masks"], inp["noise"])
+            if name.startswith("r"):
+                out["reordered"].append(y)
+            else:
+                out[name] = y
+        _FULL[seed] = (cfg, sd, inp, out)
+    return _FULL[seed]
+
+
 @pytest.fixture(scope="module")
 def full_case():
-    """Benchmark config 5 at full depth (18 + 18 layers, 27 vision layers, 2 cameras, 200 tokens, 10 steps, zero
-    noise) with the CPU oracle's chunk in the reference's dtypes and with every activation kept in fp32."""
-    cfg, sd, inp = cases.pi05_build(cases.PI05_CASES["full"])
-    shape = _shape(cfg)
-    out = {}
-    for name, dt in (("bf16", torch.bfloat16), ("fp32", torch.float32)):
-        w = Weights(sd, O.fp8_linear_names(shape, True, True), act_dtype=dt)
-        with torch.no_grad():
-            out[name] = O.sample_actions(w, shape, [i * 2.0 - 1.0 for i in inp["images"]], inp["img_masks"], inp["lang_tokens"], inp["lang_masks"], inp["noise"])
-    return cfg, sd, inp, out
+    return _full_case(0)
 
 
 def _errs(a, b):
@@ -118,27 +133,52 @@ def _errs(a, b):
     return float(d.max()), float(d.mean())
 
 
+TEXT_TIERS = dict(fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True, fused_prefill=True)
+
+
+@pytest.mark.timeout(1500)
+def test_full_depth_zero_noise_chunk_against_oracle_and_noise_floor():
+    # `sample_actions` of the full-depth model (tybok/policies/pi05/models/flow_matching.py:761-838), three seeded
+    # frames (weights and inputs), fp8 + every text tier.  Same construction as the SmolVLA-shaped test: the stated
+    # bound (max-abs <= 1e-2) sits at the noise floor of a bf16 execution of 36 layers x 10 steps, and the test
+    # measures that floor twice instead of asserting it in prose --
+    #   * `fp32`: the oracle on the same weights with every activation in fp32; the reference-dtype oracle's distance
+    #     from it is what bf16 rounding alone costs;
+    #   * `reordered`: the oracle's own arithmetic with every linear's k range summed in another order (same
+    #     operations, same rounding points): the distance between two executions of the REFERENCE arithmetic.
+    # Held per frame: the HIP path is no farther from the fp32 run than the bf16 oracle is (x1.15 mean, x1.5 max: the
+    # maximum of 1600 values re-draws by +-25 % between equally good executions), no farther from the bf16 oracle
+    # than x1.5 (max) / x1.15 (mean) of the oracle's distance from its re-ordered self, and <= 1.25e-2 max / 3e-3
+    # mean in absolute terms.  Held over the three frames, so that one rounding flip does not decide: the median of
+    # the per-frame maxima <= 1e-2, the stated bound.
+    maxima = []
+    for seed in (0, 1, 2):
+        cfg, sd, inp, ref = _full_case(seed)
+        floor_max, floor_mean = _errs(ref["bf16"], ref["fp32"])
+        self_max = max(_errs(r, ref["bf16"])[0] for r in ref["reordered"])
+        self_mean = max(_errs(r, ref["bf16"])[1] for r in ref["reordered"])
+        got = _gpu_chunk(cfg, sd, inp, **TEXT_TIERS)
+        e_max, e_mean = _errs(got, ref["bf16"])
+        d_max, d_mean = _errs(got, ref["fp32"])
+        print(
+            f"pi05 full depth, seed {seed}, fp8 + every text tier: vs bf16 oracle {e_max:.4g} / {e_mean:.4g}; vs fp32-activation run "
+            f"{d_max:.4g} / {d_mean:.4g} (bf16 oracle: {floor_max:.4g} / {floor_mean:.4g}); the oracle in another summation order vs "
+            f"itself: {self_max:.4g} / {self_mean:.4g}; |chunk|max {float(ref['bf16'].abs().max()):.3g}"
+        )
+        assert torch.isfinite(got).all()
+        assert d_mean <= 1.15 * floor_mean and d_max <= 1.5 * floor_max
+        assert e_mean <= 1.15 * self_mean and e_max <= 1.5 * self_max
+        assert e_max <= 1.25e-2 and e_mean <= 3e-3
+        maxima.append(e_max)
+    assert sorted(maxima)[1] <= 1e-2, f"median of the per-frame maxima {sorted(maxima)} exceeds 1e-2"
+
+
 @pytest.mark.timeout(900)
-def test_full_depth_zero_noise_chunk_against_oracle_golden_and_noise_floor(full_case):
-    # `sample_actions` of the full-depth model (tybok/policies/pi05/models/flow_matching.py:761-838).
-    # Bounds as for the SmolVLA-shaped model: the stated 1e-2 sits at the noise floor of a bf16 execution of 36
-    # layers x 10 steps (the bf16 oracle itself is 1.1e-2 max / 2.1e-3 mean from the run that keeps every
-    # activation in fp32), so the HIP path is held to be no farther from that run than the bf16 oracle is
-    # (x1.15 mean, x1.5 max), and to 1.25e-2 max / 3e-3 mean against the bf16 oracle.
-    cfg, sd, inp, ref = full_case
-    floor_max, floor_mean = _errs(ref["bf16"], ref["fp32"])
-    print(f"pi05 full depth: bf16 oracle vs fp32-activation run {floor_max:.4g} / {floor_mean:.4g}, |chunk|max {float(ref['bf16'].abs().max()):.3g}")
-    text = dict(fused_expert=True, fp8_expert_mlp=True, fp8_llm_mlp=True, fused_prefill=True)
-    got = _gpu_chunk(cfg, sd, inp, **text)
-    e_max, e_mean = _errs(got, ref["bf16"])
-    d_max, d_mean = _errs(got, ref["fp32"])
-    print(f"pi05 full depth, fp8 + every text tier: vs bf16 oracle {e_max:.4g} / {e_mean:.4g}; vs fp32-activation run {d_max:.4g} / {d_mean:.4g}")
-    assert torch.isfinite(got).all()
-    assert d_mean <= 1.15 * floor_mean and d_max <= 1.5 * floor_max
-    assert e_max <= 1.25e-2 and e_mean <= 3e-3
+def test_full_depth_benched_tier_set_against_the_oracle(full_case):
     # the set the benchmark times adds the bf16 vision tier, a drift tier (its distance from the fp32 tower is
-    # part of the number): reported against the same oracle, bounded by twice the text tiers' bound
-    got_all = _gpu_chunk(cfg, sd, inp, **text, vit_mlp_dtype=torch.bfloat16, vit_lowp_attn=True)
+    # part of the number): reported against the oracle with the fp32 tower, bounded by twice the text tiers' bound
+    cfg, sd, inp, ref = full_case
+    got_all = _gpu_chunk(cfg, sd, inp, **TEXT_TIERS, vit_mlp_dtype=torch.bfloat16, vit_lowp_attn=True)
     a_max, a_mean = _errs(got_all, ref["bf16"])
     print(f"pi05 full depth, every tier incl. the bf16 vision tier: vs bf16 oracle (fp32 tower) {a_max:.4g} / {a_mean:.4g}")
     assert a_max <= 2.5e-2 and a_mean <= 6e-3

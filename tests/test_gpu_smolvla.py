@@ -130,6 +130,10 @@ def test_full_model_zero_noise_chunk_against_oracle_and_noise_floor(cameras):
             assert d_mean <= 1.15 * floor_mean and d_max <= 1.5 * floor_max
             assert e_mean <= 1.15 * self_mean and e_all <= 1.5 * self_max
             assert e_act <= 1.25e-2 and e_all <= 1.5e-2 and e_mean <= 3e-3
+            if cameras == 3 and seed == 0:
+                # the frame the benchmark times and reports under `parity` (measured 0.92e-2): the stated bound, on this
+                # one frame, so that a regression of the benchmarked configuration trips whatever the medians do
+                assert e_act <= 1e-2 and (name != "benched" or e_all <= 1e-2)
             maxima[name].append(e_all)
             chunk_maxima[name].append(e_act)
     for name, vals in maxima.items():
