@@ -646,8 +646,9 @@ def main() -> None:
         "data": "synthetic (random-init weights, uniform-noise images, random token ids, zero noise)",
         "config": {
             "workload": "SmolVLA-shaped predict_action_chunk: 16+16 layers, 3 cameras 512x512, 48 tokens, chunk 50, 10 Euler steps, fp8 MLP weights, fused expert + prefill tiers, hipGraph",
-            "inputs": "HBM-resident observation",
+            "inputs": "HBM-resident observation (value); the same request with the frame's tensors on the host, as the reference's harness hands them over (tybok/base.py:182-214), is smolvla_3cam_host_inputs_p50_ms",
             "graph": graph_ok,
+            "spin_up": "a loop of 4096^3 bf16 matmuls (60-150 ms) runs before every timed block so the clocks have left the idle state; it is outside every timed region",
         },
         "p95_ms": round(float(np.percentile(samples3, 95)), 3),
         "smolvla_2cam_p50_ms": round(float(np.percentile(samples2, 50)), 3),

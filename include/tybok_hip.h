@@ -106,8 +106,11 @@ int tk_fp8w_gemm(const void* x, int ldx, const void* w_packed, const void* scale
  * + 8 MiB of partials) that each GPU the library runs on holds until the process ends.
  *   Limits: M <= 64 (the action chunk); an explicit split_k whose partials exceed the 8 MiB is
  *   rejected with TK_EWORKSPACE; split_k = 0 never chooses more than fits.
- *   The first call on a device looks the array's address up (make it outside stream capture).  No
- *   call allocates, frees or synchronises.  All calls on one GPU share the one array: calls that
+ *   The first call on a device looks the array's address up; on a capturing stream that first call is
+ *   refused with TK_EINVAL -- tk_static_scratch_bytes() resolves the address for the current device, call
+ *   it (or run one launch) before capturing.  "Same bits" holds because the automatic split never needs
+ *   more than the 8 MiB here on a 256-CU device; a device with more CUs could pick another split under
+ *   tk_fp8w_gemm's larger workspace.  No call allocates, frees or synchronises.  All calls on one GPU share the one array: calls that
  *   may overlap in time (two streams, two threads) race -- serialise them or use tk_fp8w_gemm with
  *   one workspace per stream.  The counters a split launch uses are cleared by a fill kernel
  *   right before it, so a call does not depend on what the previous one left behind. */
@@ -413,7 +416,7 @@ int tk_expert_tail_embed(const void* x, int ldx, const void* norm_w, const void*
                          int K, const void* emb_w, const void* emb_b, int emb_n, int emb_act, void* emb_out, int emb_ld,
                          int emb_dtype, void* stream);
 
-/* ---- diagnostics ------------------------------------------------------------------------------- */
+/* ---- diagnostics: helpers of the tests and the benchmark; no policy path calls them -------------- */
 /* out_f32[256] = value of every e4m3fn code as decoded by the device's conversion instruction
  * (the weight path of the GEMM); used to assert the OCP (not FNUZ) flavour on the box. */
 int tk_debug_decode_fp8(void* out_f32, void* stream);

@@ -69,3 +69,30 @@ def test_static_scratch_rejects_what_it_cannot_hold():
     # the automatic choice stays inside the scratch and matches the workspace entry point
     got, want = _both(xg, w, 0)
     assert torch.equal(got, want)
+
+
+def test_static_scratch_split_launch_replays_in_a_graph():
+    # a K-split launch of the static entry point captured into a graph (the address lookup happened in the calls
+    # above or in tk_static_scratch_bytes(); the counters are cleared by a fill kernel, which a graph may hold):
+    # every replay gives the eager bits, with eager launches that reuse the scratch between the replays
+    lib = native.lib()
+    lib.tk_static_scratch_bytes()
+    x, w8, s = gemm_case(50, 4096, 1024)
+    w = tk.pack_fp8_weight(w8.cuda(), s)
+    xg = x.cuda()
+    eager, _ = _both(xg, w, 8)
+    out = torch.zeros(50, 1024, dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        st = torch.cuda.current_stream().cuda_stream
+        native.check(lib.tk_fp8w_gemm_static(xg.data_ptr(), 4096, w.data.data_ptr(), w.scale.data_ptr(), out.data_ptr(), 1024, None, 0, 0, None, 50, 1024, 4096, 8, st), "tk_fp8w_gemm_static")
+    x2, w82, s2 = gemm_case(16, 2048, 2048)
+    w2 = tk.pack_fp8_weight(w82.cuda(), s2)
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        got2, want2 = _both(x2.cuda(), w2, 4)  # eager work on the same scratch between the replays
+        assert torch.equal(got2, want2)

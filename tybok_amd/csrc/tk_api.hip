@@ -1,5 +1,6 @@
 // extern "C" entry points of libtybok_hip.so (declared in include/tybok_hip.h).
 // Host-side argument checks, launch geometry, workspace carving.  No allocation, no sync.
+#include <atomic>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -40,7 +41,7 @@ constexpr size_t kStaticBytes = kCounterBytes + kStaticPartialBytes;
 constexpr int kStaticMaxRows = 64;
 static __device__ __align__(256) unsigned char scratch[kStaticBytes];
 constexpr int kMaxDevices = 64;
-void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` per device ordinal, nullptr = not looked up yet
+std::atomic<void*> g_scratch_ptr[kMaxDevices];  // device address of `scratch` per device ordinal, nullptr = not looked up yet
 
 bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 bool aligned8(const void* p) { return (((uintptr_t)p) & 7) == 0; }
@@ -56,19 +57,27 @@ int device_cus() {
   return g_cus;
 }
 
-// Device address of this device's copy of `scratch` (looked up on the first call per device, with that
-// device current; concurrent first calls would store the same value twice).
-int static_scratch(void** out) {
+// Device address of this device's copy of `scratch`: looked up on the first call per device, with that device
+// current (concurrent first calls store the same value twice, atomically).  The lookup is a runtime call that
+// does not belong inside a stream capture: a first call on a capturing stream is refused instead -- call
+// tk_static_scratch_bytes() (which resolves the address for the current device) or run one launch before
+// capturing.
+int static_scratch(void** out, hipStream_t st, bool may_fail_capture) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
     return fail(TK_ELAUNCH, "static scratch: no current device (or ordinal >= %d)", kMaxDevices);
-  if (!g_scratch_ptr[dev]) {
-    void* p = nullptr;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (may_fail_capture) {
+      hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+      if (hipStreamIsCapturing(st, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+        return fail(TK_EINVAL, "gemm_static: first call on this device under stream capture (call tk_static_scratch_bytes() before capturing)");
+    }
     const hipError_t rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (rc != hipSuccess || !p) return fail(TK_ELAUNCH, "static scratch: hipGetSymbolAddress failed (%s)", hipGetErrorString(rc));
-    g_scratch_ptr[dev] = p;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
   }
-  *out = g_scratch_ptr[dev];
+  *out = p;
   return TK_OK;
 }
 
@@ -360,14 +369,19 @@ int tk_fp8w_gemm_static(const void* x, int ldx, const void* w_packed, const void
     return fail(TK_EINVAL, "gemm_static: M=%d exceeds the %d rows this entry point is built for (use tk_fp8w_gemm with a workspace)",
                 M, kStaticMaxRows);
   void* ws = nullptr;
-  if (int rc = static_scratch(&ws)) return rc;
+  if (int rc = static_scratch(&ws, (hipStream_t)stream, true)) return rc;
   GemmExtra e;
   e.clear_counters = 1;
   return gemm_common(x, ldx, w_packed, (const float*)scale, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, N, K, split_k,
                      0, ws, kStaticBytes, (hipStream_t)stream, e);
 }
 
-size_t tk_static_scratch_bytes(void) { return kStaticBytes; }
+size_t tk_static_scratch_bytes(void) {
+  // also resolves the array's address for the current device, so that no later call has to (stream capture)
+  void* p = nullptr;
+  (void)static_scratch(&p, nullptr, false);
+  return kStaticBytes;
+}
 
 int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void* sg, const void* su,
                       const void* wd_packed, const void* sd, void* y, int ldy, const void* resid, int ldr,

@@ -105,7 +105,10 @@ __device__ __forceinline__ unsigned long long ld_agent64(const unsigned long lon
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Ordering of such a hand-off.  The writer's partials are write-through stores, visible to every block once
+// Ordering of such a hand-off.  RULE: every byte one block hands to another is written with st_agent* and read
+// with ld_agent* -- a plain store would sit in this XCD's L2 and a plain load could hit a stale line there; the
+// scheme below orders the accesses, it does not make ordinary ones coherent.
+// The writer's partials are write-through stores, visible to every block once
 // the wave's memory counters have drained; handoff_publish() drains them and pins the compiler on both sides
 // (no memory access may be moved across it), and the arrival count that follows it publishes the data.  On the
 // reader's side handoff_acquire() pins the compiler between seeing the count and reading the partials (the

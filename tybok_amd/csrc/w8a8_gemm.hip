@@ -213,9 +213,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void w8a8_wide_kernel(GemmArgs a, int
         st_agent64(dst + 1, c[4 * g + 2], c[4 * g + 3]);
       }
     __shared__ int s_last;
-    asm volatile("" ::: "memory");
     handoff_publish();  // the write-through stores are acknowledged: visible to every block
-    asm volatile("" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
       int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -152,16 +152,21 @@ class SmolVLAModel:
             # and every linear of the tower in the tile order of the many-row MFMA kernel
             self.vis_qkv = []
             self.vis_dense: dict[str, tuple] = {}
+
+            def packed(w: torch.Tensor):
+                # the many-row kernel takes K % 16 == 0 and N % 8 == 0; another shape stays a plain linear
+                return tk.pack_bf16_weight(w) if w.shape[1] % 16 == 0 and w.shape[0] % 8 == 0 else w
+
             for i in range(cfg.vlm_config.vision_config.num_hidden_layers):
                 lp = f"{VIS}encoder.layers.{i}."
                 w = torch.cat([self.p[lp + "self_attn." + n + "_proj.weight"] for n in "qkv"], dim=0).contiguous()
                 b = torch.cat([self.p[lp + "self_attn." + n + "_proj.bias"] for n in "qkv"], dim=0).contiguous()
-                self.vis_qkv.append((tk.pack_bf16_weight(w), b))
+                self.vis_qkv.append((packed(w), b))
                 for n in ("self_attn.out_proj", "mlp.fc1", "mlp.fc2"):
-                    self.vis_dense[lp + n] = (tk.pack_bf16_weight(self.p[lp + n + ".weight"]), self.p[lp + n + ".bias"].contiguous())
+                    self.vis_dense[lp + n] = (packed(self.p[lp + n + ".weight"]), self.p[lp + n + ".bias"].contiguous())
             pw = self.p[VIS + "embeddings.patch_embedding.weight"]
-            self.vis_dense["patch"] = (tk.pack_bf16_weight(pw.reshape(pw.shape[0], -1).contiguous()), self.p[VIS + "embeddings.patch_embedding.bias"].contiguous())
-            self.vis_dense["connector"] = (tk.pack_bf16_weight(self.p[CONNECTOR + ".weight"]), self.p.get(CONNECTOR + ".bias"))
+            self.vis_dense["patch"] = (packed(pw.reshape(pw.shape[0], -1).contiguous()), self.p[VIS + "embeddings.patch_embedding.bias"].contiguous())
+            self.vis_dense["connector"] = (packed(self.p[CONNECTOR + ".weight"]), self.p.get(CONNECTOR + ".bias"))
         if self.fused_expert:
             self._pack_expert_projections()
             # V^T of the action tokens [G, D, chunk rounded up to 32]; the projection kernel writes
@@ -262,7 +267,7 @@ class SmolVLAModel:
                 # packed q|k|v GEMM, then the HIP attention (one problem per camera): q.K^T rounded to
                 # bf16 before the fp32 scale and softmax, exactly what the bf16 matmul below produces
                 w_qkv, b_qkv = self.vis_qkv[i]
-                qkv = tk.bf16w_dense(h.view(-1, h.shape[-1]), w_qkv, b_qkv, ws=self.ws).view(b, -1, 3, heads, hd)
+                qkv = self._dense_w(w_qkv, b_qkv, h).view(b, -1, 3, heads, hd)
                 vt = tk.transpose_v(qkv[:, :, 2])
                 a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, ws=self.ws)
                 x, h = tk.add_layer_norm(x, self._dense(lp + "self_attn.out_proj", a), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
@@ -294,6 +299,12 @@ class SmolVLAModel:
     def _dense(self, name: str, x: torch.Tensor, act: str | None = None) -> torch.Tensor:
         """A linear of the vision tower on the many-row MFMA kernel; ``x [..., K]`` bf16 -> ``[..., N]`` bf16."""
         w, bias = self.vis_dense[name]
+        return self._dense_w(w, bias, x, act)
+
+    def _dense_w(self, w, bias, x: torch.Tensor, act: str | None = None) -> torch.Tensor:
+        if isinstance(w, torch.Tensor):  # a shape the many-row kernel does not take: the same arithmetic in torch
+            y = F.linear(x, w, bias)
+            return F.gelu(y, approximate="tanh") if act else y
         return tk.bf16w_dense(x.reshape(-1, x.shape[-1]), w, bias, act, ws=self.ws).view(*x.shape[:-1], w.n)
 
     def embed_prefix(self, images, img_masks, lang_tokens, lang_masks, state):
