@@ -148,6 +148,23 @@ int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float nor
                            const void* resid, int ldr, int resid_dtype, const void* gate, int M, int K, int I,
                            int act, void* ws, size_t ws_bytes, void* stream);
 
+/* The action chunk's FFN (M <= 64, the expert shapes of both models) can run as ONE launch: its down blocks
+ * request their weights, then wait inside the kernel until the gate/up blocks their k range depends on have
+ * written their slices of the intermediate through and raised their flags -- the fusion `triton_norm_gate_up` +
+ * down (tybok/policies/smolvla/models/triton_mlp.py:30-144) and `triton_mlp_fp8_chain`
+ * (tybok/policies/pi05/models/triton_expert_mlp_fp8.py:438-469) stand for.  Same bits as the two-launch form,
+ * which every other shape takes.  On MI355X the hand-off between blocks of different XCDs costs more than the
+ * launch boundary it replaces (measured: 10.9 against 8.6 us per FFN), so the single-launch form is OFF unless
+ * asked for.  The three calls below have no counterpart in the reference:
+ *   tk_set_ffn_fusion(on): 1 runs the action chunk's FFN as one launch; returns the previous setting (default 0).
+ *   tk_set_handoff_spin(polls): how often a waiting block polls before it gives up (default 200000, about 0.1 s);
+ *     returns the previous value.  A block that gives up sets the workspace's sticky error word (int32 at byte
+ *     offset tk_workspace_handoff_error_offset()) and goes on, so the launch always ends; its output is then
+ *     undefined and the workspace must be re-initialised (tk_workspace_init) before the next call. */
+int tk_set_ffn_fusion(int on);
+int tk_set_handoff_spin(int polls);
+size_t tk_workspace_handoff_error_offset(void);
+
 /* ---- W8A8 tier: per-token activation quantisation + fp8 x fp8 GEMM (VLM prefill MLP) --------- */
 /* Per-token (per-row) activation quantisation to e4m3fn:
  *   sa[m] = max_k |x[m, k]| / 448 (fp32),  a8[m, k] = RNE(x[m, k] / sa[m]) computed in fp32, one rounding;

@@ -21,6 +21,21 @@
 #include "tk_kernels.h"
 
 
+#ifdef TK_PHASE_TIMING
+// development aid (never built into the shipped library): per-block phase timestamps of the single-launch FFN,
+// 10 ns units; [half][block][slot]
+__device__ long long tk_phase_stamps[2 * 1024 * 8];
+extern "C" int tk_debug_read_phases(void* host_out) {
+  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(tk_phase_stamps), sizeof(long long) * 2 * 1024 * 8);
+}
+#define TK_MARK(i)                                                                                                \
+  do {                                                                                                            \
+    if (FUSE != 0 && threadIdx.x == 0 && blockIdx.x < 1024) tk_phase_stamps[((FUSE - 1) * 1024 + blockIdx.x) * 8 + (i)] = wall_clock64(); \
+  } while (0)
+#else
+#define TK_MARK(i)
+#endif
+
 namespace {
 
 // LDS-only barrier: waits for this wave's LDS traffic, not for the global prefetch queue
@@ -40,8 +55,16 @@ __device__ __forceinline__ void lds_barrier() {
 //      bf16 input: bf16(w * bf16(x * rstd));  fp32 input: bf16(w * (x * rstd)).
 //  NR: number of block rounds when the host knows it (every block walks the same number of k tiles), else 0:
 //      with a constant count the pipeline below is straight-line code -- no tail conditions, exact wait counts.
-template <int MT, int NT, int NW, int EPI, int PF, int TPW, bool W16, int PRO, int NR = 0>
-__global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
+// FUSE: 0 a launch of its own.  1 / 2: the two halves of the single-launch gated FFN -- 1 is a gate/up block, which
+//      writes its 32 x 32 slice of the intermediate through to memory and raises its flag; 2 is a down block, which
+//      requests its first weight rounds, THEN waits (bounded) for the flags of the gate/up strips its k range
+//      covers, and reads their slices.  The intermediate is kept tile by tile -- slice (row block, strip) is 2 KiB
+//      of its own, [32 rows][32 columns] -- so every 128-byte line of it has ONE writer: a down block's plain loads
+//      then either miss in their L2 (nobody there touched the line since the launch began) and fetch what was
+//      written through, or hit the copy the writer's own write-through stores left in the same L2.
+// (strip, split, mblock): the block's position; nstrips: strips per row block (the arrival counters' pitch).
+template <int MT, int NT, int NW, int EPI, int PF, int TPW, bool W16, int PRO, int NR, int FUSE>
+__device__ __forceinline__ void gemm_block(const GemmArgs& a, const int strip, const int split, const int mblock, const int nstrips) {
   constexpr bool GATED = EPI == 1;
   // every round of the block in flight from the start (PF == NR) with the bf16 RMSNorm prologue: the staged pieces
   // stay in registers until the row statistics are known, so the statistics come from them -- no second pass over
@@ -67,12 +90,10 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   __shared__ __align__(16) unsigned char lds[LDS_BYTES];
   __shared__ float rstd_s[ROWS];
 
+  TK_MARK(0);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps k-tile indices scalar
-  const int strip = blockIdx.x;
-  const int split = blockIdx.y;
-  const int mblock = blockIdx.z;
   const int half = lane >> 5;
   const int l32 = lane & 31;
   // k tiles of this split: KT = ksplit * kt_q + kt_r, the first kt_r splits take one more (host-side
@@ -102,10 +123,14 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 #pragma unroll
   for (int i = 0; i < XPT; ++i) {
     const int p = tid + i * NW * 64;
-    const int r = p / PPR, c = p % PPR;
+    // FUSE == 2: consecutive threads walk a 2 KiB slice (k tile, row, 16-byte piece): whole lines per request
+    const int r = FUSE == 2 ? (p % 128) / 4 : p / PPR, c = FUSE == 2 ? (p / 128) * 4 + p % 4 : p % PPR;
     int m = mblock * ROWS + r;
     if (m > a.M - 1) m = a.M - 1;
-    xsrc[i] = (const char*)a.x + (size_t)m * a.ldx * (XF32 ? 4 : 2);
+    if (FUSE == 2)
+      xsrc[i] = (const char*)a.x + (((size_t)mblock * a.KT + kt_lo + c / 4) * 32 + r) * 64 + (c % 4) * 16;
+    else
+      xsrc[i] = (const char*)a.x + (size_t)m * a.ldx * (XF32 ? 4 : 2);
     xcol[i] = c * 8;
     xdst[i] = r * PITCH + c * 16;
     xrow[i] = r;
@@ -158,6 +183,8 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
         const i32x4* p = (const i32x4*)(xsrc[i] + (size_t)k * 4);
         f.v[i][0] = p[0];
         f.v[i][XF32 ? 1 : 0] = p[1];
+      } else if (FUSE == 2) {
+        f.v[i][0] = *(const i32x4*)(xsrc[i] + (size_t)r * (RKT * 2048));  // round r: RKT slices on
       } else {
         f.v[i][0] = *(const i32x4*)(xsrc[i] + (size_t)k * 2);
       }
@@ -280,7 +307,37 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   // valid tiles: a branch here would make the compiler's wait-count analysis assume, at the head
   // of the steady-state loop, that the first stage's loads might be the youngest in flight, and
   // drain the whole queue once per pass)
-  if (FULL) {
+  int fuse_ticket = -1;
+  if (FUSE == 2) {
+    static_assert(FUSE != 2 || (PRO == 0 && MT == 1), "the down half reads a finished intermediate, 32 rows of it");
+    // the weights do not depend on the other half: on their way before the wait
+#pragma unroll
+    for (int p = 0; p < PF; ++p) wload(wbuf[p], p);
+    if (wave == 0) {
+      // lanes poll the flags of the strips [kt_lo, kt_hi) -- the slices this block's k range reads
+      const int* flags = a.fuse + mblock * TK_FUSE_STRIPS;
+      bool ready = false;
+      for (int n = 0;; ++n) {
+        bool mine = true;
+        for (int sidx = kt_lo + lane; sidx < kt_hi; sidx += 64)
+          mine = mine && __hip_atomic_load(flags + sidx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+        ready = __builtin_amdgcn_ballot_w64(!mine) == 0;
+        if (ready || n >= a.fuse_spin) break;
+        __builtin_amdgcn_s_sleep(2);
+      }
+      if (!ready && lane == 0)  // gave up: say so (this launch's output is then undefined) and go on, so that the grid drains
+        __hip_atomic_store(a.fuse + TK_FUSE_ERROR, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    handoff_acquire();
+    TK_MARK(1);
+#pragma unroll
+    for (int p = 0; p < PF; ++p) xload(xbuf[p], p);
+    // count this block past its wait (behind the loads above: memory returns in order); the answer is looked at
+    // after the k loop
+    if (tid == 0) fuse_ticket = __hip_atomic_fetch_add(a.fuse + TK_FUSE_PAST + mblock, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    TK_MARK(2);
+  } else if (FULL) {
     // the activations first: memory returns in order, and the statistics below need every piece of the rows
 #pragma unroll
     for (int p = 0; p < PF; ++p) xload(xbuf[p], p);
@@ -380,6 +437,15 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
       }
     }
   }
+  TK_MARK(3);
+  if (FUSE == 2 && wave == 0) {
+    // the last down block of the row block to get past its wait leaves the flags and the count ready for the next launch
+    if (__builtin_amdgcn_readfirstlane(fuse_ticket) == a.fuse_consumers - 1) {
+      for (int sidx = lane; sidx < a.KT; sidx += 64)
+        __hip_atomic_store(a.fuse + mblock * TK_FUSE_STRIPS + sidx, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) __hip_atomic_store(a.fuse + TK_FUSE_PAST + mblock, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
   __syncthreads();  // staging buffers are dead; the reduction reuses the LDS
 
   // The accumulators hold C^T tiles: lane l of a tile owns activation row m = l % 32 and, in
@@ -476,7 +542,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
   }
 
   // ---- K-split reduction through global partials; the last-arriving block finishes ----
-  const int blk_lin = mblock * gridDim.x + strip;
+  const int blk_lin = mblock * nstrips + strip;
   if (a.ksplit > 1) {
     // partial layout: [(block, split)][tile][group][lane][4 floats], written and read as 8-byte
     // device-coherent accesses (write-through, so the hand-off needs no cache flush)
@@ -531,6 +597,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
     }
   }
 
+  TK_MARK(6);
   // ---- epilogue: this lane finishes row m (per m tile), columns n0 .. n0+3 of each n tile ----
   if (EPI == 0) {
 #pragma unroll
@@ -562,6 +629,7 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
         }
       }
     }
+    TK_MARK(7);
   } else if (EPI == 1) {
     // tiles come in (gate, up) pairs over the same logical columns; I % 32 == 0
     const int col = strip * 32 + ng;  // logical column in [0, I)
@@ -577,8 +645,23 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) act[j] = a.act == 0 ? silu_f(g[j]) : gelu_tanh_f(g[j]);
         act = unpack_bf16x4(pack_bf16x4(act));
-        *(i32x2*)(a.y + (size_t)m * a.ldy + col) = pack_bf16x4(act * up);
+        const i32x2 hv = pack_bf16x4(act * up);
+        if (FUSE == 1)  // slice (row block, strip), written through
+          __hip_atomic_store((unsigned long long*)(a.y + (((size_t)mblock * nstrips + strip) * 32 + l32) * 32 + ng),
+                             (unsigned long long)(unsigned)hv[0] | ((unsigned long long)(unsigned)hv[1] << 32), __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+        else
+          *(i32x2*)(a.y + (size_t)m * a.ldy + col) = hv;
       }
+    }
+    if (FUSE == 1) {
+      // this block's slice of the intermediate is written through: raise its flag
+      TK_MARK(4);
+      handoff_publish();
+      __syncthreads();
+      TK_MARK(5);
+      if (threadIdx.x == 0) __hip_atomic_store(a.fuse + mblock * TK_FUSE_STRIPS + strip, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      TK_MARK(7);
     }
   } else {
     // the two tiles of a strip hold columns (c, c + rope_half) of one head: logical tile of
@@ -630,6 +713,29 @@ __global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
         }
       }
     }
+  }
+}
+
+template <int MT, int NT, int NW, int EPI, int PF, int TPW, bool W16, int PRO, int NR = 0>
+__global__ __launch_bounds__(NW * 64) void fp8w_gemm_kernel(GemmArgs a) {
+  gemm_block<MT, NT, NW, EPI, PF, TPW, W16, PRO, NR, 0>(a, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.x);
+}
+
+// The gated FFN of the action chunk in ONE launch: blocks [0, nprod) are gate/up blocks (strip-major within a row
+// block), the rest down blocks (strip, K split, row block).  Blocks are dispatched in index order, so every gate/up
+// block is resident (or done) before a down block can wait for it; the wait is bounded all the same.
+//   G*: the gate/up half's <NW, PF, PRO, NR>;  D*: the down half's <NT, NW, PF, NR>.
+template <int GNW, int GPF, int GPRO, int GNR, int DNT, int DNW, int DPF, int DNR>
+__global__ __launch_bounds__((GNW > DNW ? GNW : DNW) * 64) void ffn_fused_kernel(GemmArgs g, GemmArgs d, int nprod, int gstrips, int dstrips) {
+  const int b = blockIdx.x;
+  if (b < nprod) {
+    if (GNW < DNW && threadIdx.x >= GNW * 64) return;
+    gemm_block<1, 2, GNW, 1, GPF, 1, false, GPRO, GNR, 1>(g, b % gstrips, 0, b / gstrips, gstrips);
+  } else {
+    if (DNW < GNW && threadIdx.x >= DNW * 64) return;
+    const int c = b - nprod;
+    const int strip = c % dstrips, rest = c / dstrips;
+    gemm_block<1, DNT, DNW, 0, DPF, 1, false, 0, DNR, 2>(d, strip, rest % d.ksplit, rest / d.ksplit, dstrips);
   }
 }
 
@@ -771,6 +877,33 @@ int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st) {
   if (pro) return -1;
   if (NT == 1) return MT == 1 ? launch<1, 1, 0, false, 0>(a, grid, nw, st) : launch<2, 1, 0, false, 0>(a, grid, nw, st);
   return MT == 1 ? launch<1, 2, 0, false, 0>(a, grid, nw, st) : launch<2, 2, 0, false, 0>(a, grid, nw, st);
+}
+
+int tk_launch_ffn_fused(GemmArgs g, GemmArgs d, int d_nt, int mblocks, hipStream_t st) {
+  // the same wave and round counts tk_launch_gemm would pick for the two launches (32-row blocks)
+  if (g.w16 || d.w16 || g.s1 == nullptr || g.rope_pos != nullptr || d.s1 != nullptr || d.rope_pos != nullptr || g.ada_scale != nullptr ||
+      g.x_f32 || d.norm_w != nullptr || d.ada_scale != nullptr || g.ksplit != 1 || g.kt_r != 0 || d.kt_r != 0 || mblocks > TK_FUSE_ROWBLOCKS || (g.ntiles + 1) / 2 > TK_FUSE_STRIPS ||
+      d.KT != (g.ntiles + 1) / 2)
+    return -1;
+  const int gpro = g.norm_w != nullptr ? 1 : 0;
+  const int gnw = (g.kt_q >= 48 || gpro == 1) ? 8 : 4, dnw = d.kt_q >= 48 ? 8 : 4;
+  const int gnr = (g.kt_q + gnw - 1) / gnw, dnr = (d.kt_q + dnw - 1) / dnw;
+  const int gstrips = (g.ntiles + 1) / 2, dstrips = (d.ntiles + d_nt - 1) / d_nt;
+  const int nprod = gstrips * mblocks;
+  const dim3 grid(nprod + dstrips * d.ksplit * mblocks);
+#define TK_FUSED(GNW, GPF, GPRO, GNR, DNT, DNW, DPF, DNR)                                                                              \
+  if (gnw == GNW && gpro == GPRO && gnr == GNR && d_nt == DNT && dnw == DNW && dnr == DNR) {                                           \
+    hipLaunchKernelGGL((ffn_fused_kernel<GNW, GPF, GPRO, GNR, DNT, DNW, DPF, DNR>), grid, dim3((GNW > DNW ? GNW : DNW) * 64), 0, st, g, \
+                       d, nprod, gstrips, dstrips);                                                                                    \
+    return hipGetLastError() == hipSuccess ? 0 : -3;                                                                                   \
+  }
+  // K = 720 with the RMSNorm prologue -> I = 2048 -> 720 (SmolVLA's expert), the same without the prologue, and
+  // K = 1024 -> I = 4096 -> 1024 with the down projection in four K splits (pi0.5's expert)
+  TK_FUSED(8, 3, 1, 3, 1, 8, kPF8, 8)
+  TK_FUSED(4, kPF, 0, 6, 1, 8, kPF8, 8)
+  TK_FUSED(4, kPF, 0, 8, 1, 4, kPF, 8)
+#undef TK_FUSED
+  return -1;
 }
 
 int tk_launch_pack_bf16(const void* w, void* out, int N, int K, int pair_off, hipStream_t st) {

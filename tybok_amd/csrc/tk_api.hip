@@ -30,7 +30,14 @@ constexpr size_t kNormOff = kPartialOff + kPartialBytes;
 constexpr size_t kNormBytes = 8ull << 20;  // normalised activations of a many-row GEMM
 constexpr size_t kHiddenOff = kNormOff + kNormBytes;
 constexpr size_t kHiddenBytes = TK_WS_TOTAL_BYTES - kHiddenOff;  // FFN [M, I] bf16 intermediate
-constexpr int kMaxCounters = (int)(kCounterBytes / 4);
+// the last TK_FUSE_WORDS int32 of the counter region belong to the single-launch FFN's hand-off
+constexpr int kMaxCounters = (int)(kCounterBytes / 4) - TK_FUSE_WORDS;
+constexpr size_t kFuseOff = (size_t)kMaxCounters * 4;
+// (off unless asked for: on MI355X the in-kernel hand-off -- write-through acknowledge, flag, poll round trip, first read of
+// the intermediate: 2.6 us from the last flag raised to the flags seen -- costs more than the launch boundary it
+// replaces; measured 10.9 against 8.6 us per FFN at (50, 720, 2048), 13.3 against 10.9 us at (50, 1024, 4096))
+std::atomic<int> g_ffn_fusion{0};          // tk_set_ffn_fusion
+std::atomic<int> g_handoff_spin{200000};   // tk_set_handoff_spin: polls a waiting block makes before it gives up
 
 // Scratch of tk_fp8w_gemm_static (callers that cannot allocate): arrival counters followed by split-K
 // partials, the head of the workspace layout above at a modest size.  Every device the library runs on
@@ -98,10 +105,17 @@ struct GemmExtra {
   int clear_counters = 0;  // zero the arrival counters a split launch uses right before it (shared static scratch)
 };
 
+// What gemm_common decided for a launch it was asked to plan instead of run.
+struct GemmPlan {
+  GemmArgs a;
+  int MT = 0, NT = 0, mblocks = 0;
+  bool skinny = false;  // fp8w_gemm_kernel (not the many-row or the weight-streaming kernel)
+};
+
 // One GEMM launch (plain, gated or rotary).  `N` is the logical output width.
 int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, const float* s1, void* y, int ldy,
                 const void* resid, int ldr, int resid_dtype, const void* gate, int M, int N, int K, int split_k,
-                int act, void* ws, size_t ws_bytes, hipStream_t st, const GemmExtra& e = GemmExtra()) {
+                int act, void* ws, size_t ws_bytes, hipStream_t st, const GemmExtra& e = GemmExtra(), GemmPlan* plan = nullptr) {
   if (M <= 0 || N <= 0 || K <= 0) return fail(TK_EINVAL, "gemm: non-positive shape M=%d N=%d K=%d", M, N, K);
   if (K % 16) return fail(TK_EINVAL, "gemm: K=%d must be a multiple of 16", K);
   if (ldx % 8 || ldx < K) return fail(TK_EINVAL, "gemm: ldx=%d must be >= K and a multiple of 8", ldx);
@@ -182,6 +196,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   if (!e.w16 && !rope && !e.x_f32 && a.vec && (M >= 256 || (M > 64 && wide_blocks >= cus)) &&
       (!has_norm || (ws && ws_bytes >= kNormOff + (size_t)M * K * 2 && (size_t)M * K * 2 <= kNormBytes))) {
     // many rows: MFMA-bound kernel with a 128 x 256 block tile
+    if (plan) return TK_OK;  // (plan->skinny stays false)
     if (has_norm) {
       NormRowsArgs nr;
       nr.x = (const u16*)x;
@@ -305,14 +320,54 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
       return fail(TK_EWORKSPACE, "gemm: workspace too small (need %zu partial bytes, %d counters)", need, blocks0);
     a.partial = (float*)((char*)ws + kPartialOff);
     a.counters = (int*)ws;
-    if (e.clear_counters && tk_launch_fill_zero(a.counters, blocks0, st)) return fail(TK_ELAUNCH, "gemm: counter fill launch failed");
+    if (!plan && e.clear_counters && tk_launch_fill_zero(a.counters, blocks0, st)) return fail(TK_ELAUNCH, "gemm: counter fill launch failed");
   }
   // 33..64 rows over a large fp8 matrix: the weight-streaming schedule
   const bool stream = MT == 2 && NT == 2 && mblocks == 1 && tk_gemm_stream_takes(a);
+  if (plan) {
+    plan->a = a;
+    plan->MT = MT;
+    plan->NT = NT;
+    plan->mblocks = mblocks;
+    plan->skinny = !stream;
+    return TK_OK;
+  }
   int rc = stream ? tk_launch_gemm_stream(a, st) : tk_launch_gemm(a, MT, NT, mblocks, st);
   if (rc == -1) return fail(TK_EINVAL, "gemm: this combination of weight type, prologue and epilogue is not built");
   if (rc) return fail(TK_ELAUNCH, "gemm: launch failed (%s)", hipGetErrorString(hipGetLastError()));
   return TK_OK;
+}
+
+// gate/up (+ norm prologue) -> h [M, I] in the workspace -> down (+ gate, residual).  The action chunk (at most 64
+// rows, 32-row blocks on both sides, a pair of shapes the fused kernel is built for) runs as ONE launch whose down
+// blocks wait for the gate/up blocks inside the kernel; everything else as two launches.  Same arithmetic and
+// summation order either way: the same bits.
+int ffn_launches(const void* x, int ldx, const GemmExtra& e, const void* wgu_packed, const void* sg, const void* su, void* hbuf,
+                 const void* wd_packed, const void* sd, void* y, int ldy, const void* resid, int ldr, int resid_dtype, const void* gate,
+                 int M, int K, int I, int act, void* ws, size_t ws_bytes, hipStream_t st) {
+  // (the fused form keeps the intermediate in 32-row slices: whole row blocks of it must fit)
+  if (M <= 64 && g_ffn_fusion.load(std::memory_order_relaxed) && ws_bytes >= kHiddenOff + (size_t)((M + 31) / 32) * 32 * I * 2) {
+    GemmPlan pg, pd;
+    int rc = gemm_common(x, ldx, wgu_packed, (const float*)sg, (const float*)su, hbuf, I, nullptr, 0, 0, nullptr, M, I, K, 0, act, ws,
+                         ws_bytes, st, e, &pg);
+    if (rc) return rc;
+    rc = gemm_common(hbuf, I, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, K, I, 0, 0, ws, ws_bytes, st,
+                     GemmExtra(), &pd);
+    if (rc) return rc;
+    if (pg.skinny && pd.skinny && pg.MT == 1 && pd.MT == 1 && pg.NT == 2 && pg.a.ksplit == 1 && pg.mblocks == pd.mblocks) {
+      int* fuse = (int*)((char*)ws + kFuseOff);
+      pg.a.fuse = pd.a.fuse = fuse;
+      pd.a.fuse_consumers = ((pd.a.ntiles + pd.NT - 1) / pd.NT) * pd.a.ksplit;
+      pd.a.fuse_spin = g_handoff_spin.load(std::memory_order_relaxed);
+      rc = tk_launch_ffn_fused(pg.a, pd.a, pd.NT, pg.mblocks, st);
+      if (rc == 0) return TK_OK;
+      if (rc != -1) return fail(TK_ELAUNCH, "ffn: launch failed (%s)", hipGetErrorString(hipGetLastError()));
+    }
+  }
+  int rc = gemm_common(x, ldx, wgu_packed, (const float*)sg, (const float*)su, hbuf, I, nullptr, 0, 0, nullptr, M, I, K, 0, act, ws,
+                       ws_bytes, st, e);
+  if (rc) return rc;
+  return gemm_common(hbuf, I, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, K, I, 0, 0, ws, ws_bytes, st);
 }
 
 }  // namespace
@@ -327,10 +382,14 @@ size_t tk_workspace_bytes(void) { return TK_WS_TOTAL_BYTES; }
 
 int tk_workspace_init(void* ws, size_t ws_bytes, void* stream) {
   if (!ws || ws_bytes < kCounterBytes) return fail(TK_EWORKSPACE, "workspace_init: need >= %zu bytes", kCounterBytes);
-  if (tk_launch_fill_zero((int*)ws, kMaxCounters, (hipStream_t)stream))
+  if (tk_launch_fill_zero((int*)ws, (int)(kCounterBytes / 4), (hipStream_t)stream))
     return fail(TK_ELAUNCH, "workspace_init: launch failed");
   return TK_OK;
 }
+
+int tk_set_ffn_fusion(int on) { return g_ffn_fusion.exchange(on ? 1 : 0); }
+int tk_set_handoff_spin(int polls) { return g_handoff_spin.exchange(polls < 0 ? 0 : polls); }
+size_t tk_workspace_handoff_error_offset(void) { return kFuseOff + (size_t)TK_FUSE_ERROR * 4; }
 
 size_t tk_fp8w_packed_bytes(int N, int K) {
   if (N <= 0 || K <= 0) return 0;
@@ -397,12 +456,8 @@ int tk_fp8w_gated_ffn(const void* x, int ldx, const void* wgu_packed, const void
     return fail(TK_EWORKSPACE, "ffn: workspace too small for the [%d, %d] intermediate", M, I);
   void* hbuf = (char*)ws + kHiddenOff;
   // gate/up + activation-multiply -> h[M, I] (bf16, workspace)
-  int rc = gemm_common(x, ldx, wgu_packed, (const float*)sg, (const float*)su, hbuf, I, nullptr, 0, 0, nullptr, M, I, K, 0,
-                       act, ws, ws_bytes, (hipStream_t)stream);
-  if (rc) return rc;
-  // down projection (+ residual)
-  return gemm_common(hbuf, I, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, K, I, 0, 0,
-                     ws, ws_bytes, (hipStream_t)stream);
+  return ffn_launches(x, ldx, GemmExtra(), wgu_packed, sg, su, hbuf, wd_packed, sd, y, ldy, resid, ldr, resid_dtype, gate, M, K, I, act, ws,
+                      ws_bytes, (hipStream_t)stream);
 }
 
 // ---- W8A8 tier ---------------------------------------------------------------------------------
@@ -705,11 +760,8 @@ int tk_fp8w_norm_gated_ffn(const void* x, int ldx, const void* norm_w, float nor
   e.norm_eps = norm_eps;
   e.ada_scale = ada_scale;
   e.ada_shift = ada_shift;
-  int rc = gemm_common(x, ldx, wgu_packed, (const float*)sg, (const float*)su, hbuf, I, nullptr, 0, 0, nullptr, M, I, K, 0,
-                       act, ws, ws_bytes, (hipStream_t)stream, e);
-  if (rc) return rc;
-  return gemm_common(hbuf, I, wd_packed, (const float*)sd, nullptr, y, ldy, resid, ldr, resid_dtype, gate, M, K, I, 0, 0,
-                     ws, ws_bytes, (hipStream_t)stream);
+  return ffn_launches(x, ldx, e, wgu_packed, sg, su, hbuf, wd_packed, sd, y, ldy, resid, ldr, resid_dtype, gate, M, K, I, act, ws, ws_bytes,
+                      (hipStream_t)stream);
 }
 
 int tk_attn_prepare_kv(const void* k, const void* v, int kv_dtype, int sl, int sh, int L, int G, int D, void* k_hi,

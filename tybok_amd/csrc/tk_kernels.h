@@ -55,7 +55,18 @@ struct GemmArgs {
   const unsigned short* bias;
   // many-row fp8 kernels: 32-row tiles per block (2 or 4), chosen by the host
   int mtiles;
+  // single-launch gated FFN only: the hand-off words in the workspace (TK_FUSE_* below), the down blocks per row
+  // block, and the bound on a down block's wait (polls)
+  int* fuse;
+  int fuse_consumers, fuse_spin;
 };
+// int32 words of the single-launch FFN's hand-off: a flag per (row block, gate/up strip), the number of down blocks
+// past their wait per row block, then the sticky error word
+#define TK_FUSE_ROWBLOCKS 2
+#define TK_FUSE_STRIPS 512
+#define TK_FUSE_PAST (TK_FUSE_ROWBLOCKS * TK_FUSE_STRIPS)
+#define TK_FUSE_ERROR (TK_FUSE_PAST + TK_FUSE_ROWBLOCKS)
+#define TK_FUSE_WORDS 2048
 
 struct QuantActArgs {
   const unsigned short* x;  // bf16 [M, K], element pitch ldx
@@ -210,6 +221,9 @@ int tk_wide_cols();  // columns of the many-row GEMM's block tile (rows: 32 * Ge
 int tk_launch_gemm_wide(GemmArgs a, hipStream_t st);
 int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st);
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st);
+// the action chunk's gated FFN in one launch (32-row blocks; g: the gate/up half without a K split, d: the down half
+// with NT n tiles per strip); -1 when the pair of shapes is not one of the built combinations
+int tk_launch_ffn_fused(GemmArgs g, GemmArgs d, int d_nt, int mblocks, hipStream_t st);
 // at most 64 rows over a large fp8 matrix, plain epilogue, every block 8 or 16 rounds of four k tiles: the
 // software-pipelined kernel of fp8w_gemm_stream.hip (same grid and partial layout as tk_launch_gemm with MT = NT = 2)
 bool tk_gemm_stream_takes(const GemmArgs& a);

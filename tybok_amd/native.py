@@ -45,6 +45,9 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
          c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),  # fmt: skip
+    "tk_set_ffn_fusion": (c_int, [c_int]),
+    "tk_set_handoff_spin": (c_int, [c_int]),
+    "tk_workspace_handoff_error_offset": (c_size_t, []),
     "tk_quant_act_rows": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tk_w8a8_gemm": (
         c_int,

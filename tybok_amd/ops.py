@@ -42,6 +42,15 @@ class Workspace:
     def ptr(self) -> int:
         return self.buf.data_ptr()
 
+    def reset(self) -> None:
+        """Zero every arrival counter and the hand-off error word (after a launch that gave up waiting)."""
+        native.check(native.lib().tk_workspace_init(self.buf.data_ptr(), self.nbytes, _stream()), "tk_workspace_init")
+
+    def handoff_error(self) -> bool:
+        """Whether a block of the single-launch FFN has given up its bounded wait since the last reset (synchronises)."""
+        off = int(native.lib().tk_workspace_handoff_error_offset())
+        return bool(self.buf[off : off + 4].view(torch.int32).item())
+
 
 _default_ws: dict[int, Workspace] = {}
 
@@ -234,6 +243,16 @@ def fp8w_gated_ffn(
     )  # fmt: skip
     native.check(rc, "tk_fp8w_gated_ffn")
     return out
+
+
+def set_ffn_fusion(on: bool) -> bool:
+    """Single-launch FFN for the action chunk on / off (the default: two launches everywhere); returns the previous setting."""
+    return bool(native.lib().tk_set_ffn_fusion(1 if on else 0))
+
+
+def set_handoff_spin(polls: int) -> int:
+    """Bound (polls) of the wait inside the single-launch FFN; returns the previous value."""
+    return int(native.lib().tk_set_handoff_spin(int(polls)))
 
 
 def quant_act_rows(x: torch.Tensor, mode: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
