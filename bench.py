@@ -519,12 +519,12 @@ def main() -> None:
     torch.cuda.empty_cache()
 
     # ---- pi0.5-shaped chunk ----
-    pi05_p50 = pi05_w8a8_p50 = None
+    pi05_p50 = pi05_w8a8_p50 = pi05_mlp_tier_p50 = None
     if not args.skip_pi05:
         ckpt5 = write_pi05_checkpoint(os.path.join(tmp, "pi05"), cameras=2, seed=0)
         flags5 = {k: v for k, v in flags.items() if k not in ("tl_llm_fused_attn", "tl_vit_oproj")}  # SmolVLA-only tiers
         flags5["tl_llm_flash_attn"] = True  # pi0.5's name for the fused prefill
-        flags5["tl_fused_vit"] = True  # SigLIP linears in bf16 (the reference's drift tier of the same name)
+        flags5["tl_fused_vit"] = True  # the reference's fused tower: fp16 q|k|v and attention, bf16 out_proj and MLP
         eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **flags5)
         frame5 = device_frame(eng5, 2)
         s5, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
@@ -536,6 +536,13 @@ def main() -> None:
         eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **{**flags5, "tl_fp8_llm_mlp": "w8a8"})
         s5w, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
         pi05_w8a8_p50 = float(np.percentile(s5w, 50))
+        del eng5
+        torch.cuda.empty_cache()
+        # and with the vision tower on the tier that a fixture from the reference's own tower pins end to end: fp32
+        # attention and norms, only fc1 / fc2 in bf16 (--vit-mlp-dtype bf16) on the many-row kernel
+        eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **{**flags5, "tl_fused_vit": False, "vit_mlp_dtype": "bf16"})
+        s5m, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
+        pi05_mlp_tier_p50 = float(np.percentile(s5m, 50))
         del eng5
         torch.cuda.empty_cache()
 
@@ -656,6 +663,7 @@ def main() -> None:
         "pi05_2cam_p50_ms": None if pi05_p50 is None else round(pi05_p50, 3),
         "pi05_tiers": "tl_fused_expert, tl_fp8_expert_mlp, tl_fp8_llm_mlp, tl_llm_flash_attn, tl_fused_vit",
         "pi05_2cam_w8a8_prefill_p50_ms": None if pi05_w8a8_p50 is None else round(pi05_w8a8_p50, 3),
+        "pi05_2cam_vit_mlp_bf16_tier_p50_ms": None if pi05_mlp_tier_p50 is None else round(pi05_mlp_tier_p50, 3),
         "gemm_sweep_M50": sweep,
         "ops_action_chunk_shape": ops_small,
         "pi05_prefill_ffn_M712": prefill_ffn,

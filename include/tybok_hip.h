@@ -274,6 +274,15 @@ int tk_bf16w_dense(const void* x, int ldx, const void* w_packed, const void* bia
                    const void* resid, int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws,
                    size_t ws_bytes, void* stream);
 
+/* tk_bf16w_dense with every 16-bit operand in IEEE fp16 instead of bf16 (x, the packed weight -- tk_pack_bf16_weight
+ * moves 16-bit words and serves both --, bias, y and a TK_BF16-typed residual, which is then read as fp16), on
+ * `v_mfma_f32_32x32x16_f16`: the fp16 GEMMs of pi0.5's vision tower -- the `--vit-mlp-dtype fp16` tier
+ * (tybok/policies/pi05/models/vision.py:79-87,223-235) and the fused tier's q|k|v projection
+ * (`_vision_qkv_kernel`, tybok/policies/pi05/models/triton_vision.py:38-110: fp16 operands, fp32 accumulate). */
+int tk_f16w_dense(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy,
+                   const void* resid, int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws,
+                   size_t ws_bytes, void* stream);
+
 /* ---- action-expert attention over the cached prefix ------------------------------------------ */
 /* Lays one layer's prefix K/V out for tk_expert_attn, once per request (the counterpart of the
  * reference filling its static per-layer prefix cache after the VLM prefill,
@@ -352,7 +361,10 @@ int tk_expert_cross_attn_fused(const void* x, int ldx, const void* norm_w, float
  * operands of tk_expert_attn (K [P, G, D]; V^T [G, D, >= P rounded up to 32], zero padded), with
  * element strides q_sb / k_sb / vt_sb / out_sb between problems.  logits_bf16 = 1 rounds q.K^T to
  * bf16 before the fp32 scale and softmax, as a bf16 matmul followed by `.float() * scale` does
- * (tybok/policies/smolvla/models/vision.py:197-257).  scale > 0 replaces D^-0.5: a head whose true
+ * (tybok/policies/smolvla/models/vision.py:197-257).  logits_bf16 = 2: q, K and V^T hold IEEE fp16 values
+ * and the probabilities are rounded to fp16 for P.V, both products on the fp16 matrix instruction with fp32
+ * logits and accumulation, bf16 output -- `_vision_attn_kernel` of pi0.5's fused tower
+ * (tybok/policies/pi05/models/triton_vision.py:248-326); built for D = 96 and >= 128 queries and keys.  scale > 0 replaces D^-0.5: a head whose true
  * size is not supported (SigLIP-So400m: 72) is padded with zero columns to the next D and passes
  * 72^-0.5 (tybok/policies/pi05/models/vision.py:52-66); scale = 0 keeps the default. */
 int tk_batched_attn(const void* q, long long q_sb, int q_sm, int q_sh, const void* k, long long k_sb, int k_sl, int k_sh,
@@ -404,6 +416,16 @@ int tk_layer_norm(const void* x, int ldx, int x_dtype, const void* w, const void
  * tybok/policies/smolvla/models/vision.py:197-257, tybok/policies/pi05/models/vision.py:115-170). */
 int tk_add_layer_norm(const void* x, int ldx, int x_dtype, const void* r, int ldr, void* xsum, int ldxs, const void* w,
                       const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream);
+
+/* tk_layer_norm for fp32 rows and fp32 parameters with the normalised row rounded to IEEE fp16 instead of bf16:
+ * the LayerNorm + cast in front of the fp16 q|k|v projection of pi0.5's fused tower (`n.to(tl.float16)`,
+ * tybok/policies/pi05/models/triton_vision.py:93-95) and of the `--vit-mlp-dtype fp16` MLP
+ * (tybok/policies/pi05/models/vision.py:79-87). */
+int tk_layer_norm_f16(const void* x, int ldx, const void* w, const void* b, float eps, void* y, int ldy, int M, int K,
+                      void* stream);
+/* tk_add_layer_norm for fp32 rows and parameters (bf16 residual branch) with the normalised row rounded to fp16. */
+int tk_add_layer_norm_f16(const void* x, int ldx, const void* r, int ldr, void* xsum, int ldxs, const void* w, const void* b,
+                          float eps, void* y, int ldy, int M, int K, void* stream);
 
 /* ---- tail of a denoising step ---------------------------------------------------------------- */
 /* Final norm of the expert hidden state + fp32 action projection + Euler update in one launch:

@@ -61,13 +61,19 @@ class PI05Shape:
     #   vit_mlp_dtype: fc1 / gelu / fc2 run in that dtype, cast at the boundary (vision.py:79-87); pinned by a
     #                  fixture written from the reference's own tower after set_mlp_dtype
     #                  (tests/golden/pi05_small_vit_tiers.npz);
-    #   vit_lowp_attn: q/k/v and out_proj run in bf16 too; attention scores and softmax in fp32, the
-    #                  probabilities rounded to bf16 for P.V (fp32 accumulate, bf16 result).  PARITY UNPINNED:
-    #                  this restates the HIP backend's own tier, not the reference's fused tower kernels
-    #                  (vision.py:116-173 run q|k|v in fp16 on Triton kernels that cannot run here); it is a
-    #                  regression check of that tier, bounded against the fp32 tower, not a parity claim.
     vit_mlp_dtype: torch.dtype | None = None
-    vit_lowp_attn: bool = False
+    #   vit_fused: the reference's fused tower (``--tl-fused-vit``), restated from its kernels' source
+    #                  (tybok/policies/pi05/models/triton_vision.py): LayerNorm in fp32; q|k|v from fp16 operands with
+    #                  fp32 accumulation, kept as fp16; fp32 logits and softmax, probabilities rounded to fp16 for P.V,
+    #                  bf16 attention output; out_proj, fc1, fc2 and the projector from bf16 operands with fp32
+    #                  accumulation and fp32 results; tanh-GELU on the fp32 pre-activation, rounded to bf16 for fc2;
+    #                  residuals in fp32.  The fp16 half (LayerNorm + q|k|v + attention) is pinned by a fixture written
+    #                  from those kernels through Triton's CPU interpreter (tests/golden/pi05_small_vit_fused.npz).
+    #                  The bf16 kernels (out_proj, MLP, projector) are restated from source only -- that interpreter
+    #                  multiplies bf16 operands as raw integers and has no libdevice tanh -- PARITY UNPINNED for them;
+    #                  what they compute (a 16-bit-operand linear with an fp32 accumulator, the tanh-GELU) is pinned
+    #                  as arithmetic by the closed-form tests of oracle/ops.py.
+    vit_fused: bool = False
     # W8A8 tier of the VLM MLP (tybok/policies/pi05/models/triton_prefill_mlp.py:145-166): activations quantised
     # per token as well; only with the VLM MLP's weights in fp8 (``fp8_linear_names(..., llm_mlp=True, ...)``)
     llm_w8a8: bool = False
@@ -84,6 +90,62 @@ def fp8_linear_names(shape: PI05Shape, llm_mlp: bool, expert_mlp: bool) -> froze
     return frozenset(names)
 
 
+def _lin16(t: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, dt: torch.dtype) -> torch.Tensor:
+    """``t . weight^T + bias`` with every operand rounded to the 16-bit type ``dt``, fp32 products and accumulation,
+    fp32 result -- what a 16-bit matrix instruction with an fp32 accumulator computes, up to summation order."""
+    return t.to(dt).float() @ weight.to(dt).float().t() + bias.to(dt).float()
+
+
+def vit_fused_qkv_attention(w: Weights, shape: PI05Shape, layer: int, x: torch.Tensor):
+    """The fp16 half of an attention block of the reference's fused tower: ``x [B, L, C]`` fp32 ->
+    ``(q, k, v)`` fp32 ``[B, H, L, hd]`` as the projection kernel stores them and the attention output bf16
+    ``[B, H, L, hd]`` (`_fused_qkv`, tybok/policies/pi05/models/vision.py:133-156; `_vision_qkv_kernel`,
+    `_vision_attn_kernel`, triton_vision.py:38-110, 248-326): LayerNorm in fp32, the normalised row and the
+    weights as fp16, fp32 accumulation; q, k, v rounded to fp16 by the attention kernel; fp32 logits and softmax;
+    exp(s - max) rounded to fp16 for P.V; the normalised result rounded to bf16.  The kernel walks the keys in
+    blocks with a running maximum; this is the same computation with all keys in one block."""
+    p = f"{VIS}encoder.layers.{layer}."
+    b, hd = x.shape[0], shape.vis_hidden // shape.vis_heads
+    h = F.layer_norm(x, (shape.vis_hidden,), w[p + "layer_norm1.weight"], w[p + "layer_norm1.bias"], EPS)
+    q, k, v = (
+        _lin16(h, w[p + f"self_attn.{n}_proj.weight"], w[p + f"self_attn.{n}_proj.bias"], torch.float16)
+        .view(b, -1, shape.vis_heads, hd).transpose(1, 2)
+        for n in "qkv"
+    )  # fmt: skip
+    q16, k16, v16 = (t.to(torch.float16).float() for t in (q, k, v))
+    s = torch.matmul(q16, k16.transpose(2, 3)) * hd**-0.5
+    e = torch.exp(s - s.amax(dim=-1, keepdim=True))
+    o = torch.matmul(e.to(torch.float16).float(), v16) / e.sum(dim=-1, keepdim=True)
+    return (q, k, v), o.to(BF16)
+
+
+def vit_fused_attn_block(w: Weights, shape: PI05Shape, layer: int, x: torch.Tensor) -> torch.Tensor:
+    """One attention block of the fused tower, fp32 in and out (`SiglipEncoderLayer._attn_block`,
+    tybok/policies/pi05/models/vision.py:120-131): the fp16 half above, then out_proj from bf16 operands with
+    fp32 accumulation, bias and the fp32 residual added before the one fp32 store (`_vision_attn_out_kernel`,
+    triton_vision.py:437-497)."""
+    p = f"{VIS}encoder.layers.{layer}."
+    _, a = vit_fused_qkv_attention(w, shape, layer, x)
+    a = a.transpose(1, 2).reshape(x.shape[0], -1, shape.vis_hidden)
+    return x + _lin16(a, w[p + "self_attn.out_proj.weight"], w[p + "self_attn.out_proj.bias"], BF16)
+
+
+def vit_fused_mlp_block(w: Weights, shape: PI05Shape, layer: int, x: torch.Tensor) -> torch.Tensor:
+    """One MLP block of the fused tower (`triton_vision_mlp`, triton_vision.py:113-245, 550-622): bf16 operands, the
+    tanh-GELU on the fp32 pre-activation, the activation rounded to bf16 for fc2, fp32 residual."""
+    p = f"{VIS}encoder.layers.{layer}."
+    h = F.layer_norm(x, (shape.vis_hidden,), w[p + "layer_norm2.weight"], w[p + "layer_norm2.bias"], EPS)
+    act = F.gelu(_lin16(h, w[p + "mlp.fc1.weight"], w[p + "mlp.fc1.bias"], BF16), approximate="tanh")
+    return x + _lin16(act, w[p + "mlp.fc2.weight"], w[p + "mlp.fc2.bias"], BF16)
+
+
+def vit_fused_projector(w: Weights, shape: PI05Shape, x: torch.Tensor) -> torch.Tensor:
+    """post_layernorm + projector of the fused tower (`_vision_projector_kernel`, triton_vision.py:625-702): the
+    normalised row rounded to bf16, bf16 weights, fp32 result."""
+    h = F.layer_norm(x, (shape.vis_hidden,), w[VIS + "post_layernorm.weight"], w[VIS + "post_layernorm.bias"], EPS)
+    return _lin16(h, w[PROJ + ".weight"], w[PROJ + ".bias"], BF16)
+
+
 def embed_image(w: Weights, shape: PI05Shape, image: torch.Tensor) -> torch.Tensor:
     """``[1, 3, 224, 224]`` fp32 in [-1, 1] -> ``[1, 256, vlm_width]`` fp32 (vision.py + projector)."""
     x = F.conv2d(image.float(), w[VIS + "embeddings.patch_embedding.weight"], w[VIS + "embeddings.patch_embedding.bias"], stride=shape.patch)
@@ -96,21 +158,19 @@ def embed_image(w: Weights, shape: PI05Shape, image: torch.Tensor) -> torch.Tens
     def lowp(name, t, dt):  # Linear with weights and bias converted to dt (vision.py:223-235)
         return F.linear(t.to(dt), w[name + ".weight"].to(dt), w[name + ".bias"].to(dt))
 
+    if shape.vit_fused:
+        for i in range(shape.vis_layers):
+            x = vit_fused_mlp_block(w, shape, i, vit_fused_attn_block(w, shape, i, x))
+        return vit_fused_projector(w, shape, x)
     for i in range(shape.vis_layers):
         p = f"{VIS}encoder.layers.{i}."
         h = F.layer_norm(x, (shape.vis_hidden,), w[p + "layer_norm1.weight"], w[p + "layer_norm1.bias"], EPS)
-        if shape.vit_lowp_attn:
-            q, k, v = (lowp(p + f"self_attn.{n}_proj", h, torch.bfloat16).view(b, -1, shape.vis_heads, hd).transpose(1, 2) for n in "qkv")
-            probs = torch.softmax(torch.matmul(q.float(), k.float().transpose(2, 3)) * hd**-0.5, dim=-1).to(torch.bfloat16)
-            a = torch.matmul(probs.float(), v.float()).to(torch.bfloat16).transpose(1, 2).reshape(b, -1, shape.vis_hidden)
-            x = x + lowp(p + "self_attn.out_proj", a, torch.bfloat16).float()
-        else:
-            q = w.linear(p + "self_attn.q_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
-            k = w.linear(p + "self_attn.k_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
-            v = w.linear(p + "self_attn.v_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
-            a = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, scale=hd**-0.5, is_causal=False)
-            a = a.transpose(1, 2).contiguous().reshape(b, -1, shape.vis_hidden)
-            x = x + w.linear(p + "self_attn.out_proj", a)
+        q = w.linear(p + "self_attn.q_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
+        k = w.linear(p + "self_attn.k_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
+        v = w.linear(p + "self_attn.v_proj", h).view(b, -1, shape.vis_heads, hd).transpose(1, 2)
+        a = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, scale=hd**-0.5, is_causal=False)
+        a = a.transpose(1, 2).contiguous().reshape(b, -1, shape.vis_hidden)
+        x = x + w.linear(p + "self_attn.out_proj", a)
         h = F.layer_norm(x, (shape.vis_hidden,), w[p + "layer_norm2.weight"], w[p + "layer_norm2.bias"], EPS)
         if mdt is not None:
             x = x + lowp(p + "mlp.fc2", F.gelu(lowp(p + "mlp.fc1", h, mdt), approximate="tanh"), mdt).float()

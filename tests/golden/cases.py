@@ -92,3 +92,18 @@ def pi05_inputs(cfg, case: dict) -> dict:
         lang_masks=lang_masks,
         noise=noise,
     )
+
+
+def pi05_vit_fused_hidden(cfg) -> dict:
+    """Seeded fp32 hidden states ``[1, patches, vision_hidden]`` fed to the fused tower's q|k|v projection and
+    attention by the fixture ``pi05_small_vit_fused.npz`` and by the tests that read it (unit scale, a per-channel
+    offset and gain so that the LayerNorm has something to do)."""
+    g = torch.Generator().manual_seed(4242)
+    side = cfg.image_resolution[0] // cfg.vision_patch
+    n, c = side * side, cfg.vision_hidden
+    out = {}
+    for name in [f"layer{i}" for i in range(cfg.vision_layers)]:
+        gain = 0.5 + torch.rand(c, generator=g)
+        offset = 0.3 * torch.randn(c, generator=g)
+        out[name] = (torch.randn(1, n, c, generator=g) * gain + offset).contiguous()
+    return out

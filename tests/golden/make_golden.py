@@ -2,7 +2,7 @@
 
 Run ONCE in the build container (the reference is not available elsewhere):
 
-    python tests/golden/make_golden.py [smolvla|pi05|pi05_vit|all] [case]
+    python tests/golden/make_golden.py [smolvla|pi05|pi05_vit|pi05_vit_fused|all] [case]
 
 For each case the reference's eager model classes (``/root/reference/tybok/policies/<model>/models``)
 are constructed on the CPU from plain config dataclasses (no checkpoint, no tokenizer), loaded with
@@ -186,8 +186,65 @@ def pi05_vit_tiers() -> dict:
     return out
 
 
+def pi05_vit_fused() -> dict:
+    """The fp16 half of the reference's FUSED SigLIP tier (``--tl-fused-vit``): LayerNorm + packed fp16 q|k|v
+    projection (`_vision_qkv_kernel`) and the flash attention over fp16 q, k, v with fp16 probabilities
+    (`_vision_attn_kernel`), tybok/policies/pi05/models/vision.py:133-156 and triton_vision.py:38-110, 248-326 --
+    run through Triton's CPU interpreter (``TRITON_INTERPRET=1``; set by ``main`` before anything imports triton):
+    both layers of the small case's tower applied to seeded fp32 hidden states.  The bf16 kernels of that tier
+    (out_proj, MLP, projector) get no fixture: this interpreter multiplies bf16 operands as their raw 16-bit
+    integers (its out_proj returns 1e12 for inputs of order one), and the MLP kernel calls CUDA's libdevice tanh,
+    which it does not have."""
+    assert os.environ.get("TRITON_INTERPRET") == "1"
+    _import_reference()
+    from tybok.policies.pi05 import config as rcfg
+    from tybok.policies.pi05.models.flow_matching import PI05FlowMatching
+    from tybok.policies.pi05.models.triton_vision import triton_vision_attention
+
+    case = cases.PI05_CASES["small"]
+    cfg, sd, _ = cases.pi05_build(case)
+    rcfg.GEMMA_VARIANTS["golden_vlm"] = dict(cfg.paligemma_dims)
+    rcfg.GEMMA_VARIANTS["golden_expert"] = dict(cfg.expert_dims)
+    ref_cfg = rcfg.PI05Config(
+        paligemma_variant="golden_vlm", action_expert_variant="golden_expert", num_steps=cfg.num_steps,
+        tokenizer_max_length=cfg.tokenizer_max_length,
+    )  # fmt: skip
+    ref_cfg._image_features = list(cfg.image_features)
+    default = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        model = PI05FlowMatching(ref_cfg)
+    finally:
+        torch.set_default_dtype(default)
+    vt = model.paligemma_with_expert.paligemma.model.vision_tower.vision_model
+    vt.encoder.layers = vt.encoder.layers[: cfg.vision_layers]
+    model.eval()
+    _load(model, sd)
+    vt.set_fused_attn()
+    hidden = cases.pi05_vit_fused_hidden(cfg)
+    out: dict[str, np.ndarray] = {}
+    with torch.inference_mode():
+        for i, layer in enumerate(vt.encoder.layers):
+            q, k, v, b, length, c, attn = layer._fused_qkv(hidden[f"layer{i}"])  # fp32 [B, H, L, HD]
+            a = triton_vision_attention(q, k, v, attn.scale)  # bf16 [B, H, L, HD]
+            assert q.dtype == torch.float32 and a.dtype == torch.bfloat16
+            for name, t in (("q", q), ("k", k), ("v", v)):
+                out[f"{name}_layer{i}"] = t[0, ::4, ::8, ::4].numpy()  # 4 heads x 32 patches x 18 channels
+            out[f"attn_layer{i}"] = a[0, :, ::4].float().numpy()  # every head, 64 patches, 72 channels
+    return out
+
+
 def main() -> None:
     which = sys.argv[1] if len(sys.argv) > 1 else "all"
+    if which == "pi05_vit_fused":
+        # the reference's fused tower kernels, through Triton's interpreter: its own run (the variable must be set
+        # before triton is imported, and it changes nothing for the other fixtures, which launch no Triton kernel)
+        os.environ["TRITON_INTERPRET"] = "1"
+        t0 = time.time()
+        path = os.path.join(HERE, "pi05_small_vit_fused.npz")
+        np.savez_compressed(path, **pi05_vit_fused())
+        print(f"pi05 fused vit (fp16 q|k|v + attention): wrote {path} ({os.path.getsize(path) / 1024:.0f} KiB) in {time.time() - t0:.1f}s", flush=True)
+        return
     torch.manual_seed(0)
     jobs = []
     if which in ("smolvla", "all"):

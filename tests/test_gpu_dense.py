@@ -114,3 +114,36 @@ def test_dense_rejects_bad_arguments(tk):
         tk.bf16w_dense(x.cuda(), pw, b.cuda(), tile=33)
     with pytest.raises(ValueError):
         tk.bf16w_dense(x.cuda()[:, :32], pw, b.cuda())
+
+
+F16 = torch.float16
+
+
+@pytest.mark.parametrize("tile", [0, 42, 31, 21, 11])
+@pytest.mark.parametrize("m,k,n,act", [(512, 1152, 3456, None), (512, 1152, 4304, "gelu_tanh"), (512, 4304, 1152, None), (257, 80, 40, "gelu_tanh_fp32"), (130, 208, 264, None)])
+def test_dense_fp16_flavour_matches_torch(tk, tile, m, k, n, act):
+    # every 16-bit operand in fp16 (tk_f16w_dense): pi0.5's fp16 tower tiers.  Reference arithmetic: exact products
+    # of the fp16 operands summed in float64, one rounding to fp16 (then the GELU on that value or on the fp32 one).
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(m, k, generator=g).to(F16)
+    w = (torch.randn(n, k, generator=g) / k**0.5).to(F16)
+    b = torch.randn(n, generator=g).to(F16)
+    y = (x.double() @ w.double().t() + b.double()).float()
+    if act == "gelu_tanh":
+        y = F.gelu(y.to(F16).float(), approximate="tanh")
+    elif act == "gelu_tanh_fp32":
+        y = F.gelu(y, approximate="tanh")
+    want = y.to(F16)
+    got = tk.bf16w_dense(x.cuda(), tk.pack_bf16_weight(w.cuda()), b.cuda(), act, tile=tile)
+    assert got.dtype == F16
+    err = (got.float().cpu() - want.float()).abs()
+    tol = 2e-3 + 2**-10 * want.float().abs()  # one fp16 ulp of the result plus a floor near zero
+    assert not (err > tol).any(), f"fp16 dense M={m} K={k} N={n} tile={tile}: max |err| {err.max():.4g}"
+    assert (got.cpu() == want).float().mean().item() >= 0.97
+    # fp32 and fp16 residuals
+    r32 = torch.randn(m, n, generator=g)
+    got_r = tk.bf16w_dense(x.cuda(), tk.pack_bf16_weight(w.cuda()), b.cuda(), act, resid=r32.cuda(), tile=tile)
+    assert torch.equal(got_r.cpu(), (got.float().cpu() + r32).to(F16))
+    r16 = r32.to(F16)
+    got_r = tk.bf16w_dense(x.cuda(), tk.pack_bf16_weight(w.cuda()), b.cuda(), act, resid=r16.cuda(), tile=tile)
+    assert torch.equal(got_r.cpu(), (got.float().cpu() + r16.float()).to(F16))

@@ -64,3 +64,39 @@ def test_oracle_vision_mlp_tiers_match_the_reference_eager_tower(tag, dt):
     # the tiers are real: the low-precision fixtures differ from the fp32 one
     assert _maxdiff(gold["emb_bf16_cam0"], gold["emb_fp32_cam0"]) > 1e-4
     assert _maxdiff(gold["emb_fp16_cam0"], gold["emb_fp32_cam0"]) > 1e-6
+
+
+def test_oracle_fused_vision_fp16_half_matches_the_reference_kernels():
+    # The fp16 kernels of the reference's fused tower (triton_vision.py: `_vision_qkv_kernel`, `_vision_attn_kernel`)
+    # run through Triton's CPU interpreter by tests/golden/make_golden.py pi05_vit_fused on seeded hidden states:
+    # q, k, v as the projection stores them (fp32) and the attention output (bf16).  The restatement differs from
+    # the kernels in summation order and in how many key blocks share a running maximum (the probabilities are
+    # rounded to fp16 relative to it): rounding-level differences.  The last assertions show what the fixture pins:
+    # a q|k|v projection in bf16 instead of fp16 -- what this backend's tier used to compute -- sits an order of
+    # magnitude farther away.
+    gold = np.load(os.path.join(HERE, "golden", "pi05_small_vit_fused.npz"))
+    cfg, sd, _ = cases.pi05_build(cases.PI05_CASES["small"])
+    shape = O.PI05Shape(depth=cfg.paligemma_dims["depth"], vis_layers=cfg.vision_layers, num_steps=cfg.num_steps, vit_fused=True)
+    w = Weights(sd)
+    hidden = cases.pi05_vit_fused_hidden(cfg)
+    with torch.no_grad():
+        for i in range(cfg.vision_layers):
+            x = hidden[f"layer{i}"]
+            (q, k, v), a = O.vit_fused_qkv_attention(w, shape, i, x)
+            for name, t in (("q", q), ("k", k), ("v", v)):
+                want = gold[f"{name}_layer{i}"]
+                err = _maxdiff(t[0, ::4, ::8, ::4].numpy(), want)
+                print(f"fused tower layer {i} {name}: oracle vs the reference kernel {err:.3g}, |{name}|max {float(np.abs(want).max()):.3g}")
+                assert err <= 1e-4 * float(np.abs(want).max())  # fp16 products are exact in fp32: summation order, and a normalised value that rounds to the other fp16 neighbour under the kernel's two-pass variance
+            want = gold[f"attn_layer{i}"]
+            err = _maxdiff(a[0, :, ::4].float().numpy(), want)
+            scale = float(np.abs(want).max())
+            print(f"fused tower layer {i} attention: oracle vs the reference kernel {err:.3g}, |out|max {scale:.3g}")
+            assert err <= 2.0 ** (np.floor(np.log2(scale)) - 7)  # one bf16 step at the magnitude of the largest output
+            # the same half with bf16 in place of fp16 (q|k|v operands, q, k, v and the probabilities)
+            p = f"{O.VIS}encoder.layers.{i}."
+            h = torch.nn.functional.layer_norm(x, (shape.vis_hidden,), w[p + "layer_norm1.weight"], w[p + "layer_norm1.bias"], O.EPS)
+            qb = O._lin16(h, w[p + "self_attn.q_proj.weight"], w[p + "self_attn.q_proj.bias"], torch.bfloat16)
+            hd = shape.vis_hidden // shape.vis_heads
+            qb = qb.view(1, -1, shape.vis_heads, hd).transpose(1, 2)
+            assert _maxdiff(qb[0, ::4, ::8, ::4].numpy(), gold[f"q_layer{i}"]) >= 10 * _maxdiff(q[0, ::4, ::8, ::4].numpy(), gold[f"q_layer{i}"])

@@ -33,7 +33,8 @@ __device__ __forceinline__ void lds_barrier() {
 constexpr int NW = 4;  // waves per block
 constexpr int RK = 2;  // k tiles (of 32) per round
 
-template <int MT, int NT, int PF, int OCC>
+// F16: the operands are fp16 (v_mfma_f32_32x32x16_f16) instead of bf16; same tile order, same epilogues
+template <int MT, int NT, int PF, int OCC, bool F16>
 __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, int nblk_m, int ngroups) {
   constexpr int ROWS = MT * 32;
   constexpr int ROWB = RK * 64;     // bytes of one staged activation row per round
@@ -132,7 +133,10 @@ __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, in
   };
   auto mma1 = [&](int set, const WFrag& f, int j, int t) {  // t in [0, 2*MT*NT): k step, m tile, n tile
     const int h2 = t / (MT * NT), mt = (t / NT) % MT, nt = t % NT;
-    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(f.w[j][nt][h2]), as_bf16x8(xa[set][mt][h2]), acc[mt][nt], 0, 0, 0);
+    if (F16)
+      acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_f16x8(f.w[j][nt][h2]), as_f16x8(xa[set][mt][h2]), acc[mt][nt], 0, 0, 0);
+    else
+      acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(f.w[j][nt][h2]), as_bf16x8(xa[set][mt][h2]), acc[mt][nt], 0, 0, 0);
   };
 
   // PF rounds in flight; every load is unconditional (clamped addresses; columns past the block's k range are
@@ -279,7 +283,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, in
     for (int g = 0; g < 4; ++g) {
       int n0 = ncol0 + nt * 32 + 8 * g + 4 * half;
       if (n0 > a.N - 4) n0 = a.N - 4;  // columns past N are never stored
-      bias[nt][g] = a.bias ? unpack_bf16x4(*(const i32x2*)(a.bias + n0)) : f32x4{0.f, 0.f, 0.f, 0.f};
+      bias[nt][g] = a.bias ? unpack_16x4<F16>(*(const i32x2*)(a.bias + n0)) : f32x4{0.f, 0.f, 0.f, 0.f};
     }
   const int lrow = lane / LPR, lchunk = lane % LPR;
 #pragma unroll
@@ -291,12 +295,12 @@ __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, in
         const f32x16& c = acc[mt][nt];
         f32x4 v = {c[4 * g], c[4 * g + 1], c[4 * g + 2], c[4 * g + 3]};
         v = v + bias[nt][g];
-        if (a.act == 1) v = unpack_bf16x4(pack_bf16x4(v));  // the linear's bf16 output, then the activation on it
+        if (a.act == 1) v = unpack_16x4<F16>(pack_16x4<F16>(v));  // the linear's 16-bit output, then the activation on it
         if (a.act) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) v[j] = gelu_tanh_f(v[j]);
         }
-        *(i32x2*)(wl + l32 * EP + (nt * 32 + 8 * g + 4 * half) * 2) = pack_bf16x4(v);
+        *(i32x2*)(wl + l32 * EP + (nt * 32 + 8 * g + 4 * half) * 2) = pack_16x4<F16>(v);
       }
 #pragma unroll
     for (int j = 0; j < 32 / RPI; ++j) {
@@ -313,12 +317,12 @@ __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, in
           if (n + 8 <= a.N) r1 = rp[1];
         } else if (n + 8 <= a.N) {
           const i32x4 rr = *(const i32x4*)((const u16*)a.resid + (size_t)m * a.ldr + n);
-          r0 = unpack_bf16x4(i32x2{rr[0], rr[1]});
-          r1 = unpack_bf16x4(i32x2{rr[2], rr[3]});
+          r0 = unpack_16x4<F16>(i32x2{rr[0], rr[1]});
+          r1 = unpack_16x4<F16>(i32x2{rr[2], rr[3]});
         } else {
-          r0 = unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n));
+          r0 = unpack_16x4<F16>(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n));
         }
-        const i32x2 lo = pack_bf16x4(unpack_bf16x4(i32x2{t[0], t[1]}) + r0), hi = pack_bf16x4(unpack_bf16x4(i32x2{t[2], t[3]}) + r1);
+        const i32x2 lo = pack_16x4<F16>(unpack_16x4<F16>(i32x2{t[0], t[1]}) + r0), hi = pack_16x4<F16>(unpack_16x4<F16>(i32x2{t[2], t[3]}) + r1);
         t = i32x4{lo[0], lo[1], hi[0], hi[1]};
       }
       u16* dst = a.y + (size_t)m * a.ldy + n;
@@ -334,7 +338,10 @@ int launch(const GemmArgs& a, hipStream_t st) {
   const int nblk_n = (a.ntiles + NW * NT - 1) / (NW * NT);
   const int ngroups = nblk_n * a.ksplit;
   const unsigned blocks = (unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m;
-  hipLaunchKernelGGL((bf16w_wide_kernel<MT, NT, PF, OCC>), dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
+  if (a.f16)
+    hipLaunchKernelGGL((bf16w_wide_kernel<MT, NT, PF, OCC, true>), dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
+  else
+    hipLaunchKernelGGL((bf16w_wide_kernel<MT, NT, PF, OCC, false>), dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -131,7 +131,10 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(LayerNormArgs a) {
       union { i32x4 q; unsigned u[4]; } o4;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        o4.u[e] = pack_bf16x2((v[i][2 * e] - mean) * rstd * w[2 * e] + b[2 * e], (v[i][2 * e + 1] - mean) * rstd * w[2 * e + 1] + b[2 * e + 1]);
+      {
+        const float y0 = (v[i][2 * e] - mean) * rstd * w[2 * e] + b[2 * e], y1 = (v[i][2 * e + 1] - mean) * rstd * w[2 * e + 1] + b[2 * e + 1];
+        o4.u[e] = a.y_f16 ? pack_f16x2(y0, y1) : pack_bf16x2(y0, y1);
+      }
       *(i32x4*)(a.y + (size_t)row * a.ldy + 8 * p) = o4.q;
     }
   }

@@ -561,8 +561,10 @@ float dense_cost(const DenseTile& t, int M, int N, int KT, int ks, int cus) {
 }
 }  // namespace
 
-int tk_bf16w_dense(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy, const void* resid,
-                   int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws, size_t ws_bytes, void* stream) {
+namespace {
+int dense_common(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy, const void* resid,
+                 int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws, size_t ws_bytes, void* stream,
+                 int f16) {
   if (M <= 0 || N <= 0 || K <= 0) return fail(TK_EINVAL, "bf16w_dense: non-positive shape M=%d N=%d K=%d", M, N, K);
   if (K % 16 || ldx % 8 || ldx < K) return fail(TK_EINVAL, "bf16w_dense: K=%d must be a multiple of 16 and ldx=%d a multiple of 8 >= K", K, ldx);
   if (!x || !w_packed || !y) return fail(TK_EINVAL, "bf16w_dense: null pointer");
@@ -591,6 +593,7 @@ int tk_bf16w_dense(const void* x, int ldx, const void* w_packed, const void* bia
   a.KT = (K + 31) / 32;
   a.ntiles = (N + 31) / 32;
   a.act = act;
+  a.f16 = f16;
   a.vec = a.vec16 = 1;
   const int cus = device_cus();
   const DenseTile* best = nullptr;
@@ -629,6 +632,17 @@ int tk_bf16w_dense(const void* x, int ldx, const void* w_packed, const void* bia
   a.counters = ks > 1 ? (int*)ws : nullptr;
   if (tk_launch_bf16w_wide(a, best->id, (hipStream_t)stream)) return fail(TK_ELAUNCH, "bf16w_dense: launch failed (%s)", hipGetErrorString(hipGetLastError()));
   return TK_OK;
+}
+}  // namespace
+
+int tk_bf16w_dense(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy, const void* resid,
+                   int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws, size_t ws_bytes, void* stream) {
+  return dense_common(x, ldx, w_packed, bias, act, y, ldy, resid, ldr, resid_dtype, M, N, K, tile, split_k, ws, ws_bytes, stream, 0);
+}
+
+int tk_f16w_dense(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy, const void* resid,
+                  int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws, size_t ws_bytes, void* stream) {
+  return dense_common(x, ldx, w_packed, bias, act, y, ldy, resid, ldr, resid_dtype, M, N, K, tile, split_k, ws, ws_bytes, stream, 1);
 }
 
 int tk_quant_act_rows(const void* x, int ldx, void* a8, int lda, void* sa, int M, int K, int mode, void* stream) {
@@ -880,8 +894,11 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   a.H = H;
   a.G = G;
   a.mask_mode = mask_mode;
-  a.logits_bf16 = logits_bf16;
+  a.logits_bf16 = logits_bf16 == 1;
+  a.f16 = logits_bf16 == 2;
   a.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
+  if (a.f16 && !(batch > 0 && !split && S == 0 && !mask2d && !pad && D == 96 && P >= 128 && M >= 128))
+    return fail(TK_EINVAL, "attn: fp16 operands are built for the batched tower shape only (D = 96, >= 128 queries and keys)");
 
   if (batch > 0 && !split && S == 0 && !mask2d && !pad && (D == 64 || D == 96) && P >= 128 && M >= 128) {
     // vision towers: many query tiles over a long key range -- K / V^T staged through LDS once per 128 queries
@@ -1151,7 +1168,8 @@ int tk_rope_rows(void* y, int ldy, const void* rope_pos, const void* rope_cos, c
 }
 
 static int layer_norm_impl(const char* who, const void* x, int ldx, int x_dtype, const void* r, int ldr, void* xsum, int ldxs,
-                           const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream) {
+                           const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream,
+                           int y_f16 = 0) {
   if (M <= 0 || K <= 0 || K % 8 || K > tk_layer_norm_max_k()) return fail(TK_EINVAL, "%s: K=%d must be a multiple of 8, at most %d", who, K, tk_layer_norm_max_k());
   if ((x_dtype != TK_BF16 && x_dtype != TK_F32) || x_dtype != wb_dtype) return fail(TK_EINVAL, "%s: rows and parameters must both be bf16 or both fp32", who);
   if (!x || !w || !b || !y || ldx < K || ldy < K || ldx % 8 || ldy % 8) return fail(TK_EINVAL, "%s: null pointer or row pitch not a multiple of 8 >= K", who);
@@ -1168,6 +1186,7 @@ static int layer_norm_impl(const char* who, const void* x, int ldx, int x_dtype,
   a.eps = eps;
   a.y = (u16*)y;
   a.ldy = ldy;
+  a.y_f16 = y_f16;
   a.M = M;
   a.K = K;
   a.r = (const u16*)r;
@@ -1187,6 +1206,16 @@ int tk_add_layer_norm(const void* x, int ldx, int x_dtype, const void* r, int ld
                       const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream) {
   if (!r) return fail(TK_EINVAL, "add_layer_norm: null residual branch");
   return layer_norm_impl("add_layer_norm", x, ldx, x_dtype, r, ldr, xsum, ldxs, w, b, wb_dtype, eps, y, ldy, M, K, stream);
+}
+
+int tk_layer_norm_f16(const void* x, int ldx, const void* w, const void* b, float eps, void* y, int ldy, int M, int K, void* stream) {
+  return layer_norm_impl("layer_norm_f16", x, ldx, TK_F32, nullptr, 0, nullptr, 0, w, b, TK_F32, eps, y, ldy, M, K, stream, 1);
+}
+
+int tk_add_layer_norm_f16(const void* x, int ldx, const void* r, int ldr, void* xsum, int ldxs, const void* w, const void* b, float eps,
+                          void* y, int ldy, int M, int K, void* stream) {
+  if (!r) return fail(TK_EINVAL, "add_layer_norm_f16: null residual branch");
+  return layer_norm_impl("add_layer_norm_f16", x, ldx, TK_F32, r, ldr, xsum, ldxs, w, b, TK_F32, eps, y, ldy, M, K, stream, 1);
 }
 
 int tk_debug_stream_read(const void* src, size_t bytes, int blocks, void* sink, void* stream) {

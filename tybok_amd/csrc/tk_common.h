@@ -54,6 +54,40 @@ __device__ __forceinline__ float sub_rn(float a, float b) {
 #pragma clang fp contract(off)
   return a - b;
 }
+// fp16 counterparts (round-to-nearest-even conversions), for the kernels that also come in an fp16 flavour
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ unsigned pack_f16x2(float a, float b) {
+  f32x2 v = {a, b};
+  union { f16x2 h; unsigned u; } r;
+  r.h = __builtin_convertvector(v, f16x2);
+  return r.u;
+}
+__device__ __forceinline__ i32x2 pack_f16x4(f32x4 v) {
+  i32x2 r = {(int)pack_f16x2(v[0], v[1]), (int)pack_f16x2(v[2], v[3])};
+  return r;
+}
+__device__ __forceinline__ f32x4 unpack_f16x4(i32x2 r) {
+  union { i32x2 i; f16x2 h[2]; } u;
+  u.i = r;
+  f32x4 v = {(float)u.h[0][0], (float)u.h[0][1], (float)u.h[1][0], (float)u.h[1][1]};
+  return v;
+}
+__device__ __forceinline__ f16x8 as_f16x8(i32x4 v) {
+  union { i32x4 i; f16x8 h; } u;
+  u.i = v;
+  return u.h;
+}
+// four fp32 <-> four 16-bit floats of the kernel's flavour
+template <bool F16>
+__device__ __forceinline__ i32x2 pack_16x4(f32x4 v) {
+  return F16 ? pack_f16x4(v) : pack_bf16x4(v);
+}
+template <bool F16>
+__device__ __forceinline__ f32x4 unpack_16x4(i32x2 r) {
+  return F16 ? unpack_f16x4(r) : unpack_bf16x4(r);
+}
+
 __device__ __forceinline__ float round_bf16(float f) { return __uint_as_float(pack_bf16x2(f, 0.f) << 16); }
 
 // 4 e4m3fn bytes (one dword) -> 4 bf16 (exact: every e4m3 value is a bf16 value).

@@ -55,6 +55,8 @@ struct GemmArgs {
   const unsigned short* bias;
   // many-row fp8 kernels: 32-row tiles per block (2 or 4), chosen by the host
   int mtiles;
+  // many-row 16-bit-weight kernel only: activations, weights, bias, output and a 16-bit residual are fp16, not bf16
+  int f16;
   // single-launch gated FFN only: the hand-off words in the workspace (TK_FUSE_* below), the down blocks per row
   // block, and the bound on a down block's wait (polls)
   int* fuse;
@@ -102,6 +104,7 @@ struct AttnArgs {
   int xcd_remap;  // batched, unsplit launches: 1-D grid with (problem, head) pairs pinned to an XCD
   long long q_sb, k_sb, vt_sb, out_sb;
   int mask_mode, logits_bf16;
+  int f16;  // tower kernel only: q, K, V^T and the probabilities are fp16 (the output stays bf16)
   int kv_splits;
   int tile_q, tile_r;  // key tiles = kv_splits * tile_q + tile_r
   int gqa_mul;         // kv head of query head h = (h * gqa_mul) >> 16
@@ -157,8 +160,9 @@ struct LayerNormArgs {
   const void* b;
   int wb_f32;
   float eps;
-  unsigned short* y;  // bf16 [M, K], element pitch ldy
+  unsigned short* y;  // bf16 (fp16 when y_f16) [M, K], element pitch ldy
   int ldy;
+  int y_f16;
   int M, K;
   // optional residual branch: rows are x + r (r bf16, pitch ldr), the sum goes to xsum in x's type
   // (pitch ldxs; may be x itself)

@@ -30,11 +30,19 @@ constexpr int kStageKeys = 64;
 // 16*(i/8) + 8*hf + i%8 of the tile: registers 8s..8s+7 are then the B operand of k step s.
 __device__ __forceinline__ int key_of_row(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
 
-__device__ __forceinline__ bf16x8 pack8(const float* v) {
-  union { unsigned u[4]; bf16x8 b; } r;
+// eight fp32 -> one 16-byte matrix operand of the kernel's flavour (bf16 or fp16), round to nearest even
+template <bool F16>
+__device__ __forceinline__ i32x4 pack8(const float* v) {
+  i32x4 r;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) r.u[j] = pack_bf16x2(v[2 * j], v[2 * j + 1]);
-  return r.b;
+  for (int j = 0; j < 4; ++j) r[j] = (int)(F16 ? pack_f16x2(v[2 * j], v[2 * j + 1]) : pack_bf16x2(v[2 * j], v[2 * j + 1]));
+  return r;
+}
+// one 32 x 32 x 16 product with the operands read as bf16 or as fp16
+template <bool F16>
+__device__ __forceinline__ f32x16 mma16(i32x4 a, i32x4 b, f32x16 c) {
+  if (F16) return __builtin_amdgcn_mfma_f32_32x32x16_f16(as_f16x8(a), as_f16x8(b), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
 }
 
 // max / sum of a value over the two lanes that share a query (lane l and l ^ 32), without an LDS trip:
@@ -68,7 +76,9 @@ struct TowerLds {
 
 // LB: the logits are rounded to bf16 before the scale and the softmax (what a bf16 matmul hands to a
 // fp32 softmax); otherwise they stay fp32.
-template <int D, bool LB>
+// F16: q, K, V^T are fp16 and the probabilities are rounded to fp16 for P.V (both products on the fp16 matrix
+// instruction); the output stays bf16.
+template <int D, bool LB, bool F16>
 __global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kernel(AttnArgs a, int qblocks) {
   using L = TowerLds<D>;
   constexpr int DS = D / 16;            // k steps of Q.K^T
@@ -138,11 +148,11 @@ __global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kerne
 
   gload(s_lo);
   // Q^T operands of this wave's tile: lane (query l32, half) holds columns 16 s + 8 half .. + 8
-  bf16x8 qf[DS];
+  i32x4 qf[DS];
   {
     const u16* qrow = qp + (size_t)(q_ok ? qi : a.M - 1) * a.q_sm;
 #pragma unroll
-    for (int s = 0; s < DS; ++s) qf[s] = as_bf16x8(*(const i32x4*)(qrow + 16 * s + 8 * half));
+    for (int s = 0; s < DS; ++s) qf[s] = *(const i32x4*)(qrow + 16 * s + 8 * half);
   }
   f32x16 o[DT];
 #pragma unroll
@@ -174,8 +184,8 @@ __global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kerne
       for (int ks = 0; ks < DS; ++ks)
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
-          const bf16x8 kop = as_bf16x8(*(const i32x4*)(kb + (kt * 32 + krow) * KP + (16 * ks + 8 * half) * 2));
-          sT[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop, qf[ks], sT[kt], 0, 0, 0);
+          const i32x4 kop = *(const i32x4*)(kb + (kt * 32 + krow) * KP + (16 * ks + 8 * half) * 2);
+          sT[kt] = mma16<F16>(kop, qf[ks], sT[kt]);
         }
       // ---- one online-softmax step over the stage's 64 keys, one query per lane; register i of tile
       //      kt = key 64 s + 32 kt + 16*(i/8) + 8*half + i%8 ----
@@ -231,11 +241,11 @@ __global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kerne
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-          const bf16x8 pb = pack8(p[kt] + 8 * ks);
+          const i32x4 pb = pack8<F16>(p[kt] + 8 * ks);
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) {
-            const bf16x8 vop = as_bf16x8(*(const i32x4*)(vb + (32 * dt + l32) * VP + (kt * 32 + 16 * ks + 8 * half) * 2));
-            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vop, pb, o[dt], 0, 0, 0);
+            const i32x4 vop = *(const i32x4*)(vb + (32 * dt + l32) * VP + (kt * 32 + 16 * ks + 8 * half) * 2);
+            o[dt] = mma16<F16>(vop, pb, o[dt]);
           }
         }
       if (it + 1 < s_n) lstore(buf ^ 1);  // the other buffer: every wave of the group left it at the last barrier
@@ -275,12 +285,12 @@ __global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kerne
   }
 }
 
-template <int D, bool LB>
+template <int D, bool LB, bool F16 = false>
 int launch_tower(const AttnArgs& a, hipStream_t st) {
   // more LDS than a launch gets by default: raise the kernel's limit once per process
   static int raised = 0;
   if (!raised) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&tower_attn_kernel<D, LB>), hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&tower_attn_kernel<D, LB, F16>), hipFuncAttributeMaxDynamicSharedMemorySize,
                             TowerLds<D>::TOTAL) != hipSuccess)
       return -3;
     raised = 1;
@@ -288,7 +298,7 @@ int launch_tower(const AttnArgs& a, hipStream_t st) {
   const int qblocks = (a.M + kQTiles * 32 - 1) / (kQTiles * 32);
   const int pairs = a.batch * a.H;
   dim3 grid(8 * ((pairs + 7) / 8) * qblocks);
-  hipLaunchKernelGGL((tower_attn_kernel<D, LB>), grid, dim3(kWaves * 64), TowerLds<D>::TOTAL, st, a, qblocks);
+  hipLaunchKernelGGL((tower_attn_kernel<D, LB, F16>), grid, dim3(kWaves * 64), TowerLds<D>::TOTAL, st, a, qblocks);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
@@ -349,6 +359,7 @@ int tk_launch_transpose_v(TransposeVArgs a, int D, hipStream_t st) {
 // kernel.
 int tk_launch_tower_attn(AttnArgs a, int D, hipStream_t st) {
   if (a.P <= kStageKeys) return -1;
+  if (a.f16) return D == 96 && !a.logits_bf16 ? launch_tower<96, false, true>(a, st) : -1;  // (pi0.5's tower)
   if (D == 64) return a.logits_bf16 ? launch_tower<64, true>(a, st) : launch_tower<64, false>(a, st);
   if (D == 96) return a.logits_bf16 ? launch_tower<96, true>(a, st) : launch_tower<96, false>(a, st);
   return -1;

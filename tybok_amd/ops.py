@@ -98,6 +98,7 @@ class PackedBf16Weight:
     n: int
     k: int
     rope_half: int = 0
+    dtype: torch.dtype = torch.bfloat16  # the 16-bit type of the packed words (fp16: the many-row kernel only)
 
 
 @dataclass
@@ -333,15 +334,18 @@ def w8a8_ffn_intermediates(ws: Workspace, m: int, k: int, i: int) -> tuple[torch
 
 
 def pack_bf16_weight(w: torch.Tensor, rope_half: int = 0) -> PackedBf16Weight:
-    """Row-major bf16 ``[N, K]`` -> :class:`PackedBf16Weight` (once per model)."""
+    """Row-major bf16 ``[N, K]`` -> :class:`PackedBf16Weight` (once per model).  An fp16 matrix is packed the same way
+    (the tile order moves 16-bit words) for :func:`bf16w_dense` on fp16 activations."""
     lib = native.lib()
-    if w.dtype != torch.bfloat16 or not w.is_cuda or w.dim() != 2:
-        raise TypeError("expected a bf16 CUDA matrix")
+    if w.dtype not in (torch.bfloat16, torch.float16) or not w.is_cuda or w.dim() != 2:
+        raise TypeError("expected a bf16 (or fp16) CUDA matrix")
+    if w.dtype == torch.float16 and rope_half:
+        raise ValueError("fp16 weights serve the many-row kernel only (natural tile order)")
     w = w.contiguous()
     n, k = w.shape
     out = torch.empty(int(lib.tk_bf16w_packed_bytes(n, k)), dtype=torch.uint8, device=w.device)
     native.check(lib.tk_pack_bf16_weight(w.data_ptr(), out.data_ptr(), n, k, rope_half, _stream()), "tk_pack_bf16_weight")
-    return PackedBf16Weight(out, n, k, rope_half)
+    return PackedBf16Weight(out, n, k, rope_half, w.dtype)
 
 
 _DENSE_ACTS = {None: 0, "none": 0, "gelu_tanh": 1, "gelu_tanh_fp32": 2}
@@ -362,24 +366,36 @@ def bf16w_dense(
     """``bf16(resid + act(bf16(x @ W^T + bias)))`` for ``x [M, K]`` bf16 and a packed bf16 weight: the linears of the
     vision towers on the many-row MFMA kernel.  ``act``: ``"gelu_tanh"`` applies the tanh GELU to the bf16-rounded
     linear output (what ``gelu(linear(x))`` on bf16 tensors computes), ``"gelu_tanh_fp32"`` to the fp32 one (a GEMM
-    with the activation in its epilogue).  ``tile`` picks the block tile (0 = by shape)."""
+    with the activation in its epilogue).  ``tile`` picks the block tile (0 = by shape).  With fp16 activations and
+    a weight packed from an fp16 matrix every 16-bit operand is fp16 (``tk_f16w_dense``: pi0.5's fp16 tower tiers)."""
     lib = native.lib()
     if w.rope_half:
         raise ValueError("bf16w_dense takes weights packed in natural tile order (rope_half = 0)")
-    m, ldx = _check_act(x, w.k)
-    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != w.n or not bias.is_contiguous() or bias.device != x.device):
-        raise ValueError(f"bias must be a contiguous bf16 vector of {w.n} elements on the activations' device")
+    dt = w.dtype
+    if x.dtype != dt or not x.is_cuda or x.dim() != 2 or x.shape[1] != w.k or x.stride(1) != 1:
+        raise ValueError(f"activations must be a CUDA [M, {w.k}] matrix of the weight's type with unit inner stride")
+    m, ldx = x.shape[0], x.stride(0)
+    if bias is not None and (bias.dtype != dt or bias.numel() != w.n or not bias.is_contiguous() or bias.device != x.device):
+        raise ValueError(f"bias must be a contiguous vector of {w.n} elements of the weight's type on the activations' device")
     if out is None:
-        out = torch.empty(m, w.n, dtype=torch.bfloat16, device=x.device)
-    if out.dtype != torch.bfloat16 or out.shape != (m, w.n) or out.stride(1) != 1:
-        raise ValueError("out must be bf16 [M, N] with unit inner stride")
-    rp, ldr, rdt = _resid_args(resid, m, w.n)
+        out = torch.empty(m, w.n, dtype=dt, device=x.device)
+    if out.dtype != dt or out.shape != (m, w.n) or out.stride(1) != 1:
+        raise ValueError("out must be [M, N] of the weight's type with unit inner stride")
+    if resid is not None and resid.dtype == torch.float16 and dt == torch.float16:
+        if resid.shape != (m, w.n) or resid.stride(1) != 1:
+            raise ValueError("residual must be [M, N] with unit inner stride")
+        rp, ldr, rdt = resid.data_ptr(), resid.stride(0), _BF16  # the 16-bit residual of the kernel's flavour
+    else:
+        rp, ldr, rdt = _resid_args(resid, m, w.n)
+        if dt == torch.float16 and resid is not None and resid.dtype == torch.bfloat16:
+            raise TypeError("an fp16 launch takes an fp16 or fp32 residual")
     ws = ws or default_workspace(x.device)
-    rc = lib.tk_bf16w_dense(
+    entry = lib.tk_f16w_dense if dt == torch.float16 else lib.tk_bf16w_dense
+    rc = entry(
         x.data_ptr(), ldx, w.data.data_ptr(), None if bias is None else bias.data_ptr(), _DENSE_ACTS[act], out.data_ptr(),
         out.stride(0), rp, ldr, rdt, m, w.n, w.k, tile, split_k, ws.ptr, ws.nbytes, _stream(),
     )  # fmt: skip
-    native.check(rc, "tk_bf16w_dense")
+    native.check(rc, "tk_f16w_dense" if dt == torch.float16 else "tk_bf16w_dense")
     return out
 
 
@@ -699,8 +715,15 @@ def batched_attn(
     zero columns up to a supported ``D`` passes the scale of its true size)."""
     lib = native.lib()
     bf = torch.bfloat16
-    if q.dtype != bf or k.dtype != bf or vt.dtype != bf or q.dim() != 4 or k.dim() != 4 or vt.dim() != 4:
-        raise TypeError("q, k, vt must be 4-D bf16 tensors")
+    if q.dtype == torch.float16:
+        # fp16 operands (pi0.5's fused tower): fp32 logits, probabilities rounded to fp16, bf16 output
+        if logits_bf16:
+            raise ValueError("fp16 operands keep the logits in fp32")
+        logits_bf16 = 2
+    elif q.dtype != bf:
+        raise TypeError("q, k, vt must be 4-D bf16 (or fp16) tensors")
+    if k.dtype != q.dtype or vt.dtype != q.dtype or q.dim() != 4 or k.dim() != 4 or vt.dim() != 4:
+        raise TypeError("q, k, vt must be 4-D tensors of one 16-bit type")
     b, m, h, d = q.shape
     p, g = k.shape[1], k.shape[2]
     if k.shape[0] != b or k.shape[3] != d or vt.shape[:3] != (b, g, d) or vt.shape[3] < _pad32(p):
@@ -735,13 +758,13 @@ def transpose_v(v: torch.Tensor, *, out: torch.Tensor | None = None) -> torch.Te
     ``vt [B, G, D, P rounded up to 32]`` with zero-filled padding keys: the V^T operand of
     :func:`batched_attn`, one launch for all problems.  ``D`` in {64, 96}."""
     lib = native.lib()
-    if v.dtype != torch.bfloat16 or v.dim() != 4 or v.stride(3) != 1:
-        raise TypeError("v must be a 4-D bf16 tensor with a contiguous head dim")
+    if v.dtype not in (torch.bfloat16, torch.float16) or v.dim() != 4 or v.stride(3) != 1:
+        raise TypeError("v must be a 4-D bf16 (or fp16) tensor with a contiguous head dim")
     b, p, g, d = v.shape
     if out is None:
-        out = torch.empty(b, g, d, _pad32(p), dtype=torch.bfloat16, device=v.device)
-    if out.shape[:3] != (b, g, d) or out.shape[3] < _pad32(p) or out.stride(3) != 1 or out.dtype != torch.bfloat16:
-        raise ValueError("out must be bf16 [B, G, D, >= P rounded up to 32] with contiguous keys")
+        out = torch.empty(b, g, d, _pad32(p), dtype=v.dtype, device=v.device)
+    if out.shape[:3] != (b, g, d) or out.shape[3] < _pad32(p) or out.stride(3) != 1 or out.dtype != v.dtype:
+        raise ValueError("out must be [B, G, D, >= P rounded up to 32] of v's type with contiguous keys")
     rc = lib.tk_batched_transpose_v(
         v.data_ptr(), v.stride(0), v.stride(1), v.stride(2), out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
         out.shape[3], b, p, g, d, _stream(),
@@ -833,9 +856,10 @@ def expert_tail(
     return v, x_new
 
 
-def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) -> torch.Tensor:
+def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """``bf16(LayerNorm(x) * w + b)`` over the last dim of ``x [..., K]`` (fp32 with fp32 parameters, or
-    bf16 with bf16 parameters; contiguous rows), statistics in fp32.  One launch, bf16 result."""
+    bf16 with bf16 parameters; contiguous rows), statistics in fp32.  One launch, bf16 result -- or, for fp32 rows
+    and ``out_dtype=torch.float16``, an fp16 one."""
     lib = native.lib()
     if x.dtype not in (torch.float32, torch.bfloat16) or w.dtype != x.dtype or b.dtype != x.dtype:
         raise TypeError("layer_norm: x, w, b must all be fp32 or all bf16")
@@ -843,6 +867,14 @@ def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) ->
     x2 = x.reshape(-1, k)
     if x2.stride(1) != 1 or w.numel() != k or b.numel() != k:
         raise ValueError("layer_norm: rows must be contiguous and w, b hold K values")
+    if out_dtype == torch.float16:
+        if x.dtype != torch.float32:
+            raise TypeError("layer_norm: the fp16 result is built for fp32 rows")
+        y = torch.empty(x2.shape, dtype=torch.float16, device=x.device)
+        rc = lib.tk_layer_norm_f16(x2.data_ptr(), x2.stride(0), w.contiguous().data_ptr(), b.contiguous().data_ptr(), float(eps),
+                                   y.data_ptr(), y.stride(0), x2.shape[0], k, _stream())  # fmt: skip
+        native.check(rc, "tk_layer_norm_f16")
+        return y.view(x.shape)
     y = torch.empty(x2.shape, dtype=torch.bfloat16, device=x.device)
     dt = _F32 if x.dtype == torch.float32 else _BF16
     rc = lib.tk_layer_norm(x2.data_ptr(), x2.stride(0), dt, w.contiguous().data_ptr(), b.contiguous().data_ptr(), dt, float(eps),
@@ -851,7 +883,9 @@ def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) ->
     return y.view(x.shape)
 
 
-def add_layer_norm(x: torch.Tensor, r: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) -> tuple[torch.Tensor, torch.Tensor]:
+def add_layer_norm(
+    x: torch.Tensor, r: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, out_dtype: torch.dtype = torch.bfloat16
+) -> tuple[torch.Tensor, torch.Tensor]:
     """``x += r`` in place (``r`` bf16: the linear that closes a residual branch; fp32 ``x`` takes
     ``float(r)``, bf16 ``x`` rounds the sum once) and ``bf16(LayerNorm(x) * w + b)`` of the sum, one launch.
     Returns ``(x, normalised)``; ``x`` must own contiguous rows."""
@@ -864,6 +898,15 @@ def add_layer_norm(x: torch.Tensor, r: torch.Tensor, w: torch.Tensor, b: torch.T
     x2, r2 = x.view(-1, k), r.reshape(-1, k)
     if r2.stride(1) != 1:
         r2 = r2.contiguous()
+    if out_dtype == torch.float16:
+        if x.dtype != torch.float32:
+            raise TypeError("add_layer_norm: the fp16 result is built for fp32 rows")
+        y = torch.empty(x2.shape, dtype=torch.float16, device=x.device)
+        rc = lib.tk_add_layer_norm_f16(x2.data_ptr(), x2.stride(0), r2.data_ptr(), r2.stride(0), x2.data_ptr(), x2.stride(0),
+                                       w.contiguous().data_ptr(), b.contiguous().data_ptr(), float(eps), y.data_ptr(), y.stride(0),
+                                       x2.shape[0], k, _stream())  # fmt: skip
+        native.check(rc, "tk_add_layer_norm_f16")
+        return x, y.view(x.shape)
     y = torch.empty(x2.shape, dtype=torch.bfloat16, device=x.device)
     dt = _F32 if x.dtype == torch.float32 else _BF16
     rc = lib.tk_add_layer_norm(x2.data_ptr(), x2.stride(0), dt, r2.data_ptr(), r2.stride(0), x2.data_ptr(), x2.stride(0),

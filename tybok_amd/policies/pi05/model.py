@@ -150,6 +150,10 @@ class PI05Model:
         self.vis_head_pad = next((d for d in (64, 96, 128, 256) if d >= cfg.vision_hidden // cfg.vision_heads), 0)
         if self.vit_lowp_attn and not self.vis_head_pad:
             raise ValueError("vision heads wider than 256 are not supported by the attention kernel")
+        # q|k|v of the fused tier run on fp16 operands, as the reference's fused tower does (its q/k/v "need a >= 10-bit
+        # mantissa", tybok/policies/pi05/models/triton_vision.py:23-25) -- where the fp16 kernels take the shape (the
+        # tower attention kernel at a padded head size of 96 on the GPU); elsewhere bf16
+        self.vit_qkv_dtype = torch.float16 if self.device.type == "cuda" and self.vis_head_pad == 96 else BF16
         for i in range(cfg.vision_layers):
             lp = f"{VIS}encoder.layers.{i}."
             if self.vit_mlp_dtype is not None:
@@ -167,8 +171,8 @@ class PI05Model:
                     return out.view(heads * hp, *t.shape[1:])
 
                 self.vis_lowp[lp + "self_attn.qkv"] = (
-                    torch.cat([pad_rows(self.p[lp + f"self_attn.{n}_proj.weight"]) for n in "qkv"], dim=0).to(BF16).contiguous(),
-                    torch.cat([pad_rows(self.p[lp + f"self_attn.{n}_proj.bias"]) for n in "qkv"], dim=0).to(BF16).contiguous(),
+                    torch.cat([pad_rows(self.p[lp + f"self_attn.{n}_proj.weight"]) for n in "qkv"], dim=0).to(self.vit_qkv_dtype).contiguous(),
+                    torch.cat([pad_rows(self.p[lp + f"self_attn.{n}_proj.bias"]) for n in "qkv"], dim=0).to(self.vit_qkv_dtype).contiguous(),
                 )
                 self.vis_lowp[lp + "self_attn.out_proj"] = (
                     pad_rows(self.p[lp + "self_attn.out_proj.weight"].t().contiguous()).t().to(BF16).contiguous(),
@@ -178,6 +182,10 @@ class PI05Model:
         # same weights in its tile order (shapes it does not take -- K % 16, N % 8 -- stay on the library GEMM)
         self.vis_dense: dict[str, tuple] = {}
         if self.vit_lowp_attn and self.vit_mlp_dtype == BF16 and self.device.type == "cuda" and self.vis_head_pad in (64, 96):
+            if all(w.shape[1] % 16 == 0 and w.shape[0] % 8 == 0 for w, _ in self.vis_lowp.values()):
+                self.vis_dense = {n: (tk.pack_bf16_weight(w), b.contiguous()) for n, (w, b) in self.vis_lowp.items()}
+        elif self.vit_mlp_dtype is not None and not self.vit_lowp_attn and self.device.type == "cuda":
+            # the MLP-only tiers: fc1 / fc2 on the many-row kernel in their 16-bit type (bf16 or fp16)
             if all(w.shape[1] % 16 == 0 and w.shape[0] % 8 == 0 for w, _ in self.vis_lowp.values()):
                 self.vis_dense = {n: (tk.pack_bf16_weight(w), b.contiguous()) for n, (w, b) in self.vis_lowp.items()}
         self.set_num_steps(cfg.num_steps)
@@ -253,7 +261,7 @@ class PI05Model:
                 # attention, one problem per image: fp32 scores and softmax, probabilities rounded to bf16
                 # for P.V (fp32 accumulate)
                 hp = self.vis_head_pad
-                h = tk.layer_norm(x, p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], EPS)
+                h = tk.layer_norm(x, p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], EPS, out_dtype=self.vit_qkv_dtype)
                 qkv = F.linear(h, *self.vis_lowp[lp + "self_attn.qkv"]).view(b, -1, 3, heads, hp)
                 vt = tk.transpose_v(qkv[:, :, 2]) if hp in (64, 96) else qkv[:, :, 2].permute(0, 2, 3, 1).contiguous()
                 a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, scale=hd**-0.5, ws=self.ws)
@@ -269,15 +277,20 @@ class PI05Model:
             if self.vit_mlp_dtype is not None:
                 # MLP-only low precision: fc1, gelu and fc2 in that dtype, cast at the boundary (for bf16 on a
                 # GPU the LayerNorm and the cast are one launch)
-                if self.vit_mlp_dtype == BF16 and x.is_cuda:
-                    h = tk.layer_norm(x, p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS)
+                if x.is_cuda:
+                    h = tk.layer_norm(x, p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS, out_dtype=self.vit_mlp_dtype)
                 else:
                     h = F.layer_norm(x, (vh,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS).to(self.vit_mlp_dtype)
-                if self.vit_mlp_dtype == BF16 and x.is_cuda:
-                    m = tk.linear_gelu_tanh(h, *self.vis_lowp[lp + "mlp.fc1"])
+                if self.vis_dense and not self.vit_lowp_attn:
+                    # fc1 with the tanh-GELU on its 16-bit output (gelu(fc1(h)) on 16-bit tensors), then fc2: two
+                    # launches of the many-row kernel in the tier's type
+                    w1, b1 = self.vis_dense[lp + "mlp.fc1"]
+                    w2, b2 = self.vis_dense[lp + "mlp.fc2"]
+                    m = tk.bf16w_dense(h.view(-1, vh), w1, b1, "gelu_tanh", ws=self.ws)
+                    x = x + tk.bf16w_dense(m, w2, b2, ws=self.ws).view(x.shape)  # fp32 + 16-bit: promoted inside the add
                 else:
                     m = F.gelu(F.linear(h, *self.vis_lowp[lp + "mlp.fc1"]), approximate="tanh")
-                x = x + F.linear(m, *self.vis_lowp[lp + "mlp.fc2"])  # fp32 + low precision: promoted inside the add
+                    x = x + F.linear(m, *self.vis_lowp[lp + "mlp.fc2"])  # fp32 + low precision: promoted inside the add
             else:
                 h = F.layer_norm(x, (vh,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], EPS)
                 x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
@@ -285,14 +298,20 @@ class PI05Model:
         return self.lin(PROJ, x)
 
     def _tower_bf16_linears(self, x: torch.Tensor) -> torch.Tensor:
-        """The tower with every linear in bf16 (both low-precision tiers on): fp32 residual stream updated
-        in place, each residual add in the launch of the LayerNorm that follows it, attention on the HIP
-        kernel (fp32 scores and softmax, probabilities rounded to bf16 for P.V)."""
+        """The fused tower (``tl_fused_vit``), after the reference's (tybok/policies/pi05/models/vision.py:120-173,
+        237-273; triton_vision.py): q|k|v and the attention on fp16 operands (fp32 scores and softmax, probabilities
+        rounded to fp16 for P.V, bf16 attention output), out_proj / fc1 / fc2 on bf16 operands with the GELU on fc1's
+        fp32 pre-activation; fp32 residual stream updated in place, each residual add in the launch of the LayerNorm
+        that follows it.  Two things are rounded once more than there: the out_proj and fc2 results pass through bf16
+        before they join the fp32 residual stream (the reference's kernels add the residual to the fp32 accumulator),
+        and the post-LayerNorm + projector stay the fp32 pair of the unfused tower (its fused projector runs bf16
+        operands)."""
         cfg, p = self.cfg, self.p
         b, vh, heads, hp = x.shape[0], cfg.vision_hidden, cfg.vision_heads, self.vis_head_pad
         hd = vh // heads
         ln = lambda i, n: (p[f"{VIS}encoder.layers.{i}.layer_norm{n}.weight"], p[f"{VIS}encoder.layers.{i}.layer_norm{n}.bias"])  # noqa: E731
-        h = tk.layer_norm(x, *ln(0, 1), EPS)
+        qdt = self.vit_qkv_dtype
+        h = tk.layer_norm(x, *ln(0, 1), EPS, out_dtype=qdt)
 
         def dense(name: str, t: torch.Tensor, act: str | None = None) -> torch.Tensor:
             if self.vis_dense:
@@ -307,10 +326,11 @@ class PI05Model:
             qkv = dense(lp + "self_attn.qkv", h).view(b, -1, 3, heads, hp)
             a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], tk.transpose_v(qkv[:, :, 2]), scale=hd**-0.5, ws=self.ws)
             x, h = tk.add_layer_norm(x, dense(lp + "self_attn.out_proj", a), *ln(i, 2), EPS)
-            # fc1's GELU on the bf16-rounded linear output: the eager tier's gelu(fc1(h)) on bf16 tensors (vision.py:79-87)
-            m = dense(lp + "mlp.fc2", dense(lp + "mlp.fc1", h, "gelu_tanh"))
+            # fc1's GELU on the fp32 pre-activation, the activation rounded to bf16 for fc2: the reference's fused MLP
+            # (`_vision_mlp_up_kernel`, tybok/policies/pi05/models/triton_vision.py:113-187)
+            m = dense(lp + "mlp.fc2", dense(lp + "mlp.fc1", h, "gelu_tanh_fp32"))
             if i + 1 < cfg.vision_layers:
-                x, h = tk.add_layer_norm(x, m, *ln(i + 1, 1), EPS)
+                x, h = tk.add_layer_norm(x, m, *ln(i + 1, 1), EPS, out_dtype=qdt)
             else:
                 x = x + m
         x = F.layer_norm(x, (vh,), p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], EPS)
