@@ -306,6 +306,28 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
   SMARK(6);
 
   // ---- epilogue: this lane finishes row m, four groups of four columns ----
+  if (a.vec && a.vec16 && a.N % 8 == 0) {
+    // rows of y that keep 16-byte alignment: the block's 64 x 64 bf16 tile passes through LDS and leaves as whole
+    // 128-byte lines (8 lanes x 16 bytes per row), not as 16-byte pieces of 32 different rows per instruction
+    constexpr int OP = 64 * 2 + 16;  // row pitch of the output tile (bytes)
+    unsigned char* otile = lds + 4 * 4 * 64 * 16;  // behind the exchange area
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      i32x2 r = pack_bf16x4(own[g] * e_sc[g]);
+      if (a.gate) r = pack_bf16x4(unpack_bf16x4(r) * unpack_bf16x4(e_gate[g]));
+      if (a.resid) r = pack_bf16x4(unpack_bf16x4(r) + e_rv[g]);
+      *(i32x2*)(otile + m * OP + (nt * 32 + 8 * g + 4 * half) * 2) = r;
+    }
+    lds_barrier();
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {  // wave w stores rows 16w .. 16w+15
+      const int row = wave * 16 + h2 * 8 + (lane >> 3), n = strip * 64 + (lane & 7) * 8;
+      const i32x4 v = *(const i32x4*)(otile + row * OP + (lane & 7) * 16);
+      if (row < a.M && n < a.N) *(i32x4*)(a.y + (size_t)row * a.ldy + n) = v;
+    }
+    SMARK(7);
+    return;
+  }
   if (m < a.M) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
@@ -349,6 +371,7 @@ static const int kStreamRounds[] = {16, 8, 0};
 
 bool tk_gemm_stream_takes(const GemmArgs& a) {
   if (a.w16 || a.s1 != nullptr || a.rope_pos != nullptr || a.norm_w != nullptr || a.ada_scale != nullptr || a.x_f32) return false;
+  if (!a.vec) return false;  // the column scales are requested as 16-byte vectors before the loop
   if (a.M > 64 || a.M < 1 || ((size_t)a.M * a.ldx + a.K) * 2 >= 0x7f000000ull || a.N < 64 || a.K % 32 != 0 || a.kt_r != 0 || a.kt_q % 4 != 0) return false;
   for (const int* r = kStreamRounds; *r; ++r)
     if (a.kt_q == 4 * *r) return true;
