@@ -50,10 +50,12 @@ def spin_up(ms: float = 150.0) -> None:
         torch.cuda.synchronize()
 
 
-def gemm_launch_us(m: int, k: int, n: int, launches: int = 100, reps: int = 10, cold: bool = True) -> float:
-    """Average duration (us) of one fp8-weight GEMM launch inside a replayed graph."""
+def gemm_launch_us(m: int, k: int, n: int, launches: int = 100, reps: int = 10, cold: bool = True, cut: int = 0) -> float:
+    """Average duration (us) of one fp8-weight GEMM launch inside a replayed graph.  ``cut`` = 1..4 times a
+    measurement form of the weight-streaming kernel instead (its loads only ... everything but its tail)."""
     import torch
 
+    from tybok_amd import native
     from tybok_amd import ops as tk
     from tybok_amd.quant import quantize_weight_rows
 
@@ -65,16 +67,26 @@ def gemm_launch_us(m: int, k: int, n: int, launches: int = 100, reps: int = 10, 
     pws = [base] + [tk.PackedWeight(base.data.clone(), base.scale, base.n, base.k) for _ in range(copies - 1)]
     out = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
     stream = torch.cuda.Stream()
+
+    def launch(i: int) -> None:
+        pw = pws[i % copies]
+        if cut:
+            rc = native.lib().tk_debug_fp8w_gemm_cut(x.data_ptr(), k, pw.data.data_ptr(), pw.scale.data_ptr(), out.data_ptr(), n, m, n, k, cut,
+                                                     torch.cuda.current_stream().cuda_stream)
+            native.check(rc, "tk_debug_fp8w_gemm_cut")
+        else:
+            tk.fp8w_gemm(x, pw, out=out)
+
     with torch.cuda.stream(stream):
         for i in range(3):
-            tk.fp8w_gemm(x, pws[i % copies], out=out)
+            launch(i)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     # the engines capture under inference_mode; capturing outside it afterwards trips torch's
     # graph-safe RNG state (an in-place update of an inference tensor)
     with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
         for i in range(launches):
-            tk.fp8w_gemm(x, pws[i % copies], out=out)
+            launch(i)
     spin_up(60.0)  # capture and allocation idle the GPU long enough for its clocks to drop
     for _ in range(3):
         graph.replay()
@@ -419,6 +431,7 @@ def main() -> None:
     ap.add_argument("--skip-pi05", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--gemm-only", action="store_true", help="only the roofline GEMM loop plus a plain copy of known size (for rocprofv3 runs)")
+    ap.add_argument("--gemm-cuts", action="store_true", help="with --gemm-only: also time the measurement forms of the weight-streaming kernel (K = 2048 shapes)")
     ap.add_argument("--gemm-shape", type=int, nargs=3, metavar=("M", "K", "N"), default=(50, 2048, 16384), help="shape of the --gemm-only loop")
     ap.add_argument("--attn-only", action="store_true", help="only the action-expert attention loop (for rocprofv3 runs)")
     ap.add_argument("--attn-d256-only", action="store_true", help="only the pi0.5 action-expert attention loop, 256-wide heads (for rocprofv3 runs)")
@@ -449,8 +462,14 @@ def main() -> None:
         gm, gk, gn = args.gemm_shape
         us = gemm_launch_us(gm, gk, gn, launches=20, reps=args.steps)
         sc = stream_read_us(gk * gn, launches=20, reps=args.steps)
-        print(json.dumps({"gemm_only": {"M": gm, "K": gk, "N": gn, "us": round(us, 2), "GBps": round(bytes_gemm(gm, gk, gn) / us / 1e3, 1),
-                                        "stream_read_us": round(sc, 2), "stream_read_GBps": round(gk * gn / sc / 1e3, 1)}}), flush=True)  # fmt: skip
+        line = {"M": gm, "K": gk, "N": gn, "us": round(us, 2), "GBps": round(bytes_gemm(gm, gk, gn) / us / 1e3, 1),
+                "stream_read_us": round(sc, 2), "stream_read_GBps": round(gk * gn / sc / 1e3, 1)}  # fmt: skip
+        if args.gemm_cuts:
+            # the same kernel with the work behind a point dropped: where its time above the plain read goes
+            names = {1: "loads_and_barrier_us", 2: "plus_lds_staging_us", 3: "plus_lds_operand_reads_us", 4: "plus_convert_and_mfma_us"}
+            line["cuts"] = {names[c]: round(gemm_launch_us(gm, gk, gn, launches=20, reps=args.steps, cut=c), 2) for c in (1, 2, 3, 4)}
+            line["cuts"]["whole_kernel_us"] = line["us"]
+        print(json.dumps({"gemm_only": line}), flush=True)
         return
     if args.ffn_only:
         spin_up()
@@ -557,7 +576,7 @@ def main() -> None:
     achieved = bytes_gemm(50, rk, rn) / r_us / 1e3
     roofline = {
         "bound": "hbm",
-        "kernel": "fp8w_gemm_kernel (M=50, K=2048, N=16384, cold weights)",
+        "kernel": "fp8w_stream_kernel (M=50, K=2048, N=16384, cold weights)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
@@ -579,7 +598,7 @@ def main() -> None:
     roofline["frac_of_stream_ceiling"] = round(achieved / sc_gbps, 4)
     k2, n2 = 16384, 2048
     a2 = sweep[f"K{k2}_N{n2}"]["GBps"]
-    roofline["other_33MB_shape"] = {"kernel": "fp8w_gemm_kernel (M=50, K=16384, N=2048, cold weights)", "achieved": a2, "frac": round(a2 / HBM_PEAK_GBS, 4), "frac_of_stream_ceiling": round(a2 / sc_gbps, 4)}
+    roofline["other_33MB_shape"] = {"kernel": "fp8w_stream_kernel, 8 K-splits (M=50, K=16384, N=2048, cold weights)", "achieved": a2, "frac": round(a2 / HBM_PEAK_GBS, 4), "frac_of_stream_ceiling": round(a2 / sc_gbps, 4)}
     traffic_file = os.path.join(ROOT, "profiles", "fp8w_gemm_traffic.json")
     if os.path.exists(traffic_file):
         with open(traffic_file, encoding="utf-8") as f:

@@ -466,6 +466,16 @@ int tk_debug_decode_fp8(void* out_f32, void* stream);
  * `sink` (int32, may be NULL) is never written for real data.  No counterpart in the reference. */
 int tk_debug_stream_read(const void* src, size_t bytes, int blocks, void* sink, void* stream);
 
+/* Measurement forms of the weight-streaming fp8 GEMM (the kernel tk_fp8w_gemm launches for 33..64 rows
+ * over a large matrix): same grid, same schedule, the work behind a point dropped.  cut 1 = the weight
+ * and activation loads and the barrier per round only; 2 = + activations staged into LDS; 3 = + operands
+ * read back from LDS; 4 = + fp8 -> bf16 conversion and the matrix instructions (no exchange between
+ * waves, no scales, no output).  Nothing is written to y.  Timed by `bench.py --gemm-only` beside the
+ * whole kernel to show where its time above a plain read of the weights goes.  Only unsplit launches of
+ * the 16-round kernel (K = 2048, M <= 64, N >= 64); TK_EINVAL otherwise.  No counterpart in the reference. */
+int tk_debug_fp8w_gemm_cut(const void* x, int ldx, const void* w_packed, const void* scale, void* y, int ldy,
+                           int M, int N, int K, int cut, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

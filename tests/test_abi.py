@@ -116,6 +116,7 @@ def _cases():
         ("tk_bf16w_dense", dense(y=P + 8), -1, "16-byte aligned"),
         ("tk_fp8w_gemm_static", static(M=65), -1, "exceeds the 64 rows"),
         ("tk_debug_stream_read", sread(bytes=1000), -1, "multiple"),
+        ("tk_debug_fp8w_gemm_cut", (P, 2040, P, P, P, 16384, 50, 16384, 2040, 1, None), -1, "multiple of 16"),
         ("tk_fp8w_gemm", gemm(K=2040), -1, "multiple of 16"),
         ("tk_fp8w_gemm", gemm(ldx=1024), -1, "ldx"),
         ("tk_fp8w_gemm", gemm(x=P + 2), -1, "16-byte aligned"),

@@ -99,7 +99,7 @@ def test_single_launch_ffn_reads_this_launch_s_intermediate_not_an_older_one():
         # and under graph replay, where the launches follow each other most closely
         stream = torch.cuda.Stream()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
+        with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
             for _ in range(4):
                 for j, (_, _, wgu, wd, kw) in enumerate(cases):
                     tk.fp8w_gated_ffn(xs[j], wgu, wd, "silu", ws=ws, out=outs[j], **kw)
@@ -123,7 +123,7 @@ def test_single_launch_ffn_replays_in_a_graph():
     out = torch.zeros_like(eager)
     stream = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, stream=stream):
+    with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
         for _ in range(3):  # three dependent FFNs back to back, as consecutive layers launch them
             tk.fp8w_gated_ffn(xg, wgu, wd, "silu", ws=ws, out=out, **kw)
     for _ in range(3):

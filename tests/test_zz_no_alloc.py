@@ -84,7 +84,7 @@ def test_static_scratch_split_launch_replays_in_a_graph():
     out = torch.zeros(50, 1024, dtype=torch.bfloat16, device="cuda")
     stream = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, stream=stream):
+    with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
         st = torch.cuda.current_stream().cuda_stream
         native.check(lib.tk_fp8w_gemm_static(xg.data_ptr(), 4096, w.data.data_ptr(), w.scale.data_ptr(), out.data_ptr(), 1024, None, 0, 0, None, 50, 1024, 4096, 8, st), "tk_fp8w_gemm_static")
     x2, w82, s2 = gemm_case(16, 2048, 2048)

@@ -40,7 +40,12 @@ extern "C" int tk_debug_read_phases_s(void* host_out) {
 namespace {
 
 // waits for this wave's LDS traffic only, not for its global loads in flight
+template <bool LDS = true>
 __device__ __forceinline__ void lds_barrier() {
+  if constexpr (!LDS) {
+    __builtin_amdgcn_s_barrier();
+    return;
+  }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -59,7 +64,11 @@ constexpr int stream_issued(int r, int NR, int PF, int PRE) {
 
 // NR: rounds of four k tiles every block walks (host: KT == ksplit * 4 * NR).  PF: rounds of loads in flight.
 // PRE: rounds requested before the first one is staged.
-template <int NR, int PF, int PRE>
+// CUT: 0 in every launch of the product.  1..4 build the measurement forms that show where the time above the plain
+// weight stream goes; each keeps the schedule and drops the work behind a point, folding what it loaded into a word
+// that is never stored: 1 = the loads and the barrier per round only, 2 = + activations staged into LDS, 3 = +
+// operands read back from LDS, 4 = + conversion and matrix instructions (no exchange, no scales, no output).
+template <int NR, int PF, int PRE, int CUT = 0>
 __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
   constexpr int ROWS = 64;
   constexpr int PITCH = 4 * 64 + 16;  // LDS row pitch (bytes) of a round's 128 staged bf16 columns
@@ -112,6 +121,12 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
   i32x4 xg[PF][XPT];    // activation pieces in flight
   i32x4 xa[2][2][2][2]; // operands [round parity][k tile j][row tile][16-byte chunk]
   bf16x8 wb[2][2][2];   // converted weights [round parity][k tile j][chunk]
+  i32x4 sink = {0, 0, 0, 0};  // CUT != 0: what the dropped work would have consumed
+  // folds v into the sink where the dropped work would have used it (pinned: the fold may not drift to the end)
+  auto fold = [&](const i32x4& v) {
+    sink ^= v;
+    asm volatile("" : "+v"(sink));
+  };
 
   auto load_w = [&](int r) {
     wg[r % PF][0] = *(const i32x4*)(wptr + (size_t)r * 4096);
@@ -125,9 +140,13 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
   auto stage = [&](int r) {
 #pragma unroll
     for (int i = 0; i < XPT; ++i)
-      if (i < XSKIP || xlive[i]) *(i32x4*)(lds + (r % NBUF) * XBUF + xdst[i]) = xg[r % PF][i];
+      if (i < XSKIP || xlive[i]) {
+        if constexpr (CUT == 1) fold(xg[r % PF][i]);
+        else *(i32x4*)(lds + (r % NBUF) * XBUF + xdst[i]) = xg[r % PF][i];
+      }
   };
   auto read_ops = [&](int r, int j) {
+    if constexpr (CUT == 1 || CUT == 2) return;
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
       const i32x4* p = (const i32x4*)(lds + (r % NBUF) * XBUF + mt * 32 * PITCH + rd_off + j * 64);
@@ -136,11 +155,19 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
     }
   };
   auto convert = [&](int r, int j) {
+    if constexpr (CUT >= 1 && CUT <= 3) {
+      fold(wg[r % PF][j]);
+      return;
+    }
     wb[r & 1][j][0] = fp8x8_to_bf16x8(wg[r % PF][j][0], wg[r % PF][j][1]);
     wb[r & 1][j][1] = fp8x8_to_bf16x8(wg[r % PF][j][2], wg[r % PF][j][3]);
   };
   auto product = [&](int r, int s) {  // product s of round r: k tile j, chunk h2, row tile mt
     const int j = s >> 2, h2 = (s >> 1) & 1, mt = s & 1;
+    if constexpr (CUT >= 1 && CUT <= 3) {
+      if constexpr (CUT == 3) fold(xa[r & 1][j][mt][h2]);
+      return;
+    }
     acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[r & 1][j][h2], as_bf16x8(xa[r & 1][j][mt][h2]), acc[mt], 0, 0, 0);
   };
 
@@ -164,7 +191,7 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
   }
   SMARK(1);
   stage(0);
-  lds_barrier();
+  lds_barrier<CUT != 1>();
   read_ops(0, 0);
   read_ops(0, 1);
   convert(0, 0);
@@ -181,7 +208,7 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
     SLOT_END();
     product(r, 1);
     SLOT_END();
-    if (nxt) lds_barrier();
+    if (nxt) lds_barrier<CUT != 1>();
     SLOT_END();
     product(r, 2);
     if (nxt) read_ops(r + 1, 0);
@@ -209,6 +236,19 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
     SLOT_END();
   }
   SMARK(3);
+  if constexpr (CUT != 0) {  // measurement forms end here; the store never happens, it only keeps the work alive
+    float t = 0.f;
+    if constexpr (CUT == 4) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) t += acc[0][i] + acc[1][i];
+    }
+    if constexpr (CUT == 2) {  // staged but never read back: one read keeps the staging stores alive
+      lds_barrier();
+      sink[0] ^= *(const int*)(lds + tid * 4);
+    }
+    if ((sink[0] ^ sink[1] ^ sink[2] ^ sink[3]) == 0x12345678 || t == 1.2345e-30f) a.y[0] = 0;
+    return;
+  }
 
   // ---- the optional epilogue operands (gate, residual) of this wave's tile ----
   const int m = kh * 32 + l32;
@@ -376,6 +416,17 @@ bool tk_gemm_stream_takes(const GemmArgs& a) {
   for (const int* r = kStreamRounds; *r; ++r)
     if (a.kt_q == 4 * *r) return true;
   return false;
+}
+
+// Measurement forms of the 16-round kernel (cut = 1..4, see the kernel's CUT parameter); nothing is written to y.
+int tk_launch_gemm_stream_cut(GemmArgs a, int cut, hipStream_t st) {
+  if (!tk_gemm_stream_takes(a) || a.kt_q != 64 || cut < 1 || cut > 4) return -1;
+  dim3 grid((a.ntiles + 1) / 2, a.ksplit, 1);
+  if (cut == 1) hipLaunchKernelGGL((fp8w_stream_kernel<16, kStreamPF, kStreamPRE, 1>), grid, dim3(256), 0, st, a);
+  else if (cut == 2) hipLaunchKernelGGL((fp8w_stream_kernel<16, kStreamPF, kStreamPRE, 2>), grid, dim3(256), 0, st, a);
+  else if (cut == 3) hipLaunchKernelGGL((fp8w_stream_kernel<16, kStreamPF, kStreamPRE, 3>), grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((fp8w_stream_kernel<16, kStreamPF, kStreamPRE, 4>), grid, dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
 int tk_launch_gemm_stream(GemmArgs a, hipStream_t st) {

@@ -1225,6 +1225,17 @@ int tk_debug_stream_read(const void* src, size_t bytes, int blocks, void* sink, 
   return TK_OK;
 }
 
+int tk_debug_fp8w_gemm_cut(const void* x, int ldx, const void* w_packed, const void* scale, void* y, int ldy, int M, int N, int K,
+                           int cut, void* stream) {
+  GemmPlan plan;
+  const int rc = gemm_common(x, ldx, w_packed, (const float*)scale, nullptr, y, ldy, nullptr, 0, 0, nullptr, M, N, K, 0, 0, nullptr, 0,
+                             (hipStream_t)stream, GemmExtra(), &plan);
+  if (rc) return rc;
+  if (plan.skinny || plan.a.ksplit != 1 || tk_launch_gemm_stream_cut(plan.a, cut, (hipStream_t)stream))
+    return fail(TK_EINVAL, "gemm_cut: only for shapes the 16-round weight-streaming kernel takes unsplit (K = 2048, at most 64 rows), cut 1..4");
+  return TK_OK;
+}
+
 int tk_debug_decode_fp8(void* out_f32, void* stream) {
   if (!out_f32) return fail(TK_EINVAL, "decode: null pointer");
   if (tk_launch_decode_fp8((float*)out_f32, (hipStream_t)stream)) return fail(TK_ELAUNCH, "decode: launch failed");

@@ -232,6 +232,7 @@ int tk_launch_ffn_fused(GemmArgs g, GemmArgs d, int d_nt, int mblocks, hipStream
 // software-pipelined kernel of fp8w_gemm_stream.hip (same grid and partial layout as tk_launch_gemm with MT = NT = 2)
 bool tk_gemm_stream_takes(const GemmArgs& a);
 int tk_launch_gemm_stream(GemmArgs a, hipStream_t st);
+int tk_launch_gemm_stream_cut(GemmArgs a, int cut, hipStream_t st);  // measurement forms, nothing stored
 // W8A8 tier: per-token activation quantisation and the fp8 x fp8 many-row GEMM (block tile 32 * mtiles x tk_w8a8_cols())
 int tk_w8a8_cols();
 int tk_quant_act_max_k();

@@ -131,6 +131,7 @@ SIGNATURES: dict[str, tuple] = {
     ),  # fmt: skip
     "tk_debug_decode_fp8": (c_int, [c_void_p, c_void_p]),
     "tk_debug_stream_read": (c_int, [c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
+    "tk_debug_fp8w_gemm_cut": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
 }
 
 
