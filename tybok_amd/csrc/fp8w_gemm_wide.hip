@@ -11,8 +11,11 @@
 //     whole 128-byte lines per row, double buffered, one LDS barrier per round;
 //   * blocks that share weights (same n tiles and k range, different rows) get consecutive slots of
 //     ONE XCD, so the weight tiles are read from HBM once and served from that XCD's L2 afterwards;
-//   * K splits (few column blocks, long K: the down projection) hand fp32 partials through the
-//     workspace; the last-arriving block sums them in split order -- bit-deterministic.
+//   * K splits (few column blocks, long K: the down projection) leave fp32 partials in the workspace and a
+//     second launch over all CUs sums them in split order and runs the epilogue -- bit-deterministic.  (A
+//     gated launch that is split keeps the one-launch form: the last-arriving block sums.  Measured at
+//     M=712, K=16384, N=2048, 5 splits: 74 -> 52 + 7.7 us; one block per output tile -- 48 of 256 CUs -- pulling
+//     31 MB of partials through 8-byte coherent loads, split after split, was a fifth of the launch.)
 // The epilogues compute exactly what the skinny kernel's do (same rounding points).
 #include "tk_common.h"
 #include "tk_kernels.h"
@@ -223,6 +226,19 @@ __global__ __launch_bounds__(NW * 64, OCC) void fp8w_wide_kernel(GemmArgs a, int
 
   // ---- K-split hand-off: fp32 partials [(block, split)][wave][tile][group][lane][4] ----
   const int blk_lin = nblk * nblk_m + mblock;
+  if (a.ksplit > 1 && a.split_reduce) {
+    // the partial leaves as it is (plain 16-byte stores: the kernel boundary publishes it); wide_split_reduce_kernel
+    // finishes
+    f32x4* mine = (f32x4*)a.partial + ((size_t)blk_lin * a.ksplit + split) * (NW * TILES * 4 * 64) + (size_t)wave * TILES * 4 * 64 + lane;
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& c = acc[t / NT][t % NT];
+        mine[(t * 4 + g) * 64] = f32x4{c[4 * g], c[4 * g + 1], c[4 * g + 2], c[4 * g + 3]};
+      }
+    return;
+  }
   if (a.ksplit > 1) {
     unsigned long long* pbase = (unsigned long long*)a.partial + ((size_t)wave * TILES * 4 * 64 + lane) * 2;
     unsigned long long* mine = pbase + ((size_t)blk_lin * a.ksplit + split) * (NW * TILES * 4 * 64 * 2);
@@ -421,6 +437,51 @@ __global__ __launch_bounds__(NW * 64, OCC) void fp8w_wide_kernel(GemmArgs a, int
   }
 }
 
+// Second launch of a K-split plain GEMM (GemmArgs::split_reduce): thread (block tile, wave, tile, lane) sums its four
+// register groups over the splits in split order -- the order and the arithmetic of the last-arriving block of the
+// one-launch form, so the same bits -- and finishes them like the scattered epilogue above.  Every CU takes part.
+template <int MT>
+__global__ __launch_bounds__(256) void wide_split_reduce_kernel(GemmArgs a, int nblk_m, int nthreads) {
+  constexpr int TILES = MT * NT;
+  const int gid = blockIdx.x * 256 + threadIdx.x;
+  if (gid >= nthreads) return;
+  const int lane = gid & 63, half = lane >> 5, l32 = lane & 31;
+  const int t = (gid >> 6) % TILES;
+  const int wave = (gid >> 6) / TILES % NW;
+  const int blk_lin = (gid >> 6) / (TILES * NW);
+  const int mblock = blk_lin % nblk_m, nblk = blk_lin / nblk_m;
+  const int mt = t / NT, nt = t % NT;
+  const int strip = nblk * NW + wave;
+  const f32x4* src = (const f32x4*)a.partial + (size_t)blk_lin * a.ksplit * (NW * TILES * 4 * 64) + (size_t)wave * TILES * 4 * 64 + (size_t)t * 4 * 64 + lane;
+  f32x4 sum[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) sum[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int s = 0; s < a.ksplit; ++s) {
+    f32x4 p[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) p[g] = src[(size_t)s * (NW * TILES * 4 * 64) + g * 64];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) sum[g] += p[g];
+  }
+  const int m = (mblock * MT + mt) * 32 + l32;
+  if (m >= a.M) return;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int n0 = (strip * NT + nt) * 32 + 8 * g + 4 * half;
+    if (n0 >= a.N) continue;
+    const f32x4 sc = *(const f32x4*)(a.s0 + n0);
+    i32x2 r = pack_bf16x4(sum[g] * sc);
+    if (a.gate) r = pack_bf16x4(unpack_bf16x4(r) * unpack_bf16x4(*(const i32x2*)(a.gate + n0)));
+    if (a.resid) {
+      const f32x4 rv = a.resid_f32 ? *(const f32x4*)((const float*)a.resid + (size_t)m * a.ldr + n0)
+                                   : unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n0));
+      r = pack_bf16x4(unpack_bf16x4(r) + rv);
+    }
+    *(i32x2*)(a.y + (size_t)m * a.ldy + n0) = r;
+  }
+}
+
 // One block per row: out = bf16 norm of the bf16 row, with the rounding points of the skinny
 // kernel's prologues: RMSNorm bf16(w * bf16(x * rstd)); adaptive bf16((x * rstd) * (1 + scale) + shift).
 // A thread's first piece of the row and the norm's operands for it are requested together up front and stay in
@@ -512,6 +573,8 @@ int tk_launch_gemm_wide(GemmArgs a, hipStream_t st) {
   const int nblk_n = (a.ntiles + NW * NT - 1) / (NW * NT);
   const int ngroups = nblk_n * a.ksplit;
   const dim3 grid((unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m), block(NW * 64);
+  // K splits of a plain launch with 4-column alignment: partials out, then a reduction launch over all CUs
+  a.split_reduce = a.ksplit > 1 && !a.s1 && a.vec && a.N % 4 == 0;
   if (a.s1) {
     if (a.mtiles == 4)
       hipLaunchKernelGGL((fp8w_wide_kernel<1, 4, 4, 1>), grid, block, 0, st, a, nblk_m, ngroups);
@@ -522,6 +585,11 @@ int tk_launch_gemm_wide(GemmArgs a, hipStream_t st) {
       hipLaunchKernelGGL((fp8w_wide_kernel<0, 4, 4, 1>), grid, block, 0, st, a, nblk_m, ngroups);
     else
       hipLaunchKernelGGL((fp8w_wide_kernel<0, 2, 4, 2>), grid, block, 0, st, a, nblk_m, ngroups);
+  }
+  if (a.split_reduce) {
+    const int nthreads = nblk_n * nblk_m * NW * a.mtiles * NT * 64;
+    if (a.mtiles == 4) hipLaunchKernelGGL((wide_split_reduce_kernel<4>), dim3((nthreads + 255) / 256), dim3(256), 0, st, a, nblk_m, nthreads);
+    else hipLaunchKernelGGL((wide_split_reduce_kernel<2>), dim3((nthreads + 255) / 256), dim3(256), 0, st, a, nblk_m, nthreads);
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }

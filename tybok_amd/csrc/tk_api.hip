@@ -218,7 +218,8 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
     // 64-row blocks, two per CU, once the 128-row grid would run in several generations anyway: co-resident
     // blocks cover each other's first loads and epilogue; few blocks keep the 128-row tile
     a.mtiles = wide_blocks >= 2 * cus ? 2 : 4;
-    const int blocks0 = a.mtiles == 4 ? wide_blocks : ((a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols()) * ((M + 63) / 64);
+    const int brows = a.mtiles * 32;
+    const int blocks0 = ((a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols()) * ((M + brows - 1) / brows);
     int ks = split_k;
     if (ks <= 0) {
       // fill the device once; a split keeps at least 16 k tiles and its partials must fit
@@ -226,7 +227,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
       if (ks > a.KT / 16) ks = a.KT / 16;
       if (ks < 1) ks = 1;
     }
-    const size_t per_split = (size_t)a.mtiles * 32 * tk_wide_cols() * 4;
+    const size_t per_split = (size_t)brows * tk_wide_cols() * 4;
     if (ks > 1 && ws) {
       const size_t fit = kPartialBytes / (per_split * blocks0);
       const size_t have = ws_bytes > kPartialOff ? (ws_bytes - kPartialOff) / (per_split * blocks0) : 0;

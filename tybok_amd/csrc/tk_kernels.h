@@ -61,6 +61,9 @@ struct GemmArgs {
   // block, and the bound on a down block's wait (polls)
   int* fuse;
   int fuse_consumers, fuse_spin;
+  // many-row fp8 kernels, K splits of a plain launch: 1 = every block leaves its fp32 partial in `partial` and ends;
+  // a second launch (all CUs, not one block per output tile) sums them in split order and runs the epilogue
+  int split_reduce;
 };
 // int32 words of the single-launch FFN's hand-off: a flag per (row block, gate/up strip), the number of down blocks
 // past their wait per row block, then the sticky error word

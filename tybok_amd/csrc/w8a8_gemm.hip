@@ -200,6 +200,19 @@ __global__ __launch_bounds__(NW * 64, OCC) void w8a8_wide_kernel(GemmArgs a, int
 
   // ---- K-split hand-off: fp32 partials [(block, split)][wave][tile][group][lane][4], last arriver sums in split order
   const int blk_lin = nblk * nblk_m + mblock;
+  if (a.ksplit > 1 && a.split_reduce) {
+    // the partial leaves as it is (plain 16-byte stores: the kernel boundary publishes it); w8a8_split_reduce_kernel
+    // finishes
+    f32x4* mine = (f32x4*)a.partial + ((size_t)blk_lin * a.ksplit + split) * (NW * TILES * 4 * 64) + (size_t)wave * TILES * 4 * 64 + lane;
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& c = acc[t / NT][t % NT];
+        mine[(t * 4 + g) * 64] = f32x4{c[4 * g], c[4 * g + 1], c[4 * g + 2], c[4 * g + 3]};
+      }
+    return;
+  }
   if (a.ksplit > 1) {
     unsigned long long* pbase = (unsigned long long*)a.partial + ((size_t)wave * TILES * 4 * 64 + lane) * 2;
     unsigned long long* mine = pbase + ((size_t)blk_lin * a.ksplit + split) * (NW * TILES * 4 * 64 * 2);
@@ -414,6 +427,54 @@ __global__ __launch_bounds__(NW * 64, OCC) void w8a8_wide_kernel(GemmArgs a, int
 // One block per row.  MODE 0: sa = amax / 448 (fp32), a8 = RNE(x / sa) from fp32 -- one rounding.
 // MODE 1: the arithmetic of a torch expression on bf16 tensors, `s = x.abs().max() / 448` (a bf16 value) and
 // `(x / s).to(float8_e4m3fn)` (quotient rounded to bf16, then to fp8): sa = float(bf16(amax / 448)).
+// Second launch of a K-split plain W8A8 GEMM (GemmArgs::split_reduce): thread (block tile, wave, tile, lane) sums its
+// four register groups over the splits in split order -- the order and arithmetic of the last-arriving block of the
+// one-launch form, so the same bits -- and finishes them like the scattered epilogue above, on every CU.
+template <int MT>
+__global__ __launch_bounds__(256) void w8a8_split_reduce_kernel(GemmArgs a, int nblk_m, int nthreads) {
+  constexpr int TILES = MT * NT;
+  const int gid = blockIdx.x * 256 + threadIdx.x;
+  if (gid >= nthreads) return;
+  const int lane = gid & 63, half = lane >> 5, l32 = lane & 31;
+  const int t = (gid >> 6) % TILES;
+  const int wave = (gid >> 6) / TILES % NW;
+  const int blk_lin = (gid >> 6) / (TILES * NW);
+  const int mblock = blk_lin % nblk_m, nblk = blk_lin / nblk_m;
+  const int mt = t / NT, nt = t % NT;
+  const int strip = nblk * NW + wave;
+  const f32x4* src = (const f32x4*)a.partial + (size_t)blk_lin * a.ksplit * (NW * TILES * 4 * 64) + (size_t)wave * TILES * 4 * 64 + (size_t)t * 4 * 64 + lane;
+  f32x4 sum[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) sum[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int s = 0; s < a.ksplit; ++s) {
+    f32x4 p[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) p[g] = src[(size_t)s * (NW * TILES * 4 * 64) + g * 64];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) sum[g] += p[g];
+  }
+  const int m = (mblock * MT + mt) * 32 + l32;
+  if (m >= a.M) return;
+  const float sa = a.row_scale[m];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int n0 = (strip * NT + nt) * 32 + 8 * g + 4 * half;
+    if (n0 >= a.N) continue;
+    const f32x4 sc = *(const f32x4*)(a.s0 + n0);
+    f32x4 v = sum[g];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = mul_rn(mul_rn(v[j], sa), sc[j]);
+    i32x2 r = pack_bf16x4(v);
+    if (a.resid) {
+      const f32x4 rv = a.resid_f32 ? *(const f32x4*)((const float*)a.resid + (size_t)m * a.ldr + n0)
+                                   : unpack_bf16x4(*(const i32x2*)((const u16*)a.resid + (size_t)m * a.ldr + n0));
+      r = pack_bf16x4(unpack_bf16x4(r) + rv);
+    }
+    *(i32x2*)(a.y + (size_t)m * a.ldy + n0) = r;
+  }
+}
+
 constexpr int kQuantMaxPieces = 8;  // 16-byte pieces of a row per thread: K <= 8 * 256 * 8 = 16384
 __global__ __launch_bounds__(256) void quant_act_rows_kernel(QuantActArgs a) {
   __shared__ float part[4];
@@ -481,6 +542,7 @@ int tk_launch_w8a8_gemm(GemmArgs a, hipStream_t st) {
   const int nblk_n = (a.ntiles + NW * NT - 1) / (NW * NT);
   const int ngroups = nblk_n * a.ksplit;
   const dim3 grid((unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m), block(NW * 64);
+  a.split_reduce = a.ksplit > 1 && !a.s1;  // partials out, then a reduction launch over all CUs
   if (a.s1) {
     if (a.mtiles == 4)
       hipLaunchKernelGGL((w8a8_wide_kernel<1, 4, 1>), grid, block, 0, st, a, nblk_m, ngroups);
@@ -491,6 +553,11 @@ int tk_launch_w8a8_gemm(GemmArgs a, hipStream_t st) {
       hipLaunchKernelGGL((w8a8_wide_kernel<0, 4, 1>), grid, block, 0, st, a, nblk_m, ngroups);
     else
       hipLaunchKernelGGL((w8a8_wide_kernel<0, 2, 2>), grid, block, 0, st, a, nblk_m, ngroups);
+  }
+  if (a.split_reduce) {
+    const int nthreads = nblk_n * nblk_m * NW * a.mtiles * NT * 64;
+    if (a.mtiles == 4) hipLaunchKernelGGL((w8a8_split_reduce_kernel<4>), dim3((nthreads + 255) / 256), dim3(256), 0, st, a, nblk_m, nthreads);
+    else hipLaunchKernelGGL((w8a8_split_reduce_kernel<2>), dim3((nthreads + 255) / 256), dim3(256), 0, st, a, nblk_m, nthreads);
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
