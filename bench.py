@@ -538,7 +538,7 @@ def main() -> None:
     torch.cuda.empty_cache()
 
     # ---- pi0.5-shaped chunk ----
-    pi05_p50 = pi05_w8a8_p50 = pi05_mlp_tier_p50 = None
+    pi05_p50 = pi05_w8a8_p50 = pi05_mlp_tier_p50 = pi05_pad_free_p50 = None
     if not args.skip_pi05:
         ckpt5 = write_pi05_checkpoint(os.path.join(tmp, "pi05"), cameras=2, seed=0)
         flags5 = {k: v for k, v in flags.items() if k not in ("tl_llm_fused_attn", "tl_vit_oproj")}  # SmolVLA-only tiers
@@ -548,6 +548,16 @@ def main() -> None:
         frame5 = device_frame(eng5, 2)
         s5, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
         pi05_p50 = float(np.percentile(s5, 50))
+        del eng5
+        torch.cuda.empty_cache()
+        # the same cameras with --pad-free and a prompt of 40 tokens (a language block of 48 instead of 200: prefix
+        # 560 rows instead of 712); the first request records the (2 cameras, 48 tokens) shape
+        eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, pad_free=True, **flags5)
+        frame5p = dict(frame5)
+        frame5p["observation.language.tokens"] = torch.randint(0, eng5.config.vocab_size, (200,), generator=torch.Generator().manual_seed(1)).cuda()
+        frame5p["observation.language.attention_mask"] = torch.arange(200, device="cuda") < 40
+        s5p, _ = time_requests(eng5, frame5p, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 3)
+        pi05_pad_free_p50 = float(np.percentile(s5p, 50))
         del eng5
         torch.cuda.empty_cache()
         # the same request with the VLM MLP in W8A8 (activations quantised per token, fp8 x fp8 products): the
@@ -682,6 +692,7 @@ def main() -> None:
         "pi05_2cam_p50_ms": None if pi05_p50 is None else round(pi05_p50, 3),
         "pi05_tiers": "tl_fused_expert, tl_fp8_expert_mlp, tl_fp8_llm_mlp, tl_llm_flash_attn, tl_fused_vit",
         "pi05_2cam_w8a8_prefill_p50_ms": None if pi05_w8a8_p50 is None else round(pi05_w8a8_p50, 3),
+        "pi05_2cam_pad_free_40tok_p50_ms": None if pi05_pad_free_p50 is None else round(pi05_pad_free_p50, 3),
         "pi05_2cam_vit_mlp_bf16_tier_p50_ms": None if pi05_mlp_tier_p50 is None else round(pi05_mlp_tier_p50, 3),
         "gemm_sweep_M50": sweep,
         "ops_action_chunk_shape": ops_small,

@@ -321,12 +321,67 @@ def test_engine_api_and_graph_equals_eager(ckpt):
     chunk, normalized = graph.predict_action_chunk(frame, noise=noise, return_normalized=True)
     assert np.array_equal(chunk, a) and normalized.shape == (50, 7)
     with pytest.raises(NotImplementedError):
-        create_engine(ckpt, device="cuda", warmup=False, pad_free=True)
-    with pytest.raises(NotImplementedError):
         create_engine(ckpt, device="cuda", warmup=False, rtc_config={"enabled": True})
     with pytest.raises(ValueError):
         create_engine(ckpt, device="cuda", warmup=False, vit_mlp_dtype="fp8")
     assert create_engine(ckpt, device="cuda", warmup=False, vit_mlp_dtype="fp16").model.vit_mlp_dtype == torch.float16
+
+
+def test_pad_free_records_shapes_on_first_sight_and_graph_equals_eager(ckpt):
+    # pad_free (tybok/policies/pi05/engine.py:510-541,612-630): only the cameras a frame holds, language block on
+    # the grid of 16 tokens; one shape per requested camera count at start-up, shorter blocks and other camera
+    # counts recorded when a request first needs them; the recorded shape and the eager path build the same prefix
+    from tybok_amd.registry import create_engine
+
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_flash_attn=True, tl_fused_vit=True, pad_free=True)
+    eager = create_engine(ckpt, device="cuda", graph=False, warmup=False, **flags)
+    graph = create_engine(ckpt, device="cuda", graph=True, warmup=False, **flags)
+    assert list(graph._graph_runner.keys()) == [(2, 200)]
+    frame = eager._profile_frame(seed=3)
+    noise = torch.zeros(1, 50, 7)
+    # the synthetic tokenizer marks all 200 ids live; a prompt of 37 tokens goes in as the request's own language block
+    live, bucket = 37, 48
+    frame["observation.language.tokens"] = torch.randint(0, eager.config.vocab_size, (200,), generator=torch.Generator().manual_seed(5))
+    frame["observation.language.attention_mask"] = torch.arange(200) < live
+    a = eager.predict_action_chunk(frame, noise=noise)
+    for _ in range(2):
+        assert np.array_equal(a, graph.predict_action_chunk(frame, noise=noise))
+    assert (2, bucket) in list(graph._graph_runner.keys())
+    # one camera missing from the frame: a one-camera prefix, not a placeholder slot
+    one = {k: v for k, v in frame.items() if not k.endswith("left_wrist_0_rgb")}
+    b = eager.predict_action_chunk(one, noise=noise)
+    assert np.array_equal(b, graph.predict_action_chunk(one, noise=noise))
+    assert (1, bucket) in list(graph._graph_runner.keys())
+    assert np.isfinite(b).all() and not np.array_equal(a, b)
+    # the flag off on the same frame: the full 200-token block (another reduction length: close, not equal)
+    full = create_engine(ckpt, device="cuda", graph=False, warmup=False, **{**flags, "pad_free": False})
+    c = full.predict_action_chunk(frame, noise=noise)
+    d = float(np.abs(a - c).max())
+    print(f"pad_free vs full language block ({live} live tokens, block of {bucket}): max|diff| = {d:.3g} of |chunk|max {float(np.abs(c).max()):.3g}")
+    assert 0.0 < d <= 2e-2 * max(1.0, float(np.abs(c).max()))
+
+
+def test_skip_empty_images_on_the_eager_path(ckpt):
+    # eager path: the placeholder slot of a missing camera skips the vision tower (flow_matching.py:415-437); under
+    # graph the flag is accepted and inert.  The empty slot is pad-masked out of every attention, so nothing of it
+    # reaches the chunk -- but this backend embeds all cameras in ONE pass of the tower and picks GEMM tiles by row
+    # count, so with a slot skipped the remaining camera's embedding is summed in another order: the chunks agree to
+    # bf16 noise, not to the bit (the torch path does: tests/test_pi05_request_shape.py); with every camera present
+    # the flag changes nothing at all
+    from tybok_amd.registry import create_engine
+
+    flags = dict(tl_fused_expert=True, tl_fp8_expert_mlp=True, tl_fp8_llm_mlp=True, tl_llm_flash_attn=True, tl_fused_vit=True)
+    plain = create_engine(ckpt, device="cuda", graph=False, warmup=False, **flags)
+    skip = create_engine(ckpt, device="cuda", graph=False, warmup=False, skip_empty_images=True, **flags)
+    frame = plain._profile_frame(seed=4)
+    one = {k: v for k, v in frame.items() if not k.endswith("left_wrist_0_rgb")}
+    noise = torch.zeros(1, 50, 7)
+    p1, s1 = plain.predict_action_chunk(one, noise=noise), skip.predict_action_chunk(one, noise=noise)
+    print(f"skip_empty_images, one of two cameras missing: max|diff| = {float(np.abs(p1 - s1).max()):.3g} of |chunk|max {float(np.abs(p1).max()):.3g}")
+    assert float(np.abs(p1 - s1).max()) <= 1e-2 * max(1.0, float(np.abs(p1).max()))
+    assert np.array_equal(plain.predict_action_chunk(frame, noise=noise), skip.predict_action_chunk(frame, noise=noise))
+    inert = create_engine(ckpt, device="cuda", graph=True, warmup=False, skip_empty_images=True, **flags)
+    assert np.array_equal(plain.predict_action_chunk(one, noise=noise), inert.predict_action_chunk(one, noise=noise))
 
 
 def test_validate_against_an_oracle_dump(ckpt, tmp_path):

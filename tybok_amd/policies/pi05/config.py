@@ -61,6 +61,12 @@ class PI05Config:
     def real_camera_keys(self) -> list[str]:
         return [k for k in self.image_features if "empty_camera" not in k]
 
+    def live_camera_keys(self, batch: dict) -> list[str]:
+        """``pad_free``: the camera slots a request populates -- no ``empty_camera_*`` placeholder slots, no real
+        camera missing from the frame (tybok/policies/pi05/config.py:113-123).  One rule for the eager path and for
+        the recorded shapes, so both build the same prefix length."""
+        return [k for k in self.real_camera_keys if k in batch]
+
     @property
     def image_tokens(self) -> int:
         return (self.image_resolution[0] // self.vision_patch) ** 2

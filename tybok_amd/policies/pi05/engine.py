@@ -14,8 +14,14 @@ flags wired to the HIP kernels:
 * ``tl_fused_vit``        every linear of the SigLIP tower in bf16, scores / softmax / norms /
                           residuals fp32 (drift tier; owns the MLP precision)
 
-``pad_free``, ``skip_empty_images``, ``compile_model`` and Real-Time Chunking are not implemented
-here and are rejected when requested.
+* ``pad_free``            the prefix holds only the cameras a request sends (no ``empty_camera_*`` placeholder
+                          slots) and the language block is cut to the next multiple of 16 live tokens; shapes
+                          are recorded per ``(cameras, language length)``, new ones on first sight
+                          (tybok/policies/pi05/engine.py:510-541,612-630; flow_matching.py:725-760)
+* ``skip_empty_images``   eager path only: a masked-out camera slot behind a real one skips the vision tower and
+                          contributes zero rows (flow_matching.py:415-437); inert under ``graph``, as in the reference
+
+``compile_model`` and Real-Time Chunking are not implemented here and are rejected when requested.
 """
 
 from __future__ import annotations
@@ -28,7 +34,7 @@ import numpy as np
 import torch
 
 from ...base import ChunkRuntime, PolicyEngine
-from ...graph import StaticCall
+from ...graph import StaticCall, camera_counts
 from ...image_utils import resize_with_pad_center
 from ...registry import register, reject_unsupported_flags
 from ..common import (
@@ -72,8 +78,6 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
     _UNSUPPORTED_FLAGS = {
         "tl_llm_fused_attn": False,
         "tl_vit_oproj": False,
-        "skip_empty_images": False,
-        "pad_free": False,
         "pack_qkv": False,
         "text_fused": False,
         "text_fused_split": False,
@@ -117,10 +121,6 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
     ):
         super().__init__(checkpoint_dir, device=device)
         reject_unsupported_flags(type(self), "pi05", kwargs)
-        reject_unsupported_flags(
-            type(self), "pi05",
-            dict(skip_empty_images=skip_empty_images, pad_free=pad_free),
-        )  # fmt: skip
         if sampler != "euler":
             raise ValueError(f"sampler {sampler!r} not supported for pi05 (only 'euler')")
         if compile_model:
@@ -197,8 +197,26 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
         self.overlap = False  # prefill x step-0 two-stream overlap is not implemented; accepted, inert
         if overlap and graph:
             log.info("overlap requested: the prefill x step-0 overlap is not built for pi0.5 here; requests run sequentially (engine.overlap is False)")
-        key = (len(self.config.image_features), self.config.tokenizer_max_length)
-        self._start(warmup=warmup, graph_keys=[key], profile=profile, logger=log)
+        self.pad_free = bool(pad_free)
+        self.model.pad_free = self.pad_free
+        self.skip_empty_images = bool(skip_empty_images)
+        self.model.skip_empty_images = self.skip_empty_images
+        if self.skip_empty_images:
+            if self.graph_enabled:
+                log.info("skip_empty_images is inert on the graph path (a recorded shape runs every slot); pad_free drops the empty slots from the prefix instead")
+            else:
+                log.info("empty camera slots skip the vision tower")
+        self._start(warmup=warmup, graph_keys=self._graph_keys(graph_cameras), profile=profile, logger=log)
+
+    def _graph_keys(self, graph_cameras) -> list[tuple[int, int]]:
+        """``(camera count, language length)`` shapes recorded at start-up (tybok/policies/pi05/engine.py:527-541):
+        every image slot plus the full language block; with ``pad_free`` one shape per requested camera count at the
+        full language length -- shorter language buckets are recorded on first sight."""
+        full_lang = self.config.tokenizer_max_length
+        if not self.pad_free:
+            return [(len(self.config.image_features), full_lang)]
+        max_cams = len(self.config.real_camera_keys)
+        return [(c, full_lang) for c in camera_counts(graph_cameras, default=min(2, max_cams), max_images=max_cams)]
 
     # ------------------------------------------------------------------ API
     def supports_rtc(self) -> bool:
@@ -284,9 +302,11 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
         return {k: v.to(self.device) for k, v in batch.items()}
 
     def prepare_images(self, batch: dict[str, torch.Tensor]):
-        """Centre-padded resize to 224x224, [0,1] -> [-1,1]; missing slots become -1 images with a zero mask (policy.py:170-234)."""
+        """Centre-padded resize to 224x224, [0,1] -> [-1,1]; missing slots become -1 images with a zero mask
+        (policy.py:170-234).  With ``pad_free`` the slots are the cameras the frame holds, nothing else."""
         h, w = self.config.image_resolution
-        present = [k for k in self.config.image_features if k in batch]
+        slots = self.config.live_camera_keys(batch) if self.pad_free else self.config.image_features
+        present = [k for k in slots if k in batch]
         if not present:
             raise ValueError(f"All image features are missing from the batch (expected {self.config.image_features})")
         images, masks = [], []
@@ -294,7 +314,7 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
             img = resize_with_pad_center(batch[key].float(), h, w) * 2.0 - 1.0
             images.append(img)
             masks.append(torch.ones(img.shape[0], dtype=torch.bool, device=img.device))
-        for _ in [k for k in self.config.image_features if k not in batch]:
+        for _ in [k for k in slots if k not in batch]:
             images.append(torch.ones_like(images[-1]) * -1)
             masks.append(torch.zeros_like(masks[-1]))
         return images, masks
@@ -302,6 +322,9 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
     def _infer(self, batch: dict[str, torch.Tensor], noise: torch.Tensor | None) -> torch.Tensor:
         images, img_masks = self.prepare_images(batch)
         tokens, masks = batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK]
+        if self.pad_free:
+            # the language block on the bucket grid, for the eager path and the recorded shapes alike
+            tokens, masks = self.model.pack_language(tokens, masks)
         if self.graph_enabled and self._graph_runner:
             entry = self._graph_runner.entry((len(images), int(tokens.shape[1])))
             return self._run_graph(entry, images, img_masks, tokens, masks, noise)

@@ -92,6 +92,10 @@ class PI05Model:
         # instruction -- what the reference's fp8 prefill tier computes (tybok/policies/pi05/models/triton_prefill_mlp.py:145-166)
         self.fp8_llm_act = bool(fp8_llm_act) and self.fp8_llm_mlp
         self.fused_prefill = bool(fused_prefill)
+        # request-shape flags the engine sets (tybok/policies/pi05/models/flow_matching.py:279-285)
+        self.pad_free = False
+        self.skip_empty_images = False
+        self.tokenizer_max_length = int(cfg.tokenizer_max_length)
         self.use_hip = self.fused_expert or self.fp8_expert_mlp or self.fp8_llm_mlp or self.fused_prefill or self.vit_lowp_attn
         if self.use_hip and self.device.type != "cuda":
             raise RuntimeError("the fused / fp8 tiers run HIP kernels and need a GPU device")
@@ -336,9 +340,55 @@ class PI05Model:
         x = F.layer_norm(x, (vh,), p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], EPS)
         return self.lin(PROJ, x)
 
+    LANG_BUCKET = 16
+
+    def packed_lang_len(self, n_live: int) -> int:
+        """Language length ``pad_free`` packs ``n_live`` live tokens into: the next multiple of ``LANG_BUCKET``,
+        at most the tokenizer's length, so that the number of distinct request shapes stays bounded
+        (tybok/policies/pi05/models/flow_matching.py:727-737)."""
+        if not self.pad_free:
+            return self.tokenizer_max_length
+        bucketed = (int(n_live) + self.LANG_BUCKET - 1) // self.LANG_BUCKET * self.LANG_BUCKET
+        return min(bucketed, self.tokenizer_max_length)
+
+    def pack_language(self, tokens: torch.Tensor, masks: torch.Tensor):
+        """The language block on the bucket grid: the live tokens, then zero ids with False masks up to the bucket
+        (flow_matching.py:739-760).  Needs the live count on the host, so never under graph capture."""
+        if not self.pad_free:
+            return tokens, masks
+        lang_len = self.packed_lang_len(int(masks.sum().item()))
+        if tokens.shape[1] == lang_len and masks.shape[1] == lang_len:
+            return tokens, masks
+        tokens_packed = torch.zeros(tokens.shape[0], lang_len, dtype=tokens.dtype, device=tokens.device)
+        masks_packed = torch.zeros(masks.shape[0], lang_len, dtype=masks.dtype, device=masks.device)
+        keep = min(lang_len, int(tokens.shape[1]))
+        tokens_packed[:, :keep] = tokens[:, :keep]
+        masks_packed[:, :keep] = masks[:, :keep]
+        return tokens_packed, masks_packed
+
     def embed_prefix(self, images, img_masks, tokens, masks):
         """-> ``(embs fp32 [1,P,W], pad_masks [1,P])``; every prefix token attends to every valid one."""
         embs, pads = [], []
+        capturing = self.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
+        if self.skip_empty_images and not capturing and not all(bool(m.all()) for m in img_masks):
+            # eager path only (the check reads the masks on the host): a masked-out slot behind a real camera skips
+            # the vision tower and contributes zero rows -- it is pad-masked out of every attention, so nothing of
+            # it reaches the chunk (flow_matching.py:415-437).  The cameras that remain go through the tower one at
+            # a time here and in one batch otherwise; the HIP linears pick tiles by row count, so their embeddings
+            # can differ in summation order (bf16 noise).  An empty slot in front of any real one is embedded
+            shape = None
+            for img, m in zip(images, img_masks):
+                if shape is not None and not bool(m.all()):
+                    e = torch.zeros(img.shape[0], *shape, dtype=torch.float32, device=img.device)
+                else:
+                    e = self.embed_image(img)
+                    shape = (e.shape[1], e.shape[2])
+                embs.append(e)
+                pads.append(m[:, None].expand(e.shape[0], e.shape[1]))
+            lang = F.embedding(tokens, self.p[VLM + "embed_tokens.weight"]) * self.embed_scale
+            embs.append(lang)
+            pads.append(masks)
+            return torch.cat(embs, dim=1), torch.cat(pads, dim=1)
         if len(images) > 1 and all(img.shape == images[0].shape for img in images):
             # one pass of the vision tower over all cameras (rows are independent)
             per_image = self.embed_image(torch.cat(list(images), dim=0)).split(images[0].shape[0], dim=0)
@@ -504,6 +554,8 @@ class PI05Model:
 
     def sample_actions(self, images, img_masks, tokens, masks, noise, trace: dict | None = None) -> torch.Tensor:
         """Prefix embed, prefill, Euler loop -> ``[1, chunk, max_action_dim]`` fp32."""
+        if self.pad_free and not (self.device.type == "cuda" and torch.cuda.is_current_stream_capturing()):
+            tokens, masks = self.pack_language(tokens, masks)  # (a recorded shape already has the bucket's length)
         embs, pads = self.embed_prefix(images, img_masks, tokens, masks)
         caches = None
         if self.fused_prefill and embs.shape[0] == 1:
