@@ -283,6 +283,20 @@ int tk_f16w_dense(const void* x, int ldx, const void* w_packed, const void* bias
                    const void* resid, int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws,
                    size_t ws_bytes, void* stream);
 
+/* The many-row linear with the rotary epilogue of tk_bf16w_linear: y[M, N] = bf16(x . W^T) with the columns
+ * < rope_cols rotated in pairs (i, i + rope_half) of heads of 2 * rope_half columns by the table row of rope_pos[m]
+ * (int32 [M], clamped into fp32 tables [rope_positions, rope_half]; rope_bf16 selects pi0.5's bf16 arithmetic) and,
+ * when vt is given, the columns >= vt_col0 also written transposed, vt[(n - vt_col0) * vt_ld + m] (rows past M of
+ * vt are left as they are: the caller zero-fills it once) -- the q|k|v projection of a many-row prefill in one
+ * launch (`_fused_gemm_rope_kernel`, tybok/policies/pi05/models/triton_expert_fused_qkv_rope_attn.py:103-251).
+ * w_packed: tk_pack_bf16_weight with the same rope_half (rotary pair order).  N, rope_cols and vt_col0 whole heads;
+ * vt_ld a multiple of 8 >= M rounded up to 32; tile 0 (automatic) or one of the two-tile shapes 42, 32, 22, 12.
+ * Same bits as tk_bf16w_dense on naturally packed weights followed by tk_rope_rows and tk_batched_transpose_v. */
+int tk_bf16w_dense_rope(const void* x, int ldx, const void* w_packed, void* y, int ldy, const void* rope_pos,
+                        const void* rope_cos, const void* rope_sin, int rope_positions, int rope_cols, int rope_half,
+                        int rope_bf16, void* vt, int vt_col0, int vt_ld, int M, int N, int K, int tile, int split_k,
+                        void* ws, size_t ws_bytes, void* stream);
+
 /* ---- action-expert attention over the cached prefix ------------------------------------------ */
 /* Lays one layer's prefix K/V out for tk_expert_attn, once per request (the counterpart of the
  * reference filling its static per-layer prefix cache after the VLM prefill,

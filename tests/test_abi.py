@@ -116,6 +116,10 @@ def _cases():
         ("tk_bf16w_dense", dense(y=P + 8), -1, "16-byte aligned"),
         ("tk_fp8w_gemm_static", static(M=65), -1, "exceeds the 64 rows"),
         ("tk_debug_stream_read", sread(bytes=1000), -1, "multiple"),
+        ("tk_bf16w_dense_rope", (P, 2048, P, P, 2560, P, P, P, 300, 2304, 128, 1, None, 0, 0, 712, 2560, 2048, 31, 0, None, 0, None), -1, "tile=31"),
+        ("tk_bf16w_dense_rope", (P, 2048, P, P, 2560, P, P, P, 300, 2300, 128, 1, None, 0, 0, 712, 2560, 2048, 0, 0, None, 0, None), -1, "whole heads"),
+        ("tk_bf16w_dense_rope", (P, 2048, P, P, 2560, None, P, P, 300, 2304, 128, 1, None, 0, 0, 712, 2560, 2048, 0, 0, None, 0, None), -1, "null table"),
+        ("tk_bf16w_dense_rope", (P, 2048, P, P, 2560, P, P, P, 300, 2304, 128, 1, P, 2304, 712, 712, 2560, 2048, 0, 0, None, 0, None), -1, "vt_ld"),
         ("tk_debug_fp8w_gemm_cut", (P, 2040, P, P, P, 16384, 50, 16384, 2040, 1, None), -1, "multiple of 16"),
         ("tk_fp8w_gemm", gemm(K=2040), -1, "multiple of 16"),
         ("tk_fp8w_gemm", gemm(ldx=1024), -1, "ldx"),

@@ -147,3 +147,67 @@ def test_dense_fp16_flavour_matches_torch(tk, tile, m, k, n, act):
     r16 = r32.to(F16)
     got_r = tk.bf16w_dense(x.cuda(), tk.pack_bf16_weight(w.cuda()), b.cuda(), act, resid=r16.cuda(), tile=tile)
     assert torch.equal(got_r.cpu(), (got.float().cpu() + r16.float()).to(F16))
+
+
+def _rope_case(m, heads_rot, heads_v, d, positions=300, seed=3):
+    g = torch.Generator().manual_seed(seed)
+    half = d // 2
+    ang = torch.rand(positions, half, generator=g) * 6.0
+    pos = torch.randint(-3, positions + 5, (m,), generator=g).to(torch.int32)  # some outside the tables: clamped
+    return ang.cos().contiguous(), ang.sin().contiguous(), pos, half, heads_rot * d, (heads_rot + heads_v) * d
+
+
+@pytest.mark.parametrize("tile", [0, 42, 32, 22, 12])
+@pytest.mark.parametrize("bf16_math", [True, False])
+@pytest.mark.parametrize("m,k,d,heads_rot,heads_v", [(712, 2048, 256, 9, 1), (300, 960, 64, 20, 5), (257, 80, 64, 3, 2), (33, 64, 128, 1, 1)])
+def test_dense_with_rotary_epilogue_gives_the_bits_of_the_three_launches(tk, tile, bf16_math, m, k, d, heads_rot, heads_v):
+    # tk_bf16w_dense_rope (weights in rotary pair order, q | k rotated in the epilogue, V^T written beside V) against
+    # tk_bf16w_dense on naturally packed weights + tk_rope_rows + tk_batched_transpose_v: the same arithmetic in the
+    # same order, so the same bits -- and the rotated columns against plain torch on the GEMM's own output
+    cos, sin, pos, half, rope_cols, n = _rope_case(m, heads_rot, heads_v, d)
+    if bf16_math:
+        cos, sin = cos.to(BF16).float(), sin.to(BF16).float()
+    x, w, _ = _case(m, k, n, seed=4)
+    tables = tk.RopeTables(cos.cuda(), sin.cuda())
+    mp = (m + 31) // 32 * 32
+    # reference path: three launches
+    # (the summation order of an output depends on the K split alone: pinned to the same value on both paths --
+    # none where a tile is forced, 2 for the automatic choice when K allows it)
+    ks = 1 if tile or k < 128 else 2
+    base = tk.bf16w_dense(x.cuda(), tk.pack_bf16_weight(w.cuda()), None, split_k=ks)
+    plain = base.clone()
+    tk.rope_rows(base, tables, pos.cuda(), rope_cols, rope_bf16=bf16_math)
+    vt_want = torch.zeros(n - rope_cols, mp, dtype=BF16, device="cuda")
+    vt_want[:, :m] = base[:, rope_cols:].t()
+    # one launch; vt_out starts with a sentinel-free zero fill (rows past M must stay zero)
+    vt = torch.zeros(n - rope_cols, mp, dtype=BF16, device="cuda")
+    got = tk.bf16w_dense_rope(x.cuda(), tk.pack_bf16_weight(w.cuda(), rope_half=half), tables, pos.cuda(), rope_cols, rope_bf16=bf16_math,
+                              vt_out=vt, vt_col0=rope_cols, tile=tile, split_k=ks)  # fmt: skip
+    assert torch.equal(got, base), f"max |diff| {float((got.float() - base.float()).abs().max())}"
+    assert torch.equal(vt, vt_want)
+    # the rotation itself, in torch, on the linear's bf16 output
+    p = pos.long().clamp(0, cos.shape[0] - 1)
+    y = plain.float().cpu()[:, :rope_cols].view(m, heads_rot, 2, half)
+    a, b = y[:, :, 0], y[:, :, 1]
+    c, s = cos[p][:, None, :], sin[p][:, None, :]
+    if bf16_math:
+        r = lambda t: t.to(BF16).float()  # noqa: E731
+        ra, rb = r(r(a * c) - r(b * s)), r(r(b * c) + r(a * s))
+    else:
+        ra, rb = (a * c - b * s).to(BF16).float(), (b * c + a * s).to(BF16).float()
+    want = torch.stack([ra, rb], dim=2).reshape(m, rope_cols)
+    err = (got.float().cpu()[:, :rope_cols] - want).abs()
+    assert float(err.max()) <= (0.0 if bf16_math else 2**-6 * float(want.abs().max())), float(err.max())
+
+
+def test_dense_rope_argument_rules(tk):
+    cos, sin, pos, half, rope_cols, n = _rope_case(64, 2, 1, 64)
+    x, w, _ = _case(64, 64, n)
+    tables = tk.RopeTables(cos.cuda(), sin.cuda())
+    with pytest.raises(ValueError, match="rotary pair order"):
+        tk.bf16w_dense_rope(x.cuda(), tk.pack_bf16_weight(w.cuda()), tables, pos.cuda(), rope_cols)
+    pw = tk.pack_bf16_weight(w.cuda(), rope_half=half)
+    with pytest.raises(RuntimeError, match="whole heads"):
+        tk.bf16w_dense_rope(x.cuda(), pw, tables, pos.cuda(), rope_cols + 32)
+    with pytest.raises(RuntimeError, match="tile"):
+        tk.bf16w_dense_rope(x.cuda(), pw, tables, pos.cuda(), rope_cols, tile=31)

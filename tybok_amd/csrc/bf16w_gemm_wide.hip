@@ -34,8 +34,13 @@ constexpr int NW = 4;  // waves per block
 constexpr int RK = 2;  // k tiles (of 32) per round
 
 // F16: the operands are fp16 (v_mfma_f32_32x32x16_f16) instead of bf16; same tile order, same epilogues
-template <int MT, int NT, int PF, int OCC, bool F16>
+// ROPE (NT == 2, bf16): the weights are packed in rotary pair order -- the two tiles of a wave hold columns
+// (c, c + rope_half) of one head -- and the epilogue is the skinny kernel's rotary one: columns < rope_cols rotated
+// by the table row of pos[m] (fp32 products rounded separately, or every product and sum rounded to bf16), columns
+// >= vt_col0 also written transposed for the attention kernel.  No bias, activation or residual in this form.
+template <int MT, int NT, int PF, int OCC, bool F16, bool ROPE = false>
 __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, int nblk_m, int ngroups) {
+  static_assert(!ROPE || (NT == 2 && !F16), "the rotary epilogue needs both halves of a pair in one wave");
   constexpr int ROWS = MT * 32;
   constexpr int ROWB = RK * 64;     // bytes of one staged activation row per round
   constexpr int PITCH = ROWB + 16;  // conflict-free 16-byte operand reads, 16-byte aligned
@@ -275,6 +280,77 @@ __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, in
   // columns: whole row segments of NT*64 bytes per 4*NT lanes. ----
   lds_barrier();  // every wave has left the staged activations behind
   unsigned char* wl = lds + wave * 32 * EP;
+  if constexpr (ROPE) {
+    // logical tile of physical tile (strip, j): (strip / PO) * 2 * PO + strip % PO + j * PO, PO = rope_half / 32
+    const int po = a.rope_half >> 5;
+    const int ca0 = ((strip / po) * 2 * po + strip % po) * 32, cb0 = ca0 + a.rope_half;  // first columns of the two tiles
+    const bool rot = ca0 < a.rope_cols;
+    const int fi0 = ca0 % (2 * a.rope_half) + 4 * half;
+    const int lrow = lane / LPR, lchunk = lane % LPR;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m0 = (mblock * MT + mt) * 32;
+      int mr = m0 + l32;
+      if (mr > a.M - 1) mr = a.M - 1;
+      int pos = a.rope_pos[mr];
+      pos = pos < 0 ? 0 : (pos > a.rope_positions - 1 ? a.rope_positions - 1 : pos);
+      const float* cs_row = a.rope_cos + (size_t)pos * a.rope_half + fi0;
+      const float* sn_row = a.rope_sin + (size_t)pos * a.rope_half + fi0;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& c0 = acc[mt][0];
+        const f32x16& c1 = acc[mt][1];
+        f32x4 va = unpack_bf16x4(pack_bf16x4(f32x4{c0[4 * g], c0[4 * g + 1], c0[4 * g + 2], c0[4 * g + 3]}));
+        f32x4 vb = unpack_bf16x4(pack_bf16x4(f32x4{c1[4 * g], c1[4 * g + 1], c1[4 * g + 2], c1[4 * g + 3]}));
+        if (rot) {
+          const f32x4 cs = *(const f32x4*)(cs_row + 8 * g), sn = *(const f32x4*)(sn_row + 8 * g);
+          f32x4 ra, rb;
+          if (a.rope_bf16) {
+            const f32x4 ac = unpack_bf16x4(pack_bf16x4(va * cs)), bs = unpack_bf16x4(pack_bf16x4(vb * sn));
+            const f32x4 bc = unpack_bf16x4(pack_bf16x4(vb * cs)), as = unpack_bf16x4(pack_bf16x4(va * sn));
+            ra = ac - bs;
+            rb = bc + as;
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              ra[j] = sub_rn(mul_rn(va[j], cs[j]), mul_rn(vb[j], sn[j]));
+              rb[j] = add_rn(mul_rn(vb[j], cs[j]), mul_rn(va[j], sn[j]));
+            }
+          }
+          va = ra;
+          vb = rb;
+        }
+        *(i32x2*)(wl + l32 * EP + (8 * g + 4 * half) * 2) = pack_bf16x4(va);
+        *(i32x2*)(wl + l32 * EP + (32 + 8 * g + 4 * half) * 2) = pack_bf16x4(vb);
+      }
+#pragma unroll
+      for (int j = 0; j < 32 / RPI; ++j) {
+        const int row = j * RPI + lrow;
+        const int m = m0 + row;
+        const int n = (lchunk < 4 ? ca0 : cb0) + (lchunk & 3) * 8;
+        const i32x4 t = *(const i32x4*)(wl + row * EP + lchunk * 16);
+        if (m >= a.M || n >= a.N) continue;
+        *(i32x4*)(a.y + (size_t)m * a.ldy + n) = t;  // N is a multiple of 64 in this form
+      }
+      if (a.vt && ca0 >= a.vt_col0) {  // wave-uniform: vt_col0 is a multiple of the head size
+        // value columns, transposed for the attention kernel: lane = one of the wave's 64 columns, eight consecutive
+        // rows per 16-byte store; rows past M stay zero (the attention kernel relies on zeros behind the last key)
+        const int n = (lane < 32 ? ca0 : cb0) + (lane & 31);
+        if (n < a.N) {
+          u16* dst = a.vt + (size_t)(n - a.vt_col0) * a.vt_ld + m0;
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg) {
+            unsigned e[8];
+#pragma unroll
+            for (int r = 0; r < 8; ++r) e[r] = m0 + 8 * rg + r < a.M ? *(const u16*)(wl + (8 * rg + r) * EP + lane * 2) : 0u;
+            if (m0 + 8 * rg < a.M)
+              *(i32x4*)(dst + 8 * rg) = i32x4{(int)(e[0] | (e[1] << 16)), (int)(e[2] | (e[3] << 16)), (int)(e[4] | (e[5] << 16)), (int)(e[6] | (e[7] << 16))};
+          }
+        }
+      }
+    }
+    return;
+  }
   const int ncol0 = strip * COLS;  // first output column of this wave
   f32x4 bias[NT][4];
 #pragma unroll
@@ -338,6 +414,15 @@ int launch(const GemmArgs& a, hipStream_t st) {
   const int nblk_n = (a.ntiles + NW * NT - 1) / (NW * NT);
   const int ngroups = nblk_n * a.ksplit;
   const unsigned blocks = (unsigned)((ngroups + 7) / 8) * 8u * (unsigned)nblk_m;
+  if (a.rope_pos) {
+    if constexpr (NT == 2) {
+      if (a.f16) return -1;
+      hipLaunchKernelGGL((bf16w_wide_kernel<MT, NT, PF, OCC, false, true>), dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
+      return hipGetLastError() == hipSuccess ? 0 : -3;
+    } else {
+      return -1;
+    }
+  }
   if (a.f16)
     hipLaunchKernelGGL((bf16w_wide_kernel<MT, NT, PF, OCC, true>), dim3(blocks), dim3(NW * 64), 0, st, a, nblk_m, ngroups);
   else

@@ -563,9 +563,19 @@ float dense_cost(const DenseTile& t, int M, int N, int KT, int ks, int cus) {
 }  // namespace
 
 namespace {
+// rotary form of the many-row linear: weights in rotary pair order, tables and positions as in tk_bf16w_linear
+struct DenseRope {
+  const int* pos = nullptr;
+  const float* cos = nullptr;
+  const float* sin = nullptr;
+  int positions = 0, cols = 0, half = 0, bf16 = 0;
+  void* vt = nullptr;
+  int vt_col0 = 0, vt_ld = 0;
+};
+
 int dense_common(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy, const void* resid,
                  int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws, size_t ws_bytes, void* stream,
-                 int f16) {
+                 int f16, const DenseRope* rope = nullptr) {
   if (M <= 0 || N <= 0 || K <= 0) return fail(TK_EINVAL, "bf16w_dense: non-positive shape M=%d N=%d K=%d", M, N, K);
   if (K % 16 || ldx % 8 || ldx < K) return fail(TK_EINVAL, "bf16w_dense: K=%d must be a multiple of 16 and ldx=%d a multiple of 8 >= K", K, ldx);
   if (!x || !w_packed || !y) return fail(TK_EINVAL, "bf16w_dense: null pointer");
@@ -596,12 +606,32 @@ int dense_common(const void* x, int ldx, const void* w_packed, const void* bias,
   a.act = act;
   a.f16 = f16;
   a.vec = a.vec16 = 1;
+  if (rope) {
+    if (f16 || bias || act || resid) return fail(TK_EINVAL, "bf16w_dense_rope: bf16 only, no bias, activation or residual");
+    if (!rope->pos || !rope->cos || !rope->sin || rope->positions <= 0) return fail(TK_EINVAL, "bf16w_dense_rope: null table or position pointer");
+    if (rope->half < 32 || rope->half % 32 || rope->cols <= 0 || rope->cols % (2 * rope->half) || rope->cols > N || N % (2 * rope->half))
+      return fail(TK_EINVAL, "bf16w_dense_rope: rope_half=%d must be a multiple of 32, rope_cols=%d and N=%d whole heads of 2 * rope_half columns", rope->half, rope->cols, N);
+    if (!aligned16(rope->cos) || !aligned16(rope->sin)) return fail(TK_EINVAL, "bf16w_dense_rope: tables must be 16-byte aligned");
+    if (rope->vt && (rope->vt_col0 % (2 * rope->half) || rope->vt_col0 < 0 || rope->vt_col0 >= N || rope->vt_ld % 8 || rope->vt_ld < (M + 31) / 32 * 32 || !aligned16(rope->vt)))
+      return fail(TK_EINVAL, "bf16w_dense_rope: vt_col0=%d must start a head, vt_ld=%d be a multiple of 8 >= M rounded up to 32, vt 16-byte aligned", rope->vt_col0, rope->vt_ld);
+    a.rope_pos = rope->pos;
+    a.rope_cos = rope->cos;
+    a.rope_sin = rope->sin;
+    a.rope_positions = rope->positions;
+    a.rope_cols = rope->cols;
+    a.rope_half = rope->half;
+    a.rope_bf16 = rope->bf16;
+    a.vt = (u16*)rope->vt;
+    a.vt_col0 = rope->vt_col0;
+    a.vt_ld = rope->vt_ld;
+  }
   const int cus = device_cus();
   const DenseTile* best = nullptr;
   int ks = split_k > 0 ? split_k : 1;
   float best_cost = 0.f;
   for (const DenseTile& t : kDenseTiles) {
     if (tile && t.id != tile) continue;
+    if (rope && t.id % 10 != 2) continue;  // the rotary epilogue needs two n tiles per wave
     const int blocks0 = ((M + t.rows - 1) / t.rows) * ((N + t.cols - 1) / t.cols);
     int k1 = 1;
     if (split_k > 0) {
@@ -639,6 +669,23 @@ int dense_common(const void* x, int ldx, const void* w_packed, const void* bias,
 int tk_bf16w_dense(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy, const void* resid,
                    int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws, size_t ws_bytes, void* stream) {
   return dense_common(x, ldx, w_packed, bias, act, y, ldy, resid, ldr, resid_dtype, M, N, K, tile, split_k, ws, ws_bytes, stream, 0);
+}
+
+int tk_bf16w_dense_rope(const void* x, int ldx, const void* w_packed, void* y, int ldy, const void* rope_pos, const void* rope_cos,
+                        const void* rope_sin, int rope_positions, int rope_cols, int rope_half, int rope_bf16, void* vt, int vt_col0,
+                        int vt_ld, int M, int N, int K, int tile, int split_k, void* ws, size_t ws_bytes, void* stream) {
+  DenseRope r;
+  r.pos = (const int*)rope_pos;
+  r.cos = (const float*)rope_cos;
+  r.sin = (const float*)rope_sin;
+  r.positions = rope_positions;
+  r.cols = rope_cols;
+  r.half = rope_half;
+  r.bf16 = rope_bf16;
+  r.vt = vt;
+  r.vt_col0 = vt_col0;
+  r.vt_ld = vt_ld;
+  return dense_common(x, ldx, w_packed, nullptr, 0, y, ldy, nullptr, 0, 0, M, N, K, tile, split_k, ws, ws_bytes, stream, 0, &r);
 }
 
 int tk_f16w_dense(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy, const void* resid,

@@ -399,6 +399,54 @@ def bf16w_dense(
     return out
 
 
+def bf16w_dense_rope(
+    x: torch.Tensor,
+    w: PackedBf16Weight,
+    rope: "RopeTables",
+    rope_pos: torch.Tensor,
+    rope_cols: int,
+    *,
+    rope_bf16: bool = False,
+    vt_out: torch.Tensor | None = None,
+    vt_col0: int = 0,
+    out: torch.Tensor | None = None,
+    tile: int = 0,
+    split_k: int = 0,
+    ws: Workspace | None = None,
+) -> torch.Tensor:
+    """The many-row linear with the rotary epilogue: ``bf16(x @ W^T)`` for ``x [M, K]`` bf16 and a weight packed in
+    rotary pair order (``pack_bf16_weight(w, rope_half)``), the columns ``< rope_cols`` rotated by the table row of
+    ``rope_pos[m]``, and with ``vt_out [N - vt_col0, >= M rounded up to 32]`` the columns from ``vt_col0`` on also
+    written transposed -- a many-row prefill's q|k|v projection in one launch (``tk_bf16w_dense_rope``)."""
+    lib = native.lib()
+    if w.dtype != torch.bfloat16 or not w.rope_half or rope.half != w.rope_half:
+        raise ValueError("the weight must be bf16, packed in rotary pair order with the tables' rope_half")
+    if x.dtype != torch.bfloat16 or not x.is_cuda or x.dim() != 2 or x.shape[1] != w.k or x.stride(1) != 1:
+        raise ValueError(f"activations must be a CUDA bf16 [M, {w.k}] matrix with unit inner stride")
+    m = x.shape[0]
+    if rope_pos.dtype != torch.int32 or rope_pos.numel() != m or not rope_pos.is_contiguous():
+        raise ValueError("rope_pos must be a contiguous int32 [M]")
+    if rope.cos.dtype != torch.float32 or not rope.cos.is_contiguous() or not rope.sin.is_contiguous():
+        raise ValueError("rotary tables must be contiguous fp32")
+    if out is None:
+        out = torch.empty(m, w.n, dtype=torch.bfloat16, device=x.device)
+    if out.dtype != torch.bfloat16 or out.shape != (m, w.n) or out.stride(1) != 1:
+        raise ValueError("out must be bf16 [M, N] with unit inner stride")
+    vt_p, vt_ld = None, 0
+    if vt_out is not None:
+        if vt_out.dtype != torch.bfloat16 or vt_out.dim() != 2 or vt_out.stride(1) != 1 or vt_out.shape[0] != w.n - vt_col0:
+            raise ValueError("vt_out must be bf16 [N - vt_col0, >= M] with unit inner stride")
+        vt_p, vt_ld = vt_out.data_ptr(), vt_out.stride(0)
+    ws = ws or default_workspace(x.device)
+    rc = lib.tk_bf16w_dense_rope(
+        x.data_ptr(), x.stride(0), w.data.data_ptr(), out.data_ptr(), out.stride(0), rope_pos.data_ptr(), rope.cos.data_ptr(),
+        rope.sin.data_ptr(), rope.positions, rope_cols, rope.half, int(rope_bf16), vt_p, vt_col0, vt_ld, m, w.n, w.k, tile, split_k,
+        ws.ptr, ws.nbytes, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_bf16w_dense_rope")
+    return out
+
+
 def _norm_ptr(norm_w: torch.Tensor | None, k: int) -> int | None:
     if norm_w is None:
         return None

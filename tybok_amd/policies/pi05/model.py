@@ -134,12 +134,6 @@ class PI05Model:
             self.exp_qkv, self.exp_o = pack_stack(EXP, self.ed["depth"])
         if self.fused_prefill:
             self.vlm_qkv, self.vlm_o = pack_stack(VLM, self.depth)
-            # the same q|k|v weights in natural tile order, for prefixes long enough that the projection runs on
-            # the many-row MFMA kernel, followed by the rotary kernel
-            self.vlm_qkv_dense = [
-                tk.pack_bf16_weight(torch.cat([self.p[f"{VLM}layers.{i}.self_attn.{n}_proj.weight"] for n in "qkv"], dim=0).to(BF16).contiguous())
-                for i in range(self.depth)
-            ]
             # Gemma RMSNorm x * rstd * (1 + w) is the adaptive norm with scale = w and shift = 0
             zeros = torch.zeros(self.vd["width"], dtype=torch.float32, device=self.device)
             self.vlm_norms = [
@@ -443,14 +437,16 @@ class PI05Model:
         vt_all = torch.zeros(self.depth, nkv, p_pad, dtype=BF16, device=self.device)
         hidden = embs[0].to(BF16)
         kv, caches = [], []
-        many_rows = p_len >= 256 and nkv % 64 == 0
+        many_rows = p_len >= 256  # the projections on the many-row MFMA kernels
         for i in range(self.depth):
             norm_in, norm_post = self.vlm_norms[i]
             if many_rows:
-                # norm, many-row GEMM, rotary embedding in place, V^T through the tiled transpose
-                qkv = tk.bf16w_dense(tk.rms_norm_rows(hidden, ada=norm_in, eps=EPS), self.vlm_qkv_dense[i], out=qkv_all[i], ws=self.ws)
-                tk.rope_rows(qkv, self.rope_tables_hip, pos32, nq + nkv, rope_bf16=True)
-                tk.transpose_v(qkv[:, nq + nkv :].view(1, p_len, nkv // 64, 64), out=vt_all[i].view(1, nkv // 64, 64, p_pad))
+                # the norm as a launch of its own, then the many-row GEMM with the rotary epilogue (q | k rotated, V^T
+                # written beside V): the skinny kernel's launch below, at many rows
+                qkv = tk.bf16w_dense_rope(
+                    tk.rms_norm_rows(hidden, ada=norm_in, eps=EPS), self.vlm_qkv[i], self.rope_tables_hip, pos32, nq + nkv, rope_bf16=True,
+                    vt_out=vt_all[i], vt_col0=nq + nkv, out=qkv_all[i], ws=self.ws,
+                )  # fmt: skip
             else:
                 qkv = tk.bf16w_linear(
                     hidden, self.vlm_qkv[i], ada=norm_in, eps=EPS, rope=self.rope_tables_hip, rope_pos=pos32, rope_cols=nq + nkv,
