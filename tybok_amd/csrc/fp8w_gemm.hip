@@ -66,10 +66,10 @@ __device__ __forceinline__ void lds_barrier() {
 template <int MT, int NT, int NW, int EPI, int PF, int TPW, bool W16, int PRO, int NR, int FUSE>
 __device__ __forceinline__ void gemm_block(const GemmArgs& a, const int strip, const int split, const int mblock, const int nstrips) {
   constexpr bool GATED = EPI == 1;
-  // every round of the block in flight from the start (PF == NR) with the bf16 RMSNorm prologue: the staged pieces
-  // stay in registers until the row statistics are known, so the statistics come from them -- no second pass over
-  // the rows.  The host picks this only when a block walks the whole K (no K split).
-  constexpr bool FULL = PRO == 1 && NR > 0 && PF == NR;
+  // every round of the block in flight from the start (PF == NR) with the bf16 RMSNorm prologue (plain or adaptive):
+  // the staged pieces stay in registers until the row statistics are known, so the statistics come from them -- no
+  // second pass over the rows.  The host picks this only when a block walks the whole K (no K split).
+  constexpr bool FULL = (PRO == 1 || PRO == 3) && NR > 0 && PF == NR;
   constexpr bool PAIRED = EPI != 0;  // both n tiles of a pair are finished by the same wave
   constexpr bool XF32 = PRO == 2;
   constexpr int TILES = MT * NT;
@@ -169,9 +169,12 @@ __device__ __forceinline__ void gemm_block(const GemmArgs& a, const int strip, c
     }
   };
   constexpr bool ADA = PRO == 3;
+  // a thread's pieces of a round are the same 8 columns of XPT different rows (the block's threads are a multiple
+  // of the pieces per row), so the norm weights of those columns are held once
+  static_assert((NW * 64) % PPR == 0, "a thread's pieces share their columns");
   struct XFrag {
     i32x4 v[XPT][XF32 ? 2 : 1];
-    i32x4 nw[PRO ? XPT : 1][ADA ? 4 : 1];  // norm weights of the piece's 8 columns (ADA: fp32 scale, shift)
+    i32x4 nw[ADA ? 4 : 1];  // norm weights of the pieces' 8 columns (ADA: fp32 scale, shift)
   };
   auto xload = [&](XFrag& f, int r) {
     const int k0 = (kt_lo + r * RKT) * 32;
@@ -188,13 +191,15 @@ __device__ __forceinline__ void gemm_block(const GemmArgs& a, const int strip, c
       } else {
         f.v[i][0] = *(const i32x4*)(xsrc[i] + (size_t)k * 2);
       }
-      if (ADA) {
-        f.nw[i][0] = *(const i32x4*)(a.ada_scale + k);
-        f.nw[i][ADA ? 1 : 0] = *(const i32x4*)(a.ada_scale + k + 4);
-        f.nw[i][ADA ? 2 : 0] = *(const i32x4*)(a.ada_shift + k);
-        f.nw[i][ADA ? 3 : 0] = *(const i32x4*)(a.ada_shift + k + 4);
-      } else if (PRO) {
-        f.nw[i][0] = *(const i32x4*)(a.norm_w + k);
+      if (i == 0) {
+        if (ADA) {
+          f.nw[0] = *(const i32x4*)(a.ada_scale + k);
+          f.nw[ADA ? 1 : 0] = *(const i32x4*)(a.ada_scale + k + 4);
+          f.nw[ADA ? 2 : 0] = *(const i32x4*)(a.ada_shift + k);
+          f.nw[ADA ? 3 : 0] = *(const i32x4*)(a.ada_shift + k + 4);
+        } else if (PRO) {
+          f.nw[0] = *(const i32x4*)(a.norm_w + k);
+        }
       }
     }
   };
@@ -218,10 +223,10 @@ __device__ __forceinline__ void gemm_block(const GemmArgs& a, const int strip, c
         union { i32x4 v; unsigned u[4]; } xu, o;
         union { i32x4 v[2]; float f[8]; } sc, sh;
         xu.v = f.v[i][0];
-        sc.v[0] = f.nw[i][0];
-        sc.v[1] = f.nw[i][ADA ? 1 : 0];
-        sh.v[0] = f.nw[i][ADA ? 2 : 0];
-        sh.v[1] = f.nw[i][ADA ? 3 : 0];
+        sc.v[0] = f.nw[0];
+        sc.v[1] = f.nw[ADA ? 1 : 0];
+        sh.v[0] = f.nw[ADA ? 2 : 0];
+        sh.v[1] = f.nw[ADA ? 3 : 0];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           // separately rounded fp32 operations, as the elementwise reference computes them
@@ -233,7 +238,7 @@ __device__ __forceinline__ void gemm_block(const GemmArgs& a, const int strip, c
         out = o.v;
       } else {
         union { i32x4 v; unsigned u[4]; } nwu, o;
-        nwu.v = f.nw[i][0];
+        nwu.v = f.nw[0];
         float xv[8];
         if (XF32) {
           union { i32x4 v; float f[4]; } lo, hi;
@@ -811,7 +816,7 @@ template <int MT, int NT, int EPI, bool W16, int PRO, int NR, int NW>
 int launch_nr(const GemmArgs& a, dim3 grid, hipStream_t st) {
   // the RMSNorm prologue over a short K that one block walks alone: all of its rounds in flight, the row
   // statistics taken from the staged pieces (SmolVLA's expert: K = 720, VLM: 960)
-  constexpr bool CAN_FULL = PRO == 1 && MT == 1 && NR > 0 && NR * NW <= 32;
+  constexpr bool CAN_FULL = (PRO == 1 || PRO == 3) && MT == 1 && NR > 0 && NR * NW <= 32;
   constexpr int PFN = NW == 8 ? kPF8 : kPF;
   if (CAN_FULL && a.ksplit == 1) {
     hipLaunchKernelGGL((fp8w_gemm_kernel<MT, NT, NW, EPI, CAN_FULL ? NR : PFN, kTPW, W16, PRO, NR>), grid, dim3(NW * 64), 0, st, a);
@@ -846,10 +851,11 @@ int launch(const GemmArgs& a, dim3 grid, int nw, hipStream_t st) {
 int tk_launch_gemm(GemmArgs a, int MT, int NT, int mblocks, hipStream_t st) {
   dim3 grid((a.ntiles + NT - 1) / NT, a.ksplit, mblocks);
   // eight waves on a 32-row block where they pay (measured per launch and in whole requests, K = 720 .. 2048): a
-  // long k range of fp8 tiles (half the rounds) or the RMSNorm prologue (half the normalisation work per thread);
+  // long k range of fp8 tiles (half the rounds) or a norm prologue, plain or adaptive (half the normalisation work
+  // per thread, and at K <= 1024 every round in flight with the row statistics taken from the staged pieces);
   // elsewhere four waves are as fast or faster (one LDS exchange less)
   const int pro_ = a.ada_scale != nullptr ? 3 : (a.norm_w == nullptr ? 0 : (a.x_f32 ? 2 : 1));
-  const int nw = (MT == 1 && ((!a.w16 && a.kt_q >= 48) || pro_ == 1)) ? 8 : 4;
+  const int nw = (MT == 1 && ((!a.w16 && a.kt_q >= 48) || pro_ == 1 || pro_ == 3)) ? 8 : 4;
   const int epi = a.s1 != nullptr ? 1 : (a.rope_pos != nullptr ? 2 : 0);
   const int pro = a.ada_scale != nullptr ? 3 : (a.norm_w == nullptr ? 0 : (a.x_f32 ? 2 : 1));
   if (a.w16) {

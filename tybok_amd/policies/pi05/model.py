@@ -496,10 +496,9 @@ class PI05Model:
             att = tk.expert_attn(qkv[:, :nq].view(s, heads, d), caches[i], suffix, pad, tk.MASK_BIDIR, logits_bf16=True, ws=self.ws)
             hidden = tk.bf16w_linear(att, self.exp_o[i], resid=hidden, gate=gate_in, ws=self.ws)
             mlp = self.exp_mlp[i]
-            # the adaptive norm as a launch of its own (2.4 us): as the gate/up launch's prologue every one of
-            # its 256 blocks would normalise its 32 rows x 1024 columns again (6.4 us on that launch)
-            normed = tk.rms_norm_rows(hidden, ada=(sc_post, sh_post), eps=EPS)
-            hidden = tk.fp8w_gated_ffn(normed, mlp.wgu, mlp.wd, "gelu_tanh", resid=hidden, gate=gate_post, ws=self.ws)
+            # the adaptive norm as the gate/up launch's prologue: eight waves per block, every round of the short K in
+            # flight, the row statistics taken from the staged pieces (no second pass over the rows)
+            hidden = tk.fp8w_gated_ffn(hidden, mlp.wgu, mlp.wd, "gelu_tanh", resid=hidden, gate=gate_post, ada=(sc_post, sh_post), eps=EPS, ws=self.ws)
         return hidden
 
     def denoise_step(self, prefix_pad, kv, x_t, step: int, caches: list | None = None) -> torch.Tensor:
