@@ -423,6 +423,56 @@ def cpu_baseline_smolvla(cameras: int, frame: dict | None = None) -> tuple[dict,
     }, chunk[0].numpy()
 
 
+def live_gemm_traffic(timeout_s: int = 90) -> dict | None:
+    """HBM bytes per launch of the roofline GEMM, counted in this run: ``bench.py --gemm-only`` twice under
+    ``rocprofv3 --pmc`` (FETCH_SIZE, then WRITE_SIZE, a run each), each counter scaled by what it reads for the
+    33,554,432-byte device copies that clone the weights in the same run.  Child processes, started before this
+    process touches the GPU; ``None`` when the profiler is missing or a run fails (the caller then falls back to
+    the figure of ``profiles/fp8w_gemm_traffic.json``)."""
+    import csv
+    import glob
+    import shutil
+    import statistics
+    import subprocess
+    import tempfile
+
+    exe = shutil.which("rocprofv3")
+    if exe is None or shutil.which("timeout") is None:
+        return None
+    copy_bytes = 2048 * 16384
+    medians: dict[str, tuple[float, float]] = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        out_dir = tempfile.mkdtemp(prefix="tk_pmc_", dir="/tmp")
+        cmd = ["timeout", "-s", "KILL", str(timeout_s), exe, "--pmc", counter, "-d", out_dir, "-o", "p", "--output-format", "csv", "--",
+               sys.executable, os.path.join(ROOT, "bench.py"), "--gemm-only", "--steps", "2"]  # fmt: skip
+        try:
+            subprocess.run(cmd, cwd="/tmp", env=dict(os.environ, TMPDIR="/tmp"), stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
+                           timeout=timeout_s + 15, check=True)  # fmt: skip
+            files = glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True)
+            gemm, copy = [], []
+            with open(files[0], newline="", encoding="utf-8") as f:
+                for row in csv.DictReader(f):
+                    if row["Counter_Name"] != counter:
+                        continue
+                    if "fp8w_stream_kernel" in row["Kernel_Name"]:
+                        gemm.append(float(row["Counter_Value"]))
+                    elif "copyBuffer" in row["Kernel_Name"]:
+                        copy.append(float(row["Counter_Value"]))
+            medians[counter] = (statistics.median(gemm), statistics.median(copy))
+        except Exception:  # noqa: BLE001 - a diagnostic leg: any failure means "not measured here"
+            return None
+        finally:
+            shutil.rmtree(out_dir, ignore_errors=True)
+    (fetch, fetch_copy), (write, write_copy) = medians["FETCH_SIZE"], medians["WRITE_SIZE"]
+    if fetch_copy <= 0 or write_copy <= 0:
+        return None
+    return {
+        "hbm_bytes_per_launch": int(round(fetch * copy_bytes / fetch_copy + write * copy_bytes / write_copy)),
+        "fetch_counts": fetch, "write_counts": write,
+        "fetch_bytes_per_count": copy_bytes / fetch_copy, "write_bytes_per_count": copy_bytes / write_copy,
+    }  # fmt: skip
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -430,6 +480,7 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-pi05", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-live-traffic", action="store_true", help="do not count the roofline GEMM's HBM traffic under rocprofv3 in this run")
     ap.add_argument("--gemm-only", action="store_true", help="only the roofline GEMM loop plus a plain copy of known size (for rocprofv3 runs)")
     ap.add_argument("--gemm-cuts", action="store_true", help="with --gemm-only: also time the measurement forms of the weight-streaming kernel (K = 2048 shapes)")
     ap.add_argument("--gemm-shape", type=int, nargs=3, metavar=("M", "K", "N"), default=(50, 2048, 16384), help="shape of the --gemm-only loop")
@@ -443,6 +494,11 @@ def main() -> None:
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is batch-1 and single-device (--gpus must be 1)")
+
+    only = (args.gemm_only or args.attn_only or args.attn_d256_only or args.dense_only or args.tower_attn_only or args.ffn_only
+            or args.request_only)  # fmt: skip
+    # the counter runs are child processes: they go first, while this process has not initialised the GPU
+    traffic_live = None if (only or args.skip_live_traffic) else live_gemm_traffic()
 
     import torch
 
@@ -610,9 +666,14 @@ def main() -> None:
     a2 = sweep[f"K{k2}_N{n2}"]["GBps"]
     roofline["other_33MB_shape"] = {"kernel": "fp8w_stream_kernel, 8 K-splits (M=50, K=16384, N=2048, cold weights)", "achieved": a2, "frac": round(a2 / HBM_PEAK_GBS, 4), "frac_of_stream_ceiling": round(a2 / sc_gbps, 4)}
     traffic_file = os.path.join(ROOT, "profiles", "fp8w_gemm_traffic.json")
-    if os.path.exists(traffic_file):
+    if traffic_live is not None:
+        roofline["traffic"] = traffic_live["hbm_bytes_per_launch"]
+        roofline["traffic_source"] = ("rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE over `bench.py --gemm-only --steps 2` in this run, "
+                                      f"{traffic_live['fetch_bytes_per_count']:.1f} / {traffic_live['write_bytes_per_count']:.1f} B per count from the 33,554,432-byte weight copies")  # fmt: skip
+    elif os.path.exists(traffic_file):
         with open(traffic_file, encoding="utf-8") as f:
             roofline["traffic"] = json.load(f).get("hbm_bytes_per_launch")
+        roofline["traffic_source"] = "profiles/fp8w_gemm_traffic.json (counter runs of an earlier day; not repeated in this run)"
 
     # ---- many-row (prefill) FFN: MFMA-bound, priced against the dense bf16 peak ----
     fm, fk, fi = 712, 2048, 16384
