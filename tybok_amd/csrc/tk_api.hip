@@ -636,6 +636,10 @@ int dense_common(const void* x, int ldx, const void* w_packed, const void* bias,
     int k1 = 1;
     if (split_k > 0) {
       k1 = split_k;
+    } else if (rope) {
+      // measured at the prefill's q|k|v shape (712 x 2048 -> 2560): 64 x 256 blocks, unsplit, 20.7 us; 32 x 256:
+      // 27.9, 96 x 256: 25.7, 128 x 256: 32.2; any K split 30-39 us (the partials weigh more than the idle CUs)
+      if (!tile && t.id != (M > 32 ? 22 : 12)) continue;
     } else {
       // few blocks and a long K: split, keeping at least 32 k tiles per split
       k1 = cus / blocks0;
