@@ -84,6 +84,26 @@ def test_many_row_split_k_is_deterministic(tk, split):
     _close(a, oops.lin_fp8w(x, w8, s), f"many-row gemm split_k={split}")
 
 
+@pytest.mark.parametrize("m,k,n", [(712, 4096, 2048), (300, 2048, 516), (257, 1024, 260)])
+def test_many_row_split_k_reduction_launch_with_gate_and_residual(tk, m, k, n):
+    # a K-split plain launch leaves fp32 partials and a second launch sums them in split order and runs the epilogue
+    # (scale, per-column gate, bf16 / fp32 residual): ragged rows, N % 8 == 4, both residual types; the same
+    # launch twice gives the same bits, and every split count agrees with the oracle
+    x, w8, s = gemm_case(m, k, n)
+    pw = tk.pack_fp8_weight(w8.cuda(), s.cuda())
+    g = torch.Generator().manual_seed(7)
+    gate = torch.randn(n, generator=g).to(BF16)
+    base = oops.lin_fp8w(x, w8, s)
+    for rdt in (BF16, torch.float32):
+        resid = torch.randn(m, n, generator=g).to(rdt)
+        want = ((base * gate).float() + resid.float()).to(BF16)
+        for split in (2, 3, 4):
+            a = tk.fp8w_gemm(x.cuda(), pw, resid=resid.cuda(), gate=gate.cuda(), split_k=split)
+            b = tk.fp8w_gemm(x.cuda(), pw, resid=resid.cuda(), gate=gate.cuda(), split_k=split)
+            assert torch.equal(a, b)
+            _close(a, want, f"many-row split_k={split} + gate + resid {rdt} M={m} K={k} N={n}")
+
+
 def test_many_row_gemm_residual_gate_and_strides(tk):
     m, k, n = 270, 720, 960
     x, w8, s = gemm_case(m, k, n)
