@@ -297,6 +297,17 @@ int tk_bf16w_dense_rope(const void* x, int ldx, const void* w_packed, void* y, i
                         int rope_bf16, void* vt, int vt_col0, int vt_ld, int M, int N, int K, int tile, int split_k,
                         void* ws, size_t ws_bytes, void* stream);
 
+/* The packed q|k|v projection of a vision tower with the value columns also written transposed, so that the
+ * attention launch needs no transpose in front of it: y[M, N] = 16-bit(x . W^T + bias) as tk_bf16w_dense
+ * (f16 = 1: tk_f16w_dense) and vt[(m / vt_rows) * vt_bs + (n - vt_col0) * vt_ld + m % vt_rows] = y[m, n] for the
+ * columns n >= vt_col0 -- the rows are vt_rows-row problems (cameras; 0 = one problem), which is the layout
+ * [B, G, D, P] that tk_batched_attn reads.  vt_col0 a multiple of 64, vt_rows of 32, vt_ld and vt_bs of 8.
+ * Replaces tk_bf16w_dense + tk_batched_transpose_v (same bits); reference: the towers' `attn @ v` operand,
+ * tybok/policies/smolvla/models/vision.py:197-257, tybok/policies/pi05/models/vision.py:115-170. */
+int tk_bf16w_dense_vt(const void* x, int ldx, const void* w_packed, const void* bias, void* y, int ldy, void* vt,
+                      int vt_col0, int vt_ld, int vt_rows, long long vt_bs, int f16, int M, int N, int K, int tile,
+                      int split_k, void* ws, size_t ws_bytes, void* stream);
+
 /* ---- action-expert attention over the cached prefix ------------------------------------------ */
 /* Lays one layer's prefix K/V out for tk_expert_attn, once per request (the counterpart of the
  * reference filling its static per-layer prefix cache after the VLM prefill,

@@ -120,6 +120,9 @@ def _cases():
         ("tk_bf16w_dense_rope", (P, 2048, P, P, 2560, P, P, P, 300, 2300, 128, 1, None, 0, 0, 712, 2560, 2048, 0, 0, None, 0, None), -1, "whole heads"),
         ("tk_bf16w_dense_rope", (P, 2048, P, P, 2560, None, P, P, 300, 2304, 128, 1, None, 0, 0, 712, 2560, 2048, 0, 0, None, 0, None), -1, "null table"),
         ("tk_bf16w_dense_rope", (P, 2048, P, P, 2560, P, P, P, 300, 2304, 128, 1, P, 2304, 712, 712, 2560, 2048, 0, 0, None, 0, None), -1, "vt_ld"),
+        ("tk_bf16w_dense_vt", (P, 768, P, P, P, 2304, P, 1500, 1024, 1024, 786432, 0, 3072, 2304, 768, 0, 0, None, 0, None), -1, "multiple of 64"),
+        ("tk_bf16w_dense_vt", (P, 768, P, P, P, 2304, P, 1536, 1024, 1000, 786432, 0, 3072, 2304, 768, 0, 0, None, 0, None), -1, "multiple of 32"),
+        ("tk_bf16w_dense_vt", (P, 768, P, P, P, 2304, None, 1536, 1024, 1024, 786432, 0, 3072, 2304, 768, 0, 0, None, 0, None), -1, "16-byte aligned"),
         ("tk_debug_fp8w_gemm_cut", (P, 2040, P, P, P, 16384, 50, 16384, 2040, 1, None), -1, "multiple of 16"),
         ("tk_fp8w_gemm", gemm(K=2040), -1, "multiple of 16"),
         ("tk_fp8w_gemm", gemm(ldx=1024), -1, "ldx"),

@@ -211,3 +211,33 @@ def test_dense_rope_argument_rules(tk):
         tk.bf16w_dense_rope(x.cuda(), pw, tables, pos.cuda(), rope_cols + 32)
     with pytest.raises(RuntimeError, match="tile"):
         tk.bf16w_dense_rope(x.cuda(), pw, tables, pos.cuda(), rope_cols, tile=31)
+
+
+@pytest.mark.parametrize("tile", [0, 42, 41, 32, 31, 22, 21, 12, 11])
+@pytest.mark.parametrize("dt", [BF16, torch.float16])
+@pytest.mark.parametrize("b,p,k,heads,d", [(3, 1024, 768, 12, 64), (2, 256, 1152, 16, 96), (1, 96, 64, 2, 64), (5, 32, 80, 1, 64)])
+def test_dense_writes_the_transposed_values_of_a_packed_qkv_projection(tk, tile, dt, b, p, k, heads, d):
+    # tk_bf16w_dense_vt: the projection's own output is unchanged and the value columns also arrive as
+    # [B, G, D, P] -- the bits tk_batched_transpose_v makes of them
+    n = 3 * heads * d
+    x, w, bias = _case(b * p, k, n, seed=5)
+    x, w, bias = x.to(dt), w.to(dt), bias.to(dt)
+    pw = tk.pack_bf16_weight(w.cuda())
+    want = tk.bf16w_dense(x.cuda(), pw, bias.cuda(), tile=tile, split_k=1)
+    vt_want = tk.transpose_v(want.view(b, p, 3, heads, d)[:, :, 2])
+    vt = torch.full((b, heads, d, p), 7.0, dtype=dt, device="cuda")
+    got = tk.bf16w_dense(x.cuda(), pw, bias.cuda(), tile=tile, split_k=1, vt_out=vt, vt_col0=2 * heads * d)
+    assert torch.equal(got, want)
+    assert torch.equal(vt, vt_want[..., :p])
+
+
+def test_dense_vt_argument_rules(tk):
+    x, w, bias = _case(64, 64, 3 * 64)
+    pw = tk.pack_bf16_weight(w.cuda())
+    vt = torch.empty(2, 1, 64, 32, dtype=BF16, device="cuda")
+    with pytest.raises(ValueError, match="no activation or residual"):
+        tk.bf16w_dense(x.cuda(), pw, bias.cuda(), "gelu_tanh", vt_out=vt, vt_col0=128)
+    with pytest.raises(ValueError, match="multiple of 32"):
+        tk.bf16w_dense(x.cuda(), pw, bias.cuda(), vt_out=torch.empty(4, 1, 64, 16, dtype=BF16, device="cuda"), vt_col0=128)
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        tk.bf16w_dense(x.cuda(), pw, bias.cuda(), vt_out=torch.empty(2, 1, 96, 32, dtype=BF16, device="cuda"), vt_col0=96)

@@ -405,6 +405,26 @@ __global__ __launch_bounds__(NW * 64, OCC) void bf16w_wide_kernel(GemmArgs a, in
       if (n + 8 <= a.N) *(i32x4*)dst = t;
       else *(i32x2*)dst = i32x2{t[0], t[1]};  // N % 8 == 4: the row's last four columns
     }
+    if (a.vt && ncol0 >= a.vt_col0) {  // wave-uniform: vt_col0 is a multiple of the wave's COLS columns
+      // value columns of a packed q|k|v projection, also written transposed for the attention kernel (no activation
+      // or residual in this form, so the LDS tile holds the final values): a lane takes one of the wave's columns
+      // and eight consecutive rows per 16-byte store.  The rows of an m tile belong to one problem (vt_rows is a
+      // multiple of 32); rows past M are written as zeros.
+      const int ccol = lane % COLS, n = ncol0 + ccol;
+      const int m0 = (mblock * MT + mt) * 32;
+      if (n < a.N && m0 < a.M) {
+        const int prob = a.vt_rows ? m0 / a.vt_rows : 0, key0 = a.vt_rows ? m0 % a.vt_rows : m0;
+        u16* dst = a.vt + (size_t)prob * a.vt_bs + (size_t)(n - a.vt_col0) * a.vt_ld + key0;
+#pragma unroll
+        for (int rg = lane / COLS; rg < 4; rg += 64 / COLS) {
+          unsigned e[8];
+#pragma unroll
+          for (int r = 0; r < 8; ++r) e[r] = m0 + 8 * rg + r < a.M ? *(const u16*)(wl + (8 * rg + r) * EP + ccol * 2) : 0u;
+          if (m0 + 8 * rg < a.M)
+            *(i32x4*)(dst + 8 * rg) = i32x4{(int)(e[0] | (e[1] << 16)), (int)(e[2] | (e[3] << 16)), (int)(e[4] | (e[5] << 16)), (int)(e[6] | (e[7] << 16))};
+        }
+      }
+    }
   }
 }
 

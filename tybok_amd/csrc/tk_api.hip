@@ -564,6 +564,13 @@ float dense_cost(const DenseTile& t, int M, int N, int KT, int ks, int cus) {
 
 namespace {
 // rotary form of the many-row linear: weights in rotary pair order, tables and positions as in tk_bf16w_linear
+// transposed copy of the columns >= col0 of a packed q|k|v projection, one problem per `rows` rows
+struct DenseVt {
+  void* vt = nullptr;
+  int col0 = 0, ld = 0, rows = 0;
+  long long bs = 0;
+};
+
 struct DenseRope {
   const int* pos = nullptr;
   const float* cos = nullptr;
@@ -575,7 +582,7 @@ struct DenseRope {
 
 int dense_common(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy, const void* resid,
                  int ldr, int resid_dtype, int M, int N, int K, int tile, int split_k, void* ws, size_t ws_bytes, void* stream,
-                 int f16, const DenseRope* rope = nullptr) {
+                 int f16, const DenseRope* rope = nullptr, const DenseVt* vt = nullptr) {
   if (M <= 0 || N <= 0 || K <= 0) return fail(TK_EINVAL, "bf16w_dense: non-positive shape M=%d N=%d K=%d", M, N, K);
   if (K % 16 || ldx % 8 || ldx < K) return fail(TK_EINVAL, "bf16w_dense: K=%d must be a multiple of 16 and ldx=%d a multiple of 8 >= K", K, ldx);
   if (!x || !w_packed || !y) return fail(TK_EINVAL, "bf16w_dense: null pointer");
@@ -624,6 +631,18 @@ int dense_common(const void* x, int ldx, const void* w_packed, const void* bias,
     a.vt = (u16*)rope->vt;
     a.vt_col0 = rope->vt_col0;
     a.vt_ld = rope->vt_ld;
+  }
+  if (vt) {
+    if (act || resid) return fail(TK_EINVAL, "bf16w_dense_vt: no activation or residual in this form");
+    if (!vt->vt || !aligned16(vt->vt) || vt->col0 < 0 || vt->col0 >= N || vt->col0 % 64 || vt->ld % 8 || vt->rows < 0 || vt->rows % 32 || vt->bs % 8 ||
+        vt->ld < (vt->rows ? vt->rows : (M + 31) / 32 * 32))
+      return fail(TK_EINVAL, "bf16w_dense_vt: vt 16-byte aligned, vt_col0=%d a multiple of 64 below N, vt_rows=%d a multiple of 32, vt_ld=%d a multiple of 8 that holds a problem's rows, vt_bs a multiple of 8",
+                  vt->col0, vt->rows, vt->ld);
+    a.vt = (u16*)vt->vt;
+    a.vt_col0 = vt->col0;
+    a.vt_ld = vt->ld;
+    a.vt_rows = vt->rows;
+    a.vt_bs = vt->bs;
   }
   const int cus = device_cus();
   const DenseTile* best = nullptr;
@@ -690,6 +709,17 @@ int tk_bf16w_dense_rope(const void* x, int ldx, const void* w_packed, void* y, i
   r.vt_col0 = vt_col0;
   r.vt_ld = vt_ld;
   return dense_common(x, ldx, w_packed, nullptr, 0, y, ldy, nullptr, 0, 0, M, N, K, tile, split_k, ws, ws_bytes, stream, 0, &r);
+}
+
+int tk_bf16w_dense_vt(const void* x, int ldx, const void* w_packed, const void* bias, void* y, int ldy, void* vt, int vt_col0, int vt_ld,
+                      int vt_rows, long long vt_bs, int f16, int M, int N, int K, int tile, int split_k, void* ws, size_t ws_bytes, void* stream) {
+  DenseVt v;
+  v.vt = vt;
+  v.col0 = vt_col0;
+  v.ld = vt_ld;
+  v.rows = vt_rows;
+  v.bs = vt_bs;
+  return dense_common(x, ldx, w_packed, bias, 0, y, ldy, nullptr, 0, 0, M, N, K, tile, split_k, ws, ws_bytes, stream, f16 ? 1 : 0, nullptr, &v);
 }
 
 int tk_f16w_dense(const void* x, int ldx, const void* w_packed, const void* bias, int act, void* y, int ldy, const void* resid,

@@ -45,6 +45,10 @@ struct GemmArgs {
   unsigned short* vt;
   int vt_col0;
   int vt_ld;
+  // many-row 16-bit kernel only: the rows are vt_rows-row problems (0 = one problem) and problem b's transposed
+  // columns start vt_bs elements after problem b-1's: vt[(m / vt_rows) * vt_bs + (n - vt_col0) * vt_ld + m % vt_rows]
+  int vt_rows;
+  long long vt_bs;
   // W8A8 launches only: x holds e4m3fn codes (ldx in bytes) and row_scale the per-token fp32 scales
   const float* row_scale;
   // many-row kernels: y (and the residual) allow 16-byte row-contiguous accesses (pitches multiples of 8

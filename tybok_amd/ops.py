@@ -362,9 +362,14 @@ def bf16w_dense(
     tile: int = 0,
     split_k: int = 0,
     ws: Workspace | None = None,
+    vt_out: torch.Tensor | None = None,
+    vt_col0: int = 0,
 ) -> torch.Tensor:
     """``bf16(resid + act(bf16(x @ W^T + bias)))`` for ``x [M, K]`` bf16 and a packed bf16 weight: the linears of the
-    vision towers on the many-row MFMA kernel.  ``act``: ``"gelu_tanh"`` applies the tanh GELU to the bf16-rounded
+    vision towers on the many-row MFMA kernel.  With ``vt_out [B, G, D, P]`` (``B * P == M``, ``P`` a multiple of 32,
+    ``G * D == N - vt_col0``) the columns from ``vt_col0`` on are also written transposed per problem -- the V^T
+    operand of :func:`batched_attn` straight from a packed q|k|v projection (``tk_bf16w_dense_vt``; no ``act`` /
+    ``resid`` in that form).  ``act``: ``"gelu_tanh"`` applies the tanh GELU to the bf16-rounded
     linear output (what ``gelu(linear(x))`` on bf16 tensors computes), ``"gelu_tanh_fp32"`` to the fp32 one (a GEMM
     with the activation in its epilogue).  ``tile`` picks the block tile (0 = by shape).  With fp16 activations and
     a weight packed from an fp16 matrix every 16-bit operand is fp16 (``tk_f16w_dense``: pi0.5's fp16 tower tiers)."""
@@ -390,6 +395,20 @@ def bf16w_dense(
         if dt == torch.float16 and resid is not None and resid.dtype == torch.bfloat16:
             raise TypeError("an fp16 launch takes an fp16 or fp32 residual")
     ws = ws or default_workspace(x.device)
+    if vt_out is not None:
+        if act is not None or resid is not None:
+            raise ValueError("vt_out: no activation or residual in this form")
+        if vt_out.dtype != dt or vt_out.dim() != 4 or vt_out.stride(3) != 1 or vt_out.stride(1) != vt_out.shape[2] * vt_out.stride(2):
+            raise ValueError("vt_out must be [B, G, D, P] of the weight's type with contiguous keys and evenly pitched (g, d) rows")
+        nb, ng, nd, npk = vt_out.shape
+        if nb * npk != m or npk % 32 or ng * nd != w.n - vt_col0:
+            raise ValueError("vt_out: B * P must equal M, P be a multiple of 32 and G * D equal N - vt_col0")
+        rc = lib.tk_bf16w_dense_vt(
+            x.data_ptr(), ldx, w.data.data_ptr(), None if bias is None else bias.data_ptr(), out.data_ptr(), out.stride(0), vt_out.data_ptr(),
+            vt_col0, vt_out.stride(2), npk, vt_out.stride(0), int(dt == torch.float16), m, w.n, w.k, tile, split_k, ws.ptr, ws.nbytes, _stream(),
+        )  # fmt: skip
+        native.check(rc, "tk_bf16w_dense_vt")
+        return out
     entry = lib.tk_f16w_dense if dt == torch.float16 else lib.tk_bf16w_dense
     rc = entry(
         x.data_ptr(), ldx, w.data.data_ptr(), None if bias is None else bias.data_ptr(), _DENSE_ACTS[act], out.data_ptr(),

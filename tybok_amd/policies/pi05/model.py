@@ -321,8 +321,16 @@ class PI05Model:
 
         for i in range(cfg.vision_layers):
             lp = f"{VIS}encoder.layers.{i}."
-            qkv = dense(lp + "self_attn.qkv", h).view(b, -1, 3, heads, hp)
-            a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], tk.transpose_v(qkv[:, :, 2]), scale=hd**-0.5, ws=self.ws)
+            tokens = h.shape[1]
+            if self.vis_dense and tokens % 32 == 0:
+                # V^T for the attention launch written by the projection's epilogue (one launch less per layer)
+                w, bias = self.vis_dense[lp + "self_attn.qkv"]
+                vt = torch.empty(b, heads, hp, tokens, dtype=qdt, device=h.device)
+                qkv = tk.bf16w_dense(h.reshape(-1, h.shape[-1]), w, bias, vt_out=vt, vt_col0=2 * heads * hp, ws=self.ws).view(b, -1, 3, heads, hp)
+            else:
+                qkv = dense(lp + "self_attn.qkv", h).view(b, -1, 3, heads, hp)
+                vt = tk.transpose_v(qkv[:, :, 2])
+            a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, scale=hd**-0.5, ws=self.ws)
             x, h = tk.add_layer_norm(x, dense(lp + "self_attn.out_proj", a), *ln(i, 2), EPS)
             # fc1's GELU on the fp32 pre-activation, the activation rounded to bf16 for fc2: the reference's fused MLP
             # (`_vision_mlp_up_kernel`, tybok/policies/pi05/models/triton_vision.py:113-187)

@@ -267,8 +267,14 @@ class SmolVLAModel:
                 # packed q|k|v GEMM, then the HIP attention (one problem per camera): q.K^T rounded to
                 # bf16 before the fp32 scale and softmax, exactly what the bf16 matmul below produces
                 w_qkv, b_qkv = self.vis_qkv[i]
-                qkv = self._dense_w(w_qkv, b_qkv, h).view(b, -1, 3, heads, hd)
-                vt = tk.transpose_v(qkv[:, :, 2])
+                tokens = h.shape[1]
+                if not isinstance(w_qkv, torch.Tensor) and tokens % 32 == 0:
+                    # V^T for the attention launch written by the projection's epilogue (one launch less per layer)
+                    vt = torch.empty(b, heads, hd, tokens, dtype=h.dtype, device=h.device)
+                    qkv = tk.bf16w_dense(h.reshape(-1, h.shape[-1]), w_qkv, b_qkv, vt_out=vt, vt_col0=2 * heads * hd, ws=self.ws).view(b, -1, 3, heads, hd)
+                else:
+                    qkv = self._dense_w(w_qkv, b_qkv, h).view(b, -1, 3, heads, hd)
+                    vt = tk.transpose_v(qkv[:, :, 2])
                 a = tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, ws=self.ws)
                 x, h = tk.add_layer_norm(x, self._dense(lp + "self_attn.out_proj", a), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
                 # fc1's GELU on the bf16-rounded linear output, as gelu(linear(h)) on bf16 tensors computes it
