@@ -52,7 +52,6 @@ __device__ __forceinline__ void lds_only_barrier() {
 __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs a) {
   constexpr int DS = kD / 16;  // k steps of Q.K^T
   __shared__ float st_m[kWaves][32], st_l[kWaves][32];
-  __shared__ int s_last;
   // dynamic LDS: the Q tile (later the P^T operands of every key tile), then one staging tile per wave
   // (its K tile, later its V^T rows); rows of 512 bytes at a pitch that keeps 16-byte operand reads of
   // 32 rows conflict-free
@@ -282,33 +281,33 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
     return;
   }
 
-  // ---- key-split merge by the last-arriving block ----
-  // partials per (block, split): [2][32] statistics, then [wave][group][lane][4 floats]
+  // ---- key-split merge, wave by wave: wave w of every split block leaves its slice of O^T (with its own copy of
+  // the statistics, which are the same in every wave) and counts itself in on counter (block, w); the wave that
+  // arrives last for a slice merges that slice.  No block barrier in the chain: a wave's store acknowledgement,
+  // count and read-back overlap with the other waves'. ----
+  // partials per (block, split): [wave][2][32] statistics, then [wave][group][lane][4 floats]
   const int blk_lin = mtile * a.H + h;
-  constexpr size_t PSTRIDE = 64 + (size_t)kWaves * 1024;  // floats
+  constexpr size_t PSTRIDE = (size_t)kWaves * 64 + (size_t)kWaves * 1024;  // floats
   float* pmine = a.partial + ((size_t)blk_lin * a.kv_splits + split) * PSTRIDE;
-  if (wave == 0 && half == 0) {
-    st_agent(pmine + l32, bm);
-    st_agent(pmine + 32 + l32, bl);
+  if (half == 0) {
+    st_agent(pmine + wave * 64 + l32, bm);
+    st_agent(pmine + wave * 64 + 32 + l32, bl);
   }
   {
-    unsigned long long* dst = (unsigned long long*)(pmine + 64) + ((size_t)wave * 256 + lane) * 2;
+    unsigned long long* dst = (unsigned long long*)(pmine + kWaves * 64) + ((size_t)wave * 256 + lane) * 2;
 #pragma unroll
     for (int g4 = 0; g4 < 4; ++g4) {
       st_agent64(dst + (size_t)g4 * 128, o[4 * g4], o[4 * g4 + 1]);
       st_agent64(dst + (size_t)g4 * 128 + 1, o[4 * g4 + 2], o[4 * g4 + 3]);
     }
   }
-  handoff_publish();  // partials acknowledged (written through) before the count
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_last = (old == a.kv_splits - 1);
-  }
-  __syncthreads();
-  if (!s_last) return;
+  handoff_publish();  // this wave's slice acknowledged (written through) before its count
+  int old = 0;
+  if (lane == 0) old = __hip_atomic_fetch_add(a.counters + blk_lin * kWaves + wave, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  old = __builtin_amdgcn_readfirstlane(old);
+  if (old != a.kv_splits - 1) return;  // wave-uniform
   handoff_acquire();
-  if (threadIdx.x == 0) __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (lane == 0) __hip_atomic_store(a.counters + blk_lin * kWaves + wave, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
   const float* pblk = a.partial + (size_t)blk_lin * a.kv_splits * PSTRIDE;
   // every read of the hand-off goes out before the first one is consumed
@@ -319,14 +318,14 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
     ms[s] = -INFINITY;
     ls[s] = 0.f;
     if (s < a.kv_splits) {  // block-uniform
-      ms[s] = ld_agent(pblk + (size_t)s * PSTRIDE + l32);
-      ls[s] = ld_agent(pblk + (size_t)s * PSTRIDE + 32 + l32);
+      ms[s] = ld_agent(pblk + (size_t)s * PSTRIDE + wave * 64 + l32);
+      ls[s] = ld_agent(pblk + (size_t)s * PSTRIDE + wave * 64 + 32 + l32);
     }
   }
 #pragma unroll
   for (int s = 0; s < kMaxSplits; ++s) {
     if (s < a.kv_splits) {
-      const unsigned long long* src = (const unsigned long long*)(pblk + (size_t)s * PSTRIDE + 64) + ((size_t)wave * 256 + lane) * 2;
+      const unsigned long long* src = (const unsigned long long*)(pblk + (size_t)s * PSTRIDE + kWaves * 64) + ((size_t)wave * 256 + lane) * 2;
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         raw[s][g4][0] = ld_agent64(src + (size_t)g4 * 128);

@@ -546,7 +546,10 @@ __device__ __forceinline__ void gemm_block(const GemmArgs& a, const int strip, c
     own[t] = sum;
   }
 
-  // ---- K-split reduction through global partials; the last-arriving block finishes ----
+  // ---- K-split reduction through global partials, wave by wave: wave w of every split block leaves register
+  // group w of its tiles and counts itself in on counter (block, w); the wave that arrives last for a group sums
+  // that group in split order and finishes it.  No block barrier in the chain: a wave's store acknowledgement,
+  // count and read-back overlap with the other waves'. ----
   const int blk_lin = mblock * nstrips + strip;
   if (a.ksplit > 1) {
     // partial layout: [(block, split)][tile][group][lane][4 floats], written and read as 8-byte
@@ -558,19 +561,15 @@ __device__ __forceinline__ void gemm_block(const GemmArgs& a, const int strip, c
       st_agent64(dst, own[t][0], own[t][1]);
       st_agent64(dst + 1, own[t][2], own[t][3]);
     }
-    // wait until the partials are acknowledged, then count this block in
-    __shared__ int s_last;
+    // wait until this wave's partials are acknowledged, then count it in
     handoff_publish();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_last = (old == a.ksplit - 1);
-    }
-    __syncthreads();
-    if (!s_last) return;
+    int* counter = a.counters + blk_lin * RW + wave;
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (__builtin_amdgcn_readfirstlane(old) != a.ksplit - 1) return;  // wave-uniform
     handoff_acquire();
-    if (threadIdx.x == 0)  // leave the counter ready for the next launch
-      __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0)  // leave the counter ready for the next launch
+      __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
     for (int t = 0; t < TILES; ++t) own[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     // sum in split order; four splits' loads are in flight together

@@ -295,7 +295,7 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
       float best = 1e30f;
       // (an automatic choice never asks for more partial space than the workspace holds)
       const size_t cap = !ws || ws_bytes <= kPartialOff ? 0 : (ws_bytes - kPartialOff < kPartialBytes ? ws_bytes - kPartialOff : kPartialBytes);
-      for (int c = 1; c <= 64 && c * NW <= a.KT && (c == 1 || (blocks0 * c <= 2 * cus && (size_t)blocks0 * c * MT * NT * 4096 <= cap && blocks0 <= kMaxCounters)); ++c) {
+      for (int c = 1; c <= 64 && c * NW <= a.KT && (c == 1 || (blocks0 * c <= 2 * cus && (size_t)blocks0 * c * MT * NT * 4096 <= cap && blocks0 * 4 <= kMaxCounters)); ++c) {
         const int rounds = (a.KT + c * NW - 1) / (c * NW);
         float t = rounds * per_round;
         if (t < 1.0f) t = 1.0f;
@@ -317,11 +317,12 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
   if (ks > 1) {
     if (!ws) return fail(TK_EWORKSPACE, "gemm: split_k=%d needs a workspace", ks);
     const size_t need = (size_t)blocks0 * ks * MT * NT * 4096;
-    if (blocks0 > kMaxCounters || need > kPartialBytes || ws_bytes < kPartialOff + need)
-      return fail(TK_EWORKSPACE, "gemm: workspace too small (need %zu partial bytes, %d counters)", need, blocks0);
+    // (an arrival counter per block and finishing wave: the four waves of a block hand over on their own)
+    if (blocks0 * 4 > kMaxCounters || need > kPartialBytes || ws_bytes < kPartialOff + need)
+      return fail(TK_EWORKSPACE, "gemm: workspace too small (need %zu partial bytes, %d counters)", need, blocks0 * 4);
     a.partial = (float*)((char*)ws + kPartialOff);
     a.counters = (int*)ws;
-    if (!plan && e.clear_counters && tk_launch_fill_zero(a.counters, blocks0, st)) return fail(TK_ELAUNCH, "gemm: counter fill launch failed");
+    if (!plan && e.clear_counters && tk_launch_fill_zero(a.counters, blocks0 * 4, st)) return fail(TK_ELAUNCH, "gemm: counter fill launch failed");
   }
   // 33..64 rows over a large fp8 matrix: the weight-streaming schedule
   const bool stream = MT == 2 && NT == 2 && mblocks == 1 && tk_gemm_stream_takes(a);
@@ -1008,8 +1009,9 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
     if (sp > tk_attn_d256_max_splits()) sp = tk_attn_d256_max_splits();
     if (H * mtiles * 2 >= device_cus()) sp = 1;  // the query tiles alone fill half the device: no hand-off
     while (sp > 1 && H * mtiles * sp > 2 * device_cus()) --sp;
-    const size_t need = (size_t)H * mtiles * sp * (64 + (size_t)(D / 32) * 1024) * 4;
-    if (sp > 1 && !(ws && H * mtiles <= kMaxCounters && need <= kPartialBytes && ws_bytes >= kPartialOff + need)) sp = 1;
+    // (a statistics record and an arrival counter per wave: the waves of a block hand over on their own)
+    const size_t need = (size_t)H * mtiles * sp * (size_t)(D / 32) * (64 + 1024) * 4;
+    if (sp > 1 && !(ws && H * mtiles * (D / 32) <= kMaxCounters && need <= kPartialBytes && ws_bytes >= kPartialOff + need)) sp = 1;
     d256 = true;
     splits = sp;
   }
@@ -1024,8 +1026,9 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   a.partial = nullptr;
   a.counters = nullptr;
   if (splits > 1) {
-    const int blocks = H * mtiles;
-    const size_t need = (size_t)blocks * splits * (64 + (size_t)(D / 32) * 1024) * 4;
+    const int blocks = H * mtiles * (d256 ? D / 32 : 1);  // arrival counters
+    const size_t need = d256 ? (size_t)H * mtiles * splits * (size_t)(D / 32) * (64 + 1024) * 4
+                             : (size_t)blocks * splits * (64 + (size_t)(D / 32) * 1024) * 4;
     if (!ws || blocks > kMaxCounters || need > kPartialBytes || ws_bytes < kPartialOff + need)
       return fail(TK_EWORKSPACE, "attn: workspace too small (need %zu bytes)", need);
     a.partial = (float*)((char*)ws + kPartialOff);
