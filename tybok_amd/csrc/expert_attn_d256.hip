@@ -303,11 +303,11 @@ __global__ __launch_bounds__(kWaves * 64) void expert_attn_d256_kernel(AttnArgs 
   }
   handoff_publish();  // this wave's slice acknowledged (written through) before its count
   int old = 0;
-  if (lane == 0) old = __hip_atomic_fetch_add(a.counters + blk_lin * kWaves + wave, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (lane == 0) old = __hip_atomic_fetch_add(a.counters + (blk_lin * kWaves + wave) * 16, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   old = __builtin_amdgcn_readfirstlane(old);
   if (old != a.kv_splits - 1) return;  // wave-uniform
   handoff_acquire();
-  if (lane == 0) __hip_atomic_store(a.counters + blk_lin * kWaves + wave, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (lane == 0) __hip_atomic_store(a.counters + (blk_lin * kWaves + wave) * 16, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
   const float* pblk = a.partial + (size_t)blk_lin * a.kv_splits * PSTRIDE;
   // every read of the hand-off goes out before the first one is consumed

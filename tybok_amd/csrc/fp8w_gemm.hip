@@ -563,7 +563,7 @@ __device__ __forceinline__ void gemm_block(const GemmArgs& a, const int strip, c
     }
     // wait until this wave's partials are acknowledged, then count it in
     handoff_publish();
-    int* counter = a.counters + blk_lin * RW + wave;
+    int* counter = a.counters + (size_t)(blk_lin * RW + wave) * a.cstride;
     int old = 0;
     if (lane == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (__builtin_amdgcn_readfirstlane(old) != a.ksplit - 1) return;  // wave-uniform

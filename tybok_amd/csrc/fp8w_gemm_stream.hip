@@ -306,14 +306,14 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
     handoff_publish();
     __syncthreads();
     if (threadIdx.x == 0) {
-      const int old = __hip_atomic_fetch_add(a.counters + blk_lin, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int old = __hip_atomic_fetch_add(a.counters + (size_t)blk_lin * a.cstride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       s_last = (old == a.ksplit - 1);
     }
     __syncthreads();
     if (!s_last) return;
     handoff_acquire();
     if (threadIdx.x == 0)  // leave the counter ready for the next launch
-      __hip_atomic_store(a.counters + blk_lin, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(a.counters + (size_t)blk_lin * a.cstride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
     for (int g = 0; g < 4; ++g) own[g] = f32x4{0.f, 0.f, 0.f, 0.f};
     constexpr int SB = 8;  // splits whose partials are in flight together

@@ -322,7 +322,9 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
       return fail(TK_EWORKSPACE, "gemm: workspace too small (need %zu partial bytes, %d counters)", need, blocks0 * 4);
     a.partial = (float*)((char*)ws + kPartialOff);
     a.counters = (int*)ws;
-    if (!plan && e.clear_counters && tk_launch_fill_zero(a.counters, blocks0 * 4, st)) return fail(TK_ELAUNCH, "gemm: counter fill launch failed");
+    // a 64-byte line per counter where the region holds that many: atomics on one line queue behind each other
+    a.cstride = blocks0 * 4 * 16 <= kMaxCounters ? 16 : 1;
+    if (!plan && e.clear_counters && tk_launch_fill_zero(a.counters, blocks0 * 4 * a.cstride, st)) return fail(TK_ELAUNCH, "gemm: counter fill launch failed");
   }
   // 33..64 rows over a large fp8 matrix: the weight-streaming schedule
   const bool stream = MT == 2 && NT == 2 && mblocks == 1 && tk_gemm_stream_takes(a);
@@ -1011,7 +1013,7 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
     while (sp > 1 && H * mtiles * sp > 2 * device_cus()) --sp;
     // (a statistics record and an arrival counter per wave: the waves of a block hand over on their own)
     const size_t need = (size_t)H * mtiles * sp * (size_t)(D / 32) * (64 + 1024) * 4;
-    if (sp > 1 && !(ws && H * mtiles * (D / 32) <= kMaxCounters && need <= kPartialBytes && ws_bytes >= kPartialOff + need)) sp = 1;
+    if (sp > 1 && !(ws && H * mtiles * (D / 32) * 16 <= kMaxCounters && need <= kPartialBytes && ws_bytes >= kPartialOff + need)) sp = 1;
     d256 = true;
     splits = sp;
   }
@@ -1026,7 +1028,7 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   a.partial = nullptr;
   a.counters = nullptr;
   if (splits > 1) {
-    const int blocks = H * mtiles * (d256 ? D / 32 : 1);  // arrival counters
+    const int blocks = H * mtiles * (d256 ? (D / 32) * 16 : 1);  // arrival counters (256-wide heads: one per wave, a 64-byte line each)
     const size_t need = d256 ? (size_t)H * mtiles * splits * (size_t)(D / 32) * (64 + 1024) * 4
                              : (size_t)blocks * splits * (64 + (size_t)(D / 32) * 1024) * 4;
     if (!ws || blocks > kMaxCounters || need > kPartialBytes || ws_bytes < kPartialOff + need)

@@ -24,6 +24,7 @@ struct GemmArgs {
   int kt_q, kt_r;  // KT = ksplit * kt_q + kt_r
   float* partial;
   int* counters;
+  int cstride;  // int32 words between two arrival counters (16: a 64-byte line each -- counters that share a line queue up)
   int act;
   int vec;  // the plain epilogue may use 8/16-byte accesses (alignment and N % 4 checked by the host)
   // RMSNorm prologue (norm_w != nullptr): bf16 [K] weight, eps
