@@ -25,9 +25,11 @@ def _both(x, w, split_k, resid=None):
     ldr = resid.stride(0) if resid is not None else 0
     args = (x.data_ptr(), x.stride(0), w.data.data_ptr(), w.scale.data_ptr())
     native.check(lib.tk_fp8w_gemm(*args, want.data_ptr(), w.n, rp, ldr, 0, None, m, w.n, k, split_k, ws.ptr, ws.nbytes, st), "tk_fp8w_gemm")
-    before = torch.cuda.memory_allocated()
+    # torch's allocator makes no allocation during the call (the cumulative count: a collection of earlier tests'
+    # garbage between the two reads may free memory, it cannot allocate)
+    before = torch.cuda.memory_stats().get("allocation.all.allocated", 0)
     native.check(lib.tk_fp8w_gemm_static(*args, got.data_ptr(), w.n, rp, ldr, 0, None, m, w.n, k, split_k, st), "tk_fp8w_gemm_static")
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.memory_stats().get("allocation.all.allocated", 0) == before
     torch.cuda.synchronize()
     return got, want
 
