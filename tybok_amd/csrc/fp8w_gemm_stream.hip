@@ -78,7 +78,6 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
   constexpr int XSKIP = 3;            // pieces from this index on are requested only where the wave has live rows
   static_assert(NR >= 2 && PF >= 2 && PF <= NR && PRE >= 1 && PRE <= PF, "pipeline shape");
   __shared__ __align__(16) unsigned char lds[NBUF * XBUF];
-  __shared__ int s_last;
 
   SMARK(0);
   const int tid = threadIdx.x;
@@ -303,17 +302,16 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
         st_agent64(dst + g * 128 + 1, own[g][2], own[g][3]);
       }
     }
+    // wave by wave (a wave owns one whole output tile): acknowledged, counted in on the wave's own counter, and the
+    // wave that arrives last for a tile sums it in split order -- no block barrier in the chain
     handoff_publish();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      const int old = __hip_atomic_fetch_add(a.counters + (size_t)blk_lin * a.cstride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_last = (old == a.ksplit - 1);
-    }
-    __syncthreads();
-    if (!s_last) return;
+    int* counter = a.counters + (size_t)(blk_lin * 4 + wave) * a.cstride;
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (__builtin_amdgcn_readfirstlane(old) != a.ksplit - 1) return;  // wave-uniform
     handoff_acquire();
-    if (threadIdx.x == 0)  // leave the counter ready for the next launch
-      __hip_atomic_store(a.counters + (size_t)blk_lin * a.cstride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0)  // leave the counter ready for the next launch
+      __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
     for (int g = 0; g < 4; ++g) own[g] = f32x4{0.f, 0.f, 0.f, 0.f};
     constexpr int SB = 8;  // splits whose partials are in flight together
@@ -346,7 +344,8 @@ __global__ __launch_bounds__(256) void fp8w_stream_kernel(GemmArgs a) {
   SMARK(6);
 
   // ---- epilogue: this lane finishes row m, four groups of four columns ----
-  if (a.vec && a.vec16 && a.N % 8 == 0) {
+  if (a.vec && a.vec16 && a.N % 8 == 0 && a.ksplit == 1) {
+    // (a split launch finishes wave by wave: the waves of a block may not meet again, so it keeps the 8-byte stores)
     // rows of y that keep 16-byte alignment: the block's 64 x 64 bf16 tile passes through LDS and leaves as whole
     // 128-byte lines (8 lanes x 16 bytes per row), not as 16-byte pieces of 32 different rows per instruction
     constexpr int OP = 64 * 2 + 16;  // row pitch of the output tile (bytes)
