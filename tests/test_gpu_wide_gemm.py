@@ -73,6 +73,24 @@ def test_many_row_gemm_matches_skinny_kernel_rows(tk):
     _close(wide, skinny.cpu(), "wide vs skinny")
 
 
+@pytest.mark.parametrize("m", [712, 1024])
+def test_eight_wave_blocks_give_the_four_wave_kernels_bits(tk, m):
+    # wide launches with enough column blocks run on eight-wave blocks of 192 (M=712) or 256 (M=1024) rows that stage
+    # both operands through LDS; a 256-row slice of the same input stays on the four-wave kernel.  A row's k tiles are
+    # accumulated in the same order in both, so the shared rows must agree bit for bit -- with and without a residual.
+    k, n = 256, 32768
+    x, w8, s = gemm_case(m, k, n)
+    pw = tk.pack_fp8_weight(w8.cuda(), s.cuda())
+    xc = x.cuda()
+    r = torch.randn(m, n, generator=torch.Generator().manual_seed(5)).to(BF16).cuda()
+    for resid in (None, r):
+        full = tk.fp8w_gemm(xc, pw, resid=resid)
+        for lo in (0, m - 256):
+            part = tk.fp8w_gemm(xc[lo : lo + 256].contiguous(), pw, resid=None if resid is None else resid[lo : lo + 256].contiguous())
+            assert torch.equal(full[lo : lo + 256], part), f"rows {lo}.. differ between the two kernels"
+    _close(full[:64], (oops.lin_fp8w(x[:64], w8, s).float() + r[:64].float().cpu()).to(BF16), "eight-wave blocks vs oracle (first rows)")
+
+
 @pytest.mark.parametrize("split", [1, 2, 5, 7])
 def test_many_row_split_k_is_deterministic(tk, split):
     x, w8, s = gemm_case(300, 4096, 512)

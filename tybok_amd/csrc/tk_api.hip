@@ -218,6 +218,16 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
     // 64-row blocks, two per CU, once the 128-row grid would run in several generations anyway: co-resident
     // blocks cover each other's first loads and epilogue; few blocks keep the 128-row tile
     a.mtiles = wide_blocks >= 2 * cus ? 2 : 4;
+    if (a.mtiles == 2 && split_k <= 1) {
+      // eight-wave blocks of 192 / 256 rows with both operands through LDS, one per CU, where a CU's share of the rows
+      // (blocks in a row on it x rows per block) is no larger than with the 64-row blocks (measured on the gated
+      // 2048 -> 2 x 16384 launch: M=712 94 -> 90 us on 192 rows, 100 us on 256 -- its 384 blocks are one and a half
+      // generations; M=512 / 968 / 1024: 256-row blocks take 6 / 8 / 9 us off the FFN)
+      const int nbn = (a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols();
+      auto share = [&](int rows) { return ((nbn * ((M + rows - 1) / rows) + cus - 1) / cus) * rows; };
+      if (share(192) <= share(64)) a.mtiles = 6;
+      if (share(256) < share(192) && share(256) <= share(64)) a.mtiles = 8;
+    }
     const int brows = a.mtiles * 32;
     const int blocks0 = ((a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols()) * ((M + brows - 1) / brows);
     int ks = split_k;
