@@ -223,14 +223,30 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
       // (blocks in a row on it x rows per block) is no larger than with the 64-row blocks (measured on the gated
       // 2048 -> 2 x 16384 launch: M=712 94 -> 90 us on 192 rows, 100 us on 256 -- its 384 blocks are one and a half
       // generations; M=512 / 968 / 1024: 256-row blocks take 6 / 8 / 9 us off the FFN)
-      const int nbn = (a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols();
-      auto share = [&](int rows) { return ((nbn * ((M + rows - 1) / rows) + cus - 1) / cus) * rows; };
+      const int nb = (a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols();
+      auto share = [&](int rows) { return ((nb * ((M + rows - 1) / rows) + cus - 1) / cus) * rows; };
       if (share(192) <= share(64)) a.mtiles = 6;
       if (share(256) < share(192) && share(256) <= share(64)) a.mtiles = 8;
     }
-    const int brows = a.mtiles * 32;
-    const int blocks0 = ((a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols()) * ((M + brows - 1) / brows);
+    const int nbn = (a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols();
     int ks = split_k;
+    if (ks <= 0 && a.mtiles == 4 && !a.s1 && a.N % 4 == 0 && ws && a.KT >= 32) {
+      // Few column blocks over a long K (the down projection): 64- or 128-row blocks and the split count by a
+      // two-term cost fitted to M = 296 .. 968 at K = 16384, N = 2048 -- the k loop of the blocks that share a CU
+      // (0.1 us per 1000 row x k products) and the partials' trip through memory (0.5 us per MB).  At 296 rows
+      // 64-row blocks x 6 splits take 31.8 us where 128-row blocks x 10 take 36.2; from 712 rows on 128 x 5 / x 4.
+      double best = 1e30;
+      for (int mt = 2; mt <= 4; mt += 2)
+        for (int sp = 1; sp <= 16 && sp <= a.KT / 16; ++sp) {
+          const int nbm = (M + mt * 32 - 1) / (mt * 32);
+          const int gens = (nbn * nbm * sp + cus - 1) / cus;
+          const double loop = 1e-4 * gens * (mt * 32) * ((double)K / sp);
+          const double part = sp > 1 ? 0.5e-6 * 4.0 * sp * nbm * (mt * 32) * nbn * tk_wide_cols() : 0.0;
+          if (loop + part < best) best = loop + part, a.mtiles = mt, ks = sp;
+        }
+    }
+    const int brows = a.mtiles * 32;
+    const int blocks0 = nbn * ((M + brows - 1) / brows);
     if (ks <= 0) {
       // fill the device once; a split keeps at least 16 k tiles and its partials must fit
       ks = cus / blocks0;
