@@ -425,6 +425,26 @@ int tk_rms_norm_rows(const void* x, int ldx, const void* norm_w, const void* ada
 int tk_rope_rows(void* y, int ldy, const void* rope_pos, const void* rope_cos, const void* rope_sin, int rope_positions,
                  int rope_cols, int rope_half, int rope_bf16, int M, void* stream);
 
+/* Per-request bookkeeping of the prefix in one launch: from the pad flags (and the attention-block flags) of the P
+ * prefix tokens, the prefill's 2-D visibility, the rotary positions of the prefix and those of the S action tokens:
+ *   mask2d[i][j] = (cumsum(att)[j] <= cumsum(att)[i]) & pad[i] & pad[j]   bytes, row pitch p_pad (columns >= P zero)
+ *   pos32[j]     = clamp(cumsum(pad)[j] - 1, 0, rope_positions - 1)       int32
+ *   suf_pos[s]   = clamp(sum(pad) + s, 0, rope_positions - 1)             int32
+ * (`make_att_2d_masks` and `position_ids = cumsum(pad_masks) - 1`, tybok/policies/smolvla/models/flow_matching.py:
+ * 40-58,527-546; `prefix_pad.sum(-1) + arange(S)`, :343-350; tybok/policies/pi05/models/flow_matching.py:
+ * 440-470,609-640 with att all zero.)  pad, att: P bytes of 0 / 1 (att may be NULL); any output may be NULL;
+ * P <= 2048; p_pad a multiple of 16 >= P; mask2d 16-byte aligned. */
+int tk_prefix_meta(const void* pad, const void* att, int P, int p_pad, int rope_positions, int S, void* mask2d, void* pos32,
+                   void* suf_pos, void* stream);
+
+/* The unfolded input of a vision tower's patch embedding in one launch: n <= 4 fp32 images [3, H, W] ->
+ * bf16 rows [(image, patch row, patch column)][(channel, i, j)] of x * scale + shift (product and sum rounded to
+ * fp32 one after the other, then to bf16) -- `images * 2 - 1`, the cast and `unfold` in front of the patch GEMM
+ * (tybok/policies/smolvla/policy.py:117-163, tybok/policies/smolvla/models/vision.py:120-160).  patch a multiple of 8
+ * that divides H and W; images and out 16-byte aligned; images beyond n are ignored. */
+int tk_patchify_images(const void* img0, const void* img1, const void* img2, const void* img3, int n, int H, int W, int patch,
+                       float scale, float shift, void* out, void* stream);
+
 /* LayerNorm of token rows with the cast to the GEMM input type folded in:
  *   y[m, :] = bf16((x[m, :] - mean) * rstd * w + b), statistics in fp32 (biased variance).
  * Replaces `layer_norm1/2(x)` (+ the `.to(bf16)` of the low-precision tiers) in the encoder layers

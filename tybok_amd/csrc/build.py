@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_DIR = os.path.join(os.path.dirname(HERE), "_lib")
 OBJ_DIR = os.path.join(LIB_DIR, "obj")
 LIB_PATH = os.path.join(LIB_DIR, "libtybok_hip.so")
-SOURCES = ("fp8w_gemm.hip", "fp8w_gemm_stream.hip", "fp8w_gemm_wide.hip", "expert_attn.hip", "expert_attn_d256.hip", "expert_attn_px.hip", "expert_tail.hip", "expert_kv_proj.hip", "layer_norm.hip", "tower_attn.hip", "rope_rows.hip", "stream_read.hip", "w8a8_gemm.hip", "bf16w_gemm_wide.hip", "tk_api.hip")
+SOURCES = ("fp8w_gemm.hip", "fp8w_gemm_stream.hip", "fp8w_gemm_wide.hip", "expert_attn.hip", "expert_attn_d256.hip", "expert_attn_px.hip", "expert_tail.hip", "expert_kv_proj.hip", "layer_norm.hip", "tower_attn.hip", "rope_rows.hip", "prefix_prep.hip", "stream_read.hip", "w8a8_gemm.hip", "bf16w_gemm_wide.hip", "tk_api.hip")
 HEADERS = ("tk_common.h", "tk_kernels.h", os.path.join("..", "..", "include", "tybok_hip.h"))
 ARCH = "gfx950"
 FLAGS = (

@@ -1,0 +1,130 @@
+// Per-request bookkeeping of the prefix and the image patches on gfx950: two launches that replace the two dozen
+// tiny elementwise / scan launches which the same work costs as separate tensor operations inside a replayed graph
+// (each of them a dependent graph node with its launch gap).
+//
+//   prefix_meta_kernel   pad[P], att[P] (bytes, 0 / 1) ->
+//                          mask2d[i][j] = (cumsum(att)[j] <= cumsum(att)[i]) & pad[i] & pad[j]   (bytes, row pitch p_pad,
+//                                         columns P .. p_pad-1 zero): the prefill's 2-D visibility
+//                          pos[j]       = clamp(cumsum(pad)[j] - 1, 0, positions - 1)            (rotary positions)
+//                          suf_pos[s]   = clamp(sum(pad) + s, 0, positions - 1)                  (the action tokens')
+//   patchify_kernel      up to four fp32 images [3][H][W] -> bf16 patch rows [(camera, py, px)][(c, i, j)] of
+//                        x * scale + shift (product and sum rounded separately, as two tensor operations round them):
+//                        the unfolded input of a non-overlapping patch convolution run as one GEMM.
+#include "tk_common.h"
+#include "tk_kernels.h"
+
+namespace {
+
+constexpr int kMaxP = 2048;  // prefix tokens (8 per thread)
+
+__global__ __launch_bounds__(256) void prefix_meta_kernel(PrefixMetaArgs a) {
+  __shared__ unsigned short c_att[kMaxP], c_pad[kMaxP];
+  __shared__ unsigned char s_pad[kMaxP];
+  __shared__ int wave_tot[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // inclusive scans of both flag rows: 8 consecutive tokens per thread, wave scan of the thread sums, wave offsets
+  int la[8], lp[8], sa = 0, sp = 0;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int j = tid * 8 + e;
+    const int pv = j < a.P ? (a.pad[j] != 0) : 0;
+    const int av = (j < a.P && a.att) ? (a.att[j] != 0) : 0;
+    sa += av;
+    sp += pv;
+    la[e] = sa;
+    lp[e] = sp;
+    if (j < kMaxP) s_pad[j] = (unsigned char)pv;
+  }
+  int xa = sa, xp = sp;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int ta = __shfl_up(xa, o), tp = __shfl_up(xp, o);
+    if (lane >= o) xa += ta, xp += tp;
+  }
+  if (lane == 63) wave_tot[0][wave] = xa, wave_tot[1][wave] = xp;
+  __syncthreads();
+  int oa = xa - sa, op = xp - sp;  // exclusive over the lanes before
+  for (int w = 0; w < wave; ++w) oa += wave_tot[0][w], op += wave_tot[1][w];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int j = tid * 8 + e;
+    c_att[j] = (unsigned short)(oa + la[e]);
+    c_pad[j] = (unsigned short)(op + lp[e]);
+  }
+  __syncthreads();
+  const int hi = a.positions - 1;
+  if (blockIdx.x == 0) {
+    if (a.pos)
+      for (int j = tid; j < a.P; j += 256) {
+        const int v = (int)c_pad[j] - 1;
+        a.pos[j] = v < 0 ? 0 : (v > hi ? hi : v);
+      }
+    if (a.suf_pos) {
+      const int total = a.P > 0 ? (int)c_pad[a.P - 1] : 0;
+      for (int s = tid; s < a.S; s += 256) {
+        const int v = total + s;
+        a.suf_pos[s] = v > hi ? hi : v;
+      }
+    }
+  }
+  if (!a.mask2d) return;
+  // rows blockIdx.x, + gridDim.x, ..: 16 bytes of a row per thread and pass
+  for (int i = blockIdx.x; i < a.P; i += gridDim.x) {
+    const int ci = c_att[i], pi = s_pad[i];
+    unsigned char* row = a.mask2d + (size_t)i * a.p_pad;
+    for (int j0 = tid * 16; j0 < a.p_pad; j0 += 256 * 16) {
+      union { i32x4 v; unsigned char b[16]; } o;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int j = j0 + e;
+        o.b[e] = (j < a.P && pi && s_pad[j] && (int)c_att[j] <= ci) ? 1 : 0;
+      }
+      *(i32x4*)(row + j0) = o.v;
+    }
+  }
+}
+
+// one thread per 8 consecutive pixels of an image row (W a multiple of 8, so is the patch size or the 8 pixels would
+// straddle two patches: the host checks ps % 8 == 0)
+__global__ __launch_bounds__(256) void patchify_kernel(PatchifyArgs a) {
+  const int per_row = a.W / 8;
+  const long long per_img = (long long)3 * a.H * per_row;
+  const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= per_img * a.n) return;
+  const int cam = (int)(gid / per_img);
+  long long r = gid % per_img;
+  const int xs = (int)(r % per_row) * 8;
+  r /= per_row;
+  const int y = (int)(r % a.H), c = (int)(r / a.H);
+  const float* src = a.img[cam] + ((size_t)c * a.H + y) * a.W + xs;
+  const f32x4 v0 = *(const f32x4*)src, v1 = *(const f32x4*)(src + 4);
+  f32x4 w0, w1;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    w0[e] = add_rn(mul_rn(v0[e], a.scale), a.shift);
+    w1[e] = add_rn(mul_rn(v1[e], a.scale), a.shift);
+  }
+  const i32x2 lo = pack_bf16x4(w0), hi = pack_bf16x4(w1);
+  const int ps = a.ps, py = y / ps, iy = y % ps, px = xs / ps, ix = xs % ps;
+  const int n_w = a.W / ps, n_h = a.H / ps;
+  u16* dst = a.out + (((size_t)cam * n_h + py) * n_w + px) * (size_t)(3 * ps * ps) + ((size_t)c * ps + iy) * ps + ix;
+  *(i32x4*)dst = i32x4{lo[0], lo[1], hi[0], hi[1]};
+}
+
+}  // namespace
+
+int tk_prefix_meta_max_tokens() { return kMaxP; }
+
+int tk_launch_prefix_meta(PrefixMetaArgs a, hipStream_t st) {
+  // every block repeats the two scans (P bytes each); a block then writes every gridDim-th row of the mask
+  int blocks = a.mask2d ? (a.P + 7) / 8 : 1;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(prefix_meta_kernel, dim3(blocks), dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int tk_launch_patchify(PatchifyArgs a, hipStream_t st) {
+  const long long threads = (long long)a.n * 3 * a.H * (a.W / 8);
+  hipLaunchKernelGGL(patchify_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}

@@ -1280,6 +1280,47 @@ int tk_rope_rows(void* y, int ldy, const void* rope_pos, const void* rope_cos, c
   return TK_OK;
 }
 
+int tk_prefix_meta(const void* pad, const void* att, int P, int p_pad, int rope_positions, int S, void* mask2d, void* pos32,
+                   void* suf_pos, void* stream) {
+  if (P <= 0 || P > tk_prefix_meta_max_tokens()) return fail(TK_EINVAL, "prefix_meta: P=%d must be in 1..%d", P, tk_prefix_meta_max_tokens());
+  if (!pad || rope_positions <= 0 || S < 0 || (S > 0 && !suf_pos)) return fail(TK_EINVAL, "prefix_meta: null pad flags, empty position range or S without an output");
+  if (mask2d && (p_pad < P || p_pad % 16 || !aligned16(mask2d))) return fail(TK_EINVAL, "prefix_meta: p_pad=%d must be a multiple of 16 >= P and the mask 16-byte aligned", p_pad);
+  PrefixMetaArgs a;
+  a.pad = (const unsigned char*)pad;
+  a.att = (const unsigned char*)att;
+  a.P = P;
+  a.p_pad = p_pad;
+  a.positions = rope_positions;
+  a.S = S;
+  a.mask2d = (unsigned char*)mask2d;
+  a.pos = (int*)pos32;
+  a.suf_pos = (int*)suf_pos;
+  if (tk_launch_prefix_meta(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "prefix_meta: launch failed");
+  return TK_OK;
+}
+
+int tk_patchify_images(const void* img0, const void* img1, const void* img2, const void* img3, int n, int H, int W, int patch,
+                       float scale, float shift, void* out, void* stream) {
+  const void* imgs[4] = {img0, img1, img2, img3};
+  if (n < 1 || n > 4 || H <= 0 || W <= 0 || patch <= 0 || patch % 8 || H % patch || W % patch)
+    return fail(TK_EINVAL, "patchify: n=%d in 1..4, patch=%d a multiple of 8 that divides H=%d and W=%d", n, patch, H, W);
+  if (!out || !aligned16(out)) return fail(TK_EINVAL, "patchify: the output must be 16-byte aligned");
+  PatchifyArgs a;
+  for (int i = 0; i < 4; ++i) {
+    if (i < n && (!imgs[i] || !aligned16(imgs[i]))) return fail(TK_EINVAL, "patchify: image %d is null or not 16-byte aligned", i);
+    a.img[i] = (const float*)imgs[i < n ? i : 0];
+  }
+  a.n = n;
+  a.H = H;
+  a.W = W;
+  a.ps = patch;
+  a.scale = scale;
+  a.shift = shift;
+  a.out = (u16*)out;
+  if (tk_launch_patchify(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "patchify: launch failed");
+  return TK_OK;
+}
+
 static int layer_norm_impl(const char* who, const void* x, int ldx, int x_dtype, const void* r, int ldr, void* xsum, int ldxs,
                            const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream,
                            int y_f16 = 0) {

@@ -223,6 +223,25 @@ struct RopeRowsArgs {
   int M;
 };
 int tk_launch_rope_rows(RopeRowsArgs a, hipStream_t st);
+
+struct PrefixMetaArgs {
+  const unsigned char* pad;  // [P] 0 / 1
+  const unsigned char* att;  // [P] 0 / 1, or null (all zero)
+  int P, p_pad, positions, S;
+  unsigned char* mask2d;  // [P][p_pad] or null
+  int* pos;               // [P] or null
+  int* suf_pos;           // [S] or null
+};
+int tk_prefix_meta_max_tokens();
+int tk_launch_prefix_meta(PrefixMetaArgs a, hipStream_t st);
+
+struct PatchifyArgs {
+  const float* img[4];  // fp32 [3][H][W] each
+  int n, H, W, ps;
+  float scale, shift;
+  unsigned short* out;  // bf16 [n * (H/ps) * (W/ps)][3 * ps * ps]
+};
+int tk_launch_patchify(PatchifyArgs a, hipStream_t st);
 int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st);
 int tk_launch_tail(TailArgs a, hipStream_t st);
 int tk_tail_embed_width();  // the embedding's input width the tail kernel is built for

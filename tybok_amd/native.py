@@ -82,6 +82,8 @@ SIGNATURES: dict[str, tuple] = {
                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "tk_bf16w_dense_vt": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_longlong, c_int, c_int, c_int,
                                   c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "tk_prefix_meta": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "tk_patchify_images": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_void_p]),
     "tk_layer_norm_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tk_add_layer_norm_f16": (
         c_int,

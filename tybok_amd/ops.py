@@ -1023,6 +1023,45 @@ def rope_rows(y: torch.Tensor, rope: RopeTables, rope_pos: torch.Tensor, rope_co
     return y
 
 
+def prefix_meta(pad: torch.Tensor, att: torch.Tensor | None, rope_positions: int, suffix_len: int = 0, *, want_mask: bool = True):
+    """Prefix bookkeeping of one request in one launch: ``pad`` / ``att`` bool ``[P]`` ->
+    ``(mask2d uint8 [P, P rounded up to 32] or None, pos32 int32 [P], suf_pos int32 [suffix_len] or None)``:
+    the prefill's 2-D visibility ``(cumsum(att)[j] <= cumsum(att)[i]) & pad[i] & pad[j]``, the prefix positions
+    ``clamp(cumsum(pad) - 1)`` and the action tokens' positions ``clamp(sum(pad) + s)``."""
+    lib = native.lib()
+    if pad.dtype != torch.bool or pad.dim() != 1 or not pad.is_contiguous():
+        raise TypeError("prefix_meta: pad must be a contiguous 1-D bool tensor")
+    if att is not None and (att.dtype != torch.bool or att.shape != pad.shape or not att.is_contiguous()):
+        raise TypeError("prefix_meta: att must be a contiguous bool tensor of pad's shape")
+    p_len = pad.shape[0]
+    p_pad = (p_len + 31) // 32 * 32
+    mask2d = torch.empty(p_len, p_pad, dtype=torch.uint8, device=pad.device) if want_mask else None
+    pos32 = torch.empty(p_len, dtype=torch.int32, device=pad.device)
+    suf = torch.empty(suffix_len, dtype=torch.int32, device=pad.device) if suffix_len > 0 else None
+    rc = lib.tk_prefix_meta(pad.data_ptr(), _ptr(att), p_len, p_pad, int(rope_positions), int(suffix_len), _ptr(mask2d), pos32.data_ptr(),
+                            _ptr(suf), _stream())  # fmt: skip
+    native.check(rc, "tk_prefix_meta")
+    return mask2d, pos32, suf
+
+
+def patchify_images(images, patch: int, scale: float = 1.0, shift: float = 0.0) -> torch.Tensor:
+    """Up to four fp32 images ``[1, 3, H, W]`` (or ``[3, H, W]``) -> bf16 ``[n, (H/patch) * (W/patch), 3 * patch * patch]``
+    rows of ``x * scale + shift`` in the order of ``unfold``: the patch embedding's GEMM input."""
+    lib = native.lib()
+    images = list(images)
+    if not 1 <= len(images) <= 4:
+        raise ValueError("patchify_images: one to four images")
+    h, w = images[0].shape[-2:]
+    for img in images:
+        if img.dtype != torch.float32 or not img.is_contiguous() or img.numel() != 3 * h * w:
+            raise TypeError("patchify_images: every image must be a contiguous fp32 tensor of 3 x H x W values")
+    out = torch.empty(len(images), (h // patch) * (w // patch), 3 * patch * patch, dtype=torch.bfloat16, device=images[0].device)
+    ptrs = [img.data_ptr() for img in images] + [None] * (4 - len(images))
+    rc = lib.tk_patchify_images(*ptrs, len(images), h, w, int(patch), float(scale), float(shift), out.data_ptr(), _stream())
+    native.check(rc, "tk_patchify_images")
+    return out
+
+
 def decode_fp8_table(device: torch.device | str = "cuda") -> torch.Tensor:
     """Values of all 256 e4m3fn codes as the device's conversion instruction decodes them."""
     out = torch.empty(256, dtype=torch.float32, device=device)

@@ -438,9 +438,8 @@ class PI05Model:
         p_pad = (p_len + 31) // 32 * 32
         heads, g, d = self.vd["num_heads"], self.vd["num_kv_heads"], self.head_dim
         nq, nkv = heads * d, g * d
-        mask2d = torch.zeros(p_len, p_pad, dtype=torch.uint8, device=self.device)
-        mask2d[:, :p_len] = pad_masks[0][:, None] & pad_masks[0][None, :]
-        pos32 = (torch.cumsum(pad_masks, dim=1) - 1)[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
+        # pad x pad visibility bytes and clamp(cumsum(pad) - 1) positions: one launch
+        mask2d, pos32, _ = tk.prefix_meta(pad_masks[0].contiguous(), None, _ROPE_POSITIONS)
         qkv_all = torch.empty(self.depth, p_len, nq + 2 * nkv, dtype=BF16, device=self.device)
         vt_all = torch.zeros(self.depth, nkv, p_pad, dtype=BF16, device=self.device)
         hidden = embs[0].to(BF16)
@@ -576,7 +575,7 @@ class PI05Model:
             s = x_t.shape[1]
             if self.vt_suf is None or self.vt_suf.shape[2] < (s + 31) // 32 * 32:
                 self.vt_suf = torch.zeros(kv[0][0].shape[1], self.head_dim, (s + 31) // 32 * 32, dtype=BF16, device=self.device)
-            pos32 = (pads.sum(dim=-1)[:, None] + torch.arange(s, device=self.device)[None, :])[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
+            pos32 = tk.prefix_meta(pads[0].contiguous(), None, _ROPE_POSITIONS, s, want_mask=False)[2]  # clamp(sum(pad) + arange(s))
             for step in range(self.num_steps):
                 hidden = self.lin("action_in_proj", x_t)[0].to(BF16)
                 hidden = self._denoise_layers_fused(pads, caches, hidden, pos32, step)

@@ -300,7 +300,7 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
 
     def _core(self, images01, img_masks, lang_tokens, lang_masks, state, noise) -> torch.Tensor:
         """The unit a graph records: input scaling and the whole model."""
-        return self.model.sample_actions(self._to_model_range(images01), img_masks, lang_tokens, lang_masks, state, noise)
+        return self.model.sample_actions(images01, img_masks, lang_tokens, lang_masks, state, noise, image_range01=True)
 
     def prepare_state(self, batch: dict[str, torch.Tensor]) -> torch.Tensor:
         state = batch[OBS_STATE]

@@ -184,6 +184,10 @@ class SmolVLAModel:
         v = cfg.vlm_config.vision_config
         side = v.image_size // v.patch_size
         self.vis_pos = torch.arange(side * side, device=self.device)
+        self._pos0_32 = torch.arange(int(cfg.chunk_size), device=self.device).clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
+        # the tower's position embedding repeated for four cameras, as the residual operand of the patch launch
+        pos_w = self.p[VIS + "embeddings.position_embedding.weight"]
+        self.vis_pos_rows = pos_w[self.vis_pos].repeat(4, 1).contiguous() if self.fused_vit and pos_w.dtype == BF16 else None
         self.img_scale = torch.tensor(t.hidden_size**0.5, dtype=BF16, device=self.device)
         self.patch_w = self.p[VIS + "embeddings.patch_embedding.weight"].reshape(v.hidden_size, -1)
 
@@ -241,21 +245,45 @@ class SmolVLAModel:
         return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1).to(x.dtype)
 
     # ------------------------------------------------------------------ vision + prefix
-    def embed_image(self, image: torch.Tensor) -> torch.Tensor:
-        """``[1, 3, H, W]`` in [-1, 1] -> ``[1, 64, hidden]`` bf16 (vision.py; plain torch)."""
+    def _patch_rows_ok(self, images01) -> bool:
+        """Whether the images of a request (still in [0, 1]) can go through the one-launch patch unfolding."""
+        ps = self.cfg.vlm_config.vision_config.patch_size
+        return (
+            self.fused_vit and 1 <= len(images01) <= 4 and ps % 8 == 0
+            and all(i.is_cuda and i.dtype == torch.float32 and i.is_contiguous() and i.shape == images01[0].shape and i.shape[0] == 1 for i in images01)
+            and images01[0].shape[2] % ps == 0 and images01[0].shape[3] % ps == 0
+        )  # fmt: skip
+
+    def embed_image(self, image: torch.Tensor | None, images01=None) -> torch.Tensor:
+        """``[1, 3, H, W]`` in [-1, 1] -> ``[1, 64, hidden]`` bf16 (vision.py; plain torch).  With ``images01`` (a list
+        of ``[1, 3, H, W]`` fp32 images still in [0, 1], see ``_patch_rows_ok``) the scaling to [-1, 1], the cast and
+        the unfolding are one launch over all of them."""
         cfg = self.cfg.vlm_config
         v = cfg.vision_config
         p = self.p
-        b = image.shape[0]
         ps = v.patch_size
-        n_h, n_w = image.shape[2] // ps, image.shape[3] // ps
-        # non-overlapping patch convolution as one GEMM over unfolded patches
-        x = image.to(BF16).view(b, 3, n_h, ps, n_w, ps).permute(0, 2, 4, 1, 3, 5).reshape(b, n_h * n_w, 3 * ps * ps)
+        if images01 is not None:
+            b = len(images01)
+            x = tk.patchify_images(images01, ps, 2.0, -1.0)
+        else:
+            b = image.shape[0]
+            n_h, n_w = image.shape[2] // ps, image.shape[3] // ps
+            # non-overlapping patch convolution as one GEMM over unfolded patches
+            x = image.to(BF16).view(b, 3, n_h, ps, n_w, ps).permute(0, 2, 4, 1, 3, 5).reshape(b, n_h * n_w, 3 * ps * ps)
+        pos_added = False
         if self.fused_vit:
-            x = self._dense("patch", x)
+            w_patch, b_patch = self.vis_dense["patch"]
+            rows = b * x.shape[1]
+            if not isinstance(w_patch, torch.Tensor) and self.vis_pos_rows is not None and rows <= self.vis_pos_rows.shape[0] and x.shape[1] == self.vis_pos.shape[0]:
+                # the position embedding enters as the launch's residual: bf16(pos + bf16(x . W^T + b)), what the add computes
+                x = tk.bf16w_dense(x.reshape(rows, -1), w_patch, b_patch, resid=self.vis_pos_rows[:rows], ws=self.ws).view(b, -1, w_patch.n)
+                pos_added = True
+            else:
+                x = self._dense("patch", x)
         else:
             x = F.linear(x, self.patch_w, p[VIS + "embeddings.patch_embedding.bias"])
-        x = x + p[VIS + "embeddings.position_embedding.weight"][self.vis_pos][None]
+        if not pos_added:
+            x = x + p[VIS + "embeddings.position_embedding.weight"][self.vis_pos][None]
         heads = v.num_attention_heads
         hd = v.hidden_size // heads
         for i in range(v.num_hidden_layers):
@@ -313,10 +341,19 @@ class SmolVLAModel:
             return F.gelu(y, approximate="tanh") if act else y
         return tk.bf16w_dense(x.reshape(-1, x.shape[-1]), w, bias, act, ws=self.ws).view(*x.shape[:-1], w.n)
 
-    def embed_prefix(self, images, img_masks, lang_tokens, lang_masks, state):
-        """-> ``(embs fp32 [1,P,hidden], pad_masks bool [1,P], att_masks bool [1,P])`` (flow_matching.py:160-257)."""
+    def embed_prefix(self, images, img_masks, lang_tokens, lang_masks, state, image_range01: bool = False):
+        """-> ``(embs fp32 [1,P,hidden], pad_masks bool [1,P], att_masks bool [1,P])`` (flow_matching.py:160-257).
+        ``image_range01``: the images are still in [0, 1] (``x * 2 - 1`` is applied here, in the patch launch where
+        that is possible)."""
         embs, pads = [], []
-        if len(images) > 1 and all(img.shape == images[0].shape for img in images):
+        if image_range01 and self._patch_rows_ok(images):
+            per_image = (self.embed_image(None, images01=list(images)) * self.img_scale).split(1, dim=0)
+            images = ()
+        elif image_range01:
+            images = [img * 2.0 - 1.0 for img in images]
+        if not images:
+            pass
+        elif len(images) > 1 and all(img.shape == images[0].shape for img in images):
             # one pass of the vision tower over all cameras: rows are independent, and the tower's
             # GEMMs fill the device three times better than one 1024-patch image at a time
             per_image = (self.embed_image(torch.cat(list(images), dim=0)) * self.img_scale).split(images[0].shape[0], dim=0)
@@ -369,17 +406,17 @@ class SmolVLAModel:
             hidden = self._layer_tail(lp, self.vlm_mlp[i], att, hidden)
         return keys, values
 
-    def _prefill_setup(self, embs, pad_masks, att_masks) -> dict:
-        """Per-request operands of the fused prefill: 2-D visibility bytes, positions, output buffers."""
+    def _prefill_setup(self, embs, pad_masks, att_masks, suffix_len: int = 0) -> dict:
+        """Per-request operands of the fused prefill: 2-D visibility bytes, positions (and those of ``suffix_len``
+        action tokens, under ``suf_pos``), output buffers.  The bookkeeping is one launch: ``make_att_2d_masks``,
+        ``cumsum(pad_masks) - 1`` and ``prefix_pad.sum() + arange(s)`` clamped into the rotary table."""
         p_len = embs.shape[1]
         p_pad = (p_len + 31) // 32 * 32
         nq, nkv = self.heads * self.head_dim, self.kv_heads * self.head_dim
-        mask2d = torch.zeros(p_len, p_pad, dtype=torch.uint8, device=self.device)
-        mask2d[:, :p_len] = self.make_att_2d_masks(pad_masks, att_masks)[0]
-        pos32 = (torch.cumsum(pad_masks, dim=1) - 1)[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
+        mask2d, pos32, suf_pos = tk.prefix_meta(pad_masks[0].contiguous(), att_masks[0].contiguous(), _ROPE_POSITIONS, suffix_len)
         qkv_all = torch.empty(self.num_layers, p_len, nq + 2 * nkv, dtype=BF16, device=self.device)
         vt_all = torch.zeros(self.num_layers, nkv, p_pad, dtype=BF16, device=self.device)
-        return dict(p_len=p_len, p_pad=p_pad, mask2d=mask2d, pos32=pos32, qkv_all=qkv_all, vt_all=vt_all)
+        return dict(p_len=p_len, p_pad=p_pad, mask2d=mask2d, pos32=pos32, suf_pos=suf_pos, qkv_all=qkv_all, vt_all=vt_all)
 
     def _prefill_layer_fused(self, i: int, hidden: torch.Tensor, c: dict) -> torch.Tensor:
         """One VLM layer on the fused launches: norm + q|k|v + RoPE, attention under the 2-D prefix
@@ -410,13 +447,20 @@ class SmolVLAModel:
         values = c["qkv_all"][:, None, :, nq + nkv :].unflatten(-1, (h_kv, d))
         return keys, values, c["vt_all"].view(self.num_layers, h_kv, d, c["p_pad"])
 
-    def prefill_fused(self, embs, pad_masks, att_masks):
-        """VLM prefill on the fused launches -> ``(K, V, V^T)`` (see ``_prefill_views``)."""
-        c = self._prefill_setup(embs, pad_masks, att_masks)
+    def prefill_fused(self, embs, pad_masks, att_masks, suffix_len: int = 0):
+        """VLM prefill on the fused launches -> ``(K, V, V^T)`` (see ``_prefill_views``); with ``suffix_len`` also
+        the int32 rotary positions of that many action tokens behind the valid prefix, as a fourth item."""
+        c = self._prefill_setup(embs, pad_masks, att_masks, suffix_len)
         hidden = embs[0]
         for i in range(self.num_layers):
             hidden = self._prefill_layer_fused(i, hidden, c)
-        return self._prefill_views(c)
+        return (*self._prefill_views(c), c["suf_pos"]) if suffix_len else self._prefill_views(c)
+
+    def _suffix_pos0(self, s: int) -> torch.Tensor:
+        """int32 ``[s]`` positions of the action tokens counted from 0 (the cross layers'): ``pos - pos.min()``."""
+        if self._pos0_32.shape[0] == s:
+            return self._pos0_32  # built with the model: a tensor first written inside a graph capture must not be kept
+        return torch.arange(s, device=self.device).clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
 
     def _expert_prefix_kv_layer(self, i: int, keys_i, values_i):
         lp = f"{EXP}layers.{i}.self_attn."
@@ -580,8 +624,8 @@ class SmolVLAModel:
         of the device idle, so they overlap almost completely.  The streams join before step 1."""
         main, side = torch.cuda.current_stream(), self.side_stream
         dt = -1.0 / self.num_steps
-        positions = tuple(t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32) for t in self.suffix_positions(pads, noise.shape[1]))
-        c = self._prefill_setup(embs, pads, att)
+        c = self._prefill_setup(embs, pads, att, noise.shape[1])
+        positions = (c["suf_pos"], self._suffix_pos0(noise.shape[1]))
         keys, values, vt = self._prefill_views(c)
         side.wait_stream(main)
         with torch.cuda.stream(side):
@@ -619,21 +663,24 @@ class SmolVLAModel:
     def sample_actions_core(self, embs, pads, att, noise, trace: dict | None = None) -> torch.Tensor:
         if self.overlap and getattr(self.cfg, "sampler", "euler") == "euler" and trace is None and embs.shape[0] == 1 and noise.shape[0] == 1 and noise.dtype == torch.float32 and noise.is_contiguous():
             return self._sample_actions_overlapped(embs, pads, att, noise)
-        vt = None
+        vt = suf_pos = None
+        fused = self.fused_expert and noise.shape[0] == 1
         if self.fused_prefill and embs.shape[0] == 1:
-            keys, values, vt = self.prefill_fused(embs, pads, att)
+            keys, values, vt, suf_pos = self.prefill_fused(embs, pads, att, noise.shape[1])
         else:
             keys, values = self.prefill(embs, pads, att)
-        fused = self.fused_expert and noise.shape[0] == 1
         # the fused tier projects the cross layers' K/V inside attention_caches (one launch per layer)
         ekv = None if fused and trace is None else self.expert_prefix_kv(keys, values)
         if trace is not None:
             trace.update(prefix_embs=embs, pad_masks=pads, keys=keys, values=values, ekv=ekv)
         dt = -1.0 / self.num_steps
         x_t = noise
-        positions = self.suffix_positions(pads, noise.shape[1])
-        if self.fused_expert and noise.shape[0] == 1:
-            positions = tuple(t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32) for t in positions)
+        if fused and suf_pos is not None:
+            positions = (suf_pos, self._suffix_pos0(noise.shape[1]))  # from the prefill's bookkeeping launch
+        else:
+            positions = self.suffix_positions(pads, noise.shape[1])
+            if fused:
+                positions = tuple(t[0].clamp(0, _ROPE_POSITIONS - 1).to(torch.int32) for t in positions)
         caches = self.attention_caches(keys, values, ekv, vt) if self.fused_expert and noise.shape[0] == 1 else None
         fused_loop = caches is not None and x_t.dtype == torch.float32 and x_t.is_contiguous()
         if getattr(self.cfg, "sampler", "euler") == "heun":
@@ -661,7 +708,7 @@ class SmolVLAModel:
             x_t = x_t + dt * v_t
         return x_t
 
-    def sample_actions(self, images, img_masks, lang_tokens, lang_masks, state, noise, trace: dict | None = None) -> torch.Tensor:
+    def sample_actions(self, images, img_masks, lang_tokens, lang_masks, state, noise, trace: dict | None = None, image_range01: bool = False) -> torch.Tensor:
         """Prefix embed, prefill, expert prefix KV, Euler loop -> ``[1, chunk, max_action_dim]`` fp32."""
-        embs, pads, att = self.embed_prefix(images, img_masks, lang_tokens, lang_masks, state)
+        embs, pads, att = self.embed_prefix(images, img_masks, lang_tokens, lang_masks, state, image_range01)
         return self.sample_actions_core(embs, pads, att, noise, trace)
