@@ -185,6 +185,19 @@ class SmolVLAModel:
         side = v.image_size // v.patch_size
         self.vis_pos = torch.arange(side * side, device=self.device)
         self._pos0_32 = torch.arange(int(cfg.chunk_size), device=self.device).clamp(0, _ROPE_POSITIONS - 1).to(torch.int32)
+        # constants of the prefix for one to four cameras: the state token's pad flag and the attention-block flags (only
+        # the state token opens a block); built here because a tensor first written inside a graph capture must not be kept
+        self._true11 = torch.ones(1, 1, dtype=torch.bool, device=self.device)
+        self._att_const = {}
+        for n_cams in range(1, 5):
+            p_len = n_cams * (side // cfg.vlm_config.scale_factor) ** 2 + int(cfg.tokenizer_max_length) + 1
+            att = torch.zeros(1, p_len, dtype=torch.bool, device=self.device)
+            att[:, -1] = True
+            self._att_const[p_len] = att
+        # pixel shuffle (scale_factor x scale_factor neighbouring tokens side by side in one row) as a permutation of tokens
+        sf, seq = cfg.vlm_config.scale_factor, side * side
+        tok = torch.arange(seq, device=self.device).view(1, side, side // sf, sf).permute(0, 2, 1, 3)
+        self.shuffle_perm = tok.reshape(1, side // sf, side // sf, sf * sf).permute(0, 2, 1, 3).reshape(seq).contiguous()
         # the tower's position embedding repeated for four cameras, as the residual operand of the patch launch
         pos_w = self.p[VIS + "embeddings.position_embedding.weight"]
         self.vis_pos_rows = pos_w[self.vis_pos].repeat(4, 1).contiguous() if self.fused_vit and pos_w.dtype == BF16 else None
@@ -270,7 +283,7 @@ class SmolVLAModel:
             n_h, n_w = image.shape[2] // ps, image.shape[3] // ps
             # non-overlapping patch convolution as one GEMM over unfolded patches
             x = image.to(BF16).view(b, 3, n_h, ps, n_w, ps).permute(0, 2, 4, 1, 3, 5).reshape(b, n_h * n_w, 3 * ps * ps)
-        pos_added = False
+        pos_added, post = False, None
         if self.fused_vit:
             w_patch, b_patch = self.vis_dense["patch"]
             rows = b * x.shape[1]
@@ -310,8 +323,8 @@ class SmolVLAModel:
                 if i + 1 < v.num_hidden_layers:
                     nx = f"{VIS}encoder.layers.{i + 1}."
                     x, h = tk.add_layer_norm(x, m, p[nx + "layer_norm1.weight"], p[nx + "layer_norm1.bias"], v.layer_norm_eps)
-                else:
-                    x = x + m
+                else:  # the last residual add in the launch of the tower's closing LayerNorm
+                    post = tk.add_layer_norm(x, m, p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], v.layer_norm_eps)[1]
                 continue
             h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], v.layer_norm_eps)
             q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
@@ -322,9 +335,16 @@ class SmolVLAModel:
             x = x + self.lin(lp + "self_attn.out_proj", a)
             h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm2.weight"], p[lp + "layer_norm2.bias"], v.layer_norm_eps)
             x = x + self.lin(lp + "mlp.fc2", F.gelu(self.lin(lp + "mlp.fc1", h), approximate="tanh"))
-        x = F.layer_norm(x, (v.hidden_size,), p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], v.layer_norm_eps)
+        if post is not None:
+            x = post
+        else:
+            x = F.layer_norm(x, (v.hidden_size,), p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], v.layer_norm_eps)
         s = cfg.scale_factor
         seq, dim = x.shape[1], x.shape[2]
+        if self.fused_vit and seq == self.shuffle_perm.shape[0]:
+            # the pixel shuffle moves whole token rows: one gather by a token permutation built with the model
+            x = torch.index_select(x, 1, self.shuffle_perm).reshape(b, seq // (s * s), dim * s * s)
+            return self._dense("connector", x)
         side = int(seq**0.5)
         x = x.view(b, side, side, dim).view(b, side, side // s, dim * s).permute(0, 2, 1, 3)
         x = x.reshape(b, side // s, side // s, dim * s * s).permute(0, 2, 1, 3).reshape(b, seq // (s * s), dim * s * s)
@@ -346,8 +366,10 @@ class SmolVLAModel:
         ``image_range01``: the images are still in [0, 1] (``x * 2 - 1`` is applied here, in the patch launch where
         that is possible)."""
         embs, pads = [], []
+        stacked = None  # the embeddings of all cameras as one [cameras, tokens, hidden] tensor, when they are batch-1 images
         if image_range01 and self._patch_rows_ok(images):
-            per_image = (self.embed_image(None, images01=list(images)) * self.img_scale).split(1, dim=0)
+            stacked = self.embed_image(None, images01=list(images)) * self.img_scale
+            per_image = stacked.split(1, dim=0)
             images = ()
         elif image_range01:
             images = [img * 2.0 - 1.0 for img in images]
@@ -356,7 +378,9 @@ class SmolVLAModel:
         elif len(images) > 1 and all(img.shape == images[0].shape for img in images):
             # one pass of the vision tower over all cameras: rows are independent, and the tower's
             # GEMMs fill the device three times better than one 1024-patch image at a time
-            per_image = (self.embed_image(torch.cat(list(images), dim=0)) * self.img_scale).split(images[0].shape[0], dim=0)
+            per_all = self.embed_image(torch.cat(list(images), dim=0)) * self.img_scale
+            per_image = per_all.split(images[0].shape[0], dim=0)
+            stacked = per_all if images[0].shape[0] == 1 else None
         else:
             per_image = [self.embed_image(img) * self.img_scale for img in images]
         for e, m in zip(per_image, img_masks):
@@ -367,6 +391,18 @@ class SmolVLAModel:
         embs.append(lang)
         pads.append(lang_masks)
         st = self.lin("state_proj", state)[:, None, :]
+        p_len = sum(e.shape[1] for e in embs) + 1
+        if stacked is not None and lang.shape[0] == 1 and st.shape[0] == 1 and p_len in self._att_const:
+            # the three pieces written (and cast) straight into the prefix buffer, the attention-block flags taken from
+            # the constants built with the model: 4 launches where concatenation, casts and fills took 10
+            n_img = stacked.shape[0] * stacked.shape[1]
+            dt = torch.promote_types(torch.promote_types(stacked.dtype, lang.dtype), st.dtype)
+            out = torch.empty(1, p_len, st.shape[-1], dtype=dt, device=self.device)
+            out[0, :n_img].copy_(stacked.reshape(n_img, -1))
+            out[0, n_img : p_len - 1].copy_(lang[0])
+            out[0, p_len - 1].copy_(st[0, 0])
+            pads.append(self._true11)
+            return out, torch.cat(pads, dim=1), self._att_const[p_len]
         embs.append(st)
         pads.append(torch.ones(st.shape[0], 1, dtype=torch.bool, device=self.device))
         embs = torch.cat(embs, dim=1)
