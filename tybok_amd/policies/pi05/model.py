@@ -576,6 +576,9 @@ class PI05Model:
             if self.vt_suf is None or self.vt_suf.shape[2] < (s + 31) // 32 * 32:
                 self.vt_suf = torch.zeros(kv[0][0].shape[1], self.head_dim, (s + 31) // 32 * 32, dtype=BF16, device=self.device)
             pos32 = tk.prefix_meta(pads[0].contiguous(), None, _ROPE_POSITIONS, s, want_mask=False)[2]  # clamp(sum(pad) + arange(s))
+            # (`action_in_proj` stays the library's fp32 product + cast, two launches a step: carried in the tail launch
+            # of the step before -- tk_expert_tail_embed -- it sums its 32 terms in another order, and that re-draw of
+            # a few bf16 roundings moved one frame's maximum error from under to over the cap held for this path)
             for step in range(self.num_steps):
                 hidden = self.lin("action_in_proj", x_t)[0].to(BF16)
                 hidden = self._denoise_layers_fused(pads, caches, hidden, pos32, step)
