@@ -231,10 +231,11 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
     const int nbn = (a.ntiles * 32 + tk_wide_cols() - 1) / tk_wide_cols();
     int ks = split_k;
     if (ks <= 0 && a.mtiles == 4 && !a.s1 && a.N % 4 == 0 && ws && a.KT >= 32) {
-      // Few column blocks over a long K (the down projection): 64- or 128-row blocks and the split count by a
-      // two-term cost fitted to M = 296 .. 968 at K = 16384, N = 2048 -- the k loop of the blocks that share a CU
-      // (0.1 us per 1000 row x k products) and the partials' trip through memory (0.5 us per MB).  At 296 rows
-      // 64-row blocks x 6 splits take 31.8 us where 128-row blocks x 10 take 36.2; from 712 rows on 128 x 5 / x 4.
+      // Few column blocks over a long K (the down projection): 64- or 128-row blocks and the split count by a cost
+      // fitted to M = 296 .. 968 at K = 16384, N = 2048 -- the k loop of the blocks that share a CU (0.1 us per 1000
+      // row x k products), the partials' trip through memory (0.5 us per MB), the weights pulled once per row block
+      // (0.005 us per MB) and 8 us that a grid of lone four-wave 64-row blocks loses to 128-row ones.  At 296 rows
+      // 64-row blocks x 6 splits take 31.8 us where 128-row blocks x 10 take 36.2; from 552 rows on 128-row blocks.
       double best = 1e30;
       for (int mt = 2; mt <= 4; mt += 2)
         for (int sp = 1; sp <= 16 && sp <= a.KT / 16; ++sp) {
@@ -242,7 +243,8 @@ int gemm_common(const void* x, int ldx, const void* w_packed, const float* s0, c
           const int gens = (nbn * nbm * sp + cus - 1) / cus;
           const double loop = 1e-4 * gens * (mt * 32) * ((double)K / sp);
           const double part = sp > 1 ? 0.5e-6 * 4.0 * sp * nbm * (mt * 32) * nbn * tk_wide_cols() : 0.0;
-          if (loop + part < best) best = loop + part, a.mtiles = mt, ks = sp;
+          const double cost = loop + part + (mt == 2 ? 8.0 : 0.0) + 0.005e-6 * nbm * (double)K * nbn * tk_wide_cols();
+          if (cost < best) best = cost, a.mtiles = mt, ks = sp;
         }
     }
     const int brows = a.mtiles * 32;
