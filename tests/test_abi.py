@@ -96,6 +96,8 @@ def _cases():
         dict(x=P, ldx=2048, w=P, scale=P, y=P, ldy=16384, resid=None, ldr=0, rdt=0, gate=None, M=50, N=16384, K=2048, split=0, st=None), kw
     )
     sread = lambda **kw: _args(dict(src=P, bytes=1 << 25, blocks=256, sink=P, st=None), kw)  # noqa: E731
+    meta = lambda **kw: _args(dict(pad=P, att=None, P=241, pp=256, pos=16384, S=50, mask=P, p32=P, suf=P, st=None), kw)  # noqa: E731
+    patch = lambda **kw: _args(dict(i0=P, i1=P, i2=P, i3=None, n=3, H=512, W=512, ps=16, scale=2.0, shift=-1.0, out=P, st=None), kw)  # noqa: E731
     return [
         ("tk_quant_act_rows", qa(K=2044), -1, "multiple of 8"),
         ("tk_quant_act_rows", qa(K=32768, ldx=32768, lda=32768), -1, "at most"),
@@ -162,6 +164,18 @@ def _cases():
         ("tk_batched_transpose_v", tv(D=128), -1, "head_dim"),
         ("tk_batched_transpose_v", tv(keys=1000), -1, "rounded up to 32"),
         ("tk_batched_transpose_v", tv(sl=2300), -1, "multiples of 8"),
+        ("tk_prefix_meta", meta(P=0), -1, "P=0"),
+        ("tk_prefix_meta", meta(P=4096, pp=4096), -1, "P=4096"),
+        ("tk_prefix_meta", meta(pad=None), -1, "null pad flags"),
+        ("tk_prefix_meta", meta(S=50, suf=None), -1, "S without an output"),
+        ("tk_prefix_meta", meta(pp=240), -1, "p_pad=240"),
+        ("tk_prefix_meta", meta(pp=250), -1, "multiple of 16"),
+        ("tk_prefix_meta", meta(mask=P + 4), -1, "16-byte aligned"),
+        ("tk_patchify_images", patch(n=5), -1, "n=5"),
+        ("tk_patchify_images", patch(ps=12), -1, "patch=12"),
+        ("tk_patchify_images", patch(H=500), -1, "divides"),
+        ("tk_patchify_images", patch(i1=None), -1, "image 1 is null"),
+        ("tk_patchify_images", patch(out=P + 8), -1, "output must be 16-byte aligned"),
     ]
 
 
