@@ -1016,7 +1016,7 @@ static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb,
   if (batch > 0 && !split && S == 0 && !mask2d && !pad && (D == 64 || D == 96) && P >= 128 && M >= 128) {
     // vision towers: many query tiles over a long key range -- K / V^T staged through LDS once per 128 queries
     a.gqa_mul = (65536 + H / G - 1) / (H / G);
-    int rc = tk_launch_tower_attn(a, D, (hipStream_t)stream);
+    int rc = tk_launch_tower_attn(a, D, device_cus(), (hipStream_t)stream);
     if (rc) return fail(TK_ELAUNCH, "attn: launch failed (%s)", hipGetErrorString(hipGetLastError()));
     return TK_OK;
   }

@@ -285,7 +285,7 @@ struct TransposeVArgs {
 };
 int tk_launch_transpose_v(TransposeVArgs a, int D, hipStream_t st);
 // vision-tower self-attention (batched, unmasked, prefix-only, head size 64 / 96): 128 queries per block
-int tk_launch_tower_attn(AttnArgs a, int D, hipStream_t st);
+int tk_launch_tower_attn(AttnArgs a, int D, int cus, hipStream_t st);  // cus: compute units of the device (block shape by grid fill)
 int tk_attn_waves(int D, int split_planes, int ntiles);
 int tk_launch_attn(AttnArgs a, int D, int waves, hipStream_t st);
 // 256-wide heads: blocks of 8 waves that walk their share of the key tiles 8 at a time (a.kv_splits blocks per query tile)

@@ -20,11 +20,12 @@
 
 namespace {
 
-constexpr int kQTiles = 4;   // query tiles (waves) per key-half group
 constexpr int kGroups = 2;   // key halves
-constexpr int kWaves = kQTiles * kGroups;
-constexpr int kGroupThreads = kQTiles * 64;
 constexpr int kStageKeys = 64;
+// QT: query tiles (waves) per key-half group.  4: 128 queries a block, two blocks per CU.  5: 160 queries a block of
+// ten waves, one block per CU (three waves on two of the SIMDs) -- for grids that four-tile blocks would spread as
+// "one block on most CUs, two on some": the doubly loaded CUs then run four waves per SIMD and set the launch's
+// duration (3 cameras x 12 heads x 1024 queries: 288 blocks on 256 CUs; 252 blocks of five tiles fit one per CU).
 
 // S^T rows are dealt to keys so that accumulator register i of lane half `hf` holds key
 // 16*(i/8) + 8*hf + i%8 of the tile: registers 8s..8s+7 are then the B operand of k step s.
@@ -63,7 +64,7 @@ __device__ __forceinline__ void stage_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-template <int D>
+template <int D, int QT>
 struct TowerLds {
   static constexpr int KP = D * 2 + 16;             // pitch of a K row (bytes): rows 16 apart share banks, nothing closer
   static constexpr int VP = kStageKeys * 2 + 16;    // pitch of a V^T row
@@ -71,37 +72,47 @@ struct TowerLds {
   static constexpr int GROUP = 2 * (KBYTES + VBYTES);  // a group's double buffer; later its merge record
   static constexpr int TOTAL = kGroups * GROUP;
   static constexpr int MERGE_WAVE = (2 + (D / 32) * 16) * 64 * 4;  // m, l and O^T of one wave
-  static_assert(kQTiles * MERGE_WAVE <= GROUP, "the merge record must fit the group's staging area");
+  // the merge record lies in the second group's staging area and, if it is longer, runs back into the first one's
+  // (every wave of the block is past its last staging read by then)
+  static constexpr int MERGE_OFF = QT * MERGE_WAVE <= GROUP ? GROUP : TOTAL - QT * MERGE_WAVE;
+  static_assert(QT * MERGE_WAVE <= TOTAL, "the merge record must fit the staging areas");
 };
 
 // LB: the logits are rounded to bf16 before the scale and the softmax (what a bf16 matmul hands to a
 // fp32 softmax); otherwise they stay fp32.
 // F16: q, K, V^T are fp16 and the probabilities are rounded to fp16 for P.V (both products on the fp16 matrix
 // instruction); the output stays bf16.
-template <int D, bool LB, bool F16>
-__global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kernel(AttnArgs a, int qblocks) {
-  using L = TowerLds<D>;
+// WPE: waves per SIMD the registers are budgeted for -- 4 lets two four-tile blocks of head size 64 share a CU (128
+// registers per lane, a few of them spilled); 2 / 3 when the grid puts one block on a CU anyway.
+template <int D, bool LB, bool F16, int QT, int WPE>
+__global__ __launch_bounds__(QT * kGroups * 64, WPE) void tower_attn_kernel(AttnArgs a, int qblocks) {
+  using L = TowerLds<D, QT>;
+  constexpr int kQTiles = QT, kGroupThreads = QT * 64;
   constexpr int DS = D / 16;            // k steps of Q.K^T
   constexpr int DT = D / 32;            // 32-row tiles of O^T
   constexpr int KT = kStageKeys / 32;   // key tiles per stage
   constexpr int KP = L::KP, VP = L::VP, KBYTES = L::KBYTES, VBYTES = L::VBYTES;
   constexpr int KCH = D / 8;            // 16-byte chunks per K row
-  constexpr int NLD = kStageKeys * KCH / kGroupThreads;  // 16-byte chunks per thread and stage, K and V^T alike
-  static_assert(kStageKeys * KCH % kGroupThreads == 0, "a stage must divide evenly over the group's threads");
+  constexpr int NCHUNK = kStageKeys * KCH;                              // 16-byte chunks of a stage, K and V^T alike
+  constexpr int NLD = (NCHUNK + kGroupThreads - 1) / kGroupThreads;     // per thread and stage
+  constexpr bool EVEN = NCHUNK % kGroupThreads == 0;                    // (five tiles: the last pass is partly empty)
   extern __shared__ __align__(16) unsigned char lds_all[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, l32 = lane & 31, half = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave / kQTiles, qt = wave % kQTiles;
-  const int gtid = tid & (kGroupThreads - 1);
+  const int gtid = (kGroupThreads & (kGroupThreads - 1)) == 0 ? (tid & (kGroupThreads - 1)) : tid - grp * kGroupThreads;
   unsigned char* lds = lds_all + grp * L::GROUP;
-  // 1-D grid dealt round-robin to the 8 XCDs: every query block of one (problem, head) pair goes to
-  // the same XCD, whose L2 then holds that pair's K / V^T for all of them
+  // 1-D grid dealt round-robin to the 8 XCDs: XCD x takes the x-th eighth of the (pair, query block) list in pair-major
+  // order, so the query blocks of one (problem, head) pair run on one XCD (two where the pair straddles a boundary),
+  // whose L2 then holds that pair's K / V^T for all of them, and every XCD gets the same number of blocks
+  const int total = a.batch * a.H * qblocks, per_xcd = (total + 7) / 8;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int pair = (slot / qblocks) * 8 + xcd;
-  if (pair >= a.batch * a.H) return;
-  const int qb = slot % qblocks;
+  const int item = xcd * per_xcd + slot;
+  if (slot >= per_xcd || item >= total) return;
+  const int pair = item / qblocks;
+  const int qb = item % qblocks;
   const int bi = pair / a.H, h = pair % a.H;
   const int g = (h * a.gqa_mul) >> 16;
   const u16* qp = a.q + (long long)bi * a.q_sb + (size_t)h * a.q_sh;
@@ -124,7 +135,8 @@ __global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kerne
   auto gload = [&](int s) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      const int c = gtid + i * kGroupThreads;
+      int c = gtid + i * kGroupThreads;
+      if (!EVEN && c > NCHUNK - 1) c = NCHUNK - 1;  // loaded again, not stored
       int key = s * kStageKeys + c / KCH;
       if (key > a.P - 1) key = a.P - 1;  // rows past the end are masked below; keep the address valid
       kreg[i] = *(const i32x4*)(kp + (size_t)key * a.pre_sl + (c % KCH) * 8);
@@ -141,6 +153,7 @@ __global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kerne
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int c = gtid + i * kGroupThreads;
+      if (!EVEN && c >= NCHUNK) continue;
       *(i32x4*)(kb + (c / KCH) * KP + (c % KCH) * 16) = kreg[i];
       *(i32x4*)(vb + (c / 8) * VP + (c % 8) * 16) = vreg[i];
     }
@@ -255,7 +268,7 @@ __global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kerne
 
   // ---- merge the two key halves of each query tile: the second group hands (m, l, O^T) over through
   //      its staging area (all of its waves are past their last read of it: the barrier above) ----
-  float* rec = (float*)(lds_all + L::GROUP + qt * L::MERGE_WAVE);
+  float* rec = (float*)(lds_all + L::MERGE_OFF + qt * L::MERGE_WAVE);
   if (grp == 1) {
     rec[lane] = m_run;
     rec[64 + lane] = l_run;
@@ -285,21 +298,37 @@ __global__ __launch_bounds__(kWaves * 64, D == 64 ? 4 : 2) void tower_attn_kerne
   }
 }
 
-template <int D, bool LB, bool F16 = false>
-int launch_tower(const AttnArgs& a, hipStream_t st) {
+template <int D, bool LB, bool F16, int QT, int WPE>
+int launch_tower_qt(const AttnArgs& a, hipStream_t st) {
   // more LDS than a launch gets by default: raise the kernel's limit once per process
   static int raised = 0;
+  constexpr int lds_bytes = TowerLds<D, QT>::TOTAL;
   if (!raised) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&tower_attn_kernel<D, LB, F16>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            TowerLds<D>::TOTAL) != hipSuccess)
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&tower_attn_kernel<D, LB, F16, QT, WPE>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            lds_bytes) != hipSuccess)
       return -3;
     raised = 1;
   }
-  const int qblocks = (a.M + kQTiles * 32 - 1) / (kQTiles * 32);
+  const int qblocks = (a.M + QT * 32 - 1) / (QT * 32);
   const int pairs = a.batch * a.H;
-  dim3 grid(8 * ((pairs + 7) / 8) * qblocks);
-  hipLaunchKernelGGL((tower_attn_kernel<D, LB, F16>), grid, dim3(kWaves * 64), TowerLds<D>::TOTAL, st, a, qblocks);
+  dim3 grid(8 * ((pairs * qblocks + 7) / 8));
+  hipLaunchKernelGGL((tower_attn_kernel<D, LB, F16, QT, WPE>), grid, dim3(QT * kGroups * 64), lds_bytes, st, a, qblocks);
   return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+template <int D, bool LB, bool F16 = false>
+int launch_tower(const AttnArgs& a, hipStream_t st, int cus) {
+  if constexpr (D == 64 && !F16) {
+    // one block per CU where the grid allows it: four-tile blocks with the whole register file to themselves, or
+    // five-tile blocks where four-tile ones would double up on some CUs (see QT above); else two blocks per CU
+    const int pairs = a.batch * a.H, tiles = (a.M + 31) / 32;
+    const int b4 = pairs * ((tiles + 3) / 4), b5 = pairs * ((tiles + 4) / 5);
+    if (b4 <= cus) return launch_tower_qt<D, LB, F16, 4, 2>(a, st);
+    if (b4 < 2 * cus && b5 <= cus) return launch_tower_qt<D, LB, F16, 5, 3>(a, st);
+    return launch_tower_qt<D, LB, F16, 4, 4>(a, st);
+  } else {
+    return launch_tower_qt<D, LB, F16, 4, 2>(a, st);
+  }
 }
 
 // V [B, P, G, D] (d contiguous) -> V^T [B, G, D, ld] (keys contiguous), zero filled from P up to the end
@@ -357,10 +386,10 @@ int tk_launch_transpose_v(TransposeVArgs a, int D, hipStream_t st) {
 // Shapes this kernel is built for (checked by the caller): batched, unmasked, prefix-only, bf16 K / V^T,
 // head size 64 or 96, at least 128 keys (two stages), strides and alignment as for the expert attention
 // kernel.
-int tk_launch_tower_attn(AttnArgs a, int D, hipStream_t st) {
+int tk_launch_tower_attn(AttnArgs a, int D, int cus, hipStream_t st) {
   if (a.P <= kStageKeys) return -1;
-  if (a.f16) return D == 96 && !a.logits_bf16 ? launch_tower<96, false, true>(a, st) : -1;  // (pi0.5's tower)
-  if (D == 64) return a.logits_bf16 ? launch_tower<64, true>(a, st) : launch_tower<64, false>(a, st);
-  if (D == 96) return a.logits_bf16 ? launch_tower<96, true>(a, st) : launch_tower<96, false>(a, st);
+  if (a.f16) return D == 96 && !a.logits_bf16 ? launch_tower<96, false, true>(a, st, cus) : -1;  // (pi0.5's tower)
+  if (D == 64) return a.logits_bf16 ? launch_tower<64, true>(a, st, cus) : launch_tower<64, false>(a, st, cus);
+  if (D == 96) return a.logits_bf16 ? launch_tower<96, true>(a, st, cus) : launch_tower<96, false>(a, st, cus);
   return -1;
 }
