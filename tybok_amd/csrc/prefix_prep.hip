@@ -23,17 +23,28 @@ __global__ __launch_bounds__(256) void prefix_meta_kernel(PrefixMetaArgs a) {
   __shared__ int wave_tot[2][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // inclusive scans of both flag rows: 8 consecutive tokens per thread, wave scan of the thread sums, wave offsets
+  // (all sixteen byte loads of a thread are unconditional -- clamped index -- so that they are in flight together:
+  // behind a range check each of them waited for the one before, 16 round trips to memory in a row)
+  unsigned char rp[8], ra[8];
+  const unsigned char* att_or_pad = a.att ? a.att : a.pad;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    int j = tid * 8 + e;
+    if (j > a.P - 1) j = a.P - 1;
+    rp[e] = a.pad[j];
+    ra[e] = att_or_pad[j];
+  }
   int la[8], lp[8], sa = 0, sp = 0;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const int j = tid * 8 + e;
-    const int pv = j < a.P ? (a.pad[j] != 0) : 0;
-    const int av = (j < a.P && a.att) ? (a.att[j] != 0) : 0;
+    const int pv = j < a.P ? (rp[e] != 0) : 0;
+    const int av = (j < a.P && a.att) ? (ra[e] != 0) : 0;
     sa += av;
     sp += pv;
     la[e] = sa;
     lp[e] = sp;
-    if (j < kMaxP) s_pad[j] = (unsigned char)pv;
+    s_pad[j] = (unsigned char)pv;
   }
   int xa = sa, xp = sp;
 #pragma unroll
@@ -68,19 +79,23 @@ __global__ __launch_bounds__(256) void prefix_meta_kernel(PrefixMetaArgs a) {
     }
   }
   if (!a.mask2d) return;
-  // rows blockIdx.x, + gridDim.x, ..: 16 bytes of a row per thread and pass
+  // rows blockIdx.x, + gridDim.x, ..: a thread owns 16 columns of every row (p_pad <= 2048: one pass) and keeps their
+  // flags and block counts in registers, so a row costs two broadcast LDS reads and one 16-byte store
+  const int j0 = tid * 16;
+  if (j0 >= a.p_pad) return;
+  unsigned short cj[16];
+  unsigned char pj[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    pj[e] = s_pad[j0 + e];  // zero from P on
+    cj[e] = c_att[j0 + e];
+  }
   for (int i = blockIdx.x; i < a.P; i += gridDim.x) {
     const int ci = c_att[i], pi = s_pad[i];
-    unsigned char* row = a.mask2d + (size_t)i * a.p_pad;
-    for (int j0 = tid * 16; j0 < a.p_pad; j0 += 256 * 16) {
-      union { i32x4 v; unsigned char b[16]; } o;
+    union { i32x4 v; unsigned char b[16]; } o;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int j = j0 + e;
-        o.b[e] = (j < a.P && pi && s_pad[j] && (int)c_att[j] <= ci) ? 1 : 0;
-      }
-      *(i32x4*)(row + j0) = o.v;
-    }
+    for (int e = 0; e < 16; ++e) o.b[e] = (unsigned char)(pi & pj[e] & ((int)cj[e] <= ci ? 1 : 0));
+    *(i32x4*)(a.mask2d + (size_t)i * a.p_pad + j0) = o.v;
   }
 }
 
