@@ -16,6 +16,9 @@
 //     gated launch that is split keeps the one-launch form: the last-arriving block sums.  Measured at
 //     M=712, K=16384, N=2048, 5 splits: 74 -> 52 + 7.7 us; one block per output tile -- 48 of 256 CUs -- pulling
 //     31 MB of partials through 8-byte coherent loads, split after split, was a fifth of the launch.)
+//   * where the grid would fill the device twice over (the gated 2048 -> 2 x 16384 launch) a block is EIGHT waves on
+//     192 or 256 rows with the weights staged through LDS too (fp8w_tile_kernel below): half the bytes per matrix
+//     instruction through the L2, the same accumulators, partials and epilogue, the same bits.
 // The epilogues compute exactly what the skinny kernel's do (same rounding points).
 #include "tk_common.h"
 #include "tk_kernels.h"
