@@ -58,8 +58,9 @@ struct GemmArgs {
   // bf16-weight many-row kernel only: bf16 [N] bias added to the accumulator, or nullptr; there act is
   // 0 none, 1 tanh-GELU of the bf16-rounded pre-activation, 2 tanh-GELU of the fp32 pre-activation
   const unsigned short* bias;
-  // many-row fp8 kernels: 32-row tiles per block (2 or 4), chosen by the host
-  int mtiles;  // many-row kernels: 32-row tiles per block (2 / 4: four-wave blocks; 6 / 8: eight-wave blocks, fp8 weights only)
+  // many-row fp8 kernels: 32-row tiles per block, chosen by the host (2 / 4: four-wave blocks; 6 / 8: eight-wave
+  // blocks with both operands through LDS, weight-only kernel)
+  int mtiles;
   // many-row 16-bit-weight kernel only: activations, weights, bias, output and a 16-bit residual are fp16, not bf16
   int f16;
   // single-launch gated FFN only: the hand-off words in the workspace (TK_FUSE_* below), the down blocks per row
