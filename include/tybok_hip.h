@@ -366,6 +366,14 @@ int tk_expert_attn(const void* q, int q_sm, int q_sh, const void* k_pre, const v
 int tk_expert_kv_project(const void* k, const void* v, int sl, int P, int KV, const void* wk, const void* wv, int N,
                          void* k_hi, void* k_lo, void* vt_hi, void* vt_lo, int vt_ld, void* stream);
 
+/* tk_expert_kv_project for several cross layers in one launch (the projections are independent; each of them alone
+ * leaves 96 of 256 compute units idle and pays a launch of its own):
+ *   k, v, wk, wv: host arrays of `layers` device pointers (1..16), shapes and strides as above, the same for every layer;
+ *   k_hi / k_lo: [layers][P, N]; vt_hi / vt_lo: [layers][N, vt_ld].  Same bits as `layers` single calls. */
+int tk_expert_kv_project_layers(int layers, const void* const* k, const void* const* v, int sl, int P, int KV,
+                                const void* const* wk, const void* const* wv, int N, void* k_hi, void* k_lo, void* vt_hi,
+                                void* vt_lo, int vt_ld, void* stream);
+
 /* Cross-attention layer of the action expert with the query projection inside the attention launch:
  *   q = rope(bf16(RMSNorm(x) . Wq^T)) per head (bf16(w * bf16(x * rstd)) norm, fp32 half-split rotary
  *   embedding with table rows rope_pos[m]), then attention over the fp32 (hi + lo planes) expert

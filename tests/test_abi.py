@@ -171,6 +171,9 @@ def _cases():
         ("tk_prefix_meta", meta(pp=240), -1, "p_pad=240"),
         ("tk_prefix_meta", meta(pp=250), -1, "multiple of 16"),
         ("tk_prefix_meta", meta(mask=P + 4), -1, "16-byte aligned"),
+        ("tk_expert_kv_project_layers", (17, P, P, 960, 241, 320, P, P, 320, P, P, P, P, 256, None), -1, "17 layers"),
+        ("tk_expert_kv_project_layers", (8, P, P, 960, 241, 320, P, P, 300, P, P, P, P, 256, None), -1, "bad shape"),
+        ("tk_expert_kv_project_layers", (8, P, P, 960, 241, 320, P, P, 320, P, P, P, P, 224, None), -1, "rounded up to 32"),
         ("tk_patchify_images", patch(n=5), -1, "n=5"),
         ("tk_patchify_images", patch(ps=12), -1, "patch=12"),
         ("tk_patchify_images", patch(H=500), -1, "divides"),

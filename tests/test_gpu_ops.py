@@ -306,6 +306,25 @@ def test_batched_attention_padded_head_with_explicit_scale(tk):
     _close(got[..., :hd], want, "padded-head batched attention")
 
 
+@pytest.mark.parametrize("layers,p,kv,n", [(8, 241, 320, 320), (16, 177, 320, 320), (3, 33, 208, 64), (1, 40, 96, 128)])
+def test_kv_projection_of_several_layers_in_one_launch_gives_the_single_launches_bits(tk, layers, p, kv, n):
+    # the cross layers' projections are independent: one launch over all of them must write, layer by layer, the
+    # planes that one launch per layer writes (inputs strided like the per-layer q|k|v rows of the prefill)
+    g = torch.Generator().manual_seed(43)
+    wide = torch.randn(layers, p, 4 * kv, generator=g).to(torch.bfloat16).cuda()
+    ks, vs = [wide[i, :, 2 * kv : 3 * kv] for i in range(layers)], [wide[i, :, 3 * kv :] for i in range(layers)]
+    wks = [(torch.randn(n, kv, generator=g) * kv**-0.5).cuda() for _ in range(layers)]
+    wvs = [(torch.randn(n, kv, generator=g) * kv**-0.5).cuda() for _ in range(layers)]
+    got = tk.project_prefix_kv_layers(ks, vs, wks, wvs, 64)
+    assert len(got) == layers
+    for i in range(layers):
+        one = tk.project_prefix_kv(ks[i], vs[i], wks[i], wvs[i], 64)
+        for name in ("k", "k_lo", "vt", "vt_lo"):
+            assert torch.equal(getattr(got[i], name), getattr(one, name)), (i, name)
+    with pytest.raises(ValueError):
+        tk.project_prefix_kv_layers(ks * 17, vs * 17, wks * 17, wvs * 17, 64)
+
+
 @pytest.mark.parametrize("p,kv,n,d", [(241, 320, 320, 64), (177, 320, 320, 64), (40, 96, 128, 64), (33, 208, 64, 64)])
 def test_expert_kv_projection_into_attention_planes(tk, p, kv, n, d):
     # float(K) @ Wk^T / float(V) @ Wv^T in fp32, delivered as the attention kernel's hi + lo planes:

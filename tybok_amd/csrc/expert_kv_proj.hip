@@ -30,11 +30,12 @@ __global__ __launch_bounds__(256) void expert_kv_proj_kernel(KvProjArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int half = lane >> 5, l32 = lane & 31;
   const int nt = blockIdx.y;  // 32-column tile of the output
-  const bool is_v = blockIdx.z != 0;
+  const bool is_v = (blockIdx.z & 1) != 0;
+  const int layer = blockIdx.z >> 1;  // (several layers' projections in one launch: independent problems)
   int p = blockIdx.x * 32 + l32;
   const int pc = p < a.P ? p : a.P - 1;  // rows past P: valid data, zeroed / skipped below
-  const u16* xrow = (is_v ? a.v : a.k) + (size_t)pc * a.sl + 8 * half;
-  const float* wrow = (is_v ? a.wv : a.wk) + (size_t)(nt * 32 + l32) * a.KV + 8 * half;
+  const u16* xrow = (is_v ? a.v[layer] : a.k[layer]) + (size_t)pc * a.sl + 8 * half;
+  const float* wrow = (is_v ? a.wv[layer] : a.wk[layer]) + (size_t)(nt * 32 + l32) * a.KV + 8 * half;
 
   f32x16 acc;
 #pragma unroll
@@ -78,15 +79,17 @@ __global__ __launch_bounds__(256) void expert_kv_proj_kernel(KvProjArgs a) {
     const i32x2 lo = pack_bf16x4(v - unpack_bf16x4(hi));
     if (!is_v) {
       if (p < a.P) {
-        *(i32x2*)(a.k_hi + (size_t)p * a.N + n) = hi;
-        *(i32x2*)(a.k_lo + (size_t)p * a.N + n) = lo;
+        const size_t o = ((size_t)layer * a.P + p) * a.N + n;
+        *(i32x2*)(a.k_hi + o) = hi;
+        *(i32x2*)(a.k_lo + o) = lo;
       }
     } else if (p < a.ld) {
       // V^T rows are output columns, keys contiguous: the 32 lanes of a half write 64 contiguous bytes
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        a.vt_hi[(size_t)(n + j) * a.ld + p] = (u16)(((unsigned)hi[j >> 1]) >> (16 * (j & 1)));
-        a.vt_lo[(size_t)(n + j) * a.ld + p] = (u16)(((unsigned)lo[j >> 1]) >> (16 * (j & 1)));
+        const size_t o = ((size_t)layer * a.N + n + j) * a.ld + p;
+        a.vt_hi[o] = (u16)(((unsigned)hi[j >> 1]) >> (16 * (j & 1)));
+        a.vt_lo[o] = (u16)(((unsigned)lo[j >> 1]) >> (16 * (j & 1)));
       }
     }
   }
@@ -95,7 +98,7 @@ __global__ __launch_bounds__(256) void expert_kv_proj_kernel(KvProjArgs a) {
 }  // namespace
 
 int tk_launch_kv_proj(KvProjArgs a, hipStream_t st) {
-  dim3 grid((a.P + 31) / 32, a.N / 32, 2);
+  dim3 grid((a.P + 31) / 32, a.N / 32, 2 * a.L);
   hipLaunchKernelGGL(expert_kv_proj_kernel, grid, dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }

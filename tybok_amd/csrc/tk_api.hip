@@ -916,21 +916,27 @@ int tk_attn_prepare_kv(const void* k, const void* v, int kv_dtype, int sl, int s
   return TK_OK;
 }
 
-int tk_expert_kv_project(const void* k, const void* v, int sl, int P, int KV, const void* wk, const void* wv, int N,
-                         void* k_hi, void* k_lo, void* vt_hi, void* vt_lo, int vt_ld, void* stream) {
+static int kv_project_impl(int L, const void* const* k, const void* const* v, int sl, int P, int KV, const void* const* wk,
+                           const void* const* wv, int N, void* k_hi, void* k_lo, void* vt_hi, void* vt_lo, int vt_ld, void* stream) {
+  if (L < 1 || L > kKvProjMaxLayers) return fail(TK_EINVAL, "kv_project: %d layers in one launch (1..%d)", L, kKvProjMaxLayers);
   if (P <= 0 || KV <= 0 || N <= 0 || N % 32 || KV % 16)
     return fail(TK_EINVAL, "kv_project: bad shape P=%d KV=%d N=%d (N a multiple of 32, KV of 16)", P, KV, N);
   if (!k || !v || !wk || !wv || !k_hi || !k_lo || !vt_hi || !vt_lo) return fail(TK_EINVAL, "kv_project: null pointer");
   if (sl < KV || sl % 8) return fail(TK_EINVAL, "kv_project: row stride %d must be >= KV=%d and a multiple of 8", sl, KV);
-  if (!aligned16(k) || !aligned16(v) || !aligned16(wk) || !aligned16(wv)) return fail(TK_EINVAL, "kv_project: inputs must be 16-byte aligned");
   if (vt_ld < ((P + 31) / 32) * 32) return fail(TK_EINVAL, "kv_project: vt_ld=%d must hold P rounded up to 32", vt_ld);
   if (!aligned8(k_hi) || !aligned8(k_lo)) return fail(TK_EINVAL, "kv_project: K planes must be 8-byte aligned");
   KvProjArgs a;
-  a.k = (const u16*)k;
-  a.v = (const u16*)v;
+  memset(&a, 0, sizeof(a));
+  a.L = L;
+  for (int l = 0; l < L; ++l) {
+    if (!k[l] || !v[l] || !wk[l] || !wv[l]) return fail(TK_EINVAL, "kv_project: null pointer (layer %d)", l);
+    if (!aligned16(k[l]) || !aligned16(v[l]) || !aligned16(wk[l]) || !aligned16(wv[l])) return fail(TK_EINVAL, "kv_project: inputs must be 16-byte aligned");
+    a.k[l] = (const u16*)k[l];
+    a.v[l] = (const u16*)v[l];
+    a.wk[l] = (const float*)wk[l];
+    a.wv[l] = (const float*)wv[l];
+  }
   a.sl = sl;
-  a.wk = (const float*)wk;
-  a.wv = (const float*)wv;
   a.P = P;
   a.KV = KV;
   a.N = N;
@@ -941,6 +947,17 @@ int tk_expert_kv_project(const void* k, const void* v, int sl, int P, int KV, co
   a.ld = vt_ld;
   if (tk_launch_kv_proj(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "kv_project: launch failed");
   return TK_OK;
+}
+
+int tk_expert_kv_project(const void* k, const void* v, int sl, int P, int KV, const void* wk, const void* wv, int N,
+                         void* k_hi, void* k_lo, void* vt_hi, void* vt_lo, int vt_ld, void* stream) {
+  return kv_project_impl(1, &k, &v, sl, P, KV, &wk, &wv, N, k_hi, k_lo, vt_hi, vt_lo, vt_ld, stream);
+}
+
+int tk_expert_kv_project_layers(int layers, const void* const* k, const void* const* v, int sl, int P, int KV, const void* const* wk,
+                                const void* const* wv, int N, void* k_hi, void* k_lo, void* vt_hi, void* vt_lo, int vt_ld,
+                                void* stream) {
+  return kv_project_impl(layers, k, v, sl, P, KV, wk, wv, N, k_hi, k_lo, vt_hi, vt_lo, vt_ld, stream);
 }
 
 static int attn_impl(int batch, long long q_sb, long long k_sb, long long vt_sb, long long out_sb, const void* q, int q_sm, int q_sh, const void* k_pre, const void* k_pre_lo, int pre_sl, int pre_sh,

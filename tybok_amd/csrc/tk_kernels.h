@@ -148,16 +148,18 @@ struct KvPrepArgs {
   int ld;
 };
 
+constexpr int kKvProjMaxLayers = 16;
 struct KvProjArgs {
-  const unsigned short* k;  // bf16 [P, KV] rows (element stride sl)
-  const unsigned short* v;
+  int L;                                        // layers in this launch (<= kKvProjMaxLayers)
+  const unsigned short* k[kKvProjMaxLayers];    // per layer: bf16 [P, KV] rows (element stride sl)
+  const unsigned short* v[kKvProjMaxLayers];
   int sl;
-  const float* wk;  // fp32 [N, KV]
-  const float* wv;
+  const float* wk[kKvProjMaxLayers];            // per layer: fp32 [N, KV]
+  const float* wv[kKvProjMaxLayers];
   int P, KV, N;
-  unsigned short* k_hi;  // [P, N]
+  unsigned short* k_hi;  // [L][P, N]
   unsigned short* k_lo;
-  unsigned short* vt_hi;  // [N, ld], ld >= P rounded up to 32
+  unsigned short* vt_hi;  // [L][N, ld], ld >= P rounded up to 32
   unsigned short* vt_lo;
   int ld;
 };

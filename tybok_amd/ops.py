@@ -638,6 +638,39 @@ def project_prefix_kv(k: torch.Tensor, v: torch.Tensor, wk: torch.Tensor, wv: to
     return PrefixKV(k_hi, vt_hi, k_lo, vt_lo)
 
 
+def project_prefix_kv_layers(ks, vs, wks, wvs, d: int) -> list[PrefixKV]:
+    """:func:`project_prefix_kv` for several layers (at most 16) in one launch: lists of per-layer ``k, v [P, KV]`` views
+    (one shape and row stride) and ``wk, wv [N, KV]`` fp32 weights -> one :class:`PrefixKV` per layer (views of stacked
+    planes).  Same bits as one call per layer."""
+    import ctypes
+
+    lib = native.lib()
+    bf = torch.bfloat16
+    n_layers = len(ks)
+    if not (1 <= n_layers <= 16) or not (len(vs) == len(wks) == len(wvs) == n_layers):
+        raise ValueError("project_prefix_kv_layers: 1..16 layers, four lists of the same length")
+    p, kv = ks[0].shape
+    n = wks[0].shape[0]
+    sl = ks[0].stride(0)
+    wks, wvs = [w.contiguous() for w in wks], [w.contiguous() for w in wvs]
+    for k, v, wk, wv in zip(ks, vs, wks, wvs):
+        if k.dtype != bf or v.dtype != bf or wk.dtype != torch.float32 or wv.dtype != torch.float32:
+            raise TypeError("project_prefix_kv_layers: k, v bf16 and wk, wv fp32")
+        if k.shape != (p, kv) or v.shape != (p, kv) or wk.shape != (n, kv) or wv.shape != (n, kv) or n % d or k.stride(1) != 1 or v.stride(1) != 1 or k.stride(0) != sl or v.stride(0) != sl:
+            raise ValueError("project_prefix_kv_layers: every layer k, v [P, KV] with one row stride; wk, wv [N, KV]; N a multiple of d")
+    g = n // d
+    opts = dict(dtype=bf, device=ks[0].device)
+    k_hi, k_lo = torch.empty(n_layers, p, g, d, **opts), torch.empty(n_layers, p, g, d, **opts)
+    vt_hi, vt_lo = torch.empty(n_layers, g, d, _pad32(p), **opts), torch.empty(n_layers, g, d, _pad32(p), **opts)
+    arr = ctypes.c_void_p * n_layers
+    rc = lib.tk_expert_kv_project_layers(
+        n_layers, arr(*(t.data_ptr() for t in ks)), arr(*(t.data_ptr() for t in vs)), sl, p, kv, arr(*(t.data_ptr() for t in wks)),
+        arr(*(t.data_ptr() for t in wvs)), n, k_hi.data_ptr(), k_lo.data_ptr(), vt_hi.data_ptr(), vt_lo.data_ptr(), vt_hi.shape[3], _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_expert_kv_project_layers")
+    return [PrefixKV(k_hi[i], vt_hi[i], k_lo[i], vt_lo[i]) for i in range(n_layers)]
+
+
 def expert_attn(
     q: torch.Tensor,
     prefix: PrefixKV | None,

@@ -533,10 +533,21 @@ class SmolVLAModel:
         (self layers, bf16 cache; ``vt`` when the prefill already produced it) or K and V^T split
         into bf16 hi + lo planes (cross layers, fp32)."""
         caches = []
+        crossed = {}
+        if ekv is None:  # projection and operand layout of every cross layer in one launch (16 layers at most each)
+            idx = [i for i in range(self.num_layers) if self.cfg.is_cross_layer(i)]
+            for c0 in range(0, len(idx), 16):
+                part = idx[c0 : c0 + 16]
+                lps = [f"{EXP}layers.{i}.self_attn." for i in part]
+                planes = tk.project_prefix_kv_layers(
+                    [keys[i, 0].flatten(1) for i in part], [values[i, 0].flatten(1) for i in part],
+                    [self.p[lp + "k_proj.weight"] for lp in lps], [self.p[lp + "v_proj.weight"] for lp in lps], self.head_dim,
+                )  # fmt: skip
+                crossed.update(zip(part, planes))
         for i in range(self.num_layers):
             if self.cfg.is_cross_layer(i):
-                if ekv is None:  # projection and operand layout in one launch
-                    caches.append(self._cross_cache(i, keys[i, 0], values[i, 0]))
+                if ekv is None:
+                    caches.append(crossed[i])
                     continue
                 ek, ev = ekv[i]
                 caches.append(tk.prepare_prefix_kv(ek[0], ev[0]))
