@@ -193,10 +193,17 @@ class ChunkRuntime:
         return torch.normal(0.0, 1.0, size=shape, dtype=torch.float32, device=self.device, generator=self._noise_gen, out=out)
 
     def _prepare_noise(self, noise: torch.Tensor | None) -> torch.Tensor | None:
-        """A caller's noise on the device in fp32, zero-padded to the model's action width."""
+        """A caller's noise on the device in fp32, at the caller's width (at most the model's action width):
+        :meth:`_pad_noise` widens it for the eager path, a recorded shape takes it as it is
+        (``StaticCall.store_leading``)."""
         if noise is None:
             return None
-        noise = noise.to(self.device, dtype=torch.float32)
+        if noise.shape[-1] > self.config.max_action_dim:
+            raise ValueError(f"noise has {noise.shape[-1]} action columns, the model {self.config.max_action_dim}")
+        return noise.to(self.device, dtype=torch.float32)
+
+    def _pad_noise(self, noise: torch.Tensor) -> torch.Tensor:
+        """Zero-padded to the model's action width."""
         missing = self.config.max_action_dim - noise.shape[-1]
         return torch.nn.functional.pad(noise, (0, missing)) if missing else noise
 

@@ -81,6 +81,7 @@ class StaticCall:
         """Copy a request's values into the static tensors of the same names (on the current stream)."""
         for name, value in values.items():
             slot = self.inputs[name]
+            getattr(self, "_stored_width", {}).pop(name, None)
             if isinstance(slot, (list, tuple)):
                 if len(value) != len(slot):
                     raise ValueError(f"{name}: {len(value)} tensors for {len(slot)} static slots")
@@ -88,6 +89,25 @@ class StaticCall:
                     dst.copy_(src)
             else:
                 slot.copy_(value)
+
+    def store_leading(self, **values: torch.Tensor) -> None:
+        """:meth:`store` for values that may be narrower than their static tensor in the last dimension: the value
+        goes into the leading columns and the rest stays zero (zeroed again only after a wider value was stored),
+        which is what zero-padding the value first and copying it whole would leave -- with one launch, not three."""
+        if not hasattr(self, "_stored_width"):
+            self._stored_width: dict[str, int] = {}
+        for name, value in values.items():
+            slot = self.inputs[name]
+            width = int(value.shape[-1])
+            if value.shape[:-1] != slot.shape[:-1] or width > slot.shape[-1]:
+                raise ValueError(f"{name}: {tuple(value.shape)} does not fit the static {tuple(slot.shape)}")
+            if width == slot.shape[-1]:
+                slot.copy_(value)
+            else:
+                if self._stored_width.get(name, slot.shape[-1]) > width:  # (the first store: whatever recording left there)
+                    slot[..., width:].zero_()
+                slot[..., :width].copy_(value)
+            self._stored_width[name] = width
 
     def store_owned(self, **values: Any) -> None:
         """:meth:`store` for tensors the backend owns and never changes in place (cached token ids, all-true
@@ -100,6 +120,12 @@ class StaticCall:
             if len(last) != len(objects) or any(a is not b for a, b in zip(last, objects)):
                 self.store(**{name: value})
                 self._last_owned[name] = objects
+
+    def forget_leading(self, *names: str) -> None:
+        """The static tensors ``names`` were written in full by something else (noise drawn in place): the next
+        :meth:`store_leading` of a narrower value clears the columns behind it."""
+        for name in names:
+            getattr(self, "_stored_width", {}).pop(name, None)
 
     def forget_owned(self, *names: str) -> None:
         """The static tensors ``names`` were overwritten by a plain :meth:`store`: the next

@@ -192,6 +192,7 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
             self.camera_alias[s] = d
 
         self._init_sampling(seed)
+        self._mask_cache: dict[tuple[int, bool, str], torch.Tensor] = {}
         self.rtc_processor = None
         self._init_graphs(graph, "pi05 graph", log)
         self.overlap = False  # prefill x step-0 two-stream overlap is not implemented; accepted, inert
@@ -309,18 +310,40 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
         present = [k for k in slots if k in batch]
         if not present:
             raise ValueError(f"All image features are missing from the batch (expected {self.config.image_features})")
+        images01, masks = self.prepare_images01(batch)
+        return [img * 2.0 - 1.0 for img in images01], masks
+
+    def prepare_images01(self, batch: dict[str, torch.Tensor]):
+        """:meth:`prepare_images` before the change of range: images in [0, 1] (an empty slot all zeros, which
+        ``x * 2 - 1`` turns into the -1 filler) and the cached all-true / all-false masks."""
+        h, w = self.config.image_resolution
+        slots = self.config.live_camera_keys(batch) if self.pad_free else self.config.image_features
+        present = [k for k in slots if k in batch]
+        if not present:
+            raise ValueError(f"All image features are missing from the batch (expected {self.config.image_features})")
         images, masks = [], []
         for key in present:
-            img = resize_with_pad_center(batch[key].float(), h, w) * 2.0 - 1.0
+            img = resize_with_pad_center(batch[key].float(), h, w)
             images.append(img)
-            masks.append(torch.ones(img.shape[0], dtype=torch.bool, device=img.device))
+            masks.append(self._mask(img.shape[0], True, img.device))
         for _ in [k for k in slots if k not in batch]:
-            images.append(torch.ones_like(images[-1]) * -1)
-            masks.append(torch.zeros_like(masks[-1]))
+            images.append(torch.zeros_like(images[-1]))
+            masks.append(self._mask(images[-1].shape[0], False, images[-1].device))
         return images, masks
 
+    def _mask(self, batch_size: int, value: bool, device) -> torch.Tensor:
+        """A cached all-true / all-false image mask (never written to) on the images' device."""
+        key = (batch_size, value, str(device))
+        if key not in self._mask_cache:
+            self._mask_cache[key] = torch.full((batch_size,), value, dtype=torch.bool, device=device)
+        return self._mask_cache[key]
+
+    def _core(self, images01, img_masks, tokens, masks, noise) -> torch.Tensor:
+        """The unit a graph records: the change of range of the images and the whole model."""
+        return self.model.sample_actions([img * 2.0 - 1.0 for img in images01], img_masks, tokens, masks, noise)
+
     def _infer(self, batch: dict[str, torch.Tensor], noise: torch.Tensor | None) -> torch.Tensor:
-        images, img_masks = self.prepare_images(batch)
+        images, img_masks = self.prepare_images01(batch)
         tokens, masks = batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK]
         if self.pad_free:
             # the language block on the bucket grid, for the eager path and the recorded shapes alike
@@ -328,9 +351,8 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
         if self.graph_enabled and self._graph_runner:
             entry = self._graph_runner.entry((len(images), int(tokens.shape[1])))
             return self._run_graph(entry, images, img_masks, tokens, masks, noise)
-        if noise is None:
-            noise = self._sample_noise()
-        return self.model.sample_actions(images, img_masks, tokens, masks, noise)
+        noise = self._sample_noise() if noise is None else self._pad_noise(noise)
+        return self._core(images, img_masks, tokens, masks, noise)
 
     # ------------------------------------------------------------------ hipGraph path
     def _capture_graph(self, key, request=None) -> StaticCall:
@@ -343,22 +365,26 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
         f32 = dict(dtype=torch.float32, device=dev)
         call = StaticCall(
             torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, **f32),
-            images=[torch.zeros(1, 3, height, width, **f32) for _ in range(n_cams)],
+            images01=[torch.zeros(1, 3, height, width, **f32) for _ in range(n_cams)],
             img_masks=[torch.ones(1, dtype=torch.bool, device=dev) for _ in range(n_cams)],
             tokens=torch.zeros(1, lang_len, dtype=torch.int64, device=dev),
             masks=torch.ones(1, lang_len, dtype=torch.bool, device=dev),
             noise=torch.zeros(1, cfg.chunk_size, cfg.max_action_dim, **f32),
         )
         log.info(f"capturing one graph for {n_cams} camera(s), lang={lang_len}, steps={cfg.num_steps}")
-        return call.record(self._sess, self.model.sample_actions)
+        return call.record(self._sess, self._core)
 
     def _run_graph(self, call: StaticCall, images, img_masks, tokens, masks, noise) -> torch.Tensor:
-        """The request's tensors go into the static ones on the input stream, then the replay."""
+        """The request's tensors go into the static ones on the input stream (images still in [0, 1]: the change
+        of range is part of the recorded unit; the noise at the caller's width), then the replay.  Returns the
+        graph's static output: every caller is done with it, or has copied it, before the next request replays."""
         with self._graph_runner.copy_inputs():
-            call.store(images=images, img_masks=img_masks, tokens=tokens, masks=masks)
+            call.store(images01=images, tokens=tokens, masks=masks)
+            call.store_owned(img_masks=img_masks)  # always the engine's cached all-true / all-false masks
             if noise is None:
                 self._sample_noise(out=call.inputs["noise"])  # drawn outside the graph, from the engine's generator
+                call.forget_leading("noise")
             else:
-                call.store(noise=noise)
+                call.store_leading(noise=noise)
         self._graph_runner.wait_inputs()
-        return call.replay()
+        return call.replay(copy=False)

@@ -310,7 +310,6 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
 
     def _infer(self, batch: dict[str, torch.Tensor], noise: torch.Tensor | None) -> torch.Tensor:
         images, img_masks = self.prepare_images01(batch)
-        state = self.prepare_state(batch)
         tokens, lang_masks = batch[OBS_LANGUAGE_TOKENS], batch[OBS_LANGUAGE_ATTENTION_MASK]
         if self.graph_enabled and self._graph_runner:
             entry = None
@@ -320,11 +319,10 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
                 if not self._graph_fallback_warned:
                     log.warning(f"graph replay skipped ({e}); falling back to eager for this request")
                     self._graph_fallback_warned = True
-            if entry is not None:
-                return self._run_graph(entry, images, img_masks, tokens, lang_masks, state, noise)
-        if noise is None:
-            noise = self._sample_noise()
-        return self._core(images, img_masks, tokens, lang_masks, state, noise)
+            if entry is not None:  # state and noise at the frame's widths: the static tensors hold the zero padding
+                return self._run_graph(entry, images, img_masks, tokens, lang_masks, batch[OBS_STATE], noise)
+        noise = self._sample_noise() if noise is None else self._pad_noise(noise)
+        return self._core(images, img_masks, tokens, lang_masks, self.prepare_state(batch), noise)
 
     # ------------------------------------------------------------------ hipGraph path
     def _prefix_len_for(self, n_cams: int) -> int:
@@ -350,12 +348,13 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
         return call.record(self._sess, self._core)
 
     def _run_graph(self, call: StaticCall, images01, img_masks, tokens, lang_masks, state, noise) -> torch.Tensor:
-        """The request's tensors go into the static ones on the input stream (one copy per camera and
-        one for the state; token ids and masks only when they are not the cached objects stored last
-        time), then the replay.  Returns the graph's static output: every caller is done with it, or has
+        """The request's tensors go into the static ones on the input stream (one copy per camera, one for
+        the state and one for the noise, each at the frame's width: the static tensors keep the zero padding;
+        token ids and masks only when they are not the cached objects stored last time), then the replay.  Returns the graph's static output: every caller is done with it, or has
         copied it, before the next request replays."""
         with self._graph_runner.copy_inputs():
-            call.store(images01=images01, state=state)
+            call.store(images01=images01)
+            call.store_leading(state=state)
             call.store_owned(img_masks=img_masks)  # always the engine's cached all-true / all-false masks
             # token ids and masks: skipped only when they are the engine's own cached pair for the task; a
             # frame that carries its own token tensors may change them in place between requests
@@ -366,7 +365,8 @@ class SmolVLAEngine(ChunkRuntime, PolicyEngine):
                 call.forget_owned("lang_tokens", "lang_masks")
             if noise is None:
                 self._sample_noise(out=call.inputs["noise"])  # drawn outside the graph, from the engine's generator
+                call.forget_leading("noise")
             else:
-                call.store(noise=noise)
+                call.store_leading(noise=noise)
         self._graph_runner.wait_inputs()
         return call.replay(copy=False)
