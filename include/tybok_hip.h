@@ -453,6 +453,19 @@ int tk_prefix_meta(const void* pad, const void* att, int P, int p_pad, int rope_
 int tk_patchify_images(const void* img0, const void* img1, const void* img2, const void* img3, int n, int H, int W, int patch,
                        float scale, float shift, void* out, void* stream);
 
+/* The prefix rows of a request in one launch, in the type the prefill reads (fp32): the connector's rows of all cameras
+ * times the image scale, the language tokens' embedding rows times theirs (both products rounded to bf16 first, as a bf16
+ * tensor times a scalar is), then closing rows as they are (the projected state) -- what scaling, embedding lookup and
+ * concatenation build in `embed_prefix` (tybok/policies/smolvla/models/flow_matching.py:160-257) -- and, optionally, the
+ * pad flags of the same rows (a flag per camera, a flag per token, 1 for the closing rows).
+ *   img: bf16 [n_img, H]; table: bf16 [vocab, H]; tokens: int64 [n_tok] (ids are clamped into the table);
+ *   last: fp32 [n_last, H]; out: fp32 [n_img + n_tok + n_last, H]; H a multiple of 8; 16-byte aligned rows.
+ *   pad_out: bytes [n_img + n_tok + n_last] or NULL; cam_flag0..3: one byte each (the first `cams` are read, n_img a
+ *   multiple of cams); tok_flag: bytes [n_tok]. */
+int tk_prefix_rows(const void* img, int n_img, float img_scale, const void* table, const void* tokens, int n_tok, int vocab,
+                   float tok_scale, const void* last, int n_last, void* out, int H, const void* cam_flag0, const void* cam_flag1,
+                   const void* cam_flag2, const void* cam_flag3, int cams, const void* tok_flag, void* pad_out, void* stream);
+
 /* LayerNorm of token rows with the cast to the GEMM input type folded in:
  *   y[m, :] = bf16((x[m, :] - mean) * rstd * w + b), statistics in fp32 (biased variance).
  * Replaces `layer_norm1/2(x)` (+ the `.to(bf16)` of the low-precision tiers) in the encoder layers
@@ -469,6 +482,15 @@ int tk_layer_norm(const void* x, int ldx, int x_dtype, const void* w, const void
  * tybok/policies/smolvla/models/vision.py:197-257, tybok/policies/pi05/models/vision.py:115-170). */
 int tk_add_layer_norm(const void* x, int ldx, int x_dtype, const void* r, int ldr, void* xsum, int ldxs, const void* w,
                       const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream);
+
+/* tk_add_layer_norm with the normalised rows written in another order: row m of the result goes to row y_rows[m] of y
+ * (int32 [M] on the device, a permutation of 0..M-1; values outside that range are clamped into it).  The tower's
+ * closing LayerNorm followed by the pixel shuffle, which moves whole token rows
+ * (tybok/policies/smolvla/models/vision.py:197-257 and the connector's `pixel_shuffle` in front of its projection).
+ * y must not alias x or xsum. */
+int tk_add_layer_norm_rows(const void* x, int ldx, int x_dtype, const void* r, int ldr, void* xsum, int ldxs, const void* w,
+                           const void* b, int wb_dtype, float eps, void* y, int ldy, const void* y_rows, int M, int K,
+                           void* stream);
 
 /* tk_layer_norm for fp32 rows and fp32 parameters with the normalised row rounded to IEEE fp16 instead of bf16:
  * the LayerNorm + cast in front of the fp16 q|k|v projection of pi0.5's fused tower (`n.to(tl.float16)`,

@@ -161,6 +161,9 @@ def _cases():
         ("tk_layer_norm", ln(K=4096, ldx=4096, ldy=4096), -1, "at most"),
         ("tk_layer_norm", ln(wdt=1), -1, "both"),
         ("tk_layer_norm", ln(ldy=760), -1, "row pitch"),
+        ("tk_add_layer_norm_rows", (P, 768, 0, P, 768, P, 768, P, P, 0, 1e-6, P + 65536, 768, None, 3072, 768, None), -1, "row map is null"),
+        ("tk_add_layer_norm_rows", (P, 768, 0, P, 768, P, 768, P, P, 0, 1e-6, P, 768, P, 3072, 768, None), -1, "must not be x or xsum"),
+        ("tk_add_layer_norm_rows", (P, 768, 0, None, 768, P, 768, P, P, 0, 1e-6, P + 65536, 768, P, 3072, 768, None), -1, "null residual"),
         ("tk_batched_transpose_v", tv(D=128), -1, "head_dim"),
         ("tk_batched_transpose_v", tv(keys=1000), -1, "rounded up to 32"),
         ("tk_batched_transpose_v", tv(sl=2300), -1, "multiples of 8"),
@@ -174,6 +177,11 @@ def _cases():
         ("tk_expert_kv_project_layers", (17, P, P, 960, 241, 320, P, P, 320, P, P, P, P, 256, None), -1, "17 layers"),
         ("tk_expert_kv_project_layers", (8, P, P, 960, 241, 320, P, P, 300, P, P, P, P, 256, None), -1, "bad shape"),
         ("tk_expert_kv_project_layers", (8, P, P, 960, 241, 320, P, P, 320, P, P, P, P, 224, None), -1, "rounded up to 32"),
+        ("tk_prefix_rows", (P, 192, 30.0, P, P, 48, 49280, 30.9, P, 1, P, 964, P, P, P, None, 3, P, P, None), -1, "H=964"),
+        ("tk_prefix_rows", (P, 192, 30.0, P, P + 4, 48, 49280, 30.9, P, 1, P, 960, P, P, P, None, 3, P, P, None), -1, "8-byte aligned ids"),
+        ("tk_prefix_rows", (P, 192, 30.0, P, P, 48, 49280, 30.9, P, 1, P, 960, P, P, None, None, 3, P, P, None), -1, "camera 2 is null"),
+        ("tk_prefix_rows", (P, 190, 30.0, P, P, 48, 49280, 30.9, P, 1, P, 960, P, P, P, None, 3, P, P, None), -1, "do not split"),
+        ("tk_prefix_rows", (P, 192, 30.0, P, P, 48, 49280, 30.9, P, 1, None, 960, P, P, P, None, 3, P, P, None), -1, "output is null"),
         ("tk_patchify_images", patch(n=5), -1, "n=5"),
         ("tk_patchify_images", patch(ps=12), -1, "patch=12"),
         ("tk_patchify_images", patch(H=500), -1, "divides"),

@@ -392,6 +392,26 @@ def test_residual_add_and_layer_norm_in_one_launch(tk, dtype, m, k):
     assert torch.equal(got, tk.layer_norm(got_x, w.cuda(), b.cuda(), 1e-6))  # same kernel arithmetic after the add
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,k", [(3072, 768), (64, 1152), (5, 8)])
+def test_residual_add_and_layer_norm_with_a_row_permutation(tk, dtype, m, k):
+    # the normalised rows written in another order (the pixel shuffle behind a tower's closing LayerNorm): row i of
+    # the plain launch must be row y_rows[i] here, bit for bit, and the in-place sum stays where it is
+    g = torch.Generator().manual_seed(63)
+    x = (torch.randn(m, k, generator=g) * 2.0).to(dtype).cuda()
+    r = torch.randn(m, k, generator=g).to(torch.bfloat16).cuda()
+    w, b = (1.0 + 0.3 * torch.randn(k, generator=g)).to(dtype).cuda(), (0.2 * torch.randn(k, generator=g)).to(dtype).cuda()
+    rows = torch.randperm(m, generator=g).to(torch.int32).cuda()
+    plain_x, plain = tk.add_layer_norm(x.clone(), r, w, b, 1e-6)
+    got_x, got = tk.add_layer_norm(x.clone(), r, w, b, 1e-6, y_rows=rows)
+    assert torch.equal(got_x, plain_x)
+    assert torch.equal(got[rows.long()], plain)
+    with pytest.raises(ValueError):
+        tk.add_layer_norm(x.clone(), r, w, b, 1e-6, y_rows=rows.long())
+    with pytest.raises(ValueError):
+        tk.add_layer_norm(x.clone(), r, w, b, 1e-6, y_rows=rows[: m - 1])
+
+
 def test_gated_residual_epilogue(tk):
     # pi0.5 AdaRMS gated residual: y = resid + bf16(ffn(x) * gate)
     x, wg8, sg, wu8, su, wd8, sd = ffn_case(50, 1024, 4096, seed=3)

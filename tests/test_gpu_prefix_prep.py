@@ -5,6 +5,8 @@
 440-470 with no attention blocks) -- integer / byte results, compared exactly.
 `tk_patchify_images`: `images * 2 - 1`, the cast to bf16 and the unfolding in front of the patch GEMM
 (tybok/policies/smolvla/policy.py:117-163, tybok/policies/smolvla/models/vision.py:120-160) -- compared exactly.
+`tk_prefix_rows`: the scaled image rows, the scaled embedding rows of the language tokens and the state row concatenated
+in fp32, with their pad flags (tybok/policies/smolvla/models/flow_matching.py:160-257) -- compared exactly.
 """
 
 import pytest
@@ -97,3 +99,31 @@ def test_patchify_images_argument_rules(tk):
         tk.patchify_images([img], 12)  # not a multiple of 8
     with pytest.raises(RuntimeError, match="patch"):
         tk.patchify_images([torch.zeros(1, 3, 40, 40, device="cuda")], 16)  # does not divide the image
+
+
+@pytest.mark.parametrize("cams,per_cam,n_tok,h", [(3, 64, 48, 960), (1, 64, 48, 960), (4, 16, 7, 64), (2, 5, 1, 8)])
+def test_prefix_rows_are_the_scaled_concatenation(tk, cams, per_cam, n_tok, h):
+    # image rows times a bf16-rounded scale, gathered embedding rows times sqrt(H), the projected state row, all
+    # widened to fp32, and the pad flags of those rows: bit for bit what the tensor operations build
+    import math
+
+    g = torch.Generator().manual_seed(70 + cams)
+    img = torch.randn(cams, per_cam, h, generator=g).to(torch.bfloat16).cuda()
+    table = torch.randn(300, h, generator=g).to(torch.bfloat16).cuda()
+    tokens = torch.randint(0, 300, (n_tok,), generator=g).cuda()
+    last = torch.randn(1, h, generator=g).cuda()
+    scale = torch.tensor(h**0.5, dtype=torch.bfloat16)
+    cam_flags = [torch.tensor([bool(i != 1)]).cuda() for i in range(cams)]
+    tok_flags = (torch.rand(n_tok, generator=g) < 0.7).cuda()
+    got, flags = tk.prefix_rows(img, float(scale), table, tokens, math.sqrt(h), last, cam_flags=cam_flags, tok_flags=tok_flags)
+    lang = torch.nn.functional.embedding(tokens[None], table) * math.sqrt(h)
+    want = torch.cat([(img * scale.cuda()).reshape(1, -1, h).float(), lang.float(), last[None]], dim=1)
+    assert got.dtype == torch.float32 and torch.equal(got, want)
+    want_flags = torch.cat([f[:, None].expand(1, per_cam) for f in cam_flags] + [tok_flags[None], torch.ones(1, 1, dtype=torch.bool).cuda()], dim=1)
+    assert flags.dtype == torch.bool and torch.equal(flags, want_flags)
+    plain, none = tk.prefix_rows(img, float(scale), table, tokens, math.sqrt(h), last)
+    assert none is None and torch.equal(plain, want)
+    with pytest.raises(TypeError):
+        tk.prefix_rows(img.float(), float(scale), table, tokens, math.sqrt(h), last)
+    with pytest.raises(ValueError):
+        tk.prefix_rows(img, float(scale), table, tokens, math.sqrt(h), last, cam_flags=cam_flags[:-1] or [None, None], tok_flags=tok_flags)

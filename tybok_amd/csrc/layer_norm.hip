@@ -21,6 +21,8 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(LayerNormArgs a) {
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= a.M) return;
   const int pieces = a.K / 8;
+  int yrow = a.y_rows ? a.y_rows[row] : row;  // (requested with everything else)
+  yrow = yrow < 0 ? 0 : (yrow > a.M - 1 ? a.M - 1 : yrow);
   // the parameters of this lane's pieces are requested with the row (they depend on nothing computed here): asked
   // for after the two reductions they would cost the launch one more memory round trip
   i32x4 wq[PMAX][WF32 ? 2 : 1], bq[PMAX][WF32 ? 2 : 1];
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(LayerNormArgs a) {
         const float y0 = (v[i][2 * e] - mean) * rstd * w[2 * e] + b[2 * e], y1 = (v[i][2 * e + 1] - mean) * rstd * w[2 * e + 1] + b[2 * e + 1];
         o4.u[e] = a.y_f16 ? pack_f16x2(y0, y1) : pack_bf16x2(y0, y1);
       }
-      *(i32x4*)(a.y + (size_t)row * a.ldy + 8 * p) = o4.q;
+      *(i32x4*)(a.y + (size_t)yrow * a.ldy + 8 * p) = o4.q;
     }
   }
 }

@@ -7,6 +7,10 @@
 //                                         columns P .. p_pad-1 zero): the prefill's 2-D visibility
 //                          pos[j]       = clamp(cumsum(pad)[j] - 1, 0, positions - 1)            (rotary positions)
 //                          suf_pos[s]   = clamp(sum(pad) + s, 0, positions - 1)                  (the action tokens')
+//   prefix_rows_kernel   the fp32 prefix rows [image tokens; language tokens; closing rows] from the connector's bf16 rows
+//                        (times a scale, rounded to bf16 as the tensor product rounds it), the bf16 embedding table
+//                        gathered by token id (times its scale, likewise) and fp32 closing rows (the state token), and the
+//                        pad flags of the same rows from per-camera and per-token flags.
 //   patchify_kernel      up to four fp32 images [3][H][W] -> bf16 patch rows [(camera, py, px)][(c, i, j)] of
 //                        x * scale + shift (product and sum rounded separately, as two tensor operations round them):
 //                        the unfolded input of a non-overlapping patch convolution run as one GEMM.
@@ -126,7 +130,58 @@ __global__ __launch_bounds__(256) void patchify_kernel(PatchifyArgs a) {
   *(i32x4*)dst = i32x4{lo[0], lo[1], hi[0], hi[1]};
 }
 
+// one thread per 8 consecutive columns of a prefix row: image rows and token rows are scaled in bf16 (product in fp32,
+// rounded once, which is what a bf16 tensor times a scalar gives) and widened to fp32; the closing rows are copied
+__global__ __launch_bounds__(256) void prefix_rows_kernel(PrefixRowsArgs a) {
+  const int per_row = a.H / 8;
+  const int rows = a.n_img + a.n_tok + a.n_last;
+  const int gid = blockIdx.x * 256 + threadIdx.x;
+  if (gid >= rows * per_row) return;
+  const int row = gid / per_row, c0 = (gid % per_row) * 8;
+  float* dst = a.out + (size_t)row * a.H + c0;
+  unsigned char flag = 1;
+  if (row >= a.n_img + a.n_tok) {
+    const float* src = a.last + (size_t)(row - a.n_img - a.n_tok) * a.H + c0;
+    const f32x4 lo = *(const f32x4*)src, hi = *(const f32x4*)(src + 4);
+    *(f32x4*)dst = lo;
+    *(f32x4*)(dst + 4) = hi;
+  } else {
+    const u16* src;
+    float scale;
+    if (row < a.n_img) {
+      src = a.img + (size_t)row * a.H + c0;
+      scale = a.img_scale;
+      if (a.pad_out) flag = a.cam_flag[row / a.per_cam][0];
+    } else {
+      const int t = row - a.n_img;
+      long long id = a.tokens[t];
+      id = id < 0 ? 0 : (id > a.vocab - 1 ? a.vocab - 1 : id);
+      src = a.table + (size_t)id * a.H + c0;
+      scale = a.tok_scale;
+      if (a.pad_out) flag = a.tok_flag[t];
+    }
+    union { i32x4 q; unsigned u[4]; } x;
+    x.q = *(const i32x4*)src;
+    f32x4 lo, hi;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const unsigned pk = pack_bf16x2(mul_rn(__uint_as_float(x.u[e] << 16), scale), mul_rn(__uint_as_float(x.u[e] & 0xffff0000u), scale));
+      const float v0 = __uint_as_float(pk << 16), v1 = __uint_as_float(pk & 0xffff0000u);
+      if (e < 2) { lo[2 * e] = v0; lo[2 * e + 1] = v1; } else { hi[2 * (e - 2)] = v0; hi[2 * (e - 2) + 1] = v1; }
+    }
+    *(f32x4*)dst = lo;
+    *(f32x4*)(dst + 4) = hi;
+  }
+  if (a.pad_out && c0 == 0) a.pad_out[row] = flag ? 1 : 0;
+}
+
 }  // namespace
+
+int tk_launch_prefix_rows(PrefixRowsArgs a, hipStream_t st) {
+  const long long threads = (long long)(a.n_img + a.n_tok + a.n_last) * (a.H / 8);
+  hipLaunchKernelGGL(prefix_rows_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
 
 int tk_prefix_meta_max_tokens() { return kMaxP; }
 

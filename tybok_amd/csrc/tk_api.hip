@@ -1340,9 +1340,50 @@ int tk_patchify_images(const void* img0, const void* img1, const void* img2, con
   return TK_OK;
 }
 
+int tk_prefix_rows(const void* img, int n_img, float img_scale, const void* table, const void* tokens, int n_tok, int vocab,
+                   float tok_scale, const void* last, int n_last, void* out, int H, const void* cam_flag0, const void* cam_flag1,
+                   const void* cam_flag2, const void* cam_flag3, int cams, const void* tok_flag, void* pad_out, void* stream) {
+  if (n_img < 0 || n_tok < 0 || n_last < 0 || n_img + n_tok + n_last < 1 || H <= 0 || H % 8)
+    return fail(TK_EINVAL, "prefix_rows: row counts %d + %d + %d must be non-negative with a row in all, H=%d a multiple of 8", n_img, n_tok,
+                n_last, H);
+  if (!out || !aligned16(out)) return fail(TK_EINVAL, "prefix_rows: the output is null or not 16-byte aligned");
+  if ((n_img && (!img || !aligned16(img))) || (n_last && (!last || !aligned16(last))))
+    return fail(TK_EINVAL, "prefix_rows: image rows and closing rows must be 16-byte aligned");
+  if (n_tok && (!table || !aligned16(table) || !tokens || ((uintptr_t)tokens & 7) || vocab < 1))
+    return fail(TK_EINVAL, "prefix_rows: the token rows need a 16-byte aligned table, vocab >= 1 and 8-byte aligned ids");
+  const void* flags[4] = {cam_flag0, cam_flag1, cam_flag2, cam_flag3};
+  PrefixRowsArgs a;
+  memset(&a, 0, sizeof(a));
+  if (pad_out) {
+    if (n_img && (cams < 1 || cams > 4 || n_img % cams)) return fail(TK_EINVAL, "prefix_rows: %d image rows do not split over cams=%d (1..4)", n_img, cams);
+    for (int i = 0; n_img && i < cams; ++i)
+      if (!flags[i]) return fail(TK_EINVAL, "prefix_rows: the flag of camera %d is null", i);
+    if (n_tok && !tok_flag) return fail(TK_EINVAL, "prefix_rows: pad flags asked for without the tokens' flags");
+    a.cams = n_img ? cams : 1;
+    a.per_cam = n_img ? n_img / cams : 1;
+    for (int i = 0; i < 4; ++i) a.cam_flag[i] = (const unsigned char*)flags[(n_img && i < cams) ? i : 0];
+  }
+  a.img = (const u16*)img;
+  a.n_img = n_img;
+  a.img_scale = img_scale;
+  a.table = (const u16*)table;
+  a.tokens = (const long long*)tokens;
+  a.n_tok = n_tok;
+  a.vocab = vocab;
+  a.tok_scale = tok_scale;
+  a.last = (const float*)last;
+  a.n_last = n_last;
+  a.out = (float*)out;
+  a.H = H;
+  a.tok_flag = (const unsigned char*)tok_flag;
+  a.pad_out = (unsigned char*)pad_out;
+  if (tk_launch_prefix_rows(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "prefix_rows: launch failed");
+  return TK_OK;
+}
+
 static int layer_norm_impl(const char* who, const void* x, int ldx, int x_dtype, const void* r, int ldr, void* xsum, int ldxs,
                            const void* w, const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream,
-                           int y_f16 = 0) {
+                           int y_f16 = 0, const int* y_rows = nullptr) {
   if (M <= 0 || K <= 0 || K % 8 || K > tk_layer_norm_max_k()) return fail(TK_EINVAL, "%s: K=%d must be a multiple of 8, at most %d", who, K, tk_layer_norm_max_k());
   if ((x_dtype != TK_BF16 && x_dtype != TK_F32) || x_dtype != wb_dtype) return fail(TK_EINVAL, "%s: rows and parameters must both be bf16 or both fp32", who);
   if (!x || !w || !b || !y || ldx < K || ldy < K || ldx % 8 || ldy % 8) return fail(TK_EINVAL, "%s: null pointer or row pitch not a multiple of 8 >= K", who);
@@ -1366,6 +1407,7 @@ static int layer_norm_impl(const char* who, const void* x, int ldx, int x_dtype,
   a.ldr = ldr;
   a.xsum = xsum;
   a.ldxs = ldxs;
+  a.y_rows = y_rows;
   if (tk_launch_layer_norm(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "%s: launch failed", who);
   return TK_OK;
 }
@@ -1379,6 +1421,15 @@ int tk_add_layer_norm(const void* x, int ldx, int x_dtype, const void* r, int ld
                       const void* b, int wb_dtype, float eps, void* y, int ldy, int M, int K, void* stream) {
   if (!r) return fail(TK_EINVAL, "add_layer_norm: null residual branch");
   return layer_norm_impl("add_layer_norm", x, ldx, x_dtype, r, ldr, xsum, ldxs, w, b, wb_dtype, eps, y, ldy, M, K, stream);
+}
+
+int tk_add_layer_norm_rows(const void* x, int ldx, int x_dtype, const void* r, int ldr, void* xsum, int ldxs, const void* w,
+                           const void* b, int wb_dtype, float eps, void* y, int ldy, const void* y_rows, int M, int K, void* stream) {
+  if (!r) return fail(TK_EINVAL, "add_layer_norm_rows: null residual branch");
+  if (!y_rows || ((uintptr_t)y_rows & 3)) return fail(TK_EINVAL, "add_layer_norm_rows: the row map is null or not 4-byte aligned");
+  if (y == xsum || y == x) return fail(TK_EINVAL, "add_layer_norm_rows: rows move, so y must not be x or xsum");
+  return layer_norm_impl("add_layer_norm_rows", x, ldx, x_dtype, r, ldr, xsum, ldxs, w, b, wb_dtype, eps, y, ldy, M, K, stream, 0,
+                         (const int*)y_rows);
 }
 
 int tk_layer_norm_f16(const void* x, int ldx, const void* w, const void* b, float eps, void* y, int ldy, int M, int K, void* stream) {

@@ -181,6 +181,8 @@ struct LayerNormArgs {
   int ldr;
   void* xsum;
   int ldxs;
+  // optional: row m of the result goes to row y_rows[m] of y (a permutation of 0..M-1; values outside are clamped)
+  const int* y_rows;
 };
 
 struct TailArgs {
@@ -245,6 +247,26 @@ struct PatchifyArgs {
   unsigned short* out;  // bf16 [n * (H/ps) * (W/ps)][3 * ps * ps]
 };
 int tk_launch_patchify(PatchifyArgs a, hipStream_t st);
+
+struct PrefixRowsArgs {
+  const unsigned short* img;  // bf16 [n_img, H]: rows 0 .. n_img-1 of the result are bf16(img * img_scale)
+  int n_img;
+  float img_scale;
+  const unsigned short* table;  // bf16 [vocab, H]: rows n_img .. n_img+n_tok-1 are bf16(table[tokens[t]] * tok_scale)
+  const long long* tokens;
+  int n_tok, vocab;
+  float tok_scale;
+  const float* last;  // fp32 [n_last, H]: the closing rows, as they are
+  int n_last;
+  float* out;  // fp32 [n_img + n_tok + n_last, H]
+  int H;
+  // optional pad flags of the same rows: a flag per camera (n_img = cams * per_cam rows), a flag per token, 1 for the closing rows
+  const unsigned char* cam_flag[4];
+  int cams, per_cam;
+  const unsigned char* tok_flag;
+  unsigned char* pad_out;
+};
+int tk_launch_prefix_rows(PrefixRowsArgs a, hipStream_t st);
 int tk_launch_norm_rows(NormRowsArgs a, hipStream_t st);
 int tk_launch_tail(TailArgs a, hipStream_t st);
 int tk_tail_embed_width();  // the embedding's input width the tail kernel is built for

@@ -131,6 +131,14 @@ SIGNATURES: dict[str, tuple] = {
         c_int,
         [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     ),  # fmt: skip
+    "tk_prefix_rows": (
+        c_int,
+        [c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+    ),  # fmt: skip
+    "tk_add_layer_norm_rows": (
+        c_int,
+        [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    ),  # fmt: skip
     "tk_rms_norm_rows": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tk_rope_rows": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "tk_expert_attn": (

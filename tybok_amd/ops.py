@@ -984,11 +984,13 @@ def layer_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, ou
 
 
 def add_layer_norm(
-    x: torch.Tensor, r: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, out_dtype: torch.dtype = torch.bfloat16
-) -> tuple[torch.Tensor, torch.Tensor]:
+    x: torch.Tensor, r: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, out_dtype: torch.dtype = torch.bfloat16,
+    *, y_rows: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, torch.Tensor]:  # fmt: skip
     """``x += r`` in place (``r`` bf16: the linear that closes a residual branch; fp32 ``x`` takes
     ``float(r)``, bf16 ``x`` rounds the sum once) and ``bf16(LayerNorm(x) * w + b)`` of the sum, one launch.
-    Returns ``(x, normalised)``; ``x`` must own contiguous rows."""
+    Returns ``(x, normalised)``; ``x`` must own contiguous rows.  ``y_rows`` (int32, one entry per row of the
+    flattened ``x``, a permutation): normalised row ``m`` is written as row ``y_rows[m]`` (bf16 result only)."""
     lib = native.lib()
     if x.dtype not in (torch.float32, torch.bfloat16) or w.dtype != x.dtype or b.dtype != x.dtype or r.dtype != torch.bfloat16:
         raise TypeError("add_layer_norm: x, w, b all fp32 or all bf16; r bf16")
@@ -999,8 +1001,8 @@ def add_layer_norm(
     if r2.stride(1) != 1:
         r2 = r2.contiguous()
     if out_dtype == torch.float16:
-        if x.dtype != torch.float32:
-            raise TypeError("add_layer_norm: the fp16 result is built for fp32 rows")
+        if x.dtype != torch.float32 or y_rows is not None:
+            raise TypeError("add_layer_norm: the fp16 result is built for fp32 rows in place")
         y = torch.empty(x2.shape, dtype=torch.float16, device=x.device)
         rc = lib.tk_add_layer_norm_f16(x2.data_ptr(), x2.stride(0), r2.data_ptr(), r2.stride(0), x2.data_ptr(), x2.stride(0),
                                        w.contiguous().data_ptr(), b.contiguous().data_ptr(), float(eps), y.data_ptr(), y.stride(0),
@@ -1009,6 +1011,14 @@ def add_layer_norm(
         return x, y.view(x.shape)
     y = torch.empty(x2.shape, dtype=torch.bfloat16, device=x.device)
     dt = _F32 if x.dtype == torch.float32 else _BF16
+    if y_rows is not None:
+        if y_rows.dtype != torch.int32 or y_rows.numel() < x2.shape[0] or not y_rows.is_contiguous() or y_rows.device != x.device:
+            raise ValueError("add_layer_norm: y_rows must be a contiguous int32 tensor on x's device with an entry per row")
+        rc = lib.tk_add_layer_norm_rows(x2.data_ptr(), x2.stride(0), dt, r2.data_ptr(), r2.stride(0), x2.data_ptr(), x2.stride(0),
+                                        w.contiguous().data_ptr(), b.contiguous().data_ptr(), dt, float(eps), y.data_ptr(), y.stride(0),
+                                        y_rows.data_ptr(), x2.shape[0], k, _stream())  # fmt: skip
+        native.check(rc, "tk_add_layer_norm_rows")
+        return x, y.view(x.shape)
     rc = lib.tk_add_layer_norm(x2.data_ptr(), x2.stride(0), dt, r2.data_ptr(), r2.stride(0), x2.data_ptr(), x2.stride(0),
                                w.contiguous().data_ptr(), b.contiguous().data_ptr(), dt, float(eps), y.data_ptr(), y.stride(0),
                                x2.shape[0], k, _stream())  # fmt: skip
@@ -1093,6 +1103,40 @@ def patchify_images(images, patch: int, scale: float = 1.0, shift: float = 0.0) 
     rc = lib.tk_patchify_images(*ptrs, len(images), h, w, int(patch), float(scale), float(shift), out.data_ptr(), _stream())
     native.check(rc, "tk_patchify_images")
     return out
+
+
+def prefix_rows(img, img_scale: float, table, tokens, tok_scale: float, last, *, cam_flags=None, tok_flags=None):
+    """The fp32 prefix ``[1, P, H]`` of one request in one launch: ``img`` bf16 ``[cams, per_cam, H]`` times ``img_scale``
+    and ``table[tokens]`` (bf16 ``[vocab, H]``, ids int64 ``[n_tok]``) times ``tok_scale`` -- both products rounded to
+    bf16 as the tensor products are -- then ``last`` fp32 ``[n_last, H]`` as it is.  With ``cam_flags`` (a bool tensor of
+    one element per camera) and ``tok_flags`` (bool ``[n_tok]``) also the pad flags ``[1, P]`` of those rows (the closing
+    rows are always valid); returns ``(rows, flags or None)``."""
+    lib = native.lib()
+    bf = torch.bfloat16
+    if img.dtype != bf or table.dtype != bf or last.dtype != torch.float32 or tokens.dtype != torch.int64:
+        raise TypeError("prefix_rows: img and table bf16, tokens int64, last fp32")
+    h = table.shape[1]
+    if img.dim() != 3 or img.shape[2] != h or last.dim() != 2 or last.shape[1] != h or not (img.is_contiguous() and table.is_contiguous() and last.is_contiguous() and tokens.is_contiguous()):
+        raise ValueError("prefix_rows: img [cams, per_cam, H], table [vocab, H], last [n_last, H], all contiguous")
+    cams, n_img, n_tok, n_last = img.shape[0], img.shape[0] * img.shape[1], tokens.numel(), last.shape[0]
+    total = n_img + n_tok + n_last
+    out = torch.empty(1, total, h, dtype=torch.float32, device=img.device)
+    flags, fl = None, [None] * 4
+    if cam_flags is not None:
+        cam_flags = list(cam_flags)
+        if len(cam_flags) != cams or not 1 <= cams <= 4 or tok_flags is None or tok_flags.numel() != n_tok or not tok_flags.is_contiguous():
+            raise ValueError("prefix_rows: a flag per camera (one to four) and a contiguous flag per token")
+        if any(f.dtype != torch.bool or f.numel() != 1 for f in cam_flags) or tok_flags.dtype != torch.bool:
+            raise TypeError("prefix_rows: flags are bool tensors")
+        flags = torch.empty(1, total, dtype=torch.bool, device=img.device)
+        fl = [f.data_ptr() for f in cam_flags] + [None] * (4 - cams)
+    rc = lib.tk_prefix_rows(
+        img.data_ptr(), n_img, float(img_scale), table.data_ptr(), tokens.data_ptr(), n_tok, table.shape[0], float(tok_scale),
+        last.data_ptr(), n_last, out.data_ptr(), h, *fl, cams, tok_flags.data_ptr() if flags is not None else None,
+        flags.data_ptr() if flags is not None else None, _stream(),
+    )  # fmt: skip
+    native.check(rc, "tk_prefix_rows")
+    return out, flags
 
 
 def decode_fp8_table(device: torch.device | str = "cuda") -> torch.Tensor:

@@ -198,10 +198,16 @@ class SmolVLAModel:
         sf, seq = cfg.vlm_config.scale_factor, side * side
         tok = torch.arange(seq, device=self.device).view(1, side, side // sf, sf).permute(0, 2, 1, 3)
         self.shuffle_perm = tok.reshape(1, side // sf, side // sf, sf * sf).permute(0, 2, 1, 3).reshape(seq).contiguous()
+        # ... and as destination rows of the tower's closing LayerNorm, for up to four cameras: token i of camera c goes
+        # where the shuffle puts it (the inverse permutation), so the norm launch writes the shuffled layout itself
+        inv = torch.empty_like(self.shuffle_perm)
+        inv[self.shuffle_perm] = torch.arange(seq, device=self.device)
+        self.shuffle_rows = torch.cat([inv + c * seq for c in range(4)]).to(torch.int32).contiguous()
         # the tower's position embedding repeated for four cameras, as the residual operand of the patch launch
         pos_w = self.p[VIS + "embeddings.position_embedding.weight"]
         self.vis_pos_rows = pos_w[self.vis_pos].repeat(4, 1).contiguous() if self.fused_vit and pos_w.dtype == BF16 else None
         self.img_scale = torch.tensor(t.hidden_size**0.5, dtype=BF16, device=self.device)
+        self._img_scale_value = float(torch.tensor(t.hidden_size**0.5, dtype=BF16))  # the same bf16-rounded factor, on the host
         self.patch_w = self.p[VIS + "embeddings.patch_embedding.weight"].reshape(v.hidden_size, -1)
 
     def set_num_steps(self, n: int) -> None:
@@ -283,7 +289,7 @@ class SmolVLAModel:
             n_h, n_w = image.shape[2] // ps, image.shape[3] // ps
             # non-overlapping patch convolution as one GEMM over unfolded patches
             x = image.to(BF16).view(b, 3, n_h, ps, n_w, ps).permute(0, 2, 4, 1, 3, 5).reshape(b, n_h * n_w, 3 * ps * ps)
-        pos_added, post = False, None
+        pos_added, post, shuffled = False, None, False
         if self.fused_vit:
             w_patch, b_patch = self.vis_dense["patch"]
             rows = b * x.shape[1]
@@ -323,8 +329,10 @@ class SmolVLAModel:
                 if i + 1 < v.num_hidden_layers:
                     nx = f"{VIS}encoder.layers.{i + 1}."
                     x, h = tk.add_layer_norm(x, m, p[nx + "layer_norm1.weight"], p[nx + "layer_norm1.bias"], v.layer_norm_eps)
-                else:  # the last residual add in the launch of the tower's closing LayerNorm
-                    post = tk.add_layer_norm(x, m, p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], v.layer_norm_eps)[1]
+                else:  # the last residual add in the launch of the tower's closing LayerNorm (and the pixel shuffle's row moves)
+                    shuffled = x.shape[1] == self.shuffle_perm.shape[0] and b * x.shape[1] <= self.shuffle_rows.shape[0]
+                    post = tk.add_layer_norm(x, m, p[VIS + "post_layernorm.weight"], p[VIS + "post_layernorm.bias"], v.layer_norm_eps,
+                                             y_rows=self.shuffle_rows if shuffled else None)[1]  # fmt: skip
                 continue
             h = F.layer_norm(x, (v.hidden_size,), p[lp + "layer_norm1.weight"], p[lp + "layer_norm1.bias"], v.layer_norm_eps)
             q = self.lin(lp + "self_attn.q_proj", h).view(b, -1, heads, hd).transpose(1, 2)
@@ -342,9 +350,11 @@ class SmolVLAModel:
         s = cfg.scale_factor
         seq, dim = x.shape[1], x.shape[2]
         if self.fused_vit and seq == self.shuffle_perm.shape[0]:
-            # the pixel shuffle moves whole token rows: one gather by a token permutation built with the model
-            x = torch.index_select(x, 1, self.shuffle_perm).reshape(b, seq // (s * s), dim * s * s)
-            return self._dense("connector", x)
+            # the pixel shuffle moves whole token rows: done by the closing norm's launch, or one gather by the token
+            # permutation built with the model
+            if not shuffled:
+                x = torch.index_select(x, 1, self.shuffle_perm)
+            return self._dense("connector", x.reshape(b, seq // (s * s), dim * s * s))
         side = int(seq**0.5)
         x = x.view(b, side, side, dim).view(b, side, side // s, dim * s).permute(0, 2, 1, 3)
         x = x.reshape(b, side // s, side // s, dim * s * s).permute(0, 2, 1, 3).reshape(b, seq // (s * s), dim * s * s)
@@ -368,7 +378,23 @@ class SmolVLAModel:
         embs, pads = [], []
         stacked = None  # the embeddings of all cameras as one [cameras, tokens, hidden] tensor, when they are batch-1 images
         if image_range01 and self._patch_rows_ok(images):
-            stacked = self.embed_image(None, images01=list(images)) * self.img_scale
+            raw = self.embed_image(None, images01=list(images))
+            table = self.p[TXT + "embed_tokens.weight"]
+            p_len = raw.shape[0] * raw.shape[1] + lang_tokens.shape[1] + 1
+            if (
+                state.shape[0] == 1 and lang_tokens.shape[0] == 1 and p_len in self._att_const and raw.dtype == BF16 and table.dtype == BF16
+                and lang_tokens.dtype == torch.int64 and lang_masks.dtype == torch.bool and raw.shape[0] <= 4
+                and len(img_masks) == raw.shape[0] and all(m.dtype == torch.bool and m.numel() == 1 for m in img_masks)
+            ):  # fmt: skip
+                st = self.lin("state_proj", state)
+                if st.dtype == torch.float32:
+                    # scaling, embedding lookup, casts, concatenation and the pad flags in one launch
+                    out, pads = tk.prefix_rows(
+                        raw.contiguous(), self._img_scale_value, table, lang_tokens[0].contiguous(), math.sqrt(table.shape[1]), st.contiguous(),
+                        cam_flags=img_masks, tok_flags=lang_masks[0].contiguous(),
+                    )  # fmt: skip
+                    return out, pads, self._att_const[p_len]
+            stacked = raw * self.img_scale
             per_image = stacked.split(1, dim=0)
             images = ()
         elif image_range01:
