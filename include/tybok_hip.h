@@ -452,19 +452,27 @@ int tk_prefix_meta(const void* pad, const void* att, int P, int p_pad, int rope_
  * that divides H and W; images and out 16-byte aligned; images beyond n are ignored. */
 int tk_patchify_images(const void* img0, const void* img1, const void* img2, const void* img3, int n, int H, int W, int patch,
                        float scale, float shift, void* out, void* stream);
+/* The same with fp32 patch rows and any even patch size (pi0.5's SigLIP tower: 14 x 14 patches, fp32 patch embedding,
+ * tybok/policies/pi05/models/vision.py:100-118 after `img * 2 - 1` of tybok/policies/pi05/policy.py:170-234). */
+int tk_patchify_images_f32(const void* img0, const void* img1, const void* img2, const void* img3, int n, int H, int W, int patch,
+                           float scale, float shift, void* out, void* stream);
 
 /* The prefix rows of a request in one launch, in the type the prefill reads (fp32): the connector's rows of all cameras
  * times the image scale, the language tokens' embedding rows times theirs (both products rounded to bf16 first, as a bf16
  * tensor times a scalar is), then closing rows as they are (the projected state) -- what scaling, embedding lookup and
  * concatenation build in `embed_prefix` (tybok/policies/smolvla/models/flow_matching.py:160-257) -- and, optionally, the
  * pad flags of the same rows (a flag per camera, a flag per token, 1 for the closing rows).
- *   img: bf16 [n_img, H]; table: bf16 [vocab, H]; tokens: int64 [n_tok] (ids are clamped into the table);
- *   last: fp32 [n_last, H]; out: fp32 [n_img + n_tok + n_last, H]; H a multiple of 8; 16-byte aligned rows.
+ *   img: bf16 [n_img, H] (img_dtype TK_BF16), or fp32 (TK_F32: pi0.5's projector output,
+ *   tybok/policies/pi05/models/flow_matching.py:415-437 -- those rows are taken as they are, img_scale unused);
+ *   table: bf16 [vocab, H]; tokens: int64 [n_tok] (ids are clamped into the table); last: fp32 [n_last, H];
+ *   out: [n_img + n_tok + n_last, H] fp32 (out_dtype TK_F32) or rounded to bf16 (TK_BF16: the prefill's hidden rows,
+ *   `embs.to(bfloat16)`); H a multiple of 8; 16-byte aligned rows.
  *   pad_out: bytes [n_img + n_tok + n_last] or NULL; cam_flag0..3: one byte each (the first `cams` are read, n_img a
  *   multiple of cams); tok_flag: bytes [n_tok]. */
-int tk_prefix_rows(const void* img, int n_img, float img_scale, const void* table, const void* tokens, int n_tok, int vocab,
-                   float tok_scale, const void* last, int n_last, void* out, int H, const void* cam_flag0, const void* cam_flag1,
-                   const void* cam_flag2, const void* cam_flag3, int cams, const void* tok_flag, void* pad_out, void* stream);
+int tk_prefix_rows(const void* img, int img_dtype, int n_img, float img_scale, const void* table, const void* tokens, int n_tok,
+                   int vocab, float tok_scale, const void* last, int n_last, void* out, int out_dtype, int H, const void* cam_flag0,
+                   const void* cam_flag1, const void* cam_flag2, const void* cam_flag3, int cams, const void* tok_flag, void* pad_out,
+                   void* stream);
 
 /* LayerNorm of token rows with the cast to the GEMM input type folded in:
  *   y[m, :] = bf16((x[m, :] - mean) * rstd * w + b), statistics in fp32 (biased variance).

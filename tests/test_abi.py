@@ -177,11 +177,14 @@ def _cases():
         ("tk_expert_kv_project_layers", (17, P, P, 960, 241, 320, P, P, 320, P, P, P, P, 256, None), -1, "17 layers"),
         ("tk_expert_kv_project_layers", (8, P, P, 960, 241, 320, P, P, 300, P, P, P, P, 256, None), -1, "bad shape"),
         ("tk_expert_kv_project_layers", (8, P, P, 960, 241, 320, P, P, 320, P, P, P, P, 224, None), -1, "rounded up to 32"),
-        ("tk_prefix_rows", (P, 192, 30.0, P, P, 48, 49280, 30.9, P, 1, P, 964, P, P, P, None, 3, P, P, None), -1, "H=964"),
-        ("tk_prefix_rows", (P, 192, 30.0, P, P + 4, 48, 49280, 30.9, P, 1, P, 960, P, P, P, None, 3, P, P, None), -1, "8-byte aligned ids"),
-        ("tk_prefix_rows", (P, 192, 30.0, P, P, 48, 49280, 30.9, P, 1, P, 960, P, P, None, None, 3, P, P, None), -1, "camera 2 is null"),
-        ("tk_prefix_rows", (P, 190, 30.0, P, P, 48, 49280, 30.9, P, 1, P, 960, P, P, P, None, 3, P, P, None), -1, "do not split"),
-        ("tk_prefix_rows", (P, 192, 30.0, P, P, 48, 49280, 30.9, P, 1, None, 960, P, P, P, None, 3, P, P, None), -1, "output is null"),
+        ("tk_prefix_rows", (P, 0, 192, 30.0, P, P, 48, 49280, 30.9, P, 1, P, 1, 964, P, P, P, None, 3, P, P, None), -1, "H=964"),
+        ("tk_prefix_rows", (P, 0, 192, 30.0, P, P + 4, 48, 49280, 30.9, P, 1, P, 1, 960, P, P, P, None, 3, P, P, None), -1, "8-byte aligned ids"),
+        ("tk_prefix_rows", (P, 0, 192, 30.0, P, P, 48, 49280, 30.9, P, 1, P, 1, 960, P, P, None, None, 3, P, P, None), -1, "camera 2 is null"),
+        ("tk_prefix_rows", (P, 0, 190, 30.0, P, P, 48, 49280, 30.9, P, 1, P, 1, 960, P, P, P, None, 3, P, P, None), -1, "do not split"),
+        ("tk_prefix_rows", (P, 0, 192, 30.0, P, P, 48, 49280, 30.9, P, 1, None, 1, 960, P, P, P, None, 3, P, P, None), -1, "output is null"),
+        ("tk_prefix_rows", (P, 2, 192, 30.0, P, P, 48, 49280, 30.9, P, 1, P, 1, 960, P, P, P, None, 3, P, P, None), -1, "img_dtype=2"),
+        ("tk_patchify_images_f32", patch(H=224, W=224, ps=7), -1, "multiple of 2"),
+        ("tk_patchify_images_f32", patch(H=224, W=224, ps=14, i2=None), -1, "image 2 is null"),
         ("tk_patchify_images", patch(n=5), -1, "n=5"),
         ("tk_patchify_images", patch(ps=12), -1, "patch=12"),
         ("tk_patchify_images", patch(H=500), -1, "divides"),

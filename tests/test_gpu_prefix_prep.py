@@ -89,6 +89,21 @@ def test_patchify_images_matches_scale_cast_unfold(tk, n, h, w, ps):
     assert torch.equal(got2.cpu(), want2)
 
 
+@pytest.mark.parametrize("n,h,w,ps", [(2, 224, 224, 14), (1, 28, 42, 14), (4, 24, 24, 6), (3, 32, 32, 16)])
+def test_patchify_images_in_fp32_with_any_even_patch(tk, n, h, w, ps):
+    # the fp32 form (14 x 14 patches in front of an fp32 patch embedding): x * 2 - 1 and the unfolding, bit for bit
+    g = torch.Generator().manual_seed(n * 100 + ps)
+    images = [torch.rand(1, 3, h, w, generator=g) for _ in range(n)]
+    for scale, shift in ((2.0, -1.0), (0.3, 0.1)):
+        x = torch.cat([img * scale + shift for img in images], dim=0)
+        want = x.view(n, 3, h // ps, ps, w // ps, ps).permute(0, 2, 4, 1, 3, 5).reshape(n, (h // ps) * (w // ps), 3 * ps * ps)
+        got = tk.patchify_images([img.cuda() for img in images], ps, scale, shift, out_dtype=torch.float32)
+        assert got.dtype == torch.float32 and got.shape == want.shape
+        assert torch.equal(got.cpu(), want)
+    with pytest.raises(RuntimeError, match="patch"):
+        tk.patchify_images([torch.zeros(1, 3, 21, 21, device="cuda")], 7, out_dtype=torch.float32)  # odd patch size
+
+
 def test_patchify_images_argument_rules(tk):
     img = torch.zeros(1, 3, 32, 32, device="cuda")
     with pytest.raises(ValueError):
@@ -124,6 +139,27 @@ def test_prefix_rows_are_the_scaled_concatenation(tk, cams, per_cam, n_tok, h):
     plain, none = tk.prefix_rows(img, float(scale), table, tokens, math.sqrt(h), last)
     assert none is None and torch.equal(plain, want)
     with pytest.raises(TypeError):
-        tk.prefix_rows(img.float(), float(scale), table, tokens, math.sqrt(h), last)
+        tk.prefix_rows(img.half(), float(scale), table, tokens, math.sqrt(h), last)
     with pytest.raises(ValueError):
         tk.prefix_rows(img, float(scale), table, tokens, math.sqrt(h), last, cam_flags=cam_flags[:-1] or [None, None], tok_flags=tok_flags)
+
+
+@pytest.mark.parametrize("cams,per_cam,n_tok,h", [(2, 256, 200, 2048), (1, 256, 40, 2048), (3, 7, 5, 64)])
+def test_prefix_rows_from_fp32_image_rows_in_bf16(tk, cams, per_cam, n_tok, h):
+    # fp32 image rows as they are, embedding rows times a bf16-rounded scale, no closing rows, everything rounded to
+    # bf16: the hidden rows a prefill takes from `cat(...).to(bfloat16)`, bit for bit; and the same in fp32
+    g = torch.Generator().manual_seed(80 + cams)
+    img = (torch.randn(cams, per_cam, h, generator=g) * 3.0).cuda()
+    table = torch.randn(500, h, generator=g).to(torch.bfloat16).cuda()
+    tokens = torch.randint(0, 500, (n_tok,), generator=g).cuda()
+    scale = torch.tensor(h**0.5, dtype=torch.bfloat16)
+    cam_flags = [torch.tensor([bool(i != 0)]).cuda() for i in range(cams)]
+    tok_flags = (torch.rand(n_tok, generator=g) < 0.5).cuda()
+    lang = torch.nn.functional.embedding(tokens[None], table) * scale.cuda()
+    want = torch.cat([img.reshape(1, -1, h), lang], dim=1)
+    assert want.dtype == torch.float32
+    got, flags = tk.prefix_rows(img, 1.0, table, tokens, float(scale), None, cam_flags=cam_flags, tok_flags=tok_flags, out_dtype=torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and torch.equal(got, want.to(torch.bfloat16))
+    assert torch.equal(flags, torch.cat([f[:, None].expand(1, per_cam) for f in cam_flags] + [tok_flags[None]], dim=1))
+    got32, _ = tk.prefix_rows(img, 1.0, table, tokens, float(scale))
+    assert torch.equal(got32, want)

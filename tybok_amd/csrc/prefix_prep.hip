@@ -126,30 +126,52 @@ __global__ __launch_bounds__(256) void patchify_kernel(PatchifyArgs a) {
   const i32x2 lo = pack_bf16x4(w0), hi = pack_bf16x4(w1);
   const int ps = a.ps, py = y / ps, iy = y % ps, px = xs / ps, ix = xs % ps;
   const int n_w = a.W / ps, n_h = a.H / ps;
-  u16* dst = a.out + (((size_t)cam * n_h + py) * n_w + px) * (size_t)(3 * ps * ps) + ((size_t)c * ps + iy) * ps + ix;
+  u16* dst = (u16*)a.out + (((size_t)cam * n_h + py) * n_w + px) * (size_t)(3 * ps * ps) + ((size_t)c * ps + iy) * ps + ix;
   *(i32x4*)dst = i32x4{lo[0], lo[1], hi[0], hi[1]};
 }
 
-// one thread per 8 consecutive columns of a prefix row: image rows and token rows are scaled in bf16 (product in fp32,
-// rounded once, which is what a bf16 tensor times a scalar gives) and widened to fp32; the closing rows are copied
+// the same with fp32 patch rows and any even patch size: one thread per 2 consecutive pixels of an image row
+__global__ __launch_bounds__(256) void patchify_f32_kernel(PatchifyArgs a) {
+  const int per_row = a.W / 2;
+  const long long per_img = (long long)3 * a.H * per_row;
+  const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= per_img * a.n) return;
+  const int cam = (int)(gid / per_img);
+  long long r = gid % per_img;
+  const int xs = (int)(r % per_row) * 2;
+  r /= per_row;
+  const int y = (int)(r % a.H), c = (int)(r / a.H);
+  const f32x2 v = *(const f32x2*)(a.img[cam] + ((size_t)c * a.H + y) * a.W + xs);
+  const f32x2 w = {add_rn(mul_rn(v[0], a.scale), a.shift), add_rn(mul_rn(v[1], a.scale), a.shift)};
+  const int ps = a.ps, py = y / ps, iy = y % ps, px = xs / ps, ix = xs % ps;
+  const int n_w = a.W / ps, n_h = a.H / ps;
+  float* dst = (float*)a.out + (((size_t)cam * n_h + py) * n_w + px) * (size_t)(3 * ps * ps) + ((size_t)c * ps + iy) * ps + ix;
+  *(f32x2*)dst = w;
+}
+
+// one thread per 8 consecutive columns of a prefix row: bf16 image rows and the token rows are scaled in bf16 (product in
+// fp32, rounded once, which is what a bf16 tensor times a scalar gives); fp32 image rows and the closing rows are taken
+// as they are; the result is written in fp32 or rounded to bf16
 __global__ __launch_bounds__(256) void prefix_rows_kernel(PrefixRowsArgs a) {
   const int per_row = a.H / 8;
   const int rows = a.n_img + a.n_tok + a.n_last;
   const int gid = blockIdx.x * 256 + threadIdx.x;
   if (gid >= rows * per_row) return;
   const int row = gid / per_row, c0 = (gid % per_row) * 8;
-  float* dst = a.out + (size_t)row * a.H + c0;
+  const size_t o = (size_t)row * a.H + c0;
   unsigned char flag = 1;
-  if (row >= a.n_img + a.n_tok) {
-    const float* src = a.last + (size_t)(row - a.n_img - a.n_tok) * a.H + c0;
-    const f32x4 lo = *(const f32x4*)src, hi = *(const f32x4*)(src + 4);
-    *(f32x4*)dst = lo;
-    *(f32x4*)(dst + 4) = hi;
+  f32x4 lo, hi;
+  const bool closing = row >= a.n_img + a.n_tok;
+  if (closing || (row < a.n_img && a.img_f32)) {
+    const float* src = closing ? a.last + (size_t)(row - a.n_img - a.n_tok) * a.H + c0 : (const float*)a.img + (size_t)row * a.H + c0;
+    lo = *(const f32x4*)src;
+    hi = *(const f32x4*)(src + 4);
+    if (!closing && a.pad_out) flag = a.cam_flag[row / a.per_cam][0];
   } else {
     const u16* src;
     float scale;
     if (row < a.n_img) {
-      src = a.img + (size_t)row * a.H + c0;
+      src = (const u16*)a.img + (size_t)row * a.H + c0;
       scale = a.img_scale;
       if (a.pad_out) flag = a.cam_flag[row / a.per_cam][0];
     } else {
@@ -162,15 +184,19 @@ __global__ __launch_bounds__(256) void prefix_rows_kernel(PrefixRowsArgs a) {
     }
     union { i32x4 q; unsigned u[4]; } x;
     x.q = *(const i32x4*)src;
-    f32x4 lo, hi;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const unsigned pk = pack_bf16x2(mul_rn(__uint_as_float(x.u[e] << 16), scale), mul_rn(__uint_as_float(x.u[e] & 0xffff0000u), scale));
       const float v0 = __uint_as_float(pk << 16), v1 = __uint_as_float(pk & 0xffff0000u);
       if (e < 2) { lo[2 * e] = v0; lo[2 * e + 1] = v1; } else { hi[2 * (e - 2)] = v0; hi[2 * (e - 2) + 1] = v1; }
     }
-    *(f32x4*)dst = lo;
-    *(f32x4*)(dst + 4) = hi;
+  }
+  if (a.out_bf16) {
+    const i32x2 p0 = pack_bf16x4(lo), p1 = pack_bf16x4(hi);
+    *(i32x4*)((u16*)a.out + o) = i32x4{p0[0], p0[1], p1[0], p1[1]};
+  } else {
+    *(f32x4*)((float*)a.out + o) = lo;
+    *(f32x4*)((float*)a.out + o + 4) = hi;
   }
   if (a.pad_out && c0 == 0) a.pad_out[row] = flag ? 1 : 0;
 }
@@ -194,7 +220,10 @@ int tk_launch_prefix_meta(PrefixMetaArgs a, hipStream_t st) {
 }
 
 int tk_launch_patchify(PatchifyArgs a, hipStream_t st) {
-  const long long threads = (long long)a.n * 3 * a.H * (a.W / 8);
-  hipLaunchKernelGGL(patchify_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a);
+  const long long threads = (long long)a.n * 3 * a.H * (a.W / (a.out_f32 ? 2 : 8));
+  if (a.out_f32)
+    hipLaunchKernelGGL(patchify_f32_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL(patchify_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }

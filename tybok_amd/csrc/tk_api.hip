@@ -1318,11 +1318,11 @@ int tk_prefix_meta(const void* pad, const void* att, int P, int p_pad, int rope_
   return TK_OK;
 }
 
-int tk_patchify_images(const void* img0, const void* img1, const void* img2, const void* img3, int n, int H, int W, int patch,
-                       float scale, float shift, void* out, void* stream) {
-  const void* imgs[4] = {img0, img1, img2, img3};
-  if (n < 1 || n > 4 || H <= 0 || W <= 0 || patch <= 0 || patch % 8 || H % patch || W % patch)
-    return fail(TK_EINVAL, "patchify: n=%d in 1..4, patch=%d a multiple of 8 that divides H=%d and W=%d", n, patch, H, W);
+static int patchify_impl(const void* const* imgs, int n, int H, int W, int patch, float scale, float shift, void* out, int out_f32,
+                         void* stream) {
+  const int unit = out_f32 ? 2 : 8;  // pixels per thread: a thread's pixels must not straddle two patches
+  if (n < 1 || n > 4 || H <= 0 || W <= 0 || patch <= 0 || patch % unit || H % patch || W % patch)
+    return fail(TK_EINVAL, "patchify: n=%d in 1..4, patch=%d a multiple of %d that divides H=%d and W=%d", n, patch, unit, H, W);
   if (!out || !aligned16(out)) return fail(TK_EINVAL, "patchify: the output must be 16-byte aligned");
   PatchifyArgs a;
   for (int i = 0; i < 4; ++i) {
@@ -1335,14 +1335,30 @@ int tk_patchify_images(const void* img0, const void* img1, const void* img2, con
   a.ps = patch;
   a.scale = scale;
   a.shift = shift;
-  a.out = (u16*)out;
+  a.out = out;
+  a.out_f32 = out_f32;
   if (tk_launch_patchify(a, (hipStream_t)stream)) return fail(TK_ELAUNCH, "patchify: launch failed");
   return TK_OK;
 }
 
-int tk_prefix_rows(const void* img, int n_img, float img_scale, const void* table, const void* tokens, int n_tok, int vocab,
-                   float tok_scale, const void* last, int n_last, void* out, int H, const void* cam_flag0, const void* cam_flag1,
-                   const void* cam_flag2, const void* cam_flag3, int cams, const void* tok_flag, void* pad_out, void* stream) {
+int tk_patchify_images(const void* img0, const void* img1, const void* img2, const void* img3, int n, int H, int W, int patch,
+                       float scale, float shift, void* out, void* stream) {
+  const void* imgs[4] = {img0, img1, img2, img3};
+  return patchify_impl(imgs, n, H, W, patch, scale, shift, out, 0, stream);
+}
+
+int tk_patchify_images_f32(const void* img0, const void* img1, const void* img2, const void* img3, int n, int H, int W, int patch,
+                           float scale, float shift, void* out, void* stream) {
+  const void* imgs[4] = {img0, img1, img2, img3};
+  return patchify_impl(imgs, n, H, W, patch, scale, shift, out, 1, stream);
+}
+
+int tk_prefix_rows(const void* img, int img_dtype, int n_img, float img_scale, const void* table, const void* tokens, int n_tok,
+                   int vocab, float tok_scale, const void* last, int n_last, void* out, int out_dtype, int H, const void* cam_flag0,
+                   const void* cam_flag1, const void* cam_flag2, const void* cam_flag3, int cams, const void* tok_flag, void* pad_out,
+                   void* stream) {
+  if ((img_dtype != TK_BF16 && img_dtype != TK_F32) || (out_dtype != TK_BF16 && out_dtype != TK_F32))
+    return fail(TK_EINVAL, "prefix_rows: image rows and result are bf16 or fp32 (img_dtype=%d, out_dtype=%d)", img_dtype, out_dtype);
   if (n_img < 0 || n_tok < 0 || n_last < 0 || n_img + n_tok + n_last < 1 || H <= 0 || H % 8)
     return fail(TK_EINVAL, "prefix_rows: row counts %d + %d + %d must be non-negative with a row in all, H=%d a multiple of 8", n_img, n_tok,
                 n_last, H);
@@ -1363,7 +1379,8 @@ int tk_prefix_rows(const void* img, int n_img, float img_scale, const void* tabl
     a.per_cam = n_img ? n_img / cams : 1;
     for (int i = 0; i < 4; ++i) a.cam_flag[i] = (const unsigned char*)flags[(n_img && i < cams) ? i : 0];
   }
-  a.img = (const u16*)img;
+  a.img = img;
+  a.img_f32 = img_dtype == TK_F32;
   a.n_img = n_img;
   a.img_scale = img_scale;
   a.table = (const u16*)table;
@@ -1373,7 +1390,8 @@ int tk_prefix_rows(const void* img, int n_img, float img_scale, const void* tabl
   a.tok_scale = tok_scale;
   a.last = (const float*)last;
   a.n_last = n_last;
-  a.out = (float*)out;
+  a.out = out;
+  a.out_bf16 = out_dtype == TK_BF16;
   a.H = H;
   a.tok_flag = (const unsigned char*)tok_flag;
   a.pad_out = (unsigned char*)pad_out;

@@ -244,13 +244,14 @@ struct PatchifyArgs {
   const float* img[4];  // fp32 [3][H][W] each
   int n, H, W, ps;
   float scale, shift;
-  unsigned short* out;  // bf16 [n * (H/ps) * (W/ps)][3 * ps * ps]
+  void* out;  // bf16 (ps a multiple of 8) or fp32 (out_f32; ps even) [n * (H/ps) * (W/ps)][3 * ps * ps]
+  int out_f32;
 };
 int tk_launch_patchify(PatchifyArgs a, hipStream_t st);
 
 struct PrefixRowsArgs {
-  const unsigned short* img;  // bf16 [n_img, H]: rows 0 .. n_img-1 of the result are bf16(img * img_scale)
-  int n_img;
+  const void* img;  // bf16 [n_img, H]: rows 0 .. n_img-1 of the result are bf16(img * img_scale); fp32 (img_f32): the rows as they are
+  int n_img, img_f32;
   float img_scale;
   const unsigned short* table;  // bf16 [vocab, H]: rows n_img .. n_img+n_tok-1 are bf16(table[tokens[t]] * tok_scale)
   const long long* tokens;
@@ -258,8 +259,8 @@ struct PrefixRowsArgs {
   float tok_scale;
   const float* last;  // fp32 [n_last, H]: the closing rows, as they are
   int n_last;
-  float* out;  // fp32 [n_img + n_tok + n_last, H]
-  int H;
+  void* out;  // fp32, or bf16 (out_bf16: every value rounded once more, a no-op for the scaled rows) [n_img + n_tok + n_last, H]
+  int H, out_bf16;
   // optional pad flags of the same rows: a flag per camera (n_img = cams * per_cam rows), a flag per token, 1 for the closing rows
   const unsigned char* cam_flag[4];
   int cams, per_cam;

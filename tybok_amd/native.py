@@ -84,6 +84,7 @@ SIGNATURES: dict[str, tuple] = {
                                   c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "tk_prefix_meta": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "tk_patchify_images": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_void_p]),
+    "tk_patchify_images_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_void_p]),
     "tk_layer_norm_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p]),
     "tk_add_layer_norm_f16": (
         c_int,
@@ -133,7 +134,7 @@ SIGNATURES: dict[str, tuple] = {
     ),  # fmt: skip
     "tk_prefix_rows": (
         c_int,
-        [c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+        [c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
     ),  # fmt: skip
     "tk_add_layer_norm_rows": (
         c_int,

@@ -1087,9 +1087,10 @@ def prefix_meta(pad: torch.Tensor, att: torch.Tensor | None, rope_positions: int
     return mask2d, pos32, suf
 
 
-def patchify_images(images, patch: int, scale: float = 1.0, shift: float = 0.0) -> torch.Tensor:
-    """Up to four fp32 images ``[1, 3, H, W]`` (or ``[3, H, W]``) -> bf16 ``[n, (H/patch) * (W/patch), 3 * patch * patch]``
-    rows of ``x * scale + shift`` in the order of ``unfold``: the patch embedding's GEMM input."""
+def patchify_images(images, patch: int, scale: float = 1.0, shift: float = 0.0, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """Up to four fp32 images ``[1, 3, H, W]`` (or ``[3, H, W]``) -> ``[n, (H/patch) * (W/patch), 3 * patch * patch]``
+    rows of ``x * scale + shift`` in the order of ``unfold``: the patch embedding's GEMM input, in bf16 (patch sizes
+    that are multiples of 8) or fp32 (any even patch size)."""
     lib = native.lib()
     images = list(images)
     if not 1 <= len(images) <= 4:
@@ -1098,29 +1099,37 @@ def patchify_images(images, patch: int, scale: float = 1.0, shift: float = 0.0) 
     for img in images:
         if img.dtype != torch.float32 or not img.is_contiguous() or img.numel() != 3 * h * w:
             raise TypeError("patchify_images: every image must be a contiguous fp32 tensor of 3 x H x W values")
-    out = torch.empty(len(images), (h // patch) * (w // patch), 3 * patch * patch, dtype=torch.bfloat16, device=images[0].device)
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("patchify_images: bf16 or fp32 patch rows")
+    out = torch.empty(len(images), (h // patch) * (w // patch), 3 * patch * patch, dtype=out_dtype, device=images[0].device)
     ptrs = [img.data_ptr() for img in images] + [None] * (4 - len(images))
-    rc = lib.tk_patchify_images(*ptrs, len(images), h, w, int(patch), float(scale), float(shift), out.data_ptr(), _stream())
+    fn = lib.tk_patchify_images if out_dtype == torch.bfloat16 else lib.tk_patchify_images_f32
+    rc = fn(*ptrs, len(images), h, w, int(patch), float(scale), float(shift), out.data_ptr(), _stream())
     native.check(rc, "tk_patchify_images")
     return out
 
 
-def prefix_rows(img, img_scale: float, table, tokens, tok_scale: float, last, *, cam_flags=None, tok_flags=None):
-    """The fp32 prefix ``[1, P, H]`` of one request in one launch: ``img`` bf16 ``[cams, per_cam, H]`` times ``img_scale``
-    and ``table[tokens]`` (bf16 ``[vocab, H]``, ids int64 ``[n_tok]``) times ``tok_scale`` -- both products rounded to
-    bf16 as the tensor products are -- then ``last`` fp32 ``[n_last, H]`` as it is.  With ``cam_flags`` (a bool tensor of
-    one element per camera) and ``tok_flags`` (bool ``[n_tok]``) also the pad flags ``[1, P]`` of those rows (the closing
-    rows are always valid); returns ``(rows, flags or None)``."""
+def prefix_rows(img, img_scale: float, table, tokens, tok_scale: float, last=None, *, cam_flags=None, tok_flags=None, out_dtype: torch.dtype = torch.float32):
+    """The prefix ``[1, P, H]`` of one request in one launch: ``img [cams, per_cam, H]`` -- bf16: times ``img_scale``,
+    rounded to bf16 as the tensor product is; fp32: as it is -- then ``table[tokens]`` (bf16 ``[vocab, H]``, ids int64
+    ``[n_tok]``) times ``tok_scale``, rounded likewise, then ``last`` fp32 ``[n_last, H]`` (or None) as it is; written
+    in fp32 or rounded to bf16 (``out_dtype``).  With ``cam_flags`` (a bool tensor of one element per camera) and
+    ``tok_flags`` (bool ``[n_tok]``) also the pad flags ``[1, P]`` of those rows (the closing rows are always valid);
+    returns ``(rows, flags or None)``."""
     lib = native.lib()
     bf = torch.bfloat16
-    if img.dtype != bf or table.dtype != bf or last.dtype != torch.float32 or tokens.dtype != torch.int64:
-        raise TypeError("prefix_rows: img and table bf16, tokens int64, last fp32")
+    if img.dtype not in (bf, torch.float32) or table.dtype != bf or tokens.dtype != torch.int64 or (last is not None and last.dtype != torch.float32):
+        raise TypeError("prefix_rows: img bf16 or fp32, table bf16, tokens int64, last fp32")
+    if out_dtype not in (bf, torch.float32):
+        raise TypeError("prefix_rows: fp32 or bf16 rows")
     h = table.shape[1]
-    if img.dim() != 3 or img.shape[2] != h or last.dim() != 2 or last.shape[1] != h or not (img.is_contiguous() and table.is_contiguous() and last.is_contiguous() and tokens.is_contiguous()):
-        raise ValueError("prefix_rows: img [cams, per_cam, H], table [vocab, H], last [n_last, H], all contiguous")
-    cams, n_img, n_tok, n_last = img.shape[0], img.shape[0] * img.shape[1], tokens.numel(), last.shape[0]
+    if img.dim() != 3 or img.shape[2] != h or not (img.is_contiguous() and table.is_contiguous() and tokens.is_contiguous()):
+        raise ValueError("prefix_rows: img [cams, per_cam, H], table [vocab, H], tokens, all contiguous")
+    if last is not None and (last.dim() != 2 or last.shape[1] != h or not last.is_contiguous()):
+        raise ValueError("prefix_rows: last [n_last, H], contiguous")
+    cams, n_img, n_tok, n_last = img.shape[0], img.shape[0] * img.shape[1], tokens.numel(), 0 if last is None else last.shape[0]
     total = n_img + n_tok + n_last
-    out = torch.empty(1, total, h, dtype=torch.float32, device=img.device)
+    out = torch.empty(1, total, h, dtype=out_dtype, device=img.device)
     flags, fl = None, [None] * 4
     if cam_flags is not None:
         cam_flags = list(cam_flags)
@@ -1131,9 +1140,9 @@ def prefix_rows(img, img_scale: float, table, tokens, tok_scale: float, last, *,
         flags = torch.empty(1, total, dtype=torch.bool, device=img.device)
         fl = [f.data_ptr() for f in cam_flags] + [None] * (4 - cams)
     rc = lib.tk_prefix_rows(
-        img.data_ptr(), n_img, float(img_scale), table.data_ptr(), tokens.data_ptr(), n_tok, table.shape[0], float(tok_scale),
-        last.data_ptr(), n_last, out.data_ptr(), h, *fl, cams, tok_flags.data_ptr() if flags is not None else None,
-        flags.data_ptr() if flags is not None else None, _stream(),
+        img.data_ptr(), _BF16 if img.dtype == bf else _F32, n_img, float(img_scale), table.data_ptr(), tokens.data_ptr(), n_tok, table.shape[0],
+        float(tok_scale), None if last is None else last.data_ptr(), n_last, out.data_ptr(), _BF16 if out_dtype == bf else _F32, h, *fl, cams,
+        tok_flags.data_ptr() if flags is not None else None, flags.data_ptr() if flags is not None else None, _stream(),
     )  # fmt: skip
     native.check(rc, "tk_prefix_rows")
     return out, flags

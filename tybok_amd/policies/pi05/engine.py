@@ -340,7 +340,7 @@ class PI05Engine(ChunkRuntime, PolicyEngine):
 
     def _core(self, images01, img_masks, tokens, masks, noise) -> torch.Tensor:
         """The unit a graph records: the change of range of the images and the whole model."""
-        return self.model.sample_actions([img * 2.0 - 1.0 for img in images01], img_masks, tokens, masks, noise)
+        return self.model.sample_actions(images01, img_masks, tokens, masks, noise, image_range01=True)
 
     def _infer(self, batch: dict[str, torch.Tensor], noise: torch.Tensor | None) -> torch.Tensor:
         images, img_masks = self.prepare_images01(batch)

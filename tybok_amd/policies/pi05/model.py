@@ -141,6 +141,7 @@ class PI05Model:
                 for i in range(self.depth)
             ]
         self.embed_scale = torch.tensor(self.vd["width"] ** 0.5, dtype=BF16, device=self.device)
+        self._embed_scale_value = float(torch.tensor(self.vd["width"] ** 0.5, dtype=BF16))  # the same bf16-rounded factor, on the host
         self.patch_w = self.p[VIS + "embeddings.patch_embedding.weight"].reshape(cfg.vision_hidden, -1)
         # low-precision copies of the vision tower's linears (the drift tiers convert weights and bias)
         self.vis_lowp: dict[str, tuple[torch.Tensor, torch.Tensor]] = {}
@@ -239,13 +240,29 @@ class PI05Model:
         return self.rope_cos[pos].to(dtype), self.rope_sin[pos].to(dtype)
 
     # ------------------------------------------------------------------ vision + prefix
-    def embed_image(self, image: torch.Tensor) -> torch.Tensor:
-        """``[1, 3, 224, 224]`` fp32 in [-1, 1] -> ``[1, 256, vlm_width]`` fp32 (SigLIP tower + projector, fp32)."""
+    def _patch_rows_ok(self, images01) -> bool:
+        """One launch can scale and unfold these [0, 1] images: one to four fp32 batch-1 images of one size on the GPU,
+        an even patch size that divides them."""
+        ps = self.cfg.vision_patch
+        first = images01[0]
+        return (
+            1 <= len(images01) <= 4 and first.is_cuda and ps % 2 == 0 and first.dim() == 4 and first.shape[2] % ps == 0 and first.shape[3] % ps == 0
+            and all(i.dtype == torch.float32 and i.shape == first.shape and i.shape[0] == 1 and i.shape[1] == 3 and i.is_contiguous() for i in images01)
+        )  # fmt: skip
+
+    def embed_image(self, image: torch.Tensor | None, images01=None) -> torch.Tensor:
+        """``[1, 3, 224, 224]`` fp32 in [-1, 1] -> ``[1, 256, vlm_width]`` fp32 (SigLIP tower + projector, fp32).
+        ``images01``: a list of batch-1 images still in [0, 1] instead (see :meth:`_patch_rows_ok`): ``x * 2 - 1`` and
+        the unfolding of all of them are one launch."""
         cfg, p = self.cfg, self.p
-        b = image.shape[0]
         ps = cfg.vision_patch
-        n_h, n_w = image.shape[2] // ps, image.shape[3] // ps
-        x = image.float().view(b, 3, n_h, ps, n_w, ps).permute(0, 2, 4, 1, 3, 5).reshape(b, n_h * n_w, 3 * ps * ps)
+        if images01 is not None:
+            b = len(images01)
+            x = tk.patchify_images(images01, ps, 2.0, -1.0, out_dtype=torch.float32)
+        else:
+            b = image.shape[0]
+            n_h, n_w = image.shape[2] // ps, image.shape[3] // ps
+            x = image.float().view(b, 3, n_h, ps, n_w, ps).permute(0, 2, 4, 1, 3, 5).reshape(b, n_h * n_w, 3 * ps * ps)
         x = F.linear(x, self.patch_w, p[VIS + "embeddings.patch_embedding.bias"])
         x = x + p[VIS + "embeddings.position_embedding.weight"][None]
         vh, heads = cfg.vision_hidden, cfg.vision_heads
@@ -404,6 +421,26 @@ class PI05Model:
         pads.append(masks)
         return torch.cat(embs, dim=1), torch.cat(pads, dim=1)
 
+    def prefix_hidden(self, images01, img_masks, tokens, masks):
+        """The prefill's bf16 hidden rows ``[P, W]`` and the pad flags ``[1, P]`` straight from [0, 1] images, for one
+        request on the GPU: what ``embed_prefix(images * 2 - 1, ...)`` followed by ``.to(bfloat16)`` gives, with the
+        change of range and the unfolding in one launch and the embedding lookup, its scale, the concatenation, the cast
+        and the flags in another.  None when a piece does not have the form those launches take."""
+        table = self.p[VLM + "embed_tokens.weight"]
+        if not (
+            self._patch_rows_ok(images01) and tokens.shape[0] == 1 and tokens.dtype == torch.int64 and masks.dtype == torch.bool
+            and table.dtype == BF16 and len(img_masks) == len(images01) and all(m.dtype == torch.bool and m.numel() == 1 for m in img_masks)
+        ):  # fmt: skip
+            return None
+        per_all = self.embed_image(None, images01=list(images01))
+        if per_all.dtype != torch.float32:
+            return None
+        hidden, pads = tk.prefix_rows(
+            per_all.contiguous(), 1.0, table, tokens[0].contiguous(), self._embed_scale_value, None, cam_flags=img_masks,
+            tok_flags=masks[0].contiguous(), out_dtype=BF16,
+        )  # fmt: skip
+        return hidden[0], pads
+
     def _attn_proj(self, lp: str, h: torch.Tensor, cos, sin):
         b, length = h.shape[0], h.shape[1]
         q = self.lin(lp + "q_proj", h).view(b, length, -1, self.head_dim).transpose(1, 2)
@@ -430,19 +467,23 @@ class PI05Model:
             hidden = self.vlm_mlp[i](h, hidden)
         return kv
 
-    def prefill_fused(self, embs: torch.Tensor, pad_masks: torch.Tensor):
+    def prefill_fused(self, embs: torch.Tensor | None, pad_masks: torch.Tensor, hidden: torch.Tensor | None = None, suffix_len: int = 0):
         """VLM prefill on the fused launches (norm + q|k|v + RoPE, attention under the pad x pad mask,
         o_proj + residual, GeGLU FFN) -> ``(kv, caches)``: ``kv`` per-layer ``(K, V) [1, G, P, D]`` views
-        of the projection outputs, ``caches`` the same keys with V^T in the attention kernel's layout."""
-        p_len = embs.shape[1]
+        of the projection outputs, ``caches`` the same keys with V^T in the attention kernel's layout.
+        ``hidden``: the bf16 rows ``[P, W]`` when the caller already has them (``embs`` is then not read).
+        ``suffix_len``: also return, as a third value, the rotary positions of that many action tokens behind the
+        valid prefix (from the bookkeeping launch that writes the mask and the prefix positions)."""
+        p_len = pad_masks.shape[1]
         p_pad = (p_len + 31) // 32 * 32
         heads, g, d = self.vd["num_heads"], self.vd["num_kv_heads"], self.head_dim
         nq, nkv = heads * d, g * d
         # pad x pad visibility bytes and clamp(cumsum(pad) - 1) positions: one launch
-        mask2d, pos32, _ = tk.prefix_meta(pad_masks[0].contiguous(), None, _ROPE_POSITIONS)
+        mask2d, pos32, suf_pos = tk.prefix_meta(pad_masks[0].contiguous(), None, _ROPE_POSITIONS, suffix_len)
         qkv_all = torch.empty(self.depth, p_len, nq + 2 * nkv, dtype=BF16, device=self.device)
         vt_all = torch.zeros(self.depth, nkv, p_pad, dtype=BF16, device=self.device)
-        hidden = embs[0].to(BF16)
+        if hidden is None:
+            hidden = embs[0].to(BF16)
         kv, caches = [], []
         many_rows = p_len >= 256  # the projections on the many-row MFMA kernels
         for i in range(self.depth):
@@ -477,7 +518,7 @@ class PI05Model:
                 hidden = mlp(h, out[None])[0]
             kv.append((k.transpose(0, 1)[None], qkv[:, nq + nkv :].view(p_len, g, d).transpose(0, 1)[None]))
             caches.append(cache)
-        return kv, caches
+        return (kv, caches, suf_pos) if suffix_len else (kv, caches)
 
     # ------------------------------------------------------------------ denoising
     def attention_caches(self, kv) -> list:
@@ -554,28 +595,43 @@ class PI05Model:
         out, _ = gemma_norm(hidden, modulation=self.final_mods[step])
         return self.lin("action_out_proj", out.to(torch.float32))
 
-    def sample_actions(self, images, img_masks, tokens, masks, noise, trace: dict | None = None) -> torch.Tensor:
-        """Prefix embed, prefill, Euler loop -> ``[1, chunk, max_action_dim]`` fp32."""
-        if self.pad_free and not (self.device.type == "cuda" and torch.cuda.is_current_stream_capturing()):
+    def sample_actions(self, images, img_masks, tokens, masks, noise, trace: dict | None = None, image_range01: bool = False) -> torch.Tensor:
+        """Prefix embed, prefill, Euler loop -> ``[1, chunk, max_action_dim]`` fp32.  ``image_range01``: the images are
+        still in [0, 1] (``x * 2 - 1`` is applied here, inside the unfolding launch where that is possible)."""
+        capturing = self.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
+        if self.pad_free and not capturing:
             tokens, masks = self.pack_language(tokens, masks)  # (a recorded shape already has the bucket's length)
-        embs, pads = self.embed_prefix(images, img_masks, tokens, masks)
-        caches = None
-        if self.fused_prefill and embs.shape[0] == 1:
-            kv, caches = self.prefill_fused(embs, pads)
+        fused_loop = self.fused_expert and noise.shape[0] == 1 and noise.dtype == torch.float32 and noise.is_contiguous() and all(m.fp8 for m in self.exp_mlp)
+        suffix_len = noise.shape[1] if fused_loop else 0
+        caches = suf_pos = direct = None
+        if image_range01 and trace is None and self.fused_prefill and (capturing or not self.skip_empty_images):
+            direct = self.prefix_hidden(images, img_masks, tokens, masks)
+        if direct is not None:
+            hidden, pads = direct
+            kv, caches, *rest = self.prefill_fused(None, pads, hidden=hidden, suffix_len=suffix_len)
+            suf_pos = rest[0] if rest else None
         else:
-            kv = self.prefill(embs, pads)
-        if trace is not None:
-            trace.update(prefix_embs=embs, pad_masks=pads, kv=kv)
+            if image_range01:
+                images = [img * 2.0 - 1.0 for img in images]
+            embs, pads = self.embed_prefix(images, img_masks, tokens, masks)
+            if self.fused_prefill and embs.shape[0] == 1:
+                kv, caches, *rest = self.prefill_fused(embs, pads, suffix_len=suffix_len)
+                suf_pos = rest[0] if rest else None
+            else:
+                kv = self.prefill(embs, pads)
+            if trace is not None:
+                trace.update(prefix_embs=embs, pad_masks=pads, kv=kv)
         dt = -1.0 / self.num_steps
         x_t = noise
         if caches is None or not self.fused_expert:
             caches = self.attention_caches(kv) if self.fused_expert else None
-        if self.fused_expert and x_t.shape[0] == 1 and x_t.dtype == torch.float32 and x_t.is_contiguous() and all(m.fp8 for m in self.exp_mlp):
+        if fused_loop:
             # fused loop: positions once per request, Euler update inside the step's last launch
             s = x_t.shape[1]
             if self.vt_suf is None or self.vt_suf.shape[2] < (s + 31) // 32 * 32:
                 self.vt_suf = torch.zeros(kv[0][0].shape[1], self.head_dim, (s + 31) // 32 * 32, dtype=BF16, device=self.device)
-            pos32 = tk.prefix_meta(pads[0].contiguous(), None, _ROPE_POSITIONS, s, want_mask=False)[2]  # clamp(sum(pad) + arange(s))
+            # clamp(sum(pad) + arange(s)): from the prefill's bookkeeping launch, or a launch of its own
+            pos32 = suf_pos if suf_pos is not None else tk.prefix_meta(pads[0].contiguous(), None, _ROPE_POSITIONS, s, want_mask=False)[2]
             # (`action_in_proj` stays the library's fp32 product + cast, two launches a step: carried in the tail launch
             # of the step before -- tk_expert_tail_embed -- it sums its 32 terms in another order, and that re-draw of
             # a few bf16 roundings moved one frame's maximum error from under to over the cap held for this path)
