@@ -586,8 +586,10 @@ def main() -> None:
         oracle_frame.update(tokens=b3["observation.language.tokens"].cpu(), lang_masks=b3["observation.language.attention_mask"].cpu(), state=engine.prepare_state(b3).cpu())
     unnorm = engine.unnormalizer
     frame2 = device_frame(engine, 2)
+    spin_up()  # (building the frames above is tens of milliseconds of host work: the clocks have fallen back)
     samples2, _ = time_requests(engine, frame2, noise, max(5, args.steps // 2), 2)
     host_frame = {k: (v.cpu() if hasattr(v, "cpu") else v) for k, v in frame3.items()}
+    spin_up()
     samples_host, _ = time_requests(engine, host_frame, noise.cpu(), max(5, args.steps // 2), 2)
     graph_ok = bool(engine.graph_enabled)
     del engine
@@ -602,6 +604,7 @@ def main() -> None:
         flags5["tl_fused_vit"] = True  # the reference's fused tower: fp16 q|k|v and attention, bf16 out_proj and MLP
         eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **flags5)
         frame5 = device_frame(eng5, 2)
+        spin_up()
         s5, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
         pi05_p50 = float(np.percentile(s5, 50))
         del eng5
@@ -612,6 +615,7 @@ def main() -> None:
         frame5p = dict(frame5)
         frame5p["observation.language.tokens"] = torch.randint(0, eng5.config.vocab_size, (200,), generator=torch.Generator().manual_seed(1)).cuda()
         frame5p["observation.language.attention_mask"] = torch.arange(200, device="cuda") < 40
+        spin_up()
         s5p, _ = time_requests(eng5, frame5p, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 3)
         pi05_pad_free_p50 = float(np.percentile(s5p, 50))
         del eng5
@@ -619,6 +623,7 @@ def main() -> None:
         # the same request with the VLM MLP in W8A8 (activations quantised per token, fp8 x fp8 products): the
         # arithmetic of the reference's own --tl-fp8-llm-mlp tier; an opt-in drift tier here
         eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **{**flags5, "tl_fp8_llm_mlp": "w8a8"})
+        spin_up()
         s5w, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
         pi05_w8a8_p50 = float(np.percentile(s5w, 50))
         del eng5
@@ -626,6 +631,7 @@ def main() -> None:
         # and with the vision tower on the tier that a fixture from the reference's own tower pins end to end: fp32
         # attention and norms, only fc1 / fc2 in bf16 (--vit-mlp-dtype bf16) on the many-row kernel
         eng5 = create_engine(ckpt5, device="cuda", graph=True, warmup=True, **{**flags5, "tl_fused_vit": False, "vit_mlp_dtype": "bf16"})
+        spin_up()
         s5m, _ = time_requests(eng5, frame5, torch.zeros(1, 50, 7, device="cuda"), max(5, args.steps // 3), 2)
         pi05_mlp_tier_p50 = float(np.percentile(s5m, 50))
         del eng5
