@@ -249,15 +249,16 @@ def test_batched_vision_attention(tk):
 
 @pytest.mark.parametrize(
     "b,m,p,h,g,d",
-    [(3, 1024, 1024, 12, 12, 64), (3, 1000, 1000, 12, 12, 64), (6, 520, 300, 12, 4, 64), (2, 200, 200, 4, 4, 64), (1, 130, 300, 6, 2, 64),
-     (2, 160, 160, 3, 3, 96), (1, 128, 129, 2, 1, 96)],
+    [(3, 1024, 1024, 12, 12, 64), (3, 1000, 1000, 12, 12, 64), (6, 520, 300, 12, 4, 64), (2, 1024, 640, 12, 12, 64), (2, 200, 200, 4, 4, 64),
+     (1, 130, 300, 6, 2, 64), (2, 160, 160, 3, 3, 96), (1, 128, 129, 2, 1, 96), (5, 1024, 320, 16, 16, 96)],
 )  # fmt: skip
 def test_tower_attention_ragged_shapes(tk, b, m, p, h, g, d):
     # the many-query path (128 queries per block, keys in stages of 64): full SmolVLA tower shape, query and
     # key counts that end inside a tile / a stage, grouped heads, both head sizes; zero-padded V^T keys.  On a
     # 256-CU device the first two shapes take the five-tile blocks (288 four-tile blocks would double up on some
     # CUs, 252 five-tile blocks fit one per CU; the second ends inside a block, a tile and a stage), the third the
-    # four-tile blocks two per CU (360 blocks), the others the four-tile blocks one per CU
+    # four-tile blocks two per CU (360 blocks), the fourth the four-tile blocks one per CU (192), the next four the
+    # two-tile blocks (grids that would leave more than half of the CUs idle), the last the four-tile blocks at head size 96
     gen = torch.Generator().manual_seed(17)
     q = torch.randn(b, m, h, d, generator=gen).to(torch.bfloat16)
     k = torch.randn(b, p, g, d, generator=gen).to(torch.bfloat16)

@@ -82,6 +82,10 @@ struct TowerLds {
 // fp32 softmax); otherwise they stay fp32.
 // F16: q, K, V^T are fp16 and the probabilities are rounded to fp16 for P.V (both products on the fp16 matrix
 // instruction); the output stays bf16.
+// QT: query tiles per block (each group of QT waves walks one half of the keys): 4, 5 where four-tile blocks would put two
+// blocks on some CUs and one on the rest, 2 where four-tile blocks would leave more than half of the CUs idle (pi0.5's
+// tower: 2 x 256 tokens, 16 heads: 64 -> 128 blocks, 9.9 -> 7.0 us; one 1024-token camera: 17.9 -> 13.3 us); a wave's
+// arithmetic does not depend on it, so every form gives the same bits.
 // WPE: waves per SIMD the registers are budgeted for -- 4 lets two four-tile blocks of head size 64 share a CU (128
 // registers per lane, a few of them spilled); 2 / 3 when the grid puts one block on a CU anyway.
 template <int D, bool LB, bool F16, int QT, int WPE>
@@ -323,10 +327,13 @@ int launch_tower(const AttnArgs& a, hipStream_t st, int cus) {
     // five-tile blocks where four-tile ones would double up on some CUs (see QT above); else two blocks per CU
     const int pairs = a.batch * a.H, tiles = (a.M + 31) / 32;
     const int b4 = pairs * ((tiles + 3) / 4), b5 = pairs * ((tiles + 4) / 5);
+    if (2 * b4 <= cus && tiles >= 2) return launch_tower_qt<D, LB, F16, 2, 2>(a, st);  // few blocks: two-tile blocks on twice the CUs
     if (b4 <= cus) return launch_tower_qt<D, LB, F16, 4, 2>(a, st);
     if (b4 < 2 * cus && b5 <= cus) return launch_tower_qt<D, LB, F16, 5, 3>(a, st);
     return launch_tower_qt<D, LB, F16, 4, 4>(a, st);
   } else {
+    const int pairs = a.batch * a.H, tiles = (a.M + 31) / 32;
+    if (2 * pairs * ((tiles + 3) / 4) <= cus && tiles >= 2) return launch_tower_qt<D, LB, F16, 2, 2>(a, st);
     return launch_tower_qt<D, LB, F16, 4, 2>(a, st);
   }
 }
