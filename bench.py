@@ -212,26 +212,31 @@ def attn_launch_us(launches: int = 100, reps: int = 10) -> float:
     return e0.elapsed_time(e1) * 1e3 / (reps * launches)
 
 
-def tower_attn_launch_us(cameras: int = 3, tokens: int = 1024, heads: int = 12, d: int = 64, launches: int = 20, reps: int = 10) -> float:
-    """Average duration (us) of one vision-tower attention launch (SmolVLA tower: one 1024-token problem
-    per camera, 12 heads of 64, bf16-rounded logits) inside a replayed graph."""
+def tower_attn_launch_us(cameras: int = 3, tokens: int = 1024, heads: int = 12, d: int = 64, launches: int = 20, reps: int = 10,
+                         fp16_head: int | None = None) -> float:
+    """Average duration (us) of one vision-tower attention launch inside a replayed graph: SmolVLA's tower (one
+    1024-token problem per camera, 12 heads of 64, bf16 operands, bf16-rounded logits) or, with ``fp16_head`` = the
+    true head size, pi0.5's fused tower tier (fp16 operands, heads of ``fp16_head`` columns zero-padded to ``d``)."""
     import torch
 
     from tybok_amd import ops as tk
 
     g = torch.Generator().manual_seed(0)
-    qkv = torch.randn(cameras, tokens, 3, heads, d, generator=g).to(torch.bfloat16).cuda()
+    qkv = torch.randn(cameras, tokens, 3, heads, d, generator=g).to(torch.float16 if fp16_head else torch.bfloat16).cuda()
+    kw = dict(scale=fp16_head**-0.5) if fp16_head else dict(logits_bf16=True)
+    if fp16_head:
+        qkv[..., fp16_head:] = 0
     vt = tk.transpose_v(qkv[:, :, 2])
     out = torch.empty(cameras, tokens, heads * d, dtype=torch.bfloat16, device="cuda")
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         for _ in range(3):
-            tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, out=out)
+            tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, out=out, **kw)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.inference_mode(), torch.cuda.graph(graph, stream=stream):
         for _ in range(launches):
-            tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, logits_bf16=True, out=out)
+            tk.batched_attn(qkv[:, :, 0], qkv[:, :, 1], vt, out=out, **kw)
     spin_up(60.0)
     for _ in range(3):
         graph.replay()
@@ -549,7 +554,9 @@ def main() -> None:
         spin_up()
         us = tower_attn_launch_us(launches=20, reps=args.steps)
         flops = 4.0 * 3 * 12 * 1024 * 1024 * 64
-        print(json.dumps({"tower_attn_only": {"B": 3, "M": 1024, "P": 1024, "H": 12, "D": 64, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1)}}), flush=True)
+        us5 = tower_attn_launch_us(cameras=2, tokens=256, heads=16, d=96, launches=20, reps=args.steps, fp16_head=72)
+        print(json.dumps({"tower_attn_only": {"B": 3, "M": 1024, "P": 1024, "H": 12, "D": 64, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
+                                              "pi05_fp16_B2_M256_H16_D96": {"us": round(us5, 2)}}}), flush=True)  # fmt: skip
         return
     if args.attn_only:
         spin_up()
@@ -714,6 +721,7 @@ def main() -> None:
         "ffn_M50_K720_I2048": {"us": round(c1_us, 2), "GBps": round(c1_bytes / c1_us / 1e3, 1), "launches": 2},
         "expert_attn_M50_P241_S50_H15_G5_D64": {"us": round(attn_launch_us(launches=50, reps=10), 2)},
         "tower_attn_B3_M1024_H12_D64": {"us": round(tower_attn_launch_us(launches=20, reps=10), 2)},
+        "pi05_tower_attn_fp16_B2_M256_H16_D96": {"us": round(tower_attn_launch_us(cameras=2, tokens=256, heads=16, d=96, launches=20, reps=10, fp16_head=72), 2)},
         "pi05_expert_attn_M50_P712_S50_H8_G1_D256": {"us": round(attn_d256_launch_us(launches=20, reps=10), 2)},
     }
     for name, dm, dk, dn, dact in TOWER_LINEARS:  # the vision tower's linears on the many-row bf16 kernel
